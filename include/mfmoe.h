@@ -1,0 +1,250 @@
+/*
+ * mfmoe.h — C ABI of libmfmoe: the MoE expert hot path of Mference on MI355X
+ * (gfx950), hand-written HIP behind plain pointers and sizes.
+ *
+ * The reference has no C/FFI interface; its operator surface is a set of Swift
+ * classes under Sources/Mference/Kernels/ whose encode…() methods append
+ * dispatches to a caller-owned MTLCommandBuffer.  Each entry point below names
+ * the Swift method (file:line, relative to the Mference repository root) it
+ * replaces.  Conventions of the mapping:
+ *
+ *   MetalContext                    -> mf_ctx*            (device + kernel state)
+ *   MTLCommandBuffer                -> mf_stream          (a hipStream_t; work is
+ *                                      ordered by the stream, nothing is synchronised)
+ *   (MTLBuffer, byte offset)        -> device pointer, the caller adds the offset
+ *   `throws` / precondition         -> negative mf_status, nothing is launched
+ *   half activations                -> bf16 bit patterns (uint16_t); accumulation
+ *                                      is fp32 and the reference's narrowing points
+ *                                      are kept, narrowing to bf16 instead of fp16
+ *
+ * All pointers are DEVICE pointers unless a parameter says "host".  Activations
+ * and scale/bias tables must be 2-byte aligned; packed weights may have any
+ * alignment (16-byte aligned tensors take the fast 128-bit-load kernels).
+ * A handle (mf_moe*) owns a small device workspace and is therefore serial:
+ * do not use one handle from two streams at once (MapleMoE.swift:3-6).
+ */
+#ifndef MFMOE_H
+#define MFMOE_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define MF_GROUP_SIZE 64 /* Quantization.groupSize, Quantization.swift:5 */
+#define MF_MAX_TOKENS 8  /* kMultiXMaxT, dequant_int4.metal:356 */
+#define MF_MAX_TOPK 8    /* kMaxStreamedExperts, moe.metal:5 */
+#define MF_MAX_EXPERTS 512
+
+typedef enum {
+  MF_OK = 0,
+  MF_ERR_INVALID_ARGUMENT = -1,   /* precondition failures (MoE.swift:165-167) */
+  MF_ERR_DIMENSION_MISMATCH = -2, /* SharedExpertError.dimensionMismatch */
+  MF_ERR_UNSUPPORTED_BITS = -3,   /* SharedExpertError.unsupportedWeightBits */
+  MF_ERR_SCRATCH_TOO_SMALL = -4,  /* SharedExpertError.scratchTooSmall */
+  MF_ERR_NO_DEVICE = -5,          /* MetalError.noDevice */
+  MF_ERR_OUT_OF_MEMORY = -6,
+  MF_ERR_LAUNCH = -7,             /* a HIP call failed; see mf_last_hip_error */
+  /* PrefillMoEGroupingError, PrefillMoEGrouping.swift:52-88 */
+  MF_ERR_QUERY_COUNT = -10,
+  MF_ERR_TOPK = -11,
+  MF_ERR_NUM_EXPERTS = -12,
+  MF_ERR_TILE_EXPERT_COUNT = -13,
+  MF_ERR_PAIR_COUNT = -14,
+  MF_ERR_TOKEN_RANGE = -15,
+  MF_ERR_RANK_RANGE = -16,
+  MF_ERR_EXPERT_RANGE = -17,
+  MF_ERR_DUPLICATE_TOKEN_RANK = -18,
+  MF_ERR_SORT_KEY_COUNT = -19
+} mf_status;
+
+/* weight formats (bits per code) */
+typedef enum {
+  MF_BITS_TERNARY = 1, /* 2-bit codes {0,1,2}, bf16 scale per 64, bias = -scale */
+  MF_BITS_2 = 2,       /* 2-bit affine: 16 codes per uint32, element j at bit 2*(j%16) */
+  MF_BITS_4 = 4        /* 4-bit affine: 8 codes per uint32, element j at bit 4*(j%8)   */
+} mf_bits;
+
+typedef enum {
+  MF_ROUTER_TOPK_SOFTMAX = 0, /* select on logits, softmax over the selected
+                                 (router_topk_select_k8, moe.metal:190-240) */
+  MF_ROUTER_FULL_SOFTMAX = 1  /* softmax over all experts, k x argmax, renormalise
+                                 (maple_router_top8_full_softmax, maple_moe.metal:62-119) */
+} mf_router_mode;
+
+typedef struct mf_ctx mf_ctx;
+typedef struct mf_moe mf_moe;
+typedef void* mf_stream; /* hipStream_t; NULL = the default stream */
+
+/* MoEExpertOffsets, Kernels/MoE/MoE.swift:4-29: byte offsets of the nine
+ * sub-tensors inside one expert blob. */
+typedef struct {
+  uint32_t gate_w, gate_s, gate_b;
+  uint32_t up_w, up_s, up_b;
+  uint32_t down_w, down_s, down_b;
+} mf_expert_offsets;
+
+/* One quantized projection: SharedExpertProjection (SharedExpertInt4.swift). */
+typedef struct {
+  const void* weights;    /* packed codes, rows x cols*bits/8 bytes */
+  const uint16_t* scales; /* bf16 [rows, cols/64] */
+  const uint16_t* biases; /* bf16 [rows, cols/64]; ignored for MF_BITS_TERNARY */
+} mf_qtensor;
+
+/* PrefillTokenExpertPair, Kernels/Prefill/MoE/PrefillRouter.swift:4-28
+ * (16-byte POD).  weight_bits carries the fp32 bit pattern of the routing
+ * weight (the reference carries fp16 bits in the same field). */
+typedef struct {
+  uint32_t token, expert, rank, weight_bits;
+} mf_pair;
+
+/* ---------------------------------------------------------------- context */
+
+/* MetalContext.init, Infrastructure/Metal/MetalContext.swift:45-65 */
+mf_status mf_ctx_create(int device, mf_ctx** out);
+void mf_ctx_destroy(mf_ctx* ctx);
+const char* mf_status_string(mf_status s);
+/* text of the last failing HIP call on this context ("" if none) */
+const char* mf_last_hip_error(const mf_ctx* ctx);
+int mf_abi_version(void);
+
+/* ----------------------------------------------------------------- format */
+
+/* Quantization.quantizeInt4Affine (Infrastructure/ModelIO/Quantization.swift:50-102)
+ * and Int4AffineEncoder.encodeTensor (MferenceRepack/Core/Quantization/
+ * Int4AffineEncoder.swift:41-97), on device: w fp32 [rows, n] -> packed codes,
+ * bf16 scales, bf16 biases.  bits = 4 or 2. */
+mf_status mf_quantize_affine(mf_ctx* ctx, mf_stream stream, const float* w, size_t rows,
+                             size_t n, mf_bits bits, void* packed, uint16_t* scales,
+                             uint16_t* biases);
+/* Quantization.dequantizeInt4Affine (Quantization.swift:104-119): out fp32
+ * [rows, n] = float(q) * scale + bias, two roundings (the bit-exact target). */
+mf_status mf_dequantize(mf_ctx* ctx, mf_stream stream, mf_qtensor q, size_t rows, size_t n,
+                        mf_bits bits, float* out);
+
+/* ------------------------------------------------------------------- GEMV */
+
+/* DequantInt4GEMV.encode (Kernels/Quant/DequantInt4GEMV.swift:57-103) for t = 1,
+ * DequantInt4GEMVMultiX.encode (Kernels/Quant/DequantInt4GEMVMultiX.swift:48-82)
+ * for 1 < t <= 8, MapleTernaryGEMV.encode (Kernels/Quant/MapleTernaryGEMV.swift:
+ * 29-45) for ternary.  x bf16 [t, n], y [t, m] bf16 or fp32 (out_f32 != 0,
+ * the _f32out kernels).  Each weight row is read once for all t tokens. */
+mf_status mf_gemv(mf_ctx* ctx, mf_stream stream, mf_qtensor w, mf_bits bits, const uint16_t* x,
+                  void* y, uint32_t m, uint32_t n, uint32_t t, int out_f32);
+
+/* Elementwise.encode… (Kernels/Primitives/Elementwise.swift:60-87):
+ * silu_mul (utility.metal:21-33), sigmoid_scalar_mul (:49-59), residual_add (:83-92).
+ * gate in mf_sigmoid_scalar_mul is one bf16 value per row of `row` elements. */
+mf_status mf_silu_mul(mf_ctx* ctx, mf_stream stream, const uint16_t* gate, const uint16_t* up,
+                      uint16_t* out, uint32_t count);
+mf_status mf_sigmoid_scalar_mul(mf_ctx* ctx, mf_stream stream, uint16_t* y,
+                                const uint16_t* gate, uint32_t row, uint32_t rows);
+mf_status mf_residual_add(mf_ctx* ctx, mf_stream stream, uint16_t* hidden,
+                          const uint16_t* delta, uint32_t count);
+
+/* SharedExpertInt4.encode (Kernels/MoE/SharedExpertInt4.swift:70-165) /
+ * SharedExpertRuntime.encode (:193-202): y[t,d] = bf16(down . act),
+ * act = bf16(silu(bf16(gate.x)) * bf16(up.x)).  scratch_act holds t*f bf16.
+ * Also the dense SwiGLU MLP of Qwen38ForwardRunner (mlp.encode, :1094). */
+mf_status mf_shared_expert(mf_ctx* ctx, mf_stream stream, const uint16_t* x, mf_qtensor gate,
+                           mf_qtensor up, mf_qtensor down, mf_bits bits, uint32_t d, uint32_t f,
+                           uint32_t t, uint16_t* y, uint16_t* scratch_act,
+                           size_t scratch_act_bytes);
+
+/* ---------------------------------------------------------- MoE operator */
+
+/* Shape/activation specialisation of one operator instance: MoE.init
+ * (Kernels/MoE/MoE.swift:65-151), MoEDeepseekV4.init (MoEDeepseekV4.swift:31-87),
+ * MapleMoE.init (MapleMoE.swift). */
+typedef struct {
+  uint32_t d;            /* hidden size, multiple of 64 */
+  uint32_t f;            /* routed expert intermediate, multiple of 64 */
+  uint32_t num_experts;  /* <= MF_MAX_EXPERTS */
+  uint32_t top_k;        /* 1..MF_MAX_TOPK */
+  mf_bits bits;          /* routed expert format */
+  mf_router_mode router_mode;
+  float swiglu_limit;    /* FC_MOE_SWIGLU_LIMIT, moe.metal:27-34; <= 0: none */
+  uint32_t shared_f;     /* shared expert intermediate; 0 = no shared expert */
+  mf_bits shared_bits;
+} mf_moe_config;
+
+mf_status mf_moe_create(mf_ctx* ctx, const mf_moe_config* cfg, mf_moe** out);
+void mf_moe_destroy(mf_moe* h);
+
+/* Router: bf16 GEMV + top-k + routing weights.
+ * MoEDeepseekV4.encodeRouterGemv + encodeRouterTopK (MoEDeepseekV4.swift:153-173,
+ * 92-100), MoE.encodeRouterGemma4 (MoE.swift:153-203), MapleMoE.encodeRouterTop8
+ * (MapleMoE.swift:81-131), PrefillRouter.encodeGemma4Block for t > 1
+ * (Kernels/Prefill/MoE/PrefillRouter.swift:37-89).
+ * router_w bf16 [num_experts, d]; x bf16, row t at x + t*x_stride elements;
+ * out_idx uint32 [t, top_k]; out_w fp32 [t, top_k]; out_logits fp32
+ * [t, num_experts] or NULL.  Any t >= 1. */
+mf_status mf_moe_router(mf_moe* h, mf_stream stream, const uint16_t* router_w,
+                        const uint16_t* x, uint32_t t, uint32_t x_stride, uint32_t* out_idx,
+                        float* out_w, float* out_logits);
+
+/* Routed phase 1: acts[t,k,f] = bf16(act(gate.x) * up.x).
+ * MoE.encodeRoutedPersistentPhase1U16Load (MoE.swift:220-253),
+ * MoEDeepseekV4.encodeRoutedPhase1 (MoEDeepseekV4.swift:191-199),
+ * MapleMoE.encodePhase1 (MapleMoE.swift:146-150).  Experts are resident:
+ * blob of expert e at expert_base + e*expert_stride (the slab + slot-offset
+ * addressing of MoE.encodeSlotMapGuardedFFN, MoE.swift:333-346), selected on
+ * device by idx[t,k]; idx >= num_experts (router sentinel) gives zero acts. */
+mf_status mf_moe_phase1(mf_moe* h, mf_stream stream, const void* expert_base,
+                        size_t expert_stride, const mf_expert_offsets* offsets,
+                        const uint32_t* idx, const uint16_t* x, uint32_t t, uint32_t x_stride,
+                        uint16_t* acts);
+
+/* Routed phase 2: y[t,d] = bf16(residual[t,d] + sum_k w[t,k] * (down_k . acts[t,k]))
+ * in rank order.  MoE.encodeRoutedPersistentPhase2Reduce (MoE.swift:400-440),
+ * MoEDeepseekV4.encodeRoutedPhase2Reduce (MoEDeepseekV4.swift:265-274).
+ * residual may be NULL (MapleMoE.encodePhase2, MapleMoE.swift:214-219). */
+mf_status mf_moe_phase2(mf_moe* h, mf_stream stream, const void* expert_base,
+                        size_t expert_stride, const mf_expert_offsets* offsets,
+                        const uint32_t* idx, const float* w, const uint16_t* acts,
+                        const uint16_t* residual, uint32_t t, uint16_t* y);
+
+/* Everything one layer reads. */
+typedef struct {
+  const uint16_t* router_w;   /* bf16 [num_experts, d] */
+  const void* expert_base;
+  size_t expert_stride;
+  mf_expert_offsets offsets;
+  mf_qtensor shared_gate, shared_up, shared_down; /* used when shared_f > 0 */
+  const uint16_t* w_sg;       /* bf16 [d] scalar shared gate, or NULL */
+} mf_moe_layer_weights;
+
+/* The fused decode layer, one launch: router -> top-k -> routed gate/up/act ->
+ * down + weighted sum, + gated shared expert.  Replaces the per-layer chain of
+ * RealForwardRunner.produceToken (Runtime/Inference/RealForwardRunner.swift:
+ * 2811-2820 router, :2910-2942 shared expert + sigmoid gate, :3181-3218 routed
+ * phases) with no host readback between router and experts.
+ * x, y bf16 [t, d], t <= MF_MAX_TOKENS; out_idx / out_w may be NULL.
+ * If `hidden` is not NULL, hidden[t,d] = bf16(hidden + y) is applied in the same
+ * launch (residual_add_fp16, utility.metal:83-92). */
+mf_status mf_moe_decode_layer(mf_moe* h, mf_stream stream, const mf_moe_layer_weights* wts,
+                              const uint16_t* x, uint32_t t, uint16_t* y, uint16_t* hidden,
+                              uint32_t* out_idx, float* out_w);
+
+/* ------------------------------------------------------- ragged prefill */
+
+/* PrefillMoEGrouping.groupTokenExpertPairs (Kernels/Prefill/MoE/
+ * PrefillMoEGrouping.swift:91-192) with the reference's full result and error
+ * contract, on HOST pointers: pairs sorted by (sort key, expert, token, rank),
+ * per-expert offsets (0xFFFFFFFF when empty) and counts, groups, and tiles of
+ * <= tile_expert_count live experts.  groups/tiles need room for min(num_experts, n_pairs). */
+typedef struct { uint32_t expert, pair_start, pair_count; } mf_group;
+typedef struct { uint32_t group_start, group_count, pair_start, pair_count; } mf_tile;
+mf_status mf_group_pairs_host(const mf_pair* pairs, size_t n_pairs, int query_count, int top_k,
+                              int num_experts, int tile_expert_count,
+                              const uint64_t* sort_keys, size_t n_sort_keys, mf_pair* sorted,
+                              uint32_t* offsets, uint32_t* counts, mf_group* groups,
+                              size_t* n_groups, mf_tile* tiles, size_t* n_tiles,
+                              uint32_t err_detail[2]);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* MFMOE_H */

@@ -1,0 +1,419 @@
+// The C ABI (include/mfmoe.h): argument validation, workspace ownership and
+// kernel dispatch.  Bad arguments return a negative status and launch nothing.
+#include <stdio.h>
+#include <string.h>
+
+#include <algorithm>
+#include <new>
+#include <vector>
+
+#include "mf_internal.h"
+
+namespace {
+
+constexpr int kAbiVersion = 1;
+
+mf_status fail_hip(mf_ctx* ctx, hipError_t e, const char* what) {
+  if (ctx) snprintf(ctx->hip_error, sizeof ctx->hip_error, "%s: %s", what, hipGetErrorString(e));
+  return e == hipErrorOutOfMemory ? MF_ERR_OUT_OF_MEMORY : MF_ERR_LAUNCH;
+}
+
+#define MF_HIP(ctx, call)                                  \
+  do {                                                     \
+    hipError_t e_ = (call);                                \
+    if (e_ != hipSuccess) return fail_hip(ctx, e_, #call); \
+  } while (0)
+
+bool bits_ok(int bits) { return bits == MF_BITS_4 || bits == MF_BITS_2 || bits == MF_BITS_TERNARY; }
+
+bool qtensor_ok(const mf_qtensor& q, int bits) {
+  if (!q.weights || !q.scales || !mf::aligned2(q.scales)) return false;
+  if (bits != MF_BITS_TERNARY && (!q.biases || !mf::aligned2(q.biases))) return false;
+  return true;
+}
+
+bool offsets_ok(const mf_expert_offsets& o, int bits) {
+  uint32_t tables = o.gate_s | o.up_s | o.down_s;
+  if (bits != MF_BITS_TERNARY) tables |= o.gate_b | o.up_b | o.down_b;
+  return (tables & 1u) == 0;
+}
+
+size_t round_up(size_t v, size_t a) { return (v + a - 1) / a * a; }
+
+}  // namespace
+
+extern "C" {
+
+int mf_abi_version(void) { return kAbiVersion; }
+
+const char* mf_status_string(mf_status s) {
+  switch (s) {
+    case MF_OK: return "ok";
+    case MF_ERR_INVALID_ARGUMENT: return "invalid argument";
+    case MF_ERR_DIMENSION_MISMATCH: return "dimension mismatch";
+    case MF_ERR_UNSUPPORTED_BITS: return "unsupported weight bits";
+    case MF_ERR_SCRATCH_TOO_SMALL: return "scratch too small";
+    case MF_ERR_NO_DEVICE: return "no device";
+    case MF_ERR_OUT_OF_MEMORY: return "out of device memory";
+    case MF_ERR_LAUNCH: return "HIP call failed";
+    case MF_ERR_QUERY_COUNT: return "queryCount must be non-negative";
+    case MF_ERR_TOPK: return "topK must be positive";
+    case MF_ERR_NUM_EXPERTS: return "numExperts must be positive";
+    case MF_ERR_TILE_EXPERT_COUNT: return "tileExpertCount must be in 1...16";
+    case MF_ERR_PAIR_COUNT: return "route pair count mismatch";
+    case MF_ERR_TOKEN_RANGE: return "route token out of range";
+    case MF_ERR_RANK_RANGE: return "route rank out of range";
+    case MF_ERR_EXPERT_RANGE: return "route expert out of range";
+    case MF_ERR_DUPLICATE_TOKEN_RANK: return "duplicate route pair";
+    case MF_ERR_SORT_KEY_COUNT: return "expert sort key count mismatch";
+  }
+  return "unknown status";
+}
+
+mf_status mf_ctx_create(int device, mf_ctx** out) {
+  if (!out) return MF_ERR_INVALID_ARGUMENT;
+  *out = nullptr;
+  int count = 0;
+  if (hipGetDeviceCount(&count) != hipSuccess || device < 0 || device >= count)
+    return MF_ERR_NO_DEVICE;
+  if (hipSetDevice(device) != hipSuccess) return MF_ERR_NO_DEVICE;
+  hipDeviceProp_t prop;
+  if (hipGetDeviceProperties(&prop, device) != hipSuccess) return MF_ERR_NO_DEVICE;
+  auto* ctx = new (std::nothrow) mf_ctx();
+  if (!ctx) return MF_ERR_OUT_OF_MEMORY;
+  ctx->device = device;
+  ctx->num_cu = prop.multiProcessorCount;
+  *out = ctx;
+  return MF_OK;
+}
+
+void mf_ctx_destroy(mf_ctx* ctx) { delete ctx; }
+
+const char* mf_last_hip_error(const mf_ctx* ctx) { return ctx ? ctx->hip_error : ""; }
+
+/* ----------------------------------------------------------------- format */
+
+mf_status mf_quantize_affine(mf_ctx* ctx, mf_stream stream, const float* w, size_t rows,
+                             size_t n, mf_bits bits, void* packed, uint16_t* scales,
+                             uint16_t* biases) {
+  if (!ctx || !w || !packed || !scales || !biases) return MF_ERR_INVALID_ARGUMENT;
+  if (bits != MF_BITS_4 && bits != MF_BITS_2) return MF_ERR_UNSUPPORTED_BITS;
+  if (n % MF_GROUP_SIZE != 0) return MF_ERR_INVALID_ARGUMENT;
+  if (!mf::aligned16(w) || !mf::aligned2(packed) || !mf::aligned2(scales) || !mf::aligned2(biases))
+    return MF_ERR_INVALID_ARGUMENT;
+  MF_HIP(ctx, mf::launch_quantize(static_cast<hipStream_t>(stream), w, rows, n, bits, packed,
+                                  scales, biases));
+  return MF_OK;
+}
+
+mf_status mf_dequantize(mf_ctx* ctx, mf_stream stream, mf_qtensor q, size_t rows, size_t n,
+                        mf_bits bits, float* out) {
+  if (!ctx || !out) return MF_ERR_INVALID_ARGUMENT;
+  if (!bits_ok(bits)) return MF_ERR_UNSUPPORTED_BITS;
+  if (!qtensor_ok(q, bits) || n % MF_GROUP_SIZE != 0) return MF_ERR_INVALID_ARGUMENT;
+  MF_HIP(ctx, mf::launch_dequantize(static_cast<hipStream_t>(stream), q, rows, n, bits, out));
+  return MF_OK;
+}
+
+/* ------------------------------------------------------------------- GEMV */
+
+mf_status mf_gemv(mf_ctx* ctx, mf_stream stream, mf_qtensor w, mf_bits bits, const uint16_t* x,
+                  void* y, uint32_t m, uint32_t n, uint32_t t, int out_f32) {
+  if (!ctx || !x || !y) return MF_ERR_INVALID_ARGUMENT;
+  if (!bits_ok(bits)) return MF_ERR_UNSUPPORTED_BITS;
+  if (!qtensor_ok(w, bits) || !mf::aligned2(x) || !mf::aligned2(y)) return MF_ERR_INVALID_ARGUMENT;
+  if (n == 0 || n % MF_GROUP_SIZE != 0 || t == 0 || t > MF_MAX_TOKENS)
+    return MF_ERR_INVALID_ARGUMENT;
+  if (m == 0) return MF_OK;
+  MF_HIP(ctx, mf::launch_gemv(static_cast<hipStream_t>(stream), w, bits, x, y, m, n, t,
+                              out_f32 != 0));
+  return MF_OK;
+}
+
+mf_status mf_silu_mul(mf_ctx* ctx, mf_stream stream, const uint16_t* gate, const uint16_t* up,
+                      uint16_t* out, uint32_t count) {
+  if (!ctx || !gate || !up || !out) return MF_ERR_INVALID_ARGUMENT;
+  MF_HIP(ctx, mf::launch_silu_mul(static_cast<hipStream_t>(stream), gate, up, out, count));
+  return MF_OK;
+}
+
+mf_status mf_sigmoid_scalar_mul(mf_ctx* ctx, mf_stream stream, uint16_t* y, const uint16_t* gate,
+                                uint32_t row, uint32_t rows) {
+  if (!ctx || !y || !gate) return MF_ERR_INVALID_ARGUMENT;
+  MF_HIP(ctx, mf::launch_sigmoid_scalar_mul(static_cast<hipStream_t>(stream), y, gate, row, rows));
+  return MF_OK;
+}
+
+mf_status mf_residual_add(mf_ctx* ctx, mf_stream stream, uint16_t* hidden, const uint16_t* delta,
+                          uint32_t count) {
+  if (!ctx || !hidden || !delta) return MF_ERR_INVALID_ARGUMENT;
+  MF_HIP(ctx, mf::launch_residual_add(static_cast<hipStream_t>(stream), hidden, delta, count));
+  return MF_OK;
+}
+
+mf_status mf_shared_expert(mf_ctx* ctx, mf_stream stream, const uint16_t* x, mf_qtensor gate,
+                           mf_qtensor up, mf_qtensor down, mf_bits bits, uint32_t d, uint32_t f,
+                           uint32_t t, uint16_t* y, uint16_t* scratch_act,
+                           size_t scratch_act_bytes) {
+  if (!ctx || !x || !y || !scratch_act) return MF_ERR_INVALID_ARGUMENT;
+  if (!bits_ok(bits)) return MF_ERR_UNSUPPORTED_BITS;
+  if (d == 0 || f == 0 || d % MF_GROUP_SIZE != 0 || f % MF_GROUP_SIZE != 0)
+    return MF_ERR_DIMENSION_MISMATCH;
+  if (t == 0 || t > MF_MAX_TOKENS) return MF_ERR_INVALID_ARGUMENT;
+  if (!qtensor_ok(gate, bits) || !qtensor_ok(up, bits) || !qtensor_ok(down, bits))
+    return MF_ERR_INVALID_ARGUMENT;
+  if (!mf::aligned2(x) || !mf::aligned2(y) || !mf::aligned2(scratch_act))
+    return MF_ERR_INVALID_ARGUMENT;
+  if (scratch_act_bytes < static_cast<size_t>(t) * f * sizeof(uint16_t))
+    return MF_ERR_SCRATCH_TOO_SMALL;
+  auto s = static_cast<hipStream_t>(stream);
+  MF_HIP(ctx, mf::launch_gate_up_act(s, gate, up, bits, x, scratch_act, f, d, t));
+  MF_HIP(ctx, mf::launch_gemv(s, down, bits, scratch_act, y, d, f, t, false));
+  return MF_OK;
+}
+
+/* ---------------------------------------------------------- MoE operator */
+
+mf_status mf_moe_create(mf_ctx* ctx, const mf_moe_config* cfg, mf_moe** out) {
+  if (!ctx || !cfg || !out) return MF_ERR_INVALID_ARGUMENT;
+  *out = nullptr;
+  if (!bits_ok(cfg->bits)) return MF_ERR_UNSUPPORTED_BITS;
+  if (cfg->shared_f && !bits_ok(cfg->shared_bits)) return MF_ERR_UNSUPPORTED_BITS;
+  if (cfg->d == 0 || cfg->d % MF_GROUP_SIZE != 0 || cfg->f == 0 || cfg->f % MF_GROUP_SIZE != 0 ||
+      cfg->shared_f % MF_GROUP_SIZE != 0)
+    return MF_ERR_DIMENSION_MISMATCH;
+  if (cfg->num_experts == 0 || cfg->num_experts > MF_MAX_EXPERTS) return MF_ERR_INVALID_ARGUMENT;
+  if (cfg->top_k == 0 || cfg->top_k > MF_MAX_TOPK) return MF_ERR_INVALID_ARGUMENT;
+  if (cfg->router_mode != MF_ROUTER_TOPK_SOFTMAX && cfg->router_mode != MF_ROUTER_FULL_SOFTMAX)
+    return MF_ERR_INVALID_ARGUMENT;
+  if (cfg->router_mode == MF_ROUTER_FULL_SOFTMAX && cfg->num_experts % 32 != 0)
+    return MF_ERR_INVALID_ARGUMENT;
+
+  auto* h = new (std::nothrow) mf_moe();
+  if (!h) return MF_ERR_OUT_OF_MEMORY;
+  h->ctx = ctx;
+  h->cfg = *cfg;
+  const size_t T = MF_MAX_TOKENS;
+  size_t pos = 0;
+  auto take = [&](size_t bytes) {
+    size_t at = pos;
+    pos = round_up(pos + bytes, 256);
+    return at;
+  };
+  const size_t o_logits = take(T * cfg->num_experts * sizeof(float));
+  const size_t o_idx = take(T * cfg->top_k * sizeof(uint32_t));
+  const size_t o_w = take(T * cfg->top_k * sizeof(float));
+  const size_t o_acts = take(T * cfg->top_k * cfg->f * sizeof(uint16_t));
+  const size_t o_sact = take(T * std::max<uint32_t>(cfg->shared_f, 64) * sizeof(uint16_t));
+  const size_t o_sy = take(T * cfg->d * sizeof(uint16_t));
+  const size_t o_gate = take(T * sizeof(uint16_t));
+  const size_t o_sync = take(64 * sizeof(uint32_t));
+  h->ws_bytes = pos;
+  if (hipSetDevice(ctx->device) != hipSuccess) {
+    delete h;
+    return MF_ERR_NO_DEVICE;
+  }
+  hipError_t e = hipMalloc(&h->ws_base, h->ws_bytes);
+  if (e != hipSuccess) {
+    delete h;
+    return fail_hip(ctx, e, "hipMalloc(workspace)");
+  }
+  e = hipMemset(h->ws_base, 0, h->ws_bytes);
+  if (e != hipSuccess) {
+    (void)hipFree(h->ws_base);
+    delete h;
+    return fail_hip(ctx, e, "hipMemset(workspace)");
+  }
+  auto* b = static_cast<uint8_t*>(h->ws_base);
+  h->ws.logits = reinterpret_cast<float*>(b + o_logits);
+  h->ws.idx = reinterpret_cast<uint32_t*>(b + o_idx);
+  h->ws.w = reinterpret_cast<float*>(b + o_w);
+  h->ws.acts = reinterpret_cast<uint16_t*>(b + o_acts);
+  h->ws.shared_act = reinterpret_cast<uint16_t*>(b + o_sact);
+  h->ws.shared_y = reinterpret_cast<uint16_t*>(b + o_sy);
+  h->ws.gate = reinterpret_cast<uint16_t*>(b + o_gate);
+  h->ws.sync = reinterpret_cast<uint32_t*>(b + o_sync);
+  *out = h;
+  return MF_OK;
+}
+
+void mf_moe_destroy(mf_moe* h) {
+  if (!h) return;
+  if (h->ws_base) (void)hipFree(h->ws_base);
+  delete h;
+}
+
+mf_status mf_moe_router(mf_moe* h, mf_stream stream, const uint16_t* router_w, const uint16_t* x,
+                        uint32_t t, uint32_t x_stride, uint32_t* out_idx, float* out_w,
+                        float* out_logits) {
+  if (!h || !router_w || !x || !out_idx || !out_w) return MF_ERR_INVALID_ARGUMENT;
+  if (t == 0 || x_stride < h->cfg.d) return MF_ERR_INVALID_ARGUMENT;
+  if (!mf::aligned2(router_w) || !mf::aligned2(x)) return MF_ERR_INVALID_ARGUMENT;
+  auto s = static_cast<hipStream_t>(stream);
+  const uint32_t e = h->cfg.num_experts;
+  // logits go to the caller's buffer when given, else through the handle's
+  // workspace in chunks of MF_MAX_TOKENS rows
+  for (uint32_t t0 = 0; t0 < t;) {
+    const uint32_t tc = out_logits ? t - t0 : std::min<uint32_t>(t - t0, MF_MAX_TOKENS);
+    float* lg = out_logits ? out_logits + static_cast<size_t>(t0) * e : h->ws.logits;
+    MF_HIP(h->ctx, mf::launch_router_logits(s, router_w, x + static_cast<size_t>(t0) * x_stride, e,
+                                            h->cfg.d, tc, x_stride, lg, nullptr));
+    MF_HIP(h->ctx, mf::launch_topk(s, lg, e, h->cfg.top_k, tc, h->cfg.router_mode,
+                                   out_idx + static_cast<size_t>(t0) * h->cfg.top_k,
+                                   out_w + static_cast<size_t>(t0) * h->cfg.top_k));
+    t0 += tc;
+  }
+  return MF_OK;
+}
+
+mf_status mf_moe_phase1(mf_moe* h, mf_stream stream, const void* expert_base,
+                        size_t expert_stride, const mf_expert_offsets* offsets,
+                        const uint32_t* idx, const uint16_t* x, uint32_t t, uint32_t x_stride,
+                        uint16_t* acts) {
+  if (!h || !expert_base || !offsets || !idx || !x || !acts) return MF_ERR_INVALID_ARGUMENT;
+  if (t == 0 || x_stride < h->cfg.d) return MF_ERR_INVALID_ARGUMENT;
+  if (!offsets_ok(*offsets, h->cfg.bits) || !mf::aligned2(expert_base) || (expert_stride & 1) ||
+      !mf::aligned2(x) || !mf::aligned2(acts))
+    return MF_ERR_INVALID_ARGUMENT;
+  MF_HIP(h->ctx, mf::launch_phase1(static_cast<hipStream_t>(stream), h->cfg, expert_base,
+                                   expert_stride, *offsets, idx, x, t, x_stride, acts));
+  return MF_OK;
+}
+
+mf_status mf_moe_phase2(mf_moe* h, mf_stream stream, const void* expert_base,
+                        size_t expert_stride, const mf_expert_offsets* offsets,
+                        const uint32_t* idx, const float* w, const uint16_t* acts,
+                        const uint16_t* residual, uint32_t t, uint16_t* y) {
+  if (!h || !expert_base || !offsets || !idx || !w || !acts || !y) return MF_ERR_INVALID_ARGUMENT;
+  if (t == 0) return MF_ERR_INVALID_ARGUMENT;
+  if (!offsets_ok(*offsets, h->cfg.bits) || !mf::aligned2(expert_base) || (expert_stride & 1) ||
+      !mf::aligned2(acts) || !mf::aligned2(y) || (residual && !mf::aligned2(residual)))
+    return MF_ERR_INVALID_ARGUMENT;
+  MF_HIP(h->ctx, mf::launch_phase2(static_cast<hipStream_t>(stream), h->cfg, expert_base,
+                                   expert_stride, *offsets, idx, w, acts, residual, t, y));
+  return MF_OK;
+}
+
+mf_status mf_moe_decode_layer(mf_moe* h, mf_stream stream, const mf_moe_layer_weights* wts,
+                              const uint16_t* x, uint32_t t, uint16_t* y, uint16_t* hidden,
+                              uint32_t* out_idx, float* out_w) {
+  if (!h || !wts || !x || !y) return MF_ERR_INVALID_ARGUMENT;
+  if (t == 0 || t > MF_MAX_TOKENS) return MF_ERR_INVALID_ARGUMENT;
+  const mf_moe_config& c = h->cfg;
+  if (!wts->router_w || !wts->expert_base || !offsets_ok(wts->offsets, c.bits) ||
+      !mf::aligned2(wts->expert_base) || (wts->expert_stride & 1) || !mf::aligned2(x) ||
+      !mf::aligned2(y) || (hidden && !mf::aligned2(hidden)))
+    return MF_ERR_INVALID_ARGUMENT;
+  if (c.shared_f && (!qtensor_ok(wts->shared_gate, c.shared_bits) ||
+                     !qtensor_ok(wts->shared_up, c.shared_bits) ||
+                     !qtensor_ok(wts->shared_down, c.shared_bits)))
+    return MF_ERR_INVALID_ARGUMENT;
+  auto s = static_cast<hipStream_t>(stream);
+  uint32_t* idx = h->ws.idx;
+  float* w = h->ws.w;
+  MF_HIP(h->ctx, mf::launch_router_logits(s, wts->router_w, x, c.num_experts, c.d, t, c.d,
+                                          h->ws.logits, nullptr));
+  MF_HIP(h->ctx, mf::launch_topk(s, h->ws.logits, c.num_experts, c.top_k, t, c.router_mode, idx, w));
+  const uint16_t* residual = nullptr;
+  if (c.shared_f) {
+    MF_HIP(h->ctx, mf::launch_gate_up_act(s, wts->shared_gate, wts->shared_up, c.shared_bits, x,
+                                          h->ws.shared_act, c.shared_f, c.d, t));
+    MF_HIP(h->ctx, mf::launch_gemv(s, wts->shared_down, c.shared_bits, h->ws.shared_act,
+                                   h->ws.shared_y, c.d, c.shared_f, t, false));
+    if (wts->w_sg) {
+      MF_HIP(h->ctx, mf::launch_router_logits(s, wts->w_sg, x, 1, c.d, t, c.d, nullptr, h->ws.gate));
+      MF_HIP(h->ctx, mf::launch_sigmoid_scalar_mul(s, h->ws.shared_y, h->ws.gate, c.d, t));
+    }
+    residual = h->ws.shared_y;
+  }
+  MF_HIP(h->ctx, mf::launch_phase1(s, c, wts->expert_base, wts->expert_stride, wts->offsets, idx, x,
+                                   t, c.d, h->ws.acts));
+  MF_HIP(h->ctx, mf::launch_phase2(s, c, wts->expert_base, wts->expert_stride, wts->offsets, idx, w,
+                                   h->ws.acts, residual, t, y));
+  if (hidden) MF_HIP(h->ctx, mf::launch_residual_add(s, hidden, y, t * c.d));
+  if (out_idx)
+    MF_HIP(h->ctx, hipMemcpyAsync(out_idx, idx, sizeof(uint32_t) * t * c.top_k,
+                                  hipMemcpyDeviceToDevice, s));
+  if (out_w)
+    MF_HIP(h->ctx, hipMemcpyAsync(out_w, w, sizeof(float) * t * c.top_k, hipMemcpyDeviceToDevice, s));
+  return MF_OK;
+}
+
+/* ------------------------------------------------------- ragged prefill */
+
+mf_status mf_group_pairs_host(const mf_pair* pairs, size_t n_pairs, int query_count, int top_k,
+                              int num_experts, int tile_expert_count,
+                              const uint64_t* sort_keys, size_t n_sort_keys, mf_pair* sorted,
+                              uint32_t* offsets, uint32_t* counts, mf_group* groups,
+                              size_t* n_groups, mf_tile* tiles, size_t* n_tiles,
+                              uint32_t err_detail[2]) {
+  uint32_t dummy[2];
+  uint32_t* det = err_detail ? err_detail : dummy;
+  det[0] = det[1] = 0;
+  // validation order of PrefillMoEGrouping.swift:99-141
+  if (query_count < 0) return MF_ERR_QUERY_COUNT;
+  if (top_k <= 0) return MF_ERR_TOPK;
+  if (num_experts <= 0) return MF_ERR_NUM_EXPERTS;
+  if (tile_expert_count < 1 || tile_expert_count > 16) return MF_ERR_TILE_EXPERT_COUNT;
+  if (sort_keys && n_sort_keys != static_cast<size_t>(num_experts)) {
+    det[0] = static_cast<uint32_t>(num_experts);
+    det[1] = static_cast<uint32_t>(n_sort_keys);
+    return MF_ERR_SORT_KEY_COUNT;
+  }
+  const size_t expected = static_cast<size_t>(query_count) * static_cast<size_t>(top_k);
+  if (n_pairs != expected) {
+    det[0] = static_cast<uint32_t>(expected);
+    det[1] = static_cast<uint32_t>(n_pairs);
+    return MF_ERR_PAIR_COUNT;
+  }
+  if (n_pairs && (!pairs || !sorted)) return MF_ERR_INVALID_ARGUMENT;
+  if (!offsets || !counts || !groups || !tiles || !n_groups || !n_tiles)
+    return MF_ERR_INVALID_ARGUMENT;
+
+  std::vector<uint8_t> seen(n_pairs, 0);
+  for (size_t i = 0; i < n_pairs; ++i) {
+    const mf_pair& p = pairs[i];
+    if (p.token >= static_cast<uint32_t>(query_count)) { det[0] = p.token; return MF_ERR_TOKEN_RANGE; }
+    if (p.rank >= static_cast<uint32_t>(top_k)) { det[0] = p.rank; return MF_ERR_RANK_RANGE; }
+    if (p.expert >= static_cast<uint32_t>(num_experts)) { det[0] = p.expert; return MF_ERR_EXPERT_RANGE; }
+    const size_t key = static_cast<size_t>(p.token) * top_k + p.rank;
+    if (seen[key]) { det[0] = p.token; det[1] = p.rank; return MF_ERR_DUPLICATE_TOKEN_RANK; }
+    seen[key] = 1;
+  }
+
+  std::copy(pairs, pairs + n_pairs, sorted);
+  std::sort(sorted, sorted + n_pairs, [&](const mf_pair& a, const mf_pair& b) {
+    if (sort_keys) {
+      const uint64_t ka = sort_keys[a.expert], kb = sort_keys[b.expert];
+      if (ka != kb) return ka < kb;
+    }
+    if (a.expert != b.expert) return a.expert < b.expert;
+    if (a.token != b.token) return a.token < b.token;
+    return a.rank < b.rank;
+  });
+  std::fill(offsets, offsets + num_experts, 0xFFFFFFFFu);
+  std::fill(counts, counts + num_experts, 0u);
+  size_t ng = 0;
+  for (size_t i = 0; i < n_pairs;) {
+    const uint32_t expert = sorted[i].expert;
+    const size_t start = i;
+    while (i < n_pairs && sorted[i].expert == expert) ++i;
+    offsets[expert] = static_cast<uint32_t>(start);
+    counts[expert] = static_cast<uint32_t>(i - start);
+    groups[ng++] = mf_group{expert, static_cast<uint32_t>(start), static_cast<uint32_t>(i - start)};
+  }
+  size_t nt = 0;
+  for (size_t gs = 0; gs < ng;) {
+    const size_t ge = std::min(ng, gs + static_cast<size_t>(tile_expert_count));
+    const mf_group& first = groups[gs];
+    const mf_group& last = groups[ge - 1];
+    tiles[nt++] = mf_tile{static_cast<uint32_t>(gs), static_cast<uint32_t>(ge - gs), first.pair_start,
+                          last.pair_start + last.pair_count - first.pair_start};
+    gs = ge;
+  }
+  *n_groups = ng;
+  *n_tiles = nt;
+  return MF_OK;
+}
+
+}  // extern "C"

@@ -1,0 +1,84 @@
+// Host-side state and kernel launchers behind the C ABI (include/mfmoe.h).
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stddef.h>
+#include <stdint.h>
+
+#include "../../include/mfmoe.h"
+
+struct mf_ctx {
+  int device = 0;
+  int num_cu = 0;
+  char hip_error[256] = {0};
+};
+
+// Per-operator device workspace (the routerLogits buffer and argument table the
+// reference's MoE class owns, MoE.swift:136-150).
+struct mf_moe_workspace {
+  float* logits;        // [MF_MAX_TOKENS, num_experts]
+  uint32_t* idx;        // [MF_MAX_TOKENS, top_k]
+  float* w;             // [MF_MAX_TOKENS, top_k]
+  uint16_t* acts;       // [MF_MAX_TOKENS, top_k, f]
+  uint16_t* shared_act; // [MF_MAX_TOKENS, shared_f]
+  uint16_t* shared_y;   // [MF_MAX_TOKENS, d]
+  uint16_t* gate;       // [MF_MAX_TOKENS]
+  uint32_t* sync;       // grid-sync counters of the fused kernel
+};
+
+struct mf_moe {
+  mf_ctx* ctx = nullptr;
+  mf_moe_config cfg{};
+  void* ws_base = nullptr;
+  size_t ws_bytes = 0;
+  mf_moe_workspace ws{};
+};
+
+namespace mf {
+
+inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+inline bool aligned2(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 1u) == 0; }
+
+// lanes of a wave that share one row of n elements (power of two, <= 64)
+inline uint32_t lanes_per_row_log2(uint32_t n, int elems_per_lane) {
+  uint32_t need = (n + elems_per_lane - 1) / elems_per_lane;
+  uint32_t l = 0;
+  while ((1u << l) < need && l < 6) ++l;
+  return l;
+}
+
+// format.hip
+hipError_t launch_quantize(hipStream_t s, const float* w, size_t rows, size_t n, int bits,
+                           void* packed, uint16_t* scales, uint16_t* biases);
+hipError_t launch_dequantize(hipStream_t s, const mf_qtensor& q, size_t rows, size_t n, int bits,
+                             float* out);
+
+// gemv.hip
+hipError_t launch_gemv(hipStream_t s, const mf_qtensor& w, int bits, const uint16_t* x, void* y,
+                       uint32_t m, uint32_t n, uint32_t t, bool out_f32);
+hipError_t launch_gate_up_act(hipStream_t s, const mf_qtensor& gate, const mf_qtensor& up,
+                              int bits, const uint16_t* x, uint16_t* act, uint32_t f, uint32_t d,
+                              uint32_t t);
+hipError_t launch_silu_mul(hipStream_t s, const uint16_t* gate, const uint16_t* up, uint16_t* out,
+                           uint32_t count);
+hipError_t launch_sigmoid_scalar_mul(hipStream_t s, uint16_t* y, const uint16_t* gate,
+                                     uint32_t row, uint32_t rows);
+hipError_t launch_residual_add(hipStream_t s, uint16_t* hidden, const uint16_t* delta,
+                               uint32_t count);
+
+// router.hip
+hipError_t launch_router_logits(hipStream_t s, const uint16_t* w, const uint16_t* x, uint32_t e,
+                                uint32_t d, uint32_t t, uint32_t x_stride, float* logits,
+                                uint16_t* logits_bf16);
+hipError_t launch_topk(hipStream_t s, const float* logits, uint32_t e, uint32_t k, uint32_t t,
+                       int mode, uint32_t* idx, float* w);
+
+// moe_decode.hip
+hipError_t launch_phase1(hipStream_t s, const mf_moe_config& cfg, const void* base, size_t stride,
+                         const mf_expert_offsets& off, const uint32_t* idx, const uint16_t* x,
+                         uint32_t t, uint32_t x_stride, uint16_t* acts);
+hipError_t launch_phase2(hipStream_t s, const mf_moe_config& cfg, const void* base, size_t stride,
+                         const mf_expert_offsets& off, const uint32_t* idx, const float* w,
+                         const uint16_t* acts, const uint16_t* residual, uint32_t t, uint16_t* y);
+
+}  // namespace mf

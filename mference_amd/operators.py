@@ -1,0 +1,358 @@
+"""Host-side mirror of Mference's Swift operator surface over the C ABI.
+
+Class and method names follow Sources/Mference/Kernels/** (Swift camelCase
+turned into snake_case); a command buffer becomes a HIP stream, an
+(MTLBuffer, offset) pair becomes a torch tensor (device memory only: torch is
+the allocator and stream provider, every computation is libmfmoe's).
+Argument errors raise MfError carrying the mf_status the C ABI returned.
+"""
+from __future__ import annotations
+
+import ctypes as C
+from dataclasses import dataclass
+from typing import Optional, Sequence
+
+import numpy as np
+import torch
+
+from . import _capi
+from ._capi import (BITS_2, BITS_4, BITS_TERNARY, GROUP_SIZE, MAX_TOKENS, ROUTER_FULL_SOFTMAX,
+                    ROUTER_TOPK_SOFTMAX, ExpertOffsets, MfError, check)
+
+__all__ = [
+    "MetalContext", "QuantizedTensor", "Quantization", "DequantInt4GEMV", "DequantInt4GEMVMultiX",
+    "Elementwise", "SharedExpertInt4", "MoEExpertOffsets", "MoE", "MoELayerWeights",
+    "PrefillMoEGrouping", "PrefillTokenExpertPair", "MfError", "BITS_2", "BITS_4", "BITS_TERNARY",
+    "ROUTER_TOPK_SOFTMAX", "ROUTER_FULL_SOFTMAX", "bf16_tensor", "bf16_bits",
+]
+
+MoEExpertOffsets = ExpertOffsets
+
+
+def _ptr(t: Optional[torch.Tensor]) -> Optional[int]:
+    if t is None:
+        return None
+    if not t.is_cuda:
+        raise ValueError("libmfmoe operates on device memory; got a CPU tensor")
+    return t.data_ptr()
+
+
+def _stream(stream) -> int:
+    if stream is None:
+        return torch.cuda.current_stream().cuda_stream
+    if isinstance(stream, torch.cuda.Stream):
+        return stream.cuda_stream
+    return int(stream)
+
+
+def bf16_tensor(bits: np.ndarray, device="cuda") -> torch.Tensor:
+    """uint16 bf16 bit patterns (host) -> torch.bfloat16 tensor on `device`."""
+    a = np.ascontiguousarray(bits, dtype=np.uint16)
+    return torch.from_numpy(a.view(np.int16)).to(device).view(torch.bfloat16)
+
+
+def bf16_bits(t: torch.Tensor) -> np.ndarray:
+    """torch.bfloat16 tensor -> uint16 bit patterns on the host."""
+    return t.detach().contiguous().view(torch.int16).cpu().numpy().view(np.uint16)
+
+
+class MetalContext:
+    """Device + kernel state every operator is built from
+    (Infrastructure/Metal/MetalContext.swift:45-65)."""
+
+    def __init__(self, device: int = 0):
+        self._h = C.c_void_p()
+        check(_capi.lib().mf_ctx_create(device, C.byref(self._h)))
+        self.device = torch.device("cuda", device)
+
+    @property
+    def handle(self):
+        return self._h
+
+    def close(self):
+        if self._h:
+            _capi.lib().mf_ctx_destroy(self._h)
+            self._h = C.c_void_p()
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
+
+
+@dataclass
+class QuantizedTensor:
+    """rows x n group-quantized tensor in device memory
+    (Quantization.Int4AffineRow for every row, Quantization.swift:34-46)."""
+    packed: torch.Tensor            # uint8 [rows, n*bits/8]
+    scales: torch.Tensor            # bf16 [rows, n/64]
+    biases: Optional[torch.Tensor]  # bf16 [rows, n/64]; None for ternary
+    bits: int
+    rows: int
+    n: int
+
+    def c(self) -> _capi.QTensor:
+        return _capi.QTensor(_ptr(self.packed), _ptr(self.scales), _ptr(self.biases))
+
+    @classmethod
+    def from_host(cls, packed: np.ndarray, scales: np.ndarray, biases: Optional[np.ndarray],
+                  bits: int, rows: int, n: int, device="cuda") -> "QuantizedTensor":
+        return cls(torch.from_numpy(np.ascontiguousarray(packed)).to(device),
+                   bf16_tensor(scales, device),
+                   None if biases is None else bf16_tensor(biases, device), bits, rows, n)
+
+
+class Quantization:
+    """Infrastructure/ModelIO/Quantization.swift:3 on device."""
+    group_size = GROUP_SIZE
+
+    def __init__(self, context: MetalContext):
+        self.context = context
+
+    def quantize_affine(self, w: torch.Tensor, bits: int = BITS_4, stream=None) -> QuantizedTensor:
+        """quantizeInt4Affine (Quantization.swift:50-102) for every row of w (fp32)."""
+        if w.dtype != torch.float32 or w.dim() != 2:
+            raise ValueError("w must be a 2-D float32 tensor")
+        w = w.contiguous()
+        rows, n = w.shape
+        store = 4 if bits == BITS_4 else 2
+        packed = torch.empty((rows, n * store // 8), dtype=torch.uint8, device=w.device)
+        scales = torch.empty((rows, n // GROUP_SIZE), dtype=torch.bfloat16, device=w.device)
+        biases = torch.empty_like(scales)
+        check(_capi.lib().mf_quantize_affine(self.context.handle, _stream(stream), _ptr(w), rows, n,
+                                             bits, _ptr(packed), _ptr(scales), _ptr(biases)),
+              self.context.handle)
+        return QuantizedTensor(packed, scales, biases, bits, rows, n)
+
+    def dequantize(self, q: QuantizedTensor, stream=None) -> torch.Tensor:
+        """dequantizeInt4Affine (Quantization.swift:104-119): fp32 [rows, n]."""
+        out = torch.empty((q.rows, q.n), dtype=torch.float32, device=q.packed.device)
+        check(_capi.lib().mf_dequantize(self.context.handle, _stream(stream), q.c(), q.rows, q.n,
+                                        q.bits, _ptr(out)), self.context.handle)
+        return out
+
+
+class DequantInt4GEMV:
+    """Kernels/Quant/DequantInt4GEMV.swift:57-103 (any supported bit width)."""
+
+    def __init__(self, context: MetalContext):
+        self.context = context
+
+    def encode(self, weights: QuantizedTensor, x: torch.Tensor, y: torch.Tensor, m: int, n: int,
+               output_float32: bool = False, stream=None, t: int = 1) -> None:
+        check(_capi.lib().mf_gemv(self.context.handle, _stream(stream), weights.c(), weights.bits,
+                                  _ptr(x), _ptr(y), m, n, t, 1 if output_float32 else 0),
+              self.context.handle)
+
+
+class DequantInt4GEMVMultiX(DequantInt4GEMV):
+    """Kernels/Quant/DequantInt4GEMVMultiX.swift:48-82: x [t, n], y [t, m], t <= 8."""
+    max_tokens = MAX_TOKENS
+
+    def encode(self, weights: QuantizedTensor, x: torch.Tensor, y: torch.Tensor, m: int, n: int,
+               t: int, output_float32: bool = False, stream=None) -> None:
+        super().encode(weights, x, y, m, n, output_float32, stream, t)
+
+
+class Elementwise:
+    """Kernels/Primitives/Elementwise.swift:60-87."""
+
+    def __init__(self, context: MetalContext):
+        self.context = context
+
+    def encode_silu_mul(self, gate, up, out, count: int, stream=None):
+        check(_capi.lib().mf_silu_mul(self.context.handle, _stream(stream), _ptr(gate), _ptr(up),
+                                      _ptr(out), count), self.context.handle)
+
+    def encode_sigmoid_scalar_mul(self, y, gate, count: int, rows: int = 1, stream=None):
+        check(_capi.lib().mf_sigmoid_scalar_mul(self.context.handle, _stream(stream), _ptr(y),
+                                                _ptr(gate), count, rows), self.context.handle)
+
+    def encode_residual_add(self, hidden, delta, count: int, stream=None):
+        check(_capi.lib().mf_residual_add(self.context.handle, _stream(stream), _ptr(hidden),
+                                          _ptr(delta), count), self.context.handle)
+
+
+class SharedExpertInt4:
+    """Kernels/MoE/SharedExpertInt4.swift:70-165 (also the dense SwiGLU MLP)."""
+
+    def __init__(self, context: MetalContext):
+        self.context = context
+
+    def encode(self, x: torch.Tensor, gate: QuantizedTensor, up: QuantizedTensor,
+               down: QuantizedTensor, y: torch.Tensor, scratch_act: torch.Tensor, t: int = 1,
+               stream=None) -> None:
+        if not (gate.rows == up.rows and gate.n == up.n and down.rows == gate.n
+                and down.n == gate.rows):
+            raise MfError(-2, f"gate=({gate.rows},{gate.n}) up=({up.rows},{up.n}) "
+                              f"down=({down.rows},{down.n})")
+        check(_capi.lib().mf_shared_expert(
+            self.context.handle, _stream(stream), _ptr(x), gate.c(), up.c(), down.c(), gate.bits,
+            gate.n, gate.rows, t, _ptr(y), _ptr(scratch_act),
+            scratch_act.numel() * scratch_act.element_size()), self.context.handle)
+
+
+@dataclass
+class MoELayerWeights:
+    """Everything one MoE layer reads, resident in device memory."""
+    router_w: torch.Tensor                 # bf16 [e, d]
+    experts: torch.Tensor                  # uint8 [e, stride]
+    offsets: ExpertOffsets
+    shared: Optional[Sequence[QuantizedTensor]] = None  # gate, up, down
+    w_sg: Optional[torch.Tensor] = None    # bf16 [d]
+
+    def c(self) -> _capi.LayerWeights:
+        L = _capi.LayerWeights()
+        L.router_w = _ptr(self.router_w)
+        L.expert_base = _ptr(self.experts)
+        L.expert_stride = self.experts.stride(0)
+        L.offsets = self.offsets
+        if self.shared is not None:
+            L.shared_gate, L.shared_up, L.shared_down = (q.c() for q in self.shared)
+        L.w_sg = _ptr(self.w_sg)
+        return L
+
+
+class MoE:
+    """Router + routed experts operator: MoE (Kernels/MoE/MoE.swift),
+    MoEDeepseekV4 (2-bit, top-6) and MapleMoE (ternary) in one class, selected
+    by `bits`, `top_k` and `router_mode`."""
+
+    def __init__(self, context: MetalContext, d: int, f: int, num_experts: int, top_k: int,
+                 bits: int = BITS_4, router_mode: int = ROUTER_TOPK_SOFTMAX,
+                 swiglu_limit: float = 0.0, shared_f: int = 0, shared_bits: int = BITS_4):
+        self.context = context
+        self.cfg = _capi.MoEConfig(d, f, num_experts, top_k, bits, router_mode, swiglu_limit,
+                                   shared_f, shared_bits)
+        self._h = C.c_void_p()
+        check(_capi.lib().mf_moe_create(context.handle, C.byref(self.cfg), C.byref(self._h)),
+              context.handle)
+
+    def close(self):
+        if self._h:
+            _capi.lib().mf_moe_destroy(self._h)
+            self._h = C.c_void_p()
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
+
+    def encode_router(self, router_w, x, out_indices, out_weights, t: int = 1,
+                      x_stride: Optional[int] = None, out_logits=None, stream=None):
+        """encodeRouterGemma4 (MoE.swift:153-203) / encodeRouterTopK / encodeRouterTop8."""
+        check(_capi.lib().mf_moe_router(self._h, _stream(stream), _ptr(router_w), _ptr(x), t,
+                                        self.cfg.d if x_stride is None else x_stride,
+                                        _ptr(out_indices), _ptr(out_weights), _ptr(out_logits)),
+              self.context.handle)
+
+    def encode_routed_phase1(self, experts: torch.Tensor, offsets: ExpertOffsets, indices, x, acts,
+                             t: int = 1, x_stride: Optional[int] = None, stream=None):
+        """encodeRoutedPersistentPhase1U16Load (MoE.swift:220-253)."""
+        check(_capi.lib().mf_moe_phase1(self._h, _stream(stream), _ptr(experts), experts.stride(0),
+                                        C.byref(offsets), _ptr(indices), _ptr(x), t,
+                                        self.cfg.d if x_stride is None else x_stride, _ptr(acts)),
+              self.context.handle)
+
+    def encode_routed_phase2_reduce(self, experts: torch.Tensor, offsets: ExpertOffsets, indices,
+                                    routing_weights, acts, residual, y, t: int = 1, stream=None):
+        """encodeRoutedPersistentPhase2Reduce (MoE.swift:400-440)."""
+        check(_capi.lib().mf_moe_phase2(self._h, _stream(stream), _ptr(experts), experts.stride(0),
+                                        C.byref(offsets), _ptr(indices), _ptr(routing_weights),
+                                        _ptr(acts), _ptr(residual), t, _ptr(y)),
+              self.context.handle)
+
+    def encode_decode_layer(self, weights: MoELayerWeights, x, y, t: int = 1, hidden=None,
+                            out_indices=None, out_weights=None, stream=None):
+        """The fused decode layer (router -> experts -> shared add), one call."""
+        lw = weights.c()
+        check(_capi.lib().mf_moe_decode_layer(self._h, _stream(stream), C.byref(lw), _ptr(x), t,
+                                              _ptr(y), _ptr(hidden), _ptr(out_indices),
+                                              _ptr(out_weights)), self.context.handle)
+
+
+PAIR_DTYPE = np.dtype([("token", "<u4"), ("expert", "<u4"), ("rank", "<u4"),
+                       ("weight_bits", "<u4")])
+GROUP_DTYPE = np.dtype([("expert", "<u4"), ("pair_start", "<u4"), ("pair_count", "<u4")])
+TILE_DTYPE = np.dtype([("group_start", "<u4"), ("group_count", "<u4"), ("pair_start", "<u4"),
+                       ("pair_count", "<u4")])
+
+
+def PrefillTokenExpertPair(token: int, expert: int, rank: int, weight_bits: int):
+    """One route record (Kernels/Prefill/MoE/PrefillRouter.swift:4-28)."""
+    return (token, expert, rank, weight_bits)
+
+
+@dataclass
+class PrefillMoEGroupedRoutes:
+    """Kernels/Prefill/MoE/PrefillMoEGrouping.swift:32-50."""
+    sorted_pairs: np.ndarray
+    per_expert_offsets: np.ndarray
+    per_expert_counts: np.ndarray
+    groups: np.ndarray
+    tiles: np.ndarray
+    query_count: int
+
+    @property
+    def max_pairs_per_expert(self) -> int:
+        return int(self.groups["pair_count"].max()) if self.groups.size else 0
+
+    @property
+    def max_pairs_per_tile(self) -> int:
+        return int(self.tiles["pair_count"].max()) if self.tiles.size else 0
+
+    @property
+    def max_live_experts_per_tile(self) -> int:
+        return int(self.tiles["group_count"].max()) if self.tiles.size else 0
+
+
+class PrefillMoEGrouping:
+    """Kernels/Prefill/MoE/PrefillMoEGrouping.swift:90-192 (host, integer)."""
+
+    @staticmethod
+    def make_token_expert_pairs(indices: np.ndarray, weight_bits: np.ndarray, query_count: int,
+                                top_k: int) -> np.ndarray:
+        """PrefillRouter.makeTokenExpertPairs (PrefillRouter.swift:91-111)."""
+        indices = np.asarray(indices, np.uint32).reshape(-1)
+        weight_bits = np.asarray(weight_bits, np.uint32).reshape(-1)
+        if indices.size != query_count * top_k or weight_bits.size != query_count * top_k:
+            raise ValueError("indices / weights count mismatch")
+        out = np.empty(query_count * top_k, PAIR_DTYPE)
+        out["token"] = np.repeat(np.arange(query_count, dtype=np.uint32), top_k)
+        out["rank"] = np.tile(np.arange(top_k, dtype=np.uint32), query_count)
+        out["expert"] = indices
+        out["weight_bits"] = weight_bits
+        return out
+
+    @staticmethod
+    def group_token_expert_pairs(pairs, query_count: int, top_k: int, num_experts: int,
+                                 tile_expert_count: int = 16,
+                                 expert_sort_keys=None) -> PrefillMoEGroupedRoutes:
+        if isinstance(pairs, np.ndarray) and pairs.dtype == PAIR_DTYPE:
+            p = np.ascontiguousarray(pairs)
+        else:
+            p = np.array([tuple(x) for x in pairs], dtype=PAIR_DTYPE)
+        n = p.size
+        sorted_ = np.empty(n, PAIR_DTYPE)
+        ne = max(num_experts, 1)
+        offsets = np.empty(ne, np.uint32)
+        counts = np.empty(ne, np.uint32)
+        cap = max(min(ne, n), 1)
+        groups = np.empty(cap, GROUP_DTYPE)
+        tiles = np.empty(cap, TILE_DTYPE)
+        ng, nt = C.c_size_t(0), C.c_size_t(0)
+        keys = None if expert_sort_keys is None else np.ascontiguousarray(expert_sort_keys, np.uint64)
+        detail = (C.c_uint32 * 2)()
+        vp = lambda a: None if a is None else a.ctypes.data_as(C.c_void_p)
+        rc = _capi.lib().mf_group_pairs_host(
+            vp(p), n, query_count, top_k, num_experts, tile_expert_count, vp(keys),
+            0 if keys is None else keys.size, vp(sorted_), vp(offsets), vp(counts), vp(groups),
+            C.byref(ng), vp(tiles), C.byref(nt), C.cast(detail, C.c_void_p))
+        if rc != 0:
+            err = MfError(rc, f"detail={detail[0]},{detail[1]}")
+            err.detail = (int(detail[0]), int(detail[1]))
+            raise err
+        return PrefillMoEGroupedRoutes(sorted_, offsets[:num_experts], counts[:num_experts],
+                                       groups[:ng.value], tiles[:nt.value], query_count)

@@ -1,0 +1,222 @@
+"""GPU parity of the decode path against the CPU oracle, through the C ABI."""
+import numpy as np
+import pytest
+import torch
+
+from mference_amd import operators as ops
+from helpers import ROOT_SEED, assert_layer_close, errors, make_moe, to_device_layer, to_device_q
+
+pytestmark = pytest.mark.gpu
+
+
+def _sync():
+    torch.cuda.synchronize()
+
+
+@pytest.mark.parametrize("bits", [4, 2])
+@pytest.mark.parametrize("rows,n", [(7, 64), (16, 256), (33, 2048), (5, 4096)])
+def test_quantize_bit_exact(gpu, oracle, bits, rows, n):
+    rng = oracle.Rng.key(0x51A71001, f"quant-{bits}-{rows}-{n}")
+    w = rng.uniform_fill(-1.0, 1.0, rows * n).reshape(rows, n)
+    w[0, :64] = 0.42                      # constant group
+    if rows > 1:
+        w[1, :64] = np.arange(64) * 1e-30  # denormal-scale group
+    ref = oracle.quantize(w, bits)
+    q = ops.Quantization(gpu).quantize_affine(torch.from_numpy(w).cuda(), bits)
+    _sync()
+    assert np.array_equal(q.packed.cpu().numpy(), ref.packed)
+    assert np.array_equal(ops.bf16_bits(q.scales), ref.scales)
+    assert np.array_equal(ops.bf16_bits(q.biases), ref.biases)
+
+
+@pytest.mark.parametrize("bits", [4, 2, 1])
+def test_dequantize_bit_exact(gpu, oracle, bits):
+    rows, n = 9, 512
+    rng = oracle.Rng.key(0xF5, f"dequant-{bits}")
+    if bits == 1:
+        codes = (np.array([rng.next() % 3 for _ in range(rows * n)], np.uint8)).reshape(rows, n)
+        q = oracle.QTensor(oracle.pack_codes(codes, 1),
+                           oracle.bf16_bits(rng.uniform_fill(0.01, 0.2, rows * n // 64).reshape(rows, -1)),
+                           None, 1, rows, n)
+    else:
+        q = oracle.quantize(rng.uniform_fill(-2.0, 2.0, rows * n).reshape(rows, n), bits)
+        # adversarial scale/bias pairs: denormal bf16, negative scale, large bias
+        q.scales[0, 0], q.biases[0, 0] = 0x0001, 0x8001
+        q.scales[1, 1], q.biases[1, 1] = 0xBF80, 0x4700
+    ref = oracle.dequantize(q)
+    out = ops.Quantization(gpu).dequantize(to_device_q(q))
+    _sync()
+    assert np.array_equal(out.cpu().numpy().view(np.uint32), ref.view(np.uint32))
+
+
+@pytest.mark.parametrize("bits", [4, 2, 1])
+@pytest.mark.parametrize("m,n,t", [(64, 64, 1), (65, 128, 2), (129, 512, 1), (40, 2048, 4),
+                                   (24, 4096, 7), (17, 192, 3), (8, 5120, 8)])
+def test_gemv_matches_oracle(gpu, oracle, bits, m, n, t):
+    rng = oracle.Rng.key(0xF1, f"gemv-{bits}-{m}-{n}-{t}")
+    if bits == 1:
+        u = rng.uniform_fill(0, 1, m * n).reshape(m, n)
+        codes = np.where(u < 0.25, 0, np.where(u < 0.75, 1, 2)).astype(np.uint8)
+        q = oracle.QTensor(oracle.pack_codes(codes, 1),
+                           oracle.bf16_bits(rng.uniform_fill(0.01, 0.05, m * n // 64).reshape(m, -1)),
+                           None, 1, m, n)
+    else:
+        q = oracle.quantize(rng.uniform_fill(-1.0, 1.0, m * n).reshape(m, n), bits)
+    x = oracle.bf16_bits(rng.uniform_fill(-1.0, 1.0, t * n).reshape(t, n))
+    ref = oracle.gemv_multix(q, x)
+    xd = ops.bf16_tensor(x)
+    y32 = torch.full((t, m), 7.0, dtype=torch.float32, device="cuda")
+    y16 = torch.zeros((t, m), dtype=torch.bfloat16, device="cuda")
+    g = ops.DequantInt4GEMVMultiX(gpu)
+    dq = to_device_q(q)
+    g.encode(dq, xd, y32, m, n, t, output_float32=True)
+    g.encode(dq, xd, y16, m, n, t)
+    _sync()
+    got = y32.cpu().numpy()
+    scale = max(np.abs(ref).max(), 1e-6)
+    assert np.abs(got - ref).max() / scale < 2e-5
+    assert np.array_equal(ops.bf16_bits(y16), oracle.bf16_bits(got))
+    # multi-token rows are bit-identical to single-token calls
+    # (MultiXKernelParityTests.swift:50-77)
+    for i in range(t):
+        yi = torch.zeros((1, m), dtype=torch.float32, device="cuda")
+        g.encode(dq, xd[i:i + 1].contiguous(), yi, m, n, 1, output_float32=True)
+        _sync()
+        assert np.array_equal(yi.cpu().numpy()[0].view(np.uint32), got[i].view(np.uint32))
+
+
+def test_gemv_misaligned_pointers(gpu, oracle):
+    m, n = 9, 256
+    rng = oracle.Rng.key(0xF2, "gemv-misaligned")
+    q = oracle.quantize(rng.uniform_fill(-1.0, 1.0, m * n).reshape(m, n), 4)
+    x = oracle.bf16_bits(rng.uniform_fill(-1.0, 1.0, n))
+    ref = oracle.gemv_multix(q, x.reshape(1, n))
+    # weights at a 1-byte offset, x at a 2-byte offset, sentinel-padded output
+    wbuf = torch.full((q.packed.size + 7,), 0xA5, dtype=torch.uint8, device="cuda")
+    wbuf[1:1 + q.packed.size] = torch.from_numpy(q.packed.reshape(-1)).cuda()
+    xbuf = torch.zeros(n + 8, dtype=torch.bfloat16, device="cuda")
+    xbuf[1:1 + n] = ops.bf16_tensor(x)
+    dq = to_device_q(q)
+    dq.packed = wbuf[1:1 + q.packed.size]
+    ybuf = torch.full((m + 8,), 123.0, dtype=torch.float32, device="cuda")
+    ops.DequantInt4GEMV(gpu).encode(dq, xbuf[1:1 + n], ybuf[4:4 + m], m, n, output_float32=True)
+    _sync()
+    y = ybuf.cpu().numpy()
+    assert np.all(y[:4] == 123.0) and np.all(y[4 + m:] == 123.0)
+    assert np.abs(y[4:4 + m] - ref[0]).max() / np.abs(ref).max() < 2e-5
+
+
+@pytest.mark.parametrize("e,d,k,t", [(256, 2048, 8, 1), (16, 128, 8, 3), (64, 2048, 8, 5),
+                                     (256, 4096, 6, 2), (100, 192, 4, 9), (8, 64, 8, 1)])
+@pytest.mark.parametrize("mode", [0, 1])
+def test_router_bit_exact(gpu, oracle, e, d, k, t, mode):
+    if mode == 1 and e % 32:
+        pytest.skip("full-softmax mode needs num_experts % 32 == 0")
+    rng = oracle.Rng.key(0xA5B61234, f"router-{e}-{d}-{k}-{t}")
+    wr = oracle.bf16_bits(rng.normal(0.0, 0.02, e * d).reshape(e, d))
+    x = oracle.bf16_bits(rng.normal(0.0, 1.0, t * d).reshape(t, d))
+    moe = ops.MoE(gpu, d, 64, e, k, router_mode=mode)
+    idx = torch.zeros((t, k), dtype=torch.int32, device="cuda")
+    w = torch.zeros((t, k), dtype=torch.float32, device="cuda")
+    lg = torch.zeros((t, e), dtype=torch.float32, device="cuda")
+    moe.encode_router(ops.bf16_tensor(wr), ops.bf16_tensor(x), idx, w, t=t, out_logits=lg)
+    _sync()
+    for i in range(t):
+        ref_lg = oracle.router_logits(wr, x[i])
+        assert np.array_equal(lg[i].cpu().numpy().view(np.uint32), ref_lg.view(np.uint32))
+        ri, rw = oracle.topk_softmax(ref_lg, k, full_softmax=bool(mode))
+        assert np.array_equal(idx[i].cpu().numpy().astype(np.uint32), ri)
+        assert np.array_equal(w[i].cpu().numpy().view(np.uint32), rw.view(np.uint32))
+
+
+def _tie_logits(oracle, count, trial, rng):
+    """the four logit families of RouterTopKParityTests.swift:109-127"""
+    kind = trial % 4
+    if kind == 0:
+        return np.array([rng.uniform(-4.0, 4.0) for _ in range(count)], np.float32)
+    if kind == 1:
+        return np.array([np.float32(np.round(np.float32(rng.uniform(-3.0, 3.0) * np.float32(4))) / 4)
+                         for _ in range(count)], np.float32)
+    if kind == 2:
+        levels = [1.5, 0.5, -0.5]
+        return np.array([levels[rng.next() % 3] for _ in range(count)], np.float32)
+    return np.full(count, 0.75, np.float32)
+
+
+@pytest.mark.parametrize("e", [8, 16, 24, 33, 100, 128, 168, 255, 256])
+def test_topk_ties_match_serial(gpu, oracle, e):
+    """tie-heavy logits straight into the selector through a one-hot x."""
+    from mference_amd import _capi
+    import ctypes as C
+    rng = oracle.Rng(0x5EED0001 + e)
+    k = 8
+    for trial in range(12):
+        logits = _tie_logits(oracle, e, trial, rng)
+        for _ in range(e):
+            rng.uniform(0.6, 1.4)  # the reference draws per-expert scales here
+        # router weights = bf16(logit) column against x = e_0 reproduces bf16-rounded logits
+        wr = np.zeros((e, 64), np.uint16)
+        wr[:, 0] = oracle.bf16_bits(logits)
+        x = np.zeros(64, np.uint16)
+        x[0] = oracle.bf16_bits(np.array([1.0], np.float32))[0]
+        lg_ref = oracle.bf16_to_float(wr[:, 0])
+        for mode in ((0, 1) if e % 32 == 0 else (0,)):
+            moe = ops.MoE(gpu, 64, 64, e, k, router_mode=mode)
+            idx = torch.zeros((1, k), dtype=torch.int32, device="cuda")
+            w = torch.zeros((1, k), dtype=torch.float32, device="cuda")
+            moe.encode_router(ops.bf16_tensor(wr), ops.bf16_tensor(x), idx, w)
+            _sync()
+            ri, rw = oracle.topk_softmax(lg_ref, k, full_softmax=bool(mode))
+            assert np.array_equal(idx[0].cpu().numpy().astype(np.uint32), ri), (e, trial, mode)
+            assert np.array_equal(w[0].cpu().numpy().view(np.uint32), rw.view(np.uint32))
+
+
+@pytest.mark.parametrize("bits,d,f,e,k,fs,t", [
+    (4, 128, 64, 16, 8, 64, 1),
+    (4, 256, 128, 32, 6, 0, 3),
+    (4, 2048, 512, 32, 8, 512, 1),
+    (2, 512, 256, 16, 6, 128, 4),
+    (1, 512, 256, 16, 8, 0, 2),
+    (4, 192, 320, 12, 4, 192, 2),
+])
+def test_decode_layer_matches_oracle(gpu, oracle, bits, d, f, e, k, fs, t):
+    root = ROOT_SEED + 0x9000 + bits
+    layer = oracle.synth_layer(root, d, f, e, k, bits=bits, fs=fs)
+    x = oracle.synth_x(root, t, d)
+    ref_y, ref_idx, ref_w = oracle.moe_layer(layer, x)
+    moe = make_moe(gpu, layer)
+    wts = to_device_layer(layer)
+    xd = ops.bf16_tensor(x)
+    y = torch.zeros((t, d), dtype=torch.bfloat16, device="cuda")
+    idx = torch.zeros((t, k), dtype=torch.int32, device="cuda")
+    w = torch.zeros((t, k), dtype=torch.float32, device="cuda")
+    moe.encode_decode_layer(wts, xd, y, t=t, out_indices=idx, out_weights=w)
+    _sync()
+    assert np.array_equal(idx.cpu().numpy().astype(np.uint32), ref_idx)
+    assert np.array_equal(w.cpu().numpy().view(np.uint32), ref_w.view(np.uint32))
+    assert_layer_close(oracle.bf16_to_float(ops.bf16_bits(y)), oracle.bf16_to_float(ref_y),
+                       f"decode layer bits={bits} d={d} f={f}")
+
+
+def test_two_phase_matches_oracle_and_fused(gpu, oracle):
+    """phase 1 + phase 2 as separate calls (MoEFusedFFNTests.swift:44-190 shape D 128, F 64)."""
+    d, f, e, k = 128, 64, 16, 8
+    root = ROOT_SEED + 0x2D3
+    layer = oracle.synth_layer(root, d, f, e, k, bits=4, fs=0)
+    x = oracle.synth_x(root, 1, d)
+    ref_y, ref_idx, ref_w = oracle.moe_layer(layer, x)
+    moe = make_moe(gpu, layer)
+    wts = to_device_layer(layer)
+    xd = ops.bf16_tensor(x)
+    idx = torch.from_numpy(ref_idx.astype(np.int32)).cuda()
+    w = torch.from_numpy(ref_w).cuda()
+    acts = torch.zeros((1, k, f), dtype=torch.bfloat16, device="cuda")
+    y = torch.zeros((1, d), dtype=torch.bfloat16, device="cuda")
+    moe.encode_routed_phase1(wts.experts, wts.offsets, idx, xd, acts)
+    moe.encode_routed_phase2_reduce(wts.experts, wts.offsets, idx, w, acts, None, y)
+    _sync()
+    for s in range(k):
+        ref_act = oracle.expert_phase1(layer.experts[ref_idx[0, s]], layer.off, 4, d, f, x[0])
+        ma, rl = errors(oracle.bf16_to_float(ops.bf16_bits(acts[0, s])), oracle.bf16_to_float(ref_act))
+        assert rl < 1e-3
+    assert_layer_close(oracle.bf16_to_float(ops.bf16_bits(y)), oracle.bf16_to_float(ref_y), "two-phase")

@@ -228,6 +228,19 @@ mf_status mf_moe_decode_layer(mf_moe* h, mf_stream stream, const mf_moe_layer_we
                               const uint16_t* x, uint32_t t, uint16_t* y, uint16_t* hidden,
                               uint32_t* out_idx, float* out_w);
 
+/* Chooses between the single fused launch (default) and the chain of separate
+ * launches (router, top-k, shared expert, phase 1, phase 2) inside
+ * mf_moe_decode_layer.  Both give bit-identical results; the chain is the
+ * structure of the reference's decode step and handles operands that are not
+ * 16-byte aligned.  No counterpart in the reference. */
+mf_status mf_moe_set_fused(mf_moe* h, int enabled);
+
+/* Synchronises `stream` and reports whether any fused launch of this handle
+ * gave up on a grid barrier (MF_ERR_LAUNCH) since the handle was created.
+ * No counterpart in the reference (Metal reports this through
+ * MTLCommandBuffer.error). */
+mf_status mf_moe_status(mf_moe* h, mf_stream stream);
+
 /* ------------------------------------------------------- ragged prefill */
 
 /* PrefillMoEGrouping.groupTokenExpertPairs (Kernels/Prefill/MoE/

@@ -84,6 +84,8 @@ SIGNATURES = {
     "mf_moe_phase1": (_I, [_P, _P, _P, _SZ, C.POINTER(ExpertOffsets), _P, _P, _U32, _U32, _P]),
     "mf_moe_phase2": (_I, [_P, _P, _P, _SZ, C.POINTER(ExpertOffsets), _P, _P, _P, _P, _U32, _P]),
     "mf_moe_decode_layer": (_I, [_P, _P, C.POINTER(LayerWeights), _P, _U32, _P, _P, _P, _P]),
+    "mf_moe_set_fused": (_I, [_P, _I]),
+    "mf_moe_status": (_I, [_P, _P]),
     "mf_group_pairs_host": (_I, [_P, _SZ, _I, _I, _I, _I, _P, _SZ, _P, _P, _P, _P,
                                  C.POINTER(_SZ), _P, C.POINTER(_SZ), _P]),
 }
@@ -103,6 +105,10 @@ def lib() -> C.CDLL:
             raise LibraryMissing(
                 f"{LIB_PATH} is missing: build it with `python -m mference_amd.build` "
                 "(there is no CPU fallback)")
+        # torch carries its own HIP runtime; it has to be the one already loaded
+        # when libmfmoe resolves libamdhip64, or device pointers and streams
+        # would belong to a different runtime instance than the kernels.
+        import torch  # noqa: F401
         L = C.CDLL(LIB_PATH)
         for name, (res, args) in SIGNATURES.items():
             fn = getattr(L, name)

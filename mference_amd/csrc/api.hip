@@ -309,6 +309,10 @@ mf_status mf_moe_decode_layer(mf_moe* h, mf_stream stream, const mf_moe_layer_we
                      !qtensor_ok(wts->shared_down, c.shared_bits)))
     return MF_ERR_INVALID_ARGUMENT;
   auto s = static_cast<hipStream_t>(stream);
+  if (h->fused && mf::fused_supported(c, *wts, x, y, hidden)) {
+    MF_HIP(h->ctx, mf::launch_fused_decode(s, *h, *wts, x, t, y, hidden, out_idx, out_w));
+    return MF_OK;
+  }
   uint32_t* idx = h->ws.idx;
   float* w = h->ws.w;
   MF_HIP(h->ctx, mf::launch_router_logits(s, wts->router_w, x, c.num_experts, c.d, t, c.d,
@@ -336,6 +340,26 @@ mf_status mf_moe_decode_layer(mf_moe* h, mf_stream stream, const mf_moe_layer_we
                                   hipMemcpyDeviceToDevice, s));
   if (out_w)
     MF_HIP(h->ctx, hipMemcpyAsync(out_w, w, sizeof(float) * t * c.top_k, hipMemcpyDeviceToDevice, s));
+  return MF_OK;
+}
+
+mf_status mf_moe_set_fused(mf_moe* h, int enabled) {
+  if (!h) return MF_ERR_INVALID_ARGUMENT;
+  h->fused = enabled != 0;
+  return MF_OK;
+}
+
+mf_status mf_moe_status(mf_moe* h, mf_stream stream) {
+  if (!h) return MF_ERR_INVALID_ARGUMENT;
+  uint32_t word = 0;
+  auto s = static_cast<hipStream_t>(stream);
+  MF_HIP(h->ctx, hipMemcpyAsync(&word, h->ws.sync + 3, sizeof word, hipMemcpyDeviceToHost, s));
+  MF_HIP(h->ctx, hipStreamSynchronize(s));
+  if (word != 0) {
+    snprintf(h->ctx->hip_error, sizeof h->ctx->hip_error,
+             "fused decode layer: a grid barrier timed out (status word %u)", word);
+    return MF_ERR_LAUNCH;
+  }
   return MF_OK;
 }
 

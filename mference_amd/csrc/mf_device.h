@@ -220,6 +220,14 @@ __device__ __forceinline__ void load_scale_bias(const uint16_t* srow, const uint
   else b = bf16_to_f(brow[g]);
 }
 
+// lanes of a wave that share one row of n elements (power of two, <= 64)
+__host__ __device__ __forceinline__ uint32_t lanes_per_row_log2_dev(uint32_t n, uint32_t elems_per_lane) {
+  const uint32_t need = (n + elems_per_lane - 1) / elems_per_lane;
+  uint32_t l = 0;
+  while ((1u << l) < need && l < 6) ++l;
+  return l;
+}
+
 // storage width of a format in bits per element
 template <int BITS> struct Store { static constexpr int kBits = (BITS == kBits4) ? 4 : 2; };
 

@@ -29,6 +29,7 @@ struct mf_moe_workspace {
 struct mf_moe {
   mf_ctx* ctx = nullptr;
   mf_moe_config cfg{};
+  bool fused = true;  // mf_moe_set_fused
   void* ws_base = nullptr;
   size_t ws_bytes = 0;
   mf_moe_workspace ws{};
@@ -80,5 +81,13 @@ hipError_t launch_phase1(hipStream_t s, const mf_moe_config& cfg, const void* ba
 hipError_t launch_phase2(hipStream_t s, const mf_moe_config& cfg, const void* base, size_t stride,
                          const mf_expert_offsets& off, const uint32_t* idx, const float* w,
                          const uint16_t* acts, const uint16_t* residual, uint32_t t, uint16_t* y);
+
+
+// moe_fused.hip
+bool fused_supported(const mf_moe_config& c, const mf_moe_layer_weights& w, const void* x,
+                     const void* y, const void* hidden);
+hipError_t launch_fused_decode(hipStream_t s, const mf_moe& h, const mf_moe_layer_weights& w,
+                               const uint16_t* x, uint32_t t, uint16_t* y, uint16_t* hidden,
+                               uint32_t* out_idx, float* out_w);
 
 }  // namespace mf

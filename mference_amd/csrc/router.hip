@@ -3,41 +3,11 @@
 // dot_bf16_row) and exp/divide are IEEE sequences shared with it.
 #include "mf_device.h"
 #include "mf_internal.h"
+#include "mf_router.h"
 
 #pragma clang fp contract(off)
 
 namespace mf {
-
-// One wave per (token, expert) row.  Elements are split into 8-wide chunks;
-// chunk c belongs to lane c % 64; a lane accumulates its elements in ascending
-// order with fmaf into one fp32 accumulator; lanes are combined by an xor
-// butterfly with strides 32..1.  Replaces router_gemv_bf16_r4
-// (moe.metal:162-185) / maple_router_bf16_gemv (maple_moe.metal:25-60).
-__device__ __forceinline__ float dot_bf16_row(const uint16_t* __restrict__ w,
-                                              const uint16_t* __restrict__ x, uint32_t d,
-                                              uint32_t lane, bool aligned) {
-  float acc = 0.0f;
-  const uint32_t chunks = d / 8;
-  for (uint32_t c = lane; c < chunks; c += kWave) {
-    uint4 wv, xv;
-    if (aligned) {
-      wv = load_x8<true>(w + c * 8);
-      xv = load_x8<true>(x + c * 8);
-    } else {
-      wv = load_x8<false>(w + c * 8);
-      xv = load_x8<false>(x + c * 8);
-    }
-    acc = __builtin_fmaf(bf16_lo(wv.x), bf16_lo(xv.x), acc);
-    acc = __builtin_fmaf(bf16_hi(wv.x), bf16_hi(xv.x), acc);
-    acc = __builtin_fmaf(bf16_lo(wv.y), bf16_lo(xv.y), acc);
-    acc = __builtin_fmaf(bf16_hi(wv.y), bf16_hi(xv.y), acc);
-    acc = __builtin_fmaf(bf16_lo(wv.z), bf16_lo(xv.z), acc);
-    acc = __builtin_fmaf(bf16_hi(wv.z), bf16_hi(xv.z), acc);
-    acc = __builtin_fmaf(bf16_lo(wv.w), bf16_lo(xv.w), acc);
-    acc = __builtin_fmaf(bf16_hi(wv.w), bf16_hi(xv.w), acc);
-  }
-  return wave_sum(acc);
-}
 
 __global__ __launch_bounds__(256) void router_logits_kernel(const uint16_t* __restrict__ w,
                                                             const uint16_t* __restrict__ x,
@@ -58,162 +28,14 @@ __global__ __launch_bounds__(256) void router_logits_kernel(const uint16_t* __re
   }
 }
 
-constexpr int kMaxPerLane = MF_MAX_EXPERTS / kWave;  // 8
-constexpr uint32_t kNoWinner = 0xFFFFFFFFu;
-
-// argmax over the wave with "equal score keeps the lower index"; all lanes
-// return the winner.
-__device__ __forceinline__ void wave_argmax(float& bv, uint32_t& bi) {
-#pragma unroll
-  for (int o = 32; o > 0; o >>= 1) {
-    const float ov = __shfl_xor(bv, o, kWave);
-    const uint32_t oi = __shfl_xor(bi, o, kWave);
-    if (ov > bv || (ov == bv && oi < bi)) {
-      bv = ov;
-      bi = oi;
-    }
-  }
-}
-
-// One wave per token.  Lane l owns experts l, l+64, ...  (ownership does not
-// change the result: every step picks the highest score, lowest index first).
-//
-// mode 0 = router_topk_select_k8 (moe.metal:190-240) for any k <= 8: k rounds of
-//   strict-greater / lower-index argmax over the logits (never selecting NaN or
-//   -inf, unfilled slots stay at index 0), then w_i = exp(s_i - s_0) / sum.
-// mode 1 = maple_router_top8_full_softmax (maple_moe.metal:62-119): any
-//   non-finite logit -> idx = e, w = 0; softmax over all experts with the
-//   32-wide tree sums added block by block, k rounds of argmax on the
-//   probabilities, renormalise with the 1e-20 guards.
+// one wave per token
 __global__ __launch_bounds__(64) void topk_kernel(const float* __restrict__ logits, uint32_t e,
                                                   uint32_t k, int mode,
                                                   uint32_t* __restrict__ idx,
                                                   float* __restrict__ w) {
-  const uint32_t lane = threadIdx.x;
   const uint32_t tok = blockIdx.x;
-  const float* lg = logits + static_cast<size_t>(tok) * e;
-  const uint32_t per = (e + kWave - 1) / kWave;
-  float ch[kMaxPerLane];
-#pragma unroll
-  for (int j = 0; j < kMaxPerLane; ++j) {
-    const uint32_t x = lane + j * kWave;
-    ch[j] = (static_cast<uint32_t>(j) < per && x < e) ? lg[x] : -__builtin_inff();
-  }
-  float top_s[MF_MAX_TOPK];
-  uint32_t top_i[MF_MAX_TOPK];
-
-  if (mode == 1) {
-    bool bad = false;
-    float mx = -1.0e30f;
-#pragma unroll
-    for (int j = 0; j < kMaxPerLane; ++j) {
-      const uint32_t x = lane + j * kWave;
-      if (static_cast<uint32_t>(j) < per && x < e) {
-        if (!__builtin_isfinite(ch[j])) bad = true;
-        if (ch[j] > mx) mx = ch[j];
-      }
-    }
-    bad = __any(bad);
-    if (bad) {
-      if (lane < k) {
-        idx[static_cast<size_t>(tok) * k + lane] = e;
-        w[static_cast<size_t>(tok) * k + lane] = 0.0f;
-      }
-      return;
-    }
-#pragma unroll
-    for (int o = 32; o > 0; o >>= 1) {
-      const float other = __shfl_xor(mx, o, kWave);
-      if (other > mx) mx = other;
-    }
-    // scores and the blocked sum: block g = experts [32g, 32g+32) = half a wave
-    // row j (g = 2j + (lane >= 32)); tree over 16,8,4,2,1 then blocks in order.
-    float total = 0.0f;
-#pragma unroll
-    for (int j = 0; j < kMaxPerLane; ++j) {
-      const uint32_t x = lane + j * kWave;
-      const bool live = static_cast<uint32_t>(j) < per && x < e;
-      ch[j] = live ? mf_exp(ch[j] - mx) : 0.0f;
-      float part = ch[j];
-#pragma unroll
-      for (int o = 16; o > 0; o >>= 1) part = part + __shfl_xor(part, o, kWave);
-      const float lo = __shfl(part, 0, kWave), hi = __shfl(part, 32, kWave);
-      if (static_cast<uint32_t>(2 * j) < e / 32) total += lo;
-      if (static_cast<uint32_t>(2 * j + 1) < e / 32) total += hi;
-    }
-    const float recip = 1.0f / (total + 1.0e-20f);
-#pragma unroll
-    for (int j = 0; j < kMaxPerLane; ++j) {
-      const uint32_t x = lane + j * kWave;
-      const bool live = static_cast<uint32_t>(j) < per && x < e;
-      ch[j] = live ? ch[j] * recip : -__builtin_inff();
-    }
-  }
-
-  uint32_t taken = 0;
-  for (uint32_t r = 0; r < k; ++r) {
-    float bv = (mode == 1) ? -1.0e30f : -__builtin_inff();
-    uint32_t bi = kNoWinner;
-#pragma unroll
-    for (int j = 0; j < kMaxPerLane; ++j) {
-      if (!(taken & (1u << j)) && ch[j] > bv) {
-        bv = ch[j];
-        bi = lane + j * kWave;
-      }
-    }
-    wave_argmax(bv, bi);
-    if (bi != kNoWinner && (bi & (kWave - 1)) == lane) taken |= 1u << (bi / kWave);
-#pragma unroll
-    for (int i = 0; i < MF_MAX_TOPK; ++i) {
-      if (static_cast<uint32_t>(i) == r) {
-        top_s[i] = bv;
-        top_i[i] = bi;
-      }
-    }
-  }
-  if (lane != 0) return;
-
-  float wt[MF_MAX_TOPK];
-  if (mode == 1) {
-    float sel = 0.0f;
-#pragma unroll
-    for (int i = 0; i < MF_MAX_TOPK; ++i) {
-      if (static_cast<uint32_t>(i) < k) {
-        if (top_i[i] == kNoWinner) top_i[i] = 0;  // maple: bestIndex stays 0
-        sel += top_s[i];
-      }
-    }
-#pragma unroll
-    for (int i = 0; i < MF_MAX_TOPK; ++i)
-      if (static_cast<uint32_t>(i) < k) wt[i] = top_s[i] / (sel + 1.0e-20f);
-  } else {
-#pragma unroll
-    for (int i = 0; i < MF_MAX_TOPK; ++i) {
-      if (static_cast<uint32_t>(i) < k && top_i[i] == kNoWinner) {
-        top_i[i] = 0;
-        top_s[i] = -__builtin_inff();
-      }
-    }
-    const float max_s = top_s[0];
-    float sum = 0.0f;
-#pragma unroll
-    for (int i = 0; i < MF_MAX_TOPK; ++i) {
-      if (static_cast<uint32_t>(i) < k) {
-        wt[i] = mf_exp(top_s[i] - max_s);
-        sum += wt[i];
-      }
-    }
-#pragma unroll
-    for (int i = 0; i < MF_MAX_TOPK; ++i)
-      if (static_cast<uint32_t>(i) < k) wt[i] = wt[i] / sum;
-  }
-#pragma unroll
-  for (int i = 0; i < MF_MAX_TOPK; ++i) {
-    if (static_cast<uint32_t>(i) < k) {
-      idx[static_cast<size_t>(tok) * k + i] = top_i[i];
-      w[static_cast<size_t>(tok) * k + i] = wt[i];
-    }
-  }
+  topk_wave(logits + static_cast<size_t>(tok) * e, e, k, mode, idx + static_cast<size_t>(tok) * k,
+            w + static_cast<size_t>(tok) * k, threadIdx.x);
 }
 
 hipError_t launch_router_logits(hipStream_t s, const uint16_t* w, const uint16_t* x, uint32_t e,

@@ -240,6 +240,14 @@ class MoE:
         except Exception:
             pass
 
+    def set_fused(self, enabled: bool) -> None:
+        """single fused launch (default) or the chain of separate launches"""
+        check(_capi.lib().mf_moe_set_fused(self._h, 1 if enabled else 0), self.context.handle)
+
+    def status(self, stream=None) -> None:
+        """synchronises and raises if a fused launch gave up on a grid barrier"""
+        check(_capi.lib().mf_moe_status(self._h, _stream(stream)), self.context.handle)
+
     def encode_router(self, router_w, x, out_indices, out_weights, t: int = 1,
                       x_stride: Optional[int] = None, out_logits=None, stream=None):
         """encodeRouterGemma4 (MoE.swift:153-203) / encodeRouterTopK / encodeRouterTop8."""

@@ -187,15 +187,44 @@ def test_decode_layer_matches_oracle(gpu, oracle, bits, d, f, e, k, fs, t):
     moe = make_moe(gpu, layer)
     wts = to_device_layer(layer)
     xd = ops.bf16_tensor(x)
-    y = torch.zeros((t, d), dtype=torch.bfloat16, device="cuda")
-    idx = torch.zeros((t, k), dtype=torch.int32, device="cuda")
-    w = torch.zeros((t, k), dtype=torch.float32, device="cuda")
-    moe.encode_decode_layer(wts, xd, y, t=t, out_indices=idx, out_weights=w)
-    _sync()
-    assert np.array_equal(idx.cpu().numpy().astype(np.uint32), ref_idx)
-    assert np.array_equal(w.cpu().numpy().view(np.uint32), ref_w.view(np.uint32))
-    assert_layer_close(oracle.bf16_to_float(ops.bf16_bits(y)), oracle.bf16_to_float(ref_y),
-                       f"decode layer bits={bits} d={d} f={f}")
+    results = {}
+    for fused in (True, False):
+        moe.set_fused(fused)
+        y = torch.zeros((t, d), dtype=torch.bfloat16, device="cuda")
+        idx = torch.zeros((t, k), dtype=torch.int32, device="cuda")
+        w = torch.zeros((t, k), dtype=torch.float32, device="cuda")
+        for rep in range(3):  # the fused launch re-arms its own barrier counters
+            y.zero_()
+            moe.encode_decode_layer(wts, xd, y, t=t, out_indices=idx, out_weights=w)
+            moe.status()
+        assert np.array_equal(idx.cpu().numpy().astype(np.uint32), ref_idx)
+        assert np.array_equal(w.cpu().numpy().view(np.uint32), ref_w.view(np.uint32))
+        assert_layer_close(oracle.bf16_to_float(ops.bf16_bits(y)), oracle.bf16_to_float(ref_y),
+                           f"decode layer fused={fused} bits={bits} d={d} f={f}")
+        results[fused] = ops.bf16_bits(y)
+    # one fused launch == the chain of separate launches, bit for bit
+    # (the reference's fused == 3-dispatch gate, SharedExpertInt4Tests.swift:55-115)
+    assert np.array_equal(results[True], results[False])
+
+
+def test_decode_layer_residual_add_in_place(gpu, oracle):
+    d, f, e, k, fs, t = 256, 128, 16, 4, 128, 2
+    root = ROOT_SEED + 0x9100
+    layer = oracle.synth_layer(root, d, f, e, k, bits=4, fs=fs)
+    x = oracle.synth_x(root, t, d)
+    ref_y, _, _ = oracle.moe_layer(layer, x)
+    moe = make_moe(gpu, layer)
+    wts = to_device_layer(layer)
+    for fused in (True, False):
+        moe.set_fused(fused)
+        hidden = ops.bf16_tensor(x)
+        y = torch.zeros((t, d), dtype=torch.bfloat16, device="cuda")
+        moe.encode_decode_layer(wts, hidden, y, t=t, hidden=hidden)
+        moe.status()
+        yb = ops.bf16_bits(y)
+        want = oracle.bf16_bits(oracle.bf16_to_float(x) + oracle.bf16_to_float(yb))
+        assert np.array_equal(ops.bf16_bits(hidden), want)
+        assert_layer_close(oracle.bf16_to_float(yb), oracle.bf16_to_float(ref_y), "residual")
 
 
 def test_two_phase_matches_oracle_and_fused(gpu, oracle):

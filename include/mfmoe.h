@@ -235,6 +235,15 @@ mf_status mf_moe_decode_layer(mf_moe* h, mf_stream stream, const mf_moe_layer_we
  * 16-byte aligned.  No counterpart in the reference. */
 mf_status mf_moe_set_fused(mf_moe* h, int enabled);
 
+/* Phase trace of the fused launch: when device_buffer is not NULL every
+ * workgroup writes the 100 MHz wall clock at its stage boundaries (slots:
+ * 0 start, 1 stage A done, 2 barrier 1 passed, 3 top-k done, 4 stage B done,
+ * 5 barrier 2 passed, 6 end) to device_buffer[workgroup*8 + slot]; needs
+ * mf_ctx_num_cu()*8*8 bytes.  The counterpart of the reference's
+ * MFERENCE_PHASES=1 phase counters (RealForwardRunner.swift:397-398). */
+mf_status mf_moe_set_phase_trace(mf_moe* h, uint64_t* device_buffer, size_t bytes);
+int mf_ctx_num_cu(const mf_ctx* ctx);
+
 /* Synchronises `stream` and reports whether any fused launch of this handle
  * gave up on a grid barrier (MF_ERR_LAUNCH) since the handle was created.
  * No counterpart in the reference (Metal reports this through

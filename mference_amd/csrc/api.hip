@@ -206,8 +206,8 @@ mf_status mf_moe_create(mf_ctx* ctx, const mf_moe_config* cfg, mf_moe** out) {
   const size_t o_acts = take(T * cfg->top_k * cfg->f * sizeof(uint16_t));
   const size_t o_sact = take(T * std::max<uint32_t>(cfg->shared_f, 64) * sizeof(uint16_t));
   const size_t o_sy = take(T * cfg->d * sizeof(uint16_t));
-  const size_t o_gate = take(T * sizeof(uint16_t));
-  const size_t o_sync = take(64 * sizeof(uint32_t));
+  const size_t o_gate = take(T * sizeof(float));
+  const size_t o_sync = take((2 * 512 + 64) * sizeof(uint32_t));
   h->ws_bytes = pos;
   if (hipSetDevice(ctx->device) != hipSuccess) {
     delete h;
@@ -349,11 +349,21 @@ mf_status mf_moe_set_fused(mf_moe* h, int enabled) {
   return MF_OK;
 }
 
+mf_status mf_moe_set_phase_trace(mf_moe* h, uint64_t* device_buffer, size_t bytes) {
+  if (!h) return MF_ERR_INVALID_ARGUMENT;
+  if (device_buffer && bytes < static_cast<size_t>(h->ctx->num_cu) * 8 * sizeof(uint64_t))
+    return MF_ERR_SCRATCH_TOO_SMALL;
+  h->trace = reinterpret_cast<unsigned long long*>(device_buffer);
+  return MF_OK;
+}
+
+int mf_ctx_num_cu(const mf_ctx* ctx) { return ctx ? ctx->num_cu : 0; }
+
 mf_status mf_moe_status(mf_moe* h, mf_stream stream) {
   if (!h) return MF_ERR_INVALID_ARGUMENT;
   uint32_t word = 0;
   auto s = static_cast<hipStream_t>(stream);
-  MF_HIP(h->ctx, hipMemcpyAsync(&word, h->ws.sync + 3, sizeof word, hipMemcpyDeviceToHost, s));
+  MF_HIP(h->ctx, hipMemcpyAsync(&word, h->ws.sync + 2 * 512, sizeof word, hipMemcpyDeviceToHost, s));
   MF_HIP(h->ctx, hipStreamSynchronize(s));
   if (word != 0) {
     snprintf(h->ctx->hip_error, sizeof h->ctx->hip_error,

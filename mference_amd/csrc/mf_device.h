@@ -18,6 +18,17 @@ enum : int { kBitsTernary = 1, kBits2 = 2, kBits4 = 4 };
 
 // elements covered by one 16-byte load of packed codes
 template <int BITS> struct Fmt { static constexpr int kElemsPer16B = (BITS == kBits4) ? 32 : 64; };
+// storage width of a format in bits per element (ternary is stored as 2-bit codes)
+template <int BITS> struct Store { static constexpr int kBits = (BITS == kBits4) ? 4 : 2; };
+
+// lanes of a wave that share one row of n elements (power of two, <= 64)
+__host__ __device__ __forceinline__ uint32_t lanes_per_row_log2_dev(uint32_t n,
+                                                                    uint32_t elems_per_lane) {
+  const uint32_t need = (n + elems_per_lane - 1) / elems_per_lane;
+  uint32_t l = 0;
+  while ((1u << l) < need && l < 6) ++l;
+  return l;
+}
 
 // ------------------------------------------------------------------ bf16
 
@@ -63,15 +74,91 @@ __device__ __forceinline__ float mf_silu(float x) { return x / (1.0f + mf_exp(-x
 
 // --------------------------------------------------------- wave reductions
 
-// xor butterfly over the low `lanes` lanes of each aligned lane group
-// (lanes = power of two <= 64); every lane of the group ends with the sum.
-// Strides run from lanes/2 down to 1: this order is part of the router's
-// bit-exact contract.
+// cross-lane move inside a row of 16 lanes (DPP); CTRL: 0xB1 = swap lanes
+// (l, l^1), 0x4E = (l, l^2), 0x141 = mirror inside 8, 0x140 = mirror inside 16
+template <int CTRL> __device__ __forceinline__ float dpp_f(float v) {
+  return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), CTRL, 0xF, 0xF, true));
+}
+__device__ __forceinline__ float readlane_f(float v, int lane) {
+  return __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), lane));
+}
+
+// Sum over aligned groups of `lanes` lanes (power of two <= 64); every lane of
+// a group ends with the group's sum.  The tree pairs neighbours first:
+// (l, l^1), then (l, l^2), 4, 8, 16, 32 -- identical to an xor butterfly with
+// ascending strides, which is the order the router's bit-exact contract names.
 __device__ __forceinline__ float group_sum(float v, int lanes) {
-  for (int o = lanes >> 1; o > 0; o >>= 1) v = v + __shfl_xor(v, o, kWave);
+  if (lanes >= 2) v = v + dpp_f<0xB1>(v);
+  if (lanes >= 4) v = v + dpp_f<0x4E>(v);
+  if (lanes >= 8) v = v + dpp_f<0x141>(v);
+  if (lanes >= 16) v = v + dpp_f<0x140>(v);
+  if (lanes >= 32) {
+    const float r0 = readlane_f(v, 0), r1 = readlane_f(v, 16);
+    const float r2 = readlane_f(v, 32), r3 = readlane_f(v, 48);
+    const float lo = r0 + r1, hi = r2 + r3;
+    if (lanes >= 64) v = lo + hi;
+    else v = (threadIdx.x & 32) ? hi : lo;
+  }
   return v;
 }
 __device__ __forceinline__ float wave_sum(float v) { return group_sum(v, kWave); }
+
+// maximum over the wave, returned in every lane (no NaN inputs)
+__device__ __forceinline__ float wave_max(float v) {
+  v = fmaxf(v, dpp_f<0xB1>(v));
+  v = fmaxf(v, dpp_f<0x4E>(v));
+  v = fmaxf(v, dpp_f<0x141>(v));
+  v = fmaxf(v, dpp_f<0x140>(v));
+  const float r0 = readlane_f(v, 0), r1 = readlane_f(v, 16);
+  const float r2 = readlane_f(v, 32), r3 = readlane_f(v, 48);
+  return fmaxf(fmaxf(r0, r1), fmaxf(r2, r3));
+}
+
+// ------------------------------------------- device-coherent accesses
+//
+// Data that workgroups on different XCDs exchange inside one launch goes
+// through these: `sc1` makes a store write through, and a load miss, every
+// cache that is private to a CU or an XCD, so no bulk cache write-back or
+// invalidate is needed around the grid barriers.
+
+__device__ __forceinline__ void store_u16_agent(uint16_t* p, uint16_t v) {
+  const uint32_t vv = v;
+  asm volatile("global_store_short %0, %1, off sc1" : : "v"(p), "v"(vv) : "memory");
+}
+__device__ __forceinline__ uint16_t load_u16_agent(const uint16_t* p) {
+  uint32_t r;
+  asm volatile("global_load_ushort %0, %1, off sc1\n\ts_waitcnt vmcnt(0)" : "=v"(r) : "v"(p) : "memory");
+  return static_cast<uint16_t>(r);
+}
+__device__ __forceinline__ void store_u32_agent(uint32_t* p, uint32_t v) {
+  __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ void store_f32_agent(float* p, float v) {
+  __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ float load_f32_agent(const float* p) {
+  return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ uint4 load_u32x4_agent(const void* p) {
+  uint4 r;
+  asm volatile("global_load_dwordx4 %0, %1, off sc1\n\ts_waitcnt vmcnt(0)" : "=v"(r) : "v"(p) : "memory");
+  return r;
+}
+// every store this wave has issued is acknowledged at its scope
+__device__ __forceinline__ void wait_stores() { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); }
+
+// 32 bf16 (64 bytes) of exchanged activations
+__device__ __forceinline__ void load_x32_agent(const uint16_t* p, uint4 (&x)[4]) {
+  asm volatile(
+      "global_load_dwordx4 %0, %4, off sc1\n\t"
+      "global_load_dwordx4 %1, %4, off offset:16 sc1\n\t"
+      "global_load_dwordx4 %2, %4, off offset:32 sc1\n\t"
+      "global_load_dwordx4 %3, %4, off offset:48 sc1\n\t"
+      "s_waitcnt vmcnt(0)"
+      : "=&v"(x[0]), "=&v"(x[1]), "=&v"(x[2]), "=&v"(x[3])
+      : "v"(p)
+      : "memory");
+}
 
 // ------------------------------------------------------------- raw loads
 
@@ -112,101 +199,128 @@ __device__ __forceinline__ uint4 load_x8(const uint16_t* p) {
 }
 
 // ------------------------------------------------- per-lane code x x dots
+//
+// One lane's share of a row is 16 bytes of codes: 32 four-bit elements (half a
+// quantization group) or 64 two-bit elements (one group).  The dot product
+// sum(q*x) runs on v_dot2c_f32_bf16: two codes are masked out of the packed
+// word straight into the mantissas of a bf16 pair (0x4300 | q = 128 + q,
+// exact), multiplied with a matching bf16 pair of x and accumulated in fp32;
+// the 128 * sum(x) this adds is taken off once per lane share.  Codes are
+// paired (j, j + 4) for 4-bit and (j, j + 8) for 2-bit because those pairs sit
+// 16 bits apart in the packed word; the x slice is permuted once to match and
+// reused for every row that meets it (gate and up, several tokens' rows).
 
-// byte i of v as float (v_cvt_f32_ubyte{i})
-__device__ __forceinline__ float ubyte_f(uint32_t v, int i) {
-  return static_cast<float>((v >> (8 * i)) & 0xFFu);
+typedef __attribute__((ext_vector_type(2))) short mf_bf16x2;
+
+__device__ __forceinline__ float dot2_bf16(uint32_t a, uint32_t b, float acc) {
+  return __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(mf_bf16x2, a),
+                                         __builtin_bit_cast(mf_bf16x2, b), acc, false);
 }
 
-// 8 consecutive 4-bit codes (one uint32, element j at bit 4j) against 8 bf16
-// (four packed pairs).  dot += sum q*x, sum += sum x.
-__device__ __forceinline__ void dot8_q4(uint32_t w, const uint4& x, float& dot, float& sum) {
-  const uint32_t lo = w & 0x0F0F0F0Fu;         // byte i = code of element 2i
-  const uint32_t hi = (w >> 4) & 0x0F0F0F0Fu;  // byte i = code of element 2i+1
-  const uint32_t xs[4] = {x.x, x.y, x.z, x.w};
-#pragma unroll
-  for (int i = 0; i < 4; ++i) {
-    const float x0 = bf16_lo(xs[i]), x1 = bf16_hi(xs[i]);
-    dot = __builtin_fmaf(ubyte_f(lo, i), x0, dot);
-    dot = __builtin_fmaf(ubyte_f(hi, i), x1, dot);
-    sum += x0 + x1;
-  }
-}
+constexpr uint32_t kMagic128 = 0x43004300u;  // bf16 pair (128.0, 128.0)
+constexpr uint32_t kOnes = 0x3F803F80u;      // bf16 pair (1.0, 1.0)
 
-// 16 consecutive 2-bit codes (one uint32, element j at bit 2j) against 16 bf16.
-__device__ __forceinline__ void dot16_q2(uint32_t w, const uint4& xa, const uint4& xb,
-                                         float& dot, float& sum) {
-  // plane p, byte i = code of element 4i + p
-  const uint32_t p0 = w & 0x03030303u;
-  const uint32_t p1 = (w >> 2) & 0x03030303u;
-  const uint32_t p2 = (w >> 4) & 0x03030303u;
-  const uint32_t p3 = (w >> 6) & 0x03030303u;
-  const uint32_t xs[8] = {xa.x, xa.y, xa.z, xa.w, xb.x, xb.y, xb.z, xb.w};
-#pragma unroll
-  for (int i = 0; i < 4; ++i) {  // byte i covers elements 4i..4i+3 = pairs 2i, 2i+1
-    const float x0 = bf16_lo(xs[2 * i]), x1 = bf16_hi(xs[2 * i]);
-    const float x2 = bf16_lo(xs[2 * i + 1]), x3 = bf16_hi(xs[2 * i + 1]);
-    dot = __builtin_fmaf(ubyte_f(p0, i), x0, dot);
-    dot = __builtin_fmaf(ubyte_f(p1, i), x1, dot);
-    dot = __builtin_fmaf(ubyte_f(p2, i), x2, dot);
-    dot = __builtin_fmaf(ubyte_f(p3, i), x3, dot);
-    sum += (x0 + x1) + (x2 + x3);
-  }
-}
+// The activations one lane meets, permuted for the pairing above, plus their sum.
+template <int BITS> struct XSlice {
+  static constexpr int kPairs = Fmt<BITS>::kElemsPer16B / 2;
+  uint32_t p[kPairs];
+  float sum;
+};
 
-// One lane's share of a row: 16 bytes of codes (32 four-bit or 64 two-bit
-// elements, never straddling a 64-group for 4-bit: a lane covers half a
-// group; exactly one group for 2-bit) against the matching slice of x.
-template <int BITS, bool ALIGNED>
-__device__ __forceinline__ void lane_dot(const uint4& codes, const uint16_t* x, float& dot,
-                                         float& sum) {
-  dot = 0.0f;
-  sum = 0.0f;
-  if constexpr (BITS == kBits4) {
-    dot8_q4(codes.x, load_x8<ALIGNED>(x), dot, sum);
-    dot8_q4(codes.y, load_x8<ALIGNED>(x + 8), dot, sum);
-    dot8_q4(codes.z, load_x8<ALIGNED>(x + 16), dot, sum);
-    dot8_q4(codes.w, load_x8<ALIGNED>(x + 24), dot, sum);
-  } else {
-    dot16_q2(codes.x, load_x8<ALIGNED>(x), load_x8<ALIGNED>(x + 8), dot, sum);
-    dot16_q2(codes.y, load_x8<ALIGNED>(x + 16), load_x8<ALIGNED>(x + 24), dot, sum);
-    dot16_q2(codes.z, load_x8<ALIGNED>(x + 32), load_x8<ALIGNED>(x + 40), dot, sum);
-    dot16_q2(codes.w, load_x8<ALIGNED>(x + 48), load_x8<ALIGNED>(x + 56), dot, sum);
-  }
-}
-
-// Same with the code part only (x already turned into fp32 by the caller,
-// `xf` holds kElemsPer16B values): used when one x slice meets many rows.
+// raw: consecutive bf16 pairs (x0,x1),(x2,x3),... of the lane's slice
 template <int BITS>
-__device__ __forceinline__ float lane_dot_xf(const uint4& codes, const float* xf) {
-  float dot = 0.0f;
+__device__ __forceinline__ void permute_x(const uint32_t* raw, XSlice<BITS>& xs) {
+  float sum = 0.0f;
+#pragma unroll
+  for (int i = 0; i < XSlice<BITS>::kPairs; ++i) sum = dot2_bf16(raw[i], kOnes, sum);
+  xs.sum = sum;
+  if constexpr (BITS == kBits4) {
+    // per packed word: 8 elements = raw pairs r0..r3 -> (x0,x4),(x1,x5),(x2,x6),(x3,x7)
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const uint32_t r0 = raw[4 * j], r1 = raw[4 * j + 1], r2 = raw[4 * j + 2], r3 = raw[4 * j + 3];
+      xs.p[4 * j + 0] = __builtin_amdgcn_perm(r2, r0, 0x05040100u);
+      xs.p[4 * j + 1] = __builtin_amdgcn_perm(r2, r0, 0x07060302u);
+      xs.p[4 * j + 2] = __builtin_amdgcn_perm(r3, r1, 0x05040100u);
+      xs.p[4 * j + 3] = __builtin_amdgcn_perm(r3, r1, 0x07060302u);
+    }
+  } else {
+    // per packed word: 16 elements = raw pairs r0..r7 -> (x_i, x_{i+8}), i = 0..7
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const uint32_t lo = raw[8 * j + i], hi = raw[8 * j + 4 + i];
+        xs.p[8 * j + 2 * i] = __builtin_amdgcn_perm(hi, lo, 0x05040100u);
+        xs.p[8 * j + 2 * i + 1] = __builtin_amdgcn_perm(hi, lo, 0x07060302u);
+      }
+    }
+  }
+}
+
+enum XLoad : int { kXAligned = 0, kXUnaligned = 1, kXAgent = 2 };
+
+// loads and permutes the lane's slice of x starting at element pointer x
+template <int BITS, int MODE>
+__device__ __forceinline__ XSlice<BITS> load_xslice(const uint16_t* x) {
+  constexpr int kQuads = Fmt<BITS>::kElemsPer16B / 8;
+  uint32_t raw[kQuads * 4];
+  if constexpr (MODE == kXAgent) {
+#pragma unroll
+    for (int q = 0; q < kQuads; q += 4) {
+      uint4 a[4];
+      load_x32_agent(x + 8 * q, a);
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        raw[4 * (q + i)] = a[i].x; raw[4 * (q + i) + 1] = a[i].y;
+        raw[4 * (q + i) + 2] = a[i].z; raw[4 * (q + i) + 3] = a[i].w;
+      }
+    }
+  } else {
+#pragma unroll
+    for (int q = 0; q < kQuads; ++q) {
+      const uint4 a = load_x8<MODE == kXAligned>(x + 8 * q);
+      raw[4 * q] = a.x; raw[4 * q + 1] = a.y; raw[4 * q + 2] = a.z; raw[4 * q + 3] = a.w;
+    }
+  }
+  XSlice<BITS> xs;
+  permute_x<BITS>(raw, xs);
+  return xs;
+}
+
+// sum over the lane's share of q * x
+template <int BITS>
+__device__ __forceinline__ float codes_dot(const uint4& codes, const XSlice<BITS>& xs) {
   const uint32_t ws[4] = {codes.x, codes.y, codes.z, codes.w};
+  float dot = 0.0f;
   if constexpr (BITS == kBits4) {
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
-      const uint32_t lo = ws[j] & 0x0F0F0F0Fu, hi = (ws[j] >> 4) & 0x0F0F0F0Fu;
-#pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        dot = __builtin_fmaf(ubyte_f(lo, i), xf[8 * j + 2 * i], dot);
-        dot = __builtin_fmaf(ubyte_f(hi, i), xf[8 * j + 2 * i + 1], dot);
-      }
+      const uint32_t w = ws[j];
+      dot = dot2_bf16((w & 0x000F000Fu) | kMagic128, xs.p[4 * j + 0], dot);
+      dot = dot2_bf16(((w >> 4) & 0x000F000Fu) | kMagic128, xs.p[4 * j + 1], dot);
+      dot = dot2_bf16(((w >> 8) & 0x000F000Fu) | kMagic128, xs.p[4 * j + 2], dot);
+      dot = dot2_bf16(((w >> 12) & 0x000F000Fu) | kMagic128, xs.p[4 * j + 3], dot);
     }
   } else {
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
       const uint32_t w = ws[j];
-      const uint32_t p0 = w & 0x03030303u, p1 = (w >> 2) & 0x03030303u;
-      const uint32_t p2 = (w >> 4) & 0x03030303u, p3 = (w >> 6) & 0x03030303u;
 #pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        dot = __builtin_fmaf(ubyte_f(p0, i), xf[16 * j + 4 * i], dot);
-        dot = __builtin_fmaf(ubyte_f(p1, i), xf[16 * j + 4 * i + 1], dot);
-        dot = __builtin_fmaf(ubyte_f(p2, i), xf[16 * j + 4 * i + 2], dot);
-        dot = __builtin_fmaf(ubyte_f(p3, i), xf[16 * j + 4 * i + 3], dot);
-      }
+      for (int i = 0; i < 8; ++i)
+        dot = dot2_bf16(((w >> (2 * i)) & 0x00030003u) | kMagic128, xs.p[8 * j + i], dot);
     }
   }
-  return dot;
+  return __builtin_fmaf(-128.0f, xs.sum, dot);
+}
+
+// convenience form: one row against a slice loaded on the spot
+template <int BITS, bool ALIGNED>
+__device__ __forceinline__ void lane_dot(const uint4& codes, const uint16_t* x, float& dot,
+                                         float& sum) {
+  const XSlice<BITS> xs = load_xslice<BITS, ALIGNED ? kXAligned : kXUnaligned>(x);
+  dot = codes_dot<BITS>(codes, xs);
+  sum = xs.sum;
 }
 
 // scale / bias of the group that holds element e0 of a row whose tables start
@@ -219,19 +333,5 @@ __device__ __forceinline__ void load_scale_bias(const uint16_t* srow, const uint
   if constexpr (BITS == kBitsTernary) b = -s;
   else b = bf16_to_f(brow[g]);
 }
-
-// lanes of a wave that share one row of n elements (power of two, <= 64)
-__host__ __device__ __forceinline__ uint32_t lanes_per_row_log2_dev(uint32_t n, uint32_t elems_per_lane) {
-  const uint32_t need = (n + elems_per_lane - 1) / elems_per_lane;
-  uint32_t l = 0;
-  while ((1u << l) < need && l < 6) ++l;
-  return l;
-}
-
-// storage width of a format in bits per element
-template <int BITS> struct Store { static constexpr int kBits = (BITS == kBits4) ? 4 : 2; };
-
-// the dot-product flavour of a format (ternary shares the 2-bit unpack)
-template <int BITS> struct DotBits { static constexpr int k = (BITS == kBits4) ? kBits4 : kBits2; };
 
 }  // namespace mf

@@ -22,7 +22,7 @@ struct mf_moe_workspace {
   uint16_t* acts;       // [MF_MAX_TOKENS, top_k, f]
   uint16_t* shared_act; // [MF_MAX_TOKENS, shared_f]
   uint16_t* shared_y;   // [MF_MAX_TOKENS, d]
-  uint16_t* gate;       // [MF_MAX_TOKENS]
+  uint16_t* gate;       // [MF_MAX_TOKENS] (x2: the fused kernel keeps fp32 there)
   uint32_t* sync;       // grid-sync counters of the fused kernel
 };
 
@@ -30,6 +30,7 @@ struct mf_moe {
   mf_ctx* ctx = nullptr;
   mf_moe_config cfg{};
   bool fused = true;  // mf_moe_set_fused
+  unsigned long long* trace = nullptr;  // mf_moe_set_phase_trace
   void* ws_base = nullptr;
   size_t ws_bytes = 0;
   mf_moe_workspace ws{};

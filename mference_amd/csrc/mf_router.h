@@ -13,7 +13,7 @@ namespace mf {
 // One wave per (token, expert) row.  Elements are split into 8-wide chunks;
 // chunk c belongs to lane c % 64; a lane accumulates its elements in ascending
 // order with fmaf into one fp32 accumulator; lanes are combined by an xor
-// butterfly with strides 32..1.  Replaces router_gemv_bf16_r4
+// butterfly with strides 1..32 (neighbours first).  Replaces router_gemv_bf16_r4
 // (moe.metal:162-185) / maple_router_bf16_gemv (maple_moe.metal:25-60).
 __device__ __forceinline__ float dot_bf16_row(const uint16_t* __restrict__ w,
                                               const uint16_t* __restrict__ x, uint32_t d,
@@ -58,7 +58,8 @@ __device__ __forceinline__ void wave_argmax(float& bv, uint32_t& bi) {
   }
 }
 
-// One wave per token (all 64 lanes call it; idx / w may be LDS or global).  Lane l owns experts l, l+64, ...  (ownership does not
+// One wave per token (all 64 lanes call it; idx / w may be LDS or global;
+// AGENT_LOGITS: the logits were written by other workgroups of this launch).  Lane l owns experts l, l+64, ...  (ownership does not
 // change the result: every step picks the highest score, lowest index first).
 //
 // mode 0 = router_topk_select_k8 (moe.metal:190-240) for any k <= 8: k rounds of
@@ -68,6 +69,7 @@ __device__ __forceinline__ void wave_argmax(float& bv, uint32_t& bi) {
 //   non-finite logit -> idx = e, w = 0; softmax over all experts with the
 //   32-wide tree sums added block by block, k rounds of argmax on the
 //   probabilities, renormalise with the 1e-20 guards.
+template <bool AGENT_LOGITS = false>
 __device__ __forceinline__ void topk_wave(const float* lg, uint32_t e, uint32_t k, int mode,
                                           uint32_t* idx, float* w, uint32_t lane) {
   const uint32_t per = (e + kWave - 1) / kWave;
@@ -75,7 +77,8 @@ __device__ __forceinline__ void topk_wave(const float* lg, uint32_t e, uint32_t 
 #pragma unroll
   for (int j = 0; j < kMaxPerLane; ++j) {
     const uint32_t x = lane + j * kWave;
-    ch[j] = (static_cast<uint32_t>(j) < per && x < e) ? lg[x] : -__builtin_inff();
+    ch[j] = -__builtin_inff();
+    if (static_cast<uint32_t>(j) < per && x < e) ch[j] = AGENT_LOGITS ? load_f32_agent(lg + x) : lg[x];
   }
   float top_s[MF_MAX_TOPK];
   uint32_t top_i[MF_MAX_TOPK];
@@ -191,6 +194,67 @@ __device__ __forceinline__ void topk_wave(const float* lg, uint32_t e, uint32_t 
       idx[i] = top_i[i];
       w[i] = wt[i];
     }
+  }
+}
+
+// mode 0 selector, all-register form: lane l owns the `per` consecutive experts
+// from l*per (the blocked ownership of router_topk_select_k8_par,
+// moe.metal:262-345).  Each of the k rounds takes the wave maximum of the
+// lanes' best unretired score; among the lanes that hold it the lowest lane --
+// and inside a lane the lowest index -- wins, which is the serial kernel's
+// "strictly greater wins, equal score keeps the earlier expert".  NaN and -inf
+// are never selected; a round without a winner gives index 0, score -inf.
+// Rank r's result lives in lane r; weights are exp(s_r - s_0) / sum with the sum
+// taken in rank order.  All 64 lanes call it.
+__device__ __forceinline__ void topk_select_fast(const float* lg, uint32_t e, uint32_t k,
+                                                 uint32_t* idx, float* w, uint32_t lane) {
+  const uint32_t per = (e + kWave - 1) / kWave;
+  const uint32_t base = lane * per;
+  float ch[kMaxPerLane];
+#pragma unroll
+  for (int j = 0; j < kMaxPerLane; ++j) {
+    ch[j] = -__builtin_inff();
+    if (static_cast<uint32_t>(j) < per && base + j < e) ch[j] = lg[base + j];
+  }
+  uint32_t taken = 0;
+  float my_score = -__builtin_inff();
+  uint32_t my_idx = 0;
+  for (uint32_t r = 0; r < k; ++r) {
+    float bv = -__builtin_inff();
+    int bj = -1;
+#pragma unroll
+    for (int j = 0; j < kMaxPerLane; ++j) {
+      if (!(taken & (1u << j)) && ch[j] > bv) {
+        bv = ch[j];
+        bj = j;
+      }
+    }
+    const float m = wave_max(bv);
+    const bool cand = bj >= 0 && bv == m;
+    const unsigned long long mask = __ballot(cand);
+    uint32_t widx = 0;
+    float ws = -__builtin_inff();
+    if (mask != 0) {
+      const int wl = __ffsll(static_cast<long long>(mask)) - 1;
+      widx = static_cast<uint32_t>(
+          __builtin_amdgcn_readlane(static_cast<int>(base + static_cast<uint32_t>(bj < 0 ? 0 : bj)), wl));
+      ws = m;
+      if (static_cast<int>(lane) == wl) taken |= 1u << bj;
+    }
+    if (lane == r) {
+      my_score = ws;
+      my_idx = widx;
+    }
+  }
+  const float s0 = readlane_f(my_score, 0);
+  const float my_e = mf_exp(my_score - s0);
+  float sum = 0.0f;
+#pragma unroll
+  for (int i = 0; i < MF_MAX_TOPK; ++i)
+    if (static_cast<uint32_t>(i) < k) sum += readlane_f(my_e, i);
+  if (lane < k) {
+    idx[lane] = my_idx;
+    w[lane] = my_e / sum;
   }
 }
 

@@ -21,6 +21,7 @@
 // launcher never asks for more workgroups than CUs and the kernel needs a whole
 // CU (1024 threads, <= 128 VGPRs).  Waits are bounded: a barrier that does not
 // complete within kSpinLimit polls sets the status word and lets the grid drain.
+// (The logits buffer is read 16 bytes at a time: [T, E] fp32 with E % 4 == 0.)
 #include "mf_device.h"
 #include "mf_internal.h"
 #include "mf_router.h"
@@ -48,8 +49,9 @@ __device__ __forceinline__ Chunk<BITS> load_chunk(const uint8_t* wrow, const uin
 }
 
 // lane partial of one row of N elements against x (16-byte aligned bf16);
-// `first` may carry the already loaded chunk of the first step.
-template <int BITS>
+// `first` may carry the already loaded chunk of the first step.  AGENT_X: x was
+// written by other workgroups during this launch.
+template <int BITS, bool AGENT_X>
 __device__ __forceinline__ float row_partial(const uint8_t* wrow, const uint16_t* srow,
                                              const uint16_t* brow, const uint16_t* x, uint32_t N,
                                              uint32_t sub, uint32_t lpr, bool have_first,
@@ -60,7 +62,9 @@ __device__ __forceinline__ float row_partial(const uint8_t* wrow, const uint16_t
     const Chunk<BITS> c = (have_first && e0 == sub * EPL) ? first
                                                            : load_chunk<BITS>(wrow, srow, brow, e0);
     float dot, sum;
-    lane_dot<BITS, true>(c.codes, x + e0, dot, sum);
+    const XSlice<BITS> xs = load_xslice<BITS, AGENT_X ? kXAgent : kXAligned>(x + e0);
+    dot = codes_dot<BITS>(c.codes, xs);
+    sum = xs.sum;
     acc = __builtin_fmaf(c.s, dot, acc);
     acc = __builtin_fmaf(c.b, sum, acc);
   }
@@ -79,9 +83,9 @@ __device__ __forceinline__ void gate_up_partial(const uint8_t* gw, const uint16_
   for (uint32_t e0 = sub * EPL; e0 < N; e0 += lpr * EPL) {
     const Chunk<BITS> g = load_chunk<BITS>(gw, gs, gb, e0);
     const Chunk<BITS> u = load_chunk<BITS>(uw, us, ub, e0);
-    float gd, ud, sum, sum2;
-    lane_dot<BITS, true>(g.codes, x + e0, gd, sum);
-    lane_dot<BITS, true>(u.codes, x + e0, ud, sum2);
+    const XSlice<BITS> xs = load_xslice<BITS, kXAligned>(x + e0);
+    const float gd = codes_dot<BITS>(g.codes, xs), ud = codes_dot<BITS>(u.codes, xs);
+    const float sum = xs.sum;
     ga = __builtin_fmaf(g.s, gd, ga);
     ga = __builtin_fmaf(g.b, sum, ga);
     ua = __builtin_fmaf(u.s, ud, ua);
@@ -105,33 +109,59 @@ struct FusedArgs {
   uint16_t* acts;
   uint16_t* shared_act;
   uint16_t* shared_y;
-  uint16_t* gate;
-  uint32_t* sync;  // [0] barrier 1, [1] barrier 2, [2] finished workgroups, [3] status
+  float* gate;  // bf16-rounded scalar shared gate per token
+  unsigned long long* trace;  // phase timestamps, 8 per workgroup, or nullptr
+  uint32_t* sync;  // kMaxGrid flags of barrier 1, kMaxGrid of barrier 2, status word
   uint32_t D, F, E, K, T, Fs;
   int router_mode;
   float limit;
 };
 
-__device__ __forceinline__ void grid_arrive(uint32_t* ctr) {
-  __threadfence();
+// Grid barrier without read-modify-write atomics (256 workgroups adding to one
+// counter serialise at the memory side for microseconds): every workgroup owns
+// one flag per barrier and raises it by one each time it arrives; a waiter
+// polls all flags with one 16-byte device-coherent load per lane until none
+// lags behind its own.  Flags only ever count up, so nothing has to be reset
+// between launches (HIP-graph replay safe).  Exchanged data is written with
+// device-coherent stores that are acknowledged before the flag is raised.
+constexpr uint32_t kMaxGrid = 512;  // flags per barrier
+constexpr uint32_t kSyncFlags1 = 0, kSyncFlags2 = kMaxGrid, kSyncStatus = 2 * kMaxGrid;
+
+__device__ __forceinline__ void grid_arrive(uint32_t* flags, uint32_t target) {
+  wait_stores();
   __syncthreads();
-  if (threadIdx.x == 0)
-    __hip_atomic_fetch_add(ctr, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  if (threadIdx.x == 0) store_u32_agent(&flags[blockIdx.x], target);
 }
 
-__device__ __forceinline__ void grid_wait(uint32_t* ctr, uint32_t target, uint32_t* status) {
-  if (threadIdx.x == 0) {
+__device__ __forceinline__ void grid_wait(const uint32_t* flags, uint32_t target, uint32_t G,
+                                          uint32_t* status) {
+  if (threadIdx.x < kWave) {
+    const uint32_t lane = threadIdx.x;
     uint32_t spins = 0;
-    while (__hip_atomic_load(ctr, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) < target) {
-      __builtin_amdgcn_s_sleep(2);
+    for (;;) {
+      bool ok = true;
+      for (uint32_t b = 0; b < G; b += 4 * kWave) {
+        const uint32_t i = b + 4 * lane;
+        const uint4 f = load_u32x4_agent(flags + i);
+        ok = ok && (i + 0 >= G || static_cast<int32_t>(f.x - target) >= 0) &&
+             (i + 1 >= G || static_cast<int32_t>(f.y - target) >= 0) &&
+             (i + 2 >= G || static_cast<int32_t>(f.z - target) >= 0) &&
+             (i + 3 >= G || static_cast<int32_t>(f.w - target) >= 0);
+      }
+      if (__all(ok)) break;
+      __builtin_amdgcn_s_sleep(1);
       if (++spins > kSpinLimit) {
-        __hip_atomic_store(status, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        if (lane == 0) store_u32_agent(status, 1u);
         break;
       }
     }
   }
   __syncthreads();
-  __threadfence();
+}
+
+// phase trace: the shader clock at every stage boundary, thread 0 of each workgroup
+__device__ __forceinline__ void trace_mark(const FusedArgs& a, uint32_t slot) {
+  if (a.trace && threadIdx.x == 0) a.trace[blockIdx.x * 8 + slot] = wall_clock64();
 }
 
 template <int BITS, int SBITS>
@@ -139,6 +169,7 @@ __global__ __launch_bounds__(kFusedThreads) void fused_decode_kernel(const Fused
   __shared__ uint32_t s_idx[MF_MAX_TOKENS * MF_MAX_TOPK];
   __shared__ float s_w[MF_MAX_TOKENS * MF_MAX_TOPK];
   __shared__ float s_v[kFusedWaves][kWave];
+  __shared__ float s_lg[MF_MAX_TOKENS][MF_MAX_EXPERTS];
 
   const uint32_t lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
   const uint32_t G = gridDim.x, wg = blockIdx.x;
@@ -146,6 +177,12 @@ __global__ __launch_bounds__(kFusedThreads) void fused_decode_kernel(const Fused
   const uint32_t total_waves = kFusedWaves * G;
   const uint32_t D = a.D, F = a.F, E = a.E, K = a.K, T = a.T, Fs = a.Fs;
 
+  // this launch's barrier targets: one above the workgroup's own flags
+  const uint32_t target1 =
+      __hip_atomic_load(&a.sync[kSyncFlags1 + wg], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) + 1u;
+  const uint32_t target2 =
+      __hip_atomic_load(&a.sync[kSyncFlags2 + wg], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) + 1u;
+  trace_mark(a, 0);
   // ------------------------------------------------------------- stage A
   {
     const uint32_t lpr_log2 = Fs ? lanes_per_row_log2_dev(D, Fmt<SBITS>::kElemsPer16B) : 0;
@@ -159,11 +196,11 @@ __global__ __launch_bounds__(kFusedThreads) void fused_decode_kernel(const Fused
         const uint32_t tok = item / E, row = item % E;
         const float v = dot_bf16_row(a.router_w + static_cast<size_t>(row) * D,
                                      a.x + static_cast<size_t>(tok) * D, D, lane, true);
-        if (lane == 0) a.logits[item] = v;
+        if (lane == 0) store_f32_agent(&a.logits[item], v);
       } else if (item < n_router + n_gate) {
         const uint32_t tok = item - n_router;
         const float v = dot_bf16_row(a.w_sg, a.x + static_cast<size_t>(tok) * D, D, lane, true);
-        if (lane == 0) a.gate[tok] = f_to_bf16(v);
+        if (lane == 0) store_f32_agent(&a.gate[tok], round_bf16(v));
       } else {
         const uint32_t it = item - n_router - n_gate;
         const uint32_t tok = it / srg;
@@ -185,18 +222,31 @@ __global__ __launch_bounds__(kFusedThreads) void fused_decode_kernel(const Fused
         if (ok && sub == 0) {
           // dequant_int4.metal:240-245: gate and up narrowed before the activation
           const float rg = round_bf16(g), ru = round_bf16(u);
-          a.shared_act[static_cast<size_t>(tok) * Fs + row] = f_to_bf16(mf_silu(rg) * ru);
+          store_u16_agent(&a.shared_act[static_cast<size_t>(tok) * Fs + row],
+                          f_to_bf16(mf_silu(rg) * ru));
         }
       }
     }
   }
-  grid_arrive(&a.sync[0]);
-  grid_wait(&a.sync[0], G, &a.sync[3]);
+  trace_mark(a, 1);
+  grid_arrive(a.sync + kSyncFlags1, target1);
+  grid_wait(a.sync + kSyncFlags1, target1, G, a.sync + kSyncStatus);
+  trace_mark(a, 2);
 
   // ------------------------------------------------------------- top-k
+  if (wv < T) {  // stage the token's logits in LDS: 4 consecutive experts per lane and load
+    for (uint32_t e0 = 4 * lane; e0 < E; e0 += 4 * kWave) {
+      const uint4 v = load_u32x4_agent(a.logits + static_cast<size_t>(wv) * E + e0);
+      s_lg[wv][e0] = __uint_as_float(v.x);
+      if (e0 + 1 < E) s_lg[wv][e0 + 1] = __uint_as_float(v.y);
+      if (e0 + 2 < E) s_lg[wv][e0 + 2] = __uint_as_float(v.z);
+      if (e0 + 3 < E) s_lg[wv][e0 + 3] = __uint_as_float(v.w);
+    }
+  }
+  __syncthreads();
   if (wv < T) {
-    topk_wave(a.logits + static_cast<size_t>(wv) * E, E, K, a.router_mode, s_idx + wv * K,
-              s_w + wv * K, lane);
+    if (a.router_mode == 0) topk_select_fast(s_lg[wv], E, K, s_idx + wv * K, s_w + wv * K, lane);
+    else topk_wave(s_lg[wv], E, K, a.router_mode, s_idx + wv * K, s_w + wv * K, lane);
   }
   __syncthreads();
   if (wg == 0 && threadIdx.x < T * K) {
@@ -204,6 +254,7 @@ __global__ __launch_bounds__(kFusedThreads) void fused_decode_kernel(const Fused
     if (a.out_w) a.out_w[threadIdx.x] = s_w[threadIdx.x];
   }
 
+  trace_mark(a, 3);
   // ------------------------------------------------------------- stage B
   {
     const uint32_t lpr_log2 = lanes_per_row_log2_dev(D, Fmt<BITS>::kElemsPer16B);
@@ -222,7 +273,7 @@ __global__ __launch_bounds__(kFusedThreads) void fused_decode_kernel(const Fused
         const bool ok = row < F;
         const uint32_t expert = s_idx[pair];
         if (expert >= E) {
-          if (ok && sub == 0) a.acts[static_cast<size_t>(pair) * F + row] = 0;
+          if (ok && sub == 0) store_u16_agent(&a.acts[static_cast<size_t>(pair) * F + row], 0);
           continue;
         }
         const uint8_t* blob = a.expert_base + static_cast<size_t>(expert) * a.expert_stride;
@@ -246,7 +297,7 @@ __global__ __launch_bounds__(kFusedThreads) void fused_decode_kernel(const Fused
             g = fminf(g, a.limit);
             u = fminf(fmaxf(u, -a.limit), a.limit);
           }
-          a.acts[static_cast<size_t>(pair) * F + row] = f_to_bf16(mf_silu(g) * u);
+          store_u16_agent(&a.acts[static_cast<size_t>(pair) * F + row], f_to_bf16(mf_silu(g) * u));
         }
       } else {
         const uint32_t it = item - n_routed;
@@ -259,7 +310,7 @@ __global__ __launch_bounds__(kFusedThreads) void fused_decode_kernel(const Fused
         const size_t rb = static_cast<size_t>(Fs) * Store<SBITS>::kBits / 8;
         float part = 0.0f;
         if (ok)
-          part = row_partial<SBITS>(static_cast<const uint8_t*>(a.sd.weights) + r * rb,
+          part = row_partial<SBITS, true>(static_cast<const uint8_t*>(a.sd.weights) + r * rb,
                                     a.sd.scales + r * ng, a.sd.biases + r * ng,
                                     a.shared_act + static_cast<size_t>(tok) * Fs, Fs, sub, slpr,
                                     false, Chunk<SBITS>{});
@@ -267,10 +318,10 @@ __global__ __launch_bounds__(kFusedThreads) void fused_decode_kernel(const Fused
         if (ok && sub == 0) {
           uint16_t h = f_to_bf16(v);  // dequant_int4.metal:177-180
           if (a.w_sg) {               // utility.metal:49-59
-            const float gt = bf16_to_f(a.gate[tok]);
+            const float gt = load_f32_agent(&a.gate[tok]);
             h = f_to_bf16(bf16_to_f(h) / (1.0f + mf_exp(-gt)));
           }
-          a.shared_y[static_cast<size_t>(tok) * D + row] = h;
+          store_u16_agent(&a.shared_y[static_cast<size_t>(tok) * D + row], h);
         }
       }
     }
@@ -288,7 +339,8 @@ __global__ __launch_bounds__(kFusedThreads) void fused_decode_kernel(const Fused
   const uint32_t ng = F / kGroup;
   const size_t rb = static_cast<size_t>(F) * Store<BITS>::kBits / 8;
 
-  grid_arrive(&a.sync[1]);
+  trace_mark(a, 4);
+  grid_arrive(a.sync + kSyncFlags2, target2);
   // request round 0's codes while the barrier completes
   Chunk<BITS> pre{};
   bool have_pre = false;
@@ -308,7 +360,8 @@ __global__ __launch_bounds__(kFusedThreads) void fused_decode_kernel(const Fused
       }
     }
   }
-  grid_wait(&a.sync[1], G, &a.sync[3]);
+  grid_wait(a.sync + kSyncFlags2, target2, G, a.sync + kSyncStatus);
+  trace_mark(a, 5);
 
   for (uint32_t round = 0; round < rounds; ++round) {
     const uint32_t unit = (round * G + wg) * ub + unit_local;
@@ -322,7 +375,7 @@ __global__ __launch_bounds__(kFusedThreads) void fused_decode_kernel(const Fused
       float part = 0.0f;
       if (ok && expert < E) {
         const uint8_t* blob = a.expert_base + static_cast<size_t>(expert) * a.expert_stride;
-        part = row_partial<BITS>(blob + a.off.down_w + row * rb,
+        part = row_partial<BITS, true>(blob + a.off.down_w + row * rb,
                                  reinterpret_cast<const uint16_t*>(blob + a.off.down_s) + row * ng,
                                  reinterpret_cast<const uint16_t*>(blob + a.off.down_b) + row * ng,
                                  a.acts + static_cast<size_t>(pair) * F, F, sub, lpr,
@@ -340,7 +393,7 @@ __global__ __launch_bounds__(kFusedThreads) void fused_decode_kernel(const Fused
         const uint32_t row = (u2 % rg_per_tok) * rpw + rr;
         if (row < D) {
           const size_t o = static_cast<size_t>(tok) * D + row;
-          float acc = Fs ? bf16_to_f(a.shared_y[o]) : 0.0f;  // residual first (moe.metal:1265)
+          float acc = Fs ? bf16_to_f(load_u16_agent(&a.shared_y[o])) : 0.0f;  // residual first (moe.metal:1265)
           for (uint32_t k = 0; k < K; ++k)
             if (s_idx[tok * K + k] < E) acc = acc + s_v[ul * K + k][rr];
           const uint16_t yb = f_to_bf16(acc);
@@ -353,21 +406,12 @@ __global__ __launch_bounds__(kFusedThreads) void fused_decode_kernel(const Fused
     __syncthreads();
   }
 
-  // the last workgroup to finish re-arms the barrier counters for the next launch
-  __syncthreads();
-  if (threadIdx.x == 0) {
-    const uint32_t done = __hip_atomic_fetch_add(&a.sync[2], 1u, __ATOMIC_RELAXED,
-                                                 __HIP_MEMORY_SCOPE_AGENT);
-    if (done == G - 1) {
-      __hip_atomic_store(&a.sync[0], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-      __hip_atomic_store(&a.sync[1], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-      __hip_atomic_store(&a.sync[2], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    }
-  }
+  trace_mark(a, 6);
 }
 
 bool fused_supported(const mf_moe_config& c, const mf_moe_layer_weights& w, const void* x,
                      const void* y, const void* hidden) {
+  if (c.num_experts % 4 != 0) return false;  // logits are staged 4 at a time
   const bool combo = (c.bits == MF_BITS_4 && (!c.shared_f || c.shared_bits == MF_BITS_4)) ||
                      (c.bits == MF_BITS_2 && (!c.shared_f || c.shared_bits == MF_BITS_4 ||
                                               c.shared_bits == MF_BITS_2)) ||
@@ -408,8 +452,9 @@ hipError_t launch_fused_decode(hipStream_t s, const mf_moe& h, const mf_moe_laye
   a.acts = h.ws.acts;
   a.shared_act = h.ws.shared_act;
   a.shared_y = h.ws.shared_y;
-  a.gate = h.ws.gate;
+  a.gate = reinterpret_cast<float*>(h.ws.gate);
   a.sync = h.ws.sync;
+  a.trace = h.trace;
   a.D = c.d;
   a.F = c.f;
   a.E = c.num_experts;

@@ -34,8 +34,12 @@ __global__ __launch_bounds__(64) void topk_kernel(const float* __restrict__ logi
                                                   uint32_t* __restrict__ idx,
                                                   float* __restrict__ w) {
   const uint32_t tok = blockIdx.x;
-  topk_wave(logits + static_cast<size_t>(tok) * e, e, k, mode, idx + static_cast<size_t>(tok) * k,
-            w + static_cast<size_t>(tok) * k, threadIdx.x);
+  if (mode == 0)
+    topk_select_fast(logits + static_cast<size_t>(tok) * e, e, k, idx + static_cast<size_t>(tok) * k,
+                     w + static_cast<size_t>(tok) * k, threadIdx.x);
+  else
+    topk_wave(logits + static_cast<size_t>(tok) * e, e, k, mode, idx + static_cast<size_t>(tok) * k,
+              w + static_cast<size_t>(tok) * k, threadIdx.x);
 }
 
 hipError_t launch_router_logits(hipStream_t s, const uint16_t* w, const uint16_t* x, uint32_t e,

@@ -244,6 +244,13 @@ class MoE:
         """single fused launch (default) or the chain of separate launches"""
         check(_capi.lib().mf_moe_set_fused(self._h, 1 if enabled else 0), self.context.handle)
 
+    def set_phase_trace(self, buffer: Optional[torch.Tensor]) -> None:
+        """int64 device tensor of num_cu*8 entries receiving per-workgroup stage
+        timestamps of the fused launch (100 MHz clock); None switches it off"""
+        check(_capi.lib().mf_moe_set_phase_trace(
+            self._h, _ptr(buffer), 0 if buffer is None else buffer.numel() * 8),
+            self.context.handle)
+
     def status(self, stream=None) -> None:
         """synchronises and raises if a fused launch gave up on a grid barrier"""
         check(_capi.lib().mf_moe_status(self._h, _stream(stream)), self.context.handle)

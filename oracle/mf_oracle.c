@@ -295,7 +295,7 @@ float mfo_exp(float x) {
  * bit: elements are split into 8-wide chunks; chunk c belongs to lane c % 64;
  * each lane accumulates its elements in ascending order with fmaf into one
  * fp32 accumulator; the 64 lane sums are combined by an xor butterfly with
- * strides 32,16,8,4,2,1 (p[l] = p[l] + p[l^s]).  The reference's order is one
+ * strides 1,2,4,8,16,32 (p[l] = p[l] + p[l^s]): neighbours first.  The reference's order is one
  * Metal SIMD's (moe.metal:162-185); only a fixed order is needed, because the
  * reference itself compares logits under tolerances. */
 float mfo_dot_bf16_laneorder(const uint16_t* w, const uint16_t* x, size_t d) {
@@ -309,7 +309,7 @@ float mfo_dot_bf16_laneorder(const uint16_t* w, const uint16_t* x, size_t d) {
       acc = fmaf(mfo_bf16_to_float(w[c * 8 + j]), mfo_bf16_to_float(x[c * 8 + j]), acc);
     p[l] = acc;
   }
-  for (int s = 32; s >= 1; s >>= 1) {
+  for (int s = 1; s <= 32; s <<= 1) {
     float q[64];
     for (int l = 0; l < 64; ++l) q[l] = p[l] + p[l ^ s];
     memcpy(p, q, sizeof p);

@@ -170,6 +170,8 @@ typedef struct {
   mf_bits shared_bits;
 } mf_moe_config;
 
+/* MoE.init (Kernels/MoE/MoE.swift:65-151): one operator instance per shape; owns the
+ * router-logit and activation workspace (MoE.swift:136-150). */
 mf_status mf_moe_create(mf_ctx* ctx, const mf_moe_config* cfg, mf_moe** out);
 void mf_moe_destroy(mf_moe* h);
 
@@ -237,15 +239,15 @@ mf_status mf_moe_set_fused(mf_moe* h, int enabled);
 
 /* Phase trace of the fused launch: when device_buffer is not NULL every
  * workgroup writes the 100 MHz wall clock at its stage boundaries (slots:
- * 0 start, 1 stage A done, 2 barrier 1 passed, 3 top-k done, 4 stage B done,
- * 5 barrier 2 passed, 6 end) to device_buffer[workgroup*8 + slot]; needs
+ * 0 start, 1 stage A done, 2 logits gathered, 3 top-k done, 4 stage B done,
+ * 5 routed activations gathered, 6 end) to device_buffer[workgroup*8 + slot]; needs
  * mf_ctx_num_cu()*8*8 bytes.  The counterpart of the reference's
  * MFERENCE_PHASES=1 phase counters (RealForwardRunner.swift:397-398). */
 mf_status mf_moe_set_phase_trace(mf_moe* h, uint64_t* device_buffer, size_t bytes);
 int mf_ctx_num_cu(const mf_ctx* ctx);
 
 /* Synchronises `stream` and reports whether any fused launch of this handle
- * gave up on a grid barrier (MF_ERR_LAUNCH) since the handle was created.
+ * gave up waiting for data of another workgroup (MF_ERR_LAUNCH) since the handle was created.
  * No counterpart in the reference (Metal reports this through
  * MTLCommandBuffer.error). */
 mf_status mf_moe_status(mf_moe* h, mf_stream stream);

@@ -206,8 +206,13 @@ mf_status mf_moe_create(mf_ctx* ctx, const mf_moe_config* cfg, mf_moe** out) {
   const size_t o_acts = take(T * cfg->top_k * cfg->f * sizeof(uint16_t));
   const size_t o_sact = take(T * std::max<uint32_t>(cfg->shared_f, 64) * sizeof(uint16_t));
   const size_t o_sy = take(T * cfg->d * sizeof(uint16_t));
-  const size_t o_gate = take(T * sizeof(float));
-  const size_t o_sync = take((2 * 512 + 64) * sizeof(uint32_t));
+  const size_t o_gate = take(T * sizeof(uint16_t));
+  const size_t o_tlogits = take(T * cfg->num_experts * sizeof(uint64_t));
+  const size_t o_tgate = take(T * sizeof(uint64_t));
+  const size_t o_tsact = take(T * (std::max<uint32_t>(cfg->shared_f, 64) + 4) * sizeof(uint32_t));
+  const size_t o_tacts = take(T * cfg->top_k * cfg->f * sizeof(uint32_t));
+  const size_t o_epoch = take(512 * sizeof(uint32_t));
+  const size_t o_status = take(64);
   h->ws_bytes = pos;
   if (hipSetDevice(ctx->device) != hipSuccess) {
     delete h;
@@ -232,7 +237,12 @@ mf_status mf_moe_create(mf_ctx* ctx, const mf_moe_config* cfg, mf_moe** out) {
   h->ws.shared_act = reinterpret_cast<uint16_t*>(b + o_sact);
   h->ws.shared_y = reinterpret_cast<uint16_t*>(b + o_sy);
   h->ws.gate = reinterpret_cast<uint16_t*>(b + o_gate);
-  h->ws.sync = reinterpret_cast<uint32_t*>(b + o_sync);
+  h->ws.t_logits = reinterpret_cast<unsigned long long*>(b + o_tlogits);
+  h->ws.t_gate = reinterpret_cast<unsigned long long*>(b + o_tgate);
+  h->ws.t_sact = reinterpret_cast<uint32_t*>(b + o_tsact);
+  h->ws.t_acts = reinterpret_cast<uint32_t*>(b + o_tacts);
+  h->ws.epoch = reinterpret_cast<uint32_t*>(b + o_epoch);
+  h->ws.status = reinterpret_cast<uint32_t*>(b + o_status);
   *out = h;
   return MF_OK;
 }
@@ -309,7 +319,7 @@ mf_status mf_moe_decode_layer(mf_moe* h, mf_stream stream, const mf_moe_layer_we
                      !qtensor_ok(wts->shared_down, c.shared_bits)))
     return MF_ERR_INVALID_ARGUMENT;
   auto s = static_cast<hipStream_t>(stream);
-  if (h->fused && mf::fused_supported(c, *wts, x, y, hidden)) {
+  if (h->fused && mf::fused_supported(*h, *wts, x, y, hidden)) {
     MF_HIP(h->ctx, mf::launch_fused_decode(s, *h, *wts, x, t, y, hidden, out_idx, out_w));
     return MF_OK;
   }
@@ -363,11 +373,11 @@ mf_status mf_moe_status(mf_moe* h, mf_stream stream) {
   if (!h) return MF_ERR_INVALID_ARGUMENT;
   uint32_t word = 0;
   auto s = static_cast<hipStream_t>(stream);
-  MF_HIP(h->ctx, hipMemcpyAsync(&word, h->ws.sync + 2 * 512, sizeof word, hipMemcpyDeviceToHost, s));
+  MF_HIP(h->ctx, hipMemcpyAsync(&word, h->ws.status, sizeof word, hipMemcpyDeviceToHost, s));
   MF_HIP(h->ctx, hipStreamSynchronize(s));
   if (word != 0) {
     snprintf(h->ctx->hip_error, sizeof h->ctx->hip_error,
-             "fused decode layer: a grid barrier timed out (status word %u)", word);
+             "fused decode layer: a bounded wait on exchanged data gave up (status word %u)", word);
     return MF_ERR_LAUNCH;
   }
   return MF_OK;

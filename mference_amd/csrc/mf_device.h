@@ -144,6 +144,23 @@ __device__ __forceinline__ uint4 load_u32x4_agent(const void* p) {
   asm volatile("global_load_dwordx4 %0, %1, off sc1\n\ts_waitcnt vmcnt(0)" : "=v"(r) : "v"(p) : "memory");
   return r;
 }
+// Device-coherent 16-byte loads the compiler can schedule and wait for itself
+// (several may be in flight): a raw buffer over [p, p + 2 GiB) read with sc1.
+typedef __attribute__((ext_vector_type(4))) unsigned int mf_u32x4;
+struct AgentBuf {
+  __amdgpu_buffer_rsrc_t rsrc;
+};
+__device__ __forceinline__ AgentBuf make_agent_buf(const void* p) {
+  AgentBuf b;
+  b.rsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(p), 0, 0x7FFFFFFF, 0x00020000);
+  return b;
+}
+__device__ __forceinline__ uint4 load_u32x4_agentbuf(const AgentBuf& b, uint32_t byte_offset) {
+  const mf_u32x4 v = __builtin_amdgcn_raw_buffer_load_b128(b.rsrc, static_cast<int>(byte_offset), 0,
+                                                           16 /* sc1 */);
+  return make_uint4(v.x, v.y, v.z, v.w);
+}
+
 // every store this wave has issued is acknowledged at its scope
 __device__ __forceinline__ void wait_stores() { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); }
 

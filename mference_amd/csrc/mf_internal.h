@@ -22,8 +22,14 @@ struct mf_moe_workspace {
   uint16_t* acts;       // [MF_MAX_TOKENS, top_k, f]
   uint16_t* shared_act; // [MF_MAX_TOKENS, shared_f]
   uint16_t* shared_y;   // [MF_MAX_TOKENS, d]
-  uint16_t* gate;       // [MF_MAX_TOKENS] (x2: the fused kernel keeps fp32 there)
-  uint32_t* sync;       // grid-sync counters of the fused kernel
+  uint16_t* gate;       // [MF_MAX_TOKENS]
+  // exchange buffers of the fused launch: every word carries an epoch tag
+  unsigned long long* t_logits;  // [MF_MAX_TOKENS, num_experts]
+  unsigned long long* t_gate;    // [MF_MAX_TOKENS]
+  uint32_t* t_sact;              // [MF_MAX_TOKENS, shared_f]
+  uint32_t* t_acts;              // [MF_MAX_TOKENS, top_k, f]
+  uint32_t* epoch;               // [512] one launch counter per workgroup
+  uint32_t* status;              // non-zero once a bounded wait gave up
 };
 
 struct mf_moe {
@@ -85,8 +91,8 @@ hipError_t launch_phase2(hipStream_t s, const mf_moe_config& cfg, const void* ba
 
 
 // moe_fused.hip
-bool fused_supported(const mf_moe_config& c, const mf_moe_layer_weights& w, const void* x,
-                     const void* y, const void* hidden);
+bool fused_supported(const mf_moe& h, const mf_moe_layer_weights& w, const void* x, const void* y,
+                     const void* hidden);
 hipError_t launch_fused_decode(hipStream_t s, const mf_moe& h, const mf_moe_layer_weights& w,
                                const uint16_t* x, uint32_t t, uint16_t* y, uint16_t* hidden,
                                uint32_t* out_idx, float* out_w);

@@ -197,49 +197,116 @@ __device__ __forceinline__ void topk_wave(const float* lg, uint32_t e, uint32_t 
   }
 }
 
-// mode 0 selector, all-register form: lane l owns the `per` consecutive experts
-// from l*per (the blocked ownership of router_topk_select_k8_par,
-// moe.metal:262-345).  Each of the k rounds takes the wave maximum of the
-// lanes' best unretired score; among the lanes that hold it the lowest lane --
-// and inside a lane the lowest index -- wins, which is the serial kernel's
-// "strictly greater wins, equal score keeps the earlier expert".  NaN and -inf
-// are never selected; a round without a winner gives index 0, score -inf.
-// Rank r's result lives in lane r; weights are exp(s_r - s_0) / sum with the sum
-// taken in rank order.  All 64 lanes call it.
-__device__ __forceinline__ void topk_select_fast(const float* lg, uint32_t e, uint32_t k,
-                                                 uint32_t* idx, float* w, uint32_t lane) {
-  const uint32_t per = (e + kWave - 1) / kWave;
-  const uint32_t base = lane * per;
-  float ch[kMaxPerLane];
-#pragma unroll
-  for (int j = 0; j < kMaxPerLane; ++j) {
-    ch[j] = -__builtin_inff();
-    if (static_cast<uint32_t>(j) < per && base + j < e) ch[j] = lg[base + j];
+// mode 0 selector for a whole workgroup (every thread calls it; blockDim a
+// multiple of 64; e % 4 == 0).  The serial kernel's order "higher score first,
+// equal score: lower index first" is a total order, so the rank of an expert is
+// the number of experts that beat it, and the top-k are the experts of rank < k.
+// Four adjacent lanes share one (token, expert) and count a quarter of the
+// candidates each.  NaN and -inf never take a rank; ranks nobody takes keep
+// index 0 / score -inf.  lg: [t, e] logits in LDS; idx / w: [t, k] in LDS;
+// score: [t, k] scratch in LDS.
+__device__ __forceinline__ void topk_rank_block(const float* lg, uint32_t e, uint32_t k,
+                                                uint32_t t, uint32_t* idx, float* w,
+                                                float* score) {
+  const uint32_t tid = threadIdx.x, nthreads = blockDim.x;
+  if (tid < t * k) {
+    idx[tid] = 0;
+    score[tid] = -__builtin_inff();
   }
-  uint32_t taken = 0;
-  float my_score = -__builtin_inff();
-  uint32_t my_idx = 0;
-  for (uint32_t r = 0; r < k; ++r) {
-    float bv = -__builtin_inff();
-    int bj = -1;
-#pragma unroll
-    for (int j = 0; j < kMaxPerLane; ++j) {
-      if (!(taken & (1u << j)) && ch[j] > bv) {
-        bv = ch[j];
-        bj = j;
+  __syncthreads();
+  const uint32_t qn = e / 4;
+  const uint32_t jobs = t * e * 4;
+  for (uint32_t it0 = 0; it0 < jobs; it0 += nthreads) {
+    const uint32_t it = it0 + tid;
+    const bool live = it < jobs;
+    const uint32_t tok = live ? it / (e * 4) : 0, ex = (it / 4) % e, q = it & 3;
+    const float* row = lg + tok * e;
+    const float v = live ? row[ex] : -__builtin_inff();
+    const bool cand = v > -__builtin_inff();
+    int cnt = 0;
+    if (cand) {
+      for (uint32_t j = q * qn; j < (q + 1) * qn; ++j) {
+        const float o = row[j];
+        cnt += (o > v || (o == v && j < ex)) ? 1 : 0;
       }
     }
-    const float m = wave_max(bv);
-    const bool cand = bj >= 0 && bv == m;
+    cnt += __builtin_amdgcn_update_dpp(0, cnt, 0xB1, 0xF, 0xF, true);
+    cnt += __builtin_amdgcn_update_dpp(0, cnt, 0x4E, 0xF, 0xF, true);
+    if (cand && q == 0 && static_cast<uint32_t>(cnt) < k) {
+      idx[tok * k + cnt] = ex;
+      score[tok * k + cnt] = v;
+    }
+  }
+  __syncthreads();
+  const uint32_t wv = tid >> 6, lane = tid & 63;
+  if (wv < t) {  // w_r = exp(s_r - s_0) / sum, the sum taken in rank order
+    const float my = lane < k ? score[wv * k + lane] : -__builtin_inff();
+    const float my_e = mf_exp(my - readlane_f(my, 0));
+    float sum = 0.0f;
+#pragma unroll
+    for (int i = 0; i < MF_MAX_TOPK; ++i)
+      if (static_cast<uint32_t>(i) < k) sum += readlane_f(my_e, i);
+    if (lane < k) w[wv * k + lane] = my_e / sum;
+  }
+  __syncthreads();
+}
+
+// mode 0 selector, all-register form: lane l owns the PER consecutive experts
+// from l*PER (the blocked ownership of router_topk_select_k8_par,
+// moe.metal:262-345) and first sorts them by (score descending, index
+// ascending).  Each of the k rounds takes the wave maximum of the lanes' heads;
+// among the lanes whose head equals it the lowest lane wins and pops its head.
+// Lower lane = lower index, so this is the serial kernel's "strictly greater
+// wins, equal score keeps the earlier expert".  NaN and -inf are never selected;
+// a round without a winner gives index 0, score -inf.  Rank r's result lives in
+// lane r; weights are exp(s_r - s_0) / sum with the sum taken in rank order.
+// All 64 lanes call it.
+template <int PER>
+__device__ __forceinline__ void topk_select_sorted(const float* lg, uint32_t e, uint32_t k,
+                                                   uint32_t* idx, float* w, uint32_t lane) {
+  const float ninf = -__builtin_inff();
+  const uint32_t base = lane * PER;
+  float v[PER];
+  uint32_t id[PER];
+#pragma unroll
+  for (int j = 0; j < PER; ++j) {
+    id[j] = base + j;
+    const float x = (base + j < e) ? lg[base + j] : ninf;
+    v[j] = (x > ninf) ? x : ninf;  // NaN and -inf are not candidates
+  }
+  // odd-even transposition, swapping only on strictly smaller: stable
+#pragma unroll
+  for (int pass = 0; pass < PER; ++pass) {
+#pragma unroll
+    for (int a = pass & 1; a + 1 < PER; a += 2) {
+      const bool sw = v[a] < v[a + 1];
+      const float tv = sw ? v[a + 1] : v[a];
+      const float bv = sw ? v[a] : v[a + 1];
+      const uint32_t ti = sw ? id[a + 1] : id[a];
+      const uint32_t bi = sw ? id[a] : id[a + 1];
+      v[a] = tv; v[a + 1] = bv; id[a] = ti; id[a + 1] = bi;
+    }
+  }
+  float my_score = ninf;
+  uint32_t my_idx = 0;
+  for (uint32_t r = 0; r < k; ++r) {
+    const float m = wave_max(v[0]);
+    const bool cand = v[0] == m && m > ninf;
     const unsigned long long mask = __ballot(cand);
     uint32_t widx = 0;
-    float ws = -__builtin_inff();
+    float ws = ninf;
     if (mask != 0) {
       const int wl = __ffsll(static_cast<long long>(mask)) - 1;
-      widx = static_cast<uint32_t>(
-          __builtin_amdgcn_readlane(static_cast<int>(base + static_cast<uint32_t>(bj < 0 ? 0 : bj)), wl));
+      widx = static_cast<uint32_t>(__builtin_amdgcn_readlane(static_cast<int>(id[0]), wl));
       ws = m;
-      if (static_cast<int>(lane) == wl) taken |= 1u << bj;
+      if (static_cast<int>(lane) == wl) {  // pop the head
+#pragma unroll
+        for (int j = 0; j + 1 < PER; ++j) {
+          v[j] = v[j + 1];
+          id[j] = id[j + 1];
+        }
+        v[PER - 1] = ninf;
+      }
     }
     if (lane == r) {
       my_score = ws;
@@ -256,6 +323,15 @@ __device__ __forceinline__ void topk_select_fast(const float* lg, uint32_t e, ui
     idx[lane] = my_idx;
     w[lane] = my_e / sum;
   }
+}
+
+__device__ __forceinline__ void topk_select_fast(const float* lg, uint32_t e, uint32_t k,
+                                                 uint32_t* idx, float* w, uint32_t lane) {
+  const uint32_t per = (e + kWave - 1) / kWave;
+  if (per <= 1) topk_select_sorted<1>(lg, e, k, idx, w, lane);
+  else if (per <= 2) topk_select_sorted<2>(lg, e, k, idx, w, lane);
+  else if (per <= 4) topk_select_sorted<4>(lg, e, k, idx, w, lane);
+  else topk_select_sorted<8>(lg, e, k, idx, w, lane);
 }
 
 }  // namespace mf

@@ -1,27 +1,43 @@
 // The fused decode layer: one launch per MoE layer.
 //
-// A grid of one 1024-thread workgroup per CU stays resident for the whole layer
-// and runs three stages separated by two grid-wide barriers:
+// A grid of one 1024-thread workgroup per CU stays resident for the whole layer:
 //
 //   A  router logits (one wave per expert row), the scalar shared gate w_sg.x,
 //      shared-expert gate/up/activation rows
-//   --- barrier 1: logits, gate and shared activations are complete ---
-//      every workgroup recomputes the (cheap, deterministic) top-k itself
-//   B  routed gate/up/activation rows of the K selected experts of every token,
-//      shared-expert down rows (-> gated h1)
-//   --- barrier 2: routed activations and h1 are complete ---
-//   C  down rows: K waves of a workgroup take the K slots of one group of output
-//      rows, weight them, and one thread per row adds them to h1 in rank order.
+//      -> every workgroup gathers the logits and recomputes the (cheap,
+//         deterministic) top-k itself
+//   B  routed gate/up/activation rows of the K selected experts of every token
+//   C  per token: the shared expert's down rows of this workgroup's output rows
+//      (-> gated h1, kept in LDS), then the routed down rows: K waves take the K
+//      slots of one group of output rows, weight them, and one thread per row
+//      adds them to h1 in rank order.
+//
+// Workgroups exchange three small vectors through HBM: logits, shared
+// activations, routed activations.  There is no grid barrier.  Every exchanged
+// word carries the launch's epoch as a tag (fp32 logits: a 32-bit tag beside the
+// value; bf16 activations: a 16-bit tag above the value), producers write them
+// with device-coherent stores and go on, consumers poll the data itself with
+// device-coherent loads into LDS until every tag they need is current.  This
+// costs one store propagation plus about one load round trip per exchange;
+// a barrier built on a flag or counter costs a store acknowledgement, the flag's
+// own propagation, a poll and then the data load (measured: 4-5 us against
+// about 2 us, two exchanges per layer).  The epoch is a per-workgroup counter
+// in the workspace that every workgroup raises by one per launch, so all
+// workgroups agree on it without talking, nothing is reset between launches
+// and a captured HIP graph can replay the launch.  One token slot of the
+// activation buffers (epoch mod 8, if unused by this launch) is re-tagged per
+// launch so that no stale word is ever older than 8 launches: a 16-bit tag can
+// never alias.
 //
 // Nothing but the router decides which weights are read, so stage C's packed
-// codes are requested right after a workgroup has arrived at barrier 2: their
-// HBM latency hides behind the wait.
+// codes are requested before the routed activations are polled: their HBM
+// latency hides behind the wait.
 //
-// The barriers need every workgroup of the grid to be resident at once; the
-// launcher never asks for more workgroups than CUs and the kernel needs a whole
-// CU (1024 threads, <= 128 VGPRs).  Waits are bounded: a barrier that does not
-// complete within kSpinLimit polls sets the status word and lets the grid drain.
-// (The logits buffer is read 16 bytes at a time: [T, E] fp32 with E % 4 == 0.)
+// Consumers spin on data other workgroups produce, so every workgroup of the
+// grid has to be resident at once: the launcher never asks for more workgroups
+// than CUs and the kernel needs a whole CU (1024 threads, <= 128 VGPRs).  Waits
+// are bounded: a poll that does not complete within kSpinLimit tries sets the
+// status word and lets the grid drain.
 #include "mf_device.h"
 #include "mf_internal.h"
 #include "mf_router.h"
@@ -32,7 +48,8 @@ namespace mf {
 
 constexpr uint32_t kFusedThreads = 1024;
 constexpr uint32_t kFusedWaves = kFusedThreads / kWave;
-constexpr uint32_t kSpinLimit = 1u << 22;  // x ~50 ns per poll
+constexpr uint32_t kSpinLimit = 1u << 20;  // x ~1 us per poll
+constexpr uint32_t kMaxH1 = 2048;          // output rows of one token a workgroup may own
 
 template <int BITS> struct Chunk {
   uint4 codes;
@@ -48,10 +65,9 @@ __device__ __forceinline__ Chunk<BITS> load_chunk(const uint8_t* wrow, const uin
   return c;
 }
 
-// lane partial of one row of N elements against x (16-byte aligned bf16);
-// `first` may carry the already loaded chunk of the first step.  AGENT_X: x was
-// written by other workgroups during this launch.
-template <int BITS, bool AGENT_X>
+// lane partial of one row of N elements against x (16-byte aligned bf16, global
+// or LDS); `first` may carry the already loaded chunk of the first step.
+template <int BITS>
 __device__ __forceinline__ float row_partial(const uint8_t* wrow, const uint16_t* srow,
                                              const uint16_t* brow, const uint16_t* x, uint32_t N,
                                              uint32_t sub, uint32_t lpr, bool have_first,
@@ -61,12 +77,9 @@ __device__ __forceinline__ float row_partial(const uint8_t* wrow, const uint16_t
   for (uint32_t e0 = sub * EPL; e0 < N; e0 += lpr * EPL) {
     const Chunk<BITS> c = (have_first && e0 == sub * EPL) ? first
                                                            : load_chunk<BITS>(wrow, srow, brow, e0);
-    float dot, sum;
-    const XSlice<BITS> xs = load_xslice<BITS, AGENT_X ? kXAgent : kXAligned>(x + e0);
-    dot = codes_dot<BITS>(c.codes, xs);
-    sum = xs.sum;
-    acc = __builtin_fmaf(c.s, dot, acc);
-    acc = __builtin_fmaf(c.b, sum, acc);
+    const XSlice<BITS> xs = load_xslice<BITS, kXAligned>(x + e0);
+    acc = __builtin_fmaf(c.s, codes_dot<BITS>(c.codes, xs), acc);
+    acc = __builtin_fmaf(c.b, xs.sum, acc);
   }
   return acc;
 }
@@ -85,11 +98,10 @@ __device__ __forceinline__ void gate_up_partial(const uint8_t* gw, const uint16_
     const Chunk<BITS> u = load_chunk<BITS>(uw, us, ub, e0);
     const XSlice<BITS> xs = load_xslice<BITS, kXAligned>(x + e0);
     const float gd = codes_dot<BITS>(g.codes, xs), ud = codes_dot<BITS>(u.codes, xs);
-    const float sum = xs.sum;
     ga = __builtin_fmaf(g.s, gd, ga);
-    ga = __builtin_fmaf(g.b, sum, ga);
+    ga = __builtin_fmaf(g.b, xs.sum, ga);
     ua = __builtin_fmaf(u.s, ud, ua);
-    ua = __builtin_fmaf(u.b, sum, ua);
+    ua = __builtin_fmaf(u.b, xs.sum, ua);
   }
 }
 
@@ -105,84 +117,108 @@ struct FusedArgs {
   uint16_t* hidden;
   uint32_t* out_idx;
   float* out_w;
-  float* logits;
-  uint16_t* acts;
-  uint16_t* shared_act;
-  uint16_t* shared_y;
-  float* gate;  // bf16-rounded scalar shared gate per token
-  unsigned long long* trace;  // phase timestamps, 8 per workgroup, or nullptr
-  uint32_t* sync;  // kMaxGrid flags of barrier 1, kMaxGrid of barrier 2, status word
+  // exchange buffers (workspace of the handle)
+  unsigned long long* t_logits;  // [T, E] (value bits | epoch << 32)
+  uint32_t* t_sact;              // [MF_MAX_TOKENS, Fs + 4] (bf16 | tag << 16); word Fs = gate
+  uint32_t* t_acts;              // [MF_MAX_TOKENS, K, F]
+  uint32_t* epoch;               // one counter per workgroup
+  uint32_t* status;
+  unsigned long long* trace;     // phase timestamps, 8 per workgroup, or nullptr
   uint32_t D, F, E, K, T, Fs;
   int router_mode;
   float limit;
 };
 
-// Grid barrier without read-modify-write atomics (256 workgroups adding to one
-// counter serialise at the memory side for microseconds): every workgroup owns
-// one flag per barrier and raises it by one each time it arrives; a waiter
-// polls all flags with one 16-byte device-coherent load per lane until none
-// lags behind its own.  Flags only ever count up, so nothing has to be reset
-// between launches (HIP-graph replay safe).  Exchanged data is written with
-// device-coherent stores that are acknowledged before the flag is raised.
-constexpr uint32_t kMaxGrid = 512;  // flags per barrier
-constexpr uint32_t kSyncFlags1 = 0, kSyncFlags2 = kMaxGrid, kSyncStatus = 2 * kMaxGrid;
-
-__device__ __forceinline__ void grid_arrive(uint32_t* flags, uint32_t target) {
-  wait_stores();
-  __syncthreads();
-  if (threadIdx.x == 0) store_u32_agent(&flags[blockIdx.x], target);
+__device__ __forceinline__ void store_u64_agent(unsigned long long* p, unsigned long long v) {
+  __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
-__device__ __forceinline__ void grid_wait(const uint32_t* flags, uint32_t target, uint32_t G,
-                                          uint32_t* status) {
-  if (threadIdx.x < kWave) {
-    const uint32_t lane = threadIdx.x;
-    uint32_t spins = 0;
-    for (;;) {
-      bool ok = true;
-      for (uint32_t b = 0; b < G; b += 4 * kWave) {
-        const uint32_t i = b + 4 * lane;
-        const uint4 f = load_u32x4_agent(flags + i);
-        ok = ok && (i + 0 >= G || static_cast<int32_t>(f.x - target) >= 0) &&
-             (i + 1 >= G || static_cast<int32_t>(f.y - target) >= 0) &&
-             (i + 2 >= G || static_cast<int32_t>(f.z - target) >= 0) &&
-             (i + 3 >= G || static_cast<int32_t>(f.w - target) >= 0);
-      }
-      if (__all(ok)) break;
-      __builtin_amdgcn_s_sleep(1);
-      if (++spins > kSpinLimit) {
-        if (lane == 0) store_u32_agent(status, 1u);
+__device__ __forceinline__ void give_up(uint32_t* status, uint32_t lane) {
+  if (lane == 0) store_u32_agent(status, 1u);
+}
+
+// One wave gathers n tagged fp32 entries (n % 2 == 0) into dst (LDS).
+__device__ __forceinline__ void poll_tagged_f32(const unsigned long long* src, float* dst,
+                                                uint32_t n, uint32_t epoch, uint32_t lane,
+                                                uint32_t* status) {
+  for (uint32_t base = 0; base < n; base += 2 * kWave) {
+    const uint32_t e0 = base + 2 * lane;
+    const bool in = e0 < n;
+    uint4 v = make_uint4(0, epoch, 0, epoch);
+    for (uint32_t spins = 0;; ++spins) {
+      if (in) v = load_u32x4_agent(src + e0);
+      if (__all(!in || (v.y == epoch && v.w == epoch))) break;
+      if (spins > kSpinLimit) {
+        give_up(status, lane);
         break;
       }
+      __builtin_amdgcn_s_sleep(1);
+    }
+    if (in) {
+      dst[e0] = __uint_as_float(v.x);
+      dst[e0 + 1] = __uint_as_float(v.z);
     }
   }
-  __syncthreads();
 }
 
-// phase trace: the shader clock at every stage boundary, thread 0 of each workgroup
+// Waves part, part + nparts, ... gather n tagged bf16 words (n % 4 == 0) into
+// packed bf16 pairs at dst (LDS, n / 2 words).
+__device__ __forceinline__ void poll_tagged_bf16(const uint32_t* src, uint32_t* dst, uint32_t n,
+                                                 uint32_t tag16, uint32_t part, uint32_t nparts,
+                                                 uint32_t lane, uint32_t* status) {
+  for (uint32_t w0 = part * 4 * kWave; w0 < n; w0 += nparts * 4 * kWave) {
+    const uint32_t i = w0 + 4 * lane;
+    const bool in = i < n;
+    const uint32_t want = tag16 << 16;
+    uint4 v = make_uint4(want, want, want, want);
+    for (uint32_t spins = 0;; ++spins) {
+      if (in) v = load_u32x4_agent(src + i);
+      const uint32_t diff = (v.x ^ want) | (v.y ^ want) | (v.z ^ want) | (v.w ^ want);
+      if (__all(!in || (diff >> 16) == 0)) break;
+      if (spins > kSpinLimit) {
+        give_up(status, lane);
+        break;
+      }
+      __builtin_amdgcn_s_sleep(1);
+    }
+    if (in) {
+      dst[i / 2] = __builtin_amdgcn_perm(v.y, v.x, 0x05040100u);
+      dst[i / 2 + 1] = __builtin_amdgcn_perm(v.w, v.z, 0x05040100u);
+    }
+  }
+}
+
+// phase trace: the 100 MHz wall clock at every stage boundary, thread 0 of each workgroup
 __device__ __forceinline__ void trace_mark(const FusedArgs& a, uint32_t slot) {
   if (a.trace && threadIdx.x == 0) a.trace[blockIdx.x * 8 + slot] = wall_clock64();
 }
 
 template <int BITS, int SBITS>
 __global__ __launch_bounds__(kFusedThreads) void fused_decode_kernel(const FusedArgs a) {
-  __shared__ uint32_t s_idx[MF_MAX_TOKENS * MF_MAX_TOPK];
-  __shared__ float s_w[MF_MAX_TOKENS * MF_MAX_TOPK];
-  __shared__ float s_v[kFusedWaves][kWave];
-  __shared__ float s_lg[MF_MAX_TOKENS][MF_MAX_EXPERTS];
+  extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
+  const uint32_t D = a.D, F = a.F, E = a.E, K = a.K, T = a.T, Fs = a.Fs;
+  // LDS carve-up (the launcher sizes it with fused_lds_bytes)
+  uint32_t* s_idx = reinterpret_cast<uint32_t*>(smem);                 // [8*8]
+  float* s_w = reinterpret_cast<float*>(smem + 256);                    // [8*8]
+  float* s_v = reinterpret_cast<float*>(smem + 1024);                   // [16][64]
+  float* s_h1 = reinterpret_cast<float*>(smem + 1024 + 4096);           // [kMaxH1]
+  uint8_t* dyn = smem + 1024 + 4096 + kMaxH1 * 4;
+  float* s_lg = reinterpret_cast<float*>(dyn);                          // [MF_MAX_TOKENS][E]
+  uint32_t* s_sact = reinterpret_cast<uint32_t*>(dyn + MF_MAX_TOKENS * E * 4);  // [(Fs+4)/2]
+  uint32_t* s_acts = s_sact + (((Fs + 4) / 2 + 3) & ~3u);               // [K*F/2], 16-byte aligned
+  const uint32_t sact_stride = Fs + 4;  // words per token in t_sact
 
   const uint32_t lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
   const uint32_t G = gridDim.x, wg = blockIdx.x;
   const uint32_t gw = wv * G + wg;  // consecutive work items land on different CUs
   const uint32_t total_waves = kFusedWaves * G;
-  const uint32_t D = a.D, F = a.F, E = a.E, K = a.K, T = a.T, Fs = a.Fs;
 
-  // this launch's barrier targets: one above the workgroup's own flags
-  const uint32_t target1 =
-      __hip_atomic_load(&a.sync[kSyncFlags1 + wg], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) + 1u;
-  const uint32_t target2 =
-      __hip_atomic_load(&a.sync[kSyncFlags2 + wg], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) + 1u;
+  const uint32_t epoch =
+      __hip_atomic_load(&a.epoch[wg], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) + 1u;
+  const uint32_t tag16 = epoch & 0xFFFFu;
+  const unsigned long long etag = static_cast<unsigned long long>(epoch) << 32;
   trace_mark(a, 0);
+
   // ------------------------------------------------------------- stage A
   {
     const uint32_t lpr_log2 = Fs ? lanes_per_row_log2_dev(D, Fmt<SBITS>::kElemsPer16B) : 0;
@@ -196,11 +232,13 @@ __global__ __launch_bounds__(kFusedThreads) void fused_decode_kernel(const Fused
         const uint32_t tok = item / E, row = item % E;
         const float v = dot_bf16_row(a.router_w + static_cast<size_t>(row) * D,
                                      a.x + static_cast<size_t>(tok) * D, D, lane, true);
-        if (lane == 0) store_f32_agent(&a.logits[item], v);
+        if (lane == 0) store_u64_agent(&a.t_logits[item], etag | __float_as_uint(v));
       } else if (item < n_router + n_gate) {
         const uint32_t tok = item - n_router;
         const float v = dot_bf16_row(a.w_sg, a.x + static_cast<size_t>(tok) * D, D, lane, true);
-        if (lane == 0) store_f32_agent(&a.gate[tok], round_bf16(v));
+        if (lane < 4)  // the gate rides behind the token's shared activations
+          store_u32_agent(&a.t_sact[static_cast<size_t>(tok) * sact_stride + Fs + lane],
+                          (lane == 0 ? static_cast<uint32_t>(f_to_bf16(v)) : 0u) | (tag16 << 16));
       } else {
         const uint32_t it = item - n_router - n_gate;
         const uint32_t tok = it / srg;
@@ -222,201 +260,264 @@ __global__ __launch_bounds__(kFusedThreads) void fused_decode_kernel(const Fused
         if (ok && sub == 0) {
           // dequant_int4.metal:240-245: gate and up narrowed before the activation
           const float rg = round_bf16(g), ru = round_bf16(u);
-          store_u16_agent(&a.shared_act[static_cast<size_t>(tok) * Fs + row],
-                          f_to_bf16(mf_silu(rg) * ru));
+          store_u32_agent(&a.t_sact[static_cast<size_t>(tok) * sact_stride + row],
+                          static_cast<uint32_t>(f_to_bf16(mf_silu(rg) * ru)) | (tag16 << 16));
         }
       }
     }
-  }
-  trace_mark(a, 1);
-  grid_arrive(a.sync + kSyncFlags1, target1);
-  grid_wait(a.sync + kSyncFlags1, target1, G, a.sync + kSyncStatus);
-  trace_mark(a, 2);
-
-  // ------------------------------------------------------------- top-k
-  if (wv < T) {  // stage the token's logits in LDS: 4 consecutive experts per lane and load
-    for (uint32_t e0 = 4 * lane; e0 < E; e0 += 4 * kWave) {
-      const uint4 v = load_u32x4_agent(a.logits + static_cast<size_t>(wv) * E + e0);
-      s_lg[wv][e0] = __uint_as_float(v.x);
-      if (e0 + 1 < E) s_lg[wv][e0 + 1] = __uint_as_float(v.y);
-      if (e0 + 2 < E) s_lg[wv][e0 + 2] = __uint_as_float(v.z);
-      if (e0 + 3 < E) s_lg[wv][e0 + 3] = __uint_as_float(v.w);
+    // keep every word of the activation buffers recently tagged (see the top)
+    const uint32_t ts = epoch % MF_MAX_TOKENS;
+    if (ts >= T) {
+      const uint32_t gtid = wg * kFusedThreads + threadIdx.x, gthreads = G * kFusedThreads;
+      for (uint32_t i = gtid; i < K * F; i += gthreads)
+        store_u32_agent(&a.t_acts[static_cast<size_t>(ts) * K * F + i], tag16 << 16);
+      for (uint32_t i = gtid; i < (Fs ? sact_stride : 0); i += gthreads)
+        store_u32_agent(&a.t_sact[static_cast<size_t>(ts) * sact_stride + i], tag16 << 16);
     }
   }
+  trace_mark(a, 1);
+
+  // ------------------------------------------------------- logits, top-k
+  if (wv < T)
+    poll_tagged_f32(a.t_logits + static_cast<size_t>(wv) * E, s_lg + wv * E, E, epoch, lane,
+                    a.status);
   __syncthreads();
+  trace_mark(a, 2);
   if (wv < T) {
-    if (a.router_mode == 0) topk_select_fast(s_lg[wv], E, K, s_idx + wv * K, s_w + wv * K, lane);
-    else topk_wave(s_lg[wv], E, K, a.router_mode, s_idx + wv * K, s_w + wv * K, lane);
+    if (a.router_mode == 0) topk_select_fast(s_lg + wv * E, E, K, s_idx + wv * K, s_w + wv * K, lane);
+    else topk_wave(s_lg + wv * E, E, K, a.router_mode, s_idx + wv * K, s_w + wv * K, lane);
   }
   __syncthreads();
   if (wg == 0 && threadIdx.x < T * K) {
     if (a.out_idx) a.out_idx[threadIdx.x] = s_idx[threadIdx.x];
     if (a.out_w) a.out_w[threadIdx.x] = s_w[threadIdx.x];
   }
-
   trace_mark(a, 3);
+
   // ------------------------------------------------------------- stage B
   {
     const uint32_t lpr_log2 = lanes_per_row_log2_dev(D, Fmt<BITS>::kElemsPer16B);
     const uint32_t lpr = 1u << lpr_log2, rpw = 64u >> lpr_log2;
     const uint32_t rgf = (F + rpw - 1) / rpw;
-    const uint32_t n_routed = T * K * rgf;
-    const uint32_t slpr_log2 = Fs ? lanes_per_row_log2_dev(Fs, Fmt<SBITS>::kElemsPer16B) : 0;
-    const uint32_t slpr = 1u << slpr_log2, srpw = 64u >> slpr_log2;
-    const uint32_t sdrg = Fs ? (D + srpw - 1) / srpw : 0;
-    const uint32_t n_items = n_routed + T * sdrg;
+    const uint32_t n_items = T * K * rgf;
     for (uint32_t item = gw; item < n_items; item += total_waves) {
-      if (item < n_routed) {
-        const uint32_t pair = item / rgf;
-        const uint32_t row = (item % rgf) * rpw + (lane >> lpr_log2);
-        const uint32_t sub = lane & (lpr - 1);
-        const bool ok = row < F;
-        const uint32_t expert = s_idx[pair];
-        if (expert >= E) {
-          if (ok && sub == 0) store_u16_agent(&a.acts[static_cast<size_t>(pair) * F + row], 0);
-          continue;
+      const uint32_t pair = item / rgf;
+      const uint32_t row = (item % rgf) * rpw + (lane >> lpr_log2);
+      const uint32_t sub = lane & (lpr - 1);
+      const bool ok = row < F;
+      const uint32_t expert = s_idx[pair];
+      uint32_t* dst = &a.t_acts[static_cast<size_t>(pair) * F + (ok ? row : 0)];
+      if (expert >= E) {  // router sentinel: the slot contributes nothing
+        if (ok && sub == 0) store_u32_agent(dst, tag16 << 16);
+        continue;
+      }
+      const uint8_t* blob = a.expert_base + static_cast<size_t>(expert) * a.expert_stride;
+      const size_t r = ok ? row : 0;
+      const uint32_t ng = D / kGroup;
+      const size_t rb = static_cast<size_t>(D) * Store<BITS>::kBits / 8;
+      float ga = 0.0f, ua = 0.0f;
+      if (ok)
+        gate_up_partial<BITS>(blob + a.off.gate_w + r * rb,
+                              reinterpret_cast<const uint16_t*>(blob + a.off.gate_s) + r * ng,
+                              reinterpret_cast<const uint16_t*>(blob + a.off.gate_b) + r * ng,
+                              blob + a.off.up_w + r * rb,
+                              reinterpret_cast<const uint16_t*>(blob + a.off.up_s) + r * ng,
+                              reinterpret_cast<const uint16_t*>(blob + a.off.up_b) + r * ng,
+                              a.x + static_cast<size_t>(pair / K) * D, D, sub, lpr, ga, ua);
+      float g = group_sum(ga, static_cast<int>(lpr));
+      float u = group_sum(ua, static_cast<int>(lpr));
+      if (ok && sub == 0) {
+        if (a.limit > 0.0f) {  // moe.metal:27-34
+          g = fminf(g, a.limit);
+          u = fminf(fmaxf(u, -a.limit), a.limit);
         }
-        const uint8_t* blob = a.expert_base + static_cast<size_t>(expert) * a.expert_stride;
-        const size_t r = ok ? row : 0;
-        const uint32_t ng = D / kGroup;
-        const size_t rb = static_cast<size_t>(D) * Store<BITS>::kBits / 8;
-        float ga = 0.0f, ua = 0.0f;
-        if (ok)
-          gate_up_partial<BITS>(
-              blob + a.off.gate_w + r * rb,
-              reinterpret_cast<const uint16_t*>(blob + a.off.gate_s) + r * ng,
-              reinterpret_cast<const uint16_t*>(blob + a.off.gate_b) + r * ng,
-              blob + a.off.up_w + r * rb,
-              reinterpret_cast<const uint16_t*>(blob + a.off.up_s) + r * ng,
-              reinterpret_cast<const uint16_t*>(blob + a.off.up_b) + r * ng,
-              a.x + static_cast<size_t>(pair / K) * D, D, sub, lpr, ga, ua);
-        float g = group_sum(ga, static_cast<int>(lpr));
-        float u = group_sum(ua, static_cast<int>(lpr));
-        if (ok && sub == 0) {
-          if (a.limit > 0.0f) {  // moe.metal:27-34
-            g = fminf(g, a.limit);
-            u = fminf(fmaxf(u, -a.limit), a.limit);
-          }
-          store_u16_agent(&a.acts[static_cast<size_t>(pair) * F + row], f_to_bf16(mf_silu(g) * u));
-        }
-      } else {
-        const uint32_t it = item - n_routed;
-        const uint32_t tok = it / sdrg;
-        const uint32_t row = (it % sdrg) * srpw + (lane >> slpr_log2);
-        const uint32_t sub = lane & (slpr - 1);
-        const bool ok = row < D;
-        const size_t r = ok ? row : 0;
-        const uint32_t ng = Fs / kGroup;
-        const size_t rb = static_cast<size_t>(Fs) * Store<SBITS>::kBits / 8;
-        float part = 0.0f;
-        if (ok)
-          part = row_partial<SBITS, true>(static_cast<const uint8_t*>(a.sd.weights) + r * rb,
-                                    a.sd.scales + r * ng, a.sd.biases + r * ng,
-                                    a.shared_act + static_cast<size_t>(tok) * Fs, Fs, sub, slpr,
-                                    false, Chunk<SBITS>{});
-        const float v = group_sum(part, static_cast<int>(slpr));
-        if (ok && sub == 0) {
-          uint16_t h = f_to_bf16(v);  // dequant_int4.metal:177-180
-          if (a.w_sg) {               // utility.metal:49-59
-            const float gt = load_f32_agent(&a.gate[tok]);
-            h = f_to_bf16(bf16_to_f(h) / (1.0f + mf_exp(-gt)));
-          }
-          store_u16_agent(&a.shared_y[static_cast<size_t>(tok) * D + row], h);
-        }
+        store_u32_agent(dst, static_cast<uint32_t>(f_to_bf16(mf_silu(g) * u)) | (tag16 << 16));
       }
     }
   }
+  trace_mark(a, 4);
 
   // ------------------------------------------------------------- stage C
   const uint32_t lpr_log2 = lanes_per_row_log2_dev(F, Fmt<BITS>::kElemsPer16B);
   const uint32_t lpr = 1u << lpr_log2, rpw = 64u >> lpr_log2;
-  const uint32_t rg_per_tok = (D + rpw - 1) / rpw;
-  const uint32_t units = T * rg_per_tok;
-  const uint32_t ub = kFusedWaves / K;  // units a workgroup handles per round
-  const uint32_t rounds = (units + G * ub - 1) / (G * ub);
+  const uint32_t rg_per_tok = (D + rpw - 1) / rpw;  // units (groups of rpw output rows) per token
+  const uint32_t ub = kFusedWaves / K;              // units a workgroup handles per round
+  const uint32_t rounds = (rg_per_tok + G * ub - 1) / (G * ub);
   const uint32_t unit_local = wv / K, slot = wv % K;
   const uint32_t sub = lane & (lpr - 1);
   const uint32_t ng = F / kGroup;
   const size_t rb = static_cast<size_t>(F) * Store<BITS>::kBits / 8;
+  const uint32_t rows_per_round = ub * rpw;
+  // shared-expert down rows: srpw rows per wave step
+  const uint32_t slpr_log2 = Fs ? lanes_per_row_log2_dev(Fs, Fmt<SBITS>::kElemsPer16B) : 0;
+  const uint32_t slpr = 1u << slpr_log2, srpw = 64u >> slpr_log2;
 
-  trace_mark(a, 4);
-  grid_arrive(a.sync + kSyncFlags2, target2);
-  // request round 0's codes while the barrier completes
-  Chunk<BITS> pre{};
-  bool have_pre = false;
-  {
-    const uint32_t unit = wg * ub + unit_local;
-    if (unit_local < ub && unit < units) {
-      const uint32_t tok = unit / rg_per_tok;
-      const uint32_t row = (unit % rg_per_tok) * rpw + (lane >> lpr_log2);
-      const uint32_t expert = s_idx[tok * K + slot];
-      if (row < D && expert < E && sub * Fmt<BITS>::kElemsPer16B < F) {
-        const uint8_t* blob = a.expert_base + static_cast<size_t>(expert) * a.expert_stride;
-        pre = load_chunk<BITS>(blob + a.off.down_w + row * rb,
-                               reinterpret_cast<const uint16_t*>(blob + a.off.down_s) + row * ng,
-                               reinterpret_cast<const uint16_t*>(blob + a.off.down_b) + row * ng,
-                               sub * Fmt<BITS>::kElemsPer16B);
-        have_pre = true;
-      }
-    }
-  }
-  grid_wait(a.sync + kSyncFlags2, target2, G, a.sync + kSyncStatus);
-  trace_mark(a, 5);
-
-  for (uint32_t round = 0; round < rounds; ++round) {
-    const uint32_t unit = (round * G + wg) * ub + unit_local;
-    const bool active = unit_local < ub && unit < units;
-    if (active) {
-      const uint32_t tok = unit / rg_per_tok;
-      const uint32_t row = (unit % rg_per_tok) * rpw + (lane >> lpr_log2);
-      const uint32_t pair = tok * K + slot;
-      const uint32_t expert = s_idx[pair];
-      const bool ok = row < D;
-      float part = 0.0f;
-      if (ok && expert < E) {
-        const uint8_t* blob = a.expert_base + static_cast<size_t>(expert) * a.expert_stride;
-        part = row_partial<BITS, true>(blob + a.off.down_w + row * rb,
+  for (uint32_t tok = 0; tok < T; ++tok) {
+    // request round 0's routed codes, then wait for what other workgroups produce
+    Chunk<BITS> pre{};
+    bool have_pre = false;
+    {
+      const uint32_t unit = wg * ub + unit_local;
+      if (unit_local < ub && unit < rg_per_tok) {
+        const uint32_t row = unit * rpw + (lane >> lpr_log2);
+        const uint32_t expert = s_idx[tok * K + slot];
+        if (row < D && expert < E && sub * Fmt<BITS>::kElemsPer16B < F) {
+          const uint8_t* blob = a.expert_base + static_cast<size_t>(expert) * a.expert_stride;
+          pre = load_chunk<BITS>(blob + a.off.down_w + row * rb,
                                  reinterpret_cast<const uint16_t*>(blob + a.off.down_s) + row * ng,
                                  reinterpret_cast<const uint16_t*>(blob + a.off.down_b) + row * ng,
-                                 a.acts + static_cast<size_t>(pair) * F, F, sub, lpr,
-                                 have_pre && round == 0, pre);
+                                 sub * Fmt<BITS>::kElemsPer16B);
+          have_pre = true;
+        }
       }
-      const float v = group_sum(part, static_cast<int>(lpr));
-      if (sub == 0) s_v[wv][lane >> lpr_log2] = s_w[pair] * v;  // moe.metal:1262
+    }
+    // first shared-expert down chunk of this wave, requested before the wait as well
+    const uint32_t sng = Fs ? Fs / kGroup : 0;
+    const size_t srb = static_cast<size_t>(Fs) * Store<SBITS>::kBits / 8;
+    const uint32_t n_slots = Fs ? rounds * rows_per_round : 0;
+    const uint32_t ssub = lane & (slpr - 1);
+    Chunk<SBITS> spre{};
+    bool have_spre = false;
+    if (Fs) {
+      const uint32_t i = wv * srpw + (lane >> slpr_log2);
+      const uint32_t round = i / rows_per_round, in_round = i % rows_per_round;
+      const uint32_t unit = (round * G + wg) * ub + in_round / rpw;
+      const uint32_t row = unit * rpw + in_round % rpw;
+      if (i < n_slots && unit < rg_per_tok && row < D && ssub * Fmt<SBITS>::kElemsPer16B < Fs) {
+        spre = load_chunk<SBITS>(static_cast<const uint8_t*>(a.sd.weights) + row * srb,
+                                 a.sd.scales + static_cast<size_t>(row) * sng,
+                                 a.sd.biases + static_cast<size_t>(row) * sng,
+                                 ssub * Fmt<SBITS>::kElemsPer16B);
+        have_spre = true;
+      }
+    }
+    // gather this token's routed activations and shared activations (+ gate) in one go:
+    // a virtual array [acts | sact], 256 words per wave step, two steps in flight
+    {
+      const uint32_t n_a = K * F, n_s = Fs ? (a.w_sg ? Fs + 4 : Fs) : 0, total = n_a + n_s;
+      const AgentBuf ba = make_agent_buf(a.t_acts + static_cast<size_t>(tok) * n_a);
+      const AgentBuf bs = make_agent_buf(a.t_sact + static_cast<size_t>(tok) * sact_stride);
+      const uint32_t want = tag16 << 16, step = kFusedWaves * 4 * kWave;
+      for (uint32_t c0 = wv * 4 * kWave; c0 < total; c0 += 2 * step) {
+        const uint32_t i0 = c0 + 4 * lane, i1 = i0 + step;
+        const bool in0 = i0 < total, in1 = i1 < total;
+        uint4 v0 = make_uint4(want, want, want, want), v1 = v0;
+        for (uint32_t spins = 0;; ++spins) {
+          if (in0) v0 = i0 < n_a ? load_u32x4_agentbuf(ba, i0 * 4) : load_u32x4_agentbuf(bs, (i0 - n_a) * 4);
+          if (in1) v1 = i1 < n_a ? load_u32x4_agentbuf(ba, i1 * 4) : load_u32x4_agentbuf(bs, (i1 - n_a) * 4);
+          const uint32_t diff = (v0.x ^ want) | (v0.y ^ want) | (v0.z ^ want) | (v0.w ^ want) |
+                                (v1.x ^ want) | (v1.y ^ want) | (v1.z ^ want) | (v1.w ^ want);
+          if (__all((diff >> 16) == 0)) break;
+          if (spins > kSpinLimit) {
+            give_up(a.status, lane);
+            break;
+          }
+          __builtin_amdgcn_s_sleep(1);
+        }
+        if (in0) {
+          uint32_t* dst = i0 < n_a ? s_acts + i0 / 2 : s_sact + (i0 - n_a) / 2;
+          dst[0] = __builtin_amdgcn_perm(v0.y, v0.x, 0x05040100u);
+          dst[1] = __builtin_amdgcn_perm(v0.w, v0.z, 0x05040100u);
+        }
+        if (in1) {
+          uint32_t* dst = i1 < n_a ? s_acts + i1 / 2 : s_sact + (i1 - n_a) / 2;
+          dst[0] = __builtin_amdgcn_perm(v1.y, v1.x, 0x05040100u);
+          dst[1] = __builtin_amdgcn_perm(v1.w, v1.z, 0x05040100u);
+        }
+      }
     }
     __syncthreads();
-    if (threadIdx.x < ub * rpw) {
-      const uint32_t ul = threadIdx.x / rpw, rr = threadIdx.x % rpw;
-      const uint32_t u2 = (round * G + wg) * ub + ul;
-      if (u2 < units) {
-        const uint32_t tok = u2 / rg_per_tok;
-        const uint32_t row = (u2 % rg_per_tok) * rpw + rr;
-        if (row < D) {
+    if (tok == 0) trace_mark(a, 5);
+    if (Fs) {
+      // gated shared output h1 of every output row this workgroup owns for this token
+      const float gate = a.w_sg ? bf16_lo(s_sact[Fs / 2]) : 0.0f;
+      for (uint32_t s0 = wv * srpw; s0 < n_slots; s0 += kFusedWaves * srpw) {
+        const uint32_t i = s0 + (lane >> slpr_log2);  // slot of (round, unit_local, row in unit)
+        const uint32_t round = i / rows_per_round, in_round = i % rows_per_round;
+        const uint32_t unit = (round * G + wg) * ub + in_round / rpw;
+        const uint32_t row = unit * rpw + in_round % rpw;
+        const bool ok = i < n_slots && unit < rg_per_tok && row < D;
+        float part = 0.0f;
+        if (ok)
+          part = row_partial<SBITS>(static_cast<const uint8_t*>(a.sd.weights) + row * srb,
+                                    a.sd.scales + static_cast<size_t>(row) * sng,
+                                    a.sd.biases + static_cast<size_t>(row) * sng,
+                                    reinterpret_cast<const uint16_t*>(s_sact), Fs, ssub, slpr,
+                                    have_spre && s0 == wv * srpw, spre);
+        const float v = group_sum(part, static_cast<int>(slpr));
+        if (ok && ssub == 0) {
+          float h = round_bf16(v);  // dequant_int4.metal:177-180
+          if (a.w_sg) h = round_bf16(h / (1.0f + mf_exp(-gate)));  // utility.metal:49-59
+          s_h1[i] = h;
+        }
+      }
+    }
+
+    for (uint32_t round = 0; round < rounds; ++round) {
+      const uint32_t unit = (round * G + wg) * ub + unit_local;
+      const bool active = unit_local < ub && unit < rg_per_tok;
+      if (active) {
+        const uint32_t row = unit * rpw + (lane >> lpr_log2);
+        const uint32_t pair = tok * K + slot;
+        const uint32_t expert = s_idx[pair];
+        float part = 0.0f;
+        if (row < D && expert < E) {
+          const uint8_t* blob = a.expert_base + static_cast<size_t>(expert) * a.expert_stride;
+          part = row_partial<BITS>(blob + a.off.down_w + row * rb,
+                                   reinterpret_cast<const uint16_t*>(blob + a.off.down_s) + row * ng,
+                                   reinterpret_cast<const uint16_t*>(blob + a.off.down_b) + row * ng,
+                                   reinterpret_cast<const uint16_t*>(s_acts) + slot * F, F, sub, lpr,
+                                   have_pre && round == 0, pre);
+        }
+        const float v = group_sum(part, static_cast<int>(lpr));
+        if (sub == 0) s_v[wv * kWave + (lane >> lpr_log2)] = s_w[pair] * v;  // moe.metal:1262
+      }
+      __syncthreads();
+      if (threadIdx.x < rows_per_round) {
+        const uint32_t ul = threadIdx.x / rpw, rr = threadIdx.x % rpw;
+        const uint32_t u2 = (round * G + wg) * ub + ul;
+        const uint32_t row = u2 * rpw + rr;
+        if (u2 < rg_per_tok && row < D) {
           const size_t o = static_cast<size_t>(tok) * D + row;
-          float acc = Fs ? bf16_to_f(load_u16_agent(&a.shared_y[o])) : 0.0f;  // residual first (moe.metal:1265)
+          float acc = Fs ? s_h1[round * rows_per_round + threadIdx.x] : 0.0f;  // residual first
           for (uint32_t k = 0; k < K; ++k)
-            if (s_idx[tok * K + k] < E) acc = acc + s_v[ul * K + k][rr];
+            if (s_idx[tok * K + k] < E) acc = acc + s_v[(ul * K + k) * kWave + rr];
           const uint16_t yb = f_to_bf16(acc);
           a.y[o] = yb;
           if (a.hidden)  // residual_add_fp16, utility.metal:83-92
             a.hidden[o] = f_to_bf16(bf16_to_f(a.hidden[o]) + bf16_to_f(yb));
         }
       }
+      __syncthreads();
     }
-    __syncthreads();
   }
-
+  if (threadIdx.x == 0) a.epoch[wg] = epoch;
   trace_mark(a, 6);
 }
 
-bool fused_supported(const mf_moe_config& c, const mf_moe_layer_weights& w, const void* x,
-                     const void* y, const void* hidden) {
-  if (c.num_experts % 4 != 0) return false;  // logits are staged 4 at a time
+size_t fused_lds_bytes(const mf_moe_config& c) {
+  return 1024 + 4096 + kMaxH1 * 4 + static_cast<size_t>(MF_MAX_TOKENS) * c.num_experts * 4 +
+         2 * static_cast<size_t>(c.shared_f) + 128 + 2 * static_cast<size_t>(c.top_k) * c.f;
+}
+
+bool fused_supported(const mf_moe& h, const mf_moe_layer_weights& w, const void* x, const void* y,
+                     const void* hidden) {
+  const mf_moe_config& c = h.cfg;
+  if (c.num_experts % 4 != 0) return false;  // tagged logits are read two entries per lane
   const bool combo = (c.bits == MF_BITS_4 && (!c.shared_f || c.shared_bits == MF_BITS_4)) ||
                      (c.bits == MF_BITS_2 && (!c.shared_f || c.shared_bits == MF_BITS_4 ||
                                               c.shared_bits == MF_BITS_2)) ||
                      (c.bits == MF_BITS_TERNARY && (!c.shared_f || c.shared_bits == MF_BITS_4));
   if (!combo || c.d % 8 != 0) return false;
+  if (fused_lds_bytes(c) > 150 * 1024) return false;
+  {  // rows of one token a workgroup owns must fit the h1 array
+    const uint32_t epl = c.bits == MF_BITS_4 ? 32 : 64;
+    const uint32_t rpw = 64u >> lanes_per_row_log2_dev(c.f, epl);
+    const uint32_t rg = (c.d + rpw - 1) / rpw, ub = kFusedWaves / c.top_k;
+    const uint32_t G = static_cast<uint32_t>(h.ctx->num_cu);
+    const uint32_t rounds = (rg + G * ub - 1) / (G * ub);
+    if (rounds * ub * rpw > kMaxH1) return false;
+  }
   const uint32_t offs = w.offsets.gate_w | w.offsets.up_w | w.offsets.down_w;
   if (!aligned16(w.expert_base) || w.expert_stride % 16 || offs % 16) return false;
   if (!aligned16(w.router_w) || !aligned16(x) || !aligned16(y)) return false;
@@ -448,12 +549,11 @@ hipError_t launch_fused_decode(hipStream_t s, const mf_moe& h, const mf_moe_laye
   a.hidden = hidden;
   a.out_idx = out_idx;
   a.out_w = out_w;
-  a.logits = h.ws.logits;
-  a.acts = h.ws.acts;
-  a.shared_act = h.ws.shared_act;
-  a.shared_y = h.ws.shared_y;
-  a.gate = reinterpret_cast<float*>(h.ws.gate);
-  a.sync = h.ws.sync;
+  a.t_logits = h.ws.t_logits;
+  a.t_sact = h.ws.t_sact;
+  a.t_acts = h.ws.t_acts;
+  a.epoch = h.ws.epoch;
+  a.status = h.ws.status;
   a.trace = h.trace;
   a.D = c.d;
   a.F = c.f;
@@ -464,7 +564,17 @@ hipError_t launch_fused_decode(hipStream_t s, const mf_moe& h, const mf_moe_laye
   a.router_mode = c.router_mode;
   a.limit = c.swiglu_limit;
   const dim3 grid(static_cast<uint32_t>(h.ctx->num_cu)), block(kFusedThreads);
-#define MF_FUSED(B, SB) fused_decode_kernel<B, SB><<<grid, block, 0, s>>>(a)
+  const size_t lds = fused_lds_bytes(c);
+#define MF_FUSED(B, SB)                                                                             \
+  do {                                                                                              \
+    if (lds > 48 * 1024) {                                                                          \
+      hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(fused_decode_kernel<B, SB>), \
+                                         hipFuncAttributeMaxDynamicSharedMemorySize,                \
+                                         static_cast<int>(lds));                                    \
+      if (e != hipSuccess) return e;                                                                \
+    }                                                                                               \
+    fused_decode_kernel<B, SB><<<grid, block, lds, s>>>(a);                                         \
+  } while (0)
   if (c.bits == MF_BITS_4) MF_FUSED(kBits4, kBits4);
   else if (c.bits == MF_BITS_2 && c.shared_f && c.shared_bits == MF_BITS_2) MF_FUSED(kBits2, kBits2);
   else if (c.bits == MF_BITS_2) MF_FUSED(kBits2, kBits4);

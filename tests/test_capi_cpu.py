@@ -1,0 +1,115 @@
+"""CPU-side checks of the C ABI: libmfmoe.so loads, exports every symbol that
+include/mfmoe.h declares, rejects bad arguments without launching, and its host
+grouping twin reproduces the reference's integer KATs.  No GPU, no compute."""
+import ctypes as C
+import os
+import re
+
+import numpy as np
+import pytest
+
+from mference_amd import _capi
+from mference_amd import operators as ops
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+HEADER = os.path.join(ROOT, "include", "mfmoe.h")
+
+
+def declared_symbols():
+    text = open(HEADER).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(mf_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_library_exports_every_declared_symbol():
+    lib = C.CDLL(_capi.LIB_PATH)
+    names = declared_symbols()
+    assert len(names) >= 20
+    for name in names:
+        assert hasattr(lib, name), f"{name} is declared in mfmoe.h but not exported"
+    # and the ctypes table covers the same set
+    assert sorted(_capi.SIGNATURES) == names
+
+
+def test_every_entry_point_cites_the_reference():
+    text = open(HEADER).read()
+    for name in declared_symbols():
+        pos = text.index(name + "(")
+        comment = text[:pos].rsplit("/*", 1)[-1]
+        assert ".swift" in comment or ".metal" in comment or "No counterpart" in comment \
+            or "no counterpart" in comment or name in ("mf_ctx_destroy", "mf_status_string",
+                                                       "mf_last_hip_error", "mf_abi_version",
+                                                       "mf_moe_destroy", "mf_ctx_num_cu"), name
+
+
+def test_status_strings_and_bad_arguments():
+    lib = _capi.lib()
+    assert lib.mf_abi_version() >= 1
+    assert lib.mf_status_string(0) == b"ok"
+    assert b"tileExpertCount" in lib.mf_status_string(-13)
+    q = _capi.QTensor(None, None, None)
+    # null context / null pointers: invalid argument, nothing launched
+    assert lib.mf_gemv(None, None, q, 4, None, None, 8, 64, 1, 0) == -1
+    assert lib.mf_dequantize(None, None, q, 1, 64, 4, None) == -1
+    assert lib.mf_moe_router(None, None, None, None, 1, 64, None, None, None) == -1
+    h = C.c_void_p()
+    assert lib.mf_moe_create(None, None, C.byref(h)) == -1
+    with pytest.raises(ops.MfError) as ei:
+        _capi.check(-2)
+    assert ei.value.name == "MF_ERR_DIMENSION_MISMATCH"
+
+
+KAT_PAIRS = [(0, 3, 0, 10), (0, 1, 1, 11), (0, 4, 2, 12), (1, 1, 0, 13), (1, 3, 1, 14), (1, 2, 2, 15),
+             (2, 4, 0, 16), (2, 3, 1, 17), (2, 1, 2, 18), (3, 5, 0, 19), (3, 1, 1, 20), (3, 4, 2, 21)]
+G = ops.PrefillMoEGrouping
+
+
+def test_grouping_kat_through_the_library():
+    # PrefillMoEGroupingTests.swift:5-53
+    g = G.group_token_expert_pairs(KAT_PAIRS[::-1], 4, 3, 6, tile_expert_count=2)
+    assert list(g.sorted_pairs["expert"]) == [1, 1, 1, 1, 2, 3, 3, 3, 4, 4, 4, 5]
+    assert list(g.per_expert_offsets) == [0xFFFFFFFF, 0, 4, 5, 8, 11]
+    assert list(g.per_expert_counts) == [0, 4, 1, 3, 3, 1]
+    assert [tuple(x) for x in g.groups] == [(1, 0, 4), (2, 4, 1), (3, 5, 3), (4, 8, 3), (5, 11, 1)]
+    assert [tuple(x) for x in g.tiles] == [(0, 2, 0, 5), (2, 2, 5, 6), (4, 1, 11, 1)]
+    assert (g.max_pairs_per_expert, g.max_pairs_per_tile, g.max_live_experts_per_tile) == (4, 6, 2)
+
+
+def test_grouping_errors_carry_the_reference_payloads():
+    # PrefillMoEGroupingTests.swift:117-173
+    cases = [
+        (dict(pairs=[(0, 0, 0, 1)], q=1, k=1, e=1, tile=17), "MF_ERR_TILE_EXPERT_COUNT", None),
+        (dict(pairs=[(0, 2, 0, 1)], q=1, k=1, e=2, tile=1), "MF_ERR_EXPERT_RANGE", (2, 0)),
+        (dict(pairs=[(0, 0, 0, 1), (0, 1, 0, 2)], q=1, k=2, e=2, tile=1),
+         "MF_ERR_DUPLICATE_TOKEN_RANK", (0, 0)),
+        (dict(pairs=[(0, 0, 0, 1)], q=1, k=1, e=2, tile=1, keys=[0]), "MF_ERR_SORT_KEY_COUNT", (2, 1)),
+        (dict(pairs=[(0, 0, 0, 1)], q=2, k=1, e=2, tile=1), "MF_ERR_PAIR_COUNT", (2, 1)),
+        (dict(pairs=[(5, 0, 0, 1)], q=1, k=1, e=2, tile=1), "MF_ERR_TOKEN_RANGE", (5, 0)),
+        (dict(pairs=[(0, 0, 3, 1)], q=1, k=1, e=2, tile=1), "MF_ERR_RANK_RANGE", (3, 0)),
+        (dict(pairs=[], q=-1, k=1, e=2, tile=1), "MF_ERR_QUERY_COUNT", None),
+        (dict(pairs=[], q=0, k=0, e=2, tile=1), "MF_ERR_TOPK", None),
+        (dict(pairs=[], q=0, k=1, e=0, tile=1), "MF_ERR_NUM_EXPERTS", None),
+    ]
+    for c, name, detail in cases:
+        with pytest.raises(ops.MfError) as ei:
+            G.group_token_expert_pairs(c["pairs"], c["q"], c["k"], c["e"], c["tile"], c.get("keys"))
+        assert ei.value.name == name
+        if detail is not None:
+            assert ei.value.detail == detail
+
+
+def test_grouping_matches_the_oracle_on_random_routes(oracle):
+    rng = np.random.default_rng(5)
+    for t, k, e, tile in [(1, 8, 256, 16), (32, 8, 128, 16), (128, 6, 64, 3), (0, 2, 4, 1)]:
+        idx = np.stack([rng.permutation(e)[:k] for _ in range(t)]).astype(np.uint32) if t else \
+            np.zeros((0, k), np.uint32)
+        wb = rng.integers(0, 2 ** 32, size=(t, k), dtype=np.uint32)
+        pairs = G.make_token_expert_pairs(idx, wb, t, k)
+        assert np.array_equal(pairs, oracle.make_pairs(idx, wb)) if t else pairs.size == 0
+        shuffled = pairs[rng.permutation(pairs.size)]
+        g = G.group_token_expert_pairs(shuffled, t, k, e, tile)
+        ref = oracle.group_pairs(shuffled, t, k, e, tile)
+        assert np.array_equal(g.sorted_pairs, ref["sorted"])
+        assert np.array_equal(g.per_expert_offsets, ref["offsets"][:e])
+        assert np.array_equal(g.per_expert_counts, ref["counts"][:e])
+        assert np.array_equal(g.groups, ref["groups"]) and np.array_equal(g.tiles, ref["tiles"])

@@ -1,0 +1,456 @@
+"""Pins the CPU oracle (oracle/) against what the reference's own tests hold for
+this path and against what the mathematics fixes.  No GPU.
+
+Each block names the reference test it follows (paths relative to the Mference
+repository root).  None of these checks re-types the oracle's formula: they are
+published constants, literal integer KATs, invariants, or an independent fp64
+numpy composition.
+"""
+import math
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import mf_oracle as O
+
+
+# ------------------------------------------------------------------ generators
+
+def test_splitmix64_published_vectors():
+    # first outputs of the public-domain splitmix64.c for seeds 0 and 1234567
+    r = O.Rng(0)
+    assert [r.next() for _ in range(3)] == [0xE220A8397B1DCDAF, 0x6E789E6AA1B965F4,
+                                            0x06C45D188009454F]
+    r = O.Rng(1234567)
+    assert [r.next() for _ in range(3)] == [6457827717110365317, 3203168211198807973,
+                                            9817491932198370423]
+
+
+def test_seed_tree_is_fnv1a64_of_label():
+    # published FNV-1a 64 test vectors: "" , "a", "foobar"
+    for label, h in (("", 0xCBF29CE484222325), ("a", 0xAF63DC4C8601EC8C),
+                     ("foobar", 0x85944171F73967E8)):
+        root = 0x1234_5678_9ABC_DEF0
+        assert O.Rng.key(root, label).next() == O.Rng(root ^ h).next()
+
+
+def test_uniform_is_24_bit_and_in_range():
+    r, r2 = O.Rng(42), O.Rng(42)
+    for _ in range(100):
+        u = r.uniform(-1.0, 3.0)
+        bits = r2.next() >> 40
+        assert u == np.float32(-1.0) + np.float32(4.0) * (np.float32(bits) / np.float32(1 << 24))
+        assert -1.0 <= u < 3.0
+
+
+# ------------------------------------------------------------------------ bf16
+
+def test_bf16_matches_torch_rne():
+    rng = np.random.default_rng(0)
+    x = np.concatenate([rng.standard_normal(20000).astype(np.float32) * 10.0 ** rng.integers(-30, 30, 20000),
+                        np.array([0.0, -0.0, 1.0, -1.0, 0.5, 1 / 3, 12345.0, 1e-30, 3.25], np.float32)])
+    want = torch.from_numpy(x).to(torch.bfloat16).view(torch.int16).numpy().view(np.uint16)
+    assert np.array_equal(O.bf16_bits(x), want)
+    back = O.bf16_to_float(want)
+    assert np.array_equal(back, torch.from_numpy(want.view(np.int16)).view(torch.bfloat16).float().numpy())
+    # QuantizationAffineTests.swift:48-58: relative error <= 2^-7 on the listed values
+    for v in [0.0, 1.0, -1.0, 0.5, -0.5, 1.0 / 3.0, 12345.0]:
+        b = float(O.bf16_to_float(O.bf16_bits(np.array([v], np.float32)))[0])
+        assert abs(b - v) / max(abs(v), 1e-6) < 8e-3
+
+
+# ------------------------------------------------------------------- quantizer
+
+def _np_unpack(q):
+    """independent numpy unpack of packed codes -> [rows, n] integer codes"""
+    p = q.packed.astype(np.uint32)
+    if q.bits == 4:
+        codes = np.empty((q.rows, q.n), np.uint32)
+        codes[:, 0::2] = p & 0xF
+        codes[:, 1::2] = p >> 4
+    else:
+        codes = np.empty((q.rows, q.n), np.uint32)
+        for j in range(4):
+            codes[:, j::4] = (p >> (2 * j)) & 3
+    return codes
+
+
+def _np_dequant64(q):
+    s = O.bf16_to_float(q.scales).astype(np.float64)
+    b = -s if q.biases is None else O.bf16_to_float(q.biases).astype(np.float64)
+    codes = _np_unpack(q).astype(np.float64)
+    return codes * np.repeat(s, 64, axis=1) + np.repeat(b, 64, axis=1)
+
+
+def test_nibble_layout_low_even_high_odd():
+    # QuantizationTests.swift:35-50
+    row = (np.arange(64, dtype=np.float32) - 31.5).reshape(1, 64)
+    q = O.quantize(row, 4)
+    s = O.bf16_to_float(q.scales)[0, 0]
+    b = O.bf16_to_float(q.biases)[0, 0]
+    lo, hi = int(q.packed[0, 0] & 0xF), int(q.packed[0, 0] >> 4)
+    assert abs(lo * s + b - row[0, 0]) <= s + 1e-3
+    assert abs(hi * s + b - row[0, 1]) <= s + 1e-3
+    assert lo == 0 and hi == 0 or hi >= lo  # monotone input -> monotone codes
+
+
+def test_constant_group_reconstructs_bf16_value_exactly():
+    # QuantizationAffineTests.swift:61-72
+    q = O.quantize(np.full((1, 64), 0.42, np.float32), 4)
+    r = O.dequantize(q)
+    want = O.bf16_to_float(O.bf16_bits(np.array([0.42], np.float32)))[0]
+    assert np.all(r == want)
+    assert O.bf16_to_float(q.scales)[0, 0] == 1.0
+
+
+def test_positive_only_range_uses_full_codebook():
+    # QuantizationAffineTests.swift:76-88
+    row = (np.arange(64, dtype=np.float32) / np.float32(63.0) + np.float32(1.0)).reshape(1, 64)
+    codes = _np_unpack(O.quantize(row, 4))
+    assert codes.min() == 0 and codes.max() == 15
+
+
+def test_roundtrip_bounds():
+    # QuantizationAffineTests.swift:10-30 and DequantInt4GEMVReferenceTests.swift:59-76
+    row = np.concatenate([0.10 + np.arange(64) * 0.01, -0.50 - np.arange(64) * 0.005]).astype(np.float32)
+    r = O.dequantize(O.quantize(row.reshape(1, -1), 4))[0]
+    assert np.abs(r - row).max() < 0.025
+    for n in (128, 256, 2816):
+        raw = O.Rng.key(0xF5, f"int4-affine-roundtrip-n{n}").uniform_fill(-1.0, 1.0, n).reshape(1, n)
+        q = O.quantize(raw, 4)
+        rec = O.dequantize(q)
+        bound = np.repeat(O.bf16_to_float(q.scales), 64, axis=1) + 1e-4
+        assert np.all(np.abs(rec - raw) <= bound)
+
+
+@pytest.mark.parametrize("bits", [4, 8])
+def test_codes_are_nearest_levels(bits):
+    """brute force: every stored code is the nearest of the 2^bits levels q*s+b"""
+    raw = O.Rng.key(0x51A71001, "int4-affine-round-trip").uniform_fill(-1.0, 1.0, 4 * 256).reshape(4, 256)
+    q = O.quantize(raw, bits)
+    s = np.repeat(O.bf16_to_float(q.scales), 64, axis=1).astype(np.float64)
+    b = np.repeat(O.bf16_to_float(q.biases), 64, axis=1).astype(np.float64)
+    codes = q.packed.astype(np.int64) if bits == 8 else _np_unpack(q).astype(np.int64)
+    levels = np.arange(2 ** bits, dtype=np.float64)
+    dist = np.abs(raw.astype(np.float64)[..., None] - (levels * s[..., None] + b[..., None]))
+    best = dist.min(axis=-1)
+    mine = np.take_along_axis(dist, codes[..., None], axis=-1)[..., 0]
+    assert np.all(mine <= best + 1e-6 * np.abs(s))  # ties/rounding of (w-b)*inv allow 1 ulp slack
+
+
+def test_quantizer_edge_cases():
+    # Int4AffineEncoderParityTests.swift:41-51: the edge list quantizes to sane codes
+    cases = [np.zeros(64), np.full(128, 3.25), np.arange(64) * 1e-30,
+             np.where(np.arange(64) == 0, -1e4, 1e4), -np.arange(64) - 1.0,
+             np.concatenate([np.full(64, -2.0), np.arange(64) / 7.0])]
+    for c in cases:
+        row = c.astype(np.float32).reshape(1, -1)
+        q = O.quantize(row, 4)
+        rec = O.dequantize(q)
+        s = np.repeat(O.bf16_to_float(q.scales), 64, axis=1)
+        tol = np.maximum(s, 1e-30) + np.abs(row) * 2.0 ** -7 + 1e-30
+        assert np.all(np.abs(rec - row) <= tol), c[:4]
+    # all-zero group: scale 1, bias 0, codes 0 (constant-group rule)
+    q = O.quantize(np.zeros((1, 64), np.float32), 4)
+    assert q.scales[0, 0] == 0x3F80 and q.biases[0, 0] == 0 and not q.packed.any()
+
+
+def test_tensor_equals_row_by_row():
+    # Int4AffineEncoderParityTests.swift:53-79 (LCG values)
+    state = 0xC0FFEE
+    vals = []
+    for _ in range(6 * 192):
+        state = (state * 6364136223846793005 + 1442695040888963407) & 0xFFFFFFFFFFFFFFFF
+        vals.append((np.float32(state >> 40) / np.float32(1 << 24) - np.float32(0.5)) * np.float32(2))
+    w = np.array(vals, np.float32).reshape(6, 192)
+    full = O.quantize(w, 4)
+    for r in range(6):
+        one = O.quantize(w[r:r + 1], 4)
+        assert np.array_equal(one.packed[0], full.packed[r])
+        assert np.array_equal(one.scales[0], full.scales[r])
+        assert np.array_equal(one.biases[0], full.biases[r])
+
+
+# --------------------------------------------------------------------- dequant
+
+def test_dequant_is_two_rounding_closed_form():
+    raw = O.Rng(7).uniform_fill(-3.0, 3.0, 5 * 128).reshape(5, 128)
+    for bits in (4, 2):
+        q = O.quantize(raw, bits)
+        s = np.repeat(O.bf16_to_float(q.scales), 64, axis=1)
+        b = np.repeat(O.bf16_to_float(q.biases), 64, axis=1)
+        want = (_np_unpack(q).astype(np.float32) * s).astype(np.float32) + b  # numpy fp32: 2 roundings
+        assert np.array_equal(O.dequantize(q).view(np.uint32), want.astype(np.float32).view(np.uint32))
+
+
+def test_two_bit_element_order_hand_built():
+    # moe.metal:948-951: byte k holds elements 4k..4k+3, element j at bit 2*(j%4)
+    codes = np.array([[(r * 5 + i * 3) & 3 for i in range(64)] for r in range(3)], np.uint8)
+    packed = O.pack_codes(codes, 2)
+    assert packed[0, 0] == (codes[0, 0] | codes[0, 1] << 2 | codes[0, 2] << 4 | codes[0, 3] << 6)
+    q = O.QTensor(packed, O.bf16_bits(np.full((3, 1), 0.5, np.float32)),
+                  O.bf16_bits(np.full((3, 1), -1.0, np.float32)), 2, 3, 64)
+    assert np.array_equal(O.dequantize(q), codes.astype(np.float32) * 0.5 - 1.0)
+
+
+def test_ternary_is_scale_times_minus_one_zero_one():
+    # RepackPlanner.swift:629,640 / MapleMoETests.swift:327-332: bias = -scale
+    codes = np.array([[i % 3 for i in range(128)]], np.uint8)
+    q = O.QTensor(O.pack_codes(codes, 1), O.bf16_bits(np.array([[0.25, 0.5]], np.float32)), None, 1, 1, 128)
+    want = (codes.astype(np.float32) - 1.0) * np.repeat(np.array([[0.25, 0.5]], np.float32), 64, axis=1)
+    assert np.array_equal(O.dequantize(q), want)
+
+
+# ------------------------------------------------------------------------- exp
+
+def test_exp_close_to_libm_and_clamped():
+    xs = np.concatenate([np.linspace(-85.9, 87.9, 4001), np.array([0.0, -0.0, 1e-8, -1e-8])])
+    for x in xs:
+        x = float(np.float32(x))
+        got, want = O.exp(x), math.exp(x)
+        assert abs(got - want) <= 3e-7 * want
+    assert O.exp(-86.5) == 0.0 and O.exp(-1e30) == 0.0 and O.exp(float("-inf")) == 0.0
+    assert O.exp(89.0) == float("inf") and math.isnan(O.exp(float("nan")))
+    assert O.exp(0.0) == 1.0
+    assert abs(O.silu(1.5) - 1.5 / (1 + math.exp(-1.5))) < 1e-6 and O.silu(-100.0) == -0.0
+
+
+# ---------------------------------------------------------------------- router
+
+def test_router_logits_against_fp64_and_unit_vectors():
+    e, d = 16, 256
+    rng = O.Rng(0xA5B61234)
+    w = O.bf16_bits((rng.uniform_fill(-0.05, 0.05, e * d)).reshape(e, d))
+    x = O.bf16_bits(rng.uniform_fill(-1.0, 1.0, d))
+    ref = O.bf16_to_float(w).astype(np.float64) @ O.bf16_to_float(x).astype(np.float64)
+    got = O.router_logits(w, x)
+    assert np.abs(got - ref).max() <= 1e-6 * np.abs(ref).max() + 1e-7
+    for i in (0, 7, 8, 63, 64, 255):  # x = e_i returns column i exactly
+        unit = np.zeros(d, np.uint16)
+        unit[i] = 0x3F80
+        assert np.array_equal(O.router_logits(w, unit), O.bf16_to_float(w[:, i]))
+    ones = np.full(d, 0x3F80, np.uint16)  # exactly representable weights: sum is exact
+    wi = O.bf16_bits(np.tile(np.arange(-8, 8, dtype=np.float32), (e, d // 16)))
+    assert np.array_equal(O.router_logits(wi, ones), np.full(e, -8.0 * (d // 16), np.float32))
+
+
+def _tie_logits(count, trial, rng):
+    # RouterTopKParityTests.swift:109-127
+    kind = trial % 4
+    if kind == 0:
+        return np.array([rng.uniform(-4.0, 4.0) for _ in range(count)], np.float32)
+    if kind == 1:
+        return np.array([np.round(np.float32(rng.uniform(-3.0, 3.0)) * np.float32(4)) / np.float32(4)
+                         for _ in range(count)], np.float32)
+    if kind == 2:
+        levels = [1.5, 0.5, -0.5]
+        return np.array([levels[rng.next() % 3] for _ in range(count)], np.float32)
+    return np.full(count, 0.75, np.float32)
+
+
+@pytest.mark.parametrize("e", [8, 16, 24, 33, 100, 128, 168, 255, 256])
+def test_topk_equals_sort_by_score_desc_index_asc(e):
+    # RouterTopKParityTests.swift:34 seeds + RouterTopKTests.swift:86-96 reference
+    rng = O.Rng(0x5EED0001 + e)
+    k = 8
+    for trial in range(12):
+        logits = _tie_logits(e, trial, rng)
+        for _ in range(e):
+            rng.uniform(0.6, 1.4)
+        idx, w = O.topk_softmax(logits, k)
+        order = sorted(range(e), key=lambda i: (-float(logits[i]), i))[:k]
+        assert list(idx) == order
+        sel = logits[order].astype(np.float64)
+        want = np.exp(sel - sel[0])
+        want /= want.sum()
+        assert np.abs(w - want).max() < 5e-7
+        assert abs(float(w.sum()) - 1.0) < 2e-6
+
+
+def test_full_softmax_router_on_the_tied_fixture():
+    # MapleMoETests.swift:24-40: deliberate score ties {3,55},{7,63},{11,71},{19,95}
+    logits = np.full(256, -4.0, np.float32)
+    for i, s in {3: 8, 55: 8, 7: 7, 63: 7, 11: 6, 71: 6, 19: 5, 95: 5}.items():
+        logits[i] = s
+    idx, w = O.topk_softmax(logits, 8, full_softmax=True)
+    assert list(idx) == [3, 55, 7, 63, 11, 71, 19, 95]
+    p = np.exp(logits.astype(np.float64) - 8.0)
+    p /= p.sum()
+    want = p[idx] / p[idx].sum()
+    assert np.abs(w - want).max() <= 2e-6 and abs(float(w.sum()) - 1) <= 2e-6
+    for bad in (np.nan, np.inf, -np.inf):  # MapleMoETests.swift:141-185: sentinels
+        l2 = logits.copy()
+        l2[0] = bad
+        idx, w = O.topk_softmax(l2, 8, full_softmax=True)
+        assert list(idx) == [256] * 8 and not w.any()
+
+
+def test_topk_fewer_experts_than_k_keeps_index_zero():
+    idx, w = O.topk_softmax(np.array([1.0, 3.0, 2.0], np.float32), 8)
+    assert list(idx[:3]) == [1, 2, 0] and list(idx[3:]) == [0] * 5 and not w[3:].any()
+
+
+# ------------------------------------------------------------------------ GEMV
+
+@pytest.mark.parametrize("bits", [4, 2])
+@pytest.mark.parametrize("m,n,seed", [(4, 128, 0xF1), (8, 256, 0xF2), (16, 512, 0xF3), (32, 2816, 0xF4)])
+def test_gemv_matches_fp64_and_structure(bits, m, n, seed):
+    # shapes / seeds of DequantInt4GEMVReferenceTests.swift:32-53
+    rng = O.Rng.key(seed, f"int4-gemv-ref-m{m}-n{n}")
+    q = O.quantize(rng.uniform_fill(-1.0, 1.0, m * n).reshape(m, n), bits)
+    x = rng.uniform_fill(-1.0, 1.0, n)
+    w64 = _np_dequant64(q)
+    y = O.gemv(q, x)
+    ref = w64 @ x.astype(np.float64)
+    assert np.abs(y - ref).max() / max(np.abs(ref).max(), 1e-6) < 1e-5  # Tolerance.identity
+    unit = np.zeros(n, np.float32)
+    unit[n // 3] = 1.0
+    assert np.array_equal(O.gemv(q, unit), O.dequantize(q)[:, n // 3])   # x = e_i -> column i
+    ones = O.gemv(q, np.ones(n, np.float32))
+    assert np.abs(ones - w64.sum(axis=1)).max() < 1e-3                   # x = 1 -> row sums
+    y2 = O.gemv(q, (2.0 * x).astype(np.float32))                         # exact power-of-two scaling
+    assert np.array_equal(y2, 2.0 * y)
+
+
+def _np_layer64(layer, x_bits):
+    """independent fp64 composition of the layer from unpacked tensors"""
+    d, f, e, k = layer.d, layer.f, layer.e, layer.k
+    x = O.bf16_to_float(x_bits).astype(np.float64)
+    bf = lambda v: O.bf16_to_float(O.bf16_bits(np.asarray(v, np.float32))).astype(np.float64)
+    silu = lambda v: v / (1.0 + np.exp(-v))
+    logits = O.bf16_to_float(layer.router_w).astype(np.float64) @ x
+    order = sorted(range(e), key=lambda i: (-logits[i], i))[:k]
+    p = np.exp(logits[order] - logits[order[0]])
+    w = p / p.sum()
+
+    def sub(blob, name, rows, cols, bits):
+        wo, so, bo = (getattr(layer.off, f"{name}_{s}") for s in "wsb")
+        nb = rows * O.packed_row_bytes(bits, cols)
+        ns = rows * (cols // 64)
+        q = O.QTensor(blob[wo:wo + nb].reshape(rows, -1), blob[so:so + 2 * ns].view(np.uint16).reshape(rows, -1),
+                      None if bits == 1 else blob[bo:bo + 2 * ns].view(np.uint16).reshape(rows, -1),
+                      bits, rows, cols)
+        return _np_dequant64(q)
+
+    acc = np.zeros(d)
+    if layer.fs:
+        g, u, dn = (_np_dequant64(q) for q in layer.shared)
+        a = bf(silu(bf(g @ x)) * bf(u @ x))
+        hs = bf(dn @ a)
+        if layer.w_sg is not None:
+            gate = bf(O.bf16_to_float(layer.w_sg).astype(np.float64) @ x)
+            hs = bf(hs / (1.0 + np.exp(-gate)))
+        acc = hs.copy()
+    for s, ex in enumerate(order):
+        blob = layer.experts[ex]
+        g = sub(blob, "gate", f, d, layer.bits) @ x
+        u = sub(blob, "up", f, d, layer.bits) @ x
+        a = bf(silu(g) * u)
+        acc = acc + w[s] * (sub(blob, "down", d, f, layer.bits) @ a)
+    return bf(acc), order, w
+
+
+@pytest.mark.parametrize("bits,d,f,e,k,fs", [(4, 128, 64, 16, 8, 64), (4, 128, 64, 12, 6, 0),
+                                             (2, 256, 128, 8, 6, 128), (1, 256, 128, 8, 4, 0)])
+def test_layer_against_independent_fp64_composition(bits, d, f, e, k, fs):
+    # MoEFusedFFNTests.swift:44-190 shape (D 128, F 64, K in {6, 8}), tolerance
+    # fp16ChainedReduction = 1e-2 relative (Tolerances.swift:4-21)
+    root = 0x2D3
+    layer = O.synth_layer(root, d, f, e, k, bits=bits, fs=fs, sigma=0.1)
+    x = O.synth_x(root, 1, d)[0]
+    y, idx, w = O.moe_layer(layer, x)
+    ref, order, wref = _np_layer64(layer, x)
+    assert list(idx) == order
+    assert np.abs(w - wref).max() < 1e-6
+    yf = O.bf16_to_float(y).astype(np.float64)
+    assert np.abs(yf - ref).max() / max(np.abs(ref).max(), 1e-6) < 1e-2
+    assert np.linalg.norm(yf - ref) / np.linalg.norm(ref) < 1e-3
+
+
+def test_shared_expert_rounding_points():
+    # SharedExpertInt4Tests.swift:11-53 shape (D 128, F 64, seed 0x604)
+    d, f = 128, 64
+    t = O.Rng.key(0x604, "shared")
+    g, u = (O.quantize(t.uniform_fill(-0.5, 0.5, f * d).reshape(f, d), 4) for _ in range(2))
+    dn = O.quantize(t.uniform_fill(-0.5, 0.5, d * f).reshape(d, f), 4)
+    x = O.bf16_bits(t.uniform_fill(-1.0, 1.0, d))
+    y = O.bf16_to_float(O.shared_expert(g, u, dn, x)).astype(np.float64)
+    xf = O.bf16_to_float(x).astype(np.float64)
+    bf = lambda v: O.bf16_to_float(O.bf16_bits(np.asarray(v, np.float32))).astype(np.float64)
+    a = bf(bf(_np_dequant64(g) @ xf) / (1 + np.exp(-bf(_np_dequant64(g) @ xf))) * bf(_np_dequant64(u) @ xf))
+    ref = bf(_np_dequant64(dn) @ a)
+    assert np.abs(y - ref).max() / np.abs(ref).max() < 6e-3
+
+
+# -------------------------------------------------------------------- grouping
+
+KAT_PAIRS = [(0, 3, 0, 10), (0, 1, 1, 11), (0, 4, 2, 12), (1, 1, 0, 13), (1, 3, 1, 14), (1, 2, 2, 15),
+             (2, 4, 0, 16), (2, 3, 1, 17), (2, 1, 2, 18), (3, 5, 0, 19), (3, 1, 1, 20), (3, 4, 2, 21)]
+
+
+def test_grouping_kat():
+    # PrefillMoEGroupingTests.swift:5-53, literal expectations
+    pairs = np.array(KAT_PAIRS[::-1], dtype=O.PAIR_DTYPE)
+    g = O.group_pairs(pairs, 4, 3, 6, tile_expert_count=2)
+    assert list(g["sorted"]["expert"]) == [1, 1, 1, 1, 2, 3, 3, 3, 4, 4, 4, 5]
+    assert [[int(p["token"]), int(p["rank"])] for p in g["sorted"]] == [
+        [0, 1], [1, 0], [2, 2], [3, 1], [1, 2], [0, 0], [1, 1], [2, 1], [0, 2], [2, 0], [3, 2], [3, 0]]
+    assert list(g["offsets"]) == [0xFFFFFFFF, 0, 4, 5, 8, 11]
+    assert list(g["counts"]) == [0, 4, 1, 3, 3, 1]
+    assert [tuple(x) for x in g["groups"]] == [(1, 0, 4), (2, 4, 1), (3, 5, 3), (4, 8, 3), (5, 11, 1)]
+    assert [tuple(x) for x in g["tiles"]] == [(0, 2, 0, 5), (2, 2, 5, 6), (4, 1, 11, 1)]
+
+
+def test_grouping_order_independent_and_keeps_weight_bits():
+    # PrefillMoEGroupingTests.swift:55-82
+    tm = [(0, 2, 0, 101), (0, 1, 1, 102), (1, 2, 0, 103), (1, 0, 1, 104), (2, 1, 0, 105), (2, 2, 1, 106)]
+    sh = [tm[5], tm[1], tm[3], tm[0], tm[4], tm[2]]
+    a = O.group_pairs(np.array(tm, O.PAIR_DTYPE), 3, 2, 3, 2)
+    b = O.group_pairs(np.array(sh, O.PAIR_DTYPE), 3, 2, 3, 2)
+    for key in a:
+        assert np.array_equal(a[key], b[key])
+    assert list(a["sorted"]["weight_bits"]) == [104, 102, 105, 101, 103, 106]
+
+
+def test_grouping_sort_keys_and_errors():
+    # PrefillMoEGroupingTests.swift:84-173
+    pairs = np.array([(0, 1, 0, 10), (0, 2, 1, 20), (1, 3, 0, 30), (1, 1, 1, 11), (2, 2, 0, 21),
+                      (2, 3, 1, 31)], O.PAIR_DTYPE)
+    g = O.group_pairs(pairs, 3, 2, 4, 2, sort_keys=[0, 30, 10, 20])
+    assert list(g["groups"]["expert"]) == [2, 3, 1]
+    assert list(g["sorted"]["expert"]) == [2, 2, 3, 3, 1, 1]
+    assert list(g["offsets"]) == [0xFFFFFFFF, 4, 0, 2]
+    assert [tuple(x) for x in g["tiles"]] == [(0, 2, 0, 4), (2, 1, 4, 2)]
+    one = lambda *p: np.array([p], O.PAIR_DTYPE)
+    with pytest.raises(O.GroupingError) as ei:
+        O.group_pairs(one(0, 0, 0, 1), 1, 1, 1, 17)
+    assert ei.value.kind == "invalidTileExpertCount"
+    with pytest.raises(O.GroupingError) as ei:
+        O.group_pairs(one(0, 2, 0, 1), 1, 1, 2, 1)
+    assert ei.value.kind == "expertOutOfRange"
+    with pytest.raises(O.GroupingError) as ei:
+        O.group_pairs(np.array([(0, 0, 0, 1), (0, 1, 0, 2)], O.PAIR_DTYPE), 1, 2, 2, 1)
+    assert ei.value.kind == "duplicateTokenRank"
+    with pytest.raises(O.GroupingError) as ei:
+        O.group_pairs(one(0, 0, 0, 1), 1, 1, 2, 1, sort_keys=[0])
+    assert ei.value.kind == "expertSortKeyCountMismatch"
+
+
+def test_grouping_pressure_case():
+    # PrefillMoEGroupingTests.swift:175-203
+    pairs = np.array([(t, (t + r * 7) % 74, r, t * 8 + r) for t in range(32) for r in range(8)], O.PAIR_DTYPE)
+    g = O.group_pairs(pairs, 32, 8, 128, 16)
+    assert g["sorted"].size == 256 and g["groups"].size <= 74
+    assert g["tiles"]["group_count"].max() <= 16 and g["tiles"]["pair_count"].min() > 0
+    assert int(g["counts"].sum()) == 256
+
+
+def test_reduce_token_major_closed_form():
+    # PrefillMoETests.swift:46-64 (cpuReduce)
+    rng = np.random.default_rng(3)
+    part = rng.standard_normal((5, 4, 16)).astype(np.float32)
+    w = rng.random((5, 4)).astype(np.float32)
+    got = O.reduce_token_major(part, w)
+    ref = (part.astype(np.float64) * w.astype(np.float64)[..., None]).sum(axis=1)
+    assert np.abs(got - ref).max() < 2e-6

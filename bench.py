@@ -105,6 +105,18 @@ def layer_to_host(wts, w):
                    w_sg=None if wts.w_sg is None else ops.bf16_bits(wts.w_sg))
 
 
+def profiled_traffic_bytes():
+    """HBM bytes per launch of the fused kernel from the committed rocprofv3 --pmc
+    summary (FETCH_SIZE + WRITE_SIZE, scaled by a copy kernel of known size)."""
+    import re
+    path = os.path.join(ROOT, "profiles", "fused_decode_qwen_t1.md")
+    try:
+        m = re.search(r"Traffic per launch = \*\*([0-9,]+) B\*\*", open(path).read())
+        return int(m.group(1).replace(",", "")) if m else None
+    except OSError:
+        return None
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -113,6 +125,9 @@ def main() -> int:
     ap.add_argument("--layers", type=int, default=40)
     ap.add_argument("--no-graph", action="store_true", help="launch eagerly instead of a HIP graph")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--pmc-calibration", action="store_true",
+                    help="also run three 256 MiB device-to-device copies (a kernel of known HBM "
+                         "traffic) so that FETCH_SIZE / WRITE_SIZE counters can be scaled")
     ap.add_argument("--cpu-seconds", type=float, default=12.0)
     args = ap.parse_args()
     if args.gpus != 1:
@@ -222,8 +237,9 @@ def main() -> int:
         "output_finite": finite,
         "parity_layer0": parity,
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS,
-                     "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBPS, 4), "traffic": None,
-                     "kernel": "decode layer (all launches of one layer)",
+                     "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBPS, 4),
+                     "traffic": profiled_traffic_bytes(),
+                     "kernel": "mf::fused_decode_kernel (one launch per layer)",
                      "algorithmic_bytes_per_layer": ab["expert_bytes"]},
     }
 
@@ -245,6 +261,13 @@ def main() -> int:
                                "kind": "port",
                                "sample": f"{n} repetitions of layer 0 of the same workload "
                                          f"(OpenMP over weight rows, {cores} threads)"}
+    if args.pmc_calibration:
+        src = torch.zeros(256 << 20, dtype=torch.uint8, device=device)
+        dst = torch.empty_like(src)
+        for _ in range(3):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        out["pmc_calibration"] = "3 x 256 MiB device-to-device copy (reads 268435456 B, writes 268435456 B)"
     print(json.dumps(out))
     return 0
 

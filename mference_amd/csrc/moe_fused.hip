@@ -71,15 +71,20 @@ template <int BITS>
 __device__ __forceinline__ float row_partial(const uint8_t* wrow, const uint16_t* srow,
                                              const uint16_t* brow, const uint16_t* x, uint32_t N,
                                              uint32_t sub, uint32_t lpr, bool have_first,
-                                             const Chunk<BITS>& first) {
+                                             const Chunk<BITS> first) {
   constexpr uint32_t EPL = Fmt<BITS>::kElemsPer16B;
   float acc = 0.0f;
   for (uint32_t e0 = sub * EPL; e0 < N; e0 += lpr * EPL) {
-    const Chunk<BITS> c = (have_first && e0 == sub * EPL) ? first
-                                                           : load_chunk<BITS>(wrow, srow, brow, e0);
+    // plain scalars, not a struct select: the prefetched chunk must stay in registers
+    uint4 codes = first.codes;
+    float s = first.s, b = first.b;
+    if (!(have_first && e0 == sub * EPL)) {
+      codes = load_codes16<true>(wrow + static_cast<size_t>(e0) * Store<BITS>::kBits / 8);
+      load_scale_bias<BITS>(srow, brow, e0, s, b);
+    }
     const XSlice<BITS> xs = load_xslice<BITS, kXAligned>(x + e0);
-    acc = __builtin_fmaf(c.s, codes_dot<BITS>(c.codes, xs), acc);
-    acc = __builtin_fmaf(c.b, xs.sum, acc);
+    acc = __builtin_fmaf(s, codes_dot<BITS>(codes, xs), acc);
+    acc = __builtin_fmaf(b, xs.sum, acc);
   }
   return acc;
 }
@@ -193,10 +198,28 @@ __device__ __forceinline__ void trace_mark(const FusedArgs& a, uint32_t slot) {
   if (a.trace && threadIdx.x == 0) a.trace[blockIdx.x * 8 + slot] = wall_clock64();
 }
 
-template <int BITS, int SBITS>
+// Shape specialisation (the reference's FC_MOE_D / FC_MOE_F / FC_MOE_TOP_K function
+// constants, moe.metal:13-16): a StaticShape turns every dimension into a
+// compile-time constant, which unrolls the row loops and removes most of the
+// control flow -- the launch executes each instruction once per wave, so code
+// size is instruction-fetch latency.  RuntimeShape reads the dimensions from
+// the arguments and handles everything else.
+struct RuntimeShape {
+  static constexpr bool kStatic = false;
+  static constexpr uint32_t D = 0, F = 0, E = 0, K = 0, T = 0, Fs = 0;
+};
+template <uint32_t D_, uint32_t F_, uint32_t E_, uint32_t K_, uint32_t T_, uint32_t Fs_>
+struct StaticShape {
+  static constexpr bool kStatic = true;
+  static constexpr uint32_t D = D_, F = F_, E = E_, K = K_, T = T_, Fs = Fs_;
+};
+
+template <int BITS, int SBITS, class S>
 __global__ __launch_bounds__(kFusedThreads) void fused_decode_kernel(const FusedArgs a) {
   extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
-  const uint32_t D = a.D, F = a.F, E = a.E, K = a.K, T = a.T, Fs = a.Fs;
+  const uint32_t D = S::kStatic ? S::D : a.D, F = S::kStatic ? S::F : a.F;
+  const uint32_t E = S::kStatic ? S::E : a.E, K = S::kStatic ? S::K : a.K;
+  const uint32_t T = S::kStatic ? S::T : a.T, Fs = S::kStatic ? S::Fs : a.Fs;
   // LDS carve-up (the launcher sizes it with fused_lds_bytes)
   uint32_t* s_idx = reinterpret_cast<uint32_t*>(smem);                 // [8*8]
   float* s_w = reinterpret_cast<float*>(smem + 256);                    // [8*8]
@@ -565,20 +588,27 @@ hipError_t launch_fused_decode(hipStream_t s, const mf_moe& h, const mf_moe_laye
   a.limit = c.swiglu_limit;
   const dim3 grid(static_cast<uint32_t>(h.ctx->num_cu)), block(kFusedThreads);
   const size_t lds = fused_lds_bytes(c);
-#define MF_FUSED(B, SB)                                                                             \
-  do {                                                                                              \
-    if (lds > 48 * 1024) {                                                                          \
-      hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(fused_decode_kernel<B, SB>), \
-                                         hipFuncAttributeMaxDynamicSharedMemorySize,                \
-                                         static_cast<int>(lds));                                    \
-      if (e != hipSuccess) return e;                                                                \
-    }                                                                                               \
-    fused_decode_kernel<B, SB><<<grid, block, lds, s>>>(a);                                         \
+#define MF_FUSED(B, SB, SHAPE)                                                                 \
+  do {                                                                                         \
+    auto kern = fused_decode_kernel<B, SB, SHAPE>;                                             \
+    if (lds > 48 * 1024) {                                                                     \
+      hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),                  \
+                                         hipFuncAttributeMaxDynamicSharedMemorySize,           \
+                                         static_cast<int>(lds));                               \
+      if (e != hipSuccess) return e;                                                           \
+    }                                                                                          \
+    kern<<<grid, block, lds, s>>>(a);                                                          \
   } while (0)
-  if (c.bits == MF_BITS_4) MF_FUSED(kBits4, kBits4);
-  else if (c.bits == MF_BITS_2 && c.shared_f && c.shared_bits == MF_BITS_2) MF_FUSED(kBits2, kBits2);
-  else if (c.bits == MF_BITS_2) MF_FUSED(kBits2, kBits4);
-  else MF_FUSED(kBitsTernary, kBits4);
+  using QwenT1 = StaticShape<2048, 512, 256, 8, 1, 512>;
+  const bool qwen_t1 = c.bits == MF_BITS_4 && c.shared_bits == MF_BITS_4 && c.d == 2048 &&
+                       c.f == 512 && c.num_experts == 256 && c.top_k == 8 && c.shared_f == 512 &&
+                       t == 1 && c.router_mode == MF_ROUTER_TOPK_SOFTMAX;
+  if (qwen_t1) MF_FUSED(kBits4, kBits4, QwenT1);
+  else if (c.bits == MF_BITS_4) MF_FUSED(kBits4, kBits4, RuntimeShape);
+  else if (c.bits == MF_BITS_2 && c.shared_f && c.shared_bits == MF_BITS_2)
+    MF_FUSED(kBits2, kBits2, RuntimeShape);
+  else if (c.bits == MF_BITS_2) MF_FUSED(kBits2, kBits4, RuntimeShape);
+  else MF_FUSED(kBitsTernary, kBits4, RuntimeShape);
 #undef MF_FUSED
   return hipGetLastError();
 }

@@ -249,3 +249,32 @@ def test_two_phase_matches_oracle_and_fused(gpu, oracle):
         ma, rl = errors(oracle.bf16_to_float(ops.bf16_bits(acts[0, s])), oracle.bf16_to_float(ref_act))
         assert rl < 1e-3
     assert_layer_close(oracle.bf16_to_float(ops.bf16_bits(y)), oracle.bf16_to_float(ref_y), "two-phase")
+
+
+def test_qwen_shape_specialised_launch(gpu, oracle):
+    """the full Qwen3.6-shaped layer (D 2048, F 512, E 256, K 8, shared 512) takes the
+    shape-specialised fused kernel; weights drawn and quantized on the GPU as bench.py does"""
+    import bench
+    w = dict(bench.QWEN)
+    stack = bench.build_stack(gpu, w, 1, torch.device("cuda", 0))
+    host = bench.layer_to_host(stack[0], w)
+    moe = ops.MoE(gpu, w["d"], w["f"], w["e"], w["k"], bits=4, shared_f=w["fs"])
+    gen = torch.Generator(device="cuda")
+    gen.manual_seed(1234)
+    outs = {}
+    for rep in range(3):
+        x = torch.randn((1, w["d"]), generator=gen, device="cuda").to(torch.bfloat16)
+        ref_y, ref_idx, ref_w = oracle.moe_layer(host, ops.bf16_bits(x))
+        for fused in (True, False):
+            moe.set_fused(fused)
+            y = torch.zeros_like(x)
+            idx = torch.zeros((1, w["k"]), dtype=torch.int32, device="cuda")
+            rw = torch.zeros((1, w["k"]), dtype=torch.float32, device="cuda")
+            moe.encode_decode_layer(stack[0], x, y, out_indices=idx, out_weights=rw)
+            moe.status()
+            assert np.array_equal(idx.cpu().numpy().astype(np.uint32), ref_idx)
+            assert np.array_equal(rw.cpu().numpy().view(np.uint32), ref_w.view(np.uint32))
+            assert_layer_close(oracle.bf16_to_float(ops.bf16_bits(y)), oracle.bf16_to_float(ref_y),
+                               f"qwen shape fused={fused}")
+            outs[fused] = ops.bf16_bits(y)
+        assert np.array_equal(outs[True], outs[False])

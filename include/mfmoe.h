@@ -254,6 +254,24 @@ mf_status mf_moe_status(mf_moe* h, mf_stream stream);
 
 /* ------------------------------------------------------- ragged prefill */
 
+/* PrefillRouter.makeTokenExpertPairs + PrefillMoEGrouping.groupTokenExpertPairs
+ * (Kernels/Prefill/MoE/PrefillRouter.swift:91-111, PrefillMoEGrouping.swift:
+ * 91-192) on device with no host readback: histogram, exclusive scan and stable
+ * scatter.  idx [t, top_k] and w [t, top_k] as written by mf_moe_router.
+ * Outputs: sorted pairs [t*top_k] ordered by (expert, token, rank);
+ * expert_offsets [num_experts] (0xFFFFFFFF for an expert with no token);
+ * expert_counts [num_experts].  Routes whose idx >= num_experts are invalid
+ * and make the call's device-side status word non-zero (checked by
+ * mf_moe_group_status). */
+mf_status mf_moe_group(mf_moe* h, mf_stream stream, const uint32_t* idx, const float* w,
+                       uint32_t t, mf_pair* sorted_pairs, uint32_t* expert_offsets,
+                       uint32_t* expert_counts);
+/* Synchronises the stream and maps the device status word of the last
+ * mf_moe_group to MF_OK / MF_ERR_EXPERT_RANGE: the device-side form of
+ * PrefillMoEGroupingError.expertOutOfRange (PrefillMoEGrouping.swift:60, 131),
+ * which the reference throws from its host loop. */
+mf_status mf_moe_group_status(mf_moe* h, mf_stream stream);
+
 /* PrefillMoEGrouping.groupTokenExpertPairs (Kernels/Prefill/MoE/
  * PrefillMoEGrouping.swift:91-192) with the reference's full result and error
  * contract, on HOST pointers: pairs sorted by (sort key, expert, token, rank),
@@ -267,6 +285,22 @@ mf_status mf_group_pairs_host(const mf_pair* pairs, size_t n_pairs, int query_co
                               uint32_t* offsets, uint32_t* counts, mf_group* groups,
                               size_t* n_groups, mf_tile* tiles, size_t* n_tiles,
                               uint32_t err_detail[2]);
+
+/* Ragged prefill layer: router -> device grouping -> per-expert gather-QMM
+ * (4-bit codes expanded to exact bf16 in registers, bf16 MFMA, per-group fp32 scale) ->
+ * SwiGLU -> down-proj -> weighted un-permute, + shared expert.  Replaces
+ * PrefillGroupedRoutedMoE.encodeStreamedBatched (Kernels/Prefill/MoE/
+ * PrefillGroupedRoutedMoE.swift:392-466) + PrefillMoE.encodeReduceTokenMajor
+ * (PrefillMoE.swift:11-38) + PrefillSharedExpert.encodeBlock/encodeQwenScalarGate
+ * (PrefillSharedExpert.swift:81-99, 27-36).  Result per token equals
+ * mf_moe_decode_layer on that token within the layer tolerance.
+ * Any t >= 1; 4-bit experts only (MF_ERR_UNSUPPORTED_BITS otherwise); d, f, shared_f
+ * multiples of 128; x, y and every weight tensor 16-byte aligned.
+ * workspace: device scratch of at least mf_moe_prefill_workspace_bytes(h, t). */
+size_t mf_moe_prefill_workspace_bytes(const mf_moe* h, uint32_t t);
+mf_status mf_moe_prefill_layer(mf_moe* h, mf_stream stream, const mf_moe_layer_weights* wts,
+                               const uint16_t* x, uint32_t t, uint16_t* y, void* workspace,
+                               size_t workspace_bytes, uint32_t* out_idx, float* out_w);
 
 #ifdef __cplusplus
 }

@@ -213,6 +213,7 @@ mf_status mf_moe_create(mf_ctx* ctx, const mf_moe_config* cfg, mf_moe** out) {
   const size_t o_tacts = take(T * cfg->top_k * cfg->f * sizeof(uint32_t));
   const size_t o_epoch = take(512 * sizeof(uint32_t));
   const size_t o_status = take(64);
+  const size_t o_group = take((3 * 512 + 64) * sizeof(uint32_t));
   h->ws_bytes = pos;
   if (hipSetDevice(ctx->device) != hipSuccess) {
     delete h;
@@ -243,6 +244,7 @@ mf_status mf_moe_create(mf_ctx* ctx, const mf_moe_config* cfg, mf_moe** out) {
   h->ws.t_acts = reinterpret_cast<uint32_t*>(b + o_tacts);
   h->ws.epoch = reinterpret_cast<uint32_t*>(b + o_epoch);
   h->ws.status = reinterpret_cast<uint32_t*>(b + o_status);
+  h->ws.group_tmp = reinterpret_cast<uint32_t*>(b + o_group);
   *out = h;
   return MF_OK;
 }
@@ -384,6 +386,57 @@ mf_status mf_moe_status(mf_moe* h, mf_stream stream) {
 }
 
 /* ------------------------------------------------------- ragged prefill */
+
+mf_status mf_moe_group(mf_moe* h, mf_stream stream, const uint32_t* idx, const float* w, uint32_t t,
+                       mf_pair* sorted_pairs, uint32_t* expert_offsets, uint32_t* expert_counts) {
+  if (!h || !idx || !w || !sorted_pairs || !expert_offsets || !expert_counts)
+    return MF_ERR_INVALID_ARGUMENT;
+  auto s = static_cast<hipStream_t>(stream);
+  uint32_t* starts = h->ws.group_tmp + 512;
+  uint32_t* status = h->ws.group_tmp + 3 * 512;
+  MF_HIP(h->ctx, mf::launch_group(s, idx, w, t, h->cfg.top_k, h->cfg.num_experts, expert_counts,
+                                  expert_offsets, starts, sorted_pairs, nullptr, nullptr, status));
+  return MF_OK;
+}
+
+mf_status mf_moe_group_status(mf_moe* h, mf_stream stream) {
+  if (!h) return MF_ERR_INVALID_ARGUMENT;
+  uint32_t word = 0;
+  auto s = static_cast<hipStream_t>(stream);
+  MF_HIP(h->ctx, hipMemcpyAsync(&word, h->ws.group_tmp + 3 * 512, sizeof word, hipMemcpyDeviceToHost, s));
+  MF_HIP(h->ctx, hipStreamSynchronize(s));
+  return word ? MF_ERR_EXPERT_RANGE : MF_OK;
+}
+
+size_t mf_moe_prefill_workspace_bytes(const mf_moe* h, uint32_t t) {
+  if (!h || t == 0) return 0;
+  return mf::prefill_workspace_bytes(h->cfg, t);
+}
+
+mf_status mf_moe_prefill_layer(mf_moe* h, mf_stream stream, const mf_moe_layer_weights* wts,
+                               const uint16_t* x, uint32_t t, uint16_t* y, void* workspace,
+                               size_t workspace_bytes, uint32_t* out_idx, float* out_w) {
+  if (!h || !wts || !x || !y || !workspace) return MF_ERR_INVALID_ARGUMENT;
+  if (t == 0 || t > (1u << 20)) return MF_ERR_INVALID_ARGUMENT;
+  const mf_moe_config& c = h->cfg;
+  if (!mf::prefill_supported(c)) return MF_ERR_UNSUPPORTED_BITS;
+  if (workspace_bytes < mf::prefill_workspace_bytes(c, t)) return MF_ERR_SCRATCH_TOO_SMALL;
+  const uint32_t offs = wts->offsets.gate_w | wts->offsets.up_w | wts->offsets.down_w;
+  if (!wts->router_w || !wts->expert_base || !offsets_ok(wts->offsets, c.bits) ||
+      !mf::aligned16(wts->expert_base) || wts->expert_stride % 16 || offs % 16 ||
+      !mf::aligned16(wts->router_w) || !mf::aligned16(x) || !mf::aligned16(y) ||
+      !mf::aligned16(workspace))
+    return MF_ERR_INVALID_ARGUMENT;
+  if (c.shared_f && (!qtensor_ok(wts->shared_gate, c.shared_bits) ||
+                     !qtensor_ok(wts->shared_up, c.shared_bits) ||
+                     !qtensor_ok(wts->shared_down, c.shared_bits) ||
+                     !mf::aligned16(wts->shared_gate.weights) || !mf::aligned16(wts->shared_up.weights) ||
+                     !mf::aligned16(wts->shared_down.weights) || (wts->w_sg && !mf::aligned16(wts->w_sg))))
+    return MF_ERR_INVALID_ARGUMENT;
+  MF_HIP(h->ctx, mf::launch_prefill_layer(static_cast<hipStream_t>(stream), *h, *wts, x, t, y, workspace,
+                                          out_idx, out_w));
+  return MF_OK;
+}
 
 mf_status mf_group_pairs_host(const mf_pair* pairs, size_t n_pairs, int query_count, int top_k,
                               int num_experts, int tile_expert_count,

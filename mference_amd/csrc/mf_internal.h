@@ -30,6 +30,7 @@ struct mf_moe_workspace {
   uint32_t* t_acts;              // [MF_MAX_TOKENS, top_k, f]
   uint32_t* epoch;               // [512] one launch counter per workgroup
   uint32_t* status;              // non-zero once a bounded wait gave up
+  uint32_t* group_tmp;           // [3*512 + 64] counts, starts of mf_moe_group + its status word
 };
 
 struct mf_moe {
@@ -97,4 +98,18 @@ hipError_t launch_fused_decode(hipStream_t s, const mf_moe& h, const mf_moe_laye
                                const uint16_t* x, uint32_t t, uint16_t* y, uint16_t* hidden,
                                uint32_t* out_idx, float* out_w);
 
+}  // namespace mf
+
+// moe_prefill.hip
+namespace mf {
+hipError_t launch_group(hipStream_t s, const uint32_t* idx, const float* w, uint32_t t, uint32_t K,
+                        uint32_t E, uint32_t* counts, uint32_t* offsets, uint32_t* starts,
+                        mf_pair* sorted, void* tiles, uint32_t* n_tiles, uint32_t* status);
+size_t prefill_workspace_bytes(const mf_moe_config& c, uint32_t t);
+bool prefill_supported(const mf_moe_config& c);
+hipError_t launch_prefill_layer(hipStream_t s, const mf_moe& h, const mf_moe_layer_weights& w,
+                                const uint16_t* x, uint32_t t, uint16_t* y, void* workspace,
+                                uint32_t* out_idx, float* out_w);
+hipError_t launch_prefill_router(hipStream_t s, const uint16_t* W, const uint16_t* x, uint32_t E,
+                                 uint32_t D, uint32_t T, uint32_t x_stride, float* logits);
 }  // namespace mf

@@ -287,6 +287,39 @@ class MoE:
                                               _ptr(y), _ptr(hidden), _ptr(out_indices),
                                               _ptr(out_weights)), self.context.handle)
 
+    def encode_group(self, indices, routing_weights, t: int, sorted_pairs, expert_offsets,
+                     expert_counts, stream=None):
+        """PrefillRouter.makeTokenExpertPairs + PrefillMoEGrouping.groupTokenExpertPairs
+        (PrefillRouter.swift:91-111, PrefillMoEGrouping.swift:91-192) on device.
+        sorted_pairs: int32/uint8 device tensor of t*top_k 16-byte records."""
+        check(_capi.lib().mf_moe_group(self._h, _stream(stream), _ptr(indices),
+                                       _ptr(routing_weights), t, _ptr(sorted_pairs),
+                                       _ptr(expert_offsets), _ptr(expert_counts)),
+              self.context.handle)
+
+    def group_status(self, stream=None) -> None:
+        """synchronises; raises MfError(expert out of range) if the last
+        encode_group saw an index >= num_experts"""
+        check(_capi.lib().mf_moe_group_status(self._h, _stream(stream)), self.context.handle)
+
+    def prefill_workspace_bytes(self, t: int) -> int:
+        return int(_capi.lib().mf_moe_prefill_workspace_bytes(self._h, t))
+
+    def encode_prefill_layer(self, weights: MoELayerWeights, x, y, t: int, workspace=None,
+                             out_indices=None, out_weights=None, stream=None):
+        """Ragged prefill layer over t tokens (PrefillGroupedRoutedMoE.encodeStreamedBatched,
+        PrefillGroupedRoutedMoE.swift:392-466, + reduce + shared expert).  `workspace`: uint8
+        device tensor of at least prefill_workspace_bytes(t); allocated when None."""
+        need = self.prefill_workspace_bytes(t)
+        if workspace is None:
+            workspace = torch.empty(need, dtype=torch.uint8, device=x.device)
+        lw = weights.c()
+        check(_capi.lib().mf_moe_prefill_layer(self._h, _stream(stream), C.byref(lw), _ptr(x), t,
+                                               _ptr(y), _ptr(workspace), workspace.numel(),
+                                               _ptr(out_indices), _ptr(out_weights)),
+              self.context.handle)
+        return workspace
+
 
 PAIR_DTYPE = np.dtype([("token", "<u4"), ("expert", "<u4"), ("rank", "<u4"),
                        ("weight_bits", "<u4")])

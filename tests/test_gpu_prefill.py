@@ -1,0 +1,133 @@
+"""GPU parity of the ragged prefill path: device grouping against the oracle's
+restatement of PrefillMoEGrouping, and the tokens-sorted-by-expert layer against
+the per-token oracle (the reference's own gate for this path: grouped prefill ==
+per-token decode, PrefillGroupedRoutedMoETests / PrefillMoETests)."""
+import numpy as np
+import pytest
+import torch
+
+from mference_amd import _capi
+from mference_amd import operators as ops
+from helpers import ROOT_SEED, assert_layer_close, make_moe, to_device_layer
+
+pytestmark = pytest.mark.gpu
+
+
+def _group_on_device(moe, idx, w, t, k, e):
+    sorted_pairs = torch.zeros((t * k, 4), dtype=torch.int32, device="cuda")
+    offsets = torch.zeros(e, dtype=torch.int32, device="cuda")
+    counts = torch.zeros(e, dtype=torch.int32, device="cuda")
+    moe.encode_group(torch.from_numpy(idx.astype(np.int32)).cuda(), torch.from_numpy(w).cuda(), t,
+                     sorted_pairs, offsets, counts)
+    return sorted_pairs, offsets, counts
+
+
+@pytest.mark.parametrize("t,k,e,live", [(1, 8, 16, 16), (37, 4, 16, 16), (300, 8, 256, 256),
+                                        (129, 8, 64, 9), (64, 2, 512, 40)])
+def test_device_grouping_matches_oracle(gpu, oracle, t, k, e, live):
+    """`live` < e leaves experts without a token: their offset is 0xFFFFFFFF
+    (PrefillMoEGrouping.swift:151-160)."""
+    rng = np.random.default_rng(t * 1000 + e)
+    idx = np.stack([rng.choice(live, size=k, replace=False) for _ in range(t)]).astype(np.uint32)
+    w = rng.random((t, k), dtype=np.float32)
+    moe = ops.MoE(gpu, 128, 64, e, k)
+    sorted_pairs, offsets, counts = _group_on_device(moe, idx, w, t, k, e)
+    moe.group_status()
+    ref = oracle.group_pairs(oracle.make_pairs(idx, w.view(np.uint32)), t, k, e)
+    got = sorted_pairs.cpu().numpy().view(np.uint32)
+    assert np.array_equal(got[:, 0], ref["sorted"]["token"])
+    assert np.array_equal(got[:, 1], ref["sorted"]["expert"])
+    assert np.array_equal(got[:, 2], ref["sorted"]["rank"])
+    assert np.array_equal(got[:, 3], ref["sorted"]["weight_bits"])
+    assert np.array_equal(offsets.cpu().numpy().view(np.uint32), ref["offsets"])
+    assert np.array_equal(counts.cpu().numpy().view(np.uint32), ref["counts"])
+
+
+def test_device_grouping_flags_expert_out_of_range(gpu):
+    t, k, e = 9, 4, 16
+    idx = np.tile(np.arange(k, dtype=np.uint32), (t, 1))
+    idx[5, 2] = e + 3
+    w = np.ones((t, k), np.float32)
+    moe = ops.MoE(gpu, 128, 64, e, k)
+    _group_on_device(moe, idx, w, t, k, e)
+    with pytest.raises(_capi.MfError) as err:
+        moe.group_status()
+    assert err.value.status == -17
+    idx[5, 2] = 1  # the status word is re-armed by the next call
+    _group_on_device(moe, idx, w, t, k, e)
+    moe.group_status()
+
+
+def _run_prefill(moe, wts, x, t, d, k):
+    xd = ops.bf16_tensor(x)
+    y = torch.zeros((t, d), dtype=torch.bfloat16, device="cuda")
+    idx = torch.zeros((t, k), dtype=torch.int32, device="cuda")
+    w = torch.zeros((t, k), dtype=torch.float32, device="cuda")
+    moe.encode_prefill_layer(wts, xd, y, t, out_indices=idx, out_weights=w)
+    torch.cuda.synchronize()
+    return ops.bf16_bits(y), idx.cpu().numpy().astype(np.uint32), w.cpu().numpy()
+
+
+@pytest.mark.parametrize("d,f,e,k,fs,t,mode,limit", [
+    (256, 128, 16, 4, 0, 5, 0, 0.0),        # fewer tokens than a tile, no shared expert
+    (256, 128, 16, 4, 128, 70, 0, 0.0),     # one full tile + a ragged tail per busy expert
+    (512, 256, 32, 8, 256, 200, 0, 7.0),    # SwiGLU clamp (moe.metal:1080-1094)
+    (384, 128, 32, 2, 128, 131, 1, 0.0),    # full-softmax router, ng not a multiple of 8
+    (2048, 512, 256, 8, 512, 96, 0, 0.0),   # the headline layer shape
+])
+def test_prefill_layer_matches_per_token_oracle(gpu, oracle, d, f, e, k, fs, t, mode, limit):
+    root = ROOT_SEED + 0xA000 + d + t
+    layer = oracle.synth_layer(root, d, f, e, k, bits=4, fs=fs, router_mode=mode, swiglu_limit=limit)
+    x = oracle.synth_x(root, t, d)
+    ref_y, ref_idx, ref_w = oracle.moe_layer(layer, x)
+    moe = make_moe(gpu, layer)
+    wts = to_device_layer(layer)
+    y, idx, w = _run_prefill(moe, wts, x, t, d, k)
+    assert np.array_equal(idx, ref_idx)
+    assert np.array_equal(w.view(np.uint32), ref_w.view(np.uint32))
+    assert_layer_close(oracle.bf16_to_float(y), oracle.bf16_to_float(ref_y),
+                       f"prefill layer d={d} f={f} e={e} k={k} t={t}")
+    # a second call into the same workspace-free handle gives the same bits (no stale state)
+    y2, _, _ = _run_prefill(moe, wts, x, t, d, k)
+    assert np.array_equal(y, y2)
+
+
+def test_prefill_skewed_routing_and_decode_agreement(gpu, oracle):
+    """All tokens identical -> every token takes the same k experts: k groups of
+    t routes and e-k empty experts; and the prefill rows agree with the decode
+    launch on the same token within the layer tolerance."""
+    d, f, e, k, fs, t = 256, 128, 16, 4, 128, 150
+    root = ROOT_SEED + 0xA100
+    layer = oracle.synth_layer(root, d, f, e, k, bits=4, fs=fs)
+    x1 = oracle.synth_x(root, 1, d)
+    x = np.repeat(x1, t, axis=0)
+    ref_y, ref_idx, _ = oracle.moe_layer(layer, x1)
+    moe = make_moe(gpu, layer)
+    wts = to_device_layer(layer)
+    y, idx, _ = _run_prefill(moe, wts, x, t, d, k)
+    assert np.array_equal(idx, np.repeat(ref_idx, t, axis=0))
+    assert np.array_equal(y, np.repeat(y[:1], t, axis=0))   # position in a tile does not matter
+    assert_layer_close(oracle.bf16_to_float(y[0]), oracle.bf16_to_float(ref_y[0]), "skewed prefill")
+    yd = torch.zeros((1, d), dtype=torch.bfloat16, device="cuda")
+    moe.encode_decode_layer(wts, ops.bf16_tensor(x1), yd, t=1)
+    moe.status()
+    assert_layer_close(oracle.bf16_to_float(y[0]), oracle.bf16_to_float(ops.bf16_bits(yd)[0]),
+                       "prefill vs decode launch")
+
+
+def test_prefill_rejects_what_it_does_not_cover(gpu, oracle):
+    layer = oracle.synth_layer(ROOT_SEED + 0xA200, 256, 128, 16, 4, bits=2, fs=0)
+    moe = make_moe(gpu, layer)
+    wts = to_device_layer(layer)
+    x = ops.bf16_tensor(oracle.synth_x(1, 4, 256))
+    y = torch.zeros((4, 256), dtype=torch.bfloat16, device="cuda")
+    with pytest.raises(_capi.MfError) as err:
+        moe.encode_prefill_layer(wts, x, y, 4, workspace=torch.empty(1 << 20, dtype=torch.uint8, device="cuda"))
+    assert err.value.status == -3
+    layer4 = oracle.synth_layer(ROOT_SEED + 0xA201, 256, 128, 16, 4, bits=4, fs=0)
+    moe4 = make_moe(gpu, layer4)
+    wts4 = to_device_layer(layer4)
+    assert moe4.prefill_workspace_bytes(4) > 0
+    with pytest.raises(_capi.MfError) as err:
+        moe4.encode_prefill_layer(wts4, x, y, 4, workspace=torch.empty(256, dtype=torch.uint8, device="cuda"))
+    assert err.value.status == -4

@@ -193,6 +193,30 @@ __global__ void zero_words_kernel(uint32_t* p, uint32_t n) {
 
 // --------------------------------------------------------------- the matmul
 
+// Activation rows as the matmul wants them: inside every run of 8 K values the
+// order is (0,4,1,5,2,6,3,7) -- the pairing a packed code word expands to --
+// and the fp32 sum of every 64-wide K group is kept beside them.  One lane per
+// run of 8; `dst` may be null when `src` is already in that order.
+__global__ __launch_bounds__(256) void prep_rows_kernel(const uint16_t* __restrict__ src,
+                                                        uint16_t* __restrict__ dst,
+                                                        float* __restrict__ sums, uint32_t chunks) {
+  const uint32_t c = blockIdx.x * blockDim.x + threadIdx.x;
+  uint4 v = make_uint4(0, 0, 0, 0);
+  if (c < chunks) v = *reinterpret_cast<const uint4*>(src + static_cast<size_t>(c) * 8);
+  float sum = 0.0f;
+  sum = dot2_bf16(v.x, kOnes, sum);
+  sum = dot2_bf16(v.y, kOnes, sum);
+  sum = dot2_bf16(v.z, kOnes, sum);
+  sum = dot2_bf16(v.w, kOnes, sum);
+  sum = group_sum(sum, 8);
+  if (c >= chunks) return;
+  if (dst)
+    *reinterpret_cast<uint4*>(dst + static_cast<size_t>(c) * 8) =
+        make_uint4(__builtin_amdgcn_perm(v.z, v.x, 0x05040100u), __builtin_amdgcn_perm(v.z, v.x, 0x07060302u),
+                   __builtin_amdgcn_perm(v.w, v.y, 0x05040100u), __builtin_amdgcn_perm(v.w, v.y, 0x07060302u));
+  if ((c & 7) == 0) sums[c >> 3] = sum;
+}
+
 struct QmmArgs {
   // weights: routed = blobs of the expert pool, dense = one projection set
   const uint8_t* expert_base;
@@ -201,8 +225,9 @@ struct QmmArgs {
   mf_qtensor dense[2];
   int dense_mode;       // 1: the "expert" is dense[], tiles are runs of consecutive rows
   uint32_t dense_rows;  // number of x rows in dense mode
-  // activations: rows of kdim bf16
+  // activations: rows of kdim bf16 in prep_rows_kernel order + their group sums [row, kdim/64]
   const uint16_t* x;
+  const float* sumx;
   uint32_t x_stride;
   int gather;           // 1: x row = sorted[pair].token, 0: x row = pair index
   const mf_pair* sorted;
@@ -210,7 +235,7 @@ struct QmmArgs {
   const uint32_t* n_tiles;
   uint32_t rows, kdim;  // weight rows (output width) and contraction length
   // epilogue
-  int epi;              // 0 swiglu -> bf16 [pair, rows]; 1 fp32 [token*K+rank, rows]; 2 bf16 [pair, rows]
+  int epi;              // 0 swiglu -> bf16 [pair, rows] in prep order; 1 fp32 [token*K+rank, rows]; 2 bf16 [pair, rows]
   int narrow;           // shared-expert rounding points (dequant_int4.metal:240-245)
   void* out;
   uint32_t top_k;
@@ -222,10 +247,22 @@ __device__ __forceinline__ f32x16_t mfma_bf16(const uint4& a, const uint4& b, co
                                                  __builtin_bit_cast(bf16x8_t, b), c, 0, 0, 0);
 }
 
+// silu with the hardware exp2 / reciprocal (1 ulp each): the result is narrowed to bf16 right after
+__device__ __forceinline__ float fast_silu(float x) {
+  return x * __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(x * -1.4426950408889634f));
+}
+
+// (v & mask) | magic in one instruction; the mask rides in a scalar register
+__device__ __forceinline__ uint32_t and_or(uint32_t v, uint32_t mask, uint32_t magic) {
+  uint32_t r;
+  asm("v_and_or_b32 %0, %1, %2, %3" : "=v"(r) : "v"(v), "s"(mask), "v"(magic));
+  return r;
+}
+
 // one packed word of 4-bit codes -> MFMA operand: pairs (q0,q4),(q1,q5),(q2,q6),(q3,q7) as 128+q
 __device__ __forceinline__ uint4 expand_q4(uint32_t w) {
-  return make_uint4((w & 0x000F000Fu) | kMagic128, ((w >> 4) & 0x000F000Fu) | kMagic128,
-                    ((w >> 8) & 0x000F000Fu) | kMagic128, ((w >> 12) & 0x000F000Fu) | kMagic128);
+  return make_uint4(and_or(w, 0x000F000Fu, kMagic128), and_or(w >> 4, 0x000F000Fu, kMagic128),
+                    and_or(w >> 8, 0x000F000Fu, kMagic128), and_or(w >> 12, 0x000F000Fu, kMagic128));
 }
 
 // 8 bf16 from p, of which only the first `avail` exist (the rest read as 0)
@@ -237,61 +274,47 @@ __device__ __forceinline__ uint4 load_bf16x8_guarded(const uint16_t* p, uint32_t
   return make_uint4(v[0] | (v[1] << 16), v[2] | (v[3] << 16), v[4] | (v[5] << 16), v[6] | (v[7] << 16));
 }
 
-// three exact bf16 terms of 8 fp32 values as MFMA operands: term k of +x and of -128*x
-__device__ __forceinline__ void split_terms(const float (&sx)[8], int k, uint4& pos, uint4& neg) {
-  float t[8];
-#pragma unroll
-  for (int e = 0; e < 8; ++e) {
-    const float t0 = __uint_as_float(__float_as_uint(sx[e]) & 0xFFFF0000u);
-    const float r1 = sx[e] - t0;
-    const float t1 = __uint_as_float(__float_as_uint(r1) & 0xFFFF0000u);
-    const float t2 = r1 - t1;
-    t[e] = k == 0 ? t0 : (k == 1 ? t1 : t2);
-  }
-  pos = make_uint4((__float_as_uint(t[0]) >> 16) | (__float_as_uint(t[1]) & 0xFFFF0000u),
-                   (__float_as_uint(t[2]) >> 16) | (__float_as_uint(t[3]) & 0xFFFF0000u),
-                   (__float_as_uint(t[4]) >> 16) | (__float_as_uint(t[5]) & 0xFFFF0000u),
-                   (__float_as_uint(t[6]) >> 16) | (__float_as_uint(t[7]) & 0xFFFF0000u));
-#pragma unroll
-  for (int e = 0; e < 8; ++e) t[e] = -128.0f * t[e];
-  neg = make_uint4((__float_as_uint(t[0]) >> 16) | (__float_as_uint(t[1]) & 0xFFFF0000u),
-                   (__float_as_uint(t[2]) >> 16) | (__float_as_uint(t[3]) & 0xFFFF0000u),
-                   (__float_as_uint(t[4]) >> 16) | (__float_as_uint(t[5]) & 0xFFFF0000u),
-                   (__float_as_uint(t[6]) >> 16) | (__float_as_uint(t[7]) & 0xFFFF0000u));
-}
-
-__device__ __forceinline__ uint32_t pack_bf16_trunc(float lo, float hi) {
-  return (__float_as_uint(lo) >> 16) | (__float_as_uint(hi) & 0xFFFF0000u);
-}
-
-// LDS layout (dynamic): x tile double buffer 2 x [2 nt][4 s][2 h][32 n] x 16 B,
-// sumx [ng][64] fp32, scale tables [NPROJ][4 waves][ng][32 rows] bf16, rows[64] u32.
+// One workgroup: 64 routes of one expert x 128 weight rows (4 waves x 32) x
+// NPROJ projections, the whole K.  The matrix core computes the TRANSPOSED
+// product: the A operand is the x tile (tokens are the rows), the B operand is
+// the expanded codes, so a lane ends up holding ONE weight row (its column
+// m = lane % 32) for 16 tokens of each 32-token block, and the per-group scale
+// is one scalar per lane.  Two waves per SIMD stay resident (the register
+// budget of 256 keeps the matrix-core results in ordinary registers, where
+// the scale multiply reads them directly).
+// LDS (dynamic): x tile double buffer 2 x [2 nt][4 s][2 h][32 n] x 16 B,
+// scale tables [NPROJ][4 waves][ng][32 rows] fp32, out slots [64] u32.
 template <int NPROJ>
-__global__ __launch_bounds__(256) void qmm_kernel(const QmmArgs a) {
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2)))
+void qmm_kernel(const QmmArgs a) {
   extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
   const uint32_t lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
   const uint32_t n_slices = a.rows / kQmmRows;
-  const uint32_t tile_id = blockIdx.x / n_slices, slice = blockIdx.x % n_slices;
+  // Workgroups go to the 8 XCDs round-robin by blockIdx; consecutive work items (the row slices of
+  // one tile share its x rows, the tiles of one expert share its weights) are laid on ONE XCD so
+  // that its L2 serves the re-reads.  The grid is a multiple of 8.
+  const uint32_t n_tiles = a.dense_mode ? (a.dense_rows + kTileTokens - 1) / kTileTokens : *a.n_tiles;
+  const uint32_t per_xcd = (n_tiles * n_slices + 7) >> 3;
+  if ((blockIdx.x >> 3) >= per_xcd) return;
+  const uint32_t work = (blockIdx.x & 7u) * per_xcd + (blockIdx.x >> 3);
+  const uint32_t tile_id = work / n_slices, slice = work % n_slices;
+  if (tile_id >= n_tiles) return;
   const uint32_t ng = a.kdim / kGroup;
 
   uint32_t expert = 0, pair_start, count;
   if (a.dense_mode) {
     pair_start = tile_id * kTileTokens;
-    if (pair_start >= a.dense_rows) return;
     count = min(kTileTokens, a.dense_rows - pair_start);
   } else {
-    if (tile_id >= *a.n_tiles) return;
     const Tile t = a.tiles[tile_id];
     expert = t.expert;
     pair_start = t.pair_start;
     count = t.count;
   }
 
-  uint4* s_x = reinterpret_cast<uint4*>(smem);                                   // 2 * 512 uint4
-  float* s_sumx = reinterpret_cast<float*>(smem + 2 * 512 * 16);                 // [ng][64]
-  uint16_t* s_scale = reinterpret_cast<uint16_t*>(smem + 2 * 512 * 16 + ng * 64 * 4);
-  uint32_t* s_rows = reinterpret_cast<uint32_t*>(smem + 2 * 512 * 16 + ng * 64 * 4 +
-                                                 NPROJ * kQmmWaves * ng * 32 * 2);
+  uint4* s_x = reinterpret_cast<uint4*>(smem);                      // 2 * 512 uint4
+  float* s_scale = reinterpret_cast<float*>(smem + 2 * 512 * 16);   // [NPROJ][4][ng][32]
+  uint32_t* s_slot = reinterpret_cast<uint32_t*>(smem + 2 * 512 * 16 + NPROJ * kQmmWaves * ng * 32 * 4);
 
   // weight pointers of this workgroup's projections
   const uint8_t* Wp[NPROJ];
@@ -314,32 +337,46 @@ __global__ __launch_bounds__(256) void qmm_kernel(const QmmArgs a) {
   const uint32_t m = lane & 31, h = lane >> 5;
   const size_t row_bytes = static_cast<size_t>(a.kdim) / 2;
 
-  // x rows of the tile
-  if (threadIdx.x < kTileTokens) {
-    uint32_t r = 0xFFFFFFFFu;
-    if (threadIdx.x < count)
-      r = a.gather ? a.sorted[pair_start + threadIdx.x].token : pair_start + threadIdx.x;
-    s_rows[threadIdx.x] = r;
+  // staging role of this thread: token i, the 16 K values (two runs of 8) from 16 * q
+  const uint32_t st_i = threadIdx.x >> 2, st_q = threadIdx.x & 3;
+  uint32_t st_row = 0xFFFFFFFFu;
+  if (st_i < count) st_row = a.gather ? a.sorted[pair_start + st_i].token : pair_start + st_i;
+  // the route of each 32-token block whose x row this lane feeds into the bias terms
+  uint32_t xrow[2] = {0xFFFFFFFFu, 0xFFFFFFFFu};
+#pragma unroll
+  for (int nt = 0; nt < 2; ++nt) {
+    const uint32_t ti = nt * 32 + m;
+    if (ti < count) xrow[nt] = a.gather ? a.sorted[pair_start + ti].token : pair_start + ti;
   }
-  // scale tables of the wave's rows, transposed to [g][row]
+  // where each route's result goes (0xFFFFFFFF: no such route in this tile)
+  if (threadIdx.x < kTileTokens) {
+    uint32_t slot = 0xFFFFFFFFu;
+    if (threadIdx.x < count) {
+      slot = pair_start + threadIdx.x;
+      if (a.epi == 1) {
+        const mf_pair pr = a.sorted[slot];
+        slot = pr.token * a.top_k + pr.rank;
+      }
+    }
+    s_slot[threadIdx.x] = slot;
+  }
+  // scale tables of the wave's rows, transposed to [g][row], widened to fp32
   {
-    uint16_t* dst = s_scale;
 #pragma unroll
     for (int p = 0; p < NPROJ; ++p) {
-      uint16_t* tab = dst + (p * kQmmWaves + wv) * ng * 32;
+      float* tab = s_scale + (p * kQmmWaves + wv) * ng * 32;
       const uint16_t* src = Sp[p] + static_cast<size_t>(row_base + m) * ng;
       for (uint32_t g0 = h * 8; g0 < ng; g0 += 16) {  // lane: row m, 8 groups from g0
         const uint4 v = load_bf16x8_guarded(src + g0, ng - g0);
         const uint32_t pr[4] = {v.x, v.y, v.z, v.w};
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
-          if (g0 + 2 * i < ng) tab[(g0 + 2 * i) * 32 + m] = static_cast<uint16_t>(pr[i] & 0xFFFFu);
-          if (g0 + 2 * i + 1 < ng) tab[(g0 + 2 * i + 1) * 32 + m] = static_cast<uint16_t>(pr[i] >> 16);
+          if (g0 + 2 * i < ng) tab[(g0 + 2 * i) * 32 + m] = bf16_lo(pr[i]);
+          if (g0 + 2 * i + 1 < ng) tab[(g0 + 2 * i + 1) * 32 + m] = bf16_hi(pr[i]);
         }
       }
     }
   }
-  __syncthreads();
 
   f32x16_t acc[NPROJ][2];
 #pragma unroll
@@ -349,94 +386,118 @@ __global__ __launch_bounds__(256) void qmm_kernel(const QmmArgs a) {
 #pragma unroll
       for (int r = 0; r < 16; ++r) acc[p][nt][r] = 0.0f;
 
-  // staging role of this thread: token i, 16 K values from 16 * q
-  const uint32_t st_i = threadIdx.x >> 2, st_q = threadIdx.x & 3;
-  const uint32_t st_row = s_rows[st_i];
-  const uint16_t* st_src = a.x + static_cast<size_t>(st_row == 0xFFFFFFFFu ? 0 : st_row) * a.x_stride + st_q * 16;
-
-  uint4 codes[NPROJ];
+  const bool st_live = st_row != 0xFFFFFFFFu;
+  const uint16_t* st_src = a.x + static_cast<size_t>(st_live ? st_row : 0) * a.x_stride + st_q * 16;
+  // run c = 2q (+1): K 8c..8c+7 -> slot (h = c / 4, s = c % 4)
+  const uint32_t st_nt = st_i >> 5, st_n = st_i & 31, c0 = 2 * st_q, c1 = c0 + 1;
+  // inside a 32-token block the column is rotated by 4 * ((s >> 1) + 2h): the four lanes that
+  // stage one token then hit four different bank groups
+  const uint32_t st_rot = 4 * ((c0 & 3) >> 1) + 8 * (c0 >> 2);
+  const uint32_t st_slot0 = ((st_nt * 4 + (c0 & 3)) * 2 + (c0 >> 2)) * 32 + ((st_n + st_rot) & 31);
+  const uint32_t st_slot1 = ((st_nt * 4 + (c1 & 3)) * 2 + (c1 >> 2)) * 32 + ((st_n + st_rot) & 31);
+  uint32_t rd_col[4];
 #pragma unroll
-  for (int p = 0; p < NPROJ; ++p)
-    codes[p] = *reinterpret_cast<const uint4*>(Wp[p] + (row_base + m) * row_bytes + h * 16);
+  for (int sidx = 0; sidx < 4; ++sidx) rd_col[sidx] = (m + 4 * (sidx >> 1) + 8 * h) & 31;
 
-  for (uint32_t g = 0; g < ng; ++g) {
-    // ---- stage x tile of group g (buffer g & 1) and its row sums
-    {
-      uint4 v0 = make_uint4(0, 0, 0, 0), v1 = v0;
-      if (st_row != 0xFFFFFFFFu) {
-        v0 = *reinterpret_cast<const uint4*>(st_src + g * kGroup);
-        v1 = *reinterpret_cast<const uint4*>(st_src + g * kGroup + 8);
+  // Weight codes run four K groups ahead in registers (the expert's bytes come
+  // from HBM); x rows come from L2 and run three groups ahead, two in registers,
+  // one in the LDS buffer that is not being read.
+  const uint8_t* wrow[NPROJ];
+  uint4 cur[NPROJ][4], nxt[NPROJ][4];
+#pragma unroll
+  for (int p = 0; p < NPROJ; ++p) {
+    wrow[p] = Wp[p] + (row_base + m) * row_bytes + h * 16;
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      cur[p][u] = make_uint4(0, 0, 0, 0);
+      if (static_cast<uint32_t>(u) < ng) cur[p][u] = *reinterpret_cast<const uint4*>(wrow[p] + u * 32);
+    }
+  }
+  uint4 xs[2][2];  // xs[k & 1] holds group k on its way to LDS
+#pragma unroll
+  for (int k = 0; k < 2; ++k) xs[k][0] = xs[k][1] = make_uint4(0, 0, 0, 0);
+  if (st_live) {
+    xs[0][0] = *reinterpret_cast<const uint4*>(st_src);
+    xs[0][1] = *reinterpret_cast<const uint4*>(st_src + 8);
+    s_x[st_slot0] = xs[0][0];
+    s_x[st_slot1] = xs[0][1];
+    if (ng > 1) {
+      xs[1][0] = *reinterpret_cast<const uint4*>(st_src + kGroup);
+      xs[1][1] = *reinterpret_cast<const uint4*>(st_src + kGroup + 8);
+    }
+    if (ng > 2) {
+      xs[0][0] = *reinterpret_cast<const uint4*>(st_src + 2 * kGroup);
+      xs[0][1] = *reinterpret_cast<const uint4*>(st_src + 2 * kGroup + 8);
+    }
+  } else {
+    s_x[st_slot0] = xs[0][0];
+    s_x[st_slot1] = xs[0][1];
+  }
+
+  for (uint32_t g0 = 0; g0 < ng; g0 += 4) {
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      const uint32_t g = g0 + u;
+      if (g >= ng) break;
+      __syncthreads();  // buffer g & 1 is complete, buffer (g + 1) & 1 is no longer read
+      // ---- x of group g + 1 into the other buffer, fetch group g + 3 into the freed registers
+      if (g + 1 < ng) {
+        uint4* wbuf = s_x + ((u + 1) & 1) * 512;
+        wbuf[st_slot0] = xs[(u + 1) & 1][0];
+        wbuf[st_slot1] = xs[(u + 1) & 1][1];
+        if (g + 3 < ng && st_live) {
+          xs[(u + 1) & 1][0] = *reinterpret_cast<const uint4*>(st_src + (g + 3) * kGroup);
+          xs[(u + 1) & 1][1] = *reinterpret_cast<const uint4*>(st_src + (g + 3) * kGroup + 8);
+        }
       }
-      float sum = 0.0f;
-      sum = dot2_bf16(v0.x, kOnes, sum); sum = dot2_bf16(v0.y, kOnes, sum);
-      sum = dot2_bf16(v0.z, kOnes, sum); sum = dot2_bf16(v0.w, kOnes, sum);
-      sum = dot2_bf16(v1.x, kOnes, sum); sum = dot2_bf16(v1.y, kOnes, sum);
-      sum = dot2_bf16(v1.z, kOnes, sum); sum = dot2_bf16(v1.w, kOnes, sum);
-      sum = sum + dpp_f<0xB1>(sum);
-      sum = sum + dpp_f<0x4E>(sum);
-      if (st_q == 0) s_sumx[g * 64 + st_i] = sum;
-      uint4* buf = s_x + (g & 1) * 512;
-      const uint32_t nt = st_i >> 5, n = st_i & 31;
-      // chunk c = 2q (+1): K 8c..8c+7 -> (h = c / 4, s = c % 4)
-      const uint32_t c0 = 2 * st_q, c1 = c0 + 1;
-      buf[((nt * 4 + (c0 & 3)) * 2 + (c0 >> 2)) * 32 + n] =
-          make_uint4(__builtin_amdgcn_perm(v0.z, v0.x, 0x05040100u), __builtin_amdgcn_perm(v0.z, v0.x, 0x07060302u),
-                     __builtin_amdgcn_perm(v0.w, v0.y, 0x05040100u), __builtin_amdgcn_perm(v0.w, v0.y, 0x07060302u));
-      buf[((nt * 4 + (c1 & 3)) * 2 + (c1 >> 2)) * 32 + n] =
-          make_uint4(__builtin_amdgcn_perm(v1.z, v1.x, 0x05040100u), __builtin_amdgcn_perm(v1.z, v1.x, 0x07060302u),
-                     __builtin_amdgcn_perm(v1.w, v1.y, 0x05040100u), __builtin_amdgcn_perm(v1.w, v1.y, 0x07060302u));
-    }
-    // next group's codes
-    uint4 next[NPROJ];
+      if (u == 0) {  // codes of the next four groups
 #pragma unroll
-    for (int p = 0; p < NPROJ; ++p) {
-      next[p] = codes[p];
-      if (g + 1 < ng)
-        next[p] = *reinterpret_cast<const uint4*>(Wp[p] + (row_base + m) * row_bytes + (g + 1) * 32 + h * 16);
-    }
-    __syncthreads();
+        for (int p = 0; p < NPROJ; ++p)
+#pragma unroll
+          for (int v = 0; v < 4; ++v) {
+            nxt[p][v] = cur[p][v];
+            if (g0 + 4 + v < ng) nxt[p][v] = *reinterpret_cast<const uint4*>(wrow[p] + (g0 + 4 + v) * 32);
+          }
+      }
 
-    // ---- matrix core: tmp = sum over the group of (128+q) * x
-    const uint4* buf = s_x + (g & 1) * 512;
-    uint4 bx[2][4];
-#pragma unroll
-    for (int nt = 0; nt < 2; ++nt)
-#pragma unroll
-      for (int s = 0; s < 4; ++s) bx[nt][s] = buf[((nt * 4 + s) * 2 + h) * 32 + m];
-#pragma unroll
-    for (int p = 0; p < NPROJ; ++p) {
-      const uint32_t cw[4] = {codes[p].x, codes[p].y, codes[p].z, codes[p].w};
-      f32x16_t tmp[2];
+      // ---- matrix core: tmp[token, row] = sum over the group of x * (128+q)
+      const uint4* buf = s_x + (u & 1) * 512;
+      uint4 bx[2][4];
 #pragma unroll
       for (int nt = 0; nt < 2; ++nt)
 #pragma unroll
-        for (int r = 0; r < 16; ++r) tmp[nt][r] = 0.0f;
+        for (int s = 0; s < 4; ++s) bx[nt][s] = buf[((nt * 4 + s) * 2 + h) * 32 + rd_col[s]];
 #pragma unroll
-      for (int s = 0; s < 4; ++s) {
-        const uint4 av = expand_q4(cw[s]);
-        tmp[0] = mfma_bf16(av, bx[0][s], tmp[0]);
-        tmp[1] = mfma_bf16(av, bx[1][s], tmp[1]);
-      }
-      // per-group scale of the 16 rows this lane holds: row = 8j + 4h + i
-      const uint16_t* tab = s_scale + ((p * kQmmWaves + wv) * ng + g) * 32 + 4 * h;
+      for (int p = 0; p < NPROJ; ++p) {
+        const uint32_t cw[4] = {cur[p][u].x, cur[p][u].y, cur[p][u].z, cur[p][u].w};
+        const float sc = s_scale[((p * kQmmWaves + wv) * ng + g) * 32 + m];
+        f32x16_t tmp[2];
 #pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        const uint2 sv = *reinterpret_cast<const uint2*>(tab + 8 * j);
-        const float s0 = bf16_lo(sv.x), s1 = bf16_hi(sv.x), s2 = bf16_lo(sv.y), s3 = bf16_hi(sv.y);
+        for (int nt = 0; nt < 2; ++nt)
 #pragma unroll
-        for (int nt = 0; nt < 2; ++nt) {
-          acc[p][nt][4 * j + 0] = __builtin_fmaf(s0, tmp[nt][4 * j + 0], acc[p][nt][4 * j + 0]);
-          acc[p][nt][4 * j + 1] = __builtin_fmaf(s1, tmp[nt][4 * j + 1], acc[p][nt][4 * j + 1]);
-          acc[p][nt][4 * j + 2] = __builtin_fmaf(s2, tmp[nt][4 * j + 2], acc[p][nt][4 * j + 2]);
-          acc[p][nt][4 * j + 3] = __builtin_fmaf(s3, tmp[nt][4 * j + 3], acc[p][nt][4 * j + 3]);
+          for (int r = 0; r < 16; ++r) tmp[nt][r] = 0.0f;
+#pragma unroll
+        for (int s = 0; s < 4; ++s) {
+          const uint4 av = expand_q4(cw[s]);
+          tmp[0] = mfma_bf16(bx[0][s], av, tmp[0]);
+          tmp[1] = mfma_bf16(bx[1][s], av, tmp[1]);
         }
+#pragma unroll
+        for (int nt = 0; nt < 2; ++nt)
+#pragma unroll
+          for (int r = 0; r < 16; ++r) acc[p][nt][r] = __builtin_fmaf(sc, tmp[nt][r], acc[p][nt][r]);
       }
-      codes[p] = next[p];
     }
+#pragma unroll
+    for (int p = 0; p < NPROJ; ++p)
+#pragma unroll
+      for (int v = 0; v < 4; ++v) cur[p][v] = nxt[p][v];
   }
-  __syncthreads();
 
-  // ---- bias and offset terms: acc += B[row, g] * sumx[g, n] - 128 * S[row, g] * sumx[g, n]
+  // ---- bias and offset terms: acc[token, row] += sumx[token, g] * B[row, g] + sumx[token, g] * (-128 S[row, g]).
+  // -128 * S is formed in place (exponent + 7, sign flipped: exact; a zero scale becomes 2^-120).
+  // sumx enters as three bf16 terms, which hold all 24 bits: the -128 * S * sumx term cancels the
+  // 128 * sum(x) the matrix core accumulated with the codes, so it has to be exact.
   for (uint32_t g0 = 0; g0 < ng; g0 += 16) {
     const uint32_t gl = g0 + 8 * h;  // this lane's 8 groups
     uint4 ab[NPROJ], as[NPROJ];
@@ -445,40 +506,58 @@ __global__ __launch_bounds__(256) void qmm_kernel(const QmmArgs a) {
       ab[p] = as[p] = make_uint4(0, 0, 0, 0);
       if (gl < ng) {
         ab[p] = load_bf16x8_guarded(Bp[p] + static_cast<size_t>(row_base + m) * ng + gl, ng - gl);
-        as[p] = load_bf16x8_guarded(Sp[p] + static_cast<size_t>(row_base + m) * ng + gl, ng - gl);
+        const uint4 sv = load_bf16x8_guarded(Sp[p] + static_cast<size_t>(row_base + m) * ng + gl, ng - gl);
+        as[p] = make_uint4((sv.x + 0x03800380u) ^ 0x80008000u, (sv.y + 0x03800380u) ^ 0x80008000u,
+                           (sv.z + 0x03800380u) ^ 0x80008000u, (sv.w + 0x03800380u) ^ 0x80008000u);
       }
     }
 #pragma unroll
     for (int nt = 0; nt < 2; ++nt) {
-      float sx[8];
+      uint32_t hi[8], mid[8], lo[8];
+      const float* sp = a.sumx + static_cast<size_t>(xrow[nt] == 0xFFFFFFFFu ? 0 : xrow[nt]) * ng;
 #pragma unroll
-      for (int e = 0; e < 8; ++e) sx[e] = gl + e < ng ? s_sumx[(gl + e) * 64 + nt * 32 + m] : 0.0f;
+      for (int e = 0; e < 8; ++e) {
+        const float v = (xrow[nt] != 0xFFFFFFFFu && gl + e < ng) ? sp[gl + e] : 0.0f;
+        hi[e] = __float_as_uint(v) & 0xFFFF0000u;
+        const float r1 = v - __uint_as_float(hi[e]);
+        mid[e] = __float_as_uint(r1) & 0xFFFF0000u;
+        lo[e] = __float_as_uint(r1 - __uint_as_float(mid[e]));
+      }
+      const uint4 b_hi = make_uint4((hi[0] >> 16) | hi[1], (hi[2] >> 16) | hi[3], (hi[4] >> 16) | hi[5],
+                                    (hi[6] >> 16) | hi[7]);
+      const uint4 b_mid = make_uint4((mid[0] >> 16) | mid[1], (mid[2] >> 16) | mid[3], (mid[4] >> 16) | mid[5],
+                                     (mid[6] >> 16) | mid[7]);
+      const uint4 b_lo = make_uint4(__builtin_amdgcn_perm(lo[1], lo[0], 0x07060302u),
+                                    __builtin_amdgcn_perm(lo[3], lo[2], 0x07060302u),
+                                    __builtin_amdgcn_perm(lo[5], lo[4], 0x07060302u),
+                                    __builtin_amdgcn_perm(lo[7], lo[6], 0x07060302u));
 #pragma unroll
-      for (int k = 0; k < 3; ++k) {
-        uint4 bpos, bneg;
-        split_terms(sx, k, bpos, bneg);
-#pragma unroll
-        for (int p = 0; p < NPROJ; ++p) {
-          acc[p][nt] = mfma_bf16(ab[p], bpos, acc[p][nt]);
-          acc[p][nt] = mfma_bf16(as[p], bneg, acc[p][nt]);
-        }
+      for (int p = 0; p < NPROJ; ++p) {
+        acc[p][nt] = mfma_bf16(b_hi, ab[p], acc[p][nt]);
+        acc[p][nt] = mfma_bf16(b_hi, as[p], acc[p][nt]);
+        acc[p][nt] = mfma_bf16(b_mid, ab[p], acc[p][nt]);
+        acc[p][nt] = mfma_bf16(b_mid, as[p], acc[p][nt]);
+        acc[p][nt] = mfma_bf16(b_lo, ab[p], acc[p][nt]);
+        acc[p][nt] = mfma_bf16(b_lo, as[p], acc[p][nt]);
       }
     }
   }
 
-  // ---- epilogue: lane holds token n = m of each token tile, rows 8j + 4h + i
+  // ---- epilogue: the lane holds weight row `row` for tokens 8j + 4h + i of each 32-token block
+  const uint32_t row = row_base + m;
+  // position of the row inside its run of 8 in the (0,4,1,5,2,6,3,7) order phase 2 reads
+  const uint32_t row_p = (row & ~7u) + ((row & 3u) << 1) + ((row >> 2) & 1u);
 #pragma unroll
   for (int nt = 0; nt < 2; ++nt) {
-    const uint32_t ti = nt * 32 + m;
-    if (ti >= count) continue;
-    const uint32_t pair = pair_start + ti;
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
-      const uint32_t row = row_base + 8 * j + 4 * h;
-      if (a.epi == 0) {
-        uint16_t o[4];
+      const uint4 sl = *reinterpret_cast<const uint4*>(s_slot + nt * 32 + 8 * j + 4 * h);
+      const uint32_t slot[4] = {sl.x, sl.y, sl.z, sl.w};
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
+      for (int i = 0; i < 4; ++i) {
+        if (slot[i] == 0xFFFFFFFFu) continue;
+        const size_t at = static_cast<size_t>(slot[i]) * a.rows;
+        if (a.epi == 0) {
           float gv = acc[0][nt][4 * j + i], uv = acc[NPROJ - 1][nt][4 * j + i];
           if (a.narrow) {
             gv = round_bf16(gv);
@@ -488,24 +567,12 @@ __global__ __launch_bounds__(256) void qmm_kernel(const QmmArgs a) {
             gv = fminf(gv, a.limit);
             uv = fminf(fmaxf(uv, -a.limit), a.limit);
           }
-          o[i] = f_to_bf16(mf_silu(gv) * uv);
+          static_cast<uint16_t*>(a.out)[at + row_p] = f_to_bf16(fast_silu(gv) * uv);
+        } else if (a.epi == 1) {
+          static_cast<float*>(a.out)[at + row] = acc[0][nt][4 * j + i];
+        } else {
+          static_cast<uint16_t*>(a.out)[at + row] = f_to_bf16(acc[0][nt][4 * j + i]);
         }
-        uint2 pk;
-        pk.x = static_cast<uint32_t>(o[0]) | (static_cast<uint32_t>(o[1]) << 16);
-        pk.y = static_cast<uint32_t>(o[2]) | (static_cast<uint32_t>(o[3]) << 16);
-        *reinterpret_cast<uint2*>(static_cast<uint16_t*>(a.out) + static_cast<size_t>(pair) * a.rows + row) = pk;
-      } else if (a.epi == 1) {
-        const mf_pair pr = a.sorted[pair];
-        const size_t slot = static_cast<size_t>(pr.token) * a.top_k + pr.rank;
-        *reinterpret_cast<float4*>(static_cast<float*>(a.out) + slot * a.rows + row) =
-            make_float4(acc[0][nt][4 * j], acc[0][nt][4 * j + 1], acc[0][nt][4 * j + 2], acc[0][nt][4 * j + 3]);
-      } else {
-        uint2 pk;
-        pk.x = static_cast<uint32_t>(f_to_bf16(acc[0][nt][4 * j])) |
-               (static_cast<uint32_t>(f_to_bf16(acc[0][nt][4 * j + 1])) << 16);
-        pk.y = static_cast<uint32_t>(f_to_bf16(acc[0][nt][4 * j + 2])) |
-               (static_cast<uint32_t>(f_to_bf16(acc[0][nt][4 * j + 3])) << 16);
-        *reinterpret_cast<uint2*>(static_cast<uint16_t*>(a.out) + static_cast<size_t>(pair) * a.rows + row) = pk;
       }
     }
   }
@@ -579,13 +646,19 @@ hipError_t launch_group(hipStream_t s, const uint32_t* idx, const float* w, uint
 
 size_t qmm_lds_bytes(uint32_t kdim, int nproj) {
   const uint32_t ng = kdim / kGroup;
-  return 2 * 512 * 16 + static_cast<size_t>(ng) * 64 * 4 + static_cast<size_t>(nproj) * kQmmWaves * ng * 32 * 2 +
-         kTileTokens * 4;
+  return 2 * 512 * 16 + static_cast<size_t>(nproj) * kQmmWaves * ng * 32 * 4 + kTileTokens * 4;
+}
+
+hipError_t launch_prep_rows(hipStream_t s, const uint16_t* src, uint16_t* dst, float* sums, size_t elems) {
+  const uint32_t chunks = static_cast<uint32_t>(elems / 8);
+  if (!chunks) return hipSuccess;
+  prep_rows_kernel<<<dim3((chunks + 255) / 256), dim3(256), 0, s>>>(src, dst, sums, chunks);
+  return hipGetLastError();
 }
 
 hipError_t launch_qmm(hipStream_t s, const QmmArgs& a, int nproj, uint32_t max_tiles) {
   const size_t lds = qmm_lds_bytes(a.kdim, nproj);
-  const dim3 grid(max_tiles * (a.rows / kQmmRows)), block(256);
+  const dim3 grid((max_tiles * (a.rows / kQmmRows) + 7) / 8 * 8), block(256);
   if (grid.x == 0) return hipSuccess;
   if (nproj == 2) {
     if (lds > 48 * 1024) {
@@ -614,6 +687,7 @@ struct PrefillWs {
   float* logits; uint32_t* idx; float* w; uint32_t* counts; uint32_t* offsets; uint32_t* starts;
   uint32_t* n_tiles; uint32_t* status; Tile* tiles; mf_pair* sorted; uint16_t* acts; float* partials;
   uint16_t* sact; uint16_t* hs; uint16_t* gate;
+  uint16_t* xp; float* sum_x; float* sum_acts; float* sum_sact;
   size_t bytes;
 };
 
@@ -642,6 +716,10 @@ PrefillWs prefill_carve(const mf_moe_config& c, uint32_t t, void* base) {
   p.sact = static_cast<uint16_t*>(take(sizeof(uint16_t) * static_cast<size_t>(t) * std::max<uint32_t>(c.shared_f, 64)));
   p.hs = static_cast<uint16_t*>(take(sizeof(uint16_t) * static_cast<size_t>(t) * c.d));
   p.gate = static_cast<uint16_t*>(take(sizeof(uint16_t) * t));
+  p.xp = static_cast<uint16_t*>(take(sizeof(uint16_t) * static_cast<size_t>(t) * c.d));
+  p.sum_x = static_cast<float*>(take(sizeof(float) * static_cast<size_t>(t) * (c.d / kGroup)));
+  p.sum_acts = static_cast<float*>(take(sizeof(float) * pairs * (c.f / kGroup)));
+  p.sum_sact = static_cast<float*>(take(sizeof(float) * static_cast<size_t>(t) * (std::max<uint32_t>(c.shared_f, 64) / kGroup)));
   p.bytes = pos;
   return p;
 }
@@ -672,6 +750,8 @@ hipError_t launch_prefill_layer(hipStream_t s, const mf_moe& h, const mf_moe_lay
   const uint32_t max_tiles =
       static_cast<uint32_t>(std::min<size_t>(c.num_experts, pairs) + pairs / kTileTokens + 1);
 
+  MF_TRY(launch_prep_rows(s, x, ws.xp, ws.sum_x, static_cast<size_t>(t) * c.d));
+
   QmmArgs q{};
   q.expert_base = static_cast<const uint8_t*>(w.expert_base);
   q.expert_stride = w.expert_stride;
@@ -683,11 +763,14 @@ hipError_t launch_prefill_layer(hipStream_t s, const mf_moe& h, const mf_moe_lay
   // routed phase 1: gate/up -> acts [pair, F]
   q.w_off[0] = w.offsets.gate_w; q.s_off[0] = w.offsets.gate_s; q.b_off[0] = w.offsets.gate_b;
   q.w_off[1] = w.offsets.up_w; q.s_off[1] = w.offsets.up_s; q.b_off[1] = w.offsets.up_b;
-  q.x = x; q.x_stride = c.d; q.gather = 1; q.rows = c.f; q.kdim = c.d; q.epi = 0; q.out = ws.acts;
+  q.x = ws.xp; q.sumx = ws.sum_x; q.x_stride = c.d; q.gather = 1; q.rows = c.f; q.kdim = c.d; q.epi = 0;
+  q.out = ws.acts;
   MF_TRY(launch_qmm(s, q, 2, max_tiles));
+  // routes past the last tile's count were never written: only pairs rows exist, all written
+  MF_TRY(launch_prep_rows(s, ws.acts, nullptr, ws.sum_acts, pairs * c.f));
   // routed phase 2: down -> fp32 partials [token*K+rank, D]
   q.w_off[0] = w.offsets.down_w; q.s_off[0] = w.offsets.down_s; q.b_off[0] = w.offsets.down_b;
-  q.x = ws.acts; q.x_stride = c.f; q.gather = 0; q.rows = c.d; q.kdim = c.f; q.epi = 1; q.out = ws.partials;
+  q.x = ws.acts; q.sumx = ws.sum_acts; q.x_stride = c.f; q.gather = 0; q.rows = c.d; q.kdim = c.f; q.epi = 1; q.out = ws.partials;
   q.limit = 0.0f;
   MF_TRY(launch_qmm(s, q, 1, max_tiles));
   const uint16_t* hs = nullptr;
@@ -696,11 +779,12 @@ hipError_t launch_prefill_layer(hipStream_t s, const mf_moe& h, const mf_moe_lay
     QmmArgs d{};
     d.dense_mode = 1; d.dense_rows = t; d.top_k = c.top_k; d.narrow = 1;
     d.dense[0] = w.shared_gate; d.dense[1] = w.shared_up;
-    d.x = x; d.x_stride = c.d; d.rows = c.shared_f; d.kdim = c.d; d.epi = 0; d.out = ws.sact;
+    d.x = ws.xp; d.sumx = ws.sum_x; d.x_stride = c.d; d.rows = c.shared_f; d.kdim = c.d; d.epi = 0; d.out = ws.sact;
     const uint32_t dense_tiles = (t + kTileTokens - 1) / kTileTokens;
     MF_TRY(launch_qmm(s, d, 2, dense_tiles));
+    MF_TRY(launch_prep_rows(s, ws.sact, nullptr, ws.sum_sact, static_cast<size_t>(t) * c.shared_f));
     d.dense[0] = w.shared_down;
-    d.x = ws.sact; d.x_stride = c.shared_f; d.rows = c.d; d.kdim = c.shared_f; d.epi = 2; d.out = ws.hs;
+    d.x = ws.sact; d.sumx = ws.sum_sact; d.x_stride = c.shared_f; d.rows = c.d; d.kdim = c.shared_f; d.epi = 2; d.out = ws.hs;
     MF_TRY(launch_qmm(s, d, 1, dense_tiles));
     hs = ws.hs;
     if (w.w_sg) {

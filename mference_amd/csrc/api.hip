@@ -213,7 +213,7 @@ mf_status mf_moe_create(mf_ctx* ctx, const mf_moe_config* cfg, mf_moe** out) {
   const size_t o_tacts = take(T * cfg->top_k * cfg->f * sizeof(uint32_t));
   const size_t o_epoch = take(512 * sizeof(uint32_t));
   const size_t o_status = take(64);
-  const size_t o_group = take((3 * 512 + 64) * sizeof(uint32_t));
+  const size_t o_group = take(mf::group_scratch_words() * sizeof(uint32_t));
   h->ws_bytes = pos;
   if (hipSetDevice(ctx->device) != hipSuccess) {
     delete h;
@@ -366,6 +366,7 @@ mf_status mf_moe_set_phase_trace(mf_moe* h, uint64_t* device_buffer, size_t byte
   if (device_buffer && bytes < static_cast<size_t>(h->ctx->num_cu) * 8 * sizeof(uint64_t))
     return MF_ERR_SCRATCH_TOO_SMALL;
   h->trace = reinterpret_cast<unsigned long long*>(device_buffer);
+  h->trace_bytes = device_buffer ? bytes : 0;
   return MF_OK;
 }
 
@@ -395,7 +396,8 @@ mf_status mf_moe_group(mf_moe* h, mf_stream stream, const uint32_t* idx, const f
   uint32_t* starts = h->ws.group_tmp + 512;
   uint32_t* status = h->ws.group_tmp + 3 * 512;
   MF_HIP(h->ctx, mf::launch_group(s, idx, w, t, h->cfg.top_k, h->cfg.num_experts, expert_counts,
-                                  expert_offsets, starts, sorted_pairs, nullptr, nullptr, status));
+                                  expert_offsets, starts, sorted_pairs, nullptr, 0, nullptr, status,
+                                  h->ws.group_tmp + 2048));
   return MF_OK;
 }
 

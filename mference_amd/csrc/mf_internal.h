@@ -30,7 +30,7 @@ struct mf_moe_workspace {
   uint32_t* t_acts;              // [MF_MAX_TOKENS, top_k, f]
   uint32_t* epoch;               // [512] one launch counter per workgroup
   uint32_t* status;              // non-zero once a bounded wait gave up
-  uint32_t* group_tmp;           // [3*512 + 64] counts, starts of mf_moe_group + its status word
+  uint32_t* group_tmp;           // grouping scratch: [512, 1024) starts, [1536] status word, [2048, ...) per-chunk counts
 };
 
 struct mf_moe {
@@ -38,6 +38,7 @@ struct mf_moe {
   mf_moe_config cfg{};
   bool fused = true;  // mf_moe_set_fused
   unsigned long long* trace = nullptr;  // mf_moe_set_phase_trace
+  size_t trace_bytes = 0;
   void* ws_base = nullptr;
   size_t ws_bytes = 0;
   mf_moe_workspace ws{};
@@ -104,7 +105,9 @@ hipError_t launch_fused_decode(hipStream_t s, const mf_moe& h, const mf_moe_laye
 namespace mf {
 hipError_t launch_group(hipStream_t s, const uint32_t* idx, const float* w, uint32_t t, uint32_t K,
                         uint32_t E, uint32_t* counts, uint32_t* offsets, uint32_t* starts,
-                        mf_pair* sorted, void* tiles, uint32_t* n_tiles, uint32_t* status);
+                        mf_pair* sorted, void* tiles, uint32_t tile_slots, uint32_t* n_tiles,
+                        uint32_t* status, uint32_t* chunk_hist);
+size_t group_scratch_words();
 size_t prefill_workspace_bytes(const mf_moe_config& c, uint32_t t);
 bool prefill_supported(const mf_moe_config& c);
 hipError_t launch_prefill_layer(hipStream_t s, const mf_moe& h, const mf_moe_layer_weights& w,

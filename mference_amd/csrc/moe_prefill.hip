@@ -3,18 +3,18 @@
 // the bf16 matrix cores.
 //
 // The matmul keeps the 4-bit codes EXACT: a lane's packed uint32 (8 codes of
-// one weight row) is masked straight into four bf16 pairs 128+q
-// (0x4300 | q), which is an MFMA A operand as it stands -- no LDS staging of
-// weights.  x is staged through LDS once per 64-wide K group, permuted to the
-// same (j, j+4) pairing.  Per K group the matrix core yields
-// sum((128+q)*x) exactly (bf16 x bf16 products are exact in fp32), and the
-// group's bf16 scale is applied in fp32: acc += s * tmp -- the reference's own
-// factoring s*sum(q*x) + b*sum(x) (Metal/Quant/dequant_int4.metal:14-17), so
-// no weight is ever rounded to bf16 (rounding q*s+b to bf16 would cost ~1.6e-3
-// relative error per weight, above the layer tolerance).  The b*sum(x) and
-// -128*s*sum(x) terms are two more small matmuls over the group index
-// (A = the bf16 bias / scale tables, exact; B = sum(x) split into three bf16
-// terms, exact), run on the matrix core after the K loop.
+// one weight row) is masked straight into four bf16 pairs 8 + q/2
+// (0x4100 | q << 3), which is a matrix-core operand as it stands -- no LDS
+// staging of weights.  x rows are pre-permuted once per call to the same
+// (j, j+4) pairing and staged through LDS per 64-wide K group.  Per K group the
+// matrix core yields sum((8 + q/2) * x) (bf16 x bf16 products are exact in
+// fp32), and the group's bf16 scale is applied in fp32: acc += 2s * tmp -- the
+// reference's own factoring s*sum(q*x) + b*sum(x)
+// (Metal/Quant/dequant_int4.metal:14-17), so no weight is ever rounded to bf16
+// (rounding q*s+b to bf16 would cost ~1.6e-3 relative error per weight, above
+// the layer tolerance).  The b*sum(x) and -16*s*sum(x) terms are two more small
+// matmuls over the group index (operands: the bf16 bias / scale tables, exact,
+// and sum(x) split into three bf16 terms, exact).
 //
 // Replaces prefill_grouped_routed_moe_batched_{phase1,down}
 // (Metal/Prefill/prefill.metal:748-820), prefill_moe_reduce_token_major
@@ -104,39 +104,56 @@ __global__ __launch_bounds__(256) void prefill_router_kernel(const uint16_t* __r
 //
 // PrefillMoEGrouping.groupTokenExpertPairs (PrefillMoEGrouping.swift:91-192) on
 // device: pairs come token-major (token, rank), so "sorted by (expert, token,
-// rank)" is a stable partition by expert.  One wave per expert counts its
-// routes, a single block scans the counts, one wave per expert emits its
-// routes in order.
+// rank)" is a stable counting sort by expert.  The pair list is cut into at
+// most kGroupChunks chunks; every chunk counts its routes per expert, one
+// block turns the counts into per-(chunk, expert) start positions, and every
+// chunk then places its routes in order.
+
+constexpr uint32_t kGroupChunks = 256;   // rows of the per-chunk count matrix
+constexpr uint32_t kGroupBlock = 256;    // pairs one workgroup handles per step
 
 __global__ __launch_bounds__(256) void group_count_kernel(const uint32_t* __restrict__ idx,
                                                           uint32_t n_pairs, uint32_t E,
-                                                          uint32_t* __restrict__ counts,
+                                                          uint32_t chunk_pairs,
+                                                          uint32_t* __restrict__ chunk_hist,
                                                           uint32_t* __restrict__ status) {
-  const uint32_t lane = threadIdx.x & 63;
-  const uint32_t e = (blockIdx.x * blockDim.x + threadIdx.x) >> 6;
-  if (e >= E) return;
-  uint32_t cnt = 0;
+  __shared__ uint32_t s_hist[MF_MAX_EXPERTS];
+  for (uint32_t e = threadIdx.x; e < E; e += blockDim.x) s_hist[e] = 0;
+  __syncthreads();
+  const uint32_t p0 = blockIdx.x * chunk_pairs, p1 = min(n_pairs, p0 + chunk_pairs);
   bool bad = false;
-  for (uint32_t p0 = 0; p0 < n_pairs; p0 += kWave) {
-    const uint32_t p = p0 + lane;
-    const uint32_t v = p < n_pairs ? idx[p] : 0xFFFFFFFFu;
-    cnt += __popcll(__ballot(v == e));
-    if (e == 0 && p < n_pairs && v >= E) bad = true;
+  for (uint32_t p = p0 + threadIdx.x; p < p1; p += blockDim.x) {
+    const uint32_t e = idx[p];
+    if (e < E) atomicAdd(&s_hist[e], 1u);
+    else bad = true;
   }
-  if (lane == 0) counts[e] = cnt;
-  if (__any(bad) && lane == 0) atomicOr(status, 2u);
+  if (__any(bad) && (threadIdx.x & 63) == 0) atomicOr(status, 2u);
+  __syncthreads();
+  for (uint32_t e = threadIdx.x; e < E; e += blockDim.x) chunk_hist[blockIdx.x * E + e] = s_hist[e];
 }
 
-// offsets (0xFFFFFFFF for an empty expert), running starts, and the tile list
-// of the matmul (every expert's routes cut into runs of kTileTokens).
-__global__ __launch_bounds__(512) void group_scan_kernel(const uint32_t* __restrict__ counts,
-                                                         uint32_t E, uint32_t* __restrict__ offsets,
+// counts, offsets (0xFFFFFFFF for an empty expert), the start of every expert's
+// run, chunk_hist turned into each chunk's first position inside its expert's
+// run, and the tile list of the matmul (runs of kTileTokens routes).
+__global__ __launch_bounds__(512) void group_scan_kernel(uint32_t* __restrict__ chunk_hist,
+                                                         uint32_t n_chunks, uint32_t E,
+                                                         uint32_t* __restrict__ counts,
+                                                         uint32_t* __restrict__ offsets,
                                                          uint32_t* __restrict__ starts,
                                                          Tile* __restrict__ tiles,
+                                                         uint32_t tile_slots,
                                                          uint32_t* __restrict__ n_tiles) {
   __shared__ uint32_t s_cnt[MF_MAX_EXPERTS], s_tile[MF_MAX_EXPERTS];
   const uint32_t e = threadIdx.x;
-  const uint32_t c = e < E ? counts[e] : 0;
+  uint32_t c = 0;
+  if (e < E) {
+    for (uint32_t k = 0; k < n_chunks; ++k) {
+      const uint32_t v = chunk_hist[k * E + e];
+      chunk_hist[k * E + e] = c;
+      c += v;
+    }
+    counts[e] = c;
+  }
   s_cnt[e] = c;
   s_tile[e] = (c + kTileTokens - 1) / kTileTokens;
   __syncthreads();
@@ -147,14 +164,25 @@ __global__ __launch_bounds__(512) void group_scan_kernel(const uint32_t* __restr
     s_tile[e] += b;
     __syncthreads();
   }
+  // The tile list has tile_slots entries (a multiple of 8).  The matmul sends the workgroups of
+  // slot range k * tile_slots/8 .. to XCD k, so every eighth of the list gets an eighth of the
+  // live tiles, in expert order; the rest of each eighth stays empty (count 0).
+  if (tiles) {
+    for (uint32_t i = e; i < tile_slots; i += MF_MAX_EXPERTS) tiles[i] = Tile{0, 0, 0, 0};
+    __syncthreads();
+  }
   if (e < E) {
     const uint32_t start = s_cnt[e] - c;
     starts[e] = start;
     offsets[e] = c ? start : 0xFFFFFFFFu;
     if (tiles) {
+      const uint32_t total = s_tile[MF_MAX_EXPERTS - 1], per_live = (total + 7) / 8, per_slot = tile_slots / 8;
       const uint32_t nt = (c + kTileTokens - 1) / kTileTokens, t0 = s_tile[e] - nt;
-      for (uint32_t j = 0; j < nt; ++j)
-        tiles[t0 + j] = Tile{e, start + j * kTileTokens, min(kTileTokens, c - j * kTileTokens), 0};
+      for (uint32_t j = 0; j < nt; ++j) {
+        const uint32_t id = t0 + j;
+        tiles[(id / per_live) * per_slot + id % per_live] =
+            Tile{e, start + j * kTileTokens, min(kTileTokens, c - j * kTileTokens), 0};
+      }
     }
   }
   if (n_tiles && e == MF_MAX_EXPERTS - 1) *n_tiles = s_tile[e];
@@ -163,18 +191,42 @@ __global__ __launch_bounds__(512) void group_scan_kernel(const uint32_t* __restr
 __global__ __launch_bounds__(256) void group_emit_kernel(const uint32_t* __restrict__ idx,
                                                          const float* __restrict__ w,
                                                          uint32_t n_pairs, uint32_t K, uint32_t E,
+                                                         uint32_t chunk_pairs,
+                                                         const uint32_t* __restrict__ chunk_base,
                                                          const uint32_t* __restrict__ starts,
                                                          mf_pair* __restrict__ sorted) {
-  const uint32_t lane = threadIdx.x & 63;
-  const uint32_t e = (blockIdx.x * blockDim.x + threadIdx.x) >> 6;
-  if (e >= E) return;
-  uint32_t running = starts[e];
-  for (uint32_t p0 = 0; p0 < n_pairs; p0 += kWave) {
-    const uint32_t p = p0 + lane;
-    const bool m = p < n_pairs && idx[p] == e;
-    const unsigned long long mask = __ballot(m);
-    if (m) {
-      const uint32_t pos = running + __popcll(mask & ((1ull << lane) - 1ull));
+  __shared__ uint32_t s_base[MF_MAX_EXPERTS];      // next free position of every expert's run
+  __shared__ uint32_t s_wave[4][MF_MAX_EXPERTS];   // routes per expert of each wave in this step
+  const uint32_t lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
+  for (uint32_t e = threadIdx.x; e < E; e += blockDim.x) {
+    s_base[e] = starts[e] + chunk_base[blockIdx.x * E + e];
+    s_wave[0][e] = s_wave[1][e] = s_wave[2][e] = s_wave[3][e] = 0;
+  }
+  __syncthreads();
+  const uint32_t p0 = blockIdx.x * chunk_pairs, p1 = min(n_pairs, p0 + chunk_pairs);
+  for (uint32_t q0 = p0; q0 < p1; q0 += kGroupBlock) {
+    const uint32_t p = q0 + threadIdx.x;
+    const bool valid = p < p1;
+    const uint32_t e = valid ? idx[p] : 0xFFFFFFFFu;
+    // rank of this route among the routes of its expert in this wave, in pair order
+    bool open = valid && e < E;
+    uint32_t rank = 0;
+    unsigned long long todo = __ballot(open);
+    while (todo) {
+      const int leader = __ffsll(static_cast<long long>(todo)) - 1;
+      const uint32_t e0 = static_cast<uint32_t>(__builtin_amdgcn_readlane(static_cast<int>(e), leader));
+      const unsigned long long same = __ballot(open && e == e0);
+      if (open && e == e0) {
+        rank = __popcll(same & ((1ull << lane) - 1ull));
+        open = false;
+      }
+      if (lane == static_cast<uint32_t>(leader)) s_wave[wv][e0] = __popcll(same);
+      todo &= ~same;
+    }
+    __syncthreads();
+    if (valid && e < E) {
+      uint32_t pos = s_base[e] + rank;
+      for (uint32_t v = 0; v < wv; ++v) pos += s_wave[v][e];
       mf_pair r;
       r.token = p / K;
       r.expert = e;
@@ -182,7 +234,14 @@ __global__ __launch_bounds__(256) void group_emit_kernel(const uint32_t* __restr
       r.weight_bits = __float_as_uint(w[p]);
       sorted[pos] = r;
     }
-    running += __popcll(mask);
+    __syncthreads();
+    if (q0 + kGroupBlock < p1) {  // another step follows: advance the bases, clear the wave counts
+      for (uint32_t x = threadIdx.x; x < E; x += blockDim.x) {
+        s_base[x] += s_wave[0][x] + s_wave[1][x] + s_wave[2][x] + s_wave[3][x];
+        s_wave[0][x] = s_wave[1][x] = s_wave[2][x] = s_wave[3][x] = 0;
+      }
+      __syncthreads();
+    }
   }
 }
 
@@ -203,11 +262,8 @@ __global__ __launch_bounds__(256) void prep_rows_kernel(const uint16_t* __restri
   const uint32_t c = blockIdx.x * blockDim.x + threadIdx.x;
   uint4 v = make_uint4(0, 0, 0, 0);
   if (c < chunks) v = *reinterpret_cast<const uint4*>(src + static_cast<size_t>(c) * 8);
-  float sum = 0.0f;
-  sum = dot2_bf16(v.x, kOnes, sum);
-  sum = dot2_bf16(v.y, kOnes, sum);
-  sum = dot2_bf16(v.z, kOnes, sum);
-  sum = dot2_bf16(v.w, kOnes, sum);
+  float sum = ((bf16_lo(v.x) + bf16_hi(v.x)) + (bf16_lo(v.y) + bf16_hi(v.y))) +
+              ((bf16_lo(v.z) + bf16_hi(v.z)) + (bf16_lo(v.w) + bf16_hi(v.w)));
   sum = group_sum(sum, 8);
   if (c >= chunks) return;
   if (dst)
@@ -223,6 +279,7 @@ struct QmmArgs {
   size_t expert_stride;
   uint32_t w_off[2], s_off[2], b_off[2];
   mf_qtensor dense[2];
+  int pair_rows;        // 1: the NPROJ blocks of a wave are consecutive 32-row blocks of projection 0
   int dense_mode;       // 1: the "expert" is dense[], tiles are runs of consecutive rows
   uint32_t dense_rows;  // number of x rows in dense mode
   // activations: rows of kdim bf16 in prep_rows_kernel order + their group sums [row, kdim/64]
@@ -240,7 +297,15 @@ struct QmmArgs {
   void* out;
   uint32_t top_k;
   float limit;
+  uint32_t dense_tiles;  // dense mode: number of 64-row tiles
+  // optional stage stamps: 8 per work item, 100 MHz clock
+  unsigned long long* trace;
+  uint32_t trace_items;
 };
+
+__device__ __forceinline__ void qmm_trace(const QmmArgs& a, uint32_t work, uint32_t k) {
+  if (a.trace && threadIdx.x == 0 && work < a.trace_items) a.trace[work * 8 + k] = wall_clock64();
+}
 
 __device__ __forceinline__ f32x16_t mfma_bf16(const uint4& a, const uint4& b, const f32x16_t& c) {
   return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, a),
@@ -259,10 +324,14 @@ __device__ __forceinline__ uint32_t and_or(uint32_t v, uint32_t mask, uint32_t m
   return r;
 }
 
-// one packed word of 4-bit codes -> MFMA operand: pairs (q0,q4),(q1,q5),(q2,q6),(q3,q7) as 128+q
+// one packed word of 4-bit codes -> MFMA operand: pairs (q0,q4),(q1,q5),(q2,q6),(q3,q7) as the
+// bf16 numbers 8 + q/2 (exponent 2^3, the code in mantissa bits 3..6).  16 is the smallest offset
+// a mask-and-or can give a 4-bit code, and the offset matters: the matrix core accumulates
+// offset * sum(x) alongside the signal and the correction term takes it out again in fp32.
+constexpr uint32_t kMagic8 = 0x41004100u;
 __device__ __forceinline__ uint4 expand_q4(uint32_t w) {
-  return make_uint4(and_or(w, 0x000F000Fu, kMagic128), and_or(w >> 4, 0x000F000Fu, kMagic128),
-                    and_or(w >> 8, 0x000F000Fu, kMagic128), and_or(w >> 12, 0x000F000Fu, kMagic128));
+  return make_uint4(and_or(w << 3, 0x00780078u, kMagic8), and_or(w >> 1, 0x00780078u, kMagic8),
+                    and_or(w >> 5, 0x00780078u, kMagic8), and_or(w >> 9, 0x00780078u, kMagic8));
 }
 
 // 8 bf16 from p, of which only the first `avail` exist (the rest read as 0)
@@ -284,29 +353,31 @@ __device__ __forceinline__ uint4 load_bf16x8_guarded(const uint16_t* p, uint32_t
 // the scale multiply reads them directly).
 // LDS (dynamic): x tile double buffer 2 x [2 nt][4 s][2 h][32 n] x 16 B,
 // scale tables [NPROJ][4 waves][ng][32 rows] fp32, out slots [64] u32.
-template <int NPROJ>
+template <int NPROJ, bool NG8>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2)))
 void qmm_kernel(const QmmArgs a) {
   extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
   const uint32_t lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
-  const uint32_t n_slices = a.rows / kQmmRows;
+  const uint32_t m = lane & 31, h = lane >> 5;
+  const uint32_t wave_rows = a.pair_rows ? 32u * NPROJ : 32u;  // weight rows of one wave
+  const uint32_t n_slices = a.rows / (kQmmWaves * wave_rows);
   // Workgroups go to the 8 XCDs round-robin by blockIdx; consecutive work items (the row slices of
   // one tile share its x rows, the tiles of one expert share its weights) are laid on ONE XCD so
-  // that its L2 serves the re-reads.  The grid is a multiple of 8.
-  const uint32_t n_tiles = a.dense_mode ? (a.dense_rows + kTileTokens - 1) / kTileTokens : *a.n_tiles;
-  const uint32_t per_xcd = (n_tiles * n_slices + 7) >> 3;
-  if ((blockIdx.x >> 3) >= per_xcd) return;
-  const uint32_t work = (blockIdx.x & 7u) * per_xcd + (blockIdx.x >> 3);
+  // that its L2 serves the re-reads.  The grid is a multiple of 8; the tile list is laid out by
+  // group_scan_kernel so that every eighth of it holds an eighth of the live tiles.
+  const uint32_t work = (blockIdx.x & 7u) * (gridDim.x >> 3) + (blockIdx.x >> 3);
   const uint32_t tile_id = work / n_slices, slice = work % n_slices;
-  if (tile_id >= n_tiles) return;
   const uint32_t ng = a.kdim / kGroup;
+  qmm_trace(a, work, 0);
 
   uint32_t expert = 0, pair_start, count;
   if (a.dense_mode) {
+    if (tile_id >= a.dense_tiles) return;
     pair_start = tile_id * kTileTokens;
     count = min(kTileTokens, a.dense_rows - pair_start);
   } else {
     const Tile t = a.tiles[tile_id];
+    if (t.count == 0) return;
     expert = t.expert;
     pair_start = t.pair_start;
     count = t.count;
@@ -320,60 +391,81 @@ void qmm_kernel(const QmmArgs a) {
   const uint8_t* Wp[NPROJ];
   const uint16_t* Sp[NPROJ];
   const uint16_t* Bp[NPROJ];
+  uint32_t row_base[NPROJ];  // first weight row of each of this wave's 32-row blocks
 #pragma unroll
   for (int p = 0; p < NPROJ; ++p) {
+    const int t = a.pair_rows ? 0 : p;
     if (a.dense_mode) {
-      Wp[p] = static_cast<const uint8_t*>(a.dense[p].weights);
-      Sp[p] = a.dense[p].scales;
-      Bp[p] = a.dense[p].biases;
+      Wp[p] = static_cast<const uint8_t*>(a.dense[t].weights);
+      Sp[p] = a.dense[t].scales;
+      Bp[p] = a.dense[t].biases;
     } else {
       const uint8_t* blob = a.expert_base + static_cast<size_t>(expert) * a.expert_stride;
-      Wp[p] = blob + a.w_off[p];
-      Sp[p] = reinterpret_cast<const uint16_t*>(blob + a.s_off[p]);
-      Bp[p] = reinterpret_cast<const uint16_t*>(blob + a.b_off[p]);
+      Wp[p] = blob + a.w_off[t];
+      Sp[p] = reinterpret_cast<const uint16_t*>(blob + a.s_off[t]);
+      Bp[p] = reinterpret_cast<const uint16_t*>(blob + a.b_off[t]);
     }
+    row_base[p] = (slice * kQmmWaves + wv) * wave_rows + (a.pair_rows ? 32u * p : 0u);
   }
-  const uint32_t row_base = slice * kQmmRows + wv * 32;  // first of this wave's 32 weight rows
-  const uint32_t m = lane & 31, h = lane >> 5;
   const size_t row_bytes = static_cast<size_t>(a.kdim) / 2;
 
-  // staging role of this thread: token i, the 16 K values (two runs of 8) from 16 * q
-  const uint32_t st_i = threadIdx.x >> 2, st_q = threadIdx.x & 3;
-  uint32_t st_row = 0xFFFFFFFFu;
-  if (st_i < count) st_row = a.gather ? a.sorted[pair_start + st_i].token : pair_start + st_i;
-  // the route of each 32-token block whose x row this lane feeds into the bias terms
-  uint32_t xrow[2] = {0xFFFFFFFFu, 0xFFFFFFFFu};
-#pragma unroll
-  for (int nt = 0; nt < 2; ++nt) {
-    const uint32_t ti = nt * 32 + m;
-    if (ti < count) xrow[nt] = a.gather ? a.sorted[pair_start + ti].token : pair_start + ti;
-  }
-  // where each route's result goes (0xFFFFFFFF: no such route in this tile)
-  if (threadIdx.x < kTileTokens) {
-    uint32_t slot = 0xFFFFFFFFu;
-    if (threadIdx.x < count) {
-      slot = pair_start + threadIdx.x;
-      if (a.epi == 1) {
-        const mf_pair pr = a.sorted[slot];
-        slot = pr.token * a.top_k + pr.rank;
-      }
+  // ---- everything the tile needs that depends only on the tile: issued back to back.
+  // Routes past `count` read the tile's last route instead (finite data, results discarded).
+  const uint32_t st_i = threadIdx.x >> 2, st_q = threadIdx.x & 3;  // staging: token i, K values 16q..16q+15
+  const uint32_t st_pair = pair_start + min(st_i, count - 1);
+  const uint32_t ti_pair[2] = {pair_start + min(m, count - 1), pair_start + min(32 + m, count - 1)};
+  uint32_t st_row = st_pair, xrow[2] = {ti_pair[0], ti_pair[1]};
+  uint32_t slot = pair_start + min(threadIdx.x & 63u, count - 1);
+  if (!a.dense_mode) {
+    const mf_pair pr = a.sorted[slot];
+    if (a.gather) {
+      st_row = a.sorted[st_pair].token;
+      xrow[0] = a.sorted[ti_pair[0]].token;
+      xrow[1] = a.sorted[ti_pair[1]].token;
     }
-    s_slot[threadIdx.x] = slot;
+    if (a.epi == 1) slot = pr.token * a.top_k + pr.rank;
   }
-  // scale tables of the wave's rows, transposed to [g][row], widened to fp32
-  {
+  const uint8_t* wrow[NPROJ];
+  uint4 cur[NPROJ][4], nxt[NPROJ][4];
 #pragma unroll
-    for (int p = 0; p < NPROJ; ++p) {
-      float* tab = s_scale + (p * kQmmWaves + wv) * ng * 32;
-      const uint16_t* src = Sp[p] + static_cast<size_t>(row_base + m) * ng;
-      for (uint32_t g0 = h * 8; g0 < ng; g0 += 16) {  // lane: row m, 8 groups from g0
-        const uint4 v = load_bf16x8_guarded(src + g0, ng - g0);
-        const uint32_t pr[4] = {v.x, v.y, v.z, v.w};
+  for (int p = 0; p < NPROJ; ++p) {
+    wrow[p] = Wp[p] + (row_base[p] + m) * row_bytes + h * 16;
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-          if (g0 + 2 * i < ng) tab[(g0 + 2 * i) * 32 + m] = bf16_lo(pr[i]);
-          if (g0 + 2 * i + 1 < ng) tab[(g0 + 2 * i + 1) * 32 + m] = bf16_hi(pr[i]);
-        }
+    for (int u = 0; u < 4; ++u) {
+      cur[p][u] = make_uint4(0, 0, 0, 0);
+      if (NG8 || static_cast<uint32_t>(u) < ng) cur[p][u] = *reinterpret_cast<const uint4*>(wrow[p] + u * 32);
+    }
+  }
+  // x rows of groups 0..2 and, for the bias terms, the group sums of the lane's two routes
+  const uint16_t* st_src = a.x + static_cast<size_t>(st_row) * a.x_stride + st_q * 16;
+  uint4 xs[2][2];  // xs[k & 1] holds group k on its way to LDS
+  uint4 x0[2];
+  x0[0] = *reinterpret_cast<const uint4*>(st_src);
+  x0[1] = *reinterpret_cast<const uint4*>(st_src + 8);
+  xs[1][0] = xs[1][1] = xs[0][0] = xs[0][1] = make_uint4(0, 0, 0, 0);
+  if (NG8 || ng > 1) {
+    xs[1][0] = *reinterpret_cast<const uint4*>(st_src + kGroup);
+    xs[1][1] = *reinterpret_cast<const uint4*>(st_src + kGroup + 8);
+  }
+  if (NG8 || ng > 2) {
+    xs[0][0] = *reinterpret_cast<const uint4*>(st_src + 2 * kGroup);
+    xs[0][1] = *reinterpret_cast<const uint4*>(st_src + 2 * kGroup + 8);
+  }
+  qmm_trace(a, work, 1);
+
+  if (threadIdx.x < kTileTokens) s_slot[threadIdx.x] = threadIdx.x < count ? slot : 0xFFFFFFFFu;
+  // 2 * scale (the codes enter as 8 + q/2) of the wave's rows, transposed to [g][row], as fp32
+#pragma unroll
+  for (int p = 0; p < NPROJ; ++p) {
+    float* tab = s_scale + (p * kQmmWaves + wv) * ng * 32;
+    const uint16_t* src = Sp[p] + static_cast<size_t>(row_base[p] + m) * ng;
+    for (uint32_t g0 = h * 8; g0 < ng; g0 += 16) {  // lane: row m, 8 groups from g0
+      const uint4 v = NG8 ? load_x8<false>(src + g0) : load_bf16x8_guarded(src + g0, ng - g0);
+      const uint32_t pr[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        if (NG8 || g0 + 2 * i < ng) tab[(g0 + 2 * i) * 32 + m] = 2.0f * bf16_lo(pr[i]);
+        if (NG8 || g0 + 2 * i + 1 < ng) tab[(g0 + 2 * i + 1) * 32 + m] = 2.0f * bf16_hi(pr[i]);
       }
     }
   }
@@ -386,8 +478,66 @@ void qmm_kernel(const QmmArgs a) {
 #pragma unroll
       for (int r = 0; r < 16; ++r) acc[p][nt][r] = 0.0f;
 
-  const bool st_live = st_row != 0xFFFFFFFFu;
-  const uint16_t* st_src = a.x + static_cast<size_t>(st_live ? st_row : 0) * a.x_stride + st_q * 16;
+  // ---- bias and offset terms: acc[token, row] += sumx[token, g] * B[row, g] + sumx[token, g] * (-16 S[row, g]).
+  // -16 * S is formed in place (exponent + 4, sign flipped: exact; a zero scale becomes 2^-123).
+  // sumx enters as three bf16 terms, which hold all 24 bits: the -16 * S * sumx term cancels the
+  // 16 * sum(x) the matrix core accumulated with the codes, so it has to be exact.
+  for (uint32_t g0 = 0; g0 < ng; g0 += 16) {
+    const uint32_t gl = g0 + 8 * h;  // this lane's 8 groups
+    const bool have = gl < ng;
+    const uint32_t gc = have ? gl : 0;  // a lane without groups reads group 0 and drops it
+    uint4 ab[NPROJ], as[NPROJ];
+#pragma unroll
+    for (int p = 0; p < NPROJ; ++p) {
+      const size_t at = static_cast<size_t>(row_base[p] + m) * ng + gc;
+      ab[p] = NG8 ? load_x8<false>(Bp[p] + at) : load_bf16x8_guarded(Bp[p] + at, ng - gc);
+      const uint4 sv = NG8 ? load_x8<false>(Sp[p] + at) : load_bf16x8_guarded(Sp[p] + at, ng - gc);
+      as[p] = make_uint4((sv.x + 0x02000200u) ^ 0x80008000u, (sv.y + 0x02000200u) ^ 0x80008000u,
+                         (sv.z + 0x02000200u) ^ 0x80008000u, (sv.w + 0x02000200u) ^ 0x80008000u);
+      if (!have) ab[p] = as[p] = make_uint4(0, 0, 0, 0);
+    }
+#pragma unroll
+    for (int nt = 0; nt < 2; ++nt) {
+      float sx[8];
+      const float* sp = a.sumx + static_cast<size_t>(xrow[nt]) * ng + gc;
+      if (NG8) {
+        const float4 s0 = *reinterpret_cast<const float4*>(sp), s1 = *reinterpret_cast<const float4*>(sp + 4);
+        sx[0] = s0.x; sx[1] = s0.y; sx[2] = s0.z; sx[3] = s0.w;
+        sx[4] = s1.x; sx[5] = s1.y; sx[6] = s1.z; sx[7] = s1.w;
+      } else {
+#pragma unroll
+        for (int e = 0; e < 8; ++e) sx[e] = gc + e < ng ? sp[e] : 0.0f;
+      }
+      uint32_t hi[8], mid[8], lo[8];
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        const float v = sx[e];
+        hi[e] = __float_as_uint(v) & 0xFFFF0000u;
+        const float r1 = v - __uint_as_float(hi[e]);
+        mid[e] = __float_as_uint(r1) & 0xFFFF0000u;
+        lo[e] = __float_as_uint(r1 - __uint_as_float(mid[e]));
+      }
+      const uint4 b_hi = make_uint4((hi[0] >> 16) | hi[1], (hi[2] >> 16) | hi[3], (hi[4] >> 16) | hi[5],
+                                    (hi[6] >> 16) | hi[7]);
+      const uint4 b_mid = make_uint4((mid[0] >> 16) | mid[1], (mid[2] >> 16) | mid[3], (mid[4] >> 16) | mid[5],
+                                     (mid[6] >> 16) | mid[7]);
+      const uint4 b_lo = make_uint4(__builtin_amdgcn_perm(lo[1], lo[0], 0x07060302u),
+                                    __builtin_amdgcn_perm(lo[3], lo[2], 0x07060302u),
+                                    __builtin_amdgcn_perm(lo[5], lo[4], 0x07060302u),
+                                    __builtin_amdgcn_perm(lo[7], lo[6], 0x07060302u));
+#pragma unroll
+      for (int p = 0; p < NPROJ; ++p) {
+        acc[p][nt] = mfma_bf16(b_hi, ab[p], acc[p][nt]);
+        acc[p][nt] = mfma_bf16(b_hi, as[p], acc[p][nt]);
+        acc[p][nt] = mfma_bf16(b_mid, ab[p], acc[p][nt]);
+        acc[p][nt] = mfma_bf16(b_mid, as[p], acc[p][nt]);
+        acc[p][nt] = mfma_bf16(b_lo, ab[p], acc[p][nt]);
+        acc[p][nt] = mfma_bf16(b_lo, as[p], acc[p][nt]);
+      }
+    }
+  }
+  qmm_trace(a, work, 2);
+
   // run c = 2q (+1): K 8c..8c+7 -> slot (h = c / 4, s = c % 4)
   const uint32_t st_nt = st_i >> 5, st_n = st_i & 31, c0 = 2 * st_q, c1 = c0 + 1;
   // inside a 32-token block the column is rotated by 4 * ((s >> 1) + 2h): the four lanes that
@@ -398,41 +548,12 @@ void qmm_kernel(const QmmArgs a) {
   uint32_t rd_col[4];
 #pragma unroll
   for (int sidx = 0; sidx < 4; ++sidx) rd_col[sidx] = (m + 4 * (sidx >> 1) + 8 * h) & 31;
+  s_x[st_slot0] = x0[0];
+  s_x[st_slot1] = x0[1];
 
   // Weight codes run four K groups ahead in registers (the expert's bytes come
   // from HBM); x rows come from L2 and run three groups ahead, two in registers,
   // one in the LDS buffer that is not being read.
-  const uint8_t* wrow[NPROJ];
-  uint4 cur[NPROJ][4], nxt[NPROJ][4];
-#pragma unroll
-  for (int p = 0; p < NPROJ; ++p) {
-    wrow[p] = Wp[p] + (row_base + m) * row_bytes + h * 16;
-#pragma unroll
-    for (int u = 0; u < 4; ++u) {
-      cur[p][u] = make_uint4(0, 0, 0, 0);
-      if (static_cast<uint32_t>(u) < ng) cur[p][u] = *reinterpret_cast<const uint4*>(wrow[p] + u * 32);
-    }
-  }
-  uint4 xs[2][2];  // xs[k & 1] holds group k on its way to LDS
-#pragma unroll
-  for (int k = 0; k < 2; ++k) xs[k][0] = xs[k][1] = make_uint4(0, 0, 0, 0);
-  if (st_live) {
-    xs[0][0] = *reinterpret_cast<const uint4*>(st_src);
-    xs[0][1] = *reinterpret_cast<const uint4*>(st_src + 8);
-    s_x[st_slot0] = xs[0][0];
-    s_x[st_slot1] = xs[0][1];
-    if (ng > 1) {
-      xs[1][0] = *reinterpret_cast<const uint4*>(st_src + kGroup);
-      xs[1][1] = *reinterpret_cast<const uint4*>(st_src + kGroup + 8);
-    }
-    if (ng > 2) {
-      xs[0][0] = *reinterpret_cast<const uint4*>(st_src + 2 * kGroup);
-      xs[0][1] = *reinterpret_cast<const uint4*>(st_src + 2 * kGroup + 8);
-    }
-  } else {
-    s_x[st_slot0] = xs[0][0];
-    s_x[st_slot1] = xs[0][1];
-  }
 
   for (uint32_t g0 = 0; g0 < ng; g0 += 4) {
 #pragma unroll
@@ -445,7 +566,7 @@ void qmm_kernel(const QmmArgs a) {
         uint4* wbuf = s_x + ((u + 1) & 1) * 512;
         wbuf[st_slot0] = xs[(u + 1) & 1][0];
         wbuf[st_slot1] = xs[(u + 1) & 1][1];
-        if (g + 3 < ng && st_live) {
+        if (g + 3 < ng) {
           xs[(u + 1) & 1][0] = *reinterpret_cast<const uint4*>(st_src + (g + 3) * kGroup);
           xs[(u + 1) & 1][1] = *reinterpret_cast<const uint4*>(st_src + (g + 3) * kGroup + 8);
         }
@@ -460,7 +581,7 @@ void qmm_kernel(const QmmArgs a) {
           }
       }
 
-      // ---- matrix core: tmp[token, row] = sum over the group of x * (128+q)
+      // ---- matrix core: tmp[token, row] = sum over the group of x * (8 + q/2)
       const uint4* buf = s_x + (u & 1) * 512;
       uint4 bx[2][4];
 #pragma unroll
@@ -494,59 +615,8 @@ void qmm_kernel(const QmmArgs a) {
       for (int v = 0; v < 4; ++v) cur[p][v] = nxt[p][v];
   }
 
-  // ---- bias and offset terms: acc[token, row] += sumx[token, g] * B[row, g] + sumx[token, g] * (-128 S[row, g]).
-  // -128 * S is formed in place (exponent + 7, sign flipped: exact; a zero scale becomes 2^-120).
-  // sumx enters as three bf16 terms, which hold all 24 bits: the -128 * S * sumx term cancels the
-  // 128 * sum(x) the matrix core accumulated with the codes, so it has to be exact.
-  for (uint32_t g0 = 0; g0 < ng; g0 += 16) {
-    const uint32_t gl = g0 + 8 * h;  // this lane's 8 groups
-    uint4 ab[NPROJ], as[NPROJ];
-#pragma unroll
-    for (int p = 0; p < NPROJ; ++p) {
-      ab[p] = as[p] = make_uint4(0, 0, 0, 0);
-      if (gl < ng) {
-        ab[p] = load_bf16x8_guarded(Bp[p] + static_cast<size_t>(row_base + m) * ng + gl, ng - gl);
-        const uint4 sv = load_bf16x8_guarded(Sp[p] + static_cast<size_t>(row_base + m) * ng + gl, ng - gl);
-        as[p] = make_uint4((sv.x + 0x03800380u) ^ 0x80008000u, (sv.y + 0x03800380u) ^ 0x80008000u,
-                           (sv.z + 0x03800380u) ^ 0x80008000u, (sv.w + 0x03800380u) ^ 0x80008000u);
-      }
-    }
-#pragma unroll
-    for (int nt = 0; nt < 2; ++nt) {
-      uint32_t hi[8], mid[8], lo[8];
-      const float* sp = a.sumx + static_cast<size_t>(xrow[nt] == 0xFFFFFFFFu ? 0 : xrow[nt]) * ng;
-#pragma unroll
-      for (int e = 0; e < 8; ++e) {
-        const float v = (xrow[nt] != 0xFFFFFFFFu && gl + e < ng) ? sp[gl + e] : 0.0f;
-        hi[e] = __float_as_uint(v) & 0xFFFF0000u;
-        const float r1 = v - __uint_as_float(hi[e]);
-        mid[e] = __float_as_uint(r1) & 0xFFFF0000u;
-        lo[e] = __float_as_uint(r1 - __uint_as_float(mid[e]));
-      }
-      const uint4 b_hi = make_uint4((hi[0] >> 16) | hi[1], (hi[2] >> 16) | hi[3], (hi[4] >> 16) | hi[5],
-                                    (hi[6] >> 16) | hi[7]);
-      const uint4 b_mid = make_uint4((mid[0] >> 16) | mid[1], (mid[2] >> 16) | mid[3], (mid[4] >> 16) | mid[5],
-                                     (mid[6] >> 16) | mid[7]);
-      const uint4 b_lo = make_uint4(__builtin_amdgcn_perm(lo[1], lo[0], 0x07060302u),
-                                    __builtin_amdgcn_perm(lo[3], lo[2], 0x07060302u),
-                                    __builtin_amdgcn_perm(lo[5], lo[4], 0x07060302u),
-                                    __builtin_amdgcn_perm(lo[7], lo[6], 0x07060302u));
-#pragma unroll
-      for (int p = 0; p < NPROJ; ++p) {
-        acc[p][nt] = mfma_bf16(b_hi, ab[p], acc[p][nt]);
-        acc[p][nt] = mfma_bf16(b_hi, as[p], acc[p][nt]);
-        acc[p][nt] = mfma_bf16(b_mid, ab[p], acc[p][nt]);
-        acc[p][nt] = mfma_bf16(b_mid, as[p], acc[p][nt]);
-        acc[p][nt] = mfma_bf16(b_lo, ab[p], acc[p][nt]);
-        acc[p][nt] = mfma_bf16(b_lo, as[p], acc[p][nt]);
-      }
-    }
-  }
-
-  // ---- epilogue: the lane holds weight row `row` for tokens 8j + 4h + i of each 32-token block
-  const uint32_t row = row_base + m;
-  // position of the row inside its run of 8 in the (0,4,1,5,2,6,3,7) order phase 2 reads
-  const uint32_t row_p = (row & ~7u) + ((row & 3u) << 1) + ((row >> 2) & 1u);
+  qmm_trace(a, work, 3);
+  // ---- epilogue: the lane holds weight row row_base[p] + m for tokens 8j + 4h + i of each 32-token block
 #pragma unroll
   for (int nt = 0; nt < 2; ++nt) {
 #pragma unroll
@@ -567,15 +637,22 @@ void qmm_kernel(const QmmArgs a) {
             gv = fminf(gv, a.limit);
             uv = fminf(fmaxf(uv, -a.limit), a.limit);
           }
-          static_cast<uint16_t*>(a.out)[at + row_p] = f_to_bf16(fast_silu(gv) * uv);
-        } else if (a.epi == 1) {
-          static_cast<float*>(a.out)[at + row] = acc[0][nt][4 * j + i];
+          // position of the row inside its run of 8 in the (0,4,1,5,2,6,3,7) order phase 2 reads
+          const uint32_t row = row_base[0] + m;
+          const uint32_t row_p = (row & ~7u) + ((row & 3u) << 1) + ((row >> 2) & 1u);
+          static_cast<uint16_t*>(a.out)[at + row_p] = f_to_bf16(mf_silu(gv) * uv);
         } else {
-          static_cast<uint16_t*>(a.out)[at + row] = f_to_bf16(acc[0][nt][4 * j + i]);
+#pragma unroll
+          for (int p = 0; p < NPROJ; ++p) {
+            if (p > 0 && !a.pair_rows) break;
+            if (a.epi == 1) static_cast<float*>(a.out)[at + row_base[p] + m] = acc[p][nt][4 * j + i];
+            else static_cast<uint16_t*>(a.out)[at + row_base[p] + m] = f_to_bf16(acc[p][nt][4 * j + i]);
+          }
         }
       }
     }
   }
+  qmm_trace(a, work, 4);
 }
 
 // y[t,d] = bf16(h1[t,d] + sum_r w[t,r] * partial[t*K+r, d]), residual first, rank
@@ -619,7 +696,7 @@ __global__ __launch_bounds__(256) void prefill_reduce_kernel(const float* __rest
 hipError_t launch_prefill_router(hipStream_t s, const uint16_t* W, const uint16_t* x, uint32_t E,
                                  uint32_t D, uint32_t T, uint32_t x_stride, float* logits) {
   const uint32_t cpl = (D / 8 + 63) / 64;
-  const uint32_t tpb = 64;
+  const uint32_t tpb = std::max(1u, std::min(64u, T / 64));  // about a thousand workgroups
 #define MF_PR(CPL, R)                                                                              \
   prefill_router_kernel<CPL, R><<<dim3((E + 4 * R - 1) / (4 * R), (T + tpb - 1) / tpb), dim3(256), 0, s>>>( \
       W, x, E, D, T, x_stride, logits, tpb)
@@ -634,15 +711,23 @@ hipError_t launch_prefill_router(hipStream_t s, const uint16_t* W, const uint16_
 
 hipError_t launch_group(hipStream_t s, const uint32_t* idx, const float* w, uint32_t t, uint32_t K,
                         uint32_t E, uint32_t* counts, uint32_t* offsets, uint32_t* starts,
-                        mf_pair* sorted, void* tiles, uint32_t* n_tiles, uint32_t* status) {
+                        mf_pair* sorted, void* tiles, uint32_t tile_slots, uint32_t* n_tiles,
+                        uint32_t* status, uint32_t* chunk_hist) {
   const uint32_t n_pairs = t * K;
+  // at most kGroupChunks chunks, each a whole number of kGroupBlock-pair steps
+  const uint32_t steps = (n_pairs + kGroupBlock - 1) / kGroupBlock;
+  const uint32_t chunk_pairs = (steps + kGroupChunks - 1) / kGroupChunks * kGroupBlock;
+  const uint32_t n_chunks = (n_pairs + chunk_pairs - 1) / chunk_pairs;
   zero_words_kernel<<<dim3(1), dim3(64), 0, s>>>(status, 1);  // a fill kernel: safe under graph capture
-  group_count_kernel<<<dim3((E + 3) / 4), dim3(256), 0, s>>>(idx, n_pairs, E, counts, status);
-  group_scan_kernel<<<dim3(1), dim3(MF_MAX_EXPERTS), 0, s>>>(counts, E, offsets, starts,
-                                                             static_cast<Tile*>(tiles), n_tiles);
-  group_emit_kernel<<<dim3((E + 3) / 4), dim3(256), 0, s>>>(idx, w, n_pairs, K, E, starts, sorted);
+  group_count_kernel<<<dim3(n_chunks), dim3(256), 0, s>>>(idx, n_pairs, E, chunk_pairs, chunk_hist, status);
+  group_scan_kernel<<<dim3(1), dim3(MF_MAX_EXPERTS), 0, s>>>(chunk_hist, n_chunks, E, counts, offsets, starts,
+                                                             static_cast<Tile*>(tiles), tile_slots, n_tiles);
+  group_emit_kernel<<<dim3(n_chunks), dim3(256), 0, s>>>(idx, w, n_pairs, K, E, chunk_pairs, chunk_hist, starts,
+                                                         sorted);
   return hipGetLastError();
 }
+
+size_t group_scratch_words() { return 2048 + static_cast<size_t>(kGroupChunks) * MF_MAX_EXPERTS; }
 
 size_t qmm_lds_bytes(uint32_t kdim, int nproj) {
   const uint32_t ng = kdim / kGroup;
@@ -656,24 +741,31 @@ hipError_t launch_prep_rows(hipStream_t s, const uint16_t* src, uint16_t* dst, f
   return hipGetLastError();
 }
 
-hipError_t launch_qmm(hipStream_t s, const QmmArgs& a, int nproj, uint32_t max_tiles) {
+// tile_slots: entries of the tile list (routed; a multiple of 8) or number of 64-row tiles (dense)
+hipError_t launch_qmm(hipStream_t s, QmmArgs a, int nproj, uint32_t tile_slots) {
   const size_t lds = qmm_lds_bytes(a.kdim, nproj);
-  const dim3 grid((max_tiles * (a.rows / kQmmRows) + 7) / 8 * 8), block(256);
+  const uint32_t n_slices = a.rows / (kQmmRows * (a.pair_rows ? nproj : 1));
+  if (a.dense_mode) {
+    a.dense_tiles = tile_slots;
+    tile_slots = (tile_slots + 7) / 8 * 8;
+  }
+  const dim3 grid(tile_slots * n_slices), block(256);
   if (grid.x == 0) return hipSuccess;
+  const bool ng8 = (a.kdim / kGroup) % 8 == 0;
+  const void* fn = nproj == 2 ? (ng8 ? reinterpret_cast<const void*>(qmm_kernel<2, true>)
+                                     : reinterpret_cast<const void*>(qmm_kernel<2, false>))
+                              : (ng8 ? reinterpret_cast<const void*>(qmm_kernel<1, true>)
+                                     : reinterpret_cast<const void*>(qmm_kernel<1, false>));
+  if (lds > 48 * 1024) {
+    hipError_t e = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds));
+    if (e != hipSuccess) return e;
+  }
   if (nproj == 2) {
-    if (lds > 48 * 1024) {
-      hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(qmm_kernel<2>),
-                                         hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds));
-      if (e != hipSuccess) return e;
-    }
-    qmm_kernel<2><<<grid, block, lds, s>>>(a);
+    if (ng8) qmm_kernel<2, true><<<grid, block, lds, s>>>(a);
+    else qmm_kernel<2, false><<<grid, block, lds, s>>>(a);
   } else {
-    if (lds > 48 * 1024) {
-      hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(qmm_kernel<1>),
-                                         hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds));
-      if (e != hipSuccess) return e;
-    }
-    qmm_kernel<1><<<grid, block, lds, s>>>(a);
+    if (ng8) qmm_kernel<1, true><<<grid, block, lds, s>>>(a);
+    else qmm_kernel<1, false><<<grid, block, lds, s>>>(a);
   }
   return hipGetLastError();
 }
@@ -681,6 +773,13 @@ hipError_t launch_qmm(hipStream_t s, const QmmArgs& a, int nproj, uint32_t max_t
 namespace {
 size_t up256(size_t v) { return (v + 255) / 256 * 256; }
 }  // namespace
+
+// entries of the tile list: every live expert may end in a partial tile; a multiple of 8
+uint32_t prefill_tile_slots(const mf_moe_config& c, uint32_t t) {
+  const size_t pairs = static_cast<size_t>(t) * c.top_k;
+  const size_t n = std::min<size_t>(c.num_experts, pairs) + pairs / kTileTokens + 1;
+  return static_cast<uint32_t>((n + 7) / 8 * 8);
+}
 
 // workspace carve-up of one prefill layer call
 struct PrefillWs {
@@ -700,7 +799,7 @@ PrefillWs prefill_carve(const mf_moe_config& c, uint32_t t, void* base) {
     return static_cast<void*>(base ? at : nullptr);
   };
   const size_t pairs = static_cast<size_t>(t) * c.top_k;
-  const size_t max_tiles = std::min<size_t>(c.num_experts, pairs) + pairs / kTileTokens + 1;
+  const size_t max_tiles = prefill_tile_slots(c, t);
   p.logits = static_cast<float*>(take(sizeof(float) * t * c.num_experts));
   p.idx = static_cast<uint32_t*>(take(sizeof(uint32_t) * pairs));
   p.w = static_cast<float*>(take(sizeof(float) * pairs));
@@ -742,13 +841,12 @@ hipError_t launch_prefill_layer(hipStream_t s, const mf_moe& h, const mf_moe_lay
   const PrefillWs ws = prefill_carve(c, t, workspace);
   hipError_t e;
 #define MF_TRY(call) do { e = (call); if (e != hipSuccess) return e; } while (0)
+  const size_t pairs = static_cast<size_t>(t) * c.top_k;
+  const uint32_t max_tiles = prefill_tile_slots(c, t);
   MF_TRY(launch_prefill_router(s, w.router_w, x, c.num_experts, c.d, t, c.d, ws.logits));
   MF_TRY(launch_topk(s, ws.logits, c.num_experts, c.top_k, t, c.router_mode, ws.idx, ws.w));
   MF_TRY(launch_group(s, ws.idx, ws.w, t, c.top_k, c.num_experts, ws.counts, ws.offsets, ws.starts,
-                      ws.sorted, ws.tiles, ws.n_tiles, ws.status));
-  const size_t pairs = static_cast<size_t>(t) * c.top_k;
-  const uint32_t max_tiles =
-      static_cast<uint32_t>(std::min<size_t>(c.num_experts, pairs) + pairs / kTileTokens + 1);
+                      ws.sorted, ws.tiles, max_tiles, ws.n_tiles, ws.status, h.ws.group_tmp + 2048));
 
   MF_TRY(launch_prep_rows(s, x, ws.xp, ws.sum_x, static_cast<size_t>(t) * c.d));
 
@@ -760,6 +858,10 @@ hipError_t launch_prefill_layer(hipStream_t s, const mf_moe& h, const mf_moe_lay
   q.n_tiles = ws.n_tiles;
   q.top_k = c.top_k;
   q.limit = c.swiglu_limit;
+  if (h.trace && h.trace_bytes >= 64) {  // stage stamps of the routed gate/up matmul
+    q.trace = h.trace;
+    q.trace_items = static_cast<uint32_t>(std::min<size_t>(h.trace_bytes / 64, 1u << 30));
+  }
   // routed phase 1: gate/up -> acts [pair, F]
   q.w_off[0] = w.offsets.gate_w; q.s_off[0] = w.offsets.gate_s; q.b_off[0] = w.offsets.gate_b;
   q.w_off[1] = w.offsets.up_w; q.s_off[1] = w.offsets.up_s; q.b_off[1] = w.offsets.up_b;
@@ -772,7 +874,9 @@ hipError_t launch_prefill_layer(hipStream_t s, const mf_moe& h, const mf_moe_lay
   q.w_off[0] = w.offsets.down_w; q.s_off[0] = w.offsets.down_s; q.b_off[0] = w.offsets.down_b;
   q.x = ws.acts; q.sumx = ws.sum_acts; q.x_stride = c.f; q.gather = 0; q.rows = c.d; q.kdim = c.f; q.epi = 1; q.out = ws.partials;
   q.limit = 0.0f;
-  MF_TRY(launch_qmm(s, q, 1, max_tiles));
+  q.trace = nullptr;
+  q.pair_rows = c.d % (2 * kQmmRows) == 0;
+  MF_TRY(launch_qmm(s, q, q.pair_rows ? 2 : 1, max_tiles));
   const uint16_t* hs = nullptr;
   const uint16_t* gate = nullptr;
   if (c.shared_f) {
@@ -785,7 +889,8 @@ hipError_t launch_prefill_layer(hipStream_t s, const mf_moe& h, const mf_moe_lay
     MF_TRY(launch_prep_rows(s, ws.sact, nullptr, ws.sum_sact, static_cast<size_t>(t) * c.shared_f));
     d.dense[0] = w.shared_down;
     d.x = ws.sact; d.sumx = ws.sum_sact; d.x_stride = c.shared_f; d.rows = c.d; d.kdim = c.shared_f; d.epi = 2; d.out = ws.hs;
-    MF_TRY(launch_qmm(s, d, 1, dense_tiles));
+    d.pair_rows = c.d % (2 * kQmmRows) == 0;
+    MF_TRY(launch_qmm(s, d, d.pair_rows ? 2 : 1, dense_tiles));
     hs = ws.hs;
     if (w.w_sg) {
       MF_TRY(launch_router_logits(s, w.w_sg, x, 1, c.d, t, c.d, nullptr, ws.gate));

@@ -24,6 +24,7 @@ if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBPS = 8000.0  # MI355X HBM3E, published peak
+MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16 matrix peak, published
 ROOT_SEED = 0x4D464D4F00000000
 
 QWEN = dict(name="qwen3.6-35b-a3b-moe-layer-decode-T1-4bit-g64", config=1, d=2048, f=512, e=256,
@@ -117,6 +118,69 @@ def profiled_traffic_bytes():
         return None
 
 
+def measure_prefill(ctx, w, layer, device, tokens=(128, 512, 2048), steps=100, warmup=100):
+    """Ragged prefill of one layer of the same shape: T tokens, top-k routing from skewed
+    logits (router weights plus a per-expert bias ~ N(0, 1.5), carried by a constant-one last
+    feature of x and the last column of the router, so expert loads are uneven and some
+    experts get no token).  Parity at the smallest T against the per-token CPU checker."""
+    import numpy as np
+    import torch
+    from mference_amd import operators as ops
+    from oracle import mf_oracle as O
+
+    gen = torch.Generator(device=device)
+    gen.manual_seed((ROOT_SEED + 0x100 * 2 + 0x7F) & 0x7FFFFFFFFFFFFFFF)
+    router = layer.router_w.clone()
+    router[:, -1] = (torch.randn((w["e"],), generator=gen, device=device) * 1.5).to(torch.bfloat16)
+    lw = ops.MoELayerWeights(router, layer.experts, layer.offsets, layer.shared, layer.w_sg)
+    moe = ops.MoE(ctx, w["d"], w["f"], w["e"], w["k"], bits=w["bits"], shared_f=w["fs"],
+                  shared_bits=w["shared_bits"])
+    out = {"workload": "qwen3.6-35b-a3b-moe-layer-ragged-prefill-4bit-g64, skewed routing",
+           "dtype": "u4 codes (exact, as bf16) x bf16 activations on bf16 MFMA, fp32 accumulate",
+           "runs": []}
+    for t in tokens:
+        x = torch.randn((t, w["d"]), generator=gen, device=device).to(torch.bfloat16)
+        x[:, -1] = 1.0
+        y = torch.zeros_like(x)
+        idx = torch.zeros((t, w["k"]), dtype=torch.int32, device=device)
+        ws = moe.encode_prefill_layer(lw, x, y, t, out_indices=idx)
+        torch.cuda.synchronize()
+        counts = torch.bincount(idx.flatten().long(), minlength=w["e"]).cpu().numpy()
+        run = {"tokens": t}
+        if t == min(tokens):
+            host = layer_to_host(lw, w)
+            ref_y, ref_idx, _ = O.moe_layer(host, ops.bf16_bits(x))
+            got = O.bf16_to_float(ops.bf16_bits(y)).astype(np.float64)
+            ref = O.bf16_to_float(ref_y).astype(np.float64)
+            run["parity"] = dict(
+                routing_bit_exact=bool(np.array_equal(idx.cpu().numpy().astype(np.uint32), ref_idx)),
+                max_abs=float(np.abs(got - ref).max()),
+                rel_l2=float(np.linalg.norm(got - ref) / np.linalg.norm(ref)))
+        for _ in range(warmup):
+            moe.encode_prefill_layer(lw, x, y, t, workspace=ws)
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(steps):
+            moe.encode_prefill_layer(lw, x, y, t, workspace=ws)
+        e1.record()
+        torch.cuda.synchronize()
+        us = e0.elapsed_time(e1) / steps * 1e3
+        flops = 2.0 * 3 * w["d"] * (t * w["k"] * w["f"] + t * w["fs"])
+        tflops = flops / us / 1e6
+        run.update(us_per_layer=round(us, 1), tokens_per_s=round(t / us * 1e6, 1),
+                   tflops=round(tflops, 1), mfma_frac=round(tflops / MFMA_BF16_PEAK_TFLOPS, 4),
+                   experts_without_tokens=int((counts == 0).sum()), max_expert_load=int(counts.max()),
+                   output_finite=bool(torch.isfinite(y.float()).all().item()))
+        out["runs"].append(run)
+    last = out["runs"][-1]
+    out["roofline"] = {"bound": "mfma", "achieved": last["tflops"], "peak": MFMA_BF16_PEAK_TFLOPS,
+                       "unit": "TFLOP/s", "frac": last["mfma_frac"], "traffic": None,
+                       "kernel": "whole layer at T=%d (router, grouping, mf::qmm_kernel x4, reduce); "
+                                 "algorithmic flops = 2*3*D*(T*K*F + T*Fs)" % last["tokens"]}
+    return out
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -129,6 +193,9 @@ def main() -> int:
                     help="also run three 256 MiB device-to-device copies (a kernel of known HBM "
                          "traffic) so that FETCH_SIZE / WRITE_SIZE counters can be scaled")
     ap.add_argument("--cpu-seconds", type=float, default=12.0)
+    ap.add_argument("--no-prefill", action="store_true", help="skip the ragged prefill section")
+    ap.add_argument("--prefill-only", action="store_true",
+                    help="one layer, the ragged prefill section only (for profiling)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build measures one GPU only (--gpus 1); no multi-GPU path exists",
@@ -144,8 +211,13 @@ def main() -> int:
     torch.cuda.set_device(device)
     w = QWEN
     L, K, W = args.layers, args.steps, args.warmup
+    if args.prefill_only:
+        L = 1
     ctx = ops.MetalContext(0)
     stack = build_stack(ctx, w, L, device)
+    if args.prefill_only:
+        print(json.dumps({"prefill": measure_prefill(ctx, w, stack[0], device)}))
+        return 0
     moes = [ops.MoE(ctx, w["d"], w["f"], w["e"], w["k"], bits=w["bits"], shared_f=w["fs"],
                     shared_bits=w["shared_bits"]) for _ in range(L)]
 
@@ -243,6 +315,8 @@ def main() -> int:
                      "algorithmic_bytes_per_layer": ab["expert_bytes"]},
     }
 
+    if not args.no_prefill:
+        out["prefill"] = measure_prefill(ctx, w, stack[0], device)
     if not args.no_cpu_baseline:
         # the CPU checker (a restatement of the reference's CPU path: bulk
         # dequantize each row, scalar fp32 dot, experts in slot order) timed on

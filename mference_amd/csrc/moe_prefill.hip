@@ -100,6 +100,115 @@ __global__ __launch_bounds__(256) void prefill_router_kernel(const uint16_t* __r
   }
 }
 
+// The same logits on the fp32 matrix core, still bit for bit: a K=1 outer-product MFMA adds
+// exactly one product to every accumulator element, c <- fl(c + x*w), and x*w is exact for
+// bf16 inputs -- so a run of K=1 MFMAs is the per-lane fmaf chain of dot_bf16_row for a whole
+// 32-token x 32-expert block at once.  "Lane l" of the reference order becomes chain l: the K
+// values 8l..8l+7, then +512, +1024, ...  The two blocks of one instruction carry chains l and
+// l+1; their accumulators are added (the stride-1 level of the butterfly), then combined with
+// the later pairs as a binary counter, which reproduces the ascending-stride tree.  Each of the
+// four waves of a workgroup owns 16 chains; the last two levels go through LDS.
+// Needs D % 512 == 0 (all 64 chains the same length) and E % 32 == 0.
+typedef __attribute__((ext_vector_type(32))) float f32x32_t;
+
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) void prefill_router_mfma_kernel(const uint16_t* __restrict__ W,
+                                                                  const uint16_t* __restrict__ x,
+                                                                  uint32_t E, uint32_t D, uint32_t T,
+                                                                  uint32_t x_stride,
+                                                                  float* __restrict__ logits) {
+  __shared__ float s_part[3][16 * 64];
+  const uint32_t lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
+  const uint32_t m = lane & 31, b = lane >> 5;
+  const uint32_t t0 = blockIdx.y * 32, e0 = blockIdx.x * 32;
+  const uint32_t n_i = D / 512;
+  const uint16_t* xrow = x + static_cast<size_t>(min(t0 + m, T - 1)) * x_stride + 8 * (16 * wv + b);
+  const uint16_t* wrow = W + static_cast<size_t>(e0 + m) * D + 8 * (16 * wv + b);
+
+  float lev0[16], lev1[16], lev2[16], total[16];
+#pragma unroll
+  for (int r = 0; r < 16; ++r) lev0[r] = lev1[r] = lev2[r] = total[r] = 0.0f;
+  // step q = pp * n_i + i: chain pair pp (chains 16 wv + 2 pp + b), K run i; operands run 4 steps ahead
+  const uint32_t steps = 8 * n_i;
+  uint4 cx[4], cw[4], nx[4], nw[4];
+#pragma unroll
+  for (int u = 0; u < 4; ++u) {
+    const uint32_t q = min(static_cast<uint32_t>(u), steps - 1), off = 16 * (q / n_i) + 512 * (q % n_i);
+    cx[u] = *reinterpret_cast<const uint4*>(xrow + off);
+    cw[u] = *reinterpret_cast<const uint4*>(wrow + off);
+  }
+  f32x32_t acc;
+#pragma unroll
+  for (int r = 0; r < 32; ++r) acc[r] = 0.0f;
+  uint32_t pp = 0, i = 0;
+  for (uint32_t q0 = 0; q0 < steps; q0 += 4) {
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      const uint32_t q = min(q0 + 4 + u, steps - 1), off = 16 * (q / n_i) + 512 * (q % n_i);
+      nx[u] = *reinterpret_cast<const uint4*>(xrow + off);
+      nw[u] = *reinterpret_cast<const uint4*>(wrow + off);
+    }
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      if (q0 + u >= steps) break;
+      const uint32_t xw[4] = {cx[u].x, cx[u].y, cx[u].z, cx[u].w}, ww[4] = {cw[u].x, cw[u].y, cw[u].z, cw[u].w};
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        acc = __builtin_amdgcn_mfma_f32_32x32x1f32(bf16_lo(xw[j]), bf16_lo(ww[j]), acc, 0, 0, 0);
+        acc = __builtin_amdgcn_mfma_f32_32x32x1f32(bf16_hi(xw[j]), bf16_hi(ww[j]), acc, 0, 0, 0);
+      }
+      if (++i == n_i) {  // the pair of chains is complete: stride-1 level, then the binary counter
+        float carry[16];
+#pragma unroll
+        for (int r = 0; r < 16; ++r) carry[r] = acc[r] + acc[16 + r];
+#pragma unroll
+        for (int r = 0; r < 32; ++r) acc[r] = 0.0f;
+        if (pp & 1) {
+#pragma unroll
+          for (int r = 0; r < 16; ++r) carry[r] = lev0[r] + carry[r];
+          if (pp & 2) {
+#pragma unroll
+            for (int r = 0; r < 16; ++r) carry[r] = lev1[r] + carry[r];
+            if (pp & 4) {
+#pragma unroll
+              for (int r = 0; r < 16; ++r) total[r] = lev2[r] + carry[r];
+            } else {
+#pragma unroll
+              for (int r = 0; r < 16; ++r) lev2[r] = carry[r];
+            }
+          } else {
+#pragma unroll
+            for (int r = 0; r < 16; ++r) lev1[r] = carry[r];
+          }
+        } else {
+#pragma unroll
+          for (int r = 0; r < 16; ++r) lev0[r] = carry[r];
+        }
+        i = 0;
+        ++pp;
+      }
+    }
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      cx[u] = nx[u];
+      cw[u] = nw[u];
+    }
+  }
+  if (wv > 0) {
+#pragma unroll
+    for (int r = 0; r < 16; ++r) s_part[wv - 1][r * 64 + lane] = total[r];
+  }
+  __syncthreads();
+  if (wv == 0) {
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+      const float s01 = total[r] + s_part[0][r * 64 + lane];
+      const float s23 = s_part[1][r * 64 + lane] + s_part[2][r * 64 + lane];
+      const uint32_t t = t0 + 8 * (r / 4) + 4 * b + (r % 4);
+      if (t < T) logits[static_cast<size_t>(t) * E + e0 + m] = s01 + s23;
+    }
+  }
+}
+
 // ---------------------------------------------------------------- grouping
 //
 // PrefillMoEGrouping.groupTokenExpertPairs (PrefillMoEGrouping.swift:91-192) on
@@ -147,7 +256,18 @@ __global__ __launch_bounds__(512) void group_scan_kernel(uint32_t* __restrict__ 
   const uint32_t e = threadIdx.x;
   uint32_t c = 0;
   if (e < E) {
-    for (uint32_t k = 0; k < n_chunks; ++k) {
+    uint32_t k = 0;
+    for (; k + 8 <= n_chunks; k += 8) {  // eight independent loads in flight
+      uint32_t v[8];
+#pragma unroll
+      for (int u = 0; u < 8; ++u) v[u] = chunk_hist[(k + u) * E + e];
+#pragma unroll
+      for (int u = 0; u < 8; ++u) {
+        chunk_hist[(k + u) * E + e] = c;
+        c += v[u];
+      }
+    }
+    for (; k < n_chunks; ++k) {
       const uint32_t v = chunk_hist[k * E + e];
       chunk_hist[k * E + e] = c;
       c += v;
@@ -695,6 +815,10 @@ __global__ __launch_bounds__(256) void prefill_reduce_kernel(const float* __rest
 
 hipError_t launch_prefill_router(hipStream_t s, const uint16_t* W, const uint16_t* x, uint32_t E,
                                  uint32_t D, uint32_t T, uint32_t x_stride, float* logits) {
+  if (D % 512 == 0 && E % 32 == 0 && aligned16(W) && aligned16(x) && x_stride % 8 == 0) {
+    prefill_router_mfma_kernel<<<dim3(E / 32, (T + 31) / 32), dim3(256), 0, s>>>(W, x, E, D, T, x_stride, logits);
+    return hipGetLastError();
+  }
   const uint32_t cpl = (D / 8 + 63) / 64;
   const uint32_t tpb = std::max(1u, std::min(64u, T / 64));  // about a thousand workgroups
 #define MF_PR(CPL, R)                                                                              \

@@ -29,18 +29,31 @@ ROOT_SEED = 0x4D464D4F00000000
 
 QWEN = dict(name="qwen3.6-35b-a3b-moe-layer-decode-T1-4bit-g64", config=1, d=2048, f=512, e=256,
             k=8, fs=512, bits=4, shared_bits=4, t=1)
+# the other decode configurations of the same path (selected with --workload; parity-test shapes,
+# measured here so that every configuration has a number)
+WORKLOADS = {
+    "qwen-decode": QWEN,
+    "dsv4-2bit": dict(name="large-2bit-moe-layer-decode-D4096-F2048-E256-K6", config=3, d=4096, f=2048,
+                      e=256, k=6, fs=2048, bits=2, shared_bits=4, t=1, layers=4),
+    "maple-ternary": dict(name="ternary-moe-layer-decode-D2048-F1024-E64-K8", config=4, d=2048, f=1024,
+                          e=64, k=8, fs=0, bits=1, shared_bits=4, t=1, layers=40),
+}
+DENSE_MLP = dict(name="dense-4bit-swiglu-mlp-D5120-F17408", d=5120, f=17408, bits=4, layers=8)
 
 
 def algorithmic_bytes(w) -> dict:
     """Bytes one layer must read at T=1: the K selected experts + the shared
     expert ("expert bytes touched"), and the same plus router, w_sg, x and y."""
     def tensor(rows, cols, bits):
+        if bits == 1:  # ternary: 2-bit codes, one bf16 scale per group, no bias table
+            return rows * cols * 2 // 8 + rows * (cols // 64) * 2
         return rows * cols * bits // 8 + 2 * rows * (cols // 64) * 2
     expert = 2 * tensor(w["f"], w["d"], w["bits"]) + tensor(w["d"], w["f"], w["bits"])
     shared = (2 * tensor(w["fs"], w["d"], w["shared_bits"]) + tensor(w["d"], w["fs"], w["shared_bits"])
               if w["fs"] else 0)
-    expert_bytes = w["k"] * expert + shared
-    total = expert_bytes + w["e"] * w["d"] * 2 + w["d"] * 2 + 2 * w["d"] * 2
+    n_sel = w.get("experts_touched", w["k"])
+    expert_bytes = n_sel * expert + shared
+    total = expert_bytes + w["e"] * w["d"] * 2 + w["d"] * 2 + 2 * w["t"] * w["d"] * 2
     return dict(expert=expert, expert_bytes=expert_bytes, total=total)
 
 
@@ -64,16 +77,20 @@ def build_stack(ctx, w, layers, device):
         gen.manual_seed((ROOT_SEED + 0x100 * w["config"] + l) & 0x7FFFFFFFFFFFFFFF)
         experts = torch.zeros((E, stride), dtype=torch.uint8, device=device)
         for name, rows, cols in (("gate", F, D), ("up", F, D), ("down", D, F)):
-            raw = torch.randn((E * rows, cols), generator=gen, device=device,
-                              dtype=torch.float32) * 0.02
-            q = quant.quantize_affine(raw, w["bits"])
-            del raw
+            if w["bits"] == 1:
+                q = ternary_tensor(gen, E * rows, cols, device)
+            else:
+                raw = torch.randn((E * rows, cols), generator=gen, device=device,
+                                  dtype=torch.float32) * 0.02
+                q = quant.quantize_affine(raw, w["bits"])
+                del raw
             wo, so, bo = (getattr(off, f"{name}_{s}") for s in "wsb")
             nb = q.packed.shape[1] * rows
             experts[:, wo:wo + nb] = q.packed.view(E, nb)
             ns = q.scales.shape[1] * rows * 2
             experts[:, so:so + ns] = q.scales.view(torch.uint8).view(E, ns)
-            experts[:, bo:bo + ns] = q.biases.view(torch.uint8).view(E, ns)
+            if w["bits"] != 1:
+                experts[:, bo:bo + ns] = q.biases.view(torch.uint8).view(E, ns)
             del q
         router_w = (torch.randn((E, D), generator=gen, device=device) * 0.02).to(torch.bfloat16)
         shared = None
@@ -89,6 +106,20 @@ def build_stack(ctx, w, layers, device):
     return stack
 
 
+def ternary_tensor(gen, rows, cols, device):
+    """codes {0,1,2} with p = .25/.5/.25, four per byte; bf16 scale per group of 64 and bias = -scale
+    (the stored form of the reference's row_alpha expansion)"""
+    import torch
+    from mference_amd import operators as ops
+    u = torch.rand((rows, cols), generator=gen, device=device)
+    codes = (u >= 0.25).to(torch.uint8) + (u >= 0.75).to(torch.uint8)
+    c4 = codes.view(rows, cols // 4, 4)
+    packed = (c4[..., 0] | (c4[..., 1] << 2) | (c4[..., 2] << 4) | (c4[..., 3] << 6)).contiguous()
+    scales = (torch.randn((rows, cols // 64), generator=gen, device=device).abs() * 0.02 + 1e-3)
+    scales = scales.to(torch.bfloat16)
+    return ops.QuantizedTensor(packed, scales, -scales, 1, rows, cols)
+
+
 def layer_to_host(wts, w):
     """device layer -> oracle Layer (for the parity check and the CPU baseline)"""
     from mference_amd import operators as ops
@@ -97,8 +128,8 @@ def layer_to_host(wts, w):
     for name, _ in off._fields_:
         setattr(off, name, getattr(wts.offsets, name))
     def q(t):
-        return O.QTensor(t.packed.cpu().numpy(), ops.bf16_bits(t.scales), ops.bf16_bits(t.biases),
-                         t.bits, t.rows, t.n)
+        return O.QTensor(t.packed.cpu().numpy(), ops.bf16_bits(t.scales),
+                         None if t.biases is None else ops.bf16_bits(t.biases), t.bits, t.rows, t.n)
     shared = None if wts.shared is None else tuple(q(t) for t in wts.shared)
     return O.Layer(d=w["d"], f=w["f"], e=w["e"], k=w["k"], bits=w["bits"],
                    router_w=ops.bf16_bits(wts.router_w), experts=wts.experts.cpu().numpy(), off=off,
@@ -181,12 +212,95 @@ def measure_prefill(ctx, w, layer, device, tokens=(128, 512, 2048), steps=100, w
     return out
 
 
+def bench_dense_mlp(args, device) -> int:
+    """Dense 4-bit SwiGLU MLP (hidden 5120, intermediate 17408) at T token rows: the shared-expert
+    operator on a dense layer; `layers` distinct weight sets rotate so HBM is read every step."""
+    import torch
+    from mference_amd import operators as ops
+
+    w = DENSE_MLP
+    t = args.tokens or 1
+    L = args.layers or w["layers"]
+    ctx = ops.MetalContext(0)
+    quant = ops.Quantization(ctx)
+    gen = torch.Generator(device=device)
+    gen.manual_seed((ROOT_SEED + 0x500) & 0x7FFFFFFFFFFFFFFF)
+    D, F = w["d"], w["f"]
+    sets = []
+    for _ in range(L):
+        qs = []
+        for rows, cols in ((F, D), (F, D), (D, F)):
+            raw = torch.randn((rows, cols), generator=gen, device=device) * 0.02
+            qs.append(quant.quantize_affine(raw, 4))
+            del raw
+        sets.append(qs)
+    mlp = ops.SharedExpertInt4(ctx)
+    x = torch.randn((t, D), generator=gen, device=device).to(torch.bfloat16)
+    y = torch.zeros((L, t, D), dtype=torch.bfloat16, device=device)
+    scratch = torch.zeros((t, F), dtype=torch.bfloat16, device=device)
+
+    def step():
+        for l in range(L):
+            mlp.encode(x, sets[l][0], sets[l][1], sets[l][2], y[l], scratch, t=t)
+
+    # parity of set 0 against the CPU checker
+    import numpy as np
+    from oracle import mf_oracle as O
+    def hq(q):
+        return O.QTensor(q.packed.cpu().numpy(), ops.bf16_bits(q.scales), ops.bf16_bits(q.biases), 4, q.rows, q.n)
+    step()
+    torch.cuda.synchronize()
+    ref = np.stack([O.shared_expert(hq(sets[0][0]), hq(sets[0][1]), hq(sets[0][2]), ops.bf16_bits(x[i]))
+                    for i in range(t)])
+    got = O.bf16_to_float(ops.bf16_bits(y[0])).astype(np.float64)
+    reff = O.bf16_to_float(ref).astype(np.float64)
+    parity = dict(max_abs=float(np.abs(got - reff).max()),
+                  rel_l2=float(np.linalg.norm(got - reff) / np.linalg.norm(reff)))
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        step()
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        step()
+    for _ in range(args.warmup):
+        graph.replay()
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    for _ in range(args.steps):
+        graph.replay()
+    e1.record()
+    torch.cuda.synchronize()
+    us = e0.elapsed_time(e1) / args.steps / L * 1e3
+    nbytes = 3 * (D * F // 2 + 2 * 2 * (D * F // 64))
+    achieved = nbytes / (us * 1e-6) / 1e9
+    print(json.dumps({
+        "metric": "us_per_dense_mlp_T%d" % t, "value": round(us, 3), "unit": "us", "n_gpus": 1,
+        "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(us * L / 1e3, 5),
+        "higher_is_better": False, "scaling": "weak", "vs_baseline": None,
+        "dtype": "u4 codes x bf16 activations, fp32 accumulate", "data": "synthetic (N(0,0.02) weights, 4-bit g64)",
+        "config": {"workload": w["name"] + "-T%d" % t, "weight_sets": L, "tokens": t, "launch": "hip_graph"},
+        "parity_set0": parity,
+        "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+                     "frac": round(achieved / HBM_PEAK_GBPS, 4), "traffic": None,
+                     "kernel": "mf::gate_up_act_kernel + mf::gemv_kernel", "algorithmic_bytes": nbytes}}))
+    return 0
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
-    ap.add_argument("--layers", type=int, default=40)
+    ap.add_argument("--layers", type=int, default=None)
+    ap.add_argument("--workload", default="qwen-decode",
+                    choices=sorted(WORKLOADS) + ["dense-mlp"],
+                    help="qwen-decode is the headline; the others measure the remaining "
+                         "configurations of the same path")
+    ap.add_argument("--tokens", type=int, default=None, help="token rows per step (decode: 1..8)")
     ap.add_argument("--no-graph", action="store_true", help="launch eagerly instead of a HIP graph")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--pmc-calibration", action="store_true",
@@ -209,8 +323,15 @@ def main() -> int:
     assert torch.cuda.is_available(), "bench.py needs a GPU"
     device = torch.device("cuda", 0)
     torch.cuda.set_device(device)
-    w = QWEN
-    L, K, W = args.layers, args.steps, args.warmup
+    if args.workload == "dense-mlp":
+        return bench_dense_mlp(args, device)
+    w = dict(WORKLOADS[args.workload])
+    if args.tokens:
+        w["t"] = args.tokens
+        w["name"] += f"-T{args.tokens}"
+    if args.workload != "qwen-decode":
+        args.no_prefill = True
+    L, K, W = args.layers or w.get("layers", 40), args.steps, args.warmup
     if args.prefill_only:
         L = 1
     ctx = ops.MetalContext(0)
@@ -219,7 +340,9 @@ def main() -> int:
         print(json.dumps({"prefill": measure_prefill(ctx, w, stack[0], device)}))
         return 0
     moes = [ops.MoE(ctx, w["d"], w["f"], w["e"], w["k"], bits=w["bits"], shared_f=w["fs"],
-                    shared_bits=w["shared_bits"]) for _ in range(L)]
+                    shared_bits=w["shared_bits"],
+                    router_mode=ops.ROUTER_FULL_SOFTMAX if w["bits"] == 1 else ops.ROUTER_TOPK_SOFTMAX)
+            for _ in range(L)]
 
     gen = torch.Generator(device=device)
     gen.manual_seed(ROOT_SEED + 0x100 * w["config"] + 0xFF)
@@ -236,6 +359,7 @@ def main() -> int:
     # ---- parity of layer 0 at full size against the CPU checker
     from oracle import mf_oracle as O
     host0 = layer_to_host(stack[0], w)
+    host0.router_mode = 1 if w["bits"] == 1 else 0
     ref_y, ref_idx, ref_w = O.moe_layer(host0, ops.bf16_bits(x0))
     yy = torch.zeros_like(x0)
     idx = torch.zeros((w["t"], w["k"]), dtype=torch.int32, device=device)
@@ -286,10 +410,12 @@ def main() -> int:
         m.status()
     finite = bool(torch.isfinite(ys.float()).all().item())
 
+    if w["t"] > 1:  # several tokens share experts: count the union layer 0 selected
+        w["experts_touched"] = int(np.unique(ref_idx).size)
     ab = algorithmic_bytes(w)
     achieved = ab["expert_bytes"] / (us_per_layer * 1e-6) / 1e9
     out = {
-        "metric": "us_per_moe_layer_decode_T1",
+        "metric": "us_per_moe_layer_decode_T%d" % w["t"],
         "value": round(us_per_layer, 4),
         "unit": "us",
         "n_gpus": 1, "steps": K, "warmup": W,
@@ -297,8 +423,9 @@ def main() -> int:
         "higher_is_better": False,
         "scaling": "weak",
         "vs_baseline": None,
-        "dtype": "u4 codes x bf16 activations, fp32 accumulate",
-        "data": "synthetic (random-init N(0,0.02) weights quantized 4-bit g64 on device; x ~ N(0,1))",
+        "dtype": "%s codes x bf16 activations, fp32 accumulate" % {4: "u4", 2: "u2", 1: "ternary"}[w["bits"]],
+        "data": "synthetic (random-init weights quantized g64 on device: N(0,0.02) affine, or ternary "
+                "codes p=.25/.5/.25 with |N(0,0.02)| scales; x ~ N(0,1))",
         "config": {"workload": w["name"], "layers": L, "tokens": w["t"], "hidden": w["d"],
                    "experts": w["e"], "top_k": w["k"], "moe_intermediate": w["f"],
                    "shared_intermediate": w["fs"], "launch": "hip_graph" if use_graph else "eager"},
@@ -310,7 +437,7 @@ def main() -> int:
         "parity_layer0": parity,
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS,
                      "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBPS, 4),
-                     "traffic": profiled_traffic_bytes(),
+                     "traffic": profiled_traffic_bytes() if args.workload == "qwen-decode" else None,
                      "kernel": "mf::fused_decode_kernel (one launch per layer)",
                      "algorithmic_bytes_per_layer": ab["expert_bytes"]},
     }

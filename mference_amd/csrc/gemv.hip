@@ -117,6 +117,168 @@ __global__ __launch_bounds__(256) void gate_up_act_kernel(
   }
 }
 
+// Streaming form of the two kernels above for wide matrices: a wave keeps its
+// slices of x (already permuted, with their sums) in registers for the whole
+// launch and walks down the rows, so the only traffic per row is the codes and
+// the scale/bias entries.  The next row's loads are issued before the current
+// row's arithmetic.  ITS (compile time) bounds the 16-byte steps a lane takes
+// along a row; wpr waves (1, 2 or 4) split a row when it is longer than one
+// wave can hold in registers, and their partial sums meet in LDS in wave order.
+// NPROJ 2 is the gate/up pair with the shared-expert activation
+// (dequant_int4.metal:216-246); NPROJ 1 is the plain GEMV.
+struct RowsArgs {
+  const uint8_t* W[2];
+  const uint16_t* S[2];
+  const uint16_t* B[2];
+  const uint16_t* x;   // [T, N]
+  void* y;             // NPROJ 1: [T, M] bf16 or fp32; NPROJ 2: act [T, M] bf16
+  uint32_t M, N;
+  uint32_t wpr;        // waves per row
+  int out_f32;
+};
+
+template <int BITS, int T, int ITS, int NPROJ>
+__global__ __launch_bounds__(256) void rows_stream_kernel(const RowsArgs a) {
+  constexpr int EPL = Fmt<BITS>::kElemsPer16B;
+  __shared__ float s_part[4][T][NPROJ];
+  const uint32_t lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
+  const uint32_t wpr = a.wpr, slot = wv / wpr, part = wv % wpr, rows_per_wg = 4 / wpr;
+  const uint32_t n_groups = a.N / kGroup;
+  const size_t row_bytes = static_cast<size_t>(a.N) * Store<BITS>::kBits / 8;
+
+  // the lane's columns: step it covers elements [(it * wpr + part) * 64 + lane] * EPL ...
+  uint32_t e0[ITS];
+  bool live[ITS];
+  XSlice<BITS> xs[T][ITS];
+#pragma unroll
+  for (int it = 0; it < ITS; ++it) {
+    e0[it] = ((it * wpr + part) * 64 + lane) * EPL;
+    live[it] = e0[it] < a.N;
+    if (!live[it]) e0[it] = 0;
+#pragma unroll
+    for (int t = 0; t < T; ++t) {
+      xs[t][it] = load_xslice<BITS, kXAligned>(a.x + static_cast<size_t>(t) * a.N + e0[it]);
+      if (!live[it]) {
+#pragma unroll
+        for (int i = 0; i < XSlice<BITS>::kPairs; ++i) xs[t][it].p[i] = 0;
+        xs[t][it].sum = 0.0f;
+      }
+    }
+  }
+
+  // The scale / bias entries of one row: this wave's steps meet GPS = 64 * EPL / 64 groups
+  // each; one load per table brings them in (lane l holds entry l of step-major order, the
+  // wave's steps being wpr * GPS apart in the row), a cross-lane read hands each lane its own.
+  constexpr int GPS = EPL;                         // groups per wave step
+  constexpr int TW = (ITS * GPS + 63) / 64;        // table words per lane
+  uint32_t tab_g[TW];                              // group index this lane fetches
+  bool tab_ok[TW];
+#pragma unroll
+  for (int k = 0; k < TW; ++k) {
+    const uint32_t j = k * 64 + lane, it = j / GPS;
+    tab_g[k] = (it * wpr + part) * GPS + j % GPS;
+    tab_ok[k] = it < static_cast<uint32_t>(ITS) && tab_g[k] < n_groups;
+    if (!tab_ok[k]) tab_g[k] = 0;
+  }
+  int tab_src[ITS];                                // lane holding this lane's entry of step it,
+#pragma unroll                                     // in table word (it * GPS) / 64
+  for (int it = 0; it < ITS; ++it) tab_src[it] = static_cast<int>((it * GPS + lane * EPL / kGroup) & 63u) << 2;
+  uint4 codes[NPROJ][ITS];
+  uint32_t sraw[NPROJ][TW], braw[NPROJ][TW];
+  auto fetch = [&](uint32_t row) {
+    const size_t r = row < a.M ? row : a.M - 1;
+#pragma unroll
+    for (int p = 0; p < NPROJ; ++p) {
+#pragma unroll
+      for (int it = 0; it < ITS; ++it)
+        codes[p][it] = *reinterpret_cast<const uint4*>(a.W[p] + r * row_bytes +
+                                                       static_cast<size_t>(e0[it]) * Store<BITS>::kBits / 8);
+#pragma unroll
+      for (int k = 0; k < TW; ++k) {
+        sraw[p][k] = a.S[p][r * n_groups + tab_g[k]];
+        if constexpr (BITS != kBitsTernary) braw[p][k] = a.B[p][r * n_groups + tab_g[k]];
+      }
+    }
+  };
+
+  uint32_t row = blockIdx.x * rows_per_wg + slot;
+  const uint32_t stride = gridDim.x * rows_per_wg;
+  const uint32_t row_end = (a.M + stride - 1) / stride * stride;  // every wave runs the same trip count
+  fetch(row);
+  for (; row < row_end; row += stride) {
+    uint4 cur[NPROJ][ITS];
+    float sc[NPROJ][ITS], bi[NPROJ][ITS];
+#pragma unroll
+    for (int p = 0; p < NPROJ; ++p)
+#pragma unroll
+      for (int it = 0; it < ITS; ++it) {
+        cur[p][it] = codes[p][it];
+        uint32_t sv = 0, bv = 0;
+        sv = static_cast<uint32_t>(__builtin_amdgcn_ds_bpermute(tab_src[it], static_cast<int>(sraw[p][(it * GPS) / 64])));
+        if constexpr (BITS != kBitsTernary)
+          bv = static_cast<uint32_t>(__builtin_amdgcn_ds_bpermute(tab_src[it], static_cast<int>(braw[p][(it * GPS) / 64])));
+        sc[p][it] = __uint_as_float(sv << 16);
+        if constexpr (BITS == kBitsTernary) bi[p][it] = -sc[p][it];
+        else bi[p][it] = __uint_as_float(bv << 16);
+      }
+    if (row + stride < row_end) fetch(row + stride);
+
+    float acc[T][NPROJ];
+#pragma unroll
+    for (int t = 0; t < T; ++t)
+#pragma unroll
+      for (int p = 0; p < NPROJ; ++p) acc[t][p] = 0.0f;
+#pragma unroll
+    for (int it = 0; it < ITS; ++it)
+#pragma unroll
+      for (int p = 0; p < NPROJ; ++p)
+#pragma unroll
+        for (int t = 0; t < T; ++t) {
+          const float dot = codes_dot<BITS>(cur[p][it], xs[t][it]);
+          acc[t][p] = __builtin_fmaf(sc[p][it], dot, acc[t][p]);
+          acc[t][p] = __builtin_fmaf(bi[p][it], xs[t][it].sum, acc[t][p]);
+        }
+#pragma unroll
+    for (int t = 0; t < T; ++t)
+#pragma unroll
+      for (int p = 0; p < NPROJ; ++p) acc[t][p] = wave_sum(acc[t][p]);
+    if (wpr > 1) {
+      if (lane == 0) {
+#pragma unroll
+        for (int t = 0; t < T; ++t)
+#pragma unroll
+          for (int p = 0; p < NPROJ; ++p) s_part[wv][t][p] = acc[t][p];
+      }
+      __syncthreads();
+      if (part == 0) {
+#pragma unroll
+        for (int t = 0; t < T; ++t)
+#pragma unroll
+          for (int p = 0; p < NPROJ; ++p) {
+            float v = s_part[wv][t][p];
+            for (uint32_t q = 1; q < wpr; ++q) v = v + s_part[wv + q][t][p];
+            acc[t][p] = v;
+          }
+      }
+      __syncthreads();
+    }
+    if (part == 0 && lane == 0 && row < a.M) {
+#pragma unroll
+      for (int t = 0; t < T; ++t) {
+        const size_t at = static_cast<size_t>(t) * a.M + row;
+        if constexpr (NPROJ == 2) {
+          const float rg = round_bf16(acc[t][0]), ru = round_bf16(acc[t][1]);
+          static_cast<uint16_t*>(a.y)[at] = f_to_bf16(mf_silu(rg) * ru);
+        } else if (a.out_f32) {
+          static_cast<float*>(a.y)[at] = acc[t][0];
+        } else {
+          static_cast<uint16_t*>(a.y)[at] = f_to_bf16(acc[t][0]);
+        }
+      }
+    }
+  }
+}
+
 // silu_mul_fp16 (utility.metal:21-33)
 __global__ void silu_mul_kernel(const uint16_t* gate, const uint16_t* up, uint16_t* out,
                                 uint32_t count) {
@@ -191,11 +353,64 @@ hipError_t gate_up_dispatch_t(hipStream_t s, const mf_qtensor& g, const mf_qtens
   return hipGetLastError();
 }
 
+// Picks the streaming kernel when the shape fits one of its instantiations:
+// 16-byte aligned operands, N a multiple of the group, T in {1, 2, 4}, and a
+// (wpr, ITS) split with T * ITS x-slices small enough to stay in registers.
+uint32_t device_cu_count() {
+  static int cached[64] = {0};
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return 256;
+  if (!cached[dev]) {
+    int n = 0;
+    if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) n = 256;
+    cached[dev] = n;
+  }
+  return static_cast<uint32_t>(cached[dev]);
+}
+
+template <int BITS, int NPROJ>
+bool rows_stream_try(hipStream_t s, const RowsArgs& in, uint32_t t, uint32_t num_cu, hipError_t& err) {
+  constexpr int EPL = Fmt<BITS>::kElemsPer16B;
+  if (in.N % kGroup || in.N < 64 * EPL || (t != 1 && t != 2 && t != 4) || in.M < 1024) return false;
+  const uint32_t steps = (in.N + 64 * EPL - 1) / (64 * EPL);  // 16-byte steps of one wave along a row
+  const uint32_t max_its = t == 1 ? 9 : 3;
+  if (BITS == kBitsTernary) return false;
+  uint32_t wpr = 1;
+  while (wpr < 4 && (steps + wpr - 1) / wpr > max_its) wpr *= 2;
+  // few rows and long rows: split the rows so that every wave still walks a useful number of them
+  while (wpr < 4 && in.M / wpr < num_cu * 8 * 4 && (steps + wpr - 1) / wpr > 2) wpr *= 2;
+  const uint32_t its = (steps + wpr - 1) / wpr;
+  if (its > max_its) return false;
+  RowsArgs a = in;
+  a.wpr = wpr;
+  const uint32_t rows_per_wg = 4 / wpr;
+  const uint32_t grid = std::min<uint32_t>((a.M + rows_per_wg - 1) / rows_per_wg, num_cu * 2);
+#define MF_ROWS(TT, II)                                                                      \
+  rows_stream_kernel<BITS, TT, II, NPROJ><<<dim3(grid), dim3(256), 0, s>>>(a)
+  if constexpr (BITS != kBitsTernary) {
+    if (t == 1) { if (its == 1) MF_ROWS(1, 1); else if (its <= 3) MF_ROWS(1, 3); else MF_ROWS(1, 9); }
+    else if (t == 2) { if (its == 1) MF_ROWS(2, 1); else MF_ROWS(2, 3); }
+    else { if (its == 1) MF_ROWS(4, 1); else MF_ROWS(4, 3); }
+  }
+#undef MF_ROWS
+  err = hipGetLastError();
+  return true;
+}
+
 }  // namespace
 
 hipError_t launch_gemv(hipStream_t s, const mf_qtensor& w, int bits, const uint16_t* x, void* y,
                        uint32_t m, uint32_t n, uint32_t t, bool out_f32) {
   const bool al = aligned16(w.weights) && aligned16(x);
+  if (al && (bits == kBits4 || bits == kBits2)) {
+    RowsArgs a{};
+    a.W[0] = static_cast<const uint8_t*>(w.weights); a.S[0] = w.scales; a.B[0] = w.biases;
+    a.x = x; a.y = y; a.M = m; a.N = n; a.out_f32 = out_f32 ? 1 : 0;
+    hipError_t err = hipSuccess;
+    if (bits == kBits4 ? rows_stream_try<kBits4, 1>(s, a, t, device_cu_count(), err)
+                       : rows_stream_try<kBits2, 1>(s, a, t, device_cu_count(), err))
+      return err;
+  }
   switch (bits) {
     case kBits4:
       return al ? gemv_dispatch_t<kBits4, true>(s, w, x, y, m, n, t, out_f32)
@@ -214,6 +429,16 @@ hipError_t launch_gate_up_act(hipStream_t s, const mf_qtensor& gate, const mf_qt
                               int bits, const uint16_t* x, uint16_t* act, uint32_t f, uint32_t d,
                               uint32_t t) {
   const bool al = aligned16(gate.weights) && aligned16(up.weights) && aligned16(x);
+  if (al && (bits == kBits4 || bits == kBits2)) {
+    RowsArgs a{};
+    a.W[0] = static_cast<const uint8_t*>(gate.weights); a.S[0] = gate.scales; a.B[0] = gate.biases;
+    a.W[1] = static_cast<const uint8_t*>(up.weights); a.S[1] = up.scales; a.B[1] = up.biases;
+    a.x = x; a.y = act; a.M = f; a.N = d;
+    hipError_t err = hipSuccess;
+    if (bits == kBits4 ? rows_stream_try<kBits4, 2>(s, a, t, device_cu_count(), err)
+                       : rows_stream_try<kBits2, 2>(s, a, t, device_cu_count(), err))
+      return err;
+  }
   switch (bits) {
     case kBits4:
       return al ? gate_up_dispatch_t<kBits4, true>(s, gate, up, x, act, f, d, t)

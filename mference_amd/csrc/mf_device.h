@@ -220,9 +220,10 @@ __device__ __forceinline__ uint4 load_x8(const uint16_t* p) {
 // One lane's share of a row is 16 bytes of codes: 32 four-bit elements (half a
 // quantization group) or 64 two-bit elements (one group).  The dot product
 // sum(q*x) runs on v_dot2c_f32_bf16: two codes are masked out of the packed
-// word straight into the mantissas of a bf16 pair (0x4300 | q = 128 + q,
-// exact), multiplied with a matching bf16 pair of x and accumulated in fp32;
-// the 128 * sum(x) this adds is taken off once per lane share.  Codes are
+// word straight into the mantissas of a bf16 pair (0x4100 | q << 3 = 8 + q/2
+// for 4-bit codes, 0x4080 | q << 5 = 4 + q for 2-bit codes, both exact),
+// multiplied with a matching bf16 pair of x and accumulated in fp32; the
+// offset * sum(x) this adds is taken off once per lane share.  Codes are
 // paired (j, j + 4) for 4-bit and (j, j + 8) for 2-bit because those pairs sit
 // 16 bits apart in the packed word; the x slice is permuted once to match and
 // reused for every row that meets it (gate and up, several tokens' rows).
@@ -235,7 +236,21 @@ __device__ __forceinline__ float dot2_bf16(uint32_t a, uint32_t b, float acc) {
 }
 
 constexpr uint32_t kMagic128 = 0x43004300u;  // bf16 pair (128.0, 128.0)
+// A masked code lands in the mantissa of a bf16 whose exponent is the smallest that leaves
+// room for it: 4-bit codes in mantissa bits 3..6 under 2^3 (the number 8 + q/2), 2-bit codes
+// in bits 5..6 under 2^2 (4 + q).  The dot product then carries offset * sum(x), removed in
+// fp32 afterwards; the smaller the offset, the less of the fp32 mantissa that cancellation eats.
+constexpr uint32_t kMagic8 = 0x41004100u;    // bf16 pair (8.0, 8.0)
+constexpr uint32_t kMagic4 = 0x40804080u;    // bf16 pair (4.0, 4.0)
 constexpr uint32_t kOnes = 0x3F803F80u;      // bf16 pair (1.0, 1.0)
+
+// (v & mask) | magic in one instruction; the mask rides in a scalar register, the magic in a
+// vector register (a VOP3 instruction of this ISA takes one scalar source and no literal)
+__device__ __forceinline__ uint32_t and_or(uint32_t v, uint32_t mask, uint32_t magic) {
+  uint32_t r;
+  asm("v_and_or_b32 %0, %1, %2, %3" : "=v"(r) : "v"(v), "s"(mask), "v"(magic));
+  return r;
+}
 
 // The activations one lane meets, permuted for the pairing above, plus their sum.
 template <int BITS> struct XSlice {
@@ -314,21 +329,25 @@ __device__ __forceinline__ float codes_dot(const uint4& codes, const XSlice<BITS
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
       const uint32_t w = ws[j];
-      dot = dot2_bf16((w & 0x000F000Fu) | kMagic128, xs.p[4 * j + 0], dot);
-      dot = dot2_bf16(((w >> 4) & 0x000F000Fu) | kMagic128, xs.p[4 * j + 1], dot);
-      dot = dot2_bf16(((w >> 8) & 0x000F000Fu) | kMagic128, xs.p[4 * j + 2], dot);
-      dot = dot2_bf16(((w >> 12) & 0x000F000Fu) | kMagic128, xs.p[4 * j + 3], dot);
+      dot = dot2_bf16(and_or(w << 3, 0x00780078u, kMagic8), xs.p[4 * j + 0], dot);
+      dot = dot2_bf16(and_or(w >> 1, 0x00780078u, kMagic8), xs.p[4 * j + 1], dot);
+      dot = dot2_bf16(and_or(w >> 5, 0x00780078u, kMagic8), xs.p[4 * j + 2], dot);
+      dot = dot2_bf16(and_or(w >> 9, 0x00780078u, kMagic8), xs.p[4 * j + 3], dot);
     }
+    return 2.0f * __builtin_fmaf(-8.0f, xs.sum, dot);  // sum((8 + q/2) x) -> sum(q x)
   } else {
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
       const uint32_t w = ws[j];
+      dot = dot2_bf16(and_or(w << 5, 0x00600060u, kMagic4), xs.p[8 * j + 0], dot);
+      dot = dot2_bf16(and_or(w << 3, 0x00600060u, kMagic4), xs.p[8 * j + 1], dot);
+      dot = dot2_bf16(and_or(w << 1, 0x00600060u, kMagic4), xs.p[8 * j + 2], dot);
 #pragma unroll
-      for (int i = 0; i < 8; ++i)
-        dot = dot2_bf16(((w >> (2 * i)) & 0x00030003u) | kMagic128, xs.p[8 * j + i], dot);
+      for (int i = 3; i < 8; ++i)
+        dot = dot2_bf16(and_or(w >> (2 * i - 5), 0x00600060u, kMagic4), xs.p[8 * j + i], dot);
     }
+    return __builtin_fmaf(-4.0f, xs.sum, dot);  // sum((4 + q) x) -> sum(q x)
   }
-  return __builtin_fmaf(-128.0f, xs.sum, dot);
 }
 
 // convenience form: one row against a slice loaded on the spot

@@ -437,18 +437,10 @@ __device__ __forceinline__ float fast_silu(float x) {
   return x * __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(x * -1.4426950408889634f));
 }
 
-// (v & mask) | magic in one instruction; the mask rides in a scalar register
-__device__ __forceinline__ uint32_t and_or(uint32_t v, uint32_t mask, uint32_t magic) {
-  uint32_t r;
-  asm("v_and_or_b32 %0, %1, %2, %3" : "=v"(r) : "v"(v), "s"(mask), "v"(magic));
-  return r;
-}
-
 // one packed word of 4-bit codes -> MFMA operand: pairs (q0,q4),(q1,q5),(q2,q6),(q3,q7) as the
 // bf16 numbers 8 + q/2 (exponent 2^3, the code in mantissa bits 3..6).  16 is the smallest offset
 // a mask-and-or can give a 4-bit code, and the offset matters: the matrix core accumulates
 // offset * sum(x) alongside the signal and the correction term takes it out again in fp32.
-constexpr uint32_t kMagic8 = 0x41004100u;
 __device__ __forceinline__ uint4 expand_q4(uint32_t w) {
   return make_uint4(and_or(w << 3, 0x00780078u, kMagic8), and_or(w >> 1, 0x00780078u, kMagic8),
                     and_or(w >> 5, 0x00780078u, kMagic8), and_or(w >> 9, 0x00780078u, kMagic8));
@@ -681,6 +673,8 @@ void qmm_kernel(const QmmArgs a) {
       const uint32_t g = g0 + u;
       if (g >= ng) break;
       __syncthreads();  // buffer g & 1 is complete, buffer (g + 1) & 1 is no longer read
+      if (g == 9) qmm_trace(a, work, 5);
+      if (g == 10) qmm_trace(a, work, 7);
       // ---- x of group g + 1 into the other buffer, fetch group g + 3 into the freed registers
       if (g + 1 < ng) {
         uint4* wbuf = s_x + ((u + 1) & 1) * 512;
@@ -728,6 +722,7 @@ void qmm_kernel(const QmmArgs a) {
 #pragma unroll
           for (int r = 0; r < 16; ++r) acc[p][nt][r] = __builtin_fmaf(sc, tmp[nt][r], acc[p][nt][r]);
       }
+      if (g == 9) qmm_trace(a, work, 6);
     }
 #pragma unroll
     for (int p = 0; p < NPROJ; ++p)

@@ -149,6 +149,17 @@ def profiled_traffic_bytes():
         return None
 
 
+def pmc_calibration(device) -> str:
+    """a kernel of known HBM traffic, so that FETCH_SIZE / WRITE_SIZE readings can be scaled"""
+    import torch
+    src = torch.zeros(256 << 20, dtype=torch.uint8, device=device)
+    dst = torch.empty_like(src)
+    for _ in range(3):
+        dst.copy_(src)
+    torch.cuda.synchronize()
+    return "3 x 256 MiB device-to-device copy (reads 268435456 B, writes 268435456 B)"
+
+
 def measure_prefill(ctx, w, layer, device, tokens=(128, 512, 2048), steps=100, warmup=100):
     """Ragged prefill of one layer of the same shape: T tokens, top-k routing from skewed
     logits (router weights plus a per-expert bias ~ N(0, 1.5), carried by a constant-one last
@@ -337,7 +348,12 @@ def main() -> int:
     ctx = ops.MetalContext(0)
     stack = build_stack(ctx, w, L, device)
     if args.prefill_only:
-        print(json.dumps({"prefill": measure_prefill(ctx, w, stack[0], device)}))
+        tokens = (args.tokens,) if args.tokens else (128, 512, 2048)
+        res = {"prefill": measure_prefill(ctx, w, stack[0], device, tokens=tokens,
+                                          steps=min(args.steps, 100), warmup=min(args.warmup, 100))}
+        if args.pmc_calibration:
+            res["pmc_calibration"] = pmc_calibration(device)
+        print(json.dumps(res))
         return 0
     moes = [ops.MoE(ctx, w["d"], w["f"], w["e"], w["k"], bits=w["bits"], shared_f=w["fs"],
                     shared_bits=w["shared_bits"],
@@ -463,12 +479,7 @@ def main() -> int:
                                "sample": f"{n} repetitions of layer 0 of the same workload "
                                          f"(OpenMP over weight rows, {cores} threads)"}
     if args.pmc_calibration:
-        src = torch.zeros(256 << 20, dtype=torch.uint8, device=device)
-        dst = torch.empty_like(src)
-        for _ in range(3):
-            dst.copy_(src)
-        torch.cuda.synchronize()
-        out["pmc_calibration"] = "3 x 256 MiB device-to-device copy (reads 268435456 B, writes 268435456 B)"
+        out["pmc_calibration"] = pmc_calibration(device)
     print(json.dumps(out))
     return 0
 

@@ -261,7 +261,9 @@ __device__ __forceinline__ void topk_rank_block(const float* lg, uint32_t e, uin
 // a round without a winner gives index 0, score -inf.  Rank r's result lives in
 // lane r; weights are exp(s_r - s_0) / sum with the sum taken in rank order.
 // All 64 lanes call it.
-template <int PER>
+// MODE 1: lg holds probabilities of the full softmax; the weights are p_r / (sum + 1e-20)
+// with the sum in rank order (maple_moe.metal:100-118).
+template <int PER, int MODE = 0>
 __device__ __forceinline__ void topk_select_sorted(const float* lg, uint32_t e, uint32_t k,
                                                    uint32_t* idx, float* w, uint32_t lane) {
   const float ninf = -__builtin_inff();
@@ -313,6 +315,17 @@ __device__ __forceinline__ void topk_select_sorted(const float* lg, uint32_t e, 
       my_idx = widx;
     }
   }
+  if constexpr (MODE == 1) {
+    float sum = 0.0f;
+#pragma unroll
+    for (int i = 0; i < MF_MAX_TOPK; ++i)
+      if (static_cast<uint32_t>(i) < k) sum += readlane_f(my_score, i);
+    if (lane < k) {
+      idx[lane] = my_idx;
+      w[lane] = my_score / (sum + 1.0e-20f);
+    }
+    return;
+  }
   const float s0 = readlane_f(my_score, 0);
   const float my_e = mf_exp(my_score - s0);
   float sum = 0.0f;
@@ -323,6 +336,74 @@ __device__ __forceinline__ void topk_select_sorted(const float* lg, uint32_t e, 
     idx[lane] = my_idx;
     w[lane] = my_e / sum;
   }
+}
+
+// Full softmax over e logits in the reference's order (maple_moe.metal:62-99): maximum, then
+// exp(l - max) summed as 32-wide blocks, each block by a 16,8,4,2,1 tree, the blocks added in
+// order, + 1e-20; p written to `p` (may alias lg).  Returns false (nothing written) when a
+// logit is not finite.  All 64 lanes call it; lg and p are read and written by this wave only.
+__device__ __forceinline__ bool full_softmax_probs(const float* lg, float* p, uint32_t e,
+                                                   uint32_t lane) {
+  const uint32_t per = (e + kWave - 1) / kWave;
+  float ch[kMaxPerLane];
+  bool bad = false;
+  float mx = -1.0e30f;
+#pragma unroll
+  for (int j = 0; j < kMaxPerLane; ++j) {
+    const uint32_t x = lane + j * kWave;
+    ch[j] = 0.0f;
+    if (static_cast<uint32_t>(j) < per && x < e) {
+      ch[j] = lg[x];
+      if (!__builtin_isfinite(ch[j])) bad = true;
+      if (ch[j] > mx) mx = ch[j];
+    }
+  }
+  if (__any(bad)) return false;
+  mx = wave_max(mx);
+  float total = 0.0f;
+#pragma unroll
+  for (int j = 0; j < kMaxPerLane; ++j) {
+    if (static_cast<uint32_t>(j) < per) {  // uniform: rows past the last expert cost nothing
+      const uint32_t x = lane + j * kWave;
+      const bool live = x < e;
+      ch[j] = live ? mf_exp(ch[j] - mx) : 0.0f;
+      float part = ch[j];
+#pragma unroll
+      for (int o = 16; o > 0; o >>= 1) part = part + __shfl_xor(part, o, kWave);
+      const float lo = readlane_f(part, 0), hi = readlane_f(part, 32);
+      if (static_cast<uint32_t>(2 * j) < e / 32) total += lo;
+      if (static_cast<uint32_t>(2 * j + 1) < e / 32) total += hi;
+    }
+  }
+  const float recip = 1.0f / (total + 1.0e-20f);
+#pragma unroll
+  for (int j = 0; j < kMaxPerLane; ++j) {
+    const uint32_t x = lane + j * kWave;
+    if (static_cast<uint32_t>(j) < per && x < e) p[x] = ch[j] * recip;
+  }
+  return true;
+}
+
+// mode 1 selector: full softmax, then k rounds of arg-max on the probabilities (strictly
+// greater wins, so equal probabilities keep the lower index), renormalised.  `p` is scratch
+// of e floats owned by this wave (LDS).  A non-finite logit gives indices = e, weights = 0.
+__device__ __forceinline__ void topk_full_softmax_fast(const float* lg, float* p, uint32_t e,
+                                                       uint32_t k, uint32_t* idx, float* w,
+                                                       uint32_t lane) {
+  if (!full_softmax_probs(lg, p, e, lane)) {
+    if (lane < k) {
+      idx[lane] = e;
+      w[lane] = 0.0f;
+    }
+    return;
+  }
+  __builtin_amdgcn_s_waitcnt(0xc07f);  // lgkmcnt(0): p is re-read by other lanes of this wave
+  __builtin_amdgcn_wave_barrier();
+  const uint32_t per = (e + kWave - 1) / kWave;
+  if (per <= 1) topk_select_sorted<1, 1>(p, e, k, idx, w, lane);
+  else if (per <= 2) topk_select_sorted<2, 1>(p, e, k, idx, w, lane);
+  else if (per <= 4) topk_select_sorted<4, 1>(p, e, k, idx, w, lane);
+  else topk_select_sorted<8, 1>(p, e, k, idx, w, lane);
 }
 
 __device__ __forceinline__ void topk_select_fast(const float* lg, uint32_t e, uint32_t k,

@@ -264,8 +264,9 @@ __global__ __launch_bounds__(kFusedThreads) void fused_decode_kernel(const Fused
                           (lane == 0 ? static_cast<uint32_t>(f_to_bf16(v)) : 0u) | (tag16 << 16));
       } else {
         const uint32_t it = item - n_router - n_gate;
-        const uint32_t tok = it / srg;
-        const uint32_t row = (it % srg) * rpw + (lane >> lpr_log2);
+        const uint32_t srg1 = srg ? srg : 1u;  // no shared expert: this branch is never taken
+        const uint32_t tok = it / srg1;
+        const uint32_t row = (it % srg1) * rpw + (lane >> lpr_log2);
         const uint32_t sub = lane & (lpr - 1);
         const bool ok = row < Fs;
         const size_t r = ok ? row : 0;
@@ -308,7 +309,7 @@ __global__ __launch_bounds__(kFusedThreads) void fused_decode_kernel(const Fused
   trace_mark(a, 2);
   if (wv < T) {
     if (a.router_mode == 0) topk_select_fast(s_lg + wv * E, E, K, s_idx + wv * K, s_w + wv * K, lane);
-    else topk_wave(s_lg + wv * E, E, K, a.router_mode, s_idx + wv * K, s_w + wv * K, lane);
+    else topk_full_softmax_fast(s_lg + wv * E, s_lg + wv * E, E, K, s_idx + wv * K, s_w + wv * K, lane);
   }
   __syncthreads();
   if (wg == 0 && threadIdx.x < T * K) {
@@ -603,7 +604,20 @@ hipError_t launch_fused_decode(hipStream_t s, const mf_moe& h, const mf_moe_laye
   const bool qwen_t1 = c.bits == MF_BITS_4 && c.shared_bits == MF_BITS_4 && c.d == 2048 &&
                        c.f == 512 && c.num_experts == 256 && c.top_k == 8 && c.shared_f == 512 &&
                        t == 1 && c.router_mode == MF_ROUTER_TOPK_SOFTMAX;
+  // the large 2-bit layer (hidden 4096, 256 experts of 2048, top-6, 4-bit shared expert of 2048)
+  using Big2T1 = StaticShape<4096, 2048, 256, 6, 1, 2048>;
+  using Big2T4 = StaticShape<4096, 2048, 256, 6, 4, 2048>;
+  const bool big2 = c.bits == MF_BITS_2 && c.shared_bits == MF_BITS_4 && c.d == 4096 && c.f == 2048 &&
+                    c.num_experts == 256 && c.top_k == 6 && c.shared_f == 2048 &&
+                    c.router_mode == MF_ROUTER_TOPK_SOFTMAX;
+  // the ternary layer (hidden 2048, 64 experts of 1024, top-8, no shared expert)
+  using TernT1 = StaticShape<2048, 1024, 64, 8, 1, 0>;
+  const bool tern_t1 = c.bits == MF_BITS_TERNARY && c.d == 2048 && c.f == 1024 && c.num_experts == 64 &&
+                       c.top_k == 8 && c.shared_f == 0 && t == 1;
   if (qwen_t1) MF_FUSED(kBits4, kBits4, QwenT1);
+  else if (big2 && t == 1) MF_FUSED(kBits2, kBits4, Big2T1);
+  else if (big2 && t == 4) MF_FUSED(kBits2, kBits4, Big2T4);
+  else if (tern_t1) MF_FUSED(kBitsTernary, kBits4, TernT1);
   else if (c.bits == MF_BITS_4) MF_FUSED(kBits4, kBits4, RuntimeShape);
   else if (c.bits == MF_BITS_2 && c.shared_f && c.shared_bits == MF_BITS_2)
     MF_FUSED(kBits2, kBits2, RuntimeShape);

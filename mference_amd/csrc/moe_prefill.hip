@@ -119,7 +119,9 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
   __shared__ float s_part[3][16 * 64];
   const uint32_t lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
   const uint32_t m = lane & 31, b = lane >> 5;
-  const uint32_t t0 = blockIdx.y * 32, e0 = blockIdx.x * 32;
+  // token tiles vary fastest: workgroups go to the XCDs round-robin, so each XCD's L2 sees an
+  // eighth of the token rows (and all of the small router matrix)
+  const uint32_t t0 = blockIdx.x * 32, e0 = blockIdx.y * 32;
   const uint32_t n_i = D / 512;
   const uint16_t* xrow = x + static_cast<size_t>(min(t0 + m, T - 1)) * x_stride + 8 * (16 * wv + b);
   const uint16_t* wrow = W + static_cast<size_t>(e0 + m) * D + 8 * (16 * wv + b);
@@ -811,7 +813,7 @@ __global__ __launch_bounds__(256) void prefill_reduce_kernel(const float* __rest
 hipError_t launch_prefill_router(hipStream_t s, const uint16_t* W, const uint16_t* x, uint32_t E,
                                  uint32_t D, uint32_t T, uint32_t x_stride, float* logits) {
   if (D % 512 == 0 && E % 32 == 0 && aligned16(W) && aligned16(x) && x_stride % 8 == 0) {
-    prefill_router_mfma_kernel<<<dim3(E / 32, (T + 31) / 32), dim3(256), 0, s>>>(W, x, E, D, T, x_stride, logits);
+    prefill_router_mfma_kernel<<<dim3((T + 31) / 32, E / 32), dim3(256), 0, s>>>(W, x, E, D, T, x_stride, logits);
     return hipGetLastError();
   }
   const uint32_t cpl = (D / 8 + 63) / 64;

@@ -37,9 +37,11 @@ __global__ __launch_bounds__(64) void topk_kernel(const float* __restrict__ logi
   if (mode == 0)
     topk_select_fast(logits + static_cast<size_t>(tok) * e, e, k, idx + static_cast<size_t>(tok) * k,
                      w + static_cast<size_t>(tok) * k, threadIdx.x);
-  else
-    topk_wave(logits + static_cast<size_t>(tok) * e, e, k, mode, idx + static_cast<size_t>(tok) * k,
-              w + static_cast<size_t>(tok) * k, threadIdx.x);
+  else {
+    __shared__ float s_p[MF_MAX_EXPERTS];
+    topk_full_softmax_fast(logits + static_cast<size_t>(tok) * e, s_p, e, k, idx + static_cast<size_t>(tok) * k,
+                           w + static_cast<size_t>(tok) * k, threadIdx.x);
+  }
 }
 
 hipError_t launch_router_logits(hipStream_t s, const uint16_t* w, const uint16_t* x, uint32_t e,

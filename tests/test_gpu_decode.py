@@ -85,6 +85,54 @@ def test_gemv_matches_oracle(gpu, oracle, bits, m, n, t):
         assert np.array_equal(yi.cpu().numpy()[0].view(np.uint32), got[i].view(np.uint32))
 
 
+@pytest.mark.parametrize("bits,m,n,t", [
+    (4, 1024, 2048, 1),    # one wave step per row: same partition as the per-row kernel
+    (4, 1100, 5120, 1),    # 2.5 steps: the last step is half empty; rows not a multiple of the grid
+    (4, 1024, 5120, 4),    # four token rows held in registers
+    (4, 1024, 8192, 2),    # longer than one wave can hold at T=2: two waves per row, LDS combine
+    (4, 1280, 17408, 1),   # nine steps, split over waves when there are few rows
+    (2, 1024, 8192, 1),    # 2-bit: 64 elements per 16 bytes
+    (2, 1024, 4096, 4),
+])
+def test_gemv_streaming_rows_kernel(gpu, oracle, bits, m, n, t):
+    """wide matrices take the streaming form (x slices resident in registers, rows walked by
+    a wave); same contract as the per-row kernel"""
+    rng = oracle.Rng.key(0xF3, f"stream-{bits}-{m}-{n}-{t}")
+    q = oracle.quantize(rng.uniform_fill(-1.0, 1.0, m * n).reshape(m, n), bits)
+    x = oracle.bf16_bits(rng.uniform_fill(-1.0, 1.0, t * n).reshape(t, n))
+    ref = oracle.gemv_multix(q, x)
+    xd = ops.bf16_tensor(x)
+    y32 = torch.full((t, m), 7.0, dtype=torch.float32, device="cuda")
+    g = ops.DequantInt4GEMVMultiX(gpu)
+    dq = to_device_q(q)
+    g.encode(dq, xd, y32, m, n, t, output_float32=True)
+    _sync()
+    got = y32.cpu().numpy()
+    assert np.abs(got - ref).max() / max(np.abs(ref).max(), 1e-6) < 2e-5
+    if t > 1:  # multi-token rows == single-token calls, bit for bit, when the row split is the same
+        yi = torch.zeros((1, m), dtype=torch.float32, device="cuda")
+        g.encode(dq, xd[0:1].contiguous(), yi, m, n, 1, output_float32=True)
+        _sync()
+        assert np.abs(yi.cpu().numpy()[0] - got[0]).max() / max(np.abs(ref).max(), 1e-6) < 2e-6
+
+
+@pytest.mark.parametrize("d,f,t", [(2048, 1024, 1), (5120, 1536, 4)])
+def test_shared_expert_streaming_rows_kernel(gpu, oracle, d, f, t):
+    """dense SwiGLU MLP wide enough for the streaming gate/up and down kernels"""
+    rng = oracle.Rng.key(0xF4, f"mlp-{d}-{f}-{t}")
+    gq = oracle.quantize(rng.normal(0.0, 0.02, f * d).reshape(f, d), 4)
+    uq = oracle.quantize(rng.normal(0.0, 0.02, f * d).reshape(f, d), 4)
+    dq = oracle.quantize(rng.normal(0.0, 0.02, d * f).reshape(d, f), 4)
+    x = oracle.bf16_bits(rng.normal(0.0, 1.0, t * d).reshape(t, d))
+    ref = np.stack([oracle.shared_expert(gq, uq, dq, x[i]) for i in range(t)])
+    y = torch.zeros((t, d), dtype=torch.bfloat16, device="cuda")
+    scratch = torch.zeros((t, f), dtype=torch.bfloat16, device="cuda")
+    ops.SharedExpertInt4(gpu).encode(ops.bf16_tensor(x), to_device_q(gq), to_device_q(uq),
+                                     to_device_q(dq), y, scratch, t=t)
+    _sync()
+    assert_layer_close(oracle.bf16_to_float(ops.bf16_bits(y)), oracle.bf16_to_float(ref), "streaming mlp")
+
+
 def test_gemv_misaligned_pointers(gpu, oracle):
     m, n = 9, 256
     rng = oracle.Rng.key(0xF2, "gemv-misaligned")

@@ -294,9 +294,12 @@ mf_status mf_group_pairs_host(const mf_pair* pairs, size_t n_pairs, int query_co
  * (PrefillMoE.swift:11-38) + PrefillSharedExpert.encodeBlock/encodeQwenScalarGate
  * (PrefillSharedExpert.swift:81-99, 27-36).  Result per token equals
  * mf_moe_decode_layer on that token within the layer tolerance.
- * Any t >= 1; 4-bit experts only (MF_ERR_UNSUPPORTED_BITS otherwise); d, f, shared_f
- * multiples of 128; x, y and every weight tensor 16-byte aligned.
- * workspace: device scratch of at least mf_moe_prefill_workspace_bytes(h, t). */
+ * Any t >= 1.  The matrix-core path takes 4-bit experts with d, f, shared_f multiples of
+ * 128 and x, y and every weight tensor 16-byte aligned; every other configuration (2-bit,
+ * ternary, other widths) runs the same rows through the decode launch, MF_MAX_TOKENS at a
+ * time, and needs no workspace.
+ * workspace: device scratch of at least mf_moe_prefill_workspace_bytes(h, t) (0 when the
+ * configuration takes the decode launch; workspace may then be null). */
 size_t mf_moe_prefill_workspace_bytes(const mf_moe* h, uint32_t t);
 mf_status mf_moe_prefill_layer(mf_moe* h, mf_stream stream, const mf_moe_layer_weights* wts,
                                const uint16_t* x, uint32_t t, uint16_t* y, void* workspace,

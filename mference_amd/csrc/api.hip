@@ -411,17 +411,30 @@ mf_status mf_moe_group_status(mf_moe* h, mf_stream stream) {
 }
 
 size_t mf_moe_prefill_workspace_bytes(const mf_moe* h, uint32_t t) {
-  if (!h || t == 0) return 0;
+  if (!h || t == 0 || !mf::prefill_supported(h->cfg)) return 0;
   return mf::prefill_workspace_bytes(h->cfg, t);
 }
 
 mf_status mf_moe_prefill_layer(mf_moe* h, mf_stream stream, const mf_moe_layer_weights* wts,
                                const uint16_t* x, uint32_t t, uint16_t* y, void* workspace,
                                size_t workspace_bytes, uint32_t* out_idx, float* out_w) {
-  if (!h || !wts || !x || !y || !workspace) return MF_ERR_INVALID_ARGUMENT;
+  if (!h || !wts || !x || !y) return MF_ERR_INVALID_ARGUMENT;
   if (t == 0 || t > (1u << 20)) return MF_ERR_INVALID_ARGUMENT;
   const mf_moe_config& c = h->cfg;
-  if (!mf::prefill_supported(c)) return MF_ERR_UNSUPPORTED_BITS;
+  if (!mf::prefill_supported(c)) {
+    // 2-bit / ternary experts, or widths the matmul tiles do not divide: the same rows through
+    // the decode launch, MF_MAX_TOKENS at a time (correct for every configuration, not fast)
+    for (uint32_t t0 = 0; t0 < t; t0 += MF_MAX_TOKENS) {
+      const uint32_t n = t - t0 < MF_MAX_TOKENS ? t - t0 : MF_MAX_TOKENS;
+      const mf_status st = mf_moe_decode_layer(
+          h, stream, wts, x + static_cast<size_t>(t0) * c.d, n, y + static_cast<size_t>(t0) * c.d, nullptr,
+          out_idx ? out_idx + static_cast<size_t>(t0) * c.top_k : nullptr,
+          out_w ? out_w + static_cast<size_t>(t0) * c.top_k : nullptr);
+      if (st != MF_OK) return st;
+    }
+    return MF_OK;
+  }
+  if (!workspace) return MF_ERR_INVALID_ARGUMENT;
   if (workspace_bytes < mf::prefill_workspace_bytes(c, t)) return MF_ERR_SCRATCH_TOO_SMALL;
   const uint32_t offs = wts->offsets.gate_w | wts->offsets.up_w | wts->offsets.down_w;
   if (!wts->router_w || !wts->expert_base || !offsets_ok(wts->offsets, c.bits) ||

@@ -310,9 +310,9 @@ class MoE:
         """Ragged prefill layer over t tokens (PrefillGroupedRoutedMoE.encodeStreamedBatched,
         PrefillGroupedRoutedMoE.swift:392-466, + reduce + shared expert).  `workspace`: uint8
         device tensor of at least prefill_workspace_bytes(t); allocated when None."""
-        need = self.prefill_workspace_bytes(t)
+        need = self.prefill_workspace_bytes(t)  # 0 for formats that take the decode launch
         if workspace is None:
-            workspace = torch.empty(need, dtype=torch.uint8, device=x.device)
+            workspace = torch.empty(max(need, 16), dtype=torch.uint8, device=x.device)
         lw = weights.c()
         check(_capi.lib().mf_moe_prefill_layer(self._h, _stream(stream), C.byref(lw), _ptr(x), t,
                                                _ptr(y), _ptr(workspace), workspace.numel(),

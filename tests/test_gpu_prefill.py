@@ -115,18 +115,35 @@ def test_prefill_skewed_routing_and_decode_agreement(gpu, oracle):
                        "prefill vs decode launch")
 
 
-def test_prefill_rejects_what_it_does_not_cover(gpu, oracle):
-    layer = oracle.synth_layer(ROOT_SEED + 0xA200, 256, 128, 16, 4, bits=2, fs=0)
-    moe = make_moe(gpu, layer)
-    wts = to_device_layer(layer)
-    x = ops.bf16_tensor(oracle.synth_x(1, 4, 256))
-    y = torch.zeros((4, 256), dtype=torch.bfloat16, device="cuda")
-    with pytest.raises(_capi.MfError) as err:
-        moe.encode_prefill_layer(wts, x, y, 4, workspace=torch.empty(1 << 20, dtype=torch.uint8, device="cuda"))
-    assert err.value.status == -3
+def test_prefill_other_formats_take_the_decode_launch(gpu, oracle):
+    """2-bit and ternary experts have no matrix-core path: the call runs the rows through the
+    decode launch eight at a time and gives exactly the decode result."""
+    for bits, mode in ((2, 0), (1, 1)):
+        d, f, e, k, fs, t = 256, 128, 32, 4, 128 if bits == 2 else 0, 19
+        layer = oracle.synth_layer(ROOT_SEED + 0xA200 + bits, d, f, e, k, bits=bits, fs=fs, router_mode=mode)
+        x = oracle.synth_x(ROOT_SEED + 0xA200 + bits, t, d)
+        ref_y, ref_idx, ref_w = oracle.moe_layer(layer, x)
+        moe = make_moe(gpu, layer)
+        wts = to_device_layer(layer)
+        y, idx, w = _run_prefill(moe, wts, x, t, d, k)
+        assert np.array_equal(idx, ref_idx)
+        assert np.array_equal(w.view(np.uint32), ref_w.view(np.uint32))
+        assert_layer_close(oracle.bf16_to_float(y), oracle.bf16_to_float(ref_y), f"prefill bits={bits}")
+        yd = torch.zeros((t, d), dtype=torch.bfloat16, device="cuda")
+        xd = ops.bf16_tensor(x)
+        for t0 in range(0, t, 8):
+            n = min(8, t - t0)
+            moe.encode_decode_layer(wts, xd[t0:t0 + n], yd[t0:t0 + n], t=n)
+        moe.status()
+        assert np.array_equal(y, ops.bf16_bits(yd))
+
+
+def test_prefill_rejects_a_short_workspace(gpu, oracle):
     layer4 = oracle.synth_layer(ROOT_SEED + 0xA201, 256, 128, 16, 4, bits=4, fs=0)
     moe4 = make_moe(gpu, layer4)
     wts4 = to_device_layer(layer4)
+    x = ops.bf16_tensor(oracle.synth_x(1, 4, 256))
+    y = torch.zeros((4, 256), dtype=torch.bfloat16, device="cuda")
     assert moe4.prefill_workspace_bytes(4) > 0
     with pytest.raises(_capi.MfError) as err:
         moe4.encode_prefill_layer(wts4, x, y, 4, workspace=torch.empty(256, dtype=torch.uint8, device="cuda"))

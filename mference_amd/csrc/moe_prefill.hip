@@ -34,6 +34,7 @@ typedef __attribute__((ext_vector_type(16))) float f32x16_t;
 constexpr uint32_t kTileTokens = 64;   // tokens of one expert a workgroup handles
 constexpr uint32_t kQmmWaves = 4;      // waves per workgroup, 32 weight rows each
 constexpr uint32_t kQmmRows = kQmmWaves * 32;
+constexpr uint32_t kQmmXBytes = 2 * 2 * 512 * 16;  // x tile ring: 2 stages of 2 K groups
 
 struct Tile {
   uint32_t expert, pair_start, count, pad;
@@ -465,7 +466,7 @@ __device__ __forceinline__ uint4 load_bf16x8_guarded(const uint16_t* p, uint32_t
 // is one scalar per lane.  Two waves per SIMD stay resident (the register
 // budget of 256 keeps the matrix-core results in ordinary registers, where
 // the scale multiply reads them directly).
-// LDS (dynamic): x tile double buffer 2 x [2 nt][4 s][2 h][32 n] x 16 B,
+// LDS (dynamic): x tile ring, 2 stages x 2 K groups x [2 nt][4 s][2 h][32 n] x 16 B,
 // scale tables [NPROJ][4 waves][ng][32 rows] fp32, out slots [64] u32.
 template <int NPROJ, bool NG8>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2)))
@@ -497,9 +498,9 @@ void qmm_kernel(const QmmArgs a) {
     count = t.count;
   }
 
-  uint4* s_x = reinterpret_cast<uint4*>(smem);                      // 2 * 512 uint4
-  float* s_scale = reinterpret_cast<float*>(smem + 2 * 512 * 16);   // [NPROJ][4][ng][32]
-  uint32_t* s_slot = reinterpret_cast<uint32_t*>(smem + 2 * 512 * 16 + NPROJ * kQmmWaves * ng * 32 * 4);
+  uint4* s_x = reinterpret_cast<uint4*>(smem);                      // 2 stages x 2 groups x 512 uint4
+  float* s_scale = reinterpret_cast<float*>(smem + kQmmXBytes);     // [NPROJ][4][ng][32]
+  uint32_t* s_slot = reinterpret_cast<uint32_t*>(smem + kQmmXBytes + NPROJ * kQmmWaves * ng * 32 * 4);
 
   // weight pointers of this workgroup's projections
   const uint8_t* Wp[NPROJ];
@@ -552,18 +553,18 @@ void qmm_kernel(const QmmArgs a) {
   }
   // x rows of groups 0..2 and, for the bias terms, the group sums of the lane's two routes
   const uint16_t* st_src = a.x + static_cast<size_t>(st_row) * a.x_stride + st_q * 16;
-  uint4 xs[2][2];  // xs[k & 1] holds group k on its way to LDS
-  uint4 x0[2];
-  x0[0] = *reinterpret_cast<const uint4*>(st_src);
-  x0[1] = *reinterpret_cast<const uint4*>(st_src + 8);
-  xs[1][0] = xs[1][1] = xs[0][0] = xs[0][1] = make_uint4(0, 0, 0, 0);
-  if (NG8 || ng > 1) {
-    xs[1][0] = *reinterpret_cast<const uint4*>(st_src + kGroup);
-    xs[1][1] = *reinterpret_cast<const uint4*>(st_src + kGroup + 8);
-  }
-  if (NG8 || ng > 2) {
-    xs[0][0] = *reinterpret_cast<const uint4*>(st_src + 2 * kGroup);
-    xs[0][1] = *reinterpret_cast<const uint4*>(st_src + 2 * kGroup + 8);
+  // K groups travel in pairs (ng is even: kdim is a multiple of 128)
+  uint4 xs[2][2];  // the pair after the one in LDS, on its way there
+  uint4 x0[2][2];
+#pragma unroll
+  for (int gi = 0; gi < 2; ++gi) {
+    x0[gi][0] = *reinterpret_cast<const uint4*>(st_src + gi * kGroup);
+    x0[gi][1] = *reinterpret_cast<const uint4*>(st_src + gi * kGroup + 8);
+    xs[gi][0] = xs[gi][1] = make_uint4(0, 0, 0, 0);
+    if (NG8 || ng > 2) {
+      xs[gi][0] = *reinterpret_cast<const uint4*>(st_src + (2 + gi) * kGroup);
+      xs[gi][1] = *reinterpret_cast<const uint4*>(st_src + (2 + gi) * kGroup + 8);
+    }
   }
   qmm_trace(a, work, 1);
 
@@ -662,32 +663,39 @@ void qmm_kernel(const QmmArgs a) {
   uint32_t rd_col[4];
 #pragma unroll
   for (int sidx = 0; sidx < 4; ++sidx) rd_col[sidx] = (m + 4 * (sidx >> 1) + 8 * h) & 31;
-  s_x[st_slot0] = x0[0];
-  s_x[st_slot1] = x0[1];
+#pragma unroll
+  for (int gi = 0; gi < 2; ++gi) {
+    s_x[gi * 512 + st_slot0] = x0[gi][0];
+    s_x[gi * 512 + st_slot1] = x0[gi][1];
+  }
 
   // Weight codes run four K groups ahead in registers (the expert's bytes come
-  // from HBM); x rows come from L2 and run three groups ahead, two in registers,
-  // one in the LDS buffer that is not being read.
+  // from HBM); x rows come from L2 in pairs of groups, one pair in registers behind
+  // the pair in the LDS stage that is not being read.
 
   for (uint32_t g0 = 0; g0 < ng; g0 += 4) {
 #pragma unroll
-    for (int u = 0; u < 4; ++u) {
-      const uint32_t g = g0 + u;
-      if (g >= ng) break;
-      __syncthreads();  // buffer g & 1 is complete, buffer (g + 1) & 1 is no longer read
-      if (g == 9) qmm_trace(a, work, 5);
-      if (g == 10) qmm_trace(a, work, 7);
-      // ---- x of group g + 1 into the other buffer, fetch group g + 3 into the freed registers
-      if (g + 1 < ng) {
-        uint4* wbuf = s_x + ((u + 1) & 1) * 512;
-        wbuf[st_slot0] = xs[(u + 1) & 1][0];
-        wbuf[st_slot1] = xs[(u + 1) & 1][1];
-        if (g + 3 < ng) {
-          xs[(u + 1) & 1][0] = *reinterpret_cast<const uint4*>(st_src + (g + 3) * kGroup);
-          xs[(u + 1) & 1][1] = *reinterpret_cast<const uint4*>(st_src + (g + 3) * kGroup + 8);
+    for (int uu = 0; uu < 2; ++uu) {  // pair of K groups g0 + 2uu, g0 + 2uu + 1 in stage uu
+      const uint32_t gu = g0 + 2 * uu;
+      if (gu >= ng) break;
+      __syncthreads();  // stage uu is complete, stage uu ^ 1 is no longer read
+      // ---- the next pair into the other stage, fetch the pair after it into the freed registers
+      if (gu + 2 < ng) {
+        uint4* wbuf = s_x + (uu ^ 1) * 1024;
+#pragma unroll
+        for (int gi = 0; gi < 2; ++gi) {
+          wbuf[gi * 512 + st_slot0] = xs[gi][0];
+          wbuf[gi * 512 + st_slot1] = xs[gi][1];
+        }
+        if (gu + 4 < ng) {
+#pragma unroll
+          for (int gi = 0; gi < 2; ++gi) {
+            xs[gi][0] = *reinterpret_cast<const uint4*>(st_src + (gu + 4 + gi) * kGroup);
+            xs[gi][1] = *reinterpret_cast<const uint4*>(st_src + (gu + 4 + gi) * kGroup + 8);
+          }
         }
       }
-      if (u == 0) {  // codes of the next four groups
+      if (uu == 0) {  // codes of the next four groups
 #pragma unroll
         for (int p = 0; p < NPROJ; ++p)
 #pragma unroll
@@ -696,35 +704,38 @@ void qmm_kernel(const QmmArgs a) {
             if (g0 + 4 + v < ng) nxt[p][v] = *reinterpret_cast<const uint4*>(wrow[p] + (g0 + 4 + v) * 32);
           }
       }
-
-      // ---- matrix core: tmp[token, row] = sum over the group of x * (8 + q/2)
-      const uint4* buf = s_x + (u & 1) * 512;
-      uint4 bx[2][4];
 #pragma unroll
-      for (int nt = 0; nt < 2; ++nt)
-#pragma unroll
-        for (int s = 0; s < 4; ++s) bx[nt][s] = buf[((nt * 4 + s) * 2 + h) * 32 + rd_col[s]];
-#pragma unroll
-      for (int p = 0; p < NPROJ; ++p) {
-        const uint32_t cw[4] = {cur[p][u].x, cur[p][u].y, cur[p][u].z, cur[p][u].w};
-        const float sc = s_scale[((p * kQmmWaves + wv) * ng + g) * 32 + m];
-        f32x16_t tmp[2];
+      for (int gi = 0; gi < 2; ++gi) {
+        const uint32_t g = gu + gi;
+        // ---- matrix core: tmp[token, row] = sum over the group of x * (8 + q/2)
+        const uint4* buf = s_x + uu * 1024 + gi * 512;
+        uint4 bx[2][4];
 #pragma unroll
         for (int nt = 0; nt < 2; ++nt)
 #pragma unroll
-          for (int r = 0; r < 16; ++r) tmp[nt][r] = 0.0f;
+          for (int s = 0; s < 4; ++s) bx[nt][s] = buf[((nt * 4 + s) * 2 + h) * 32 + rd_col[s]];
 #pragma unroll
-        for (int s = 0; s < 4; ++s) {
-          const uint4 av = expand_q4(cw[s]);
-          tmp[0] = mfma_bf16(bx[0][s], av, tmp[0]);
-          tmp[1] = mfma_bf16(bx[1][s], av, tmp[1]);
+        for (int p = 0; p < NPROJ; ++p) {
+          const uint4 cv = cur[p][2 * uu + gi];
+          const uint32_t cw[4] = {cv.x, cv.y, cv.z, cv.w};
+          const float sc = s_scale[((p * kQmmWaves + wv) * ng + g) * 32 + m];
+          f32x16_t tmp[2];
+#pragma unroll
+          for (int nt = 0; nt < 2; ++nt)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) tmp[nt][r] = 0.0f;
+#pragma unroll
+          for (int s = 0; s < 4; ++s) {
+            const uint4 av = expand_q4(cw[s]);
+            tmp[0] = mfma_bf16(bx[0][s], av, tmp[0]);
+            tmp[1] = mfma_bf16(bx[1][s], av, tmp[1]);
+          }
+#pragma unroll
+          for (int nt = 0; nt < 2; ++nt)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) acc[p][nt][r] = __builtin_fmaf(sc, tmp[nt][r], acc[p][nt][r]);
         }
-#pragma unroll
-        for (int nt = 0; nt < 2; ++nt)
-#pragma unroll
-          for (int r = 0; r < 16; ++r) acc[p][nt][r] = __builtin_fmaf(sc, tmp[nt][r], acc[p][nt][r]);
       }
-      if (g == 9) qmm_trace(a, work, 6);
     }
 #pragma unroll
     for (int p = 0; p < NPROJ; ++p)
@@ -852,7 +863,7 @@ size_t group_scratch_words() { return 2048 + static_cast<size_t>(kGroupChunks) *
 
 size_t qmm_lds_bytes(uint32_t kdim, int nproj) {
   const uint32_t ng = kdim / kGroup;
-  return 2 * 512 * 16 + static_cast<size_t>(nproj) * kQmmWaves * ng * 32 * 4 + kTileTokens * 4;
+  return kQmmXBytes + static_cast<size_t>(nproj) * kQmmWaves * ng * 32 * 4 + kTileTokens * 4;
 }
 
 hipError_t launch_prep_rows(hipStream_t s, const uint16_t* src, uint16_t* dst, float* sums, size_t elems) {

@@ -139,6 +139,8 @@ struct RowsArgs {
 
 template <int BITS, int T, int ITS, int NPROJ>
 __global__ __launch_bounds__(256) void rows_stream_kernel(const RowsArgs a) {
+  // rows in flight per wave: HBM under load answers in 2-3 us and a row's arithmetic is under 1 us
+  constexpr int DEPTH = 2;
   constexpr int EPL = Fmt<BITS>::kElemsPer16B;
   __shared__ float s_part[4][T][NPROJ];
   const uint32_t lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
@@ -183,45 +185,45 @@ __global__ __launch_bounds__(256) void rows_stream_kernel(const RowsArgs a) {
   int tab_src[ITS];                                // lane holding this lane's entry of step it,
 #pragma unroll                                     // in table word (it * GPS) / 64
   for (int it = 0; it < ITS; ++it) tab_src[it] = static_cast<int>((it * GPS + lane * EPL / kGroup) & 63u) << 2;
-  uint4 codes[NPROJ][ITS];
-  uint32_t sraw[NPROJ][TW], braw[NPROJ][TW];
-  auto fetch = [&](uint32_t row) {
-    const size_t r = row < a.M ? row : a.M - 1;
-#pragma unroll
-    for (int p = 0; p < NPROJ; ++p) {
-#pragma unroll
-      for (int it = 0; it < ITS; ++it)
-        codes[p][it] = *reinterpret_cast<const uint4*>(a.W[p] + r * row_bytes +
-                                                       static_cast<size_t>(e0[it]) * Store<BITS>::kBits / 8);
-#pragma unroll
-      for (int k = 0; k < TW; ++k) {
-        sraw[p][k] = a.S[p][r * n_groups + tab_g[k]];
-        if constexpr (BITS != kBitsTernary) braw[p][k] = a.B[p][r * n_groups + tab_g[k]];
-      }
-    }
-  };
-
-  uint32_t row = blockIdx.x * rows_per_wg + slot;
+  uint4 codes[DEPTH][NPROJ][ITS];
+  uint32_t sraw[DEPTH][NPROJ][TW], braw[DEPTH][NPROJ][TW];
   const uint32_t stride = gridDim.x * rows_per_wg;
+  const uint32_t row0 = blockIdx.x * rows_per_wg + slot;
   const uint32_t row_end = (a.M + stride - 1) / stride * stride;  // every wave runs the same trip count
-  fetch(row);
-  for (; row < row_end; row += stride) {
-    uint4 cur[NPROJ][ITS];
+#define MF_FETCH(U, ROW)                                                                            \
+  do {                                                                                              \
+    const size_t fr = (ROW) < a.M ? (ROW) : a.M - 1;                                                \
+    _Pragma("unroll") for (int p = 0; p < NPROJ; ++p) {                                             \
+      _Pragma("unroll") for (int it = 0; it < ITS; ++it)                                            \
+        codes[U][p][it] = *reinterpret_cast<const uint4*>(                                          \
+            a.W[p] + fr * row_bytes + static_cast<size_t>(e0[it]) * Store<BITS>::kBits / 8);        \
+      _Pragma("unroll") for (int k = 0; k < TW; ++k) {                                              \
+        sraw[U][p][k] = a.S[p][fr * n_groups + tab_g[k]];                                           \
+        if constexpr (BITS != kBitsTernary) braw[U][p][k] = a.B[p][fr * n_groups + tab_g[k]];       \
+      }                                                                                             \
+    }                                                                                               \
+  } while (0)
+#pragma unroll
+  for (int u = 0; u < DEPTH; ++u) MF_FETCH(u, row0 + u * stride);
+
+  for (uint32_t base = row0; base < row_end; base += DEPTH * stride) {
+#pragma unroll
+  for (int u = 0; u < DEPTH; ++u) {
+    const uint32_t row = base + u * stride;
+    if (row >= row_end) break;
     float sc[NPROJ][ITS], bi[NPROJ][ITS];
 #pragma unroll
     for (int p = 0; p < NPROJ; ++p)
 #pragma unroll
       for (int it = 0; it < ITS; ++it) {
-        cur[p][it] = codes[p][it];
         uint32_t sv = 0, bv = 0;
-        sv = static_cast<uint32_t>(__builtin_amdgcn_ds_bpermute(tab_src[it], static_cast<int>(sraw[p][(it * GPS) / 64])));
+        sv = static_cast<uint32_t>(__builtin_amdgcn_ds_bpermute(tab_src[it], static_cast<int>(sraw[u][p][(it * GPS) / 64])));
         if constexpr (BITS != kBitsTernary)
-          bv = static_cast<uint32_t>(__builtin_amdgcn_ds_bpermute(tab_src[it], static_cast<int>(braw[p][(it * GPS) / 64])));
+          bv = static_cast<uint32_t>(__builtin_amdgcn_ds_bpermute(tab_src[it], static_cast<int>(braw[u][p][(it * GPS) / 64])));
         sc[p][it] = __uint_as_float(sv << 16);
         if constexpr (BITS == kBitsTernary) bi[p][it] = -sc[p][it];
         else bi[p][it] = __uint_as_float(bv << 16);
       }
-    if (row + stride < row_end) fetch(row + stride);
 
     float acc[T][NPROJ];
 #pragma unroll
@@ -234,7 +236,7 @@ __global__ __launch_bounds__(256) void rows_stream_kernel(const RowsArgs a) {
       for (int p = 0; p < NPROJ; ++p)
 #pragma unroll
         for (int t = 0; t < T; ++t) {
-          const float dot = codes_dot<BITS>(cur[p][it], xs[t][it]);
+          const float dot = codes_dot<BITS>(codes[u][p][it], xs[t][it]);
           acc[t][p] = __builtin_fmaf(sc[p][it], dot, acc[t][p]);
           acc[t][p] = __builtin_fmaf(bi[p][it], xs[t][it].sum, acc[t][p]);
         }
@@ -274,6 +276,207 @@ __global__ __launch_bounds__(256) void rows_stream_kernel(const RowsArgs a) {
         } else {
           static_cast<uint16_t*>(a.y)[at] = f_to_bf16(acc[t][0]);
         }
+      }
+    }
+    if (row + DEPTH * stride < row_end) MF_FETCH(u, row + DEPTH * stride);  // refill the slot just consumed
+  }
+  }
+#undef MF_FETCH
+}
+
+// Matrix-core form of the same two operations (4-bit codes, T <= 8).  The vector ALU is what
+// limits the streaming kernel: extracting a code and feeding it to a dot product costs about
+// three instructions per code.  Here a code costs one (mask-and-or into a bf16 operand) and the
+// bf16 matrix core does the products: per 64-wide K group, D[token, row] = sum x * (8 + q/2) over
+// four 32x32x16 MFMAs with the tokens as the (mostly empty) M side, so a lane ends up with ONE
+// weight row and the group's scale is a per-lane scalar, applied to the T live accumulator rows
+// only.  A workgroup is one block of 32 weight rows; its KS waves split K, each keeps the x rows
+// of its K range (pre-ordered for the code pairing, with their group sums) in its own part of
+// LDS, and the partial sums meet in LDS in wave order.  Bias and offset terms are MFMAs over the
+// group index, as in the prefill matmul.
+struct RowsMfmaArgs {
+  const uint8_t* W[2];
+  const uint16_t* S[2];
+  const uint16_t* B[2];
+  const uint16_t* x;   // [T, N]
+  void* y;             // NPROJ 1: [T, M] bf16 or fp32; NPROJ 2: act [T, M] bf16
+  uint32_t M, N, T;
+  uint32_t gps;        // K groups per wave (a multiple of 4)
+  int out_f32;
+};
+
+template <int NPROJ, int KS>
+__global__ __launch_bounds__(KS * 64) void rows_mfma_kernel(const RowsMfmaArgs a) {
+  extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
+  const uint32_t lane = threadIdx.x & 63, ks = threadIdx.x >> 6, n_ks = KS;
+  const uint32_t m = lane & 31, h = lane >> 5;
+  const uint32_t T = a.T, ng = a.N / kGroup;
+  const uint32_t gps = a.gps;                               // K groups per wave
+  const uint32_t g_begin = min(ng, ks * gps), g_end = min(ng, g_begin + gps), n_g = g_end - g_begin;
+  const uint32_t row = blockIdx.x * 32 + m, row_c = min(row, a.M - 1);
+  const size_t row_bytes = static_cast<size_t>(a.N) / 2;
+
+  // this wave's LDS: x operands [group][s][h][token] x 16 B, then group sums [token][group] fp32
+  uint4* s_xw = reinterpret_cast<uint4*>(smem + static_cast<size_t>(ks) * gps * (8 * T * 16 + T * 4));
+  float* s_sum = reinterpret_cast<float*>(s_xw + gps * 8 * T);
+
+  // codes of the first four groups are on their way while x is staged
+  const uint8_t* wrow[NPROJ];
+  uint4 cur[NPROJ][4], nxt[NPROJ][4];
+#pragma unroll
+  for (int p = 0; p < NPROJ; ++p) {
+    wrow[p] = a.W[p] + row_c * row_bytes + static_cast<size_t>(g_begin) * 32 + h * 16;
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      cur[p][u] = make_uint4(0, 0, 0, 0);
+      if (static_cast<uint32_t>(u) < n_g) cur[p][u] = *reinterpret_cast<const uint4*>(wrow[p] + u * 32);
+    }
+  }
+
+  // ---- stage x: 8-value runs re-ordered to (0,4,1,5,2,6,3,7), one lane per run
+  const uint32_t runs = n_g * 8;
+  for (uint32_t i0 = 0; i0 < T * runs; i0 += kWave) {
+    const uint32_t i = i0 + lane;
+    const bool in = i < T * runs;
+    const uint32_t t = in ? i / runs : 0, c = in ? i % runs : 0;
+    uint4 v = make_uint4(0, 0, 0, 0);
+    if (in) v = *reinterpret_cast<const uint4*>(a.x + static_cast<size_t>(t) * a.N + (g_begin * 8 + c) * 8);
+    float sum = ((bf16_lo(v.x) + bf16_hi(v.x)) + (bf16_lo(v.y) + bf16_hi(v.y))) +
+                ((bf16_lo(v.z) + bf16_hi(v.z)) + (bf16_lo(v.w) + bf16_hi(v.w)));
+    sum = group_sum(sum, 8);
+    if (in) {
+      const uint32_t gl = c >> 3, ci = c & 7;
+      s_xw[((gl * 4 + (ci & 3)) * 2 + (ci >> 2)) * T + t] =
+          make_uint4(__builtin_amdgcn_perm(v.z, v.x, 0x05040100u), __builtin_amdgcn_perm(v.z, v.x, 0x07060302u),
+                     __builtin_amdgcn_perm(v.w, v.y, 0x05040100u), __builtin_amdgcn_perm(v.w, v.y, 0x07060302u));
+      if (ci == 0) s_sum[t * gps + gl] = sum;
+    }
+  }
+  __builtin_amdgcn_s_waitcnt(0xc07f);  // lgkmcnt(0): the wave reads back what its lanes wrote
+  __builtin_amdgcn_wave_barrier();
+
+  const uint32_t tok = m < T ? m : 0;  // accumulator rows past T read token 0 and are never stored
+  f32x16_t acc[NPROJ];
+#pragma unroll
+  for (int p = 0; p < NPROJ; ++p)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) acc[p][r] = 0.0f;
+
+  // ---- bias and offset terms: acc[token, row] += sumx[token, g] * (B[row, g] - 16 S[row, g])
+  for (uint32_t g0 = 0; g0 < n_g; g0 += 16) {
+    const uint32_t gl = g0 + 8 * h;
+    const bool have = gl < n_g;
+    const uint32_t gc = have ? gl : 0;
+    uint4 ab[NPROJ], as[NPROJ];
+#pragma unroll
+    for (int p = 0; p < NPROJ; ++p) {
+      const size_t at = static_cast<size_t>(row_c) * ng + g_begin + gc;
+      ab[p] = load_bf16x8_guarded(a.B[p] + at, n_g - gc);
+      const uint4 sv = load_bf16x8_guarded(a.S[p] + at, n_g - gc);
+      as[p] = make_uint4((sv.x + 0x02000200u) ^ 0x80008000u, (sv.y + 0x02000200u) ^ 0x80008000u,
+                         (sv.z + 0x02000200u) ^ 0x80008000u, (sv.w + 0x02000200u) ^ 0x80008000u);
+      if (!have) ab[p] = as[p] = make_uint4(0, 0, 0, 0);
+    }
+    uint32_t hi[8], mid[8], lo[8];
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      const float v = (m < T && gc + e < n_g) ? s_sum[tok * gps + gc + e] : 0.0f;
+      hi[e] = __float_as_uint(v) & 0xFFFF0000u;
+      const float r1 = v - __uint_as_float(hi[e]);
+      mid[e] = __float_as_uint(r1) & 0xFFFF0000u;
+      lo[e] = __float_as_uint(r1 - __uint_as_float(mid[e]));
+    }
+    const uint4 b_hi = make_uint4((hi[0] >> 16) | hi[1], (hi[2] >> 16) | hi[3], (hi[4] >> 16) | hi[5],
+                                  (hi[6] >> 16) | hi[7]);
+    const uint4 b_mid = make_uint4((mid[0] >> 16) | mid[1], (mid[2] >> 16) | mid[3], (mid[4] >> 16) | mid[5],
+                                   (mid[6] >> 16) | mid[7]);
+    const uint4 b_lo = make_uint4(__builtin_amdgcn_perm(lo[1], lo[0], 0x07060302u),
+                                  __builtin_amdgcn_perm(lo[3], lo[2], 0x07060302u),
+                                  __builtin_amdgcn_perm(lo[5], lo[4], 0x07060302u),
+                                  __builtin_amdgcn_perm(lo[7], lo[6], 0x07060302u));
+#pragma unroll
+    for (int p = 0; p < NPROJ; ++p) {
+      acc[p] = mfma_bf16(b_hi, ab[p], acc[p]);
+      acc[p] = mfma_bf16(b_hi, as[p], acc[p]);
+      acc[p] = mfma_bf16(b_mid, ab[p], acc[p]);
+      acc[p] = mfma_bf16(b_mid, as[p], acc[p]);
+      acc[p] = mfma_bf16(b_lo, ab[p], acc[p]);
+      acc[p] = mfma_bf16(b_lo, as[p], acc[p]);
+    }
+  }
+
+  // ---- main loop, four K groups per step; the next step's codes and scales are in flight
+  for (uint32_t g0 = 0; g0 < n_g; g0 += 4) {
+    uint2 sraw[NPROJ];
+#pragma unroll
+    for (int p = 0; p < NPROJ; ++p) {
+      const uint16_t* sp = a.S[p] + static_cast<size_t>(row_c) * ng + g_begin + g0;
+      if (g0 + 4 <= n_g) {
+        sraw[p] = *reinterpret_cast<const uint2*>(sp);  // 8-byte aligned: ng, gps and g0 are multiples of 4
+      } else {
+        uint32_t q[4];
+#pragma unroll
+        for (int e = 0; e < 4; ++e) q[e] = g0 + e < n_g ? sp[e] : 0u;
+        sraw[p] = make_uint2(q[0] | (q[1] << 16), q[2] | (q[3] << 16));
+      }
+#pragma unroll
+      for (int v = 0; v < 4; ++v) {
+        nxt[p][v] = cur[p][v];
+        if (g0 + 4 + v < n_g) nxt[p][v] = *reinterpret_cast<const uint4*>(wrow[p] + (g0 + 4 + v) * 32);
+      }
+    }
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      const uint32_t gl = g0 + u;
+      if (gl >= n_g) break;
+      uint4 ax[4];
+#pragma unroll
+      for (int s4 = 0; s4 < 4; ++s4) ax[s4] = s_xw[((gl * 4 + s4) * 2 + h) * T + tok];
+#pragma unroll
+      for (int p = 0; p < NPROJ; ++p) {
+        const uint32_t cw[4] = {cur[p][u].x, cur[p][u].y, cur[p][u].z, cur[p][u].w};
+        const uint32_t sw = u < 2 ? sraw[p].x : sraw[p].y;
+        const float sc = 2.0f * ((u & 1) ? bf16_hi(sw) : bf16_lo(sw));
+        f32x16_t tmp;
+#pragma unroll
+        for (int r = 0; r < 16; ++r) tmp[r] = 0.0f;
+#pragma unroll
+        for (int s4 = 0; s4 < 4; ++s4) tmp = mfma_bf16(ax[s4], expand_q4(cw[s4]), tmp);
+#pragma unroll
+        for (int r = 0; r < 4; ++r) acc[p][r] = __builtin_fmaf(sc, tmp[r], acc[p][r]);  // tokens 4h + r
+      }
+    }
+#pragma unroll
+    for (int p = 0; p < NPROJ; ++p)
+#pragma unroll
+      for (int v = 0; v < 4; ++v) cur[p][v] = nxt[p][v];
+  }
+
+  // ---- the K splits meet: [wave][projection][token 0..7][32 rows], over the x area
+  __syncthreads();
+  float* s_comb = reinterpret_cast<float*>(smem);
+#pragma unroll
+  for (int p = 0; p < NPROJ; ++p)
+#pragma unroll
+    for (int r = 0; r < 4; ++r) s_comb[((ks * NPROJ + p) * 8 + 4 * h + r) * 32 + m] = acc[p][r];
+  __syncthreads();
+  if (threadIdx.x < T * 32) {
+    const uint32_t t = threadIdx.x >> 5, mm = threadIdx.x & 31, orow = blockIdx.x * 32 + mm;
+    float v[NPROJ];
+#pragma unroll
+    for (int p = 0; p < NPROJ; ++p) {
+      v[p] = 0.0f;
+      for (uint32_t q = 0; q < n_ks; ++q) v[p] = v[p] + s_comb[((q * NPROJ + p) * 8 + t) * 32 + mm];
+    }
+    if (orow < a.M) {
+      const size_t at = static_cast<size_t>(t) * a.M + orow;
+      if constexpr (NPROJ == 2) {
+        const float rg = round_bf16(v[0]), ru = round_bf16(v[1]);
+        static_cast<uint16_t*>(a.y)[at] = f_to_bf16(mf_silu(rg) * ru);
+      } else if (a.out_f32) {
+        static_cast<float*>(a.y)[at] = v[0];
+      } else {
+        static_cast<uint16_t*>(a.y)[at] = f_to_bf16(v[0]);
       }
     }
   }
@@ -384,7 +587,7 @@ bool rows_stream_try(hipStream_t s, const RowsArgs& in, uint32_t t, uint32_t num
   RowsArgs a = in;
   a.wpr = wpr;
   const uint32_t rows_per_wg = 4 / wpr;
-  const uint32_t grid = std::min<uint32_t>((a.M + rows_per_wg - 1) / rows_per_wg, num_cu * 2);
+  const uint32_t grid = std::min<uint32_t>((a.M + rows_per_wg - 1) / rows_per_wg, num_cu * (t == 1 ? 3u : 2u));
 #define MF_ROWS(TT, II)                                                                      \
   rows_stream_kernel<BITS, TT, II, NPROJ><<<dim3(grid), dim3(256), 0, s>>>(a)
   if constexpr (BITS != kBitsTernary) {
@@ -397,11 +600,51 @@ bool rows_stream_try(hipStream_t s, const RowsArgs& in, uint32_t t, uint32_t num
   return true;
 }
 
+// The matrix-core kernel takes 4-bit matrices with at least 1024 rows whose K is a multiple of
+// 256 (so that the per-wave group ranges start on 8-byte boundaries of the scale table), up to 8
+// token rows, when the x rows of one workgroup fit LDS.
+template <int NPROJ>
+bool rows_mfma_try(hipStream_t s, const RowsMfmaArgs& a, uint32_t num_cu, hipError_t& err) {
+  const uint32_t ng = a.N / kGroup;
+  // one or two token rows stream faster through rows_stream_kernel (1 KB contiguous per load
+  // instruction against 32-byte pieces of 32 rows here); from three rows on the dot products
+  // outweigh that
+  if (a.N % (4 * kGroup) || a.N < 2048 || a.T < 3 || a.T > 8 || a.M < 1024) return false;
+  const uint32_t blocks = (a.M + 31) / 32;
+  // enough waves to fill the chip: 4 K-splits when there are many row blocks, 16 when few
+  uint32_t n_ks = blocks * 4 >= num_cu * 8 ? 4 : 16;
+  while (n_ks > 4 && ng / n_ks < 4) n_ks /= 2;
+  uint32_t gps = (ng + n_ks - 1) / n_ks;
+  gps = (gps + 3) / 4 * 4;  // multiples of 4 groups per wave
+  const size_t lds = std::max<size_t>(static_cast<size_t>(n_ks) * gps * (8 * a.T * 16 + a.T * 4),
+                                      static_cast<size_t>(n_ks) * NPROJ * 8 * 32 * 4);
+  if (lds > 156 * 1024 || (n_ks != 4 && n_ks != 16) || (NPROJ == 2 && n_ks != 4)) return false;
+  RowsMfmaArgs b = a;
+  b.gps = gps;
+  const void* fn = n_ks == 4 ? reinterpret_cast<const void*>(rows_mfma_kernel<NPROJ, 4>)
+                             : reinterpret_cast<const void*>(rows_mfma_kernel<1, 16>);
+  if (lds > 48 * 1024) {
+    err = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds));
+    if (err != hipSuccess) return true;
+  }
+  if (n_ks == 4) rows_mfma_kernel<NPROJ, 4><<<dim3(blocks), dim3(256), lds, s>>>(b);
+  else rows_mfma_kernel<1, 16><<<dim3(blocks), dim3(1024), lds, s>>>(b);
+  err = hipGetLastError();
+  return true;
+}
+
 }  // namespace
 
 hipError_t launch_gemv(hipStream_t s, const mf_qtensor& w, int bits, const uint16_t* x, void* y,
                        uint32_t m, uint32_t n, uint32_t t, bool out_f32) {
   const bool al = aligned16(w.weights) && aligned16(x);
+  if (al && bits == kBits4 && aligned16(w.scales) && aligned16(w.biases)) {
+    RowsMfmaArgs ma{};
+    ma.W[0] = static_cast<const uint8_t*>(w.weights); ma.S[0] = w.scales; ma.B[0] = w.biases;
+    ma.x = x; ma.y = y; ma.M = m; ma.N = n; ma.T = t; ma.out_f32 = out_f32 ? 1 : 0;
+    hipError_t err = hipSuccess;
+    if (rows_mfma_try<1>(s, ma, device_cu_count(), err)) return err;
+  }
   if (al && (bits == kBits4 || bits == kBits2)) {
     RowsArgs a{};
     a.W[0] = static_cast<const uint8_t*>(w.weights); a.S[0] = w.scales; a.B[0] = w.biases;
@@ -429,6 +672,15 @@ hipError_t launch_gate_up_act(hipStream_t s, const mf_qtensor& gate, const mf_qt
                               int bits, const uint16_t* x, uint16_t* act, uint32_t f, uint32_t d,
                               uint32_t t) {
   const bool al = aligned16(gate.weights) && aligned16(up.weights) && aligned16(x);
+  if (al && bits == kBits4 && aligned16(gate.scales) && aligned16(gate.biases) && aligned16(up.scales) &&
+      aligned16(up.biases)) {
+    RowsMfmaArgs ma{};
+    ma.W[0] = static_cast<const uint8_t*>(gate.weights); ma.S[0] = gate.scales; ma.B[0] = gate.biases;
+    ma.W[1] = static_cast<const uint8_t*>(up.weights); ma.S[1] = up.scales; ma.B[1] = up.biases;
+    ma.x = x; ma.y = act; ma.M = f; ma.N = d; ma.T = t;
+    hipError_t err = hipSuccess;
+    if (rows_mfma_try<2>(s, ma, device_cu_count(), err)) return err;
+  }
   if (al && (bits == kBits4 || bits == kBits2)) {
     RowsArgs a{};
     a.W[0] = static_cast<const uint8_t*>(gate.weights); a.S[0] = gate.scales; a.B[0] = gate.biases;

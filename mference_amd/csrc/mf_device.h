@@ -252,6 +252,33 @@ __device__ __forceinline__ uint32_t and_or(uint32_t v, uint32_t mask, uint32_t m
   return r;
 }
 
+// ---- matrix-core forms of the same embedding
+typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8_t;
+typedef __attribute__((ext_vector_type(16))) float f32x16_t;
+
+__device__ __forceinline__ f32x16_t mfma_bf16(const uint4& a, const uint4& b, const f32x16_t& c) {
+  return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, a),
+                                                 __builtin_bit_cast(bf16x8_t, b), c, 0, 0, 0);
+}
+
+// one packed word of 4-bit codes -> MFMA operand: pairs (q0,q4),(q1,q5),(q2,q6),(q3,q7) as the
+// bf16 numbers 8 + q/2 (exponent 2^3, the code in mantissa bits 3..6).  16 is the smallest offset
+// a mask-and-or can give a 4-bit code, and the offset matters: the matrix core accumulates
+// offset * sum(x) alongside the signal and the correction term takes it out again in fp32.
+__device__ __forceinline__ uint4 expand_q4(uint32_t w) {
+  return make_uint4(and_or(w << 3, 0x00780078u, kMagic8), and_or(w >> 1, 0x00780078u, kMagic8),
+                    and_or(w >> 5, 0x00780078u, kMagic8), and_or(w >> 9, 0x00780078u, kMagic8));
+}
+
+// 8 bf16 from p, of which only the first `avail` exist (the rest read as 0)
+__device__ __forceinline__ uint4 load_bf16x8_guarded(const uint16_t* p, uint32_t avail) {
+  if (avail >= 8) return load_x8<false>(p);
+  uint32_t v[8];
+#pragma unroll
+  for (int i = 0; i < 8; ++i) v[i] = static_cast<uint32_t>(i) < avail ? p[i] : 0u;
+  return make_uint4(v[0] | (v[1] << 16), v[2] | (v[3] << 16), v[4] | (v[5] << 16), v[6] | (v[7] << 16));
+}
+
 // The activations one lane meets, permuted for the pairing above, plus their sum.
 template <int BITS> struct XSlice {
   static constexpr int kPairs = Fmt<BITS>::kElemsPer16B / 2;

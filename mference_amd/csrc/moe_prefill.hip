@@ -28,9 +28,6 @@
 
 namespace mf {
 
-typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8_t;
-typedef __attribute__((ext_vector_type(16))) float f32x16_t;
-
 constexpr uint32_t kTileTokens = 64;   // tokens of one expert a workgroup handles
 constexpr uint32_t kQmmWaves = 4;      // waves per workgroup, 32 weight rows each
 constexpr uint32_t kQmmRows = kQmmWaves * 32;
@@ -430,32 +427,9 @@ __device__ __forceinline__ void qmm_trace(const QmmArgs& a, uint32_t work, uint3
   if (a.trace && threadIdx.x == 0 && work < a.trace_items) a.trace[work * 8 + k] = wall_clock64();
 }
 
-__device__ __forceinline__ f32x16_t mfma_bf16(const uint4& a, const uint4& b, const f32x16_t& c) {
-  return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, a),
-                                                 __builtin_bit_cast(bf16x8_t, b), c, 0, 0, 0);
-}
-
 // silu with the hardware exp2 / reciprocal (1 ulp each): the result is narrowed to bf16 right after
 __device__ __forceinline__ float fast_silu(float x) {
   return x * __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(x * -1.4426950408889634f));
-}
-
-// one packed word of 4-bit codes -> MFMA operand: pairs (q0,q4),(q1,q5),(q2,q6),(q3,q7) as the
-// bf16 numbers 8 + q/2 (exponent 2^3, the code in mantissa bits 3..6).  16 is the smallest offset
-// a mask-and-or can give a 4-bit code, and the offset matters: the matrix core accumulates
-// offset * sum(x) alongside the signal and the correction term takes it out again in fp32.
-__device__ __forceinline__ uint4 expand_q4(uint32_t w) {
-  return make_uint4(and_or(w << 3, 0x00780078u, kMagic8), and_or(w >> 1, 0x00780078u, kMagic8),
-                    and_or(w >> 5, 0x00780078u, kMagic8), and_or(w >> 9, 0x00780078u, kMagic8));
-}
-
-// 8 bf16 from p, of which only the first `avail` exist (the rest read as 0)
-__device__ __forceinline__ uint4 load_bf16x8_guarded(const uint16_t* p, uint32_t avail) {
-  if (avail >= 8) return load_x8<false>(p);
-  uint32_t v[8];
-#pragma unroll
-  for (int i = 0; i < 8; ++i) v[i] = static_cast<uint32_t>(i) < avail ? p[i] : 0u;
-  return make_uint4(v[0] | (v[1] << 16), v[2] | (v[3] << 16), v[4] | (v[5] << 16), v[6] | (v[7] << 16));
 }
 
 // One workgroup: 64 routes of one expert x 128 weight rows (4 waves x 32) x

@@ -93,6 +93,8 @@ def test_gemv_matches_oracle(gpu, oracle, bits, m, n, t):
     (4, 1280, 17408, 1),   # nine steps, split over waves when there are few rows
     (2, 1024, 8192, 1),    # 2-bit: 64 elements per 16 bytes
     (2, 1024, 4096, 4),
+    (4, 1056, 5120, 5),    # three or more token rows of a 4-bit matrix: the matrix-core kernel
+    (4, 1024, 17408, 8),   # ... with 16 K-splits per row block
 ])
 def test_gemv_streaming_rows_kernel(gpu, oracle, bits, m, n, t):
     """wide matrices take the streaming form (x slices resident in registers, rows walked by

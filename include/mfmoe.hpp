@@ -1,0 +1,281 @@
+// mfmoe.hpp — C++ host-side mirror of Mference's Swift operator surface over the C ABI
+// of libmfmoe (mfmoe.h).  Header only, C++17.
+//
+// The reference's host code is Swift: a set of operator classes under
+// Sources/Mference/Kernels/ built from a MetalContext, whose encode…() methods append
+// dispatches to a caller-owned MTLCommandBuffer and `throw` typed errors.  The classes below
+// keep the reference's class and method names, argument order and error behaviour; a command
+// buffer becomes a hipStream_t (passed as mf_stream), an (MTLBuffer, offset) pair becomes a
+// device pointer (the caller adds the offset), `throws` becomes mf::Error carrying the
+// mf_status.  Nothing here allocates device memory or touches the HIP runtime: every call
+// goes straight to the C ABI.
+#ifndef MFMOE_HPP
+#define MFMOE_HPP
+
+#include <cstddef>
+#include <cstdint>
+#include <stdexcept>
+#include <string>
+#include <vector>
+
+#include "mfmoe.h"
+
+namespace mf {
+
+// `throws` of the reference (SharedExpertError, PrefillMoEGroupingError, MetalError, …):
+// one exception type carrying the status code; detail[] holds the payload of the grouping
+// errors (PrefillMoEGrouping.swift:52-88).
+class Error : public std::runtime_error {
+ public:
+  Error(mf_status s, const std::string& what_arg, uint32_t d0 = 0, uint32_t d1 = 0)
+      : std::runtime_error(what_arg), status(s), detail{d0, d1} {}
+  mf_status status;
+  uint32_t detail[2];
+};
+
+inline void check(mf_status s, const mf_ctx* ctx = nullptr) {
+  if (s == MF_OK) return;
+  std::string text = mf_status_string(s);
+  if (s == MF_ERR_LAUNCH && ctx) text += std::string(": ") + mf_last_hip_error(ctx);
+  throw Error(s, text);
+}
+
+// MetalContext (Infrastructure/Metal/MetalContext.swift:45-65): the device and its kernels.
+class MetalContext {
+ public:
+  explicit MetalContext(int device = 0) { check(mf_ctx_create(device, &ctx_)); }
+  ~MetalContext() { mf_ctx_destroy(ctx_); }
+  MetalContext(const MetalContext&) = delete;
+  MetalContext& operator=(const MetalContext&) = delete;
+  mf_ctx* raw() const { return ctx_; }
+  int computeUnits() const { return mf_ctx_num_cu(ctx_); }
+
+ private:
+  mf_ctx* ctx_ = nullptr;
+};
+
+// Quantization (Infrastructure/ModelIO/Quantization.swift:3-119), on device.
+class Quantization {
+ public:
+  static constexpr int groupSize = MF_GROUP_SIZE;
+  explicit Quantization(const MetalContext& context) : ctx_(context.raw()) {}
+  // quantizeInt4Affine (:50-102) for every row of w; bits 4 or 2
+  void quantizeInt4Affine(mf_stream stream, const float* w, size_t rows, size_t n, void* packed,
+                          uint16_t* scales, uint16_t* biases, mf_bits bits = MF_BITS_4) const {
+    check(mf_quantize_affine(ctx_, stream, w, rows, n, bits, packed, scales, biases), ctx_);
+  }
+  // dequantizeInt4Affine (:104-119)
+  void dequantizeInt4Affine(mf_stream stream, mf_qtensor q, size_t rows, size_t n, float* out,
+                            mf_bits bits = MF_BITS_4) const {
+    check(mf_dequantize(ctx_, stream, q, rows, n, bits, out), ctx_);
+  }
+
+ private:
+  mf_ctx* ctx_;
+};
+
+// DequantInt4GEMV (Kernels/Quant/DequantInt4GEMV.swift:57-103); any supported bit width.
+class DequantInt4GEMV {
+ public:
+  explicit DequantInt4GEMV(const MetalContext& context, mf_bits bits = MF_BITS_4)
+      : ctx_(context.raw()), bits_(bits) {}
+  void encode(mf_stream commandBuffer, mf_qtensor weights, const uint16_t* x, void* y, uint32_t m,
+              uint32_t n, bool outputFloat32 = false) const {
+    check(mf_gemv(ctx_, commandBuffer, weights, bits_, x, y, m, n, 1, outputFloat32 ? 1 : 0), ctx_);
+  }
+
+ protected:
+  mf_ctx* ctx_;
+  mf_bits bits_;
+};
+
+// DequantInt4GEMVMultiX (Kernels/Quant/DequantInt4GEMVMultiX.swift:48-82): t <= 8 token rows.
+class DequantInt4GEMVMultiX : public DequantInt4GEMV {
+ public:
+  static constexpr uint32_t maxTokens = MF_MAX_TOKENS;
+  using DequantInt4GEMV::DequantInt4GEMV;
+  void encode(mf_stream commandBuffer, mf_qtensor weights, const uint16_t* x, void* y, uint32_t m,
+              uint32_t n, uint32_t t, bool outputFloat32 = false) const {
+    check(mf_gemv(ctx_, commandBuffer, weights, bits_, x, y, m, n, t, outputFloat32 ? 1 : 0), ctx_);
+  }
+};
+
+// Elementwise (Kernels/Primitives/Elementwise.swift:60-87)
+class Elementwise {
+ public:
+  explicit Elementwise(const MetalContext& context) : ctx_(context.raw()) {}
+  void encodeSiluMul(mf_stream cb, const uint16_t* gate, const uint16_t* up, uint16_t* out,
+                     uint32_t count) const {
+    check(mf_silu_mul(ctx_, cb, gate, up, out, count), ctx_);
+  }
+  void encodeSigmoidScalarMul(mf_stream cb, uint16_t* y, const uint16_t* gate, uint32_t count,
+                              uint32_t rows = 1) const {
+    check(mf_sigmoid_scalar_mul(ctx_, cb, y, gate, count, rows), ctx_);
+  }
+  void encodeResidualAdd(mf_stream cb, uint16_t* hidden, const uint16_t* delta, uint32_t count) const {
+    check(mf_residual_add(ctx_, cb, hidden, delta, count), ctx_);
+  }
+
+ private:
+  mf_ctx* ctx_;
+};
+
+// SharedExpertInt4 (Kernels/MoE/SharedExpertInt4.swift:70-165), also the dense SwiGLU MLP.
+// Errors: MF_ERR_DIMENSION_MISMATCH / MF_ERR_SCRATCH_TOO_SMALL / MF_ERR_UNSUPPORTED_BITS are
+// SharedExpertError.dimensionMismatch / .scratchTooSmall / .unsupportedWeightBits (:4-19).
+class SharedExpertInt4 {
+ public:
+  explicit SharedExpertInt4(const MetalContext& context, mf_bits bits = MF_BITS_4)
+      : ctx_(context.raw()), bits_(bits) {}
+  void encode(mf_stream commandBuffer, const uint16_t* x, mf_qtensor gate, mf_qtensor up,
+              mf_qtensor down, uint32_t d, uint32_t f, uint16_t* y, uint16_t* scratchAct,
+              size_t scratchActBytes, uint32_t tokens = 1) const {
+    check(mf_shared_expert(ctx_, commandBuffer, x, gate, up, down, bits_, d, f, tokens, y, scratchAct,
+                           scratchActBytes), ctx_);
+  }
+
+ private:
+  mf_ctx* ctx_;
+  mf_bits bits_;
+};
+
+using MoEExpertOffsets = mf_expert_offsets;  // Kernels/MoE/MoE.swift:4-29
+
+// MoE (Kernels/MoE/MoE.swift), MoEDeepseekV4 (2-bit, top-6) and MapleMoE (ternary, full-softmax
+// router) in one class, selected by the configuration — the specialisation arguments of
+// MoE.init (MoE.swift:65-151).  An instance owns its device workspace and is serial
+// (MapleMoE.swift:3-6).
+class MoE {
+ public:
+  MoE(const MetalContext& context, uint32_t specializedD, uint32_t specializedF,
+      uint32_t specializedNumExperts, uint32_t specializedTopK = 8, mf_bits bits = MF_BITS_4,
+      mf_router_mode routerMode = MF_ROUTER_TOPK_SOFTMAX, float swigluLimit = 0.0f,
+      uint32_t sharedF = 0, mf_bits sharedBits = MF_BITS_4)
+      : ctx_(context.raw()) {
+    cfg_ = mf_moe_config{specializedD, specializedF, specializedNumExperts, specializedTopK, bits,
+                         routerMode,   swigluLimit,  sharedF,               sharedBits};
+    check(mf_moe_create(ctx_, &cfg_, &h_), ctx_);
+  }
+  ~MoE() { mf_moe_destroy(h_); }
+  MoE(const MoE&) = delete;
+  MoE& operator=(const MoE&) = delete;
+  const mf_moe_config& config() const { return cfg_; }
+
+  // encodeRouterGemma4 / encodeRouterTopK / encodeRouterTop8 (MoE.swift:153-203,
+  // MoEDeepseekV4.swift:92-100, MapleMoE.swift:81-131)
+  void encodeRouter(mf_stream cb, const uint16_t* weights, const uint16_t* hidden, uint32_t* outIndices,
+                    float* outWeights, uint32_t queryCount = 1, float* outLogits = nullptr) const {
+    check(mf_moe_router(h_, cb, weights, hidden, queryCount, cfg_.d, outIndices, outWeights, outLogits),
+          ctx_);
+  }
+  // encodeRoutedPersistentPhase1U16Load (MoE.swift:220-253)
+  void encodeRoutedPersistentPhase1U16Load(mf_stream cb, const void* experts, size_t expertStride,
+                                           const MoEExpertOffsets& routedOffsets, const uint32_t* indices,
+                                           const uint16_t* x, uint16_t* acts, uint32_t tokens = 1) const {
+    check(mf_moe_phase1(h_, cb, experts, expertStride, &routedOffsets, indices, x, tokens, cfg_.d, acts),
+          ctx_);
+  }
+  // encodeRoutedPersistentPhase2Reduce (MoE.swift:400-440)
+  void encodeRoutedPersistentPhase2Reduce(mf_stream cb, const void* experts, size_t expertStride,
+                                          const MoEExpertOffsets& routedOffsets, const uint32_t* indices,
+                                          const float* routingWeights, const uint16_t* acts,
+                                          const uint16_t* residual, uint16_t* y, uint32_t tokens = 1) const {
+    check(mf_moe_phase2(h_, cb, experts, expertStride, &routedOffsets, indices, routingWeights, acts,
+                        residual, tokens, y), ctx_);
+  }
+  // the whole decode layer in one launch (RealForwardRunner.swift:2811-3218 steps, no readback)
+  void encodeDecodeLayer(mf_stream cb, const mf_moe_layer_weights& weights, const uint16_t* x,
+                         uint16_t* y, uint32_t tokens = 1, uint16_t* hidden = nullptr,
+                         uint32_t* outIndices = nullptr, float* outWeights = nullptr) const {
+    check(mf_moe_decode_layer(h_, cb, &weights, x, tokens, y, hidden, outIndices, outWeights), ctx_);
+  }
+  // PrefillGroupedRoutedMoE.encodeStreamedBatched + PrefillMoE.encodeReduceTokenMajor +
+  // PrefillSharedExpert.encodeBlock (PrefillGroupedRoutedMoE.swift:392-466, PrefillMoE.swift:11-38,
+  // PrefillSharedExpert.swift:81-99) for `tokens` rows
+  size_t prefillWorkspaceBytes(uint32_t tokens) const { return mf_moe_prefill_workspace_bytes(h_, tokens); }
+  void encodePrefillLayer(mf_stream cb, const mf_moe_layer_weights& weights, const uint16_t* x,
+                          uint16_t* y, uint32_t tokens, void* workspace, size_t workspaceBytes,
+                          uint32_t* outIndices = nullptr, float* outWeights = nullptr) const {
+    check(mf_moe_prefill_layer(h_, cb, &weights, x, tokens, y, workspace, workspaceBytes, outIndices,
+                               outWeights), ctx_);
+  }
+  // PrefillRouter.makeTokenExpertPairs + PrefillMoEGrouping.groupTokenExpertPairs on device
+  void encodeGroup(mf_stream cb, const uint32_t* indices, const float* routingWeights, uint32_t tokens,
+                   mf_pair* sortedPairs, uint32_t* expertOffsets, uint32_t* expertCounts) const {
+    check(mf_moe_group(h_, cb, indices, routingWeights, tokens, sortedPairs, expertOffsets, expertCounts),
+          ctx_);
+  }
+  void groupStatus(mf_stream cb) const { check(mf_moe_group_status(h_, cb), ctx_); }
+  void setFused(bool enabled) const { check(mf_moe_set_fused(h_, enabled ? 1 : 0), ctx_); }
+  void status(mf_stream cb) const { check(mf_moe_status(h_, cb), ctx_); }
+
+ private:
+  mf_ctx* ctx_;
+  mf_moe_config cfg_{};
+  mf_moe* h_ = nullptr;
+};
+
+// PrefillTokenExpertPair (Kernels/Prefill/MoE/PrefillRouter.swift:4-28)
+using PrefillTokenExpertPair = mf_pair;
+
+// PrefillMoEGroupedRoutes (PrefillMoEGrouping.swift:3-50)
+struct PrefillMoEGroupedRoutes {
+  std::vector<PrefillTokenExpertPair> sortedPairs;
+  std::vector<uint32_t> expertOffsets, expertCounts;
+  std::vector<mf_group> groups;
+  std::vector<mf_tile> tiles;
+  uint32_t maxPairsPerExpert() const {
+    uint32_t m = 0;
+    for (const auto& g : groups) m = g.pair_count > m ? g.pair_count : m;
+    return m;
+  }
+  uint32_t maxPairsPerTile() const {
+    uint32_t m = 0;
+    for (const auto& t : tiles) m = t.pair_count > m ? t.pair_count : m;
+    return m;
+  }
+};
+
+// PrefillMoEGrouping (Kernels/Prefill/MoE/PrefillMoEGrouping.swift:91-192), host side.
+struct PrefillMoEGrouping {
+  // makeTokenExpertPairs (PrefillRouter.swift:91-111): token-major (token, rank) records
+  static std::vector<PrefillTokenExpertPair> makeTokenExpertPairs(const uint32_t* indices,
+                                                                  const uint32_t* weightBits,
+                                                                  uint32_t queryCount, uint32_t topK) {
+    std::vector<PrefillTokenExpertPair> pairs(static_cast<size_t>(queryCount) * topK);
+    for (uint32_t t = 0; t < queryCount; ++t)
+      for (uint32_t r = 0; r < topK; ++r) {
+        const size_t i = static_cast<size_t>(t) * topK + r;
+        pairs[i] = PrefillTokenExpertPair{t, indices[i], r, weightBits[i]};
+      }
+    return pairs;
+  }
+  // groupTokenExpertPairs; throws mf::Error with the PrefillMoEGroupingError case as status
+  static PrefillMoEGroupedRoutes groupTokenExpertPairs(const std::vector<PrefillTokenExpertPair>& pairs,
+                                                       int queryCount, int topK, int numExperts,
+                                                       int tileExpertCount = 16,
+                                                       const std::vector<uint64_t>* sortKeys = nullptr) {
+    PrefillMoEGroupedRoutes r;
+    const size_t ne = numExperts > 0 ? static_cast<size_t>(numExperts) : 1;
+    const size_t cap = pairs.size() < ne ? (pairs.empty() ? 1 : pairs.size()) : ne;
+    r.sortedPairs.resize(pairs.size());
+    r.expertOffsets.resize(ne);
+    r.expertCounts.resize(ne);
+    r.groups.resize(cap);
+    r.tiles.resize(cap);
+    size_t ng = 0, nt = 0;
+    uint32_t detail[2] = {0, 0};
+    const mf_status s = mf_group_pairs_host(
+        pairs.data(), pairs.size(), queryCount, topK, numExperts, tileExpertCount,
+        sortKeys ? sortKeys->data() : nullptr, sortKeys ? sortKeys->size() : 0, r.sortedPairs.data(),
+        r.expertOffsets.data(), r.expertCounts.data(), r.groups.data(), &ng, r.tiles.data(), &nt, detail);
+    if (s != MF_OK) throw Error(s, mf_status_string(s), detail[0], detail[1]);
+    r.groups.resize(ng);
+    r.tiles.resize(nt);
+    return r;
+  }
+};
+
+}  // namespace mf
+
+#endif  // MFMOE_HPP

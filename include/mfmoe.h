@@ -241,7 +241,10 @@ mf_status mf_moe_set_fused(mf_moe* h, int enabled);
  * workgroup writes the 100 MHz wall clock at its stage boundaries (slots:
  * 0 start, 1 stage A done, 2 logits gathered, 3 top-k done, 4 stage B done,
  * 5 routed activations gathered, 6 end) to device_buffer[workgroup*8 + slot]; needs
- * mf_ctx_num_cu()*8*8 bytes.  The counterpart of the reference's
+ * mf_ctx_num_cu()*8*8 bytes.  mf_moe_prefill_layer writes, for as many work
+ * items (tile x row slice) of its routed gate/up matmul as the buffer holds, the
+ * stamps 0 start, 1 loads issued, 2 tables and bias terms done, 3 main loop done,
+ * 4 end at device_buffer[item*8 + slot].  The counterpart of the reference's
  * MFERENCE_PHASES=1 phase counters (RealForwardRunner.swift:397-398). */
 mf_status mf_moe_set_phase_trace(mf_moe* h, uint64_t* device_buffer, size_t bytes);
 int mf_ctx_num_cu(const mf_ctx* ctx);

@@ -437,13 +437,14 @@ __device__ __forceinline__ float fast_silu(float x) {
 // product: the A operand is the x tile (tokens are the rows), the B operand is
 // the expanded codes, so a lane ends up holding ONE weight row (its column
 // m = lane % 32) for 16 tokens of each 32-token block, and the per-group scale
-// is one scalar per lane.  Two waves per SIMD stay resident (the register
-// budget of 256 keeps the matrix-core results in ordinary registers, where
-// the scale multiply reads them directly).
+// is one scalar per lane.  With two row blocks per wave two waves per SIMD stay
+// resident (the register budget of 256 keeps the matrix-core results in ordinary
+// registers, where the scale multiply reads them directly); with one row block the
+// kernel fits 168 registers and three waves stay resident.
 // LDS (dynamic): x tile ring, 2 stages x 2 K groups x [2 nt][4 s][2 h][32 n] x 16 B,
 // scale tables [NPROJ][4 waves][ng][32 rows] fp32, out slots [64] u32.
 template <int NPROJ, bool NG8>
-__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2)))
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(NPROJ == 1 ? 3 : 2, NPROJ == 1 ? 3 : 2)))
 void qmm_kernel(const QmmArgs a) {
   extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
   const uint32_t lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
@@ -515,7 +516,7 @@ void qmm_kernel(const QmmArgs a) {
     if (a.epi == 1) slot = pr.token * a.top_k + pr.rank;
   }
   const uint8_t* wrow[NPROJ];
-  uint4 cur[NPROJ][4], nxt[NPROJ][4];
+  uint4 cur[NPROJ][4];
 #pragma unroll
   for (int p = 0; p < NPROJ; ++p) {
     wrow[p] = Wp[p] + (row_base[p] + m) * row_bytes + h * 16;
@@ -643,7 +644,7 @@ void qmm_kernel(const QmmArgs a) {
     s_x[gi * 512 + st_slot1] = x0[gi][1];
   }
 
-  // Weight codes run four K groups ahead in registers (the expert's bytes come
+  // Weight codes run four K groups ahead in a ring of registers (the expert's bytes come
   // from HBM); x rows come from L2 in pairs of groups, one pair in registers behind
   // the pair in the LDS stage that is not being read.
 
@@ -668,15 +669,6 @@ void qmm_kernel(const QmmArgs a) {
             xs[gi][1] = *reinterpret_cast<const uint4*>(st_src + (gu + 4 + gi) * kGroup + 8);
           }
         }
-      }
-      if (uu == 0) {  // codes of the next four groups
-#pragma unroll
-        for (int p = 0; p < NPROJ; ++p)
-#pragma unroll
-          for (int v = 0; v < 4; ++v) {
-            nxt[p][v] = cur[p][v];
-            if (g0 + 4 + v < ng) nxt[p][v] = *reinterpret_cast<const uint4*>(wrow[p] + (g0 + 4 + v) * 32);
-          }
       }
 #pragma unroll
       for (int gi = 0; gi < 2; ++gi) {
@@ -704,6 +696,9 @@ void qmm_kernel(const QmmArgs a) {
             tmp[0] = mfma_bf16(bx[0][s], av, tmp[0]);
             tmp[1] = mfma_bf16(bx[1][s], av, tmp[1]);
           }
+          // the register that held this group's codes takes those of the group four ahead
+          // (past the end the last group is read again: no branch inside the unrolled body)
+          cur[p][2 * uu + gi] = *reinterpret_cast<const uint4*>(wrow[p] + min(g + 4, ng - 1) * 32);
 #pragma unroll
           for (int nt = 0; nt < 2; ++nt)
 #pragma unroll
@@ -711,25 +706,25 @@ void qmm_kernel(const QmmArgs a) {
         }
       }
     }
-#pragma unroll
-    for (int p = 0; p < NPROJ; ++p)
-#pragma unroll
-      for (int v = 0; v < 4; ++v) cur[p][v] = nxt[p][v];
   }
 
   qmm_trace(a, work, 3);
   // ---- epilogue: the lane holds weight row row_base[p] + m for tokens 8j + 4h + i of each 32-token block
+  if (a.epi == 0) {
+    // SwiGLU, narrowed to bf16, transposed through the (now free) x ring so that a lane stores
+    // 16 bytes of one token: [token][32 rows] per wave, the rows of a run of 8 in the
+    // (0,4,1,5,2,6,3,7) order phase 2 reads, i.e. rows r and r + 4 share a 32-bit word.
+    __syncthreads();  // every wave is past its last read of the ring
+    uint32_t* so = reinterpret_cast<uint32_t*>(s_x) + wv * 1024;
+    const bool upper = (m >> 2) & 1u;
+    const uint32_t dw = ((m & ~7u) >> 1) + (m & 3u);  // word of the row pair (r, r + 4)
 #pragma unroll
-  for (int nt = 0; nt < 2; ++nt) {
+    for (int nt = 0; nt < 2; ++nt) {
 #pragma unroll
-    for (int j = 0; j < 4; ++j) {
-      const uint4 sl = *reinterpret_cast<const uint4*>(s_slot + nt * 32 + 8 * j + 4 * h);
-      const uint32_t slot[4] = {sl.x, sl.y, sl.z, sl.w};
+      for (int j = 0; j < 4; ++j) {
+        uint32_t bits[4];
 #pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        if (slot[i] == 0xFFFFFFFFu) continue;
-        const size_t at = static_cast<size_t>(slot[i]) * a.rows;
-        if (a.epi == 0) {
+        for (int i = 0; i < 4; ++i) {
           float gv = acc[0][nt][4 * j + i], uv = acc[NPROJ - 1][nt][4 * j + i];
           if (a.narrow) {
             gv = round_bf16(gv);
@@ -739,11 +734,42 @@ void qmm_kernel(const QmmArgs a) {
             gv = fminf(gv, a.limit);
             uv = fminf(fmaxf(uv, -a.limit), a.limit);
           }
-          // position of the row inside its run of 8 in the (0,4,1,5,2,6,3,7) order phase 2 reads
-          const uint32_t row = row_base[0] + m;
-          const uint32_t row_p = (row & ~7u) + ((row & 3u) << 1) + ((row >> 2) & 1u);
-          static_cast<uint16_t*>(a.out)[at + row_p] = f_to_bf16(mf_silu(gv) * uv);
-        } else {
+          bits[i] = f_to_bf16(fast_silu(gv) * uv);
+        }
+        // lanes m and m ^ 4 trade halves: the lower lane ends with tokens i = 0, 1 of both rows,
+        // the upper lane with tokens i = 2, 3
+        const uint32_t t01 = bits[0] | (bits[1] << 16), t23 = bits[2] | (bits[3] << 16);
+        const uint32_t keep = upper ? t23 : t01;
+        const uint32_t got = static_cast<uint32_t>(
+            __builtin_amdgcn_ds_swizzle(static_cast<int>(upper ? t01 : t23), 0x101F));  // lane ^ 4
+        const uint32_t lo_row = upper ? got : keep, hi_row = upper ? keep : got;
+        const uint32_t tok = nt * 32 + 8 * j + 4 * h + (upper ? 2u : 0u);
+        so[tok * 16 + dw] = __builtin_amdgcn_perm(hi_row, lo_row, 0x05040100u);
+        so[(tok + 1) * 16 + dw] = __builtin_amdgcn_perm(hi_row, lo_row, 0x07060302u);
+      }
+    }
+    __builtin_amdgcn_wave_barrier();  // the wave reads back only what it wrote itself
+    const uint32_t lane = threadIdx.x & 63u;
+#pragma unroll
+    for (int it = 0; it < 4; ++it) {
+      const uint32_t c = it * 64 + lane, tok = c >> 2, part = c & 3u;
+      const uint32_t sl = s_slot[tok];
+      const uint4 v = reinterpret_cast<const uint4*>(so)[c];
+      if (sl != 0xFFFFFFFFu)
+        *reinterpret_cast<uint4*>(static_cast<uint16_t*>(a.out) + static_cast<size_t>(sl) * a.rows + row_base[0] +
+                                  part * 8) = v;
+    }
+  } else {
+#pragma unroll
+    for (int nt = 0; nt < 2; ++nt) {
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const uint4 sl = *reinterpret_cast<const uint4*>(s_slot + nt * 32 + 8 * j + 4 * h);
+        const uint32_t slot[4] = {sl.x, sl.y, sl.z, sl.w};
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          if (slot[i] == 0xFFFFFFFFu) continue;
+          const size_t at = static_cast<size_t>(slot[i]) * a.rows;
 #pragma unroll
           for (int p = 0; p < NPROJ; ++p) {
             if (p > 0 && !a.pair_rows) break;

@@ -482,6 +482,184 @@ __global__ __launch_bounds__(KS * 64) void rows_mfma_kernel(const RowsMfmaArgs a
   }
 }
 
+// Quad form for 1..4 token rows of a wide 4-bit matrix.  v_mfma_f32_4x4x4_16b_bf16 multiplies
+// sixteen independent 4x4x4 blocks, one per quad of lanes.  Block b takes the K positions of the
+// 16-byte code chunks b, b + 16, ... of a row, so the lanes of a wave read 4 weight rows x 256
+// contiguous bytes per load, and the x values a lane meets never change: they stay in registers
+// as the A operand (lane (b, r) holds token r), pre-ordered for the code pairing of expand_q4,
+// next to their per-chunk sums.  The B operand is the chunk's codes of weight row c = lane % 4 as
+// the bf16 numbers 8 + q/2, so the result D[token, row] puts ONE weight row in a lane (its four
+// token sums in four registers) and the group's scale is a per-lane scalar:
+//   acc[t] += 2 s * (sum x (8 + q/2))            4 fma per chunk
+//   acc[t] += b * sum(x) - 16 s * sum(x)         two more matrix instructions per chunk (sum(x) as
+//                                                three bf16 terms: exact products)
+// Every token count 1..4 runs the same instructions on its own A rows: a token's result does
+// not depend on how many tokens ride along.  The waves of a workgroup split the chunks of a row
+// set (4 rows); partial sums meet in LDS in a fixed order.
+struct RowsQuadArgs {
+  const uint8_t* W[2];
+  const uint16_t* S[2];
+  const uint16_t* B[2];
+  const uint16_t* x;   // [T, N]
+  void* y;             // NPROJ 1: [T, M] bf16 or fp32; NPROJ 2: act [T, M] bf16
+  uint32_t M, N, T;    // M % 4 == 0, N % 64 == 0, T <= 4
+  int out_f32;
+};
+
+typedef __attribute__((ext_vector_type(4))) short s16x4_t;
+typedef __attribute__((ext_vector_type(4))) float f32x4_t;
+
+__device__ __forceinline__ f32x4_t mfma_quad(uint2 a, uint2 b, f32x4_t c) {
+  return __builtin_amdgcn_mfma_f32_4x4x4bf16_1k(__builtin_bit_cast(s16x4_t, a), __builtin_bit_cast(s16x4_t, b), c,
+                                                0, 0, 0);
+}
+
+constexpr uint32_t kQuadMaxWaves = 8;
+
+template <int NPROJ, int ITS>
+__global__ __launch_bounds__(kQuadMaxWaves * 64) void rows_quad_kernel(const RowsQuadArgs a) {
+  // partial sums [buffer][projection][wave][16-lane row][weight row][token]
+  __shared__ __attribute__((aligned(16))) float s_part[2][NPROJ][kQuadMaxWaves][4][4][4];
+  const uint32_t lane = threadIdx.x & 63, wsub = threadIdx.x >> 6, wpr = blockDim.x >> 6;
+  const uint32_t b = lane >> 2, c = lane & 3;
+  const uint32_t n_chunks = a.N / 32, ng = a.N / kGroup, n_sets = a.M / 4;
+  const size_t row_bytes = static_cast<size_t>(a.N) / 2;
+
+  // ---- this lane's x: token c, chunks (wsub * ITS + j) * 16 + b
+  uint32_t chc[ITS];
+  uint2 xa[ITS][8], sx[ITS];
+#pragma unroll
+  for (int j = 0; j < ITS; ++j) {
+    const uint32_t ch = (wsub * ITS + j) * 16 + b;
+    chc[j] = min(ch, n_chunks - 1);  // a slot past the row reads the last chunk against x = 0
+    const bool live = ch < n_chunks && c < a.T;
+    float sum = 0.0f;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      uint4 v = make_uint4(0, 0, 0, 0);
+      if (live) v = *reinterpret_cast<const uint4*>(a.x + static_cast<size_t>(c) * a.N + chc[j] * 32 + 8 * i);
+      xa[j][2 * i] = make_uint2(__builtin_amdgcn_perm(v.z, v.x, 0x05040100u),   // (e0, e4)
+                                __builtin_amdgcn_perm(v.z, v.x, 0x07060302u));  // (e1, e5)
+      xa[j][2 * i + 1] = make_uint2(__builtin_amdgcn_perm(v.w, v.y, 0x05040100u),   // (e2, e6)
+                                    __builtin_amdgcn_perm(v.w, v.y, 0x07060302u));  // (e3, e7)
+      const uint32_t pr[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+      for (int e = 0; e < 4; ++e) sum = (sum + bf16_lo(pr[e])) + bf16_hi(pr[e]);
+    }
+    const uint32_t hi = __float_as_uint(sum) & 0xFFFF0000u;
+    const float r1 = sum - __uint_as_float(hi);
+    const uint32_t mid = __float_as_uint(r1) & 0xFFFF0000u;
+    const uint32_t lo = __float_as_uint(r1 - __uint_as_float(mid));
+    sx[j] = make_uint2((hi >> 16) | mid, lo >> 16);  // K slots: hi, mid, lo, 0
+  }
+
+  uint4 cw[2][ITS];
+  uint32_t sc[2][ITS], bi[2][ITS];
+  auto issue = [&](int buf, uint32_t set, int p) __attribute__((always_inline)) {
+    const size_t row = static_cast<size_t>(set) * 4 + c;
+    const uint8_t* wrow = a.W[p] + row * row_bytes;
+    const uint16_t* srow = a.S[p] + row * ng;
+    const uint16_t* brow = a.B[p] + row * ng;
+#pragma unroll
+    for (int j = 0; j < ITS; ++j) {
+      cw[buf][j] = *reinterpret_cast<const uint4*>(wrow + static_cast<size_t>(chc[j]) * 16);
+      sc[buf][j] = srow[chc[j] >> 1];
+      bi[buf][j] = brow[chc[j] >> 1];
+    }
+  };
+  // the wave's part of D[token, row] for one row set; then the four blocks of each 16-lane row
+  // are added and lanes 0..3 of the row leave [weight row][token] in LDS
+  auto compute = [&](int buf, int p, uint32_t pb) __attribute__((always_inline)) {
+    f32x4_t acc = {0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+    for (int j = 0; j < ITS; ++j) {
+      const uint32_t w[4] = {cw[buf][j].x, cw[buf][j].y, cw[buf][j].z, cw[buf][j].w};
+      f32x4_t tmp = {0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const uint4 e = expand_q4(w[i]);
+        tmp = mfma_quad(xa[j][2 * i], make_uint2(e.x, e.y), tmp);
+        tmp = mfma_quad(xa[j][2 * i + 1], make_uint2(e.z, e.w), tmp);
+      }
+      const uint32_t sb = sc[buf][j], bb = bi[buf][j];
+      const uint32_t ms = ((sb + 0x0200u) ^ 0x8000u) & 0xFFFFu;  // -16 s: exponent + 4, sign flipped
+      acc = mfma_quad(sx[j], make_uint2(bb | (bb << 16), bb), acc);
+      acc = mfma_quad(sx[j], make_uint2(ms | (ms << 16), ms), acc);
+      const float s2 = 2.0f * __uint_as_float(sb << 16);
+#pragma unroll
+      for (int t = 0; t < 4; ++t) acc[t] = __builtin_fmaf(s2, tmp[t], acc[t]);
+    }
+    float v[4];
+#pragma unroll
+    for (int t = 0; t < 4; ++t) {
+      v[t] = acc[t] + dpp_f<0x124>(acc[t]);  // + lane - 4 (rotation inside the 16-lane row)
+      v[t] = v[t] + dpp_f<0x128>(v[t]);      // + lane - 8
+    }
+    if ((lane & 12u) == 0)
+      *reinterpret_cast<float4*>(&s_part[pb][p][wsub][lane >> 4][c][0]) = make_float4(v[0], v[1], v[2], v[3]);
+  };
+  // threads 0..15: (weight row, token) totals in wave then row order
+  auto combine = [&](uint32_t set, uint32_t pb) __attribute__((always_inline)) {
+    if (threadIdx.x >= 16) return;
+    const uint32_t cc = threadIdx.x & 3, t = threadIdx.x >> 2;
+    float v[NPROJ];
+#pragma unroll
+    for (int p = 0; p < NPROJ; ++p) {
+      v[p] = 0.0f;
+      for (uint32_t w = 0; w < wpr; ++w)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) v[p] = v[p] + s_part[pb][p][w][r][cc][t];
+    }
+    if (t >= a.T) return;
+    const size_t at = static_cast<size_t>(t) * a.M + set * 4 + cc;
+    if constexpr (NPROJ == 2) {
+      const float rg = round_bf16(v[0]), ru = round_bf16(v[1]);
+      static_cast<uint16_t*>(a.y)[at] = f_to_bf16(mf_silu(rg) * ru);
+    } else if (a.out_f32) {
+      static_cast<float*>(a.y)[at] = v[0];
+    } else {
+      static_cast<uint16_t*>(a.y)[at] = f_to_bf16(v[0]);
+    }
+  };
+
+  const uint32_t G = gridDim.x;
+  uint32_t set = blockIdx.x, pb = 0;
+  if (set >= n_sets) return;
+  issue(0, set, 0);
+  if constexpr (NPROJ == 2) {
+    for (;;) {
+      issue(1, set, 1);
+      compute(0, 0, pb);
+      const uint32_t nxt = set + G;
+      if (nxt < n_sets) issue(0, nxt, 0);
+      compute(1, 1, pb);
+      __syncthreads();  // the other buffer stays untouched until every wave has passed this point again
+      combine(set, pb);
+      pb ^= 1u;
+      if (nxt >= n_sets) break;
+      set = nxt;
+    }
+  } else {
+    for (;;) {
+      const uint32_t s1 = set + G;
+      if (s1 < n_sets) issue(1, s1, 0);
+      compute(0, 0, pb);
+      __syncthreads();
+      combine(set, pb);
+      pb ^= 1u;
+      if (s1 >= n_sets) break;
+      const uint32_t s2 = s1 + G;
+      if (s2 < n_sets) issue(0, s2, 0);
+      compute(1, 0, pb);
+      __syncthreads();
+      combine(s1, pb);
+      pb ^= 1u;
+      if (s2 >= n_sets) break;
+      set = s2;
+    }
+  }
+}
+
 // silu_mul_fp16 (utility.metal:21-33)
 __global__ void silu_mul_kernel(const uint16_t* gate, const uint16_t* up, uint16_t* out,
                                 uint32_t count) {
@@ -633,6 +811,31 @@ bool rows_mfma_try(hipStream_t s, const RowsMfmaArgs& a, uint32_t num_cu, hipErr
   return true;
 }
 
+// The quad kernel takes 4-bit matrices with at least 1024 rows (a multiple of 4) and up to 4
+// token rows when the 32-element chunks of a row split over (waves, ITS slots of 16 chunks)
+// with little waste.
+template <int NPROJ>
+bool rows_quad_try(hipStream_t s, const RowsQuadArgs& a, uint32_t num_cu, hipError_t& err) {
+  if (a.N % kGroup || a.T < 1 || a.T > 4 || a.M < 1024 || a.M % 4) return false;
+  const uint32_t chunks = a.N / 32;
+  uint32_t best_its = 0, best_wpr = 0, best_waste = ~0u;
+  for (uint32_t its = 6; its >= 4; --its) {
+    const uint32_t wpr = (chunks + 16 * its - 1) / (16 * its);
+    if (wpr > kQuadMaxWaves) continue;
+    const uint32_t waste = 16 * its * wpr - chunks;
+    if (waste < best_waste) { best_waste = waste; best_its = its; best_wpr = wpr; }
+  }
+  if (!best_its || best_waste * 10 > chunks) return false;
+  const uint32_t n_sets = a.M / 4;
+  const uint32_t grid = std::min<uint32_t>(n_sets, num_cu * std::max(1u, 8u / best_wpr));
+  const dim3 block(best_wpr * 64);
+  if (best_its == 4) rows_quad_kernel<NPROJ, 4><<<dim3(grid), block, 0, s>>>(a);
+  else if (best_its == 5) rows_quad_kernel<NPROJ, 5><<<dim3(grid), block, 0, s>>>(a);
+  else rows_quad_kernel<NPROJ, 6><<<dim3(grid), block, 0, s>>>(a);
+  err = hipGetLastError();
+  return true;
+}
+
 }  // namespace
 
 hipError_t launch_gemv(hipStream_t s, const mf_qtensor& w, int bits, const uint16_t* x, void* y,
@@ -643,6 +846,10 @@ hipError_t launch_gemv(hipStream_t s, const mf_qtensor& w, int bits, const uint1
     ma.W[0] = static_cast<const uint8_t*>(w.weights); ma.S[0] = w.scales; ma.B[0] = w.biases;
     ma.x = x; ma.y = y; ma.M = m; ma.N = n; ma.T = t; ma.out_f32 = out_f32 ? 1 : 0;
     hipError_t err = hipSuccess;
+    RowsQuadArgs qa{};
+    qa.W[0] = ma.W[0]; qa.S[0] = ma.S[0]; qa.B[0] = ma.B[0];
+    qa.x = x; qa.y = y; qa.M = m; qa.N = n; qa.T = t; qa.out_f32 = ma.out_f32;
+    if (rows_quad_try<1>(s, qa, device_cu_count(), err)) return err;
     if (rows_mfma_try<1>(s, ma, device_cu_count(), err)) return err;
   }
   if (al && (bits == kBits4 || bits == kBits2)) {
@@ -679,6 +886,10 @@ hipError_t launch_gate_up_act(hipStream_t s, const mf_qtensor& gate, const mf_qt
     ma.W[1] = static_cast<const uint8_t*>(up.weights); ma.S[1] = up.scales; ma.B[1] = up.biases;
     ma.x = x; ma.y = act; ma.M = f; ma.N = d; ma.T = t;
     hipError_t err = hipSuccess;
+    RowsQuadArgs qa{};
+    for (int p = 0; p < 2; ++p) { qa.W[p] = ma.W[p]; qa.S[p] = ma.S[p]; qa.B[p] = ma.B[p]; }
+    qa.x = x; qa.y = act; qa.M = f; qa.N = d; qa.T = t;
+    if (rows_quad_try<2>(s, qa, device_cu_count(), err)) return err;
     if (rows_mfma_try<2>(s, ma, device_cu_count(), err)) return err;
   }
   if (al && (bits == kBits4 || bits == kBits2)) {

@@ -244,12 +244,24 @@ constexpr uint32_t kMagic8 = 0x41004100u;    // bf16 pair (8.0, 8.0)
 constexpr uint32_t kMagic4 = 0x40804080u;    // bf16 pair (4.0, 4.0)
 constexpr uint32_t kOnes = 0x3F803F80u;      // bf16 pair (1.0, 1.0)
 
-// (v & mask) | magic in one instruction; the mask rides in a scalar register, the magic in a
-// vector register (a VOP3 instruction of this ISA takes one scalar source and no literal)
-__device__ __forceinline__ uint32_t and_or(uint32_t v, uint32_t mask, uint32_t magic) {
+// (v & mask) | magic in one instruction (v_and_or_b32).  A VOP3 instruction of this ISA takes
+// one scalar source and no literal, so the mask has to sit in a scalar register and the magic in
+// a vector register; the two empty asm statements only pin the constants there (they are pure,
+// so the compiler hoists them out of loops) and the and-or itself stays an ordinary instruction
+// the compiler schedules and guards: written as inline asm it would escape the hazard checks
+// between a matrix instruction that still reads an operand and the next write of that register.
+__device__ __forceinline__ uint32_t pin_sgpr(uint32_t x) {
   uint32_t r;
-  asm("v_and_or_b32 %0, %1, %2, %3" : "=v"(r) : "v"(v), "s"(mask), "v"(magic));
+  asm("" : "=s"(r) : "0"(x));
   return r;
+}
+__device__ __forceinline__ uint32_t pin_vgpr(uint32_t x) {
+  uint32_t r;
+  asm("" : "=v"(r) : "0"(x));
+  return r;
+}
+__device__ __forceinline__ uint32_t and_or(uint32_t v, uint32_t mask, uint32_t magic) {
+  return (v & pin_sgpr(mask)) | pin_vgpr(magic);
 }
 
 // ---- matrix-core forms of the same embedding

@@ -520,6 +520,8 @@ template <int NPROJ, int ITS>
 __global__ __launch_bounds__(kQuadMaxWaves * 64) void rows_quad_kernel(const RowsQuadArgs a) {
   // partial sums [buffer][projection][wave][16-lane row][weight row][token]
   __shared__ __attribute__((aligned(16))) float s_part[2][NPROJ][kQuadMaxWaves][4][4][4];
+  // scale / bias pieces [wave][ring slot][(table, row, piece)][8 groups]
+  __shared__ __attribute__((aligned(16))) uint16_t s_tab[kQuadMaxWaves][2][64 * 8];
   const uint32_t lane = threadIdx.x & 63, wsub = threadIdx.x >> 6, wpr = blockDim.x >> 6;
   const uint32_t b = lane >> 2, c = lane & 3;
   const uint32_t n_chunks = a.N / 32, ng = a.N / kGroup, n_sets = a.M / 4;
@@ -553,24 +555,44 @@ __global__ __launch_bounds__(kQuadMaxWaves * 64) void rows_quad_kernel(const Row
     sx[j] = make_uint2((hi >> 16) | mid, lo >> 16);  // K slots: hi, mid, lo, 0
   }
 
+  // Codes and table entries of two stages (a stage = one projection of one row set) live in a
+  // ring of registers: a slot is refilled, as soon as it has been used, with the same slot of
+  // the stage two ahead, so between one and two stages of loads are in flight all the time.
+  // The scales and biases a wave needs for one stage are 8 * ITS consecutive groups of each of its
+  // 4 rows: lanes 0 .. 8 * ITS - 1 fetch them as 16-byte pieces ((table, row, piece) per lane) in
+  // ONE load instruction issued with the first refill of the stage that frees the ring slot; the
+  // piece goes to the wave's own LDS area when that stage ends, and a lane picks the two values of
+  // each slot from there (LDS reads cost no vector-memory issue slot,
+  // which is what limits this kernel).
   uint4 cw[2][ITS];
-  uint32_t sc[2][ITS], bi[2][ITS];
-  auto issue = [&](int buf, uint32_t set, int p) __attribute__((always_inline)) {
+  // (lanes past 8 * ITS fetch and store a copy nobody reads: no branch around the load)
+  const uint32_t tb_lane = lane % (8 * ITS);
+  const uint32_t tb_bias = tb_lane / (4 * ITS), tb_row = (tb_lane / ITS) & 3u, tb_piece = tb_lane % ITS;
+  const uint32_t tb_g = (wsub * ITS + tb_piece) * 8;
+  const uint32_t tb_group = tb_g < ng ? tb_g : 0u;  // a piece past the row is never used: read piece 0
+  uint16_t* my_tab = &s_tab[wsub][0][0];
+  auto fetch = [&](int buf, int j, uint32_t set, int p) __attribute__((always_inline)) {
     const size_t row = static_cast<size_t>(set) * 4 + c;
-    const uint8_t* wrow = a.W[p] + row * row_bytes;
-    const uint16_t* srow = a.S[p] + row * ng;
-    const uint16_t* brow = a.B[p] + row * ng;
+    cw[buf][j] = *reinterpret_cast<const uint4*>(a.W[p] + row * row_bytes + static_cast<size_t>(chc[j]) * 16);
+  };
+  auto fetch_tables = [&](uint32_t set, int p) __attribute__((always_inline)) {
+    return *reinterpret_cast<const uint4*>((tb_bias ? a.B[p] : a.S[p]) + (static_cast<size_t>(set) * 4 + tb_row) * ng +
+                                           tb_group);
+  };
+  auto issue = [&](int buf, uint32_t set, int p) __attribute__((always_inline)) {
+    const uint4 t = fetch_tables(set, p);
 #pragma unroll
-    for (int j = 0; j < ITS; ++j) {
-      cw[buf][j] = *reinterpret_cast<const uint4*>(wrow + static_cast<size_t>(chc[j]) * 16);
-      sc[buf][j] = srow[chc[j] >> 1];
-      bi[buf][j] = brow[chc[j] >> 1];
-    }
+    for (int j = 0; j < ITS; ++j) fetch(buf, j, set, p);
+    *reinterpret_cast<uint4*>(my_tab + buf * (64 * 8) + lane * 8) = t;
   };
   // the wave's part of D[token, row] for one row set; then the four blocks of each 16-lane row
-  // are added and lanes 0..3 of the row leave [weight row][token] in LDS
-  auto compute = [&](int buf, int p, uint32_t pb) __attribute__((always_inline)) {
+  // are added and lanes 0..3 of the row leave [weight row][token] in LDS.  `refill` is the row
+  // set whose stage takes over the ring slots.
+  auto compute = [&](int buf, int p, uint32_t pb, uint32_t refill) __attribute__((always_inline)) {
     f32x4_t acc = {0.0f, 0.0f, 0.0f, 0.0f};
+    uint16_t* tab = my_tab + buf * (64 * 8);
+    __builtin_amdgcn_wave_barrier();  // the wave reads back what its own lanes wrote (LDS keeps order)
+    uint4 tbn = make_uint4(0, 0, 0, 0);
 #pragma unroll
     for (int j = 0; j < ITS; ++j) {
       const uint32_t w[4] = {cw[buf][j].x, cw[buf][j].y, cw[buf][j].z, cw[buf][j].w};
@@ -581,14 +603,19 @@ __global__ __launch_bounds__(kQuadMaxWaves * 64) void rows_quad_kernel(const Row
         tmp = mfma_quad(xa[j][2 * i], make_uint2(e.x, e.y), tmp);
         tmp = mfma_quad(xa[j][2 * i + 1], make_uint2(e.z, e.w), tmp);
       }
-      const uint32_t sb = sc[buf][j], bb = bi[buf][j];
+      const uint32_t sb = tab[((c * ITS) + j) * 8 + (b >> 1)], bb = tab[(((4 + c) * ITS) + j) * 8 + (b >> 1)];
       const uint32_t ms = ((sb + 0x0200u) ^ 0x8000u) & 0xFFFFu;  // -16 s: exponent + 4, sign flipped
       acc = mfma_quad(sx[j], make_uint2(bb | (bb << 16), bb), acc);
       acc = mfma_quad(sx[j], make_uint2(ms | (ms << 16), ms), acc);
       const float s2 = 2.0f * __uint_as_float(sb << 16);
+      fetch(buf, j, refill, p);
+      if (j == 0) tbn = fetch_tables(refill, p);
 #pragma unroll
       for (int t = 0; t < 4; ++t) acc[t] = __builtin_fmaf(s2, tmp[t], acc[t]);
     }
+    // every read of this ring slot's tables is issued: the refill stage's pieces take their place
+    __builtin_amdgcn_wave_barrier();
+    *reinterpret_cast<uint4*>(tab + lane * 8) = tbn;
     float v[4];
 #pragma unroll
     for (int t = 0; t < 4; ++t) {
@@ -622,40 +649,38 @@ __global__ __launch_bounds__(kQuadMaxWaves * 64) void rows_quad_kernel(const Row
     }
   };
 
-  const uint32_t G = gridDim.x;
+  // Refills past the last row set read the last row set again (loaded, never used): no branch
+  // splits the unrolled stage.
+  const uint32_t G = gridDim.x, last = n_sets - 1;
   uint32_t set = blockIdx.x, pb = 0;
   if (set >= n_sets) return;
-  issue(0, set, 0);
   if constexpr (NPROJ == 2) {
-    for (;;) {
-      issue(1, set, 1);
-      compute(0, 0, pb);
-      const uint32_t nxt = set + G;
-      if (nxt < n_sets) issue(0, nxt, 0);
-      compute(1, 1, pb);
+    issue(0, set, 0);
+    issue(1, set, 1);
+    for (; set < n_sets; set += G) {
+      const uint32_t nxt = min(set + G, last);
+      compute(0, 0, pb, nxt);
+      compute(1, 1, pb, nxt);
       __syncthreads();  // the other buffer stays untouched until every wave has passed this point again
       combine(set, pb);
       pb ^= 1u;
-      if (nxt >= n_sets) break;
-      set = nxt;
     }
   } else {
+    issue(0, set, 0);
+    issue(1, min(set + G, last), 0);
     for (;;) {
-      const uint32_t s1 = set + G;
-      if (s1 < n_sets) issue(1, s1, 0);
-      compute(0, 0, pb);
+      compute(0, 0, pb, min(set + 2 * G, last));
       __syncthreads();
       combine(set, pb);
       pb ^= 1u;
+      const uint32_t s1 = set + G;
       if (s1 >= n_sets) break;
-      const uint32_t s2 = s1 + G;
-      if (s2 < n_sets) issue(0, s2, 0);
-      compute(1, 0, pb);
+      compute(1, 0, pb, min(s1 + 2 * G, last));
       __syncthreads();
       combine(s1, pb);
       pb ^= 1u;
-      if (s2 >= n_sets) break;
-      set = s2;
+      set = s1 + G;
+      if (set >= n_sets) break;
     }
   }
 }
@@ -816,7 +841,7 @@ bool rows_mfma_try(hipStream_t s, const RowsMfmaArgs& a, uint32_t num_cu, hipErr
 // with little waste.
 template <int NPROJ>
 bool rows_quad_try(hipStream_t s, const RowsQuadArgs& a, uint32_t num_cu, hipError_t& err) {
-  if (a.N % kGroup || a.T < 1 || a.T > 4 || a.M < 1024 || a.M % 4) return false;
+  if (a.N % (8 * kGroup) || a.T < 1 || a.T > 4 || a.M < 1024 || a.M % 4) return false;
   const uint32_t chunks = a.N / 32;
   uint32_t best_its = 0, best_wpr = 0, best_waste = ~0u;
   for (uint32_t its = 6; its >= 4; --its) {

@@ -118,6 +118,43 @@ def test_gemv_streaming_rows_kernel(gpu, oracle, bits, m, n, t):
         assert np.abs(yi.cpu().numpy()[0] - got[0]).max() / max(np.abs(ref).max(), 1e-6) < 2e-6
 
 
+@pytest.mark.parametrize("m,n,t", [
+    (1024, 2048, 3),    # one wave per row set, four slots
+    (1100, 5120, 4),    # two waves per row set, five slots; 275 row sets
+    (1280, 17408, 2),   # seven waves per row set, ragged last slot; workgroups walk several row sets
+    (2048, 4096, 1),
+])
+def test_gemv_quad_rows_kernel(gpu, oracle, m, n, t):
+    """4-bit matrices with K a multiple of 512 and up to 4 token rows take the quad matrix-core
+    kernel: every token count runs the same instructions, so a token's row does not depend on how
+    many tokens ride along (MultiXKernelParityTests.swift:50-77), bit for bit"""
+    rng = oracle.Rng.key(0xF5, f"quad-{m}-{n}-{t}")
+    q = oracle.quantize(rng.uniform_fill(-1.0, 1.0, m * n).reshape(m, n), 4)
+    x = oracle.bf16_bits(rng.uniform_fill(-1.0, 1.0, t * n).reshape(t, n))
+    ref = oracle.gemv_multix(q, x)
+    xd = ops.bf16_tensor(x)
+    g = ops.DequantInt4GEMVMultiX(gpu)
+    dq = to_device_q(q)
+    y32 = torch.full((t, m), 7.0, dtype=torch.float32, device="cuda")
+    y16 = torch.zeros((t, m), dtype=torch.bfloat16, device="cuda")
+    g.encode(dq, xd, y32, m, n, t, output_float32=True)
+    g.encode(dq, xd, y16, m, n, t)
+    _sync()
+    got = y32.cpu().numpy()
+    assert np.abs(got - ref).max() / max(np.abs(ref).max(), 1e-6) < 2e-5
+    assert np.array_equal(ops.bf16_bits(y16), oracle.bf16_bits(got))
+    for i in range(t):
+        yi = torch.zeros((1, m), dtype=torch.float32, device="cuda")
+        g.encode(dq, xd[i:i + 1].contiguous(), yi, m, n, 1, output_float32=True)
+        _sync()
+        assert np.array_equal(yi.cpu().numpy()[0].view(np.uint32), got[i].view(np.uint32))
+    # twice the same launch: the partial sums meet in a fixed order
+    y2 = torch.zeros((t, m), dtype=torch.float32, device="cuda")
+    g.encode(dq, xd, y2, m, n, t, output_float32=True)
+    _sync()
+    assert np.array_equal(y2.cpu().numpy().view(np.uint32), got.view(np.uint32))
+
+
 @pytest.mark.parametrize("d,f,t", [(2048, 1024, 1), (5120, 1536, 4)])
 def test_shared_expert_streaming_rows_kernel(gpu, oracle, d, f, t):
     """dense SwiGLU MLP wide enough for the streaming gate/up and down kernels"""

@@ -443,19 +443,31 @@ __device__ __forceinline__ float fast_silu(float x) {
 // kernel fits 168 registers and three waves stay resident.
 // LDS (dynamic): x tile ring, 2 stages x 2 K groups x [2 nt][4 s][2 h][32 n] x 16 B,
 // scale tables [NPROJ][4 waves][ng][32 rows] fp32, out slots [64] u32.
+// One launch can carry two independent problems of the same instantiation (the routed experts
+// and the shared expert of the same phase): the second problem's work items follow the first's
+// on every XCD, so they fill the slots the first problem's last round leaves empty instead of
+// running as a launch of their own that covers a quarter of the chip.
+struct QmmLaunch {
+  QmmArgs part[2];
+  uint32_t per_xcd[2];  // work items of each part on one XCD (grid = 8 * their sum)
+};
+
 template <int NPROJ, bool NG8>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(NPROJ == 1 ? 3 : 2, NPROJ == 1 ? 3 : 2)))
-void qmm_kernel(const QmmArgs a) {
+void qmm_kernel(const QmmLaunch launch) {
   extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
   const uint32_t lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
   const uint32_t m = lane & 31, h = lane >> 5;
-  const uint32_t wave_rows = a.pair_rows ? 32u * NPROJ : 32u;  // weight rows of one wave
-  const uint32_t n_slices = a.rows / (kQmmWaves * wave_rows);
   // Workgroups go to the 8 XCDs round-robin by blockIdx; consecutive work items (the row slices of
   // one tile share its x rows, the tiles of one expert share its weights) are laid on ONE XCD so
-  // that its L2 serves the re-reads.  The grid is a multiple of 8; the tile list is laid out by
-  // group_scan_kernel so that every eighth of it holds an eighth of the live tiles.
-  const uint32_t work = (blockIdx.x & 7u) * (gridDim.x >> 3) + (blockIdx.x >> 3);
+  // that its L2 serves the re-reads.  The tile list is laid out by group_scan_kernel so that every
+  // eighth of it holds an eighth of the live tiles.
+  const uint32_t xcd_slot = blockIdx.x >> 3;
+  const bool second = xcd_slot >= launch.per_xcd[0];
+  const QmmArgs& a = launch.part[second ? 1 : 0];
+  const uint32_t work = (blockIdx.x & 7u) * launch.per_xcd[second ? 1 : 0] + (xcd_slot - (second ? launch.per_xcd[0] : 0u));
+  const uint32_t wave_rows = a.pair_rows ? 32u * NPROJ : 32u;  // weight rows of one wave
+  const uint32_t n_slices = a.rows / (kQmmWaves * wave_rows);
   const uint32_t tile_id = work / n_slices, slice = work % n_slices;
   const uint32_t ng = a.kdim / kGroup;
   qmm_trace(a, work, 0);
@@ -873,17 +885,28 @@ hipError_t launch_prep_rows(hipStream_t s, const uint16_t* src, uint16_t* dst, f
   return hipGetLastError();
 }
 
-// tile_slots: entries of the tile list (routed; a multiple of 8) or number of 64-row tiles (dense)
-hipError_t launch_qmm(hipStream_t s, QmmArgs a, int nproj, uint32_t tile_slots) {
-  const size_t lds = qmm_lds_bytes(a.kdim, nproj);
-  const uint32_t n_slices = a.rows / (kQmmRows * (a.pair_rows ? nproj : 1));
-  if (a.dense_mode) {
-    a.dense_tiles = tile_slots;
-    tile_slots = (tile_slots + 7) / 8 * 8;
+// tile_slots: entries of the tile list (routed; a multiple of 8) or number of 64-row tiles (dense).
+// `b` (optional) is a second problem for the same instantiation, run behind `a` in the same launch.
+hipError_t launch_qmm(hipStream_t s, QmmArgs a, int nproj, uint32_t tile_slots, const QmmArgs* b,
+                      uint32_t b_tile_slots) {
+  QmmLaunch launch{};
+  size_t lds = 0;
+  bool ng8 = true;
+  for (int part = 0; part < (b ? 2 : 1); ++part) {
+    QmmArgs& q = launch.part[part];
+    q = part ? *b : a;
+    uint32_t slots = part ? b_tile_slots : tile_slots;
+    const uint32_t n_slices = q.rows / (kQmmRows * (q.pair_rows ? nproj : 1));
+    if (q.dense_mode) {
+      q.dense_tiles = slots;
+      slots = (slots + 7) / 8 * 8;
+    }
+    launch.per_xcd[part] = slots / 8 * n_slices;
+    lds = std::max(lds, qmm_lds_bytes(q.kdim, nproj));
+    ng8 = ng8 && (q.kdim / kGroup) % 8 == 0;
   }
-  const dim3 grid(tile_slots * n_slices), block(256);
+  const dim3 grid(8 * (launch.per_xcd[0] + launch.per_xcd[1])), block(256);
   if (grid.x == 0) return hipSuccess;
-  const bool ng8 = (a.kdim / kGroup) % 8 == 0;
   const void* fn = nproj == 2 ? (ng8 ? reinterpret_cast<const void*>(qmm_kernel<2, true>)
                                      : reinterpret_cast<const void*>(qmm_kernel<2, false>))
                               : (ng8 ? reinterpret_cast<const void*>(qmm_kernel<1, true>)
@@ -893,11 +916,11 @@ hipError_t launch_qmm(hipStream_t s, QmmArgs a, int nproj, uint32_t tile_slots) 
     if (e != hipSuccess) return e;
   }
   if (nproj == 2) {
-    if (ng8) qmm_kernel<2, true><<<grid, block, lds, s>>>(a);
-    else qmm_kernel<2, false><<<grid, block, lds, s>>>(a);
+    if (ng8) qmm_kernel<2, true><<<grid, block, lds, s>>>(launch);
+    else qmm_kernel<2, false><<<grid, block, lds, s>>>(launch);
   } else {
-    if (ng8) qmm_kernel<1, true><<<grid, block, lds, s>>>(a);
-    else qmm_kernel<1, false><<<grid, block, lds, s>>>(a);
+    if (ng8) qmm_kernel<1, true><<<grid, block, lds, s>>>(launch);
+    else qmm_kernel<1, false><<<grid, block, lds, s>>>(launch);
   }
   return hipGetLastError();
 }
@@ -994,35 +1017,38 @@ hipError_t launch_prefill_layer(hipStream_t s, const mf_moe& h, const mf_moe_lay
     q.trace = h.trace;
     q.trace_items = static_cast<uint32_t>(std::min<size_t>(h.trace_bytes / 64, 1u << 30));
   }
-  // routed phase 1: gate/up -> acts [pair, F]
+  // The shared expert's two matmuls ride in the routed launches of the same phase.
+  QmmArgs d{};
+  const uint32_t dense_tiles = c.shared_f ? (t + kTileTokens - 1) / kTileTokens : 0;
+  if (c.shared_f) {
+    d.dense_mode = 1; d.dense_rows = t; d.top_k = c.top_k; d.narrow = 1;
+    d.dense[0] = w.shared_gate; d.dense[1] = w.shared_up;
+    d.x = ws.xp; d.sumx = ws.sum_x; d.x_stride = c.d; d.rows = c.shared_f; d.kdim = c.d; d.epi = 0; d.out = ws.sact;
+  }
+  // phase 1: routed gate/up -> acts [pair, F]; shared gate/up -> sact [token, Fs]
   q.w_off[0] = w.offsets.gate_w; q.s_off[0] = w.offsets.gate_s; q.b_off[0] = w.offsets.gate_b;
   q.w_off[1] = w.offsets.up_w; q.s_off[1] = w.offsets.up_s; q.b_off[1] = w.offsets.up_b;
   q.x = ws.xp; q.sumx = ws.sum_x; q.x_stride = c.d; q.gather = 1; q.rows = c.f; q.kdim = c.d; q.epi = 0;
   q.out = ws.acts;
-  MF_TRY(launch_qmm(s, q, 2, max_tiles));
+  MF_TRY(launch_qmm(s, q, 2, max_tiles, c.shared_f ? &d : nullptr, dense_tiles));
   // routes past the last tile's count were never written: only pairs rows exist, all written
   MF_TRY(launch_prep_rows(s, ws.acts, nullptr, ws.sum_acts, pairs * c.f));
-  // routed phase 2: down -> fp32 partials [token*K+rank, D]
+  if (c.shared_f) MF_TRY(launch_prep_rows(s, ws.sact, nullptr, ws.sum_sact, static_cast<size_t>(t) * c.shared_f));
+  // phase 2: routed down -> fp32 partials [token*K+rank, D]; shared down -> hs [token, D]
   q.w_off[0] = w.offsets.down_w; q.s_off[0] = w.offsets.down_s; q.b_off[0] = w.offsets.down_b;
   q.x = ws.acts; q.sumx = ws.sum_acts; q.x_stride = c.f; q.gather = 0; q.rows = c.d; q.kdim = c.f; q.epi = 1; q.out = ws.partials;
   q.limit = 0.0f;
   q.trace = nullptr;
   q.pair_rows = c.d % (2 * kQmmRows) == 0;
-  MF_TRY(launch_qmm(s, q, q.pair_rows ? 2 : 1, max_tiles));
+  if (c.shared_f) {
+    d.dense[0] = w.shared_down;
+    d.x = ws.sact; d.sumx = ws.sum_sact; d.x_stride = c.shared_f; d.rows = c.d; d.kdim = c.shared_f; d.epi = 2; d.out = ws.hs;
+    d.pair_rows = q.pair_rows;
+  }
+  MF_TRY(launch_qmm(s, q, q.pair_rows ? 2 : 1, max_tiles, c.shared_f ? &d : nullptr, dense_tiles));
   const uint16_t* hs = nullptr;
   const uint16_t* gate = nullptr;
   if (c.shared_f) {
-    QmmArgs d{};
-    d.dense_mode = 1; d.dense_rows = t; d.top_k = c.top_k; d.narrow = 1;
-    d.dense[0] = w.shared_gate; d.dense[1] = w.shared_up;
-    d.x = ws.xp; d.sumx = ws.sum_x; d.x_stride = c.d; d.rows = c.shared_f; d.kdim = c.d; d.epi = 0; d.out = ws.sact;
-    const uint32_t dense_tiles = (t + kTileTokens - 1) / kTileTokens;
-    MF_TRY(launch_qmm(s, d, 2, dense_tiles));
-    MF_TRY(launch_prep_rows(s, ws.sact, nullptr, ws.sum_sact, static_cast<size_t>(t) * c.shared_f));
-    d.dense[0] = w.shared_down;
-    d.x = ws.sact; d.sumx = ws.sum_sact; d.x_stride = c.shared_f; d.rows = c.d; d.kdim = c.shared_f; d.epi = 2; d.out = ws.hs;
-    d.pair_rows = c.d % (2 * kQmmRows) == 0;
-    MF_TRY(launch_qmm(s, d, d.pair_rows ? 2 : 1, dense_tiles));
     hs = ws.hs;
     if (w.w_sg) {
       MF_TRY(launch_router_logits(s, w.w_sg, x, 1, c.d, t, c.d, nullptr, ws.gate));

@@ -225,7 +225,7 @@ __global__ __launch_bounds__(256) void group_count_kernel(const uint32_t* __rest
                                                           uint32_t n_pairs, uint32_t E,
                                                           uint32_t chunk_pairs,
                                                           uint32_t* __restrict__ chunk_hist,
-                                                          uint32_t* __restrict__ status) {
+                                                          uint32_t* __restrict__ chunk_bad) {
   __shared__ uint32_t s_hist[MF_MAX_EXPERTS];
   for (uint32_t e = threadIdx.x; e < E; e += blockDim.x) s_hist[e] = 0;
   __syncthreads();
@@ -236,8 +236,9 @@ __global__ __launch_bounds__(256) void group_count_kernel(const uint32_t* __rest
     if (e < E) atomicAdd(&s_hist[e], 1u);
     else bad = true;
   }
-  if (__any(bad) && (threadIdx.x & 63) == 0) atomicOr(status, 2u);
-  __syncthreads();
+  // one flag per chunk, always written: nothing has to be cleared before the launch
+  const int any_bad = __syncthreads_or(bad ? 1 : 0);
+  if (threadIdx.x == 0) chunk_bad[blockIdx.x] = any_bad ? 1u : 0u;
   for (uint32_t e = threadIdx.x; e < E; e += blockDim.x) chunk_hist[blockIdx.x * E + e] = s_hist[e];
 }
 
@@ -251,9 +252,15 @@ __global__ __launch_bounds__(512) void group_scan_kernel(uint32_t* __restrict__ 
                                                          uint32_t* __restrict__ starts,
                                                          Tile* __restrict__ tiles,
                                                          uint32_t tile_slots,
-                                                         uint32_t* __restrict__ n_tiles) {
+                                                         uint32_t* __restrict__ n_tiles,
+                                                         const uint32_t* __restrict__ chunk_bad,
+                                                         uint32_t* __restrict__ status) {
   __shared__ uint32_t s_cnt[MF_MAX_EXPERTS], s_tile[MF_MAX_EXPERTS];
   const uint32_t e = threadIdx.x;
+  {  // status word: 2 when any chunk met an expert index out of range (n_chunks <= blockDim)
+    const int any_bad = __syncthreads_or(e < n_chunks && chunk_bad[e] ? 1 : 0);
+    if (e == 0) *status = any_bad ? 2u : 0u;
+  }
   uint32_t c = 0;
   if (e < E) {
     uint32_t k = 0;
@@ -365,21 +372,27 @@ __global__ __launch_bounds__(256) void group_emit_kernel(const uint32_t* __restr
   }
 }
 
-__global__ void zero_words_kernel(uint32_t* p, uint32_t n) {
-  const uint32_t i = blockIdx.x * blockDim.x + threadIdx.x;
-  if (i < n) p[i] = 0;
-}
-
 // --------------------------------------------------------------- the matmul
 
 // Activation rows as the matmul wants them: inside every run of 8 K values the
 // order is (0,4,1,5,2,6,3,7) -- the pairing a packed code word expands to --
 // and the fp32 sum of every 64-wide K group is kept beside them.  One lane per
 // run of 8; `dst` may be null when `src` is already in that order.
-__global__ __launch_bounds__(256) void prep_rows_kernel(const uint16_t* __restrict__ src,
-                                                        uint16_t* __restrict__ dst,
-                                                        float* __restrict__ sums, uint32_t chunks) {
-  const uint32_t c = blockIdx.x * blockDim.x + threadIdx.x;
+struct PrepArgs {  // up to two row sets per launch: the second starts at workgroup `blocks0`
+  const uint16_t* src[2];
+  uint16_t* dst[2];
+  float* sums[2];
+  uint32_t chunks[2];
+  uint32_t blocks0;
+};
+
+__global__ __launch_bounds__(256) void prep_rows_kernel(const PrepArgs a) {
+  const int part = blockIdx.x >= a.blocks0 ? 1 : 0;
+  const uint16_t* src = a.src[part];
+  uint16_t* dst = a.dst[part];
+  float* sums = a.sums[part];
+  const uint32_t chunks = a.chunks[part];
+  const uint32_t c = (blockIdx.x - (part ? a.blocks0 : 0u)) * blockDim.x + threadIdx.x;
   uint4 v = make_uint4(0, 0, 0, 0);
   if (c < chunks) v = *reinterpret_cast<const uint4*>(src + static_cast<size_t>(c) * 8);
   float sum = ((bf16_lo(v.x) + bf16_hi(v.x)) + (bf16_lo(v.y) + bf16_hi(v.y))) +
@@ -862,26 +875,33 @@ hipError_t launch_group(hipStream_t s, const uint32_t* idx, const float* w, uint
   const uint32_t steps = (n_pairs + kGroupBlock - 1) / kGroupBlock;
   const uint32_t chunk_pairs = (steps + kGroupChunks - 1) / kGroupChunks * kGroupBlock;
   const uint32_t n_chunks = (n_pairs + chunk_pairs - 1) / chunk_pairs;
-  zero_words_kernel<<<dim3(1), dim3(64), 0, s>>>(status, 1);  // a fill kernel: safe under graph capture
-  group_count_kernel<<<dim3(n_chunks), dim3(256), 0, s>>>(idx, n_pairs, E, chunk_pairs, chunk_hist, status);
+  uint32_t* chunk_bad = chunk_hist + static_cast<size_t>(kGroupChunks) * MF_MAX_EXPERTS;
+  group_count_kernel<<<dim3(n_chunks), dim3(256), 0, s>>>(idx, n_pairs, E, chunk_pairs, chunk_hist, chunk_bad);
   group_scan_kernel<<<dim3(1), dim3(MF_MAX_EXPERTS), 0, s>>>(chunk_hist, n_chunks, E, counts, offsets, starts,
-                                                             static_cast<Tile*>(tiles), tile_slots, n_tiles);
+                                                             static_cast<Tile*>(tiles), tile_slots, n_tiles,
+                                                             chunk_bad, status);
   group_emit_kernel<<<dim3(n_chunks), dim3(256), 0, s>>>(idx, w, n_pairs, K, E, chunk_pairs, chunk_hist, starts,
                                                          sorted);
   return hipGetLastError();
 }
 
-size_t group_scratch_words() { return 2048 + static_cast<size_t>(kGroupChunks) * MF_MAX_EXPERTS; }
+size_t group_scratch_words() { return 2048 + static_cast<size_t>(kGroupChunks) * MF_MAX_EXPERTS + kGroupChunks; }
 
 size_t qmm_lds_bytes(uint32_t kdim, int nproj) {
   const uint32_t ng = kdim / kGroup;
   return kQmmXBytes + static_cast<size_t>(nproj) * kQmmWaves * ng * 32 * 4 + kTileTokens * 4;
 }
 
-hipError_t launch_prep_rows(hipStream_t s, const uint16_t* src, uint16_t* dst, float* sums, size_t elems) {
-  const uint32_t chunks = static_cast<uint32_t>(elems / 8);
-  if (!chunks) return hipSuccess;
-  prep_rows_kernel<<<dim3((chunks + 255) / 256), dim3(256), 0, s>>>(src, dst, sums, chunks);
+hipError_t launch_prep_rows(hipStream_t s, const uint16_t* src, uint16_t* dst, float* sums, size_t elems,
+                            const uint16_t* src1 = nullptr, uint16_t* dst1 = nullptr, float* sums1 = nullptr,
+                            size_t elems1 = 0) {
+  PrepArgs a{};
+  a.src[0] = src; a.dst[0] = dst; a.sums[0] = sums; a.chunks[0] = static_cast<uint32_t>(elems / 8);
+  a.src[1] = src1; a.dst[1] = dst1; a.sums[1] = sums1; a.chunks[1] = static_cast<uint32_t>(elems1 / 8);
+  a.blocks0 = (a.chunks[0] + 255) / 256;
+  const uint32_t blocks = a.blocks0 + (a.chunks[1] + 255) / 256;
+  if (!blocks) return hipSuccess;
+  prep_rows_kernel<<<dim3(blocks), dim3(256), 0, s>>>(a);
   return hipGetLastError();
 }
 
@@ -1032,8 +1052,8 @@ hipError_t launch_prefill_layer(hipStream_t s, const mf_moe& h, const mf_moe_lay
   q.out = ws.acts;
   MF_TRY(launch_qmm(s, q, 2, max_tiles, c.shared_f ? &d : nullptr, dense_tiles));
   // routes past the last tile's count were never written: only pairs rows exist, all written
-  MF_TRY(launch_prep_rows(s, ws.acts, nullptr, ws.sum_acts, pairs * c.f));
-  if (c.shared_f) MF_TRY(launch_prep_rows(s, ws.sact, nullptr, ws.sum_sact, static_cast<size_t>(t) * c.shared_f));
+  MF_TRY(launch_prep_rows(s, ws.acts, nullptr, ws.sum_acts, pairs * c.f, ws.sact, nullptr, ws.sum_sact,
+                          static_cast<size_t>(t) * c.shared_f));
   // phase 2: routed down -> fp32 partials [token*K+rank, D]; shared down -> hs [token, D]
   q.w_off[0] = w.offsets.down_w; q.s_off[0] = w.offsets.down_s; q.b_off[0] = w.offsets.down_b;
   q.x = ws.acts; q.sumx = ws.sum_acts; q.x_stride = c.f; q.gather = 0; q.rows = c.d; q.kdim = c.f; q.epi = 1; q.out = ws.partials;

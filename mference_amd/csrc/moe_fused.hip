@@ -415,16 +415,23 @@ __global__ __launch_bounds__(kFusedThreads) void fused_decode_kernel(const Fused
         have_spre = true;
       }
     }
-    // gather this token's routed activations and shared activations (+ gate) in one go:
-    // a virtual array [acts | sact], 256 words per wave step, two steps in flight
-    {
-      const uint32_t n_a = K * F, n_s = Fs ? (a.w_sg ? Fs + 4 : Fs) : 0, total = n_a + n_s;
-      const AgentBuf ba = make_agent_buf(a.t_acts + static_cast<size_t>(tok) * n_a);
-      const AgentBuf bs = make_agent_buf(a.t_sact + static_cast<size_t>(tok) * sact_stride);
-      const uint32_t want = tag16 << 16, step = kFusedWaves * 4 * kWave;
-      for (uint32_t c0 = wv * 4 * kWave; c0 < total; c0 += 2 * step) {
+    // Gather what other workgroups produced: the routed activations [K*F] and the shared
+    // activations (+ gate) [Fs (+4)], 256 words per wave step, two steps in flight.
+    // The shared activations were written in stage A, long ago: when the routed words fit the
+    // other waves' first poll step, the workgroup fetches the shared words first (they are there:
+    // one round trip, during which the routed words are still on their way anyway) and the few
+    // waves that own the shared-expert down rows compute the gated shared output h1 while the
+    // rest of the workgroup polls for the routed words -- h1 leaves the critical path.
+    const uint32_t n_a = K * F, n_s = Fs ? (a.w_sg ? Fs + 4 : Fs) : 0;
+    const AgentBuf ba = make_agent_buf(a.t_acts + static_cast<size_t>(tok) * n_a);
+    const AgentBuf bs = make_agent_buf(a.t_sact + static_cast<size_t>(tok) * sact_stride);
+    const uint32_t want = tag16 << 16;
+    // waves [w0, w0 + nw) gather words [first, first + count) of the virtual array [acts | sact]
+    auto gather = [&](uint32_t first, uint32_t count, uint32_t w0, uint32_t nw) __attribute__((always_inline)) {
+      const uint32_t step = nw * 4 * kWave, end = first + count;
+      for (uint32_t c0 = first + (wv - w0) * 4 * kWave; c0 < end; c0 += 2 * step) {
         const uint32_t i0 = c0 + 4 * lane, i1 = i0 + step;
-        const bool in0 = i0 < total, in1 = i1 < total;
+        const bool in0 = i0 < end, in1 = i1 < end;
         uint4 v0 = make_uint4(want, want, want, want), v1 = v0;
         for (uint32_t spins = 0;; ++spins) {
           if (in0) v0 = i0 < n_a ? load_u32x4_agentbuf(ba, i0 * 4) : load_u32x4_agentbuf(bs, (i0 - n_a) * 4);
@@ -449,13 +456,12 @@ __global__ __launch_bounds__(kFusedThreads) void fused_decode_kernel(const Fused
           dst[1] = __builtin_amdgcn_perm(v1.w, v1.z, 0x05040100u);
         }
       }
-    }
-    __syncthreads();
-    if (tok == 0) trace_mark(a, 5);
-    if (Fs) {
-      // gated shared output h1 of every output row this workgroup owns for this token
+    };
+    // gated shared output h1 of the output rows this workgroup owns for this token; waves
+    // [0, nw) share the rows
+    auto shared_rows = [&](uint32_t nw) __attribute__((always_inline)) {
       const float gate = a.w_sg ? bf16_lo(s_sact[Fs / 2]) : 0.0f;
-      for (uint32_t s0 = wv * srpw; s0 < n_slots; s0 += kFusedWaves * srpw) {
+      for (uint32_t s0 = wv * srpw; s0 < n_slots; s0 += nw * srpw) {
         const uint32_t i = s0 + (lane >> slpr_log2);  // slot of (round, unit_local, row in unit)
         const uint32_t round = i / rows_per_round, in_round = i % rows_per_round;
         const uint32_t unit = (round * G + wg) * ub + in_round / rpw;
@@ -475,6 +481,22 @@ __global__ __launch_bounds__(kFusedThreads) void fused_decode_kernel(const Fused
           s_h1[i] = h;
         }
       }
+    };
+    // waves that own shared rows when the rows are dealt one wave step each
+    const uint32_t sh_waves = Fs ? (n_slots + srpw - 1) / srpw : 0;
+    const bool split = Fs && sh_waves <= 4 && n_a <= (kFusedWaves - sh_waves) * 8 * kWave;
+    if (split) {
+      gather(n_a, n_s, 0, kFusedWaves);  // first try succeeds: one round trip
+      __syncthreads();
+      if (wv < sh_waves) shared_rows(sh_waves);
+      else gather(0, n_a, sh_waves, kFusedWaves - sh_waves);
+      __syncthreads();
+      if (tok == 0) trace_mark(a, 5);
+    } else {
+      gather(0, n_a + n_s, 0, kFusedWaves);
+      __syncthreads();
+      if (tok == 0) trace_mark(a, 5);
+      if (Fs) shared_rows(kFusedWaves);
     }
 
     for (uint32_t round = 0; round < rounds; ++round) {

@@ -208,7 +208,6 @@ mf_status mf_moe_create(mf_ctx* ctx, const mf_moe_config* cfg, mf_moe** out) {
   const size_t o_sy = take(T * cfg->d * sizeof(uint16_t));
   const size_t o_gate = take(T * sizeof(uint16_t));
   const size_t o_tlogits = take(T * cfg->num_experts * sizeof(uint64_t));
-  const size_t o_tgate = take(T * sizeof(uint64_t));
   const size_t o_tsact = take(T * (std::max<uint32_t>(cfg->shared_f, 64) + 4) * sizeof(uint32_t));
   const size_t o_tacts = take(T * cfg->top_k * cfg->f * sizeof(uint32_t));
   const size_t o_epoch = take(512 * sizeof(uint32_t));
@@ -239,7 +238,6 @@ mf_status mf_moe_create(mf_ctx* ctx, const mf_moe_config* cfg, mf_moe** out) {
   h->ws.shared_y = reinterpret_cast<uint16_t*>(b + o_sy);
   h->ws.gate = reinterpret_cast<uint16_t*>(b + o_gate);
   h->ws.t_logits = reinterpret_cast<unsigned long long*>(b + o_tlogits);
-  h->ws.t_gate = reinterpret_cast<unsigned long long*>(b + o_tgate);
   h->ws.t_sact = reinterpret_cast<uint32_t*>(b + o_tsact);
   h->ws.t_acts = reinterpret_cast<uint32_t*>(b + o_tacts);
   h->ws.epoch = reinterpret_cast<uint32_t*>(b + o_epoch);

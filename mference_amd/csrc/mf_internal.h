@@ -25,7 +25,6 @@ struct mf_moe_workspace {
   uint16_t* gate;       // [MF_MAX_TOKENS]
   // exchange buffers of the fused launch: every word carries an epoch tag
   unsigned long long* t_logits;  // [MF_MAX_TOKENS, num_experts]
-  unsigned long long* t_gate;    // [MF_MAX_TOKENS]
   uint32_t* t_sact;              // [MF_MAX_TOKENS, shared_f]
   uint32_t* t_acts;              // [MF_MAX_TOKENS, top_k, f]
   uint32_t* epoch;               // [512] one launch counter per workgroup

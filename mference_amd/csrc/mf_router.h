@@ -44,213 +44,6 @@ __device__ __forceinline__ float dot_bf16_row(const uint16_t* __restrict__ w,
 constexpr int kMaxPerLane = MF_MAX_EXPERTS / kWave;  // 8
 constexpr uint32_t kNoWinner = 0xFFFFFFFFu;
 
-// argmax over the wave with "equal score keeps the lower index"; all lanes
-// return the winner.
-__device__ __forceinline__ void wave_argmax(float& bv, uint32_t& bi) {
-#pragma unroll
-  for (int o = 32; o > 0; o >>= 1) {
-    const float ov = __shfl_xor(bv, o, kWave);
-    const uint32_t oi = __shfl_xor(bi, o, kWave);
-    if (ov > bv || (ov == bv && oi < bi)) {
-      bv = ov;
-      bi = oi;
-    }
-  }
-}
-
-// One wave per token (all 64 lanes call it; idx / w may be LDS or global;
-// AGENT_LOGITS: the logits were written by other workgroups of this launch).  Lane l owns experts l, l+64, ...  (ownership does not
-// change the result: every step picks the highest score, lowest index first).
-//
-// mode 0 = router_topk_select_k8 (moe.metal:190-240) for any k <= 8: k rounds of
-//   strict-greater / lower-index argmax over the logits (never selecting NaN or
-//   -inf, unfilled slots stay at index 0), then w_i = exp(s_i - s_0) / sum.
-// mode 1 = maple_router_top8_full_softmax (maple_moe.metal:62-119): any
-//   non-finite logit -> idx = e, w = 0; softmax over all experts with the
-//   32-wide tree sums added block by block, k rounds of argmax on the
-//   probabilities, renormalise with the 1e-20 guards.
-template <bool AGENT_LOGITS = false>
-__device__ __forceinline__ void topk_wave(const float* lg, uint32_t e, uint32_t k, int mode,
-                                          uint32_t* idx, float* w, uint32_t lane) {
-  const uint32_t per = (e + kWave - 1) / kWave;
-  float ch[kMaxPerLane];
-#pragma unroll
-  for (int j = 0; j < kMaxPerLane; ++j) {
-    const uint32_t x = lane + j * kWave;
-    ch[j] = -__builtin_inff();
-    if (static_cast<uint32_t>(j) < per && x < e) ch[j] = AGENT_LOGITS ? load_f32_agent(lg + x) : lg[x];
-  }
-  float top_s[MF_MAX_TOPK];
-  uint32_t top_i[MF_MAX_TOPK];
-
-  if (mode == 1) {
-    bool bad = false;
-    float mx = -1.0e30f;
-#pragma unroll
-    for (int j = 0; j < kMaxPerLane; ++j) {
-      const uint32_t x = lane + j * kWave;
-      if (static_cast<uint32_t>(j) < per && x < e) {
-        if (!__builtin_isfinite(ch[j])) bad = true;
-        if (ch[j] > mx) mx = ch[j];
-      }
-    }
-    bad = __any(bad);
-    if (bad) {
-      if (lane < k) {
-        idx[lane] = e;
-        w[lane] = 0.0f;
-      }
-      return;
-    }
-#pragma unroll
-    for (int o = 32; o > 0; o >>= 1) {
-      const float other = __shfl_xor(mx, o, kWave);
-      if (other > mx) mx = other;
-    }
-    // scores and the blocked sum: block g = experts [32g, 32g+32) = half a wave
-    // row j (g = 2j + (lane >= 32)); tree over 16,8,4,2,1 then blocks in order.
-    float total = 0.0f;
-#pragma unroll
-    for (int j = 0; j < kMaxPerLane; ++j) {
-      const uint32_t x = lane + j * kWave;
-      const bool live = static_cast<uint32_t>(j) < per && x < e;
-      ch[j] = live ? mf_exp(ch[j] - mx) : 0.0f;
-      float part = ch[j];
-#pragma unroll
-      for (int o = 16; o > 0; o >>= 1) part = part + __shfl_xor(part, o, kWave);
-      const float lo = __shfl(part, 0, kWave), hi = __shfl(part, 32, kWave);
-      if (static_cast<uint32_t>(2 * j) < e / 32) total += lo;
-      if (static_cast<uint32_t>(2 * j + 1) < e / 32) total += hi;
-    }
-    const float recip = 1.0f / (total + 1.0e-20f);
-#pragma unroll
-    for (int j = 0; j < kMaxPerLane; ++j) {
-      const uint32_t x = lane + j * kWave;
-      const bool live = static_cast<uint32_t>(j) < per && x < e;
-      ch[j] = live ? ch[j] * recip : -__builtin_inff();
-    }
-  }
-
-  uint32_t taken = 0;
-  for (uint32_t r = 0; r < k; ++r) {
-    float bv = (mode == 1) ? -1.0e30f : -__builtin_inff();
-    uint32_t bi = kNoWinner;
-#pragma unroll
-    for (int j = 0; j < kMaxPerLane; ++j) {
-      if (!(taken & (1u << j)) && ch[j] > bv) {
-        bv = ch[j];
-        bi = lane + j * kWave;
-      }
-    }
-    wave_argmax(bv, bi);
-    if (bi != kNoWinner && (bi & (kWave - 1)) == lane) taken |= 1u << (bi / kWave);
-#pragma unroll
-    for (int i = 0; i < MF_MAX_TOPK; ++i) {
-      if (static_cast<uint32_t>(i) == r) {
-        top_s[i] = bv;
-        top_i[i] = bi;
-      }
-    }
-  }
-  if (lane != 0) return;
-
-  float wt[MF_MAX_TOPK];
-  if (mode == 1) {
-    float sel = 0.0f;
-#pragma unroll
-    for (int i = 0; i < MF_MAX_TOPK; ++i) {
-      if (static_cast<uint32_t>(i) < k) {
-        if (top_i[i] == kNoWinner) top_i[i] = 0;  // maple: bestIndex stays 0
-        sel += top_s[i];
-      }
-    }
-#pragma unroll
-    for (int i = 0; i < MF_MAX_TOPK; ++i)
-      if (static_cast<uint32_t>(i) < k) wt[i] = top_s[i] / (sel + 1.0e-20f);
-  } else {
-#pragma unroll
-    for (int i = 0; i < MF_MAX_TOPK; ++i) {
-      if (static_cast<uint32_t>(i) < k && top_i[i] == kNoWinner) {
-        top_i[i] = 0;
-        top_s[i] = -__builtin_inff();
-      }
-    }
-    const float max_s = top_s[0];
-    float sum = 0.0f;
-#pragma unroll
-    for (int i = 0; i < MF_MAX_TOPK; ++i) {
-      if (static_cast<uint32_t>(i) < k) {
-        wt[i] = mf_exp(top_s[i] - max_s);
-        sum += wt[i];
-      }
-    }
-#pragma unroll
-    for (int i = 0; i < MF_MAX_TOPK; ++i)
-      if (static_cast<uint32_t>(i) < k) wt[i] = wt[i] / sum;
-  }
-#pragma unroll
-  for (int i = 0; i < MF_MAX_TOPK; ++i) {
-    if (static_cast<uint32_t>(i) < k) {
-      idx[i] = top_i[i];
-      w[i] = wt[i];
-    }
-  }
-}
-
-// mode 0 selector for a whole workgroup (every thread calls it; blockDim a
-// multiple of 64; e % 4 == 0).  The serial kernel's order "higher score first,
-// equal score: lower index first" is a total order, so the rank of an expert is
-// the number of experts that beat it, and the top-k are the experts of rank < k.
-// Four adjacent lanes share one (token, expert) and count a quarter of the
-// candidates each.  NaN and -inf never take a rank; ranks nobody takes keep
-// index 0 / score -inf.  lg: [t, e] logits in LDS; idx / w: [t, k] in LDS;
-// score: [t, k] scratch in LDS.
-__device__ __forceinline__ void topk_rank_block(const float* lg, uint32_t e, uint32_t k,
-                                                uint32_t t, uint32_t* idx, float* w,
-                                                float* score) {
-  const uint32_t tid = threadIdx.x, nthreads = blockDim.x;
-  if (tid < t * k) {
-    idx[tid] = 0;
-    score[tid] = -__builtin_inff();
-  }
-  __syncthreads();
-  const uint32_t qn = e / 4;
-  const uint32_t jobs = t * e * 4;
-  for (uint32_t it0 = 0; it0 < jobs; it0 += nthreads) {
-    const uint32_t it = it0 + tid;
-    const bool live = it < jobs;
-    const uint32_t tok = live ? it / (e * 4) : 0, ex = (it / 4) % e, q = it & 3;
-    const float* row = lg + tok * e;
-    const float v = live ? row[ex] : -__builtin_inff();
-    const bool cand = v > -__builtin_inff();
-    int cnt = 0;
-    if (cand) {
-      for (uint32_t j = q * qn; j < (q + 1) * qn; ++j) {
-        const float o = row[j];
-        cnt += (o > v || (o == v && j < ex)) ? 1 : 0;
-      }
-    }
-    cnt += __builtin_amdgcn_update_dpp(0, cnt, 0xB1, 0xF, 0xF, true);
-    cnt += __builtin_amdgcn_update_dpp(0, cnt, 0x4E, 0xF, 0xF, true);
-    if (cand && q == 0 && static_cast<uint32_t>(cnt) < k) {
-      idx[tok * k + cnt] = ex;
-      score[tok * k + cnt] = v;
-    }
-  }
-  __syncthreads();
-  const uint32_t wv = tid >> 6, lane = tid & 63;
-  if (wv < t) {  // w_r = exp(s_r - s_0) / sum, the sum taken in rank order
-    const float my = lane < k ? score[wv * k + lane] : -__builtin_inff();
-    const float my_e = mf_exp(my - readlane_f(my, 0));
-    float sum = 0.0f;
-#pragma unroll
-    for (int i = 0; i < MF_MAX_TOPK; ++i)
-      if (static_cast<uint32_t>(i) < k) sum += readlane_f(my_e, i);
-    if (lane < k) w[wv * k + lane] = my_e / sum;
-  }
-  __syncthreads();
-}
-
 // mode 0 selector, all-register form: lane l owns the PER consecutive experts
 // from l*PER (the blocked ownership of router_topk_select_k8_par,
 // moe.metal:262-345) and first sorts them by (score descending, index

@@ -166,33 +166,6 @@ __device__ __forceinline__ void poll_tagged_f32(const unsigned long long* src, f
   }
 }
 
-// Waves part, part + nparts, ... gather n tagged bf16 words (n % 4 == 0) into
-// packed bf16 pairs at dst (LDS, n / 2 words).
-__device__ __forceinline__ void poll_tagged_bf16(const uint32_t* src, uint32_t* dst, uint32_t n,
-                                                 uint32_t tag16, uint32_t part, uint32_t nparts,
-                                                 uint32_t lane, uint32_t* status) {
-  for (uint32_t w0 = part * 4 * kWave; w0 < n; w0 += nparts * 4 * kWave) {
-    const uint32_t i = w0 + 4 * lane;
-    const bool in = i < n;
-    const uint32_t want = tag16 << 16;
-    uint4 v = make_uint4(want, want, want, want);
-    for (uint32_t spins = 0;; ++spins) {
-      if (in) v = load_u32x4_agent(src + i);
-      const uint32_t diff = (v.x ^ want) | (v.y ^ want) | (v.z ^ want) | (v.w ^ want);
-      if (__all(!in || (diff >> 16) == 0)) break;
-      if (spins > kSpinLimit) {
-        give_up(status, lane);
-        break;
-      }
-      __builtin_amdgcn_s_sleep(1);
-    }
-    if (in) {
-      dst[i / 2] = __builtin_amdgcn_perm(v.y, v.x, 0x05040100u);
-      dst[i / 2 + 1] = __builtin_amdgcn_perm(v.w, v.z, 0x05040100u);
-    }
-  }
-}
-
 // phase trace: the 100 MHz wall clock at every stage boundary, thread 0 of each workgroup
 __device__ __forceinline__ void trace_mark(const FusedArgs& a, uint32_t slot) {
   if (a.trace && threadIdx.x == 0) a.trace[blockIdx.x * 8 + slot] = wall_clock64();

@@ -1013,7 +1013,10 @@ hipError_t launch_prefill_layer(hipStream_t s, const mf_moe& h, const mf_moe_lay
                                 const uint16_t* x, uint32_t t, uint16_t* y, void* workspace,
                                 uint32_t* out_idx, float* out_w) {
   const mf_moe_config& c = h.cfg;
-  const PrefillWs ws = prefill_carve(c, t, workspace);
+  PrefillWs ws = prefill_carve(c, t, workspace);
+  // the caller's routing outputs, when given, are the routing buffers of the whole call
+  if (out_idx) ws.idx = out_idx;
+  if (out_w) ws.w = out_w;
   hipError_t e;
 #define MF_TRY(call) do { e = (call); if (e != hipSuccess) return e; } while (0)
   const size_t pairs = static_cast<size_t>(t) * c.top_k;
@@ -1079,8 +1082,6 @@ hipError_t launch_prefill_layer(hipStream_t s, const mf_moe& h, const mf_moe_lay
   prefill_reduce_kernel<<<dim3(static_cast<uint32_t>((n4 + 255) / 256)), dim3(256), 0, s>>>(
       ws.partials, ws.w, ws.idx, hs, gate, y, t, c.top_k, c.d, c.num_experts);
   MF_TRY(hipGetLastError());
-  if (out_idx) MF_TRY(hipMemcpyAsync(out_idx, ws.idx, sizeof(uint32_t) * pairs, hipMemcpyDeviceToDevice, s));
-  if (out_w) MF_TRY(hipMemcpyAsync(out_w, ws.w, sizeof(float) * pairs, hipMemcpyDeviceToDevice, s));
 #undef MF_TRY
   return hipSuccess;
 }

@@ -527,33 +527,12 @@ __global__ __launch_bounds__(kQuadMaxWaves * 64) void rows_quad_kernel(const Row
   const uint32_t n_chunks = a.N / 32, ng = a.N / kGroup, n_sets = a.M / 4;
   const size_t row_bytes = static_cast<size_t>(a.N) / 2;
 
-  // ---- this lane's x: token c, chunks (wsub * ITS + j) * 16 + b
+  // chunk of every slot of this lane: (wsub * ITS + j) * 16 + b
   uint32_t chc[ITS];
-  uint2 xa[ITS][8], sx[ITS];
+  uint2 xa[ITS][8], sx[ITS];  // this lane's x operands and chunk sums (filled below)
 #pragma unroll
-  for (int j = 0; j < ITS; ++j) {
-    const uint32_t ch = (wsub * ITS + j) * 16 + b;
-    chc[j] = min(ch, n_chunks - 1);  // a slot past the row reads the last chunk against x = 0
-    const bool live = ch < n_chunks && c < a.T;
-    float sum = 0.0f;
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      uint4 v = make_uint4(0, 0, 0, 0);
-      if (live) v = *reinterpret_cast<const uint4*>(a.x + static_cast<size_t>(c) * a.N + chc[j] * 32 + 8 * i);
-      xa[j][2 * i] = make_uint2(__builtin_amdgcn_perm(v.z, v.x, 0x05040100u),   // (e0, e4)
-                                __builtin_amdgcn_perm(v.z, v.x, 0x07060302u));  // (e1, e5)
-      xa[j][2 * i + 1] = make_uint2(__builtin_amdgcn_perm(v.w, v.y, 0x05040100u),   // (e2, e6)
-                                    __builtin_amdgcn_perm(v.w, v.y, 0x07060302u));  // (e3, e7)
-      const uint32_t pr[4] = {v.x, v.y, v.z, v.w};
-#pragma unroll
-      for (int e = 0; e < 4; ++e) sum = (sum + bf16_lo(pr[e])) + bf16_hi(pr[e]);
-    }
-    const uint32_t hi = __float_as_uint(sum) & 0xFFFF0000u;
-    const float r1 = sum - __uint_as_float(hi);
-    const uint32_t mid = __float_as_uint(r1) & 0xFFFF0000u;
-    const uint32_t lo = __float_as_uint(r1 - __uint_as_float(mid));
-    sx[j] = make_uint2((hi >> 16) | mid, lo >> 16);  // K slots: hi, mid, lo, 0
-  }
+  for (int j = 0; j < ITS; ++j)
+    chc[j] = min((wsub * ITS + j) * 16 + b, n_chunks - 1);  // a slot past the row reads the last chunk against x = 0
 
   // Codes and table entries of two stages (a stage = one projection of one row set) live in a
   // ring of registers: a slot is refilled, as soon as it has been used, with the same slot of
@@ -578,12 +557,6 @@ __global__ __launch_bounds__(kQuadMaxWaves * 64) void rows_quad_kernel(const Row
   auto fetch_tables = [&](uint32_t set, int p) __attribute__((always_inline)) {
     return *reinterpret_cast<const uint4*>((tb_bias ? a.B[p] : a.S[p]) + (static_cast<size_t>(set) * 4 + tb_row) * ng +
                                            tb_group);
-  };
-  auto issue = [&](int buf, uint32_t set, int p) __attribute__((always_inline)) {
-    const uint4 t = fetch_tables(set, p);
-#pragma unroll
-    for (int j = 0; j < ITS; ++j) fetch(buf, j, set, p);
-    *reinterpret_cast<uint4*>(my_tab + buf * (64 * 8) + lane * 8) = t;
   };
   // the wave's part of D[token, row] for one row set; then the four blocks of each 16-lane row
   // are added and lanes 0..3 of the row leave [weight row][token] in LDS.  `refill` is the row
@@ -654,9 +627,42 @@ __global__ __launch_bounds__(kQuadMaxWaves * 64) void rows_quad_kernel(const Row
   const uint32_t G = gridDim.x, last = n_sets - 1;
   uint32_t set = blockIdx.x, pb = 0;
   if (set >= n_sets) return;
+  const uint32_t set1 = NPROJ == 2 ? set : min(set + G, last);
+  const uint4 t0 = fetch_tables(set, 0), t1 = fetch_tables(set1, NPROJ == 2 ? 1 : 0);
+#pragma unroll
+  for (int j = 0; j < ITS; ++j) {
+    fetch(0, j, set, 0);
+    fetch(1, j, set1, NPROJ == 2 ? 1 : 0);
+  }
+  // ---- this lane's x: token c, chunks (wsub * ITS + j) * 16 + b.  The first two stages' weight
+  // loads are already on their way: the x rows come from L2 behind them.
+#pragma unroll
+  for (int j = 0; j < ITS; ++j) {
+    const uint32_t ch = (wsub * ITS + j) * 16 + b;
+    const bool live = ch < n_chunks && c < a.T;
+    float sum = 0.0f;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      uint4 v = make_uint4(0, 0, 0, 0);
+      if (live) v = *reinterpret_cast<const uint4*>(a.x + static_cast<size_t>(c) * a.N + chc[j] * 32 + 8 * i);
+      xa[j][2 * i] = make_uint2(__builtin_amdgcn_perm(v.z, v.x, 0x05040100u),   // (e0, e4)
+                                __builtin_amdgcn_perm(v.z, v.x, 0x07060302u));  // (e1, e5)
+      xa[j][2 * i + 1] = make_uint2(__builtin_amdgcn_perm(v.w, v.y, 0x05040100u),   // (e2, e6)
+                                    __builtin_amdgcn_perm(v.w, v.y, 0x07060302u));  // (e3, e7)
+      const uint32_t pr[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+      for (int e = 0; e < 4; ++e) sum = (sum + bf16_lo(pr[e])) + bf16_hi(pr[e]);
+    }
+    const uint32_t hi = __float_as_uint(sum) & 0xFFFF0000u;
+    const float r1 = sum - __uint_as_float(hi);
+    const uint32_t mid = __float_as_uint(r1) & 0xFFFF0000u;
+    const uint32_t lo = __float_as_uint(r1 - __uint_as_float(mid));
+    sx[j] = make_uint2((hi >> 16) | mid, lo >> 16);  // K slots: hi, mid, lo, 0
+  }
+
+  *reinterpret_cast<uint4*>(my_tab + lane * 8) = t0;
+  *reinterpret_cast<uint4*>(my_tab + 64 * 8 + lane * 8) = t1;
   if constexpr (NPROJ == 2) {
-    issue(0, set, 0);
-    issue(1, set, 1);
     for (; set < n_sets; set += G) {
       const uint32_t nxt = min(set + G, last);
       compute(0, 0, pb, nxt);
@@ -666,8 +672,6 @@ __global__ __launch_bounds__(kQuadMaxWaves * 64) void rows_quad_kernel(const Row
       pb ^= 1u;
     }
   } else {
-    issue(0, set, 0);
-    issue(1, min(set + G, last), 0);
     for (;;) {
       compute(0, 0, pb, min(set + 2 * G, last));
       __syncthreads();

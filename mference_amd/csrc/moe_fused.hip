@@ -187,6 +187,14 @@ struct StaticShape {
   static constexpr uint32_t D = D_, F = F_, E = E_, K = K_, T = T_, Fs = Fs_;
 };
 
+// rows one wave takes per step when a row has n elements (compile-time twin of
+// 64 >> lanes_per_row_log2_dev)
+constexpr uint32_t static_rows_per_wave(uint32_t n, uint32_t elems_per_lane) {
+  uint32_t need = (n + elems_per_lane - 1) / elems_per_lane, lanes = 1;
+  while (lanes < need && lanes < 64) lanes *= 2;
+  return 64u / lanes;
+}
+
 template <int BITS, int SBITS, class S>
 __global__ __launch_bounds__(kFusedThreads) void fused_decode_kernel(const FusedArgs a) {
   extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
@@ -297,6 +305,15 @@ __global__ __launch_bounds__(kFusedThreads) void fused_decode_kernel(const Fused
     const uint32_t lpr = 1u << lpr_log2, rpw = 64u >> lpr_log2;
     const uint32_t rgf = (F + rpw - 1) / rpw;
     const uint32_t n_items = T * K * rgf;
+    // a row is one 16-byte step per lane and waves have more than one item.  A shape-specialised
+    // kernel compiles the path in only when a full grid of 256 workgroups would have such waves
+    // (on a smaller grid it then simply takes the general path).
+    constexpr uint32_t kStaticRpw = static_rows_per_wave(S::kStatic ? S::D : 64u, Fmt<BITS>::kElemsPer16B);
+    constexpr bool kMayHoist =
+        !S::kStatic || S::T * S::K * ((S::F + kStaticRpw - 1) / kStaticRpw) > kFusedWaves * 256u;
+    const bool one_step = kMayHoist && lpr * Fmt<BITS>::kElemsPer16B >= D && n_items > total_waves;
+    XSlice<BITS> xs_cur{};
+    uint32_t xs_tok = 0xFFFFFFFFu;
     for (uint32_t item = gw; item < n_items; item += total_waves) {
       const uint32_t pair = item / rgf;
       const uint32_t row = (item % rgf) * rpw + (lane >> lpr_log2);
@@ -313,7 +330,28 @@ __global__ __launch_bounds__(kFusedThreads) void fused_decode_kernel(const Fused
       const uint32_t ng = D / kGroup;
       const size_t rb = static_cast<size_t>(D) * Store<BITS>::kBits / 8;
       float ga = 0.0f, ua = 0.0f;
-      if (ok)
+      if (one_step) {
+        // the lane's slice of x depends on the token only: a wave with several items of one
+        // token builds it once (same operations as gate_up_partial, one step)
+        const uint32_t e0 = sub * Fmt<BITS>::kElemsPer16B, tok = pair / K;
+        if (tok != xs_tok) {
+          if (e0 < D) xs_cur = load_xslice<BITS, kXAligned>(a.x + static_cast<size_t>(tok) * D + e0);
+          xs_tok = tok;
+        }
+        if (ok && e0 < D) {
+          const Chunk<BITS> gc = load_chunk<BITS>(blob + a.off.gate_w + r * rb,
+                                                  reinterpret_cast<const uint16_t*>(blob + a.off.gate_s) + r * ng,
+                                                  reinterpret_cast<const uint16_t*>(blob + a.off.gate_b) + r * ng, e0);
+          const Chunk<BITS> uc = load_chunk<BITS>(blob + a.off.up_w + r * rb,
+                                                  reinterpret_cast<const uint16_t*>(blob + a.off.up_s) + r * ng,
+                                                  reinterpret_cast<const uint16_t*>(blob + a.off.up_b) + r * ng, e0);
+          const float gd = codes_dot<BITS>(gc.codes, xs_cur), ud = codes_dot<BITS>(uc.codes, xs_cur);
+          ga = __builtin_fmaf(gc.s, gd, ga);
+          ga = __builtin_fmaf(gc.b, xs_cur.sum, ga);
+          ua = __builtin_fmaf(uc.s, ud, ua);
+          ua = __builtin_fmaf(uc.b, xs_cur.sum, ua);
+        }
+      } else if (ok)
         gate_up_partial<BITS>(blob + a.off.gate_w + r * rb,
                               reinterpret_cast<const uint16_t*>(blob + a.off.gate_s) + r * ng,
                               reinterpret_cast<const uint16_t*>(blob + a.off.gate_b) + r * ng,

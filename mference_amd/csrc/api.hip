@@ -330,10 +330,11 @@ mf_status mf_moe_decode_layer(mf_moe* h, mf_stream stream, const mf_moe_layer_we
   MF_HIP(h->ctx, mf::launch_topk(s, h->ws.logits, c.num_experts, c.top_k, t, c.router_mode, idx, w));
   const uint16_t* residual = nullptr;
   if (c.shared_f) {
+    // lane order of the fused kernel: both forms of the layer give the same bits
     MF_HIP(h->ctx, mf::launch_gate_up_act(s, wts->shared_gate, wts->shared_up, c.shared_bits, x,
-                                          h->ws.shared_act, c.shared_f, c.d, t));
+                                          h->ws.shared_act, c.shared_f, c.d, t, true));
     MF_HIP(h->ctx, mf::launch_gemv(s, wts->shared_down, c.shared_bits, h->ws.shared_act,
-                                   h->ws.shared_y, c.d, c.shared_f, t, false));
+                                   h->ws.shared_y, c.d, c.shared_f, t, false, true));
     if (wts->w_sg) {
       MF_HIP(h->ctx, mf::launch_router_logits(s, wts->w_sg, x, 1, c.d, t, c.d, nullptr, h->ws.gate));
       MF_HIP(h->ctx, mf::launch_sigmoid_scalar_mul(s, h->ws.shared_y, h->ws.gate, c.d, t));

@@ -868,9 +868,9 @@ bool rows_quad_try(hipStream_t s, const RowsQuadArgs& a, uint32_t num_cu, hipErr
 }  // namespace
 
 hipError_t launch_gemv(hipStream_t s, const mf_qtensor& w, int bits, const uint16_t* x, void* y,
-                       uint32_t m, uint32_t n, uint32_t t, bool out_f32) {
+                       uint32_t m, uint32_t n, uint32_t t, bool out_f32, bool lane_order) {
   const bool al = aligned16(w.weights) && aligned16(x);
-  if (al && bits == kBits4 && aligned16(w.scales) && aligned16(w.biases)) {
+  if (!lane_order && al && bits == kBits4 && aligned16(w.scales) && aligned16(w.biases)) {
     RowsMfmaArgs ma{};
     ma.W[0] = static_cast<const uint8_t*>(w.weights); ma.S[0] = w.scales; ma.B[0] = w.biases;
     ma.x = x; ma.y = y; ma.M = m; ma.N = n; ma.T = t; ma.out_f32 = out_f32 ? 1 : 0;
@@ -881,7 +881,7 @@ hipError_t launch_gemv(hipStream_t s, const mf_qtensor& w, int bits, const uint1
     if (rows_quad_try<1>(s, qa, device_cu_count(), err)) return err;
     if (rows_mfma_try<1>(s, ma, device_cu_count(), err)) return err;
   }
-  if (al && (bits == kBits4 || bits == kBits2)) {
+  if (!lane_order && al && (bits == kBits4 || bits == kBits2)) {
     RowsArgs a{};
     a.W[0] = static_cast<const uint8_t*>(w.weights); a.S[0] = w.scales; a.B[0] = w.biases;
     a.x = x; a.y = y; a.M = m; a.N = n; a.out_f32 = out_f32 ? 1 : 0;
@@ -906,9 +906,9 @@ hipError_t launch_gemv(hipStream_t s, const mf_qtensor& w, int bits, const uint1
 
 hipError_t launch_gate_up_act(hipStream_t s, const mf_qtensor& gate, const mf_qtensor& up,
                               int bits, const uint16_t* x, uint16_t* act, uint32_t f, uint32_t d,
-                              uint32_t t) {
+                              uint32_t t, bool lane_order) {
   const bool al = aligned16(gate.weights) && aligned16(up.weights) && aligned16(x);
-  if (al && bits == kBits4 && aligned16(gate.scales) && aligned16(gate.biases) && aligned16(up.scales) &&
+  if (!lane_order && al && bits == kBits4 && aligned16(gate.scales) && aligned16(gate.biases) && aligned16(up.scales) &&
       aligned16(up.biases)) {
     RowsMfmaArgs ma{};
     ma.W[0] = static_cast<const uint8_t*>(gate.weights); ma.S[0] = gate.scales; ma.B[0] = gate.biases;
@@ -921,7 +921,7 @@ hipError_t launch_gate_up_act(hipStream_t s, const mf_qtensor& gate, const mf_qt
     if (rows_quad_try<2>(s, qa, device_cu_count(), err)) return err;
     if (rows_mfma_try<2>(s, ma, device_cu_count(), err)) return err;
   }
-  if (al && (bits == kBits4 || bits == kBits2)) {
+  if (!lane_order && al && (bits == kBits4 || bits == kBits2)) {
     RowsArgs a{};
     a.W[0] = static_cast<const uint8_t*>(gate.weights); a.S[0] = gate.scales; a.B[0] = gate.biases;
     a.W[1] = static_cast<const uint8_t*>(up.weights); a.S[1] = up.scales; a.B[1] = up.biases;

@@ -63,11 +63,15 @@ hipError_t launch_dequantize(hipStream_t s, const mf_qtensor& q, size_t rows, si
                              float* out);
 
 // gemv.hip
+// `lane_order`: keep the per-row lane partition of gemv_kernel (the fused decode kernel sums in
+// that order; the chain of separate launches of a decode layer asks for it so that both give
+// the same bits).  Without it wide matrices may take the matrix-core kernels, whose sums differ
+// in the last bits.
 hipError_t launch_gemv(hipStream_t s, const mf_qtensor& w, int bits, const uint16_t* x, void* y,
-                       uint32_t m, uint32_t n, uint32_t t, bool out_f32);
+                       uint32_t m, uint32_t n, uint32_t t, bool out_f32, bool lane_order = false);
 hipError_t launch_gate_up_act(hipStream_t s, const mf_qtensor& gate, const mf_qtensor& up,
                               int bits, const uint16_t* x, uint16_t* act, uint32_t f, uint32_t d,
-                              uint32_t t);
+                              uint32_t t, bool lane_order = false);
 hipError_t launch_silu_mul(hipStream_t s, const uint16_t* gate, const uint16_t* up, uint16_t* out,
                            uint32_t count);
 hipError_t launch_sigmoid_scalar_mul(hipStream_t s, uint16_t* y, const uint16_t* gate,

@@ -365,3 +365,37 @@ def test_qwen_shape_specialised_launch(gpu, oracle):
                                f"qwen shape fused={fused}")
             outs[fused] = ops.bf16_bits(y)
         assert np.array_equal(outs[True], outs[False])
+
+
+@pytest.mark.parametrize("workload,t", [("dsv4-2bit", 1), ("dsv4-2bit", 4), ("maple-ternary", 1)])
+def test_other_shape_specialised_launches(gpu, oracle, workload, t):
+    """the large 2-bit layer (D 4096, F 2048, E 256, K 6, 4-bit shared 2048; T = 1 and 4) and the
+    ternary layer (D 2048, F 1024, E 64, K 8, full-softmax router) at full size take their own
+    shape-specialised fused kernels; weights drawn and quantized on the GPU as bench.py does,
+    checked against the CPU checker and against the chain of separate launches"""
+    import bench
+    w = dict(bench.WORKLOADS[workload])
+    stack = bench.build_stack(gpu, w, 1, torch.device("cuda", 0))
+    host = bench.layer_to_host(stack[0], w)
+    mode = ops.ROUTER_FULL_SOFTMAX if w["bits"] == 1 else ops.ROUTER_TOPK_SOFTMAX
+    host.router_mode = 1 if w["bits"] == 1 else 0
+    moe = ops.MoE(gpu, w["d"], w["f"], w["e"], w["k"], bits=w["bits"], shared_f=w["fs"],
+                  shared_bits=w["shared_bits"], router_mode=mode)
+    gen = torch.Generator(device="cuda")
+    gen.manual_seed(4321)
+    x = torch.randn((t, w["d"]), generator=gen, device="cuda").to(torch.bfloat16)
+    ref_y, ref_idx, ref_w = oracle.moe_layer(host, ops.bf16_bits(x))
+    outs = {}
+    for fused in (True, False):
+        moe.set_fused(fused)
+        y = torch.zeros_like(x)
+        idx = torch.zeros((t, w["k"]), dtype=torch.int32, device="cuda")
+        rw = torch.zeros((t, w["k"]), dtype=torch.float32, device="cuda")
+        moe.encode_decode_layer(stack[0], x, y, t=t, out_indices=idx, out_weights=rw)
+        moe.status()
+        assert np.array_equal(idx.cpu().numpy().astype(np.uint32), ref_idx)
+        assert np.array_equal(rw.cpu().numpy().view(np.uint32), ref_w.view(np.uint32))
+        assert_layer_close(oracle.bf16_to_float(ops.bf16_bits(y)), oracle.bf16_to_float(ref_y),
+                           f"{workload} T={t} fused={fused}")
+        outs[fused] = ops.bf16_bits(y)
+    assert np.array_equal(outs[True], outs[False])

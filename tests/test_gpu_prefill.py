@@ -148,3 +148,48 @@ def test_prefill_rejects_a_short_workspace(gpu, oracle):
     with pytest.raises(_capi.MfError) as err:
         moe4.encode_prefill_layer(wts4, x, y, 4, workspace=torch.empty(256, dtype=torch.uint8, device="cuda"))
     assert err.value.status == -4
+
+
+def test_prefill_full_size_rows_do_not_depend_on_their_neighbours(gpu, oracle):
+    """Qwen-shaped layer, 2048 tokens, skewed routing (the bench.py configuration): a token's
+    output row depends on that token alone, so permuting the tokens permutes the rows bit for
+    bit (tiles, chunk boundaries and positions inside a tile all change); the routes of every
+    expert add up; sampled rows agree with the decode launch of the same token."""
+    import bench
+    w = dict(bench.QWEN)
+    dev = torch.device("cuda", 0)
+    stack = bench.build_stack(gpu, w, 1, dev)
+    lw = stack[0]
+    gen = torch.Generator(device=dev)
+    gen.manual_seed(99)
+    router = lw.router_w.clone()
+    router[:, -1] = (torch.randn((w["e"],), generator=gen, device=dev) * 1.5).to(torch.bfloat16)
+    lw = ops.MoELayerWeights(router, lw.experts, lw.offsets, lw.shared, lw.w_sg)
+    moe = ops.MoE(gpu, w["d"], w["f"], w["e"], w["k"], bits=4, shared_f=w["fs"], shared_bits=4)
+    t, d, k = 2048, w["d"], w["k"]
+    x = torch.randn((t, d), generator=gen, device=dev).to(torch.bfloat16)
+    x[:, -1] = 1.0
+    y = torch.zeros_like(x)
+    idx = torch.zeros((t, k), dtype=torch.int32, device=dev)
+    ws = moe.encode_prefill_layer(lw, x, y, t, out_indices=idx)
+    torch.cuda.synchronize()
+    assert bool(torch.isfinite(y.float()).all())
+    counts = torch.bincount(idx.flatten().long(), minlength=w["e"])
+    assert int(counts.sum()) == t * k and int((counts == 0).sum()) > 0   # skew: some experts stay empty
+    assert bool((idx.sort(dim=1).values.diff(dim=1) != 0).all())        # k distinct experts per token
+    perm = torch.randperm(t, generator=gen, device=dev)
+    xp = x[perm].contiguous()
+    yp = torch.zeros_like(x)
+    idxp = torch.zeros_like(idx)
+    moe.encode_prefill_layer(lw, xp, yp, t, out_indices=idxp, workspace=ws)
+    torch.cuda.synchronize()
+    assert torch.equal(idxp, idx[perm])
+    assert torch.equal(yp.view(torch.int16), y[perm].view(torch.int16))
+    for i in (0, 1, 777, 2047):   # the decode launch on single tokens
+        yd = torch.zeros((1, d), dtype=torch.bfloat16, device=dev)
+        idd = torch.zeros((1, k), dtype=torch.int32, device=dev)
+        moe.encode_decode_layer(lw, x[i:i + 1].contiguous(), yd, t=1, out_indices=idd)
+        moe.status()
+        assert torch.equal(idd[0], idx[i])
+        assert_layer_close(oracle.bf16_to_float(ops.bf16_bits(y[i:i + 1])),
+                           oracle.bf16_to_float(ops.bf16_bits(yd)), f"prefill row {i} vs decode")

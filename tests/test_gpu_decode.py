@@ -399,3 +399,41 @@ def test_other_shape_specialised_launches(gpu, oracle, workload, t):
                            f"{workload} T={t} fused={fused}")
         outs[fused] = ops.bf16_bits(y)
     assert np.array_equal(outs[True], outs[False])
+
+
+def test_dense_mlp_full_size(gpu, oracle):
+    """hidden 5120, intermediate 17408, 4 token rows (the dense-MLP configuration of bench.py):
+    weights drawn and quantized on the GPU, every row against the CPU checker; rows of the
+    4-token call equal the single-token calls bit for bit"""
+    d, f, t = 5120, 17408, 4
+    dev = torch.device("cuda", 0)
+    gen = torch.Generator(device=dev)
+    gen.manual_seed(2024)
+    quant = ops.Quantization(gpu)
+    qs = []
+    for rows, cols in ((f, d), (f, d), (d, f)):
+        raw = torch.randn((rows, cols), generator=gen, device=dev) * 0.02
+        qs.append(quant.quantize_affine(raw, 4))
+        del raw
+    x = torch.randn((t, d), generator=gen, device=dev).to(torch.bfloat16)
+    mlp = ops.SharedExpertInt4(gpu)
+    y = torch.zeros((t, d), dtype=torch.bfloat16, device=dev)
+    scratch = torch.zeros((t, f), dtype=torch.bfloat16, device=dev)
+    mlp.encode(x, qs[0], qs[1], qs[2], y, scratch, t=t)
+    _sync()
+
+    def hq(q):
+        return oracle.QTensor(q.packed.cpu().numpy(), ops.bf16_bits(q.scales), ops.bf16_bits(q.biases), 4, q.rows, q.n)
+    hg, hu, hd = hq(qs[0]), hq(qs[1]), hq(qs[2])
+    ref = np.stack([oracle.shared_expert(hg, hu, hd, ops.bf16_bits(x[i])) for i in range(t)])
+    got = oracle.bf16_to_float(ops.bf16_bits(y)).astype(np.float64)
+    reff = oracle.bf16_to_float(ref).astype(np.float64)
+    rel_l2 = np.linalg.norm(got - reff) / np.linalg.norm(reff)
+    # |y| reaches 8..16 here, where one bf16 step is 0.0625: the max-abs bar is one step of the output
+    assert rel_l2 <= 1e-3 and np.abs(got - reff).max() <= 0.0625 + 1e-6, (rel_l2, np.abs(got - reff).max())
+    for i in range(t):
+        yi = torch.zeros((1, d), dtype=torch.bfloat16, device=dev)
+        si = torch.zeros((1, f), dtype=torch.bfloat16, device=dev)
+        mlp.encode(x[i:i + 1].contiguous(), qs[0], qs[1], qs[2], yi, si, t=1)
+        _sync()
+        assert torch.equal(yi[0].view(torch.int16), y[i].view(torch.int16))

@@ -1,0 +1,233 @@
+"""Reader of the reference's `packed_experts/` directory: `layout.json` plus one
+`layer_XX.bin` per MoE layer, every routed expert one contiguous blob
+(gate, gate_scales, gate_biases, up, ..., down_biases) at a fixed stride.
+
+Mirrors `PackedExpertsLayoutReader.load`
+(Sources/Mference/Infrastructure/ModelIO/PackedExpertsLayout.swift:46-157: same keys, same
+checks, same error cases), `Model.routedExpertOffsets` / `routedExpertPhysicalOffsets`
+(Sources/Mference/Runtime/Inference/ModelExpertIO.swift:20-39) and `routedGateGroupSize`
+(ModelExpertIO.swift:118-135), and loads a layer file straight into the resident HBM expert
+pool the operators address as `expert_base + expert * stride`.
+
+What it does not do: the group-32 gate projection of the DeepSeek conversion is detected
+(`routed_gate_group_size`) but the kernels take group 64 only; Maple's per-row alpha tables
+are expected already expanded to per-group scale / bias entries, which is how the reference's
+repacker stores them.
+"""
+from __future__ import annotations
+
+import json
+import os
+from dataclasses import dataclass
+from typing import Dict, List, Optional
+
+DEFAULT_MAX_BYTES = 64 * 1024 * 1024   # PackedExpertsLayout.swift:49
+GROUP_SIZE = 64                        # Quantization.groupSize
+
+
+class ModelError(Exception):
+    """ModelTypes.swift:795-800: `missingFile(name)` and `indexCorrupt(detail)`."""
+
+    def __init__(self, kind: str, text: str):
+        super().__init__(f"{kind}: {text}")
+        self.kind = kind
+        self.text = text
+
+    @classmethod
+    def missing_file(cls, name: str) -> "ModelError":
+        return cls("missingFile", name)
+
+    @classmethod
+    def index_corrupt(cls, detail: str) -> "ModelError":
+        return cls("indexCorrupt", detail)
+
+
+@dataclass(frozen=True)
+class SubTensorEntry:          # PackedExpertsLayout.swift:3-6
+    offset: int                # relative to the expert blob's start
+    size: int                  # bytes; scale slices encode the group count
+
+
+@dataclass(frozen=True)
+class ExpertEntry:             # PackedExpertsLayout.swift:8-28
+    expert: int                # logical routed-expert id
+    offset: int                # absolute byte offset of the blob inside its layer file
+    size: int                  # bytes of the blob (== expert_stride)
+    sub_tensors: Dict[str, SubTensorEntry]
+
+
+@dataclass(frozen=True)
+class LayerLayout:             # PackedExpertsLayout.swift:30-34
+    layer: int
+    file: str                  # basename, e.g. "layer_00.bin"
+    experts: List[ExpertEntry]
+
+
+@dataclass(frozen=True)
+class PackedExpertsLayout:     # PackedExpertsLayout.swift:36-46
+    expert_stride: int
+    num_layers: int
+    experts_per_layer: int
+    layers: List[LayerLayout]
+
+    def expert(self, layer: int, expert: int) -> ExpertEntry:
+        return self.layers[layer].experts[expert]
+
+
+def _is_int(v) -> bool:
+    return isinstance(v, int) and not isinstance(v, bool)
+
+
+def _uint(v) -> Optional[int]:
+    """NSNumber.uint64Value of a JSON number: integers, and floats holding one"""
+    if _is_int(v) and v >= 0:
+        return v
+    if isinstance(v, float) and v >= 0 and v == int(v):
+        return int(v)
+    return None
+
+
+class PackedExpertsLayoutReader:
+    """`PackedExpertsLayoutReader.load(directoryURL:maxBytes:)`"""
+
+    default_max_bytes = DEFAULT_MAX_BYTES
+
+    @staticmethod
+    def load(directory: str, max_bytes: int = DEFAULT_MAX_BYTES) -> PackedExpertsLayout:
+        path = os.path.join(directory, "packed_experts", "layout.json")
+        if not os.path.isfile(path):
+            raise ModelError.missing_file("packed_experts/layout.json")
+        size = os.path.getsize(path)
+        if size > max_bytes:   # checked before anything is decoded
+            raise ModelError.index_corrupt(f"layout.json size {size} exceeds metadata cap {max_bytes}")
+        try:
+            with open(path, "rb") as fh:
+                root = json.loads(fh.read().decode("utf-8"))
+        except (ValueError, UnicodeDecodeError) as exc:
+            raise ModelError.index_corrupt(f"layout.json: {exc}") from None
+        if not isinstance(root, dict):
+            root = {}
+        stride = _uint(root.get("expertStride"))
+        n_layers = root.get("numLayers")
+        per_layer = root.get("expertsPerLayer")
+        layers_arr = root.get("layers")
+        if (stride is None or not _is_int(n_layers) or not _is_int(per_layer)
+                or not isinstance(layers_arr, list) or not all(isinstance(x, dict) for x in layers_arr)):
+            raise ModelError.index_corrupt("layout.json: missing top-level keys")
+
+        layers: List[LayerLayout] = []
+        for obj in layers_arr:
+            layer_idx, file, experts_arr = obj.get("layer"), obj.get("file"), obj.get("experts")
+            if (not _is_int(layer_idx) or not isinstance(file, str) or not isinstance(experts_arr, list)
+                    or not all(isinstance(x, dict) for x in experts_arr)):
+                raise ModelError.index_corrupt("layout.json: malformed layer entry")
+            if not experts_arr:   # leading dense-FFN layers: an empty entry, no blob file
+                layers.append(LayerLayout(layer_idx, file, []))
+                continue
+            experts: List[Optional[ExpertEntry]] = [None] * per_layer
+            for eobj in experts_arr:
+                off, esize, tensors = _uint(eobj.get("offset")), _uint(eobj.get("size")), eobj.get("tensors")
+                if (off is None or esize is None or not isinstance(tensors, dict)
+                        or not all(isinstance(t, dict) for t in tensors.values())):
+                    raise ModelError.index_corrupt("layout.json: malformed expert entry")
+                subs: Dict[str, SubTensorEntry] = {}
+                for role, t in tensors.items():
+                    toff, tsize = _uint(t.get("offset")), _uint(t.get("size"))
+                    shape = t.get("shape")
+                    if (toff is None or tsize is None or not isinstance(t.get("dtype"), str)
+                            or not isinstance(shape, list) or not all(_is_int(s) for s in shape)):
+                        raise ModelError.index_corrupt(f"layout.json: malformed tensor {role}")
+                    if "bits" in t and not _is_int(t["bits"]):
+                        raise ModelError.index_corrupt(f"layout.json: malformed tensor bits {role}")
+                    subs[role] = SubTensorEntry(toff, tsize)
+                expert_id = eobj.get("expert")
+                if not _is_int(expert_id):   # absent id: the next free position in file order
+                    expert_id = sum(1 for x in experts if x is not None)
+                if expert_id < 0 or expert_id >= per_layer:
+                    raise ModelError.index_corrupt("layout.json: expert id out of range")
+                rank = eobj.get("physicalRank")
+                if _is_int(rank) and (rank < 0 or rank >= per_layer):
+                    raise ModelError.index_corrupt("layout.json: physicalRank out of range")
+                experts[expert_id] = ExpertEntry(expert_id, off, esize, subs)
+            if any(x is None for x in experts):
+                raise ModelError.index_corrupt("layout.json: missing expert entries")
+            layers.append(LayerLayout(layer_idx, file, list(experts)))   # type: ignore[arg-type]
+        return PackedExpertsLayout(stride, n_layers, per_layer, layers)
+
+
+_ROLES = ("gate", "gate_scales", "gate_biases", "up", "up_scales", "up_biases",
+          "down", "down_scales", "down_biases")
+
+
+def routed_expert_offsets(layout: PackedExpertsLayout, layer: int):
+    """`Model.routedExpertOffsets(layer:)`: the nine sub-tensor offsets of expert 0 of the layer
+    (a missing role reads as 0), as the operators' MoEExpertOffsets."""
+    from .operators import MoEExpertOffsets
+    subs = layout.expert(layer, 0).sub_tensors
+    vals = [subs[r].offset if r in subs else 0 for r in _ROLES]
+    off = MoEExpertOffsets()
+    for (name, _), v in zip(off._fields_, vals):
+        setattr(off, name, v)
+    return off
+
+
+def routed_expert_physical_offsets(layout: PackedExpertsLayout, layer: int) -> List[int]:
+    """`Model.routedExpertPhysicalOffsets(layer:)`"""
+    return [e.offset for e in layout.layers[layer].experts]
+
+
+def routed_gate_group_size(layout: PackedExpertsLayout, layer: int, moe_intermediate: int, hidden: int) -> int:
+    """`Model.routedGateGroupSize(layer:)`: the gate projection's quantization group, from the
+    byte size of its scale slice (bf16 entries, one per row and group)."""
+    scales = layout.expert(layer, 0).sub_tensors.get("gate_scales")
+    if scales is None or moe_intermediate <= 0:
+        return GROUP_SIZE
+    groups = scales.size // (2 * moe_intermediate)
+    if groups <= 0 or hidden % groups:
+        return GROUP_SIZE
+    return hidden // groups
+
+
+def load_layer_experts(directory: str, layout: PackedExpertsLayout, layer: int, device="cuda"):
+    """Read `packed_experts/<layer file>` into one resident uint8 tensor of
+    experts_per_layer * expert_stride bytes in LOGICAL expert order (the operators address
+    expert e at e * stride; the file may hold the blobs in any physical order).  Returns
+    (tensor, stride).  The read goes through a pinned staging buffer in chunks, so a 453 MB
+    layer never needs a second full copy in host memory."""
+    import numpy as np
+    import torch
+
+    entry = layout.layers[layer]
+    if not entry.experts:
+        raise ModelError.index_corrupt(f"layer {layer} has no routed experts")
+    path = os.path.join(directory, "packed_experts", entry.file)
+    if not os.path.isfile(path):
+        raise ModelError.missing_file(entry.file)
+    stride, n = layout.expert_stride, layout.experts_per_layer
+    file_size = os.path.getsize(path)
+    for e in entry.experts:
+        if e.size > stride or e.offset + e.size > file_size:
+            raise ModelError.index_corrupt(f"{entry.file}: expert {e.expert} lies outside the file")
+    pool = torch.empty((n * stride,), dtype=torch.uint8, device=device)
+    src = np.memmap(path, dtype=np.uint8, mode="r")
+    in_order = all(e.offset == i * stride and e.size == stride for i, e in enumerate(entry.experts))
+    chunk = max(stride, 64 << 20) // stride * stride
+    use_pin = torch.device(device).type == "cuda"
+    stage = torch.empty((chunk,), dtype=torch.uint8, pin_memory=use_pin)
+    stage_np = stage.numpy()
+    if in_order:
+        for pos in range(0, n * stride, chunk):
+            m = min(chunk, n * stride - pos)
+            stage_np[:m] = src[pos:pos + m]
+            pool[pos:pos + m].copy_(stage[:m], non_blocking=False)
+    else:
+        per = chunk // stride
+        for e0 in range(0, n, per):
+            cnt = min(per, n - e0)
+            stage_np[:cnt * stride] = 0
+            for j in range(cnt):
+                e = entry.experts[e0 + j]
+                stage_np[j * stride:j * stride + e.size] = src[e.offset:e.offset + e.size]
+            pool[e0 * stride:(e0 + cnt) * stride].copy_(stage[:cnt * stride], non_blocking=False)
+    del src
+    return pool, stride

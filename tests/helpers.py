@@ -49,3 +49,46 @@ def assert_layer_close(actual: np.ndarray, ref: np.ndarray, what: str = ""):
     max_abs, rel_l2 = errors(actual, ref)
     assert max_abs <= MAX_ABS and rel_l2 <= REL_L2, (
         f"{what}: max_abs={max_abs:.3e} (<= {MAX_ABS}), rel_l2={rel_l2:.3e} (<= {REL_L2})")
+
+
+def write_packed_experts(directory, layer, physical_order=None, page=16384):
+    """Write `layer` (an oracle Layer) as the reference's packed_experts/ directory: layout.json
+    and layer_00.bin, every expert one blob at a stride rounded up to `page`
+    (RepackPlanner.swift:544-712); `physical_order[rank]` = logical expert stored at that rank."""
+    import json
+    import os
+    import numpy as np
+    d, f, e, bits = layer.d, layer.f, layer.e, layer.bits
+    blob = layer.experts.shape[1]
+    stride = (blob + page - 1) // page * page
+    order = list(range(e)) if physical_order is None else list(physical_order)
+    rank_of = {ex: r for r, ex in enumerate(order)}
+    pack_bits = 2 if bits == 1 else bits
+    gu_w, gu_s = f * d * pack_bits // 8, f * (d // 64) * 2
+    dn_w, dn_s = d * f * pack_bits // 8, d * (f // 64) * 2
+    off = layer.off
+    tensors = {
+        "gate": dict(offset=off.gate_w, size=gu_w, dtype="U32", shape=[f, d * pack_bits // 32], bits=pack_bits),
+        "gate_scales": dict(offset=off.gate_s, size=gu_s, dtype="BF16", shape=[f, d // 64]),
+        "up": dict(offset=off.up_w, size=gu_w, dtype="U32", shape=[f, d * pack_bits // 32], bits=pack_bits),
+        "up_scales": dict(offset=off.up_s, size=gu_s, dtype="BF16", shape=[f, d // 64]),
+        "down": dict(offset=off.down_w, size=dn_w, dtype="U32", shape=[d, f * pack_bits // 32], bits=pack_bits),
+        "down_scales": dict(offset=off.down_s, size=dn_s, dtype="BF16", shape=[d, f // 64]),
+    }
+    if bits != 1:
+        tensors["gate_biases"] = dict(offset=off.gate_b, size=gu_s, dtype="BF16", shape=[f, d // 64])
+        tensors["up_biases"] = dict(offset=off.up_b, size=gu_s, dtype="BF16", shape=[f, d // 64])
+        tensors["down_biases"] = dict(offset=off.down_b, size=dn_s, dtype="BF16", shape=[d, f // 64])
+    experts = [dict(expert=ex, physicalRank=rank_of[ex], offset=rank_of[ex] * stride, size=stride,
+                    tensors=tensors) for ex in range(e)]
+    root = dict(expertStride=stride, numLayers=1, expertsPerLayer=e,
+                layers=[dict(layer=0, file="layer_00.bin", experts=experts)])
+    pe = os.path.join(directory, "packed_experts")
+    os.makedirs(pe, exist_ok=True)
+    with open(os.path.join(pe, "layout.json"), "w") as fh:
+        json.dump(root, fh, sort_keys=True)
+    data = np.zeros((e, stride), np.uint8)
+    for r, ex in enumerate(order):
+        data[r, :blob] = layer.experts[ex]
+    data.tofile(os.path.join(pe, "layer_00.bin"))
+    return stride

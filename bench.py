@@ -218,7 +218,7 @@ def measure_prefill(ctx, w, layer, device, tokens=(128, 512, 2048), steps=100, w
     last = out["runs"][-1]
     out["roofline"] = {"bound": "mfma", "achieved": last["tflops"], "peak": MFMA_BF16_PEAK_TFLOPS,
                        "unit": "TFLOP/s", "frac": last["mfma_frac"], "traffic": None,
-                       "kernel": "whole layer at T=%d (router, grouping, mf::qmm_kernel x2, reduce); "
+                       "kernel": "whole layer at T=%d (router, grouping, mf::qmm_kernel, mf::qmm_kres_kernel, reduce); "
                                  "algorithmic flops = 2*3*D*(T*K*F + T*Fs)" % last["tokens"]}
     return out
 

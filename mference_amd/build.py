@@ -30,7 +30,25 @@ def build(verbose: bool = False) -> str:
         raise RuntimeError("hipcc failed building libmfmoe.so")
     if verbose and proc.stderr:
         sys.stderr.write(proc.stderr)
+    build_microbench(verbose)
     return LIB
+
+
+def build_microbench(verbose: bool = False) -> str:
+    """The stand-alone issue-port measurement (csrc/microbench/issue_port.hip): a program of its own,
+    not part of libmfmoe.so."""
+    hipcc = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
+    src = os.path.join(CSRC, "microbench", "issue_port.hip")
+    exe = os.path.join(CSRC, "microbench", "issue_port")
+    cmd = [hipcc, "--offload-arch=gfx950", "-O3", "-std=c++17", "-Xclang", "-target-feature", "-Xclang",
+           "-packed-fp32-ops", "-o", exe, src]
+    if verbose:
+        print(" ".join(cmd), flush=True)
+    proc = subprocess.run(cmd, capture_output=True, text=True)
+    if proc.returncode != 0:
+        sys.stderr.write(proc.stdout + proc.stderr)
+        raise RuntimeError("hipcc failed building microbench/issue_port")
+    return exe
 
 
 if __name__ == "__main__":

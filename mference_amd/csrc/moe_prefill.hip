@@ -427,6 +427,7 @@ struct QmmArgs {
   // epilogue
   int epi;              // 0 swiglu -> bf16 [pair, rows] in prep order; 1 fp32 [token*K+rank, rows]; 2 bf16 [pair, rows]
   int narrow;           // shared-expert rounding points (dequant_int4.metal:240-245)
+  int tab_aligned;      // scale / bias rows start on 16-byte boundaries (set by the launcher)
   void* out;
   uint32_t top_k;
   float limit;
@@ -566,24 +567,43 @@ void qmm_kernel(const QmmLaunch launch) {
       xs[gi][1] = *reinterpret_cast<const uint4*>(st_src + (2 + gi) * kGroup + 8);
     }
   }
+  // Scale and bias words of the lane's row and the group sums of its two routes, 8 K groups at a time
+  // (groups gl = g0 + 8h .. gl + 7 for g0 = 0, 16, ...); the loads of the first step leave now, with the
+  // codes and the x rows, the loads of every later step one step ahead of their use.
+  struct TabStep {
+    uint4 S[NPROJ], B[NPROJ];
+    float sx[2][8];
+  };
+  auto tab_fetch = [&](uint32_t g0) {
+    TabStep t;
+    const uint32_t gl = g0 + 8 * h;
+    const uint32_t gc = gl < ng ? gl : 0;  // a lane without groups reads group 0 and drops it
+#pragma unroll
+    for (int p = 0; p < NPROJ; ++p) {
+      const size_t at = static_cast<size_t>(row_base[p] + m) * ng + gc;
+      t.B[p] = NG8 ? (a.tab_aligned ? load_x8<true>(Bp[p] + at) : load_x8<false>(Bp[p] + at))
+                   : load_bf16x8_guarded(Bp[p] + at, ng - gc);
+      t.S[p] = NG8 ? (a.tab_aligned ? load_x8<true>(Sp[p] + at) : load_x8<false>(Sp[p] + at))
+                   : load_bf16x8_guarded(Sp[p] + at, ng - gc);
+    }
+#pragma unroll
+    for (int nt = 0; nt < 2; ++nt) {
+      const float* sp = a.sumx + static_cast<size_t>(xrow[nt]) * ng + gc;
+      if (NG8) {
+        const float4 s0 = *reinterpret_cast<const float4*>(sp), s1 = *reinterpret_cast<const float4*>(sp + 4);
+        t.sx[nt][0] = s0.x; t.sx[nt][1] = s0.y; t.sx[nt][2] = s0.z; t.sx[nt][3] = s0.w;
+        t.sx[nt][4] = s1.x; t.sx[nt][5] = s1.y; t.sx[nt][6] = s1.z; t.sx[nt][7] = s1.w;
+      } else {
+#pragma unroll
+        for (int e = 0; e < 8; ++e) t.sx[nt][e] = gc + e < ng ? sp[e] : 0.0f;
+      }
+    }
+    return t;
+  };
+  TabStep tab_cur = tab_fetch(0);
   qmm_trace(a, work, 1);
 
   if (threadIdx.x < kTileTokens) s_slot[threadIdx.x] = threadIdx.x < count ? slot : 0xFFFFFFFFu;
-  // 2 * scale (the codes enter as 8 + q/2) of the wave's rows, transposed to [g][row], as fp32
-#pragma unroll
-  for (int p = 0; p < NPROJ; ++p) {
-    float* tab = s_scale + (p * kQmmWaves + wv) * ng * 32;
-    const uint16_t* src = Sp[p] + static_cast<size_t>(row_base[p] + m) * ng;
-    for (uint32_t g0 = h * 8; g0 < ng; g0 += 16) {  // lane: row m, 8 groups from g0
-      const uint4 v = NG8 ? load_x8<false>(src + g0) : load_bf16x8_guarded(src + g0, ng - g0);
-      const uint32_t pr[4] = {v.x, v.y, v.z, v.w};
-#pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        if (NG8 || g0 + 2 * i < ng) tab[(g0 + 2 * i) * 32 + m] = 2.0f * bf16_lo(pr[i]);
-        if (NG8 || g0 + 2 * i + 1 < ng) tab[(g0 + 2 * i + 1) * 32 + m] = 2.0f * bf16_hi(pr[i]);
-      }
-    }
-  }
 
   f32x16_t acc[NPROJ][2];
 #pragma unroll
@@ -593,40 +613,37 @@ void qmm_kernel(const QmmLaunch launch) {
 #pragma unroll
       for (int r = 0; r < 16; ++r) acc[p][nt][r] = 0.0f;
 
-  // ---- bias and offset terms: acc[token, row] += sumx[token, g] * B[row, g] + sumx[token, g] * (-16 S[row, g]).
+  // ---- per step: 2 * scale (the codes enter as 8 + q/2) of the wave's rows into the [g][row] fp32 table,
+  // and the bias and offset terms: acc[token, row] += sumx[token, g] * B[row, g] + sumx[token, g] * (-16 S[row, g]).
   // -16 * S is formed in place (exponent + 4, sign flipped: exact; a zero scale becomes 2^-123).
   // sumx enters as three bf16 terms, which hold all 24 bits: the -16 * S * sumx term cancels the
   // 16 * sum(x) the matrix core accumulated with the codes, so it has to be exact.
   for (uint32_t g0 = 0; g0 < ng; g0 += 16) {
-    const uint32_t gl = g0 + 8 * h;  // this lane's 8 groups
+    const TabStep t = tab_cur;
+    tab_cur = tab_fetch(g0 + 16 < ng ? g0 + 16 : g0);  // past the end: the same step again, unused
+    const uint32_t gl = g0 + 8 * h;
     const bool have = gl < ng;
-    const uint32_t gc = have ? gl : 0;  // a lane without groups reads group 0 and drops it
     uint4 ab[NPROJ], as[NPROJ];
 #pragma unroll
     for (int p = 0; p < NPROJ; ++p) {
-      const size_t at = static_cast<size_t>(row_base[p] + m) * ng + gc;
-      ab[p] = NG8 ? load_x8<false>(Bp[p] + at) : load_bf16x8_guarded(Bp[p] + at, ng - gc);
-      const uint4 sv = NG8 ? load_x8<false>(Sp[p] + at) : load_bf16x8_guarded(Sp[p] + at, ng - gc);
-      as[p] = make_uint4((sv.x + 0x02000200u) ^ 0x80008000u, (sv.y + 0x02000200u) ^ 0x80008000u,
-                         (sv.z + 0x02000200u) ^ 0x80008000u, (sv.w + 0x02000200u) ^ 0x80008000u);
+      float* tab = s_scale + (p * kQmmWaves + wv) * ng * 32;
+      const uint32_t pr[4] = {t.S[p].x, t.S[p].y, t.S[p].z, t.S[p].w};
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        if (have && (NG8 || gl + 2 * i < ng)) tab[(gl + 2 * i) * 32 + m] = 2.0f * bf16_lo(pr[i]);
+        if (have && (NG8 || gl + 2 * i + 1 < ng)) tab[(gl + 2 * i + 1) * 32 + m] = 2.0f * bf16_hi(pr[i]);
+      }
+      ab[p] = t.B[p];
+      as[p] = make_uint4((t.S[p].x + 0x02000200u) ^ 0x80008000u, (t.S[p].y + 0x02000200u) ^ 0x80008000u,
+                         (t.S[p].z + 0x02000200u) ^ 0x80008000u, (t.S[p].w + 0x02000200u) ^ 0x80008000u);
       if (!have) ab[p] = as[p] = make_uint4(0, 0, 0, 0);
     }
 #pragma unroll
     for (int nt = 0; nt < 2; ++nt) {
-      float sx[8];
-      const float* sp = a.sumx + static_cast<size_t>(xrow[nt]) * ng + gc;
-      if (NG8) {
-        const float4 s0 = *reinterpret_cast<const float4*>(sp), s1 = *reinterpret_cast<const float4*>(sp + 4);
-        sx[0] = s0.x; sx[1] = s0.y; sx[2] = s0.z; sx[3] = s0.w;
-        sx[4] = s1.x; sx[5] = s1.y; sx[6] = s1.z; sx[7] = s1.w;
-      } else {
-#pragma unroll
-        for (int e = 0; e < 8; ++e) sx[e] = gc + e < ng ? sp[e] : 0.0f;
-      }
       uint32_t hi[8], mid[8], lo[8];
 #pragma unroll
       for (int e = 0; e < 8; ++e) {
-        const float v = sx[e];
+        const float v = t.sx[nt][e];
         hi[e] = __float_as_uint(v) & 0xFFFF0000u;
         const float r1 = v - __uint_as_float(hi[e]);
         mid[e] = __float_as_uint(r1) & 0xFFFF0000u;
@@ -808,6 +825,294 @@ void qmm_kernel(const QmmLaunch launch) {
   qmm_trace(a, work, 4);
 }
 
+// ---- the same product for a short contraction (K <= 512: the down projections) ----
+// With K this short the x tile of a workgroup (64 routes x K bf16 <= 64 KB) stays in LDS whole, so a
+// workgroup stages it once and then walks over `slices` consecutive 256-row slices of the weight matrix
+// without any further workgroup barrier: the waves run free, each wave's next-slice codes and scale / bias
+// words are requested while it still multiplies the current slice, and the stores of a finished slice
+// drain while the next one starts.  (qmm_kernel re-stages x through a two-stage ring for every 128 or 256
+// rows, four barriers per 8 groups, and pays its set-up -- tile, routes, tables, 3 us -- per slice.)
+// A wave owns two consecutive 32-row blocks (64 rows).  Routes past the tile's count repeat the tile's
+// last route in every respect, its output slot included: they store the same values to the same place,
+// and no store needs a branch.
+struct KresLaunch {
+  QmmArgs part[2];
+  uint32_t per_xcd[2];   // work items of each part on one XCD (grid = 8 * their sum)
+  uint32_t slices[2];    // 256-row slices one work item walks (divides rows / 256)
+};
+
+template <int NG> __device__ __forceinline__ uint4 load_groups_bf16(const uint16_t* p) {  // NG bf16, zero-padded to 8
+  if constexpr (NG >= 8) {
+    return *reinterpret_cast<const uint4*>(p);
+  } else if constexpr (NG == 4) {
+    const uint2 v = *reinterpret_cast<const uint2*>(p);
+    return make_uint4(v.x, v.y, 0, 0);
+  } else {
+    return make_uint4(*reinterpret_cast<const uint32_t*>(p), 0, 0, 0);
+  }
+}
+
+template <int NG>
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2)))
+void qmm_kres_kernel(const KresLaunch launch) {
+  static_assert(NG == 2 || NG == 4 || NG == 8, "K is 128, 256 or 512");
+  constexpr int kRing = NG < 4 ? NG : 4;  // code registers in flight per projection
+  extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
+  const uint32_t lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
+  const uint32_t m = lane & 31, h = lane >> 5;
+  const uint32_t xcd_slot = blockIdx.x >> 3;
+  const bool second = xcd_slot >= launch.per_xcd[0];
+  const QmmArgs& a = launch.part[second ? 1 : 0];
+  const uint32_t work = (blockIdx.x & 7u) * launch.per_xcd[second ? 1 : 0] + (xcd_slot - (second ? launch.per_xcd[0] : 0u));
+  const uint32_t n_walk = launch.slices[second ? 1 : 0];
+  const uint32_t items_per_tile = a.rows / (256u * n_walk);
+  const uint32_t tile_id = work / items_per_tile, slice0 = (work % items_per_tile) * n_walk;
+  qmm_trace(a, work, 0);
+
+  uint32_t expert = 0, pair_start, count;
+  if (a.dense_mode) {
+    if (tile_id >= a.dense_tiles) return;
+    pair_start = tile_id * kTileTokens;
+    count = min(kTileTokens, a.dense_rows - pair_start);
+  } else {
+    const Tile t = a.tiles[tile_id];
+    if (t.count == 0) return;
+    expert = t.expert;
+    pair_start = t.pair_start;
+    count = t.count;
+  }
+  uint4* s_x = reinterpret_cast<uint4*>(smem);                       // [NG groups][512]
+  uint32_t* s_slot = reinterpret_cast<uint32_t*>(smem + NG * 8192);  // [64]
+
+  const uint8_t* W;
+  const uint16_t* Sp;
+  const uint16_t* Bp;
+  if (a.dense_mode) {
+    W = static_cast<const uint8_t*>(a.dense[0].weights);
+    Sp = a.dense[0].scales;
+    Bp = a.dense[0].biases;
+  } else {
+    const uint8_t* blob = a.expert_base + static_cast<size_t>(expert) * a.expert_stride;
+    W = blob + a.w_off[0];
+    Sp = reinterpret_cast<const uint16_t*>(blob + a.s_off[0]);
+    Bp = reinterpret_cast<const uint16_t*>(blob + a.b_off[0]);
+  }
+  constexpr uint32_t kRowBytes = NG * 32;
+  // the lane's weight row of block p of slice w: row0 + 256 w + 32 p
+  const uint32_t row0 = (slice0 * kQmmWaves + wv) * 64 + m;
+  const uint8_t* wrow = W + static_cast<size_t>(row0) * kRowBytes + h * 16;
+  const uint16_t* srow = Sp + static_cast<size_t>(row0) * NG;
+  const uint16_t* brow = Bp + static_cast<size_t>(row0) * NG;
+
+  // ---- everything issued back to back: codes of the first slice, its scale / bias words, the x tile
+  uint4 cur[2][kRing];
+#pragma unroll
+  for (int p = 0; p < 2; ++p)
+#pragma unroll
+    for (int u = 0; u < kRing; ++u) cur[p][u] = *reinterpret_cast<const uint4*>(wrow + p * 32 * kRowBytes + u * 32);
+  uint4 nS[2], nB[2];
+#pragma unroll
+  for (int p = 0; p < 2; ++p) {
+    nS[p] = load_groups_bf16<NG>(srow + p * 32 * NG);
+    nB[p] = load_groups_bf16<NG>(brow + p * 32 * NG);
+  }
+  const uint32_t st_i = threadIdx.x >> 2, st_q = threadIdx.x & 3;  // staging: route i, K values 16q..16q+15 of a group
+  const uint16_t* st_src = a.x + static_cast<size_t>(pair_start + min(st_i, count - 1)) * a.x_stride + st_q * 16;
+  typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
+  u32x4_t xv[2 * NG];
+#pragma unroll
+  for (int g = 0; g < 2 * NG; ++g) xv[g] = *reinterpret_cast<const u32x4_t*>(st_src + (g >> 1) * kGroup + (g & 1) * 8);
+  // group sums of the lane's two routes (both halves of the wave hold them: K slots 8h..8h+7 of the
+  // bias product are the groups 0..7 again, multiplied by the biases for h = 0 and by -16 scale for h = 1)
+  float sx[2][8];
+#pragma unroll
+  for (int nt = 0; nt < 2; ++nt) {
+    const float* sp = a.sumx + static_cast<size_t>(pair_start + min(nt * 32 + m, count - 1)) * NG;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) sx[nt][e] = 0.0f;
+    if constexpr (NG >= 8) {
+      const float4 s0 = *reinterpret_cast<const float4*>(sp), s1 = *reinterpret_cast<const float4*>(sp + 4);
+      sx[nt][0] = s0.x; sx[nt][1] = s0.y; sx[nt][2] = s0.z; sx[nt][3] = s0.w;
+      sx[nt][4] = s1.x; sx[nt][5] = s1.y; sx[nt][6] = s1.z; sx[nt][7] = s1.w;
+    } else if constexpr (NG == 4) {
+      const float4 s0 = *reinterpret_cast<const float4*>(sp);
+      sx[nt][0] = s0.x; sx[nt][1] = s0.y; sx[nt][2] = s0.z; sx[nt][3] = s0.w;
+    } else {
+      const float2 s0 = *reinterpret_cast<const float2*>(sp);
+      sx[nt][0] = s0.x; sx[nt][1] = s0.y;
+    }
+  }
+  uint32_t slot = 0;
+  if (threadIdx.x < kTileTokens) {
+    const uint32_t pi = pair_start + min(threadIdx.x, count - 1);
+    slot = pi;
+    if (!a.dense_mode && a.epi == 1) {
+      const mf_pair pr = a.sorted[pi];
+      slot = pr.token * a.top_k + pr.rank;
+    }
+  }
+  qmm_trace(a, work, 1);
+
+  // ---- x tile into LDS (the layout qmm_kernel's ring uses for one group, NG times)
+  {
+    const uint32_t st_nt = st_i >> 5, st_n = st_i & 31, c0 = 2 * st_q, c1 = c0 + 1;
+    const uint32_t st_rot = 4 * ((c0 & 3) >> 1) + 8 * (c0 >> 2);
+    const uint32_t st_slot0 = ((st_nt * 4 + (c0 & 3)) * 2 + (c0 >> 2)) * 32 + ((st_n + st_rot) & 31);
+    const uint32_t st_slot1 = ((st_nt * 4 + (c1 & 3)) * 2 + (c1 >> 2)) * 32 + ((st_n + st_rot) & 31);
+#pragma unroll
+    for (int g = 0; g < NG; ++g) {
+      *reinterpret_cast<u32x4_t*>(s_x + g * 512 + st_slot0) = xv[2 * g];
+      *reinterpret_cast<u32x4_t*>(s_x + g * 512 + st_slot1) = xv[2 * g + 1];
+    }
+    if (threadIdx.x < kTileTokens) s_slot[threadIdx.x] = slot;
+  }
+  // sum(x) of a group as three bf16 terms (all 24 bits), see qmm_kernel
+  uint4 b_term[2][3];
+#pragma unroll
+  for (int nt = 0; nt < 2; ++nt) {
+    uint32_t hi[8], mid[8], lo[8];
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      const float v = sx[nt][e];
+      hi[e] = __float_as_uint(v) & 0xFFFF0000u;
+      const float r1 = v - __uint_as_float(hi[e]);
+      mid[e] = __float_as_uint(r1) & 0xFFFF0000u;
+      lo[e] = __float_as_uint(r1 - __uint_as_float(mid[e]));
+    }
+    b_term[nt][0] = make_uint4((hi[0] >> 16) | hi[1], (hi[2] >> 16) | hi[3], (hi[4] >> 16) | hi[5], (hi[6] >> 16) | hi[7]);
+    b_term[nt][1] = make_uint4((mid[0] >> 16) | mid[1], (mid[2] >> 16) | mid[3], (mid[4] >> 16) | mid[5],
+                               (mid[6] >> 16) | mid[7]);
+    b_term[nt][2] = make_uint4(__builtin_amdgcn_perm(lo[1], lo[0], 0x07060302u), __builtin_amdgcn_perm(lo[3], lo[2], 0x07060302u),
+                               __builtin_amdgcn_perm(lo[5], lo[4], 0x07060302u), __builtin_amdgcn_perm(lo[7], lo[6], 0x07060302u));
+  }
+  uint32_t rd_col[4];
+#pragma unroll
+  for (int sidx = 0; sidx < 4; ++sidx) rd_col[sidx] = (m + 4 * (sidx >> 1) + 8 * h) & 31;
+  __syncthreads();  // the only workgroup barrier: from here on the waves run on their own
+  qmm_trace(a, work, 2);
+
+  for (uint32_t w = 0; w < n_walk; ++w) {
+    const uint32_t step = w + 1 < n_walk ? 1u : 0u;  // the last slice requests itself again: no branch around loads
+    const uint8_t* wnext = wrow + static_cast<size_t>(step) * 256 * kRowBytes;
+    // scale words of this slice; bias operand: the biases for K slots 0..7, -16 scale for K slots 8..15
+    // (-16 * S formed in place: exponent + 4, sign flipped -- exact; a zero scale becomes 2^-123)
+    uint4 Sv[2], bop[2];
+#pragma unroll
+    for (int p = 0; p < 2; ++p) {
+      Sv[p] = nS[p];
+      const uint4 neg = make_uint4((nS[p].x + 0x02000200u) ^ 0x80008000u, (nS[p].y + 0x02000200u) ^ 0x80008000u,
+                                   (nS[p].z + 0x02000200u) ^ 0x80008000u, (nS[p].w + 0x02000200u) ^ 0x80008000u);
+      bop[p] = h ? neg : nB[p];
+    }
+    f32x16_t acc[2][2];
+#pragma unroll
+    for (int p = 0; p < 2; ++p)
+#pragma unroll
+      for (int nt = 0; nt < 2; ++nt) {
+#pragma unroll
+        for (int r = 0; r < 16; ++r) acc[p][nt][r] = 0.0f;
+#pragma unroll
+        for (int term = 0; term < 3; ++term) acc[p][nt] = mfma_bf16(b_term[nt][term], bop[p], acc[p][nt]);
+      }
+    // the next slice's scale / bias words (the registers are free again)
+    srow += step * 256 * NG;
+    brow += step * 256 * NG;
+#pragma unroll
+    for (int p = 0; p < 2; ++p) {
+      nS[p] = load_groups_bf16<NG>(srow + p * 32 * NG);
+      nB[p] = load_groups_bf16<NG>(brow + p * 32 * NG);
+    }
+    // x of a group comes out of LDS one group ahead, into the registers the matrix core has just read
+    uint4 bx[2][4];
+    if (w == 0) {
+#pragma unroll
+      for (int nt = 0; nt < 2; ++nt)
+#pragma unroll
+        for (int s = 0; s < 4; ++s) bx[nt][s] = s_x[((nt * 4 + s) * 2 + h) * 32 + rd_col[s]];
+    }
+#pragma unroll
+    for (int g = 0; g < NG; ++g) {
+      const uint4* nbuf = s_x + ((g + 1) % NG) * 512;  // after the last group: group 0 again, for the next slice
+#pragma unroll
+      for (int p = 0; p < 2; ++p) {
+        const uint4 cv = cur[p][g % kRing];
+        const uint32_t cw[4] = {cv.x, cv.y, cv.z, cv.w};
+        const uint32_t sw[4] = {Sv[p].x, Sv[p].y, Sv[p].z, Sv[p].w};
+        const float sc = 2.0f * ((g & 1) ? bf16_hi(sw[g >> 1]) : bf16_lo(sw[g >> 1]));  // codes enter as 8 + q/2
+        f32x16_t tmp[2];
+#pragma unroll
+        for (int nt = 0; nt < 2; ++nt)
+#pragma unroll
+          for (int r = 0; r < 16; ++r) tmp[nt][r] = 0.0f;
+#pragma unroll
+        for (int s = 0; s < 4; ++s) {
+          const uint4 av = expand_q4(cw[s]);
+          tmp[0] = mfma_bf16(bx[0][s], av, tmp[0]);
+          tmp[1] = mfma_bf16(bx[1][s], av, tmp[1]);
+          if (p == 1) {
+            bx[0][s] = nbuf[((0 * 4 + s) * 2 + h) * 32 + rd_col[s]];
+            bx[1][s] = nbuf[((1 * 4 + s) * 2 + h) * 32 + rd_col[s]];
+          }
+        }
+        // the register takes the codes kRing groups on: of this slice, or of the next one
+        const int ahead = g + kRing;
+        cur[p][g % kRing] = ahead < NG
+            ? *reinterpret_cast<const uint4*>(wrow + p * 32 * kRowBytes + ahead * 32)
+            : *reinterpret_cast<const uint4*>(wnext + p * 32 * kRowBytes + (ahead - NG) * 32);
+#pragma unroll
+        for (int nt = 0; nt < 2; ++nt)
+#pragma unroll
+          for (int r = 0; r < 16; ++r) acc[p][nt][r] = __builtin_fmaf(sc, tmp[nt][r], acc[p][nt][r]);
+        // the sums are wanted here, not after the last group: without this the compiler keeps every
+        // group's products and adds them up at the end of the slice, out of scratch memory
+        asm volatile("" : "+v"(acc[p][0]), "+v"(acc[p][1]));
+        __builtin_amdgcn_sched_barrier(0);  // one unit at a time: hoisted loads would cost more registers than exist
+      }
+    }
+    if (w + 1 == n_walk) qmm_trace(a, work, 3);
+    // ---- stores: the lane holds rows row + 32 p for routes 8j + 4h + i of each 32-route block
+    const uint32_t row = row0 + w * 256;
+    // byte offsets fit 32 bits (the launcher checks): one multiply-add per route, the base stays scalar
+    if (a.epi == 1) {
+      uint8_t* out = static_cast<uint8_t*>(a.out);
+      const uint32_t pitch = a.rows * 4, col = row * 4;
+#pragma unroll
+      for (int nt = 0; nt < 2; ++nt) {
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          const uint4 sl = *reinterpret_cast<const uint4*>(s_slot + nt * 32 + 8 * j + 4 * h);
+          const uint32_t sl4[4] = {sl.x, sl.y, sl.z, sl.w};
+#pragma unroll
+          for (int i = 0; i < 4; ++i) {
+            float* o = reinterpret_cast<float*>(out + (sl4[i] * pitch + col));
+            o[0] = acc[0][nt][4 * j + i];
+            o[32] = acc[1][nt][4 * j + i];
+          }
+        }
+      }
+    } else {
+      uint8_t* out = static_cast<uint8_t*>(a.out);
+      const uint32_t pitch = a.rows * 2, col = row * 2;
+#pragma unroll
+      for (int nt = 0; nt < 2; ++nt) {
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          const uint4 sl = *reinterpret_cast<const uint4*>(s_slot + nt * 32 + 8 * j + 4 * h);
+          const uint32_t sl4[4] = {sl.x, sl.y, sl.z, sl.w};
+#pragma unroll
+          for (int i = 0; i < 4; ++i) {
+            uint16_t* o = reinterpret_cast<uint16_t*>(out + (sl4[i] * pitch + col));
+            o[0] = f_to_bf16(acc[0][nt][4 * j + i]);
+            o[32] = f_to_bf16(acc[1][nt][4 * j + i]);
+          }
+        }
+      }
+    }
+    wrow = wnext;
+  }
+  qmm_trace(a, work, 4);
+}
+
 // y[t,d] = bf16(h1[t,d] + sum_r w[t,r] * partial[t*K+r, d]), residual first, rank
 // order, product then add (moe.metal:1262-1270; reduce of prefill.metal:631-652).
 // h1 = bf16(hs / (1 + exp(-gate_t))) when a scalar gate is given (utility.metal:49-59).
@@ -905,6 +1210,50 @@ hipError_t launch_prep_rows(hipStream_t s, const uint16_t* src, uint16_t* dst, f
   return hipGetLastError();
 }
 
+// Whether qmm_kres_kernel takes the problem: a down-projection epilogue, K of 128, 256 or 512, whole
+// 256-row slices, tables aligned for vector loads.
+bool kres_takes(const QmmArgs& q, size_t out_rows) {
+  const uint32_t ng = q.kdim / kGroup;
+  if (q.epi == 0 || q.gather || q.kdim % kGroup || !(ng == 2 || ng == 4 || ng == 8) || q.rows % 256) return false;
+  if (static_cast<uint64_t>(out_rows) * q.rows * 4 >= (1ull << 32)) return false;  // 32-bit store offsets
+  if (q.dense_mode) return aligned16(q.dense[0].scales) && aligned16(q.dense[0].biases) && aligned16(q.dense[0].weights);
+  return aligned16(q.expert_base) && q.expert_stride % 16 == 0 && (q.w_off[0] | q.s_off[0] | q.b_off[0]) % 16 == 0;
+}
+
+hipError_t launch_qmm_kres(hipStream_t s, const QmmArgs& a, uint32_t tile_slots, const QmmArgs* b, uint32_t b_tile_slots) {
+  KresLaunch launch{};
+  for (int part = 0; part < (b ? 2 : 1); ++part) {
+    QmmArgs& q = launch.part[part];
+    q = part ? *b : a;
+    uint32_t slots = part ? b_tile_slots : tile_slots;
+    if (q.dense_mode) {
+      q.dense_tiles = slots;
+      slots = (slots + 7) / 8 * 8;
+    }
+    const uint32_t n_slices = q.rows / 256;
+    // two slices per work item halve the set-up per slice and still leave several rounds of work items
+    // (Qwen shape, 2048 tokens, whole layer: 331 us with one slice, 325 with two, 330 with four, 334 with eight)
+    const uint32_t walk = n_slices % 2 == 0 ? 2 : 1;
+    launch.slices[part] = walk;
+    launch.per_xcd[part] = slots / 8 * (n_slices / walk);
+  }
+  const dim3 grid(8 * (launch.per_xcd[0] + launch.per_xcd[1])), block(256);
+  if (grid.x == 0) return hipSuccess;
+  const uint32_t ng = a.kdim / kGroup;
+  const size_t lds = static_cast<size_t>(ng) * 8192 + kTileTokens * 4;
+  const void* fn = ng == 8 ? reinterpret_cast<const void*>(qmm_kres_kernel<8>)
+                 : ng == 4 ? reinterpret_cast<const void*>(qmm_kres_kernel<4>)
+                           : reinterpret_cast<const void*>(qmm_kres_kernel<2>);
+  if (lds > 48 * 1024) {
+    hipError_t e = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds));
+    if (e != hipSuccess) return e;
+  }
+  if (ng == 8) qmm_kres_kernel<8><<<grid, block, lds, s>>>(launch);
+  else if (ng == 4) qmm_kres_kernel<4><<<grid, block, lds, s>>>(launch);
+  else qmm_kres_kernel<2><<<grid, block, lds, s>>>(launch);
+  return hipGetLastError();
+}
+
 // tile_slots: entries of the tile list (routed; a multiple of 8) or number of 64-row tiles (dense).
 // `b` (optional) is a second problem for the same instantiation, run behind `a` in the same launch.
 hipError_t launch_qmm(hipStream_t s, QmmArgs a, int nproj, uint32_t tile_slots, const QmmArgs* b,
@@ -922,6 +1271,11 @@ hipError_t launch_qmm(hipStream_t s, QmmArgs a, int nproj, uint32_t tile_slots, 
       slots = (slots + 7) / 8 * 8;
     }
     launch.per_xcd[part] = slots / 8 * n_slices;
+    q.tab_aligned = q.dense_mode
+        ? aligned16(q.dense[0].scales) && aligned16(q.dense[0].biases) && aligned16(q.dense[1].scales) &&
+              aligned16(q.dense[1].biases)
+        : aligned16(q.expert_base) && q.expert_stride % 16 == 0 &&
+              (q.s_off[0] | q.b_off[0] | q.s_off[1] | q.b_off[1]) % 16 == 0;
     lds = std::max(lds, qmm_lds_bytes(q.kdim, nproj));
     ng8 = ng8 && (q.kdim / kGroup) % 8 == 0;
   }
@@ -1068,7 +1422,10 @@ hipError_t launch_prefill_layer(hipStream_t s, const mf_moe& h, const mf_moe_lay
     d.x = ws.sact; d.sumx = ws.sum_sact; d.x_stride = c.shared_f; d.rows = c.d; d.kdim = c.shared_f; d.epi = 2; d.out = ws.hs;
     d.pair_rows = q.pair_rows;
   }
-  MF_TRY(launch_qmm(s, q, q.pair_rows ? 2 : 1, max_tiles, c.shared_f ? &d : nullptr, dense_tiles));
+  if (kres_takes(q, pairs) && (!c.shared_f || (kres_takes(d, t) && d.kdim == q.kdim)))
+    MF_TRY(launch_qmm_kres(s, q, max_tiles, c.shared_f ? &d : nullptr, dense_tiles));
+  else
+    MF_TRY(launch_qmm(s, q, q.pair_rows ? 2 : 1, max_tiles, c.shared_f ? &d : nullptr, dense_tiles));
   const uint16_t* hs = nullptr;
   const uint16_t* gate = nullptr;
   if (c.shared_f) {

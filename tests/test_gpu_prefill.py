@@ -74,6 +74,8 @@ def _run_prefill(moe, wts, x, t, d, k):
     (512, 256, 32, 8, 256, 200, 0, 7.0),    # SwiGLU clamp (moe.metal:1080-1094)
     (384, 128, 32, 2, 128, 131, 1, 0.0),    # full-softmax router, ng not a multiple of 8
     (2048, 512, 256, 8, 512, 96, 0, 0.0),   # the headline layer shape
+    (512, 256, 16, 4, 128, 90, 0, 0.0),     # shared width != routed width: the two down projections differ in K
+    (256, 384, 16, 4, 384, 67, 0, 0.0),     # K of the down projection not 128, 256 or 512
 ])
 def test_prefill_layer_matches_per_token_oracle(gpu, oracle, d, f, e, k, fs, t, mode, limit):
     root = ROOT_SEED + 0xA000 + d + t

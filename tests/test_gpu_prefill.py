@@ -195,3 +195,34 @@ def test_prefill_full_size_rows_do_not_depend_on_their_neighbours(gpu, oracle):
         assert torch.equal(idd[0], idx[i])
         assert_layer_close(oracle.bf16_to_float(ops.bf16_bits(y[i:i + 1])),
                            oracle.bf16_to_float(ops.bf16_bits(yd)), f"prefill row {i} vs decode")
+
+
+def test_prefill_16k_tokens_repeat_the_2048_token_rows(gpu):
+    """16 384 tokens (131 072 routes, 2 000+ tiles, 1 GiB of per-route partial rows -- byte offsets
+    of the down projection's stores reach 2^30): the batch is the 2048-token batch eight times
+    over, so every block of 2048 output rows equals the rows of the 2048-token call bit for bit."""
+    import bench
+    w = dict(bench.QWEN)
+    dev = torch.device("cuda", 0)
+    lw = bench.build_stack(gpu, w, 1, dev)[0]
+    gen = torch.Generator(device=dev)
+    gen.manual_seed(4242)
+    router = lw.router_w.clone()
+    router[:, -1] = (torch.randn((w["e"],), generator=gen, device=dev) * 1.5).to(torch.bfloat16)
+    lw = ops.MoELayerWeights(router, lw.experts, lw.offsets, lw.shared, lw.w_sg)
+    moe = ops.MoE(gpu, w["d"], w["f"], w["e"], w["k"], bits=4, shared_f=w["fs"], shared_bits=4)
+    t, d, k, reps = 2048, w["d"], w["k"], 8
+    x = torch.randn((t, d), generator=gen, device=dev).to(torch.bfloat16)
+    x[:, -1] = 1.0
+    y = torch.zeros_like(x)
+    idx = torch.zeros((t, k), dtype=torch.int32, device=dev)
+    moe.encode_prefill_layer(lw, x, y, t, out_indices=idx)
+    torch.cuda.synchronize()
+    xb = x.repeat(reps, 1).contiguous()
+    yb = torch.zeros_like(xb)
+    idxb = torch.zeros((t * reps, k), dtype=torch.int32, device=dev)
+    moe.encode_prefill_layer(lw, xb, yb, t * reps, out_indices=idxb)
+    torch.cuda.synchronize()
+    assert bool(torch.isfinite(yb.float()).all())
+    assert torch.equal(idxb.view(reps, t, k), idx.expand(reps, t, k))
+    assert torch.equal(yb.view(torch.int16).view(reps, t, d), y.view(torch.int16).expand(reps, t, d))

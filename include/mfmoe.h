@@ -297,10 +297,12 @@ mf_status mf_group_pairs_host(const mf_pair* pairs, size_t n_pairs, int query_co
  * (PrefillMoE.swift:11-38) + PrefillSharedExpert.encodeBlock/encodeQwenScalarGate
  * (PrefillSharedExpert.swift:81-99, 27-36).  Result per token equals
  * mf_moe_decode_layer on that token within the layer tolerance.
- * Any t >= 1.  The matrix-core path takes 4-bit experts with d, f, shared_f multiples of
- * 128 and x, y and every weight tensor 16-byte aligned; every other configuration (2-bit,
- * ternary, other widths) runs the same rows through the decode launch, MF_MAX_TOKENS at a
- * time, and needs no workspace.
+ * Any t >= 1.  The matrix-core path takes 4-bit, 2-bit and ternary experts (with a 4-bit
+ * shared expert, if any) with d, f, shared_f multiples of 128 and x, y and every weight
+ * tensor 16-byte aligned; every other configuration (other widths, another shared-expert
+ * format) runs the same rows through the decode launch, MF_MAX_TOKENS at a time, and needs
+ * no workspace.  Covers MoEDeepseekV4's pair-major 2-bit prefill
+ * (Metal/MoE/moe.metal:1293-1409) with the same call.
  * workspace: device scratch of at least mf_moe_prefill_workspace_bytes(h, t) (0 when the
  * configuration takes the decode launch; workspace may then be null). */
 size_t mf_moe_prefill_workspace_bytes(const mf_moe* h, uint32_t t);

@@ -282,6 +282,71 @@ __device__ __forceinline__ uint4 expand_q4(uint32_t w) {
                     and_or(w >> 5, 0x00780078u, kMagic8), and_or(w >> 9, 0x00780078u, kMagic8));
 }
 
+// one packed word of sixteen 2-bit codes -> two MFMA operands in the same pairing: the byte swap
+// (B0, B2, B1, B3) puts code r and code r + 4 sixteen bits apart, and likewise 8 + r and 12 + r, so
+// a = (q0,q4),(q1,q5),(q2,q6),(q3,q7) and b = (q8,q12),...,(q11,q15) as the bf16 numbers 4 + q
+// (exponent 2^2, the code in mantissa bits 5..6): the x order of the 4-bit form serves both.
+__device__ __forceinline__ void expand_q2(uint32_t w, uint4& a, uint4& b) {
+  const uint32_t v = __builtin_amdgcn_perm(w, w, 0x03010200u);
+  a = make_uint4(and_or(v << 5, 0x00600060u, kMagic4), and_or(v << 3, 0x00600060u, kMagic4),
+                 and_or(v << 1, 0x00600060u, kMagic4), and_or(v >> 1, 0x00600060u, kMagic4));
+  b = make_uint4(and_or(v >> 3, 0x00600060u, kMagic4), and_or(v >> 5, 0x00600060u, kMagic4),
+                 and_or(v >> 7, 0x00600060u, kMagic4), and_or(v >> 9, 0x00600060u, kMagic4));
+}
+
+// What the quantized matmuls need to know about a code width: a lane's share of one 64-wide group
+// of its weight row is half the group -- 16 bytes of 4-bit codes or 8 bytes of 2-bit codes (ternary
+// weights are 2-bit codes) -- and it becomes four MFMA operands of 8 bf16 numbers offset + q * step.
+template <int BITS> struct QmmCodes;
+template <> struct QmmCodes<4> {
+  static constexpr uint32_t kGroupBytes = 32;     // one group of one row
+  static constexpr uint32_t kNegOffsetAdd = 0x02000200u;  // exponent + 4: 16 * scale (offset 8 at step 1/2)
+  static constexpr float kScaleMul = 2.0f;        // codes enter as 8 + q/2
+  uint32_t w[4];
+  __device__ __forceinline__ void load(const uint8_t* p) {
+    const uint4 v = *reinterpret_cast<const uint4*>(p);
+    w[0] = v.x; w[1] = v.y; w[2] = v.z; w[3] = v.w;
+  }
+};
+template <> struct QmmCodes<2> {
+  static constexpr uint32_t kGroupBytes = 16;
+  static constexpr uint32_t kNegOffsetAdd = 0x01000100u;  // exponent + 2: 4 * scale (offset 4 at step 1)
+  static constexpr float kScaleMul = 1.0f;        // codes enter as 4 + q
+  uint32_t w[2];
+  __device__ __forceinline__ void load(const uint8_t* p) {
+    const uint2 v = *reinterpret_cast<const uint2*>(p);
+    w[0] = v.x; w[1] = v.y;
+  }
+};
+
+// tmp[token block] += x * codes over one group: 8 MFMAs; `after(s)` runs once both token blocks have
+// issued theirs on operand s (the caller may then overwrite bx[.][s])
+template <int BITS, typename After>
+__device__ __forceinline__ void group_products(const QmmCodes<BITS>& c, const uint4 (&bx)[2][4], f32x16_t (&tmp)[2],
+                                               After after) {
+  if constexpr (BITS == 4) {
+#pragma unroll
+    for (int s = 0; s < 4; ++s) {
+      const uint4 av = expand_q4(c.w[s]);
+      tmp[0] = mfma_bf16(bx[0][s], av, tmp[0]);
+      tmp[1] = mfma_bf16(bx[1][s], av, tmp[1]);
+      after(s);
+    }
+  } else {
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+      uint4 a, b;
+      expand_q2(c.w[j], a, b);
+      tmp[0] = mfma_bf16(bx[0][2 * j], a, tmp[0]);
+      tmp[1] = mfma_bf16(bx[1][2 * j], a, tmp[1]);
+      after(2 * j);
+      tmp[0] = mfma_bf16(bx[0][2 * j + 1], b, tmp[0]);
+      tmp[1] = mfma_bf16(bx[1][2 * j + 1], b, tmp[1]);
+      after(2 * j + 1);
+    }
+  }
+}
+
 // 8 bf16 from p, of which only the first `avail` exist (the rest read as 0)
 __device__ __forceinline__ uint4 load_bf16x8_guarded(const uint16_t* p, uint32_t avail) {
   if (avail >= 8) return load_x8<false>(p);

@@ -428,6 +428,7 @@ struct QmmArgs {
   int epi;              // 0 swiglu -> bf16 [pair, rows] in prep order; 1 fp32 [token*K+rank, rows]; 2 bf16 [pair, rows]
   int narrow;           // shared-expert rounding points (dequant_int4.metal:240-245)
   int tab_aligned;      // scale / bias rows start on 16-byte boundaries (set by the launcher)
+  int ternary;          // 2-bit codes {0,1,2} with bias = -scale: b_off / dense[].biases name the SCALE table
   void* out;
   uint32_t top_k;
   float limit;
@@ -466,9 +467,10 @@ struct QmmLaunch {
   uint32_t per_xcd[2];  // work items of each part on one XCD (grid = 8 * their sum)
 };
 
-template <int NPROJ, bool NG8>
+template <int BITS, int NPROJ, bool NG8>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(NPROJ == 1 ? 3 : 2, NPROJ == 1 ? 3 : 2)))
 void qmm_kernel(const QmmLaunch launch) {
+  constexpr uint32_t kGB = QmmCodes<BITS>::kGroupBytes;  // bytes of one K group of one weight row
   extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
   const uint32_t lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
   const uint32_t m = lane & 31, h = lane >> 5;
@@ -523,7 +525,7 @@ void qmm_kernel(const QmmLaunch launch) {
     }
     row_base[p] = (slice * kQmmWaves + wv) * wave_rows + (a.pair_rows ? 32u * p : 0u);
   }
-  const size_t row_bytes = static_cast<size_t>(a.kdim) / 2;
+  const size_t row_bytes = static_cast<size_t>(ng) * kGB;
 
   // ---- everything the tile needs that depends only on the tile: issued back to back.
   // Routes past `count` read the tile's last route instead (finite data, results discarded).
@@ -542,15 +544,12 @@ void qmm_kernel(const QmmLaunch launch) {
     if (a.epi == 1) slot = pr.token * a.top_k + pr.rank;
   }
   const uint8_t* wrow[NPROJ];
-  uint4 cur[NPROJ][4];
+  QmmCodes<BITS> cur[NPROJ][4];
 #pragma unroll
   for (int p = 0; p < NPROJ; ++p) {
-    wrow[p] = Wp[p] + (row_base[p] + m) * row_bytes + h * 16;
+    wrow[p] = Wp[p] + (row_base[p] + m) * row_bytes + h * (kGB / 2);
 #pragma unroll
-    for (int u = 0; u < 4; ++u) {
-      cur[p][u] = make_uint4(0, 0, 0, 0);
-      if (NG8 || static_cast<uint32_t>(u) < ng) cur[p][u] = *reinterpret_cast<const uint4*>(wrow[p] + u * 32);
-    }
+    for (int u = 0; u < 4; ++u) cur[p][u].load(wrow[p] + min(static_cast<uint32_t>(u), ng - 1) * kGB);
   }
   // x rows of groups 0..2 and, for the bias terms, the group sums of the lane's two routes
   const uint16_t* st_src = a.x + static_cast<size_t>(st_row) * a.x_stride + st_q * 16;
@@ -613,11 +612,12 @@ void qmm_kernel(const QmmLaunch launch) {
 #pragma unroll
       for (int r = 0; r < 16; ++r) acc[p][nt][r] = 0.0f;
 
-  // ---- per step: 2 * scale (the codes enter as 8 + q/2) of the wave's rows into the [g][row] fp32 table,
-  // and the bias and offset terms: acc[token, row] += sumx[token, g] * B[row, g] + sumx[token, g] * (-16 S[row, g]).
-  // -16 * S is formed in place (exponent + 4, sign flipped: exact; a zero scale becomes 2^-123).
-  // sumx enters as three bf16 terms, which hold all 24 bits: the -16 * S * sumx term cancels the
-  // 16 * sum(x) the matrix core accumulated with the codes, so it has to be exact.
+  // ---- per step: scale / code step (4-bit codes enter as 8 + q/2: 2 * scale; 2-bit codes as 4 + q: scale)
+  // of the wave's rows into the [g][row] fp32 table, and the bias and offset terms:
+  // acc[token, row] += sumx[token, g] * B[row, g] + sumx[token, g] * (-offset S[row, g]), offset 16 or 4.
+  // -offset * S is formed in place (exponent + 4 or + 2, sign flipped: exact; a zero scale becomes 2^-123 / 2^-125).
+  // sumx enters as three bf16 terms, which hold all 24 bits: the -offset * S * sumx term cancels the
+  // offset * sum(x) the matrix core accumulated with the codes, so it has to be exact.
   for (uint32_t g0 = 0; g0 < ng; g0 += 16) {
     const TabStep t = tab_cur;
     tab_cur = tab_fetch(g0 + 16 < ng ? g0 + 16 : g0);  // past the end: the same step again, unused
@@ -630,12 +630,16 @@ void qmm_kernel(const QmmLaunch launch) {
       const uint32_t pr[4] = {t.S[p].x, t.S[p].y, t.S[p].z, t.S[p].w};
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
-        if (have && (NG8 || gl + 2 * i < ng)) tab[(gl + 2 * i) * 32 + m] = 2.0f * bf16_lo(pr[i]);
-        if (have && (NG8 || gl + 2 * i + 1 < ng)) tab[(gl + 2 * i + 1) * 32 + m] = 2.0f * bf16_hi(pr[i]);
+        if (have && (NG8 || gl + 2 * i < ng)) tab[(gl + 2 * i) * 32 + m] = QmmCodes<BITS>::kScaleMul * bf16_lo(pr[i]);
+        if (have && (NG8 || gl + 2 * i + 1 < ng)) tab[(gl + 2 * i + 1) * 32 + m] = QmmCodes<BITS>::kScaleMul * bf16_hi(pr[i]);
       }
-      ab[p] = t.B[p];
-      as[p] = make_uint4((t.S[p].x + 0x02000200u) ^ 0x80008000u, (t.S[p].y + 0x02000200u) ^ 0x80008000u,
-                         (t.S[p].z + 0x02000200u) ^ 0x80008000u, (t.S[p].w + 0x02000200u) ^ 0x80008000u);
+      constexpr uint32_t kAdd = QmmCodes<BITS>::kNegOffsetAdd;
+      // ternary rows store no biases: the bias is -scale (the table pointer is the scale table then)
+      ab[p] = a.ternary ? make_uint4(t.B[p].x ^ 0x80008000u, t.B[p].y ^ 0x80008000u, t.B[p].z ^ 0x80008000u,
+                                     t.B[p].w ^ 0x80008000u)
+                        : t.B[p];
+      as[p] = make_uint4((t.S[p].x + kAdd) ^ 0x80008000u, (t.S[p].y + kAdd) ^ 0x80008000u,
+                         (t.S[p].z + kAdd) ^ 0x80008000u, (t.S[p].w + kAdd) ^ 0x80008000u);
       if (!have) ab[p] = as[p] = make_uint4(0, 0, 0, 0);
     }
 #pragma unroll
@@ -724,23 +728,16 @@ void qmm_kernel(const QmmLaunch launch) {
           for (int s = 0; s < 4; ++s) bx[nt][s] = buf[((nt * 4 + s) * 2 + h) * 32 + rd_col[s]];
 #pragma unroll
         for (int p = 0; p < NPROJ; ++p) {
-          const uint4 cv = cur[p][2 * uu + gi];
-          const uint32_t cw[4] = {cv.x, cv.y, cv.z, cv.w};
           const float sc = s_scale[((p * kQmmWaves + wv) * ng + g) * 32 + m];
           f32x16_t tmp[2];
 #pragma unroll
           for (int nt = 0; nt < 2; ++nt)
 #pragma unroll
             for (int r = 0; r < 16; ++r) tmp[nt][r] = 0.0f;
-#pragma unroll
-          for (int s = 0; s < 4; ++s) {
-            const uint4 av = expand_q4(cw[s]);
-            tmp[0] = mfma_bf16(bx[0][s], av, tmp[0]);
-            tmp[1] = mfma_bf16(bx[1][s], av, tmp[1]);
-          }
+          group_products<BITS>(cur[p][2 * uu + gi], bx, tmp, [](int) {});
           // the register that held this group's codes takes those of the group four ahead
           // (past the end the last group is read again: no branch inside the unrolled body)
-          cur[p][2 * uu + gi] = *reinterpret_cast<const uint4*>(wrow[p] + min(g + 4, ng - 1) * 32);
+          cur[p][2 * uu + gi].load(wrow[p] + min(g + 4, ng - 1) * kGB);
 #pragma unroll
           for (int nt = 0; nt < 2; ++nt)
 #pragma unroll
@@ -852,10 +849,11 @@ template <int NG> __device__ __forceinline__ uint4 load_groups_bf16(const uint16
   }
 }
 
-template <int NG>
+template <int BITS, int NG>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2)))
 void qmm_kres_kernel(const KresLaunch launch) {
   static_assert(NG == 2 || NG == 4 || NG == 8, "K is 128, 256 or 512");
+  constexpr uint32_t kGB = QmmCodes<BITS>::kGroupBytes;  // bytes of one K group of one weight row
   constexpr int kRing = NG < 4 ? NG : 4;  // code registers in flight per projection
   extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
   const uint32_t lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
@@ -897,19 +895,19 @@ void qmm_kres_kernel(const KresLaunch launch) {
     Sp = reinterpret_cast<const uint16_t*>(blob + a.s_off[0]);
     Bp = reinterpret_cast<const uint16_t*>(blob + a.b_off[0]);
   }
-  constexpr uint32_t kRowBytes = NG * 32;
+  constexpr uint32_t kRowBytes = NG * kGB;
   // the lane's weight row of block p of slice w: row0 + 256 w + 32 p
   const uint32_t row0 = (slice0 * kQmmWaves + wv) * 64 + m;
-  const uint8_t* wrow = W + static_cast<size_t>(row0) * kRowBytes + h * 16;
+  const uint8_t* wrow = W + static_cast<size_t>(row0) * kRowBytes + h * (kGB / 2);
   const uint16_t* srow = Sp + static_cast<size_t>(row0) * NG;
   const uint16_t* brow = Bp + static_cast<size_t>(row0) * NG;
 
   // ---- everything issued back to back: codes of the first slice, its scale / bias words, the x tile
-  uint4 cur[2][kRing];
+  QmmCodes<BITS> cur[2][kRing];
 #pragma unroll
   for (int p = 0; p < 2; ++p)
 #pragma unroll
-    for (int u = 0; u < kRing; ++u) cur[p][u] = *reinterpret_cast<const uint4*>(wrow + p * 32 * kRowBytes + u * 32);
+    for (int u = 0; u < kRing; ++u) cur[p][u].load(wrow + p * 32 * kRowBytes + u * kGB);
   uint4 nS[2], nB[2];
 #pragma unroll
   for (int p = 0; p < 2; ++p) {
@@ -994,15 +992,18 @@ void qmm_kres_kernel(const KresLaunch launch) {
   for (uint32_t w = 0; w < n_walk; ++w) {
     const uint32_t step = w + 1 < n_walk ? 1u : 0u;  // the last slice requests itself again: no branch around loads
     const uint8_t* wnext = wrow + static_cast<size_t>(step) * 256 * kRowBytes;
-    // scale words of this slice; bias operand: the biases for K slots 0..7, -16 scale for K slots 8..15
-    // (-16 * S formed in place: exponent + 4, sign flipped -- exact; a zero scale becomes 2^-123)
+    // scale words of this slice; bias operand: the biases for K slots 0..7, -offset * scale for K slots
+    // 8..15 (formed in place: exponent + 4 or + 2, sign flipped -- exact; a zero scale becomes 2^-123 / 2^-125);
+    // ternary rows store no biases: theirs is -scale (the bias pointer is the scale table then)
     uint4 Sv[2], bop[2];
 #pragma unroll
     for (int p = 0; p < 2; ++p) {
+      constexpr uint32_t kAdd = QmmCodes<BITS>::kNegOffsetAdd;
       Sv[p] = nS[p];
-      const uint4 neg = make_uint4((nS[p].x + 0x02000200u) ^ 0x80008000u, (nS[p].y + 0x02000200u) ^ 0x80008000u,
-                                   (nS[p].z + 0x02000200u) ^ 0x80008000u, (nS[p].w + 0x02000200u) ^ 0x80008000u);
-      bop[p] = h ? neg : nB[p];
+      const uint4 neg = make_uint4((nS[p].x + kAdd) ^ 0x80008000u, (nS[p].y + kAdd) ^ 0x80008000u,
+                                   (nS[p].z + kAdd) ^ 0x80008000u, (nS[p].w + kAdd) ^ 0x80008000u);
+      const uint32_t flip = a.ternary ? 0x80008000u : 0u;
+      bop[p] = h ? neg : make_uint4(nB[p].x ^ flip, nB[p].y ^ flip, nB[p].z ^ flip, nB[p].w ^ flip);
     }
     f32x16_t acc[2][2];
 #pragma unroll
@@ -1035,30 +1036,23 @@ void qmm_kres_kernel(const KresLaunch launch) {
       const uint4* nbuf = s_x + ((g + 1) % NG) * 512;  // after the last group: group 0 again, for the next slice
 #pragma unroll
       for (int p = 0; p < 2; ++p) {
-        const uint4 cv = cur[p][g % kRing];
-        const uint32_t cw[4] = {cv.x, cv.y, cv.z, cv.w};
         const uint32_t sw[4] = {Sv[p].x, Sv[p].y, Sv[p].z, Sv[p].w};
-        const float sc = 2.0f * ((g & 1) ? bf16_hi(sw[g >> 1]) : bf16_lo(sw[g >> 1]));  // codes enter as 8 + q/2
+        const float sc = QmmCodes<BITS>::kScaleMul * ((g & 1) ? bf16_hi(sw[g >> 1]) : bf16_lo(sw[g >> 1]));
         f32x16_t tmp[2];
 #pragma unroll
         for (int nt = 0; nt < 2; ++nt)
 #pragma unroll
           for (int r = 0; r < 16; ++r) tmp[nt][r] = 0.0f;
-#pragma unroll
-        for (int s = 0; s < 4; ++s) {
-          const uint4 av = expand_q4(cw[s]);
-          tmp[0] = mfma_bf16(bx[0][s], av, tmp[0]);
-          tmp[1] = mfma_bf16(bx[1][s], av, tmp[1]);
-          if (p == 1) {
+        group_products<BITS>(cur[p][g % kRing], bx, tmp, [&](int s) {
+          if (p == 1) {  // both row blocks have read x slot s of this group
             bx[0][s] = nbuf[((0 * 4 + s) * 2 + h) * 32 + rd_col[s]];
             bx[1][s] = nbuf[((1 * 4 + s) * 2 + h) * 32 + rd_col[s]];
           }
-        }
+        });
         // the register takes the codes kRing groups on: of this slice, or of the next one
         const int ahead = g + kRing;
-        cur[p][g % kRing] = ahead < NG
-            ? *reinterpret_cast<const uint4*>(wrow + p * 32 * kRowBytes + ahead * 32)
-            : *reinterpret_cast<const uint4*>(wnext + p * 32 * kRowBytes + (ahead - NG) * 32);
+        cur[p][g % kRing].load(ahead < NG ? wrow + p * 32 * kRowBytes + ahead * kGB
+                                          : wnext + p * 32 * kRowBytes + (ahead - NG) * kGB);
 #pragma unroll
         for (int nt = 0; nt < 2; ++nt)
 #pragma unroll
@@ -1220,7 +1214,9 @@ bool kres_takes(const QmmArgs& q, size_t out_rows) {
   return aligned16(q.expert_base) && q.expert_stride % 16 == 0 && (q.w_off[0] | q.s_off[0] | q.b_off[0]) % 16 == 0;
 }
 
-hipError_t launch_qmm_kres(hipStream_t s, const QmmArgs& a, uint32_t tile_slots, const QmmArgs* b, uint32_t b_tile_slots) {
+// bits: 4, or 2 for 2-bit and ternary codes (both problems of one launch have the same width)
+hipError_t launch_qmm_kres(hipStream_t s, int bits, const QmmArgs& a, uint32_t tile_slots, const QmmArgs* b,
+                           uint32_t b_tile_slots) {
   KresLaunch launch{};
   for (int part = 0; part < (b ? 2 : 1); ++part) {
     QmmArgs& q = launch.part[part];
@@ -1241,22 +1237,27 @@ hipError_t launch_qmm_kres(hipStream_t s, const QmmArgs& a, uint32_t tile_slots,
   if (grid.x == 0) return hipSuccess;
   const uint32_t ng = a.kdim / kGroup;
   const size_t lds = static_cast<size_t>(ng) * 8192 + kTileTokens * 4;
-  const void* fn = ng == 8 ? reinterpret_cast<const void*>(qmm_kres_kernel<8>)
-                 : ng == 4 ? reinterpret_cast<const void*>(qmm_kres_kernel<4>)
-                           : reinterpret_cast<const void*>(qmm_kres_kernel<2>);
-  if (lds > 48 * 1024) {
-    hipError_t e = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds));
-    if (e != hipSuccess) return e;
+#define MF_KRES(B, N)                                                                                  \
+  do {                                                                                                 \
+    if (lds > 48 * 1024) {                                                                             \
+      hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(qmm_kres_kernel<B, N>),         \
+                                         hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds)); \
+      if (e != hipSuccess) return e;                                                                   \
+    }                                                                                                  \
+    qmm_kres_kernel<B, N><<<grid, block, lds, s>>>(launch);                                            \
+  } while (0)
+  if (bits == 4) {
+    if (ng == 8) MF_KRES(4, 8); else if (ng == 4) MF_KRES(4, 4); else MF_KRES(4, 2);
+  } else {
+    if (ng == 8) MF_KRES(2, 8); else if (ng == 4) MF_KRES(2, 4); else MF_KRES(2, 2);
   }
-  if (ng == 8) qmm_kres_kernel<8><<<grid, block, lds, s>>>(launch);
-  else if (ng == 4) qmm_kres_kernel<4><<<grid, block, lds, s>>>(launch);
-  else qmm_kres_kernel<2><<<grid, block, lds, s>>>(launch);
+#undef MF_KRES
   return hipGetLastError();
 }
 
 // tile_slots: entries of the tile list (routed; a multiple of 8) or number of 64-row tiles (dense).
 // `b` (optional) is a second problem for the same instantiation, run behind `a` in the same launch.
-hipError_t launch_qmm(hipStream_t s, QmmArgs a, int nproj, uint32_t tile_slots, const QmmArgs* b,
+hipError_t launch_qmm(hipStream_t s, int bits, QmmArgs a, int nproj, uint32_t tile_slots, const QmmArgs* b,
                       uint32_t b_tile_slots) {
   QmmLaunch launch{};
   size_t lds = 0;
@@ -1281,21 +1282,23 @@ hipError_t launch_qmm(hipStream_t s, QmmArgs a, int nproj, uint32_t tile_slots, 
   }
   const dim3 grid(8 * (launch.per_xcd[0] + launch.per_xcd[1])), block(256);
   if (grid.x == 0) return hipSuccess;
-  const void* fn = nproj == 2 ? (ng8 ? reinterpret_cast<const void*>(qmm_kernel<2, true>)
-                                     : reinterpret_cast<const void*>(qmm_kernel<2, false>))
-                              : (ng8 ? reinterpret_cast<const void*>(qmm_kernel<1, true>)
-                                     : reinterpret_cast<const void*>(qmm_kernel<1, false>));
-  if (lds > 48 * 1024) {
-    hipError_t e = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds));
-    if (e != hipSuccess) return e;
-  }
-  if (nproj == 2) {
-    if (ng8) qmm_kernel<2, true><<<grid, block, lds, s>>>(launch);
-    else qmm_kernel<2, false><<<grid, block, lds, s>>>(launch);
-  } else {
-    if (ng8) qmm_kernel<1, true><<<grid, block, lds, s>>>(launch);
-    else qmm_kernel<1, false><<<grid, block, lds, s>>>(launch);
-  }
+#define MF_QMM(B, P, G)                                                                                \
+  do {                                                                                                 \
+    if (lds > 48 * 1024) {                                                                             \
+      hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(qmm_kernel<B, P, G>),           \
+                                         hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds)); \
+      if (e != hipSuccess) return e;                                                                   \
+    }                                                                                                  \
+    qmm_kernel<B, P, G><<<grid, block, lds, s>>>(launch);                                              \
+  } while (0)
+#define MF_QMM_B(B)                                                        \
+  do {                                                                     \
+    if (nproj == 2) { if (ng8) MF_QMM(B, 2, true); else MF_QMM(B, 2, false); } \
+    else { if (ng8) MF_QMM(B, 1, true); else MF_QMM(B, 1, false); }        \
+  } while (0)
+  if (bits == 4) MF_QMM_B(4); else MF_QMM_B(2);
+#undef MF_QMM_B
+#undef MF_QMM
   return hipGetLastError();
 }
 
@@ -1357,7 +1360,8 @@ size_t prefill_workspace_bytes(const mf_moe_config& c, uint32_t t) {
 }
 
 bool prefill_supported(const mf_moe_config& c) {
-  if (c.bits != MF_BITS_4 || (c.shared_f && c.shared_bits != MF_BITS_4)) return false;
+  if (c.bits != MF_BITS_4 && c.bits != MF_BITS_2 && c.bits != MF_BITS_TERNARY) return false;
+  if (c.shared_f && c.shared_bits != MF_BITS_4) return false;
   if (c.d % kQmmRows || c.f % kQmmRows || (c.shared_f % kQmmRows)) return false;
   if (c.d > 8192 || c.f > 8192 || c.shared_f > 8192) return false;
   return true;
@@ -1390,6 +1394,13 @@ hipError_t launch_prefill_layer(hipStream_t s, const mf_moe& h, const mf_moe_lay
   q.n_tiles = ws.n_tiles;
   q.top_k = c.top_k;
   q.limit = c.swiglu_limit;
+  // ternary experts are 2-bit codes whose bias is -scale: the kernels take the scale table as bias table
+  const int code_bits = c.bits == MF_BITS_4 ? 4 : 2;
+  const bool ternary = c.bits == MF_BITS_TERNARY;
+  q.ternary = ternary;
+  // the (4-bit) shared expert rides in the routed launches when the routed experts are 4-bit too;
+  // otherwise its matmuls are launches of their own
+  const bool shared_rides = c.shared_f && code_bits == 4;
   if (h.trace && h.trace_bytes >= 64) {  // stage stamps of the routed gate/up matmul
     q.trace = h.trace;
     q.trace_items = static_cast<uint32_t>(std::min<size_t>(h.trace_bytes / 64, 1u << 30));
@@ -1403,16 +1414,18 @@ hipError_t launch_prefill_layer(hipStream_t s, const mf_moe& h, const mf_moe_lay
     d.x = ws.xp; d.sumx = ws.sum_x; d.x_stride = c.d; d.rows = c.shared_f; d.kdim = c.d; d.epi = 0; d.out = ws.sact;
   }
   // phase 1: routed gate/up -> acts [pair, F]; shared gate/up -> sact [token, Fs]
-  q.w_off[0] = w.offsets.gate_w; q.s_off[0] = w.offsets.gate_s; q.b_off[0] = w.offsets.gate_b;
-  q.w_off[1] = w.offsets.up_w; q.s_off[1] = w.offsets.up_s; q.b_off[1] = w.offsets.up_b;
+  q.w_off[0] = w.offsets.gate_w; q.s_off[0] = w.offsets.gate_s; q.b_off[0] = ternary ? w.offsets.gate_s : w.offsets.gate_b;
+  q.w_off[1] = w.offsets.up_w; q.s_off[1] = w.offsets.up_s; q.b_off[1] = ternary ? w.offsets.up_s : w.offsets.up_b;
   q.x = ws.xp; q.sumx = ws.sum_x; q.x_stride = c.d; q.gather = 1; q.rows = c.f; q.kdim = c.d; q.epi = 0;
   q.out = ws.acts;
-  MF_TRY(launch_qmm(s, q, 2, max_tiles, c.shared_f ? &d : nullptr, dense_tiles));
+  MF_TRY(launch_qmm(s, code_bits, q, 2, max_tiles, shared_rides ? &d : nullptr, dense_tiles));
+  if (c.shared_f && !shared_rides) MF_TRY(launch_qmm(s, 4, d, 2, dense_tiles, nullptr, 0));
   // routes past the last tile's count were never written: only pairs rows exist, all written
   MF_TRY(launch_prep_rows(s, ws.acts, nullptr, ws.sum_acts, pairs * c.f, ws.sact, nullptr, ws.sum_sact,
                           static_cast<size_t>(t) * c.shared_f));
   // phase 2: routed down -> fp32 partials [token*K+rank, D]; shared down -> hs [token, D]
-  q.w_off[0] = w.offsets.down_w; q.s_off[0] = w.offsets.down_s; q.b_off[0] = w.offsets.down_b;
+  q.w_off[0] = w.offsets.down_w; q.s_off[0] = w.offsets.down_s; q.b_off[0] = ternary ? w.offsets.down_s : w.offsets.down_b;
+  q.w_off[1] = q.s_off[1] = q.b_off[1] = 0;
   q.x = ws.acts; q.sumx = ws.sum_acts; q.x_stride = c.f; q.gather = 0; q.rows = c.d; q.kdim = c.f; q.epi = 1; q.out = ws.partials;
   q.limit = 0.0f;
   q.trace = nullptr;
@@ -1422,10 +1435,18 @@ hipError_t launch_prefill_layer(hipStream_t s, const mf_moe& h, const mf_moe_lay
     d.x = ws.sact; d.sumx = ws.sum_sact; d.x_stride = c.shared_f; d.rows = c.d; d.kdim = c.shared_f; d.epi = 2; d.out = ws.hs;
     d.pair_rows = q.pair_rows;
   }
-  if (kres_takes(q, pairs) && (!c.shared_f || (kres_takes(d, t) && d.kdim == q.kdim)))
-    MF_TRY(launch_qmm_kres(s, q, max_tiles, c.shared_f ? &d : nullptr, dense_tiles));
-  else
-    MF_TRY(launch_qmm(s, q, q.pair_rows ? 2 : 1, max_tiles, c.shared_f ? &d : nullptr, dense_tiles));
+  const bool kres_q = kres_takes(q, pairs), kres_d = c.shared_f && kres_takes(d, t);
+  if (shared_rides) {
+    if (kres_q && kres_d && d.kdim == q.kdim) MF_TRY(launch_qmm_kres(s, 4, q, max_tiles, &d, dense_tiles));
+    else MF_TRY(launch_qmm(s, 4, q, q.pair_rows ? 2 : 1, max_tiles, &d, dense_tiles));
+  } else {
+    if (kres_q) MF_TRY(launch_qmm_kres(s, code_bits, q, max_tiles, nullptr, 0));
+    else MF_TRY(launch_qmm(s, code_bits, q, q.pair_rows ? 2 : 1, max_tiles, nullptr, 0));
+    if (c.shared_f) {
+      if (kres_d) MF_TRY(launch_qmm_kres(s, 4, d, dense_tiles, nullptr, 0));
+      else MF_TRY(launch_qmm(s, 4, d, d.pair_rows ? 2 : 1, dense_tiles, nullptr, 0));
+    }
+  }
   const uint16_t* hs = nullptr;
   const uint16_t* gate = nullptr;
   if (c.shared_f) {

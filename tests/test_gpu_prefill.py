@@ -68,18 +68,27 @@ def _run_prefill(moe, wts, x, t, d, k):
     return ops.bf16_bits(y), idx.cpu().numpy().astype(np.uint32), w.cpu().numpy()
 
 
-@pytest.mark.parametrize("d,f,e,k,fs,t,mode,limit", [
-    (256, 128, 16, 4, 0, 5, 0, 0.0),        # fewer tokens than a tile, no shared expert
-    (256, 128, 16, 4, 128, 70, 0, 0.0),     # one full tile + a ragged tail per busy expert
-    (512, 256, 32, 8, 256, 200, 0, 7.0),    # SwiGLU clamp (moe.metal:1080-1094)
-    (384, 128, 32, 2, 128, 131, 1, 0.0),    # full-softmax router, ng not a multiple of 8
-    (2048, 512, 256, 8, 512, 96, 0, 0.0),   # the headline layer shape
-    (512, 256, 16, 4, 128, 90, 0, 0.0),     # shared width != routed width: the two down projections differ in K
-    (256, 384, 16, 4, 384, 67, 0, 0.0),     # K of the down projection not 128, 256 or 512
+@pytest.mark.parametrize("bits,d,f,e,k,fs,t,mode,limit", [
+    (4, 256, 128, 16, 4, 0, 5, 0, 0.0),        # fewer tokens than a tile, no shared expert
+    (4, 256, 128, 16, 4, 128, 70, 0, 0.0),     # one full tile + a ragged tail per busy expert
+    (4, 512, 256, 32, 8, 256, 200, 0, 7.0),    # SwiGLU clamp (moe.metal:1080-1094)
+    (4, 384, 128, 32, 2, 128, 131, 1, 0.0),    # full-softmax router, ng not a multiple of 8
+    (4, 2048, 512, 256, 8, 512, 96, 0, 0.0),   # the headline layer shape
+    (4, 512, 256, 16, 4, 128, 90, 0, 0.0),     # shared width != routed width: the two down projections differ in K
+    (4, 256, 384, 16, 4, 384, 67, 0, 0.0),     # K of the down projection not 128, 256 or 512
+    # 2-bit routed experts with a 4-bit shared expert (the shared matmuls are launches of their own)
+    (2, 256, 128, 16, 4, 128, 70, 0, 0.0),
+    (2, 512, 256, 32, 6, 256, 200, 0, 7.0),    # top-6 + SwiGLU clamp (moe.metal:902-1195)
+    (2, 1024, 512, 16, 6, 0, 133, 0, 0.0),     # K a multiple of 512 (whole-table vector loads), no shared expert
+    (2, 384, 384, 16, 2, 128, 45, 0, 0.0),     # neither down projection has K of 128, 256 or 512
+    # ternary experts, scale-only tables, full-softmax router (maple_moe.metal:62-265)
+    (1, 256, 128, 32, 8, 0, 131, 1, 0.0),
+    (1, 512, 256, 32, 4, 0, 64, 1, 0.0),
+    (1, 1024, 512, 64, 8, 0, 77, 1, 0.0),
 ])
-def test_prefill_layer_matches_per_token_oracle(gpu, oracle, d, f, e, k, fs, t, mode, limit):
-    root = ROOT_SEED + 0xA000 + d + t
-    layer = oracle.synth_layer(root, d, f, e, k, bits=4, fs=fs, router_mode=mode, swiglu_limit=limit)
+def test_prefill_layer_matches_per_token_oracle(gpu, oracle, bits, d, f, e, k, fs, t, mode, limit):
+    root = ROOT_SEED + 0xA000 + d + t + 0x10000 * (4 - bits)
+    layer = oracle.synth_layer(root, d, f, e, k, bits=bits, fs=fs, router_mode=mode, swiglu_limit=limit)
     x = oracle.synth_x(root, t, d)
     ref_y, ref_idx, ref_w = oracle.moe_layer(layer, x)
     moe = make_moe(gpu, layer)
@@ -88,7 +97,7 @@ def test_prefill_layer_matches_per_token_oracle(gpu, oracle, d, f, e, k, fs, t, 
     assert np.array_equal(idx, ref_idx)
     assert np.array_equal(w.view(np.uint32), ref_w.view(np.uint32))
     assert_layer_close(oracle.bf16_to_float(y), oracle.bf16_to_float(ref_y),
-                       f"prefill layer d={d} f={f} e={e} k={k} t={t}")
+                       f"prefill layer bits={bits} d={d} f={f} e={e} k={k} t={t}")
     # a second call into the same workspace-free handle gives the same bits (no stale state)
     y2, _, _ = _run_prefill(moe, wts, x, t, d, k)
     assert np.array_equal(y, y2)
@@ -117,15 +126,17 @@ def test_prefill_skewed_routing_and_decode_agreement(gpu, oracle):
                        "prefill vs decode launch")
 
 
-def test_prefill_other_formats_take_the_decode_launch(gpu, oracle):
-    """2-bit and ternary experts have no matrix-core path: the call runs the rows through the
-    decode launch eight at a time and gives exactly the decode result."""
-    for bits, mode in ((2, 0), (1, 1)):
-        d, f, e, k, fs, t = 256, 128, 32, 4, 128 if bits == 2 else 0, 19
+def test_prefill_other_widths_take_the_decode_launch(gpu, oracle):
+    """widths the matmul tiles do not divide (an intermediate size of 64) have no matrix-core
+    path: the call runs the rows through the decode launch eight at a time and gives exactly
+    the decode result, and asks for no workspace."""
+    for bits, mode in ((4, 0), (2, 0), (1, 1)):
+        d, f, e, k, fs, t = 256, 64, 32, 4, 64 if bits != 1 else 0, 19
         layer = oracle.synth_layer(ROOT_SEED + 0xA200 + bits, d, f, e, k, bits=bits, fs=fs, router_mode=mode)
         x = oracle.synth_x(ROOT_SEED + 0xA200 + bits, t, d)
         ref_y, ref_idx, ref_w = oracle.moe_layer(layer, x)
         moe = make_moe(gpu, layer)
+        assert moe.prefill_workspace_bytes(t) == 0
         wts = to_device_layer(layer)
         y, idx, w = _run_prefill(moe, wts, x, t, d, k)
         assert np.array_equal(idx, ref_idx)
@@ -138,6 +149,51 @@ def test_prefill_other_formats_take_the_decode_launch(gpu, oracle):
             moe.encode_decode_layer(wts, xd[t0:t0 + n], yd[t0:t0 + n], t=n)
         moe.status()
         assert np.array_equal(y, ops.bf16_bits(yd))
+
+
+@pytest.mark.parametrize("workload,t", [("dsv4-2bit", 300), ("maple-ternary", 300)])
+def test_prefill_other_formats_full_size(gpu, oracle, workload, t):
+    """the large 2-bit layer (D 4096, F 2048, E 256, K 6, 4-bit shared 2048) and the ternary layer
+    (D 2048, F 1024, E 64, K 8, full-softmax router) at full size through the matrix-core path:
+    routing against the CPU checker for every token, sampled rows against the CPU checker and
+    against the decode launch of the same token; a second call gives the same bits"""
+    import bench
+    w = dict(bench.WORKLOADS[workload])
+    dev = torch.device("cuda", 0)
+    lw = bench.build_stack(gpu, w, 1, dev)[0]
+    host = bench.layer_to_host(lw, w)
+    mode = ops.ROUTER_FULL_SOFTMAX if w["bits"] == 1 else ops.ROUTER_TOPK_SOFTMAX
+    host.router_mode = 1 if w["bits"] == 1 else 0
+    moe = ops.MoE(gpu, w["d"], w["f"], w["e"], w["k"], bits=w["bits"], shared_f=w["fs"],
+                  shared_bits=w["shared_bits"], router_mode=mode)
+    assert moe.prefill_workspace_bytes(t) > 0
+    gen = torch.Generator(device=dev)
+    gen.manual_seed(777)
+    d, k = w["d"], w["k"]
+    x = torch.randn((t, d), generator=gen, device=dev).to(torch.bfloat16)
+    y = torch.zeros_like(x)
+    idx = torch.zeros((t, k), dtype=torch.int32, device=dev)
+    rw = torch.zeros((t, k), dtype=torch.float32, device=dev)
+    ws = moe.encode_prefill_layer(lw, x, y, t, out_indices=idx, out_weights=rw)
+    torch.cuda.synchronize()
+    sample = [0, 1, 63, 64, 150, t - 1]
+    ref_y, ref_idx, ref_w = oracle.moe_layer(host, ops.bf16_bits(x[sample].contiguous()))
+    assert np.array_equal(idx[sample].cpu().numpy().astype(np.uint32), ref_idx)
+    assert np.array_equal(rw[sample].cpu().numpy().view(np.uint32), ref_w.view(np.uint32))
+    assert_layer_close(oracle.bf16_to_float(ops.bf16_bits(y[sample].contiguous())), oracle.bf16_to_float(ref_y),
+                       f"{workload} prefill rows vs checker")
+    for i in sample[:3]:
+        yd = torch.zeros((1, d), dtype=torch.bfloat16, device=dev)
+        idd = torch.zeros((1, k), dtype=torch.int32, device=dev)
+        moe.encode_decode_layer(lw, x[i:i + 1].contiguous(), yd, t=1, out_indices=idd)
+        moe.status()
+        assert torch.equal(idd[0], idx[i])
+        assert_layer_close(oracle.bf16_to_float(ops.bf16_bits(y[i:i + 1])),
+                           oracle.bf16_to_float(ops.bf16_bits(yd)), f"{workload} prefill row {i} vs decode")
+    y2 = torch.zeros_like(x)
+    moe.encode_prefill_layer(lw, x, y2, t, workspace=ws)
+    torch.cuda.synchronize()
+    assert torch.equal(y.view(torch.int16), y2.view(torch.int16))
 
 
 def test_prefill_rejects_a_short_workspace(gpu, oracle):

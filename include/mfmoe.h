@@ -168,6 +168,13 @@ typedef struct {
   float swiglu_limit;    /* FC_MOE_SWIGLU_LIMIT, moe.metal:27-34; <= 0: none */
   uint32_t shared_f;     /* shared expert intermediate; 0 = no shared expert */
   mf_bits shared_bits;
+  uint32_t maple_rounding; /* 1: MapleMoE's rounding points -- gate and up narrowed to bf16 and
+                            * clamped at 7 / +-7, the sigmoid built in bf16 steps
+                            * (maple_swiglu, Metal/MoE/maple_moe.metal:153-164), each expert's
+                            * down output narrowed to bf16 before its routing weight
+                            * (maple_moe_phase2, maple_moe.metal:243-264); swiglu_limit is
+                            * ignored.  0: the MoE / MoEDeepseekV4 rule (moe.metal:27-34, 528,
+                            * 1262-1270) */
 } mf_moe_config;
 
 /* MoE.init (Kernels/MoE/MoE.swift:65-151): one operator instance per shape; owns the

@@ -188,6 +188,7 @@ mf_status mf_moe_create(mf_ctx* ctx, const mf_moe_config* cfg, mf_moe** out) {
     return MF_ERR_INVALID_ARGUMENT;
   if (cfg->router_mode == MF_ROUTER_FULL_SOFTMAX && cfg->num_experts % 32 != 0)
     return MF_ERR_INVALID_ARGUMENT;
+  if (cfg->maple_rounding > 1) return MF_ERR_INVALID_ARGUMENT;
 
   auto* h = new (std::nothrow) mf_moe();
   if (!h) return MF_ERR_OUT_OF_MEMORY;

@@ -72,6 +72,28 @@ __device__ __forceinline__ float mf_exp(float x) {
 // moe.metal:79-84
 __device__ __forceinline__ float mf_silu(float x) { return x / (1.0f + mf_exp(-x)); }
 
+// MapleMoE's activation (maple_swiglu, maple_moe.metal:153-164): every intermediate is a bf16 number.
+// min / clamp of bf16 numbers against +-7 and |x| stay bf16 numbers, so only the five arithmetic
+// results are narrowed here.
+__device__ __forceinline__ float maple_swiglu(float gate_projection, float up_projection) {
+  const float gate = fminf(round_bf16(gate_projection), 7.0f);
+  const float up = fminf(fmaxf(round_bf16(up_projection), -7.0f), 7.0f);
+  const float exponent = round_bf16(mf_exp(fabsf(gate)));
+  const float reciprocal = round_bf16(1.0f / round_bf16(1.0f + exponent));
+  const float sigmoid = gate < 0.0f ? reciprocal : round_bf16(1.0f - reciprocal);
+  return round_bf16(round_bf16(gate * sigmoid) * up);
+}
+
+// the routed experts' activation, narrowed once (moe.metal:27-34, 528) or in Maple's steps
+__device__ __forceinline__ uint16_t routed_activation(float g, float u, float limit, bool maple) {
+  if (maple) return f_to_bf16(maple_swiglu(g, u));
+  if (limit > 0.0f) {
+    g = fminf(g, limit);
+    u = fminf(fmaxf(u, -limit), limit);
+  }
+  return f_to_bf16(mf_silu(g) * u);
+}
+
 // --------------------------------------------------------- wave reductions
 
 // cross-lane move inside a row of 16 lanes (DPP); CTRL: 0xB1 = swap lanes

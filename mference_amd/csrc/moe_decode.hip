@@ -28,19 +28,10 @@ __device__ __forceinline__ BlobView view_blob(const uint8_t* blob, const mf_expe
   return v;
 }
 
-// moe_swiglu_clamp (moe.metal:27-34) + moe_hidden_activation (:79-84), narrowed once (:528)
-__device__ __forceinline__ uint16_t routed_act(float g, float u, float limit) {
-  if (limit > 0.0f) {
-    g = fminf(g, limit);
-    u = fminf(fmaxf(u, -limit), limit);
-  }
-  return f_to_bf16(mf_silu(g) * u);
-}
-
 // acts[(t*K+k)*F + f] for every routed (token, slot): one lane group per row,
 // gate and up rows share the x loads (moe_phase1_gate_up_act_u16load,
 // moe.metal:499-583; 2-bit twin :966-1116; ternary maple_moe_phase1,
-// maple_moe.metal:190-221 without its bf16-stepped activation).
+// maple_moe.metal:190-221; `maple` selects its bf16-stepped activation, :153-164).
 template <int BITS, bool ALIGNED>
 __global__ __launch_bounds__(256) void phase1_kernel(const uint8_t* __restrict__ base,
                                                      size_t stride, mf_expert_offsets off,
@@ -49,7 +40,8 @@ __global__ __launch_bounds__(256) void phase1_kernel(const uint8_t* __restrict__
                                                      uint32_t x_stride,
                                                      uint16_t* __restrict__ acts, uint32_t D,
                                                      uint32_t F, uint32_t E, uint32_t pairs,
-                                                     uint32_t K, float limit, uint32_t lpr_log2) {
+                                                     uint32_t K, float limit, int maple,
+                                                     uint32_t lpr_log2) {
   constexpr int EPL = Fmt<BITS>::kElemsPer16B;
   const uint32_t lane = threadIdx.x & 63;
   const uint32_t wave = (blockIdx.x * blockDim.x + threadIdx.x) >> 6;
@@ -89,12 +81,13 @@ __global__ __launch_bounds__(256) void phase1_kernel(const uint8_t* __restrict__
   }
   const float g = group_sum(ga, static_cast<int>(lpr));
   const float u = group_sum(ua, static_cast<int>(lpr));
-  if (row_ok && sub == 0) acts[static_cast<size_t>(pair) * F + row] = routed_act(g, u, limit);
+  if (row_ok && sub == 0) acts[static_cast<size_t>(pair) * F + row] = routed_activation(g, u, limit, maple != 0);
 }
 
 // y[t,d] = bf16(residual[t,d] + sum_k w[t,k] * (down_k[d,:] . acts[t,k,:])):
 // residual first, slots in rank order, product then add, one narrowing
-// (moe_phase2_down_reduce_k8, moe.metal:1235-1271).
+// (moe_phase2_down_reduce_k8, moe.metal:1235-1271); with `maple` every expert's down output is a
+// bf16 number before it meets its routing weight (maple_moe_phase2, maple_moe.metal:243-264).
 template <int BITS, bool ALIGNED>
 __global__ __launch_bounds__(256) void phase2_kernel(const uint8_t* __restrict__ base,
                                                      size_t stride, mf_expert_offsets off,
@@ -104,7 +97,7 @@ __global__ __launch_bounds__(256) void phase2_kernel(const uint8_t* __restrict__
                                                      const uint16_t* __restrict__ residual,
                                                      uint16_t* __restrict__ y, uint32_t D,
                                                      uint32_t F, uint32_t E, uint32_t T,
-                                                     uint32_t K, uint32_t lpr_log2) {
+                                                     uint32_t K, int maple, uint32_t lpr_log2) {
   constexpr int EPL = Fmt<BITS>::kElemsPer16B;
   const uint32_t lane = threadIdx.x & 63;
   const uint32_t wave = (blockIdx.x * blockDim.x + threadIdx.x) >> 6;
@@ -138,7 +131,7 @@ __global__ __launch_bounds__(256) void phase2_kernel(const uint8_t* __restrict__
       part = __builtin_fmaf(b, sum, part);
     }
     const float v = group_sum(part, static_cast<int>(lpr));
-    const float weighted = w[pair] * v;
+    const float weighted = w[pair] * (maple ? round_bf16(v) : v);
     acc = acc + weighted;
   }
   if (row_ok && sub == 0) y[static_cast<size_t>(tok) * D + row] = f_to_bf16(acc);
@@ -167,7 +160,7 @@ hipError_t launch_phase1(hipStream_t s, const mf_moe_config& cfg, const void* ba
     const uint32_t waves = pairs * ((cfg.f + rpw - 1) / rpw);                                    \
     phase1_kernel<BITS, AL><<<dim3((waves + 3) / 4), dim3(256), 0, s>>>(                         \
         b, stride, off, idx, x, x_stride, acts, cfg.d, cfg.f, cfg.num_experts, pairs, cfg.top_k, \
-        cfg.swiglu_limit, lpr_log2);                                                             \
+        cfg.swiglu_limit, static_cast<int>(cfg.maple_rounding), lpr_log2);                       \
   }
   switch (cfg.bits) {
     case MF_BITS_4: if (al) MF_P1(kBits4, true) else MF_P1(kBits4, false) break;
@@ -192,7 +185,7 @@ hipError_t launch_phase2(hipStream_t s, const mf_moe_config& cfg, const void* ba
     const uint32_t waves = t * ((cfg.d + rpw - 1) / rpw);                                    \
     phase2_kernel<BITS, AL><<<dim3((waves + 3) / 4), dim3(256), 0, s>>>(                     \
         b, stride, off, idx, w, acts, residual, y, cfg.d, cfg.f, cfg.num_experts, t,         \
-        cfg.top_k, lpr_log2);                                                                \
+        cfg.top_k, static_cast<int>(cfg.maple_rounding), lpr_log2);                          \
   }
   switch (cfg.bits) {
     case MF_BITS_4: if (al) MF_P2(kBits4, true) else MF_P2(kBits4, false) break;

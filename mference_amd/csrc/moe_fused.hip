@@ -132,6 +132,7 @@ struct FusedArgs {
   uint32_t D, F, E, K, T, Fs;
   int router_mode;
   float limit;
+  int maple;  // MapleMoE's rounding points (mf_moe_config::maple_rounding)
 };
 
 __device__ __forceinline__ void store_u64_agent(unsigned long long* p, unsigned long long v) {
@@ -362,11 +363,8 @@ __global__ __launch_bounds__(kFusedThreads) void fused_decode_kernel(const Fused
       float g = group_sum(ga, static_cast<int>(lpr));
       float u = group_sum(ua, static_cast<int>(lpr));
       if (ok && sub == 0) {
-        if (a.limit > 0.0f) {  // moe.metal:27-34
-          g = fminf(g, a.limit);
-          u = fminf(fmaxf(u, -a.limit), a.limit);
-        }
-        store_u32_agent(dst, static_cast<uint32_t>(f_to_bf16(mf_silu(g) * u)) | (tag16 << 16));
+        // moe.metal:27-34, 528; maple_moe.metal:153-164
+        store_u32_agent(dst, static_cast<uint32_t>(routed_activation(g, u, a.limit, a.maple != 0)) | (tag16 << 16));
       }
     }
   }
@@ -527,7 +525,8 @@ __global__ __launch_bounds__(kFusedThreads) void fused_decode_kernel(const Fused
                                    have_pre && round == 0, pre);
         }
         const float v = group_sum(part, static_cast<int>(lpr));
-        if (sub == 0) s_v[wv * kWave + (lane >> lpr_log2)] = s_w[pair] * v;  // moe.metal:1262
+        // moe.metal:1262; maple_moe.metal:258 (the down output is a bf16 number first)
+        if (sub == 0) s_v[wv * kWave + (lane >> lpr_log2)] = s_w[pair] * (a.maple ? round_bf16(v) : v);
       }
       __syncthreads();
       if (threadIdx.x < rows_per_round) {
@@ -620,6 +619,7 @@ hipError_t launch_fused_decode(hipStream_t s, const mf_moe& h, const mf_moe_laye
   a.Fs = c.shared_f;
   a.router_mode = c.router_mode;
   a.limit = c.swiglu_limit;
+  a.maple = static_cast<int>(c.maple_rounding);
   const dim3 grid(static_cast<uint32_t>(h.ctx->num_cu)), block(kFusedThreads);
   const size_t lds = fused_lds_bytes(c);
 #define MF_FUSED(B, SB, SHAPE)                                                                 \

@@ -429,6 +429,7 @@ struct QmmArgs {
   int narrow;           // shared-expert rounding points (dequant_int4.metal:240-245)
   int tab_aligned;      // scale / bias rows start on 16-byte boundaries (set by the launcher)
   int ternary;          // 2-bit codes {0,1,2} with bias = -scale: b_off / dense[].biases name the SCALE table
+  int maple;            // MapleMoE's bf16-stepped activation in the SwiGLU epilogue
   void* out;
   uint32_t top_k;
   float limit;
@@ -765,6 +766,10 @@ void qmm_kernel(const QmmLaunch launch) {
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
           float gv = acc[0][nt][4 * j + i], uv = acc[NPROJ - 1][nt][4 * j + i];
+          if (a.maple) {  // maple_moe.metal:153-164
+            bits[i] = f_to_bf16(maple_swiglu(gv, uv));
+            continue;
+          }
           if (a.narrow) {
             gv = round_bf16(gv);
             uv = round_bf16(uv);
@@ -1116,7 +1121,7 @@ __global__ __launch_bounds__(256) void prefill_reduce_kernel(const float* __rest
                                                              const uint16_t* __restrict__ hs,
                                                              const uint16_t* __restrict__ gate,
                                                              uint16_t* __restrict__ y, uint32_t T,
-                                                             uint32_t K, uint32_t D, uint32_t E) {
+                                                             uint32_t K, uint32_t D, uint32_t E, int maple) {
   const size_t i4 = (static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x) * 4;
   if (i4 >= static_cast<size_t>(T) * D) return;
   const uint32_t t = static_cast<uint32_t>(i4 / D), d = static_cast<uint32_t>(i4 % D);
@@ -1133,7 +1138,10 @@ __global__ __launch_bounds__(256) void prefill_reduce_kernel(const float* __rest
   for (uint32_t r = 0; r < K; ++r) {
     if (idx[t * K + r] >= E) continue;
     const float wt = w[t * K + r];
-    const float4 v = *reinterpret_cast<const float4*>(partials + (static_cast<size_t>(t) * K + r) * D + d);
+    float4 v = *reinterpret_cast<const float4*>(partials + (static_cast<size_t>(t) * K + r) * D + d);
+    if (maple) {  // maple_moe.metal:258: the down output is a bf16 number before its weight
+      v.x = round_bf16(v.x); v.y = round_bf16(v.y); v.z = round_bf16(v.z); v.w = round_bf16(v.w);
+    }
     const float p0 = wt * v.x, p1 = wt * v.y, p2 = wt * v.z, p3 = wt * v.w;
     acc[0] = acc[0] + p0; acc[1] = acc[1] + p1; acc[2] = acc[2] + p2; acc[3] = acc[3] + p3;
   }
@@ -1398,6 +1406,7 @@ hipError_t launch_prefill_layer(hipStream_t s, const mf_moe& h, const mf_moe_lay
   const int code_bits = c.bits == MF_BITS_4 ? 4 : 2;
   const bool ternary = c.bits == MF_BITS_TERNARY;
   q.ternary = ternary;
+  q.maple = static_cast<int>(c.maple_rounding);
   // the (4-bit) shared expert rides in the routed launches when the routed experts are 4-bit too;
   // otherwise its matmuls are launches of their own
   const bool shared_rides = c.shared_f && code_bits == 4;
@@ -1458,7 +1467,7 @@ hipError_t launch_prefill_layer(hipStream_t s, const mf_moe& h, const mf_moe_lay
   }
   const size_t n4 = static_cast<size_t>(t) * c.d / 4;
   prefill_reduce_kernel<<<dim3(static_cast<uint32_t>((n4 + 255) / 256)), dim3(256), 0, s>>>(
-      ws.partials, ws.w, ws.idx, hs, gate, y, t, c.top_k, c.d, c.num_experts);
+      ws.partials, ws.w, ws.idx, hs, gate, y, t, c.top_k, c.d, c.num_experts, static_cast<int>(c.maple_rounding));
   MF_TRY(hipGetLastError());
 #undef MF_TRY
   return hipSuccess;

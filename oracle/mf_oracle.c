@@ -49,6 +49,13 @@
  *                                 moe.metal:526-528, dequant_int4.metal:240-245;
  *                                 checked against an independent fp64 numpy
  *                                 composition within the reference tolerance.
+ *   mfo_maple_swiglu, the         maple_moe.metal:153-164, 243-264; the bf16 steps
+ *   maple_rounding layer          checked on seven inputs followed by hand (clamp
+ *                                 sides, both sigmoid branches, overflow, a bf16
+ *                                 tie); the layer rebuilt from the phase-1 and
+ *                                 down functions.  exp is mfo_exp, not Metal's:
+ *                                 PARITY UNPINNED where an exp result sits on a
+ *                                 bf16 rounding boundary.
  *   mfo_group_pairs               PrefillMoEGrouping.swift:91-192; checked on
  *                                 the literal integer KATs of
  *                                 PrefillMoEGroupingTests.swift:5-203.
@@ -448,12 +455,27 @@ int mfo_gemv_multix(const uint8_t* packed, const uint16_t* scales, const uint16_
 /* moe.metal:79-84: x / (1 + exp(-x)) */
 float mfo_silu(float x) { return x / (1.0f + mfo_exp(-x)); }
 
+/* maple_swiglu (maple_moe.metal:153-164): every intermediate is a bf16 number */
+static float bf16r(float x) { return mfo_bf16_to_float(mfo_bf16_bits(x)); }
+float mfo_maple_swiglu(float gate_projection, float up_projection) {
+  const float limit = 7.0f;
+  const float gate = bf16r(fminf(bf16r(gate_projection), limit));
+  const float up = bf16r(fminf(fmaxf(bf16r(up_projection), -limit), limit));
+  const float absolute = gate < 0.0f ? bf16r(-gate) : gate;
+  const float exponent = bf16r(mfo_exp(absolute));
+  const float denominator = bf16r(1.0f + exponent);
+  const float reciprocal = bf16r(1.0f / denominator);
+  const float sigmoid = gate < 0.0f ? reciprocal : bf16r(1.0f - reciprocal);
+  const float silu = bf16r(gate * sigmoid);
+  return bf16r(silu * up);
+}
+
 static const uint16_t* u16_at(const uint8_t* base, uint32_t off) {
   return (const uint16_t*)(const void*)(base + off);
 }
 
 int mfo_expert_phase1(const uint8_t* blob, const mfo_expert_offsets* off, int bits,
-                      size_t d, size_t f, float limit, const uint16_t* x, uint16_t* acts) {
+                      size_t d, size_t f, float limit, int maple, const uint16_t* x, uint16_t* acts) {
   if ((off->gate_s | off->gate_b | off->up_s | off->up_b) & 1u) return MFO_ERR_ARG;
   float* xf = (float*)malloc(d * sizeof(float));
   float* g = (float*)malloc(f * sizeof(float));
@@ -468,6 +490,10 @@ int mfo_expert_phase1(const uint8_t* blob, const mfo_expert_offsets* off, int bi
   if (!rc) {
     for (size_t i = 0; i < f; ++i) {
       float gv = g[i], uv = u[i];
+      if (maple) { /* maple_moe.metal:203 */
+        acts[i] = mfo_bf16_bits(mfo_maple_swiglu(gv, uv));
+        continue;
+      }
       if (limit > 0.0f) { /* moe.metal:27-34 */
         gv = fminf(gv, limit);
         uv = fminf(fmaxf(uv, -limit), limit);
@@ -534,7 +560,9 @@ void mfo_sigmoid_scalar_mul(uint16_t* y, size_t n, uint16_t gate_bits) {
 
 /* Moe.swift:58-88 (y = residual + sum_slot w * FFN(x), slot order) with the
  * kernels' rounding points: phase-2 product then add, residual first, one
- * narrowing at the end (moe.metal:1262-1270). */
+ * narrowing at the end (moe.metal:1262-1270).  With maple_rounding: MapleMoE's
+ * activation and bf16 down outputs (maple_moe.metal:153-164, 243-264; the sum
+ * there starts from the first product, which 0 + w*v reproduces exactly). */
 int mfo_moe_layer(const mfo_layer* L, const uint16_t* x, uint16_t* y, uint32_t* idx_out,
                   float* w_out, float* logits_out) {
   const size_t d = L->d, f = L->f, e = L->e, k = L->k;
@@ -564,11 +592,12 @@ int mfo_moe_layer(const mfo_layer* L, const uint16_t* x, uint16_t* y, uint32_t* 
   for (size_t s = 0; s < k && !rc; ++s) {
     if (idx[s] >= e) continue; /* sentinel route: contributes nothing */
     const uint8_t* blob = L->experts + (size_t)idx[s] * L->expert_stride;
-    rc = mfo_expert_phase1(blob, &L->off, L->bits, d, f, L->swiglu_limit, x, acts);
+    rc = mfo_expert_phase1(blob, &L->off, L->bits, d, f, L->swiglu_limit, L->maple_rounding, x, acts);
     if (!rc) rc = mfo_expert_down(blob, &L->off, L->bits, d, f, acts, v);
     if (!rc)
       for (size_t i = 0; i < d; ++i) {
-        float partial = w[s] * v[i];
+        /* maple_moe.metal:258: the down output is a bf16 number before it meets its weight */
+        float partial = w[s] * (L->maple_rounding ? bf16r(v[i]) : v[i]);
         acc[i] += partial;
       }
   }

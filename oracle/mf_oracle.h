@@ -98,8 +98,11 @@ float mfo_silu(float x);
 /* routed phase 1: acts[f] = bf16(silu(clamp(gate.x)) * clamp(up.x)), fp32 gate/up
  * (moe.metal:499-529, clamp :27-34).  limit <= 0 disables the clamp. */
 int mfo_expert_phase1(const uint8_t* blob, const mfo_expert_offsets* off, int bits,
-                      size_t d, size_t f, float swiglu_limit, const uint16_t* x,
+                      size_t d, size_t f, float swiglu_limit, int maple, const uint16_t* x,
                       uint16_t* acts);
+/* MapleMoE's activation, every intermediate narrowed to bf16 (maple_moe.metal:153-164);
+ * selected in mfo_expert_phase1 by maple != 0 (swiglu_limit is ignored then) */
+float mfo_maple_swiglu(float gate_projection, float up_projection);
 /* v[d] = down . acts (fp32) (moe.metal:349-404) */
 int mfo_expert_down(const uint8_t* blob, const mfo_expert_offsets* off, int bits,
                     size_t d, size_t f, const uint16_t* acts, float* v);
@@ -128,6 +131,7 @@ typedef struct {
   const uint8_t* suw; const uint16_t* sus; const uint16_t* sub; /* shared up   */
   const uint8_t* sdw; const uint16_t* sds; const uint16_t* sdb; /* shared down */
   const uint16_t* w_sg;      /* [d] bf16 scalar shared gate, may be NULL    */
+  int maple_rounding;        /* MapleMoE's activation and bf16 down outputs */
 } mfo_layer;
 
 /* one token through router -> routed experts -> shared expert -> combine.

@@ -52,7 +52,7 @@ class _Layer(C.Structure):
         ("sgw", C.c_void_p), ("sgs", C.c_void_p), ("sgb", C.c_void_p),
         ("suw", C.c_void_p), ("sus", C.c_void_p), ("sub", C.c_void_p),
         ("sdw", C.c_void_p), ("sds", C.c_void_p), ("sdb", C.c_void_p),
-        ("w_sg", C.c_void_p),
+        ("w_sg", C.c_void_p), ("maple_rounding", C.c_int),
     ]
 
 
@@ -263,12 +263,12 @@ def gemv_multix(q: QTensor, x_bits) -> np.ndarray:
 
 
 def expert_phase1(blob, off: ExpertOffsets, bits: int, d: int, f: int, x_bits,
-                  swiglu_limit: float = 0.0) -> np.ndarray:
+                  swiglu_limit: float = 0.0, maple: bool = False) -> np.ndarray:
     blob = _c(blob, np.uint8)
     x_bits = _c(x_bits, np.uint16)
     acts = np.empty(f, np.uint16)
     rc = lib().mfo_expert_phase1(_p(blob), C.byref(off), bits, C.c_size_t(d), C.c_size_t(f),
-                                 C.c_float(swiglu_limit), _p(x_bits), _p(acts))
+                                 C.c_float(swiglu_limit), C.c_int(1 if maple else 0), _p(x_bits), _p(acts))
     if rc:
         raise ValueError("mfo_expert_phase1")
     return acts
@@ -298,6 +298,14 @@ def shared_expert(gate: QTensor, up: QTensor, down: QTensor, x_bits) -> np.ndarr
     return y
 
 
+def maple_swiglu(gate: float, up: float) -> float:
+    """MapleMoE's activation, every intermediate a bf16 number (maple_moe.metal:153-164)"""
+    fn = lib().mfo_maple_swiglu
+    fn.restype = C.c_float
+    fn.argtypes = [C.c_float, C.c_float]
+    return float(fn(gate, up))
+
+
 def sigmoid_scalar_mul(y_bits, gate_bits: int) -> np.ndarray:
     y = _c(y_bits, np.uint16).copy()
     lib().mfo_sigmoid_scalar_mul(_p(y), C.c_size_t(y.size), C.c_uint16(gate_bits))
@@ -321,12 +329,14 @@ class Layer:
     w_sg: Optional[np.ndarray] = None  # uint16 [d]
     router_mode: int = 0
     swiglu_limit: float = 0.0
+    maple_rounding: bool = False    # MapleMoE's activation and bf16 down outputs
 
     def _struct(self) -> _Layer:
         L = _Layer()
         L.d, L.f, L.e, L.k, L.fs = self.d, self.f, self.e, self.k, self.fs
         L.bits, L.shared_bits = self.bits, self.shared_bits
         L.router_mode, L.swiglu_limit = self.router_mode, self.swiglu_limit
+        L.maple_rounding = 1 if self.maple_rounding else 0
         L.router_w = self.router_w.ctypes.data
         L.experts = self.experts.ctypes.data
         L.expert_stride = self.experts.strides[0]
@@ -451,7 +461,7 @@ def pack_expert_blob(gate: QTensor, up: QTensor, down: QTensor, off: ExpertOffse
 
 def synth_layer(root: int, d: int, f: int, e: int, k: int, bits: int = BITS_4, fs: int = 0,
                 shared_bits: int = BITS_4, sigma: float = 0.02, router_mode: int = 0,
-                swiglu_limit: float = 0.0, with_w_sg: bool = True) -> Layer:
+                swiglu_limit: float = 0.0, with_w_sg: bool = True, maple_rounding: bool = False) -> Layer:
     """Seeded synthetic layer: one SeedTree stream per tensor (labels "router",
     "shared.gate|up|down", "w_sg", "expert<i>.gate|up|down"), N(0, sigma)
     weights by Box-Muller, quantized per group of 64."""
@@ -488,7 +498,7 @@ def synth_layer(root: int, d: int, f: int, e: int, k: int, bits: int = BITS_4, f
             w_sg = bf16_bits(nrm("w_sg", 1, d).reshape(d))
     return Layer(d=d, f=f, e=e, k=k, bits=bits, router_w=router_w, experts=experts, off=off,
                  fs=fs, shared_bits=shared_bits, shared=shared, w_sg=w_sg,
-                 router_mode=router_mode, swiglu_limit=swiglu_limit)
+                 router_mode=router_mode, swiglu_limit=swiglu_limit, maple_rounding=maple_rounding)
 
 
 def synth_x(root: int, t: int, d: int, label: str = "x") -> np.ndarray:

@@ -34,7 +34,8 @@ def to_device_layer(layer, device="cuda") -> ops.MoELayerWeights:
 def make_moe(ctx, layer) -> ops.MoE:
     return ops.MoE(ctx, layer.d, layer.f, layer.e, layer.k, bits=layer.bits,
                    router_mode=layer.router_mode, swiglu_limit=layer.swiglu_limit,
-                   shared_f=layer.fs, shared_bits=layer.shared_bits)
+                   shared_f=layer.fs, shared_bits=layer.shared_bits,
+                   maple_rounding=getattr(layer, "maple_rounding", False))
 
 
 def errors(actual: np.ndarray, ref: np.ndarray):

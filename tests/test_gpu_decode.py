@@ -437,3 +437,35 @@ def test_dense_mlp_full_size(gpu, oracle):
         mlp.encode(x[i:i + 1].contiguous(), qs[0], qs[1], qs[2], yi, si, t=1)
         _sync()
         assert torch.equal(yi[0].view(torch.int16), y[i].view(torch.int16))
+
+
+@pytest.mark.parametrize("bits,d,f,e,k,t", [(1, 256, 128, 32, 8, 1), (1, 512, 256, 64, 8, 3), (4, 256, 128, 32, 4, 2)])
+def test_decode_layer_with_maple_rounding(gpu, oracle, bits, d, f, e, k, t):
+    """MapleMoE's rounding points (bf16-stepped activation clamped at 7, bf16 down outputs before
+    the routing weights; maple_moe.metal:153-164, 243-264) against the CPU checker, fused launch
+    and launch chain bit for bit, and different from the same layer without the flag"""
+    root = ROOT_SEED + 0x9A00 + bits + d
+    layer = oracle.synth_layer(root, d, f, e, k, bits=bits, router_mode=1, sigma=0.1, maple_rounding=True)
+    x = oracle.synth_x(root, t, d)
+    ref_y, ref_idx, _ = oracle.moe_layer(layer, x)
+    moe = make_moe(gpu, layer)
+    wts = to_device_layer(layer)
+    xd = ops.bf16_tensor(x)
+    results = {}
+    for fused in (True, False):
+        moe.set_fused(fused)
+        y = torch.zeros((t, d), dtype=torch.bfloat16, device="cuda")
+        idx = torch.zeros((t, k), dtype=torch.int32, device="cuda")
+        moe.encode_decode_layer(wts, xd, y, t=t, out_indices=idx)
+        moe.status()
+        assert np.array_equal(idx.cpu().numpy().astype(np.uint32), ref_idx)
+        assert_layer_close(oracle.bf16_to_float(ops.bf16_bits(y)), oracle.bf16_to_float(ref_y),
+                           f"maple rounding fused={fused} bits={bits}")
+        results[fused] = ops.bf16_bits(y)
+    assert np.array_equal(results[True], results[False])
+    layer.maple_rounding = False
+    plain = make_moe(gpu, layer)
+    y0 = torch.zeros((t, d), dtype=torch.bfloat16, device="cuda")
+    plain.encode_decode_layer(wts, xd, y0, t=t)
+    plain.status()
+    assert not np.array_equal(ops.bf16_bits(y0), results[True])

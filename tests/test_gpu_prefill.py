@@ -103,6 +103,26 @@ def test_prefill_layer_matches_per_token_oracle(gpu, oracle, bits, d, f, e, k, f
     assert np.array_equal(y, y2)
 
 
+@pytest.mark.parametrize("bits,d,f,e,k,t", [(1, 512, 256, 32, 8, 150), (4, 256, 128, 32, 4, 70)])
+def test_prefill_layer_with_maple_rounding(gpu, oracle, bits, d, f, e, k, t):
+    """MapleMoE's rounding points in the prefill call: the SwiGLU epilogue takes maple_swiglu,
+    the reduce narrows every down output to bf16 before its weight"""
+    root = ROOT_SEED + 0xAA00 + bits + d
+    # sigma keeps |y| below 2, where one bf16 step is still inside the max-abs bar
+    layer = oracle.synth_layer(root, d, f, e, k, bits=bits, router_mode=1, sigma=0.03, maple_rounding=True)
+    x = oracle.synth_x(root, t, d)
+    ref_y, ref_idx, ref_w = oracle.moe_layer(layer, x)
+    moe = make_moe(gpu, layer)
+    wts = to_device_layer(layer)
+    y, idx, w = _run_prefill(moe, wts, x, t, d, k)
+    assert np.array_equal(idx, ref_idx)
+    assert np.array_equal(w.view(np.uint32), ref_w.view(np.uint32))
+    assert_layer_close(oracle.bf16_to_float(y), oracle.bf16_to_float(ref_y), f"maple prefill bits={bits}")
+    layer.maple_rounding = False
+    y0, _, _ = _run_prefill(make_moe(gpu, layer), wts, x, t, d, k)
+    assert not np.array_equal(y0, y)
+
+
 def test_prefill_skewed_routing_and_decode_agreement(gpu, oracle):
     """All tokens identical -> every token takes the same k experts: k groups of
     t routes and e-k empty experts; and the prefill rows agree with the decode

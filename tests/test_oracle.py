@@ -368,6 +368,52 @@ def test_layer_against_independent_fp64_composition(bits, d, f, e, k, fs):
     assert np.linalg.norm(yf - ref) / np.linalg.norm(ref) < 1e-3
 
 
+def test_maple_swiglu_known_answers():
+    """maple_swiglu (maple_moe.metal:153-164) on values whose bf16 steps can be followed by hand
+    (the test-side restatement in MapleMoETests.swift:411-418 is the same sequence):
+    gate 0 -> exp 1, 1 + 1 = 2, 1/2, sigmoid 1 - 1/2, silu 0;
+    gate 1, up 2 -> exp bf16(2.71828) = 2.71875, denominator 3.71875 (exact), reciprocal
+      bf16(0.268908) = 0.26953125, sigmoid 1 - that = 0.73046875 (exact), silu the same, x 2;
+    gate -1 takes the reciprocal itself as sigmoid;
+    gate and up beyond the limit: gate clamps at 7 from above only, up at +-7; exp(7) = 1096.6 ->
+      1096, + 1 -> 1096, reciprocal 9.1e-4, 1 - that rounds to 1, silu 7, 7 x 7 = 49;
+    a very negative gate: exp overflows to inf, reciprocal 0, silu -0;
+    gate 1 + 2^-8 is a bf16 tie and narrows to 1 (even), up 7.5 clamps to 7: bf16(0.73046875 x 7) = 5.125."""
+    assert O.maple_swiglu(0.0, 3.0) == 0.0
+    assert O.maple_swiglu(1.0, 2.0) == 1.4609375
+    assert O.maple_swiglu(-1.0, 2.0) == -0.5390625
+    assert O.maple_swiglu(100.0, 100.0) == 49.0
+    assert O.maple_swiglu(100.0, -100.0) == -49.0
+    assert O.maple_swiglu(-100.0, 5.0) == 0.0
+    assert O.maple_swiglu(1.00390625, 7.5) == 5.125
+
+
+def test_maple_layer_is_the_composition_of_its_pinned_parts():
+    """with maple_rounding the layer is: activations through maple_swiglu, every expert's down
+    output narrowed to bf16 before its routing weight, products added in rank order from the
+    first (maple_moe_phase2, maple_moe.metal:243-264) -- rebuilt here from the phase-1 and down
+    functions, and different from the layer without the flag"""
+    d, f, e, k = 256, 128, 32, 8
+    layer = O.synth_layer(0x3A91E, d, f, e, k, bits=O.BITS_TERNARY, router_mode=1, sigma=0.1, maple_rounding=True)
+    x = O.synth_x(0x3A91E, 1, d)[0]
+    y, idx, w = O.moe_layer(layer, x)
+    bf = lambda v: O.bf16_to_float(O.bf16_bits(np.asarray(v, np.float32)))
+    acc = np.zeros(d, np.float32)
+    for s, ex in enumerate(idx):
+        acts = O.expert_phase1(layer.experts[ex], layer.off, layer.bits, d, f, x, maple=True)
+        g_u = O.expert_phase1(layer.experts[ex], layer.off, layer.bits, d, f, x, maple=False)
+        assert not np.array_equal(acts, g_u)
+        v = O.expert_down(layer.experts[ex], layer.off, layer.bits, d, f, acts)
+        acc = (acc + np.float32(w[s]) * bf(v)).astype(np.float32)
+    assert np.array_equal(y, O.bf16_bits(acc))
+    layer.maple_rounding = False
+    y0, idx0, _ = O.moe_layer(layer, x)
+    assert np.array_equal(idx0, idx) and not np.array_equal(y0, y)
+    # the two rules stay close: Maple's steps cost a few bf16 roundings
+    a, b = O.bf16_to_float(y).astype(np.float64), O.bf16_to_float(y0).astype(np.float64)
+    assert np.linalg.norm(a - b) / np.linalg.norm(b) < 2e-2
+
+
 def test_shared_expert_rounding_points():
     # SharedExpertInt4Tests.swift:11-53 shape (D 128, F 64, seed 0x604)
     d, f = 128, 64

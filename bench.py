@@ -37,7 +37,7 @@ WORKLOADS = {
     "dsv4-2bit": dict(name="large-2bit-moe-layer-decode-D4096-F2048-E256-K6", config=3, d=4096, f=2048,
                       e=256, k=6, fs=2048, bits=2, shared_bits=4, t=1, layers=4),
     "maple-ternary": dict(name="ternary-moe-layer-decode-D2048-F1024-E64-K8", config=4, d=2048, f=1024,
-                          e=64, k=8, fs=0, bits=1, shared_bits=4, t=1, layers=40),
+                          e=64, k=8, fs=0, bits=1, shared_bits=4, t=1, layers=40, maple=True),
 }
 DENSE_MLP = dict(name="dense-4bit-swiglu-mlp-D5120-F17408", d=5120, f=17408, bits=4, layers=8)
 
@@ -135,7 +135,8 @@ def layer_to_host(wts, w):
     return O.Layer(d=w["d"], f=w["f"], e=w["e"], k=w["k"], bits=w["bits"],
                    router_w=ops.bf16_bits(wts.router_w), experts=wts.experts.cpu().numpy(), off=off,
                    fs=w["fs"], shared_bits=w["shared_bits"], shared=shared,
-                   w_sg=None if wts.w_sg is None else ops.bf16_bits(wts.w_sg))
+                   w_sg=None if wts.w_sg is None else ops.bf16_bits(wts.w_sg),
+                   router_mode=1 if w["bits"] == 1 else 0, maple_rounding=bool(w.get("maple")))
 
 
 def profiled_traffic_bytes():
@@ -178,7 +179,7 @@ def measure_prefill(ctx, w, layer, device, tokens=(128, 512, 2048), steps=100, w
     lw = ops.MoELayerWeights(router, layer.experts, layer.offsets, layer.shared, layer.w_sg)
     full_softmax = w["bits"] == 1
     moe = ops.MoE(ctx, w["d"], w["f"], w["e"], w["k"], bits=w["bits"], shared_f=w["fs"],
-                  shared_bits=w["shared_bits"],
+                  shared_bits=w["shared_bits"], maple_rounding=bool(w.get("maple")),
                   router_mode=ops.ROUTER_FULL_SOFTMAX if full_softmax else ops.ROUTER_TOPK_SOFTMAX)
     qwen = w["config"] == QWEN["config"]
     import re
@@ -198,7 +199,6 @@ def measure_prefill(ctx, w, layer, device, tokens=(128, 512, 2048), steps=100, w
         run = {"tokens": t}
         if t == min(tokens):
             host = layer_to_host(lw, w)
-            host.router_mode = 1 if full_softmax else 0
             n_par = t if qwen else min(t, 16)   # the large layers: the first 16 rows (the checker is a CPU loop)
             ref_y, ref_idx, _ = O.moe_layer(host, ops.bf16_bits(x[:n_par].contiguous()))
             got = O.bf16_to_float(ops.bf16_bits(y[:n_par].contiguous())).astype(np.float64)
@@ -366,7 +366,7 @@ def main() -> int:
         print(json.dumps(res))
         return 0
     moes = [ops.MoE(ctx, w["d"], w["f"], w["e"], w["k"], bits=w["bits"], shared_f=w["fs"],
-                    shared_bits=w["shared_bits"],
+                    shared_bits=w["shared_bits"], maple_rounding=bool(w.get("maple")),
                     router_mode=ops.ROUTER_FULL_SOFTMAX if w["bits"] == 1 else ops.ROUTER_TOPK_SOFTMAX)
             for _ in range(L)]
 

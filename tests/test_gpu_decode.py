@@ -380,7 +380,7 @@ def test_other_shape_specialised_launches(gpu, oracle, workload, t):
     mode = ops.ROUTER_FULL_SOFTMAX if w["bits"] == 1 else ops.ROUTER_TOPK_SOFTMAX
     host.router_mode = 1 if w["bits"] == 1 else 0
     moe = ops.MoE(gpu, w["d"], w["f"], w["e"], w["k"], bits=w["bits"], shared_f=w["fs"],
-                  shared_bits=w["shared_bits"], router_mode=mode)
+                  shared_bits=w["shared_bits"], router_mode=mode, maple_rounding=bool(w.get("maple")))
     gen = torch.Generator(device="cuda")
     gen.manual_seed(4321)
     x = torch.randn((t, w["d"]), generator=gen, device="cuda").to(torch.bfloat16)

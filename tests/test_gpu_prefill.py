@@ -185,7 +185,7 @@ def test_prefill_other_formats_full_size(gpu, oracle, workload, t):
     mode = ops.ROUTER_FULL_SOFTMAX if w["bits"] == 1 else ops.ROUTER_TOPK_SOFTMAX
     host.router_mode = 1 if w["bits"] == 1 else 0
     moe = ops.MoE(gpu, w["d"], w["f"], w["e"], w["k"], bits=w["bits"], shared_f=w["fs"],
-                  shared_bits=w["shared_bits"], router_mode=mode)
+                  shared_bits=w["shared_bits"], router_mode=mode, maple_rounding=bool(w.get("maple")))
     assert moe.prefill_workspace_bytes(t) > 0
     gen = torch.Generator(device=dev)
     gen.manual_seed(777)

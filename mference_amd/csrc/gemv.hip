@@ -783,7 +783,10 @@ bool rows_stream_try(hipStream_t s, const RowsArgs& in, uint32_t t, uint32_t num
   constexpr int EPL = Fmt<BITS>::kElemsPer16B;
   if (in.N % kGroup || in.N < 64 * EPL || (t != 1 && t != 2 && t != 4) || in.M < 1024) return false;
   const uint32_t steps = (in.N + 64 * EPL - 1) / (64 * EPL);  // 16-byte steps of one wave along a row
-  const uint32_t max_its = t == 1 ? 9 : 3;
+  // x slices live in registers for the whole launch: T x its x (pairs + sum).  A 2-bit slice is 33
+  // registers, and with two projections in flight the 9-step and the 4-token 3-step instances spill.
+  constexpr bool wide_slices = BITS == kBits2 && NPROJ == 2;
+  const uint32_t max_its = t == 1 ? (wide_slices ? 3 : 9) : (wide_slices && t == 4 ? 1 : 3);
   if (BITS == kBitsTernary) return false;
   uint32_t wpr = 1;
   while (wpr < 4 && (steps + wpr - 1) / wpr > max_its) wpr *= 2;
@@ -798,9 +801,16 @@ bool rows_stream_try(hipStream_t s, const RowsArgs& in, uint32_t t, uint32_t num
 #define MF_ROWS(TT, II)                                                                      \
   rows_stream_kernel<BITS, TT, II, NPROJ><<<dim3(grid), dim3(256), 0, s>>>(a)
   if constexpr (BITS != kBitsTernary) {
-    if (t == 1) { if (its == 1) MF_ROWS(1, 1); else if (its <= 3) MF_ROWS(1, 3); else MF_ROWS(1, 9); }
-    else if (t == 2) { if (its == 1) MF_ROWS(2, 1); else MF_ROWS(2, 3); }
-    else { if (its == 1) MF_ROWS(4, 1); else MF_ROWS(4, 3); }
+    if (t == 1) {
+      if (its == 1) MF_ROWS(1, 1);
+      else if (its <= 3) MF_ROWS(1, 3);
+      else if constexpr (!wide_slices) MF_ROWS(1, 9);
+    } else if (t == 2) {
+      if (its == 1) MF_ROWS(2, 1); else MF_ROWS(2, 3);
+    } else {
+      if (its == 1) MF_ROWS(4, 1);
+      else if constexpr (!wide_slices) MF_ROWS(4, 3);
+    }
   }
 #undef MF_ROWS
   err = hipGetLastError();

@@ -555,16 +555,18 @@ void qmm_kernel(const QmmLaunch launch) {
   // x rows of groups 0..2 and, for the bias terms, the group sums of the lane's two routes
   const uint16_t* st_src = a.x + static_cast<size_t>(st_row) * a.x_stride + st_q * 16;
   // K groups travel in pairs (ng is even: kdim is a multiple of 128)
-  uint4 xs[2][2];  // the pair after the one in LDS, on its way there
-  uint4 x0[2][2];
+  // (arrays of a native vector type: arrays of the uint4 struct were kept in scratch memory)
+  typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
+  u32x4_t xs[2][2];  // the pair after the one in LDS, on its way there
+  u32x4_t x0[2][2];
 #pragma unroll
   for (int gi = 0; gi < 2; ++gi) {
-    x0[gi][0] = *reinterpret_cast<const uint4*>(st_src + gi * kGroup);
-    x0[gi][1] = *reinterpret_cast<const uint4*>(st_src + gi * kGroup + 8);
-    xs[gi][0] = xs[gi][1] = make_uint4(0, 0, 0, 0);
+    x0[gi][0] = *reinterpret_cast<const u32x4_t*>(st_src + gi * kGroup);
+    x0[gi][1] = *reinterpret_cast<const u32x4_t*>(st_src + gi * kGroup + 8);
+    xs[gi][0] = xs[gi][1] = u32x4_t{0, 0, 0, 0};
     if (NG8 || ng > 2) {
-      xs[gi][0] = *reinterpret_cast<const uint4*>(st_src + (2 + gi) * kGroup);
-      xs[gi][1] = *reinterpret_cast<const uint4*>(st_src + (2 + gi) * kGroup + 8);
+      xs[gi][0] = *reinterpret_cast<const u32x4_t*>(st_src + (2 + gi) * kGroup);
+      xs[gi][1] = *reinterpret_cast<const u32x4_t*>(st_src + (2 + gi) * kGroup + 8);
     }
   }
   // Scale and bias words of the lane's row and the group sums of its two routes, 8 K groups at a time
@@ -687,8 +689,8 @@ void qmm_kernel(const QmmLaunch launch) {
   for (int sidx = 0; sidx < 4; ++sidx) rd_col[sidx] = (m + 4 * (sidx >> 1) + 8 * h) & 31;
 #pragma unroll
   for (int gi = 0; gi < 2; ++gi) {
-    s_x[gi * 512 + st_slot0] = x0[gi][0];
-    s_x[gi * 512 + st_slot1] = x0[gi][1];
+    *reinterpret_cast<u32x4_t*>(s_x + gi * 512 + st_slot0) = x0[gi][0];
+    *reinterpret_cast<u32x4_t*>(s_x + gi * 512 + st_slot1) = x0[gi][1];
   }
 
   // Weight codes run four K groups ahead in a ring of registers (the expert's bytes come
@@ -706,14 +708,14 @@ void qmm_kernel(const QmmLaunch launch) {
         uint4* wbuf = s_x + (uu ^ 1) * 1024;
 #pragma unroll
         for (int gi = 0; gi < 2; ++gi) {
-          wbuf[gi * 512 + st_slot0] = xs[gi][0];
-          wbuf[gi * 512 + st_slot1] = xs[gi][1];
+          *reinterpret_cast<u32x4_t*>(wbuf + gi * 512 + st_slot0) = xs[gi][0];
+          *reinterpret_cast<u32x4_t*>(wbuf + gi * 512 + st_slot1) = xs[gi][1];
         }
         if (gu + 4 < ng) {
 #pragma unroll
           for (int gi = 0; gi < 2; ++gi) {
-            xs[gi][0] = *reinterpret_cast<const uint4*>(st_src + (gu + 4 + gi) * kGroup);
-            xs[gi][1] = *reinterpret_cast<const uint4*>(st_src + (gu + 4 + gi) * kGroup + 8);
+            xs[gi][0] = *reinterpret_cast<const u32x4_t*>(st_src + (gu + 4 + gi) * kGroup);
+            xs[gi][1] = *reinterpret_cast<const u32x4_t*>(st_src + (gu + 4 + gi) * kGroup + 8);
           }
         }
       }

@@ -264,12 +264,12 @@ __global__ __launch_bounds__(512) void group_scan_kernel(uint32_t* __restrict__ 
   uint32_t c = 0;
   if (e < E) {
     uint32_t k = 0;
-    for (; k + 8 <= n_chunks; k += 8) {  // eight independent loads in flight
-      uint32_t v[8];
+    for (; k + 32 <= n_chunks; k += 32) {  // 32 independent loads in flight: the loop is all latency
+      uint32_t v[32];
 #pragma unroll
-      for (int u = 0; u < 8; ++u) v[u] = chunk_hist[(k + u) * E + e];
+      for (int u = 0; u < 32; ++u) v[u] = chunk_hist[(k + u) * E + e];
 #pragma unroll
-      for (int u = 0; u < 8; ++u) {
+      for (int u = 0; u < 32; ++u) {
         chunk_hist[(k + u) * E + e] = c;
         c += v[u];
       }

@@ -162,7 +162,7 @@ def pmc_calibration(device) -> str:
     return "3 x 256 MiB device-to-device copy (reads 268435456 B, writes 268435456 B)"
 
 
-def measure_prefill(ctx, w, layer, device, tokens=(128, 512, 2048), steps=100, warmup=100):
+def measure_prefill(ctx, w, layer, device, tokens=(128, 512, 2048), steps=100, warmup=100, use_graph=True):
     """Ragged prefill of one layer of the same shape: T tokens, top-k routing from skewed
     logits (router weights plus a per-expert bias ~ N(0, 1.5), carried by a constant-one last
     feature of x and the last column of the router, so expert loads are uneven and some
@@ -183,7 +183,8 @@ def measure_prefill(ctx, w, layer, device, tokens=(128, 512, 2048), steps=100, w
                   router_mode=ops.ROUTER_FULL_SOFTMAX if full_softmax else ops.ROUTER_TOPK_SOFTMAX)
     qwen = w["config"] == QWEN["config"]
     import re
-    out = {"workload": ("qwen3.6-35b-a3b-moe-layer-ragged-prefill-4bit-g64" if qwen
+    out = {"launch": "hip_graph" if use_graph else "eager",
+           "workload": ("qwen3.6-35b-a3b-moe-layer-ragged-prefill-4bit-g64" if qwen
                         else re.sub(r"-T\d+$", "", w["name"]).replace("decode", "ragged-prefill")) + ", skewed routing",
            "dtype": "u%d codes (exact, as bf16) x bf16 activations on bf16 MFMA, fp32 accumulate"
                     % (4 if w["bits"] == 4 else 2),
@@ -208,16 +209,35 @@ def measure_prefill(ctx, w, layer, device, tokens=(128, 512, 2048), steps=100, w
                 routing_bit_exact=bool(np.array_equal(idx[:n_par].cpu().numpy().astype(np.uint32), ref_idx)),
                 max_abs=float(np.abs(got - ref).max()),
                 rel_l2=float(np.linalg.norm(got - ref) / np.linalg.norm(ref)))
-        for _ in range(warmup):
-            moe.encode_prefill_layer(lw, x, y, t, workspace=ws)
+        # the layer call is eleven launches: replayed from a HIP graph (ten calls per graph) so that
+        # short batches measure the kernels and not the host's launch rate
+        per_graph = 10 if use_graph else 1
+        def calls():
+            for _ in range(per_graph):
+                moe.encode_prefill_layer(lw, x, y, t, workspace=ws)
+        go = calls
+        if use_graph:
+            side = torch.cuda.Stream()
+            side.wait_stream(torch.cuda.current_stream())
+            with torch.cuda.stream(side):
+                calls()
+            torch.cuda.current_stream().wait_stream(side)
+            torch.cuda.synchronize()
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(graph):
+                calls()
+            go = graph.replay
+        reps = max(1, steps // per_graph)
+        for _ in range(max(1, warmup // per_graph)):
+            go()
         torch.cuda.synchronize()
         e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
         e0.record()
-        for _ in range(steps):
-            moe.encode_prefill_layer(lw, x, y, t, workspace=ws)
+        for _ in range(reps):
+            go()
         e1.record()
         torch.cuda.synchronize()
-        us = e0.elapsed_time(e1) / steps * 1e3
+        us = e0.elapsed_time(e1) / (reps * per_graph) * 1e3
         flops = 2.0 * 3 * w["d"] * (t * w["k"] * w["f"] + t * w["fs"])
         tflops = flops / us / 1e6
         run.update(us_per_layer=round(us, 1), tokens_per_s=round(t / us * 1e6, 1),
@@ -359,8 +379,8 @@ def main() -> int:
     stack = build_stack(ctx, w, L, device)
     if args.prefill_only:
         tokens = (args.tokens,) if args.tokens else (128, 512, 2048)
-        res = {"prefill": measure_prefill(ctx, w, stack[0], device, tokens=tokens,
-                                          steps=min(args.steps, 100), warmup=min(args.warmup, 100))}
+        res = {"prefill": measure_prefill(ctx, w, stack[0], device, tokens=tokens, steps=min(args.steps, 100),
+                                          warmup=min(args.warmup, 100), use_graph=not args.no_graph)}
         if args.pmc_calibration:
             res["pmc_calibration"] = pmc_calibration(device)
         print(json.dumps(res))
@@ -469,7 +489,7 @@ def main() -> int:
     }
 
     if not args.no_prefill:
-        out["prefill"] = measure_prefill(ctx, w, stack[0], device)
+        out["prefill"] = measure_prefill(ctx, w, stack[0], device, use_graph=not args.no_graph)
     if not args.no_cpu_baseline:
         # the CPU checker (a restatement of the reference's CPU path: bulk
         # dequantize each row, scalar fp32 dot, experts in slot order) timed on

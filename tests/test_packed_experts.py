@@ -178,3 +178,71 @@ def test_loaded_layer_runs_like_the_directly_built_one(tmp_path, gpu, oracle):
         ys.append(ops.bf16_bits(y))
     assert np.array_equal(ys[0], ys[1])
     assert_layer_close(oracle.bf16_to_float(ys[1]), oracle.bf16_to_float(ref_y), "layer from packed_experts")
+
+
+# ------------------------------------------------------- resident streamer (HBM pool behind the streamer calls)
+
+def test_stream_layout_offsets():
+    """StreamLayout.expertOffset (ExpertStreamer.swift:58-65): the explicit table for layer 0, else
+    layer * experts * stride + expert * stride"""
+    from mference_amd.resident_streamer import StreamLayout
+    plain = StreamLayout("x", 0, 4 * 4096, 4, 4096)
+    assert plain.expert_offset(0, 3) == 3 * 4096 and plain.expert_offset(2, 1) == 2 * 4 * 4096 + 4096
+    table = StreamLayout("x", 0, 4 * 4096, 4, 4096, expert_offsets=[8192, 0, 12288, 4096])
+    assert [table.expert_offset(0, e) for e in range(4)] == [8192, 0, 12288, 4096]
+    assert table.expert_offset(1, 2) == 4 * 4096 + 2 * 4096   # the table covers layer 0 only
+    assert table.expert_offset(0, 7) == 7 * 4096              # and only its own length
+
+
+def test_resident_streamer_views_and_errors(tmp_path, oracle):
+    from mference_amd import resident_streamer as rs
+    layer = oracle.synth_layer(ROOT_SEED + 0xB400, 256, 128, 8, 4, bits=4)
+    order = [5, 2, 7, 0, 1, 6, 3, 4]
+    stride = write_packed_experts(str(tmp_path), layer, physical_order=order)
+    layout = pe.PackedExpertsLayoutReader.load(str(tmp_path))
+    sl = rs.stream_layout_for_packed_layer(str(tmp_path), layout, 0)
+    assert sl.stream_offset == 0 and sl.stream_size == 8 * stride and sl.expert_stride == stride
+    st = rs.ResidentExpertStreamer(sl, device="cpu")
+    st.warm_up()
+    blob = layer.experts.shape[1]
+    for e in range(8):
+        buf, off, size = st.expert_buffer(0, e)
+        assert off == 0 and size == stride
+        assert np.array_equal(buf.numpy()[:blob], layer.experts[e])
+    with pytest.raises(rs.StreamerError) as err:
+        st.expert_buffer(0, 8)
+    assert err.value.kind == "slotOutOfRange"
+    with pytest.raises(rs.StreamerError) as err:
+        rs.ResidentExpertStreamer(rs.StreamLayout(str(tmp_path / "nothing.bin"), 0, stride, 1, stride), device="cpu")
+    assert err.value.kind == "openFailed"
+    with pytest.raises(rs.StreamerError) as err:   # the file is shorter than offset + size
+        rs.ResidentExpertStreamer(rs.StreamLayout(sl.path, stride, 8 * stride, 8, stride), device="cpu")
+    assert err.value.kind == "sizeMismatch"
+    with pytest.raises(rs.StreamerError) as err:   # an expert lies past the streamed range
+        rs.ResidentExpertStreamer(rs.StreamLayout(sl.path, 0, 4 * stride, 8, stride), device="cpu")
+    assert err.value.kind == "offsetOutOfRange"
+
+
+@pytest.mark.gpu
+def test_resident_streamer_pool_runs_a_layer(tmp_path, gpu, oracle):
+    import torch
+    from mference_amd import operators as ops
+    from mference_amd import resident_streamer as rs
+    from helpers import assert_layer_close, make_moe, to_device_layer
+    d, f, e, k = 512, 256, 16, 4
+    layer = oracle.synth_layer(ROOT_SEED + 0xB500, d, f, e, k, bits=2)
+    write_packed_experts(str(tmp_path), layer, physical_order=[(3 * i) % e for i in range(e)])
+    layout = pe.PackedExpertsLayoutReader.load(str(tmp_path))
+    st = rs.ResidentExpertStreamer(rs.stream_layout_for_packed_layer(str(tmp_path), layout, 0), device="cuda")
+    direct = to_device_layer(layer)
+    wts = ops.MoELayerWeights(router_w=direct.router_w, experts=st.pool,
+                              offsets=pe.routed_expert_offsets(layout, 0))
+    x_bits = oracle.synth_x(ROOT_SEED + 0xB500, 2, d)
+    ref_y, ref_idx, _ = oracle.moe_layer(layer, x_bits)
+    y = torch.zeros((2, d), dtype=torch.bfloat16, device="cuda")
+    idx = torch.zeros((2, k), dtype=torch.int32, device="cuda")
+    moe = make_moe(gpu, layer)
+    moe.encode_decode_layer(wts, ops.bf16_tensor(x_bits), y, t=2, out_indices=idx)
+    moe.status()
+    assert np.array_equal(idx.cpu().numpy().astype(np.uint32), ref_idx)
+    assert_layer_close(oracle.bf16_to_float(ops.bf16_bits(y)), oracle.bf16_to_float(ref_y), "layer from the streamer's pool")

@@ -302,3 +302,31 @@ def test_prefill_16k_tokens_repeat_the_2048_token_rows(gpu):
     assert bool(torch.isfinite(yb.float()).all())
     assert torch.equal(idxb.view(reps, t, k), idx.expand(reps, t, k))
     assert torch.equal(yb.view(torch.int16).view(reps, t, d), y.view(torch.int16).expand(reps, t, d))
+
+
+def test_non_finite_token_takes_sentinel_routes(gpu, oracle):
+    """full-softmax router: a token whose logits are not finite gets indices = num_experts and
+    weights 0 (maple_moe.metal:73-79); its routes contribute nothing, in the decode launch and in
+    the prefill call, and the other tokens of the batch are untouched"""
+    d, f, e, k, t = 512, 256, 32, 8, 100
+    root = ROOT_SEED + 0xAB00
+    layer = oracle.synth_layer(root, d, f, e, k, bits=1, router_mode=1)
+    x = oracle.synth_x(root, t, d)
+    bad = [3, 64, 99]
+    x[bad, 7] = 0x7FC0   # bf16 NaN
+    ref_y, ref_idx, ref_w = oracle.moe_layer(layer, x)
+    assert (ref_idx[bad] == e).all() and (ref_w[bad] == 0).all() and (ref_y[bad] == 0).all()
+    moe = make_moe(gpu, layer)
+    wts = to_device_layer(layer)
+    y, idx, w = _run_prefill(moe, wts, x, t, d, k)
+    assert np.array_equal(idx, ref_idx)
+    assert np.array_equal(w.view(np.uint32), ref_w.view(np.uint32))
+    assert (y[bad] == 0).all()
+    good = [i for i in range(t) if i not in bad]
+    assert_layer_close(oracle.bf16_to_float(y[good]), oracle.bf16_to_float(ref_y[good]), "tokens next to a NaN token")
+    yd = torch.zeros((3, d), dtype=torch.bfloat16, device="cuda")
+    idd = torch.zeros((3, k), dtype=torch.int32, device="cuda")
+    moe.encode_decode_layer(wts, ops.bf16_tensor(x[[2, 3, 4]]), yd, t=3, out_indices=idd)
+    moe.status()
+    assert np.array_equal(idd.cpu().numpy().astype(np.uint32), ref_idx[[2, 3, 4]])
+    assert (ops.bf16_bits(yd)[1] == 0).all()

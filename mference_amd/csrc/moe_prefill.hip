@@ -150,12 +150,21 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
 #pragma unroll
     for (int u = 0; u < 4; ++u) {
       if (q0 + u >= steps) break;
+      // The 16 operands of the step's 8 matrix instructions, each in a register of its own, before the
+      // first of them issues: a vector instruction that writes a register an MFMA in flight still reads
+      // as A or B waits until that MFMA is done (64 cycles here), so operands made one at a time in a
+      // recycled register pair cost 89 instead of 65 cycles per instruction.
       const uint32_t xw[4] = {cx[u].x, cx[u].y, cx[u].z, cx[u].w}, ww[4] = {cw[u].x, cw[u].y, cw[u].z, cw[u].w};
+      float xa[8], wa[8];
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
-        acc = __builtin_amdgcn_mfma_f32_32x32x1f32(bf16_lo(xw[j]), bf16_lo(ww[j]), acc, 0, 0, 0);
-        acc = __builtin_amdgcn_mfma_f32_32x32x1f32(bf16_hi(xw[j]), bf16_hi(ww[j]), acc, 0, 0, 0);
+        xa[2 * j] = bf16_lo(xw[j]); xa[2 * j + 1] = bf16_hi(xw[j]);
+        wa[2 * j] = bf16_lo(ww[j]); wa[2 * j + 1] = bf16_hi(ww[j]);
       }
+      asm volatile("" : "+v"(xa[0]), "+v"(xa[1]), "+v"(xa[2]), "+v"(xa[3]), "+v"(xa[4]), "+v"(xa[5]), "+v"(xa[6]), "+v"(xa[7]),
+                        "+v"(wa[0]), "+v"(wa[1]), "+v"(wa[2]), "+v"(wa[3]), "+v"(wa[4]), "+v"(wa[5]), "+v"(wa[6]), "+v"(wa[7]));
+#pragma unroll
+      for (int j = 0; j < 8; ++j) acc = __builtin_amdgcn_mfma_f32_32x32x1f32(xa[j], wa[j], acc, 0, 0, 0);
       if (++i == n_i) {  // the pair of chains is complete: stride-1 level, then the binary counter
         float carry[16];
 #pragma unroll

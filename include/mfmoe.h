@@ -144,6 +144,16 @@ mf_status mf_sigmoid_scalar_mul(mf_ctx* ctx, mf_stream stream, uint16_t* y,
 mf_status mf_residual_add(mf_ctx* ctx, mf_stream stream, uint16_t* hidden,
                           const uint16_t* delta, uint32_t count);
 
+/* The step in front of the MoE layer in RealForwardRunner.produceToken
+ * (Runtime/Inference/RealForwardRunner.swift:2799-2808): Elementwise.encodeResidualAdd
+ * (hidden += delta; utility.metal:83-92) followed by RMSNorm.encodeBF16W
+ * (Kernels/Primitives/RMSNorm.swift:52-64; rmsnorm_bf16w, Metal/Primitives/rmsnorm.metal:68-92),
+ * as one launch over t rows of d: hidden[t,d] = bf16(hidden + delta) when delta is not NULL, then
+ * out[t,d] = bf16(hidden * rsqrt(mean(hidden^2) + eps) * weight[d]), the sum of squares in fp32.
+ * out may not alias hidden. */
+mf_status mf_residual_rmsnorm(mf_ctx* ctx, mf_stream stream, uint16_t* hidden, const uint16_t* delta,
+                              const uint16_t* weight, uint16_t* out, uint32_t d, uint32_t t, float eps);
+
 /* SharedExpertInt4.encode (Kernels/MoE/SharedExpertInt4.swift:70-165) /
  * SharedExpertRuntime.encode (:193-202): y[t,d] = bf16(down . act),
  * act = bf16(silu(bf16(gate.x)) * bf16(up.x)).  scratch_act holds t*f bf16.

@@ -120,6 +120,20 @@ class Elementwise {
   mf_ctx* ctx_;
 };
 
+// RMSNorm.encodeBF16W (Kernels/Primitives/RMSNorm.swift:52-64); `delta`, when given, is the residual
+// add the runner issues in front of it (RealForwardRunner.swift:2799-2808), in the same launch
+class RMSNorm {
+ public:
+  explicit RMSNorm(const MetalContext& context) : ctx_(context.raw()) {}
+  void encodeBF16W(mf_stream cb, uint16_t* x, const uint16_t* weight, uint16_t* out, uint32_t d, float eps,
+                   uint32_t t = 1, const uint16_t* delta = nullptr) const {
+    check(mf_residual_rmsnorm(ctx_, cb, x, delta, weight, out, d, t, eps), ctx_);
+  }
+
+ private:
+  mf_ctx* ctx_;
+};
+
 // SharedExpertInt4 (Kernels/MoE/SharedExpertInt4.swift:70-165), also the dense SwiGLU MLP.
 // Errors: MF_ERR_DIMENSION_MISMATCH / MF_ERR_SCRATCH_TOO_SMALL / MF_ERR_UNSUPPORTED_BITS are
 // SharedExpertError.dimensionMismatch / .scratchTooSmall / .unsupportedWeightBits (:4-19).

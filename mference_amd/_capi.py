@@ -76,6 +76,7 @@ SIGNATURES = {
     "mf_silu_mul": (_I, [_P, _P, _P, _P, _P, _U32]),
     "mf_sigmoid_scalar_mul": (_I, [_P, _P, _P, _P, _U32, _U32]),
     "mf_residual_add": (_I, [_P, _P, _P, _P, _U32]),
+    "mf_residual_rmsnorm": (_I, [_P, _P, _P, _P, _P, _P, _U32, _U32, C.c_float]),
     "mf_shared_expert": (_I, [_P, _P, _P, QTensor, QTensor, QTensor, _I, _U32, _U32, _U32, _P, _P,
                               _SZ]),
     "mf_moe_create": (_I, [_P, C.POINTER(MoEConfig), C.POINTER(_P)]),

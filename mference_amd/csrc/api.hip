@@ -151,6 +151,16 @@ mf_status mf_residual_add(mf_ctx* ctx, mf_stream stream, uint16_t* hidden, const
   return MF_OK;
 }
 
+mf_status mf_residual_rmsnorm(mf_ctx* ctx, mf_stream stream, uint16_t* hidden, const uint16_t* delta,
+                              const uint16_t* weight, uint16_t* out, uint32_t d, uint32_t t, float eps) {
+  if (!ctx || !hidden || !weight || !out) return MF_ERR_INVALID_ARGUMENT;
+  if (d == 0) return MF_ERR_DIMENSION_MISMATCH;
+  if (!mf::aligned2(hidden) || !mf::aligned2(weight) || !mf::aligned2(out) || (delta && !mf::aligned2(delta)))
+    return MF_ERR_INVALID_ARGUMENT;
+  MF_HIP(ctx, mf::launch_residual_rmsnorm(static_cast<hipStream_t>(stream), hidden, delta, weight, out, d, t, eps));
+  return MF_OK;
+}
+
 mf_status mf_shared_expert(mf_ctx* ctx, mf_stream stream, const uint16_t* x, mf_qtensor gate,
                            mf_qtensor up, mf_qtensor down, mf_bits bits, uint32_t d, uint32_t f,
                            uint32_t t, uint16_t* y, uint16_t* scratch_act,

@@ -969,6 +969,45 @@ hipError_t launch_sigmoid_scalar_mul(hipStream_t s, uint16_t* y, const uint16_t*
   return hipGetLastError();
 }
 
+// The step in front of the MoE layer (RealForwardRunner.swift:2799-2808): hidden += delta
+// (residual_add_fp16, utility.metal:83-92; skipped when delta is null), then
+// out = narrow(hidden * rsqrt(mean(hidden^2) + eps) * weight) (rmsnorm_bf16w, rmsnorm.metal:68-92:
+// fp32 sum of squares by fma, the sum is taken over the narrowed hidden).  One workgroup per row.
+__global__ __launch_bounds__(256) void residual_rmsnorm_kernel(uint16_t* __restrict__ hidden,
+                                                               const uint16_t* __restrict__ delta,
+                                                               const uint16_t* __restrict__ weight,
+                                                               uint16_t* __restrict__ out, uint32_t d,
+                                                               float eps) {
+  __shared__ float s_part[4];
+  uint16_t* h = hidden + static_cast<size_t>(blockIdx.x) * d;
+  const uint16_t* dl = delta ? delta + static_cast<size_t>(blockIdx.x) * d : nullptr;
+  uint16_t* o = out + static_cast<size_t>(blockIdx.x) * d;
+  float acc = 0.0f;
+  for (uint32_t i = threadIdx.x; i < d; i += blockDim.x) {
+    uint16_t hb = h[i];
+    if (dl) {
+      hb = f_to_bf16(bf16_to_f(hb) + bf16_to_f(dl[i]));
+      h[i] = hb;
+    }
+    const float v = bf16_to_f(hb);
+    acc = __builtin_fmaf(v, v, acc);
+  }
+  acc = wave_sum(acc);
+  if ((threadIdx.x & 63) == 0) s_part[threadIdx.x >> 6] = acc;
+  __syncthreads();
+  const float total = (s_part[0] + s_part[1]) + (s_part[2] + s_part[3]);
+  const float inv = 1.0f / __builtin_sqrtf(total / static_cast<float>(d) + eps);
+  for (uint32_t i = threadIdx.x; i < d; i += blockDim.x)
+    o[i] = f_to_bf16(bf16_to_f(h[i]) * inv * bf16_to_f(weight[i]));
+}
+
+hipError_t launch_residual_rmsnorm(hipStream_t s, uint16_t* hidden, const uint16_t* delta,
+                                   const uint16_t* weight, uint16_t* out, uint32_t d, uint32_t t, float eps) {
+  if (!t) return hipSuccess;
+  residual_rmsnorm_kernel<<<dim3(t), dim3(256), 0, s>>>(hidden, delta, weight, out, d, eps);
+  return hipGetLastError();
+}
+
 hipError_t launch_residual_add(hipStream_t s, uint16_t* hidden, const uint16_t* delta,
                                uint32_t count) {
   if (!count) return hipSuccess;

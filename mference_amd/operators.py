@@ -174,6 +174,20 @@ class Elementwise:
                                           _ptr(delta), count), self.context.handle)
 
 
+class RMSNorm:
+    """Kernels/Primitives/RMSNorm.swift:52-64 (`encodeBF16W`), with the residual add that
+    precedes it in the runner folded into the same launch when `delta` is given."""
+
+    def __init__(self, context: MetalContext):
+        self.context = context
+
+    def encode_bf16w(self, x, weight, out, d: int, eps: float, t: int = 1, delta=None, stream=None):
+        """x [t, d] bf16 is the hidden state: updated in place by `delta` when given"""
+        check(_capi.lib().mf_residual_rmsnorm(self.context.handle, _stream(stream), _ptr(x), _ptr(delta),
+                                              _ptr(weight), _ptr(out), d, t, C.c_float(eps)),
+              self.context.handle)
+
+
 class SharedExpertInt4:
     """Kernels/MoE/SharedExpertInt4.swift:70-165 (also the dense SwiGLU MLP)."""
 

@@ -56,6 +56,9 @@
  *                                 down functions.  exp is mfo_exp, not Metal's:
  *                                 PARITY UNPINNED where an exp result sits on a
  *                                 bf16 rounding boundary.
+ *   mfo_residual_rmsnorm          utility.metal:83-92 + rmsnorm.metal:30-92; closed
+ *                                 form, checked on hand-computed rows (3-4-0
+ *                                 vector, unit vector, eps only) and fp64 numpy.
  *   mfo_group_pairs               PrefillMoEGrouping.swift:91-192; checked on
  *                                 the literal integer KATs of
  *                                 PrefillMoEGroupingTests.swift:5-203.
@@ -556,6 +559,26 @@ void mfo_sigmoid_scalar_mul(uint16_t* y, size_t n, uint16_t gate_bits) {
   float g = mfo_bf16_to_float(gate_bits);
   float den = 1.0f + mfo_exp(-g);
   for (size_t i = 0; i < n; ++i) y[i] = mfo_bf16_bits(mfo_bf16_to_float(y[i]) / den);
+}
+
+/* residual_add_fp16 (utility.metal:83-92) + rmsnorm_bf16w (rmsnorm.metal:30-92): hidden is
+ * narrowed after the add; the sum of squares of the narrowed values is taken here in double
+ * (the kernels sum in fp32 in an order of their own: a test compares within one bf16 step);
+ * out = narrow(h * inv * w), two fp32 products, left to right. */
+void mfo_residual_rmsnorm(uint16_t* hidden, const uint16_t* delta, const uint16_t* weight,
+                          uint16_t* out, size_t d, float eps) {
+  double sum = 0.0;
+  for (size_t i = 0; i < d; ++i) {
+    if (delta) hidden[i] = mfo_bf16_bits(mfo_bf16_to_float(hidden[i]) + mfo_bf16_to_float(delta[i]));
+    const double v = mfo_bf16_to_float(hidden[i]);
+    sum += v * v;
+  }
+  const float inv = (float)(1.0 / sqrt(sum / (double)d + (double)eps));
+  for (size_t i = 0; i < d; ++i) {
+    float v = mfo_bf16_to_float(hidden[i]) * inv;
+    v = v * mfo_bf16_to_float(weight[i]);
+    out[i] = mfo_bf16_bits(v);
+  }
 }
 
 /* Moe.swift:58-88 (y = residual + sum_slot w * FFN(x), slot order) with the

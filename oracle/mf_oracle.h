@@ -115,6 +115,11 @@ int mfo_shared_expert(const uint8_t* gw, const uint16_t* gs, const uint16_t* gb,
 /* y[i] = bf16(y[i] / (1 + exp(-gate))) (utility.metal:49-59) */
 void mfo_sigmoid_scalar_mul(uint16_t* y, size_t n, uint16_t gate_bits);
 
+/* hidden += delta (delta may be NULL), then out = narrow(hidden * rsqrt(mean(hidden^2) + eps) * weight)
+ * (utility.metal:83-92, rmsnorm.metal:30-92) */
+void mfo_residual_rmsnorm(uint16_t* hidden, const uint16_t* delta, const uint16_t* weight,
+                          uint16_t* out, size_t d, float eps);
+
 typedef struct {
   size_t d, f, e, k;         /* hidden, routed intermediate, experts, top-k */
   size_t fs;                 /* shared intermediate (0 = no shared expert)  */

@@ -306,6 +306,19 @@ def maple_swiglu(gate: float, up: float) -> float:
     return float(fn(gate, up))
 
 
+def residual_rmsnorm(hidden_bits, weight_bits, eps: float, delta_bits=None):
+    """rows of hidden [t, d] (or [d]): (hidden after the add, normalised rows), both uint16"""
+    h = _c(hidden_bits, np.uint16).copy()
+    w = _c(weight_bits, np.uint16)
+    h2 = h.reshape(-1, w.size)
+    dl = None if delta_bits is None else _c(delta_bits, np.uint16).reshape(h2.shape)
+    out = np.empty_like(h2)
+    for i in range(h2.shape[0]):
+        lib().mfo_residual_rmsnorm(_p(h2[i]), None if dl is None else _p(dl[i]), _p(w), _p(out[i]),
+                                   C.c_size_t(w.size), C.c_float(eps))
+    return h2.reshape(h.shape), out.reshape(h.shape)
+
+
 def sigmoid_scalar_mul(y_bits, gate_bits: int) -> np.ndarray:
     y = _c(y_bits, np.uint16).copy()
     lib().mfo_sigmoid_scalar_mul(_p(y), C.c_size_t(y.size), C.c_uint16(gate_bits))

@@ -469,3 +469,26 @@ def test_decode_layer_with_maple_rounding(gpu, oracle, bits, d, f, e, k, t):
     plain.encode_decode_layer(wts, xd, y0, t=t)
     plain.status()
     assert not np.array_equal(ops.bf16_bits(y0), results[True])
+
+
+@pytest.mark.parametrize("d,t,with_delta", [(2048, 1, True), (2048, 5, False), (4096, 3, True), (320, 2, True)])
+def test_residual_rmsnorm_matches_oracle(gpu, oracle, d, t, with_delta):
+    """hidden += delta, then RMSNorm with a bf16 weight, one launch (rmsnorm.metal:30-92,
+    utility.metal:83-92): the updated hidden bit for bit; the normalised rows within one bf16 step
+    of the checker (it sums the squares in double, the kernel in fp32 in lane order) and equal on
+    all but a few elements"""
+    r = oracle.Rng.key(ROOT_SEED + 0x9B00 + d, "rms")
+    hb = oracle.bf16_bits(r.normal(0.0, 1.5, t * d).reshape(t, d))
+    db = oracle.bf16_bits(r.normal(0.0, 0.5, t * d).reshape(t, d)) if with_delta else None
+    wb = oracle.bf16_bits(r.normal(1.0, 0.1, d))
+    ref_h, ref_out = oracle.residual_rmsnorm(hb, wb, 1e-6, delta_bits=db)
+    hidden = ops.bf16_tensor(hb)
+    out = torch.zeros_like(hidden)
+    ops.RMSNorm(gpu).encode_bf16w(hidden, ops.bf16_tensor(wb), out, d, 1e-6, t=t,
+                                  delta=None if db is None else ops.bf16_tensor(db))
+    torch.cuda.synchronize()
+    assert np.array_equal(ops.bf16_bits(hidden), ref_h)
+    got, ref = oracle.bf16_to_float(ops.bf16_bits(out)), oracle.bf16_to_float(ref_out)
+    step = np.maximum(np.abs(ref), 2.0 ** -126) * 2.0 ** -7
+    assert (np.abs(got - ref) <= step).all()
+    assert (ops.bf16_bits(out) != ref_out).mean() < 0.01

@@ -414,6 +414,38 @@ def test_maple_layer_is_the_composition_of_its_pinned_parts():
     assert np.linalg.norm(a - b) / np.linalg.norm(b) < 2e-2
 
 
+def test_residual_rmsnorm_hand_computed_rows():
+    """rmsnorm_bf16w (rmsnorm.metal:30-92) after residual_add_fp16 (utility.metal:83-92):
+    (3, 4, 0, ...) over 64 elements has mean square 25/64, so inv = 1.6 and the row becomes
+    bf16(4.8) = 4.8125, bf16(6.4) = 6.40625; a weight of 0.5 halves them exactly; a unit vector over
+    d = 64 becomes 8 e_i; the add is narrowed before the squares are summed: 1 + 2^-9 narrows to 1"""
+    d = 64
+    one = O.bf16_bits(np.ones(d, np.float32))
+    x = np.zeros(d, np.float32); x[0], x[1] = 3.0, 4.0
+    h, out = O.residual_rmsnorm(O.bf16_bits(x), one, 0.0)
+    got = O.bf16_to_float(out)
+    assert got[0] == 4.8125 and got[1] == 6.40625 and not got[2:].any()
+    assert np.array_equal(h, O.bf16_bits(x))
+    _, out = O.residual_rmsnorm(O.bf16_bits(x), O.bf16_bits(np.full(d, 0.5, np.float32)), 0.0)
+    assert O.bf16_to_float(out)[0] == 2.40625 and O.bf16_to_float(out)[1] == 3.203125
+    e5 = np.zeros(d, np.float32); e5[5] = -2.0
+    _, out = O.residual_rmsnorm(O.bf16_bits(e5), one, 0.0)
+    assert O.bf16_to_float(out)[5] == -8.0
+    # zeros: only eps under the root; the row stays zero
+    _, out = O.residual_rmsnorm(O.bf16_bits(np.zeros(d, np.float32)), one, 1e-6)
+    assert not O.bf16_to_float(out).any()
+    # hidden + delta is narrowed first: 1 + 2^-9 -> 1, every element 1, the norm returns 1
+    h, out = O.residual_rmsnorm(one, one, 0.0, delta_bits=O.bf16_bits(np.full(d, 2.0 ** -9, np.float32)))
+    assert np.array_equal(h, one) and np.array_equal(out, one)
+    # against fp64 on a random row, to one bf16 step
+    r = O.Rng.key(0x5151, "rms")
+    xr = O.bf16_bits(r.normal(0.0, 1.5, 2048)); wr = O.bf16_bits(r.normal(1.0, 0.1, 2048))
+    _, out = O.residual_rmsnorm(xr, wr, 1e-6)
+    xf, wf = O.bf16_to_float(xr).astype(np.float64), O.bf16_to_float(wr).astype(np.float64)
+    ref = xf / np.sqrt((xf * xf).mean() + 1e-6) * wf
+    assert np.abs(O.bf16_to_float(out) - ref).max() <= np.abs(ref).max() * 2.0 ** -8
+
+
 def test_shared_expert_rounding_points():
     # SharedExpertInt4Tests.swift:11-53 shape (D 128, F 64, seed 0x604)
     d, f = 128, 64

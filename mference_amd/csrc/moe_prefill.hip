@@ -897,6 +897,7 @@ void qmm_kres_kernel(const KresLaunch launch) {
   }
   uint4* s_x = reinterpret_cast<uint4*>(smem);                       // [NG groups][512]
   uint32_t* s_slot = reinterpret_cast<uint32_t*>(smem + NG * 8192);  // [64]
+  float* s_sum = reinterpret_cast<float*>(smem + NG * 8192 + kTileTokens * 4);  // [64 routes][NG]
 
   const uint8_t* W;
   const uint16_t* Sp;
@@ -936,26 +937,6 @@ void qmm_kres_kernel(const KresLaunch launch) {
   u32x4_t xv[2 * NG];
 #pragma unroll
   for (int g = 0; g < 2 * NG; ++g) xv[g] = *reinterpret_cast<const u32x4_t*>(st_src + (g >> 1) * kGroup + (g & 1) * 8);
-  // group sums of the lane's two routes (both halves of the wave hold them: K slots 8h..8h+7 of the
-  // bias product are the groups 0..7 again, multiplied by the biases for h = 0 and by -16 scale for h = 1)
-  float sx[2][8];
-#pragma unroll
-  for (int nt = 0; nt < 2; ++nt) {
-    const float* sp = a.sumx + static_cast<size_t>(pair_start + min(nt * 32 + m, count - 1)) * NG;
-#pragma unroll
-    for (int e = 0; e < 8; ++e) sx[nt][e] = 0.0f;
-    if constexpr (NG >= 8) {
-      const float4 s0 = *reinterpret_cast<const float4*>(sp), s1 = *reinterpret_cast<const float4*>(sp + 4);
-      sx[nt][0] = s0.x; sx[nt][1] = s0.y; sx[nt][2] = s0.z; sx[nt][3] = s0.w;
-      sx[nt][4] = s1.x; sx[nt][5] = s1.y; sx[nt][6] = s1.z; sx[nt][7] = s1.w;
-    } else if constexpr (NG == 4) {
-      const float4 s0 = *reinterpret_cast<const float4*>(sp);
-      sx[nt][0] = s0.x; sx[nt][1] = s0.y; sx[nt][2] = s0.z; sx[nt][3] = s0.w;
-    } else {
-      const float2 s0 = *reinterpret_cast<const float2*>(sp);
-      sx[nt][0] = s0.x; sx[nt][1] = s0.y;
-    }
-  }
   uint32_t slot = 0;
   if (threadIdx.x < kTileTokens) {
     const uint32_t pi = pair_start + min(threadIdx.x, count - 1);
@@ -979,15 +960,39 @@ void qmm_kres_kernel(const KresLaunch launch) {
       *reinterpret_cast<u32x4_t*>(s_x + g * 512 + st_slot1) = xv[2 * g + 1];
     }
     if (threadIdx.x < kTileTokens) s_slot[threadIdx.x] = slot;
+    // the fp32 sum of every 64-wide group of every route, for the bias and offset terms: the four
+    // threads that stage a route each hold 16 of a group's values
+#pragma unroll
+    for (int g = 0; g < NG; ++g) {
+      float part = 0.0f;
+#pragma unroll
+      for (int u = 0; u < 2; ++u) {
+        const u32x4_t v = xv[2 * g + u];
+        part += ((bf16_lo(v.x) + bf16_hi(v.x)) + (bf16_lo(v.y) + bf16_hi(v.y))) +
+                ((bf16_lo(v.z) + bf16_hi(v.z)) + (bf16_lo(v.w) + bf16_hi(v.w)));
+      }
+      part = group_sum(part, 4);
+      if (st_q == 0) s_sum[st_i * NG + g] = part;
+    }
   }
-  // sum(x) of a group as three bf16 terms (all 24 bits), see qmm_kernel
+  uint32_t rd_col[4];
+#pragma unroll
+  for (int sidx = 0; sidx < 4; ++sidx) rd_col[sidx] = (m + 4 * (sidx >> 1) + 8 * h) & 31;
+  __syncthreads();  // the only workgroup barrier: from here on the waves run on their own
+  qmm_trace(a, work, 2);
+  // sum(x) of a group as three bf16 terms (all 24 bits), see qmm_kernel.  Both halves of the wave hold
+  // the sums of groups 0..7 of the lane's two routes: K slots 8h..8h+7 of the bias product are those
+  // groups again, multiplied by the biases for h = 0 and by -offset * scale for h = 1.
   uint4 b_term[2][3];
 #pragma unroll
   for (int nt = 0; nt < 2; ++nt) {
+    float sx[8];
+#pragma unroll
+    for (int e = 0; e < 8; ++e) sx[e] = e < NG ? s_sum[(nt * 32 + m) * NG + e] : 0.0f;
     uint32_t hi[8], mid[8], lo[8];
 #pragma unroll
     for (int e = 0; e < 8; ++e) {
-      const float v = sx[nt][e];
+      const float v = sx[e];
       hi[e] = __float_as_uint(v) & 0xFFFF0000u;
       const float r1 = v - __uint_as_float(hi[e]);
       mid[e] = __float_as_uint(r1) & 0xFFFF0000u;
@@ -999,11 +1004,6 @@ void qmm_kres_kernel(const KresLaunch launch) {
     b_term[nt][2] = make_uint4(__builtin_amdgcn_perm(lo[1], lo[0], 0x07060302u), __builtin_amdgcn_perm(lo[3], lo[2], 0x07060302u),
                                __builtin_amdgcn_perm(lo[5], lo[4], 0x07060302u), __builtin_amdgcn_perm(lo[7], lo[6], 0x07060302u));
   }
-  uint32_t rd_col[4];
-#pragma unroll
-  for (int sidx = 0; sidx < 4; ++sidx) rd_col[sidx] = (m + 4 * (sidx >> 1) + 8 * h) & 31;
-  __syncthreads();  // the only workgroup barrier: from here on the waves run on their own
-  qmm_trace(a, work, 2);
 
   for (uint32_t w = 0; w < n_walk; ++w) {
     const uint32_t step = w + 1 < n_walk ? 1u : 0u;  // the last slice requests itself again: no branch around loads
@@ -1255,7 +1255,7 @@ hipError_t launch_qmm_kres(hipStream_t s, int bits, const QmmArgs& a, uint32_t t
   const dim3 grid(8 * (launch.per_xcd[0] + launch.per_xcd[1])), block(256);
   if (grid.x == 0) return hipSuccess;
   const uint32_t ng = a.kdim / kGroup;
-  const size_t lds = static_cast<size_t>(ng) * 8192 + kTileTokens * 4;
+  const size_t lds = static_cast<size_t>(ng) * 8192 + kTileTokens * 4 + kTileTokens * ng * 4;
 #define MF_KRES(B, N)                                                                                  \
   do {                                                                                                 \
     if (lds > 48 * 1024) {                                                                             \
@@ -1440,9 +1440,6 @@ hipError_t launch_prefill_layer(hipStream_t s, const mf_moe& h, const mf_moe_lay
   q.out = ws.acts;
   MF_TRY(launch_qmm(s, code_bits, q, 2, max_tiles, shared_rides ? &d : nullptr, dense_tiles));
   if (c.shared_f && !shared_rides) MF_TRY(launch_qmm(s, 4, d, 2, dense_tiles, nullptr, 0));
-  // routes past the last tile's count were never written: only pairs rows exist, all written
-  MF_TRY(launch_prep_rows(s, ws.acts, nullptr, ws.sum_acts, pairs * c.f, ws.sact, nullptr, ws.sum_sact,
-                          static_cast<size_t>(t) * c.shared_f));
   // phase 2: routed down -> fp32 partials [token*K+rank, D]; shared down -> hs [token, D]
   q.w_off[0] = w.offsets.down_w; q.s_off[0] = w.offsets.down_s; q.b_off[0] = ternary ? w.offsets.down_s : w.offsets.down_b;
   q.w_off[1] = q.s_off[1] = q.b_off[1] = 0;
@@ -1456,6 +1453,16 @@ hipError_t launch_prefill_layer(hipStream_t s, const mf_moe& h, const mf_moe_lay
     d.pair_rows = q.pair_rows;
   }
   const bool kres_q = kres_takes(q, pairs), kres_d = c.shared_f && kres_takes(d, t);
+  {
+    // group sums of the activation rows for qmm_kernel (qmm_kres_kernel sums the rows it stages itself);
+    // routes past the last tile's count were never written: only pairs rows exist, all written
+    const bool q_ring = !(kres_q && (!shared_rides || (kres_d && d.kdim == q.kdim)));
+    const bool d_ring = c.shared_f && !(kres_d && (!shared_rides || (kres_q && d.kdim == q.kdim)));
+    if (q_ring || d_ring)
+      MF_TRY(launch_prep_rows(s, q_ring ? ws.acts : nullptr, nullptr, ws.sum_acts, q_ring ? pairs * c.f : 0,
+                              d_ring ? ws.sact : nullptr, nullptr, ws.sum_sact,
+                              d_ring ? static_cast<size_t>(t) * c.shared_f : 0));
+  }
   if (shared_rides) {
     if (kres_q && kres_d && d.kdim == q.kdim) MF_TRY(launch_qmm_kres(s, 4, q, max_tiles, &d, dense_tiles));
     else MF_TRY(launch_qmm(s, 4, q, q.pair_rows ? 2 : 1, max_tiles, &d, dense_tiles));

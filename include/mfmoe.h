@@ -204,6 +204,60 @@ mf_status mf_moe_router(mf_moe* h, mf_stream stream, const uint16_t* router_w,
                         const uint16_t* x, uint32_t t, uint32_t x_stride, uint32_t* out_idx,
                         float* out_w, float* out_logits);
 
+/* ---- family-specific routers.  Stand-alone (no operator handle): the logits go through the
+ * caller's fp32 buffer `logits` [t, rows], which stands in for the operators' internal
+ * routerLogits buffer (MoEDeepseekV4.swift:31-87, InklingKernels.swift:377-417).  All keep the
+ * tie rule of mf_moe_router (equal score keeps the lower index) and write fp32 routing
+ * weights where the reference narrows to fp16.  top_k <= MF_MAX_TOPK, experts <=
+ * MF_MAX_EXPERTS, d a multiple of 8; x rows as in mf_moe_router.  Their outputs feed
+ * mf_moe_phase1 / mf_moe_phase2 like mf_moe_router's. */
+
+/* MoEDeepseekV4.encodeRouterTopK (Kernels/MoE/MoEDeepseekV4.swift:92-124): bf16 router GEMV
+ * (router_gemv_bf16_r4, Metal/MoE/moe.metal:162-185), then
+ * router_topk_select_sqrtsoftplus_k6(_par) (moe.metal:744-841): experts are picked on
+ * sqrt(softplus(logit)) + correction_bias[e], weighed by the raw scores of the picked,
+ * renormalised and times route_scale.  correction_bias fp32 [num_experts]. */
+mf_status mf_router_sqrtsoftplus(mf_ctx* ctx, mf_stream stream, const uint16_t* router_w,
+                                 const uint16_t* x, uint32_t t, uint32_t x_stride,
+                                 uint32_t num_experts, uint32_t d, uint32_t top_k,
+                                 const float* correction_bias, float route_scale, float* logits,
+                                 uint32_t* out_idx, float* out_w);
+
+/* MoEDeepseekV4.encodeRouterHashWeights (MoEDeepseekV4.swift:126-151),
+ * router_hash_weights_k6(_par) (moe.metal:847-896): the experts of every token are given
+ * (indices uint32 [t, top_k], repeats allowed); only their weights are computed.  An index
+ * >= num_experts gets weight 0. */
+mf_status mf_router_hash_weights(mf_ctx* ctx, mf_stream stream, const uint16_t* router_w,
+                                 const uint16_t* x, uint32_t t, uint32_t x_stride,
+                                 uint32_t num_experts, uint32_t d, uint32_t top_k,
+                                 const uint32_t* indices, float route_scale, float* logits,
+                                 float* out_w);
+
+/* InklingKernels.encodeRouter / encodeRouterPrefill (Kernels/Inkling/InklingKernels.swift:
+ * 377-476), inkling_router_select(_prefill) (Metal/Inkling/inkling.metal:503-626): router_w
+ * bf16 [n_routed + n_shared, d], the shared-expert sink rows last.  Experts are picked on
+ * sigmoid(logit) + gate_bias[e] (fp32 [n_routed]); weights are the softmax over logsigmoid of
+ * the raw logits of the picked experts and the sinks, times route_scale * global_scale[0]
+ * (device fp32).  out_gammas fp32 [t, n_shared] (may be NULL when n_shared == 0);
+ * n_shared <= 8; out_idx / out_w are [t, top_k] (the reference's fixed stride is 8). */
+mf_status mf_router_inkling(mf_ctx* ctx, mf_stream stream, const uint16_t* router_w,
+                            const uint16_t* x, uint32_t t, uint32_t x_stride, uint32_t n_routed,
+                            uint32_t n_shared, uint32_t d, uint32_t top_k, const float* gate_bias,
+                            const float* global_scale, float route_scale, float* logits,
+                            uint32_t* out_idx, float* out_w, float* out_gammas);
+
+/* MoE.encodeRouterGemma4 (Kernels/MoE/MoE.swift:153-202): router_gemv_gemma4_r4
+ * (moe.metal:102-157) over 8-bit affine router rows (codes uint8 [num_experts, d], bf16
+ * scales and biases [num_experts, d/64]) with x scaled element-wise by effective_scale
+ * (bf16 [d]), then router_topk_select_k8(_par) (moe.metal:190-345): softmax over the picked
+ * experts times per_expert_scale[e] (bf16 [num_experts]).  d a multiple of 64. */
+mf_status mf_router_gemma4(mf_ctx* ctx, mf_stream stream, const uint8_t* router_codes,
+                           const uint16_t* router_scales, const uint16_t* router_biases,
+                           const uint16_t* x, uint32_t t, uint32_t x_stride,
+                           const uint16_t* effective_scale, const uint16_t* per_expert_scale,
+                           uint32_t num_experts, uint32_t d, uint32_t top_k, float* logits,
+                           uint32_t* out_idx, float* out_w);
+
 /* Routed phase 1: acts[t,k,f] = bf16(act(gate.x) * up.x).
  * MoE.encodeRoutedPersistentPhase1U16Load (MoE.swift:220-253),
  * MoEDeepseekV4.encodeRoutedPhase1 (MoEDeepseekV4.swift:191-199),
@@ -227,7 +281,12 @@ mf_status mf_moe_phase2(mf_moe* h, mf_stream stream, const void* expert_base,
 
 /* Everything one layer reads. */
 typedef struct {
-  const uint16_t* router_w;   /* bf16 [num_experts, d] */
+  const uint16_t* router_w;   /* bf16 [num_experts, d]; NULL: the routing is the caller's -- the layer
+                               * calls then READ out_idx / out_w (both required, e.g. written by a
+                               * family router above; the reference's runners likewise route first and
+                               * hand the result to the expert phases,
+                               * RealForwardRunner+DSV4Prefill.swift:690-806) and run no router.  An
+                               * index >= num_experts contributes nothing. */
   const void* expert_base;
   size_t expert_stride;
   mf_expert_offsets offsets;

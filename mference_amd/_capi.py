@@ -82,6 +82,11 @@ SIGNATURES = {
     "mf_moe_create": (_I, [_P, C.POINTER(MoEConfig), C.POINTER(_P)]),
     "mf_moe_destroy": (None, [_P]),
     "mf_moe_router": (_I, [_P, _P, _P, _P, _U32, _U32, _P, _P, _P]),
+    "mf_router_sqrtsoftplus": (_I, [_P, _P, _P, _P, _U32, _U32, _U32, _U32, _U32, _P, C.c_float, _P, _P, _P]),
+    "mf_router_hash_weights": (_I, [_P, _P, _P, _P, _U32, _U32, _U32, _U32, _U32, _P, C.c_float, _P, _P]),
+    "mf_router_inkling": (_I, [_P, _P, _P, _P, _U32, _U32, _U32, _U32, _U32, _U32, _P, _P, C.c_float, _P,
+                               _P, _P, _P]),
+    "mf_router_gemma4": (_I, [_P, _P, _P, _P, _P, _P, _U32, _U32, _P, _P, _U32, _U32, _U32, _P, _P, _P]),
     "mf_moe_phase1": (_I, [_P, _P, _P, _SZ, C.POINTER(ExpertOffsets), _P, _P, _U32, _U32, _P]),
     "mf_moe_phase2": (_I, [_P, _P, _P, _SZ, C.POINTER(ExpertOffsets), _P, _P, _P, _P, _U32, _P]),
     "mf_moe_decode_layer": (_I, [_P, _P, C.POINTER(LayerWeights), _P, _U32, _P, _P, _P, _P]),

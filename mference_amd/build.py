@@ -8,7 +8,7 @@ import sys
 HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 LIB = os.path.join(HERE, "libmfmoe.so")
-SOURCES = ["format.hip", "gemv.hip", "router.hip", "moe_decode.hip", "moe_fused.hip", "moe_prefill.hip", "api.hip"]
+SOURCES = ["format.hip", "gemv.hip", "router.hip", "router_family.hip", "moe_decode.hip", "moe_fused.hip", "moe_prefill.hip", "api.hip"]
 
 FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-shared",

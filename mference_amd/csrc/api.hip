@@ -287,6 +287,85 @@ mf_status mf_moe_router(mf_moe* h, mf_stream stream, const uint16_t* router_w, c
   return MF_OK;
 }
 
+namespace {
+// the checks the four family routers share
+mf_status family_args_ok(const mf_ctx* ctx, const void* w, const uint16_t* x, uint32_t t, uint32_t x_stride,
+                         uint32_t rows, uint32_t d, uint32_t top_k, const float* logits) {
+  if (!ctx || !w || !x || !logits) return MF_ERR_INVALID_ARGUMENT;
+  if (t == 0 || d == 0 || d % 8 != 0 || x_stride < d) return MF_ERR_INVALID_ARGUMENT;
+  if (rows == 0 || rows > MF_MAX_EXPERTS) return MF_ERR_NUM_EXPERTS;
+  if (top_k == 0 || top_k > MF_MAX_TOPK) return MF_ERR_TOPK;
+  if (!mf::aligned2(x) || (reinterpret_cast<uintptr_t>(logits) & 3u)) return MF_ERR_INVALID_ARGUMENT;
+  return MF_OK;
+}
+}  // namespace
+
+mf_status mf_router_sqrtsoftplus(mf_ctx* ctx, mf_stream stream, const uint16_t* router_w, const uint16_t* x,
+                                 uint32_t t, uint32_t x_stride, uint32_t num_experts, uint32_t d,
+                                 uint32_t top_k, const float* correction_bias, float route_scale,
+                                 float* logits, uint32_t* out_idx, float* out_w) {
+  const mf_status st = family_args_ok(ctx, router_w, x, t, x_stride, num_experts, d, top_k, logits);
+  if (st != MF_OK) return st;
+  if (!correction_bias || !out_idx || !out_w || !mf::aligned2(router_w)) return MF_ERR_INVALID_ARGUMENT;
+  auto s = static_cast<hipStream_t>(stream);
+  MF_HIP(ctx, mf::launch_router_logits(s, router_w, x, num_experts, d, t, x_stride, logits, nullptr));
+  MF_HIP(ctx, mf::launch_select_sqrtsoftplus(s, logits, correction_bias, num_experts, top_k, t, route_scale,
+                                             out_idx, out_w));
+  return MF_OK;
+}
+
+mf_status mf_router_hash_weights(mf_ctx* ctx, mf_stream stream, const uint16_t* router_w, const uint16_t* x,
+                                 uint32_t t, uint32_t x_stride, uint32_t num_experts, uint32_t d,
+                                 uint32_t top_k, const uint32_t* indices, float route_scale, float* logits,
+                                 float* out_w) {
+  const mf_status st = family_args_ok(ctx, router_w, x, t, x_stride, num_experts, d, top_k, logits);
+  if (st != MF_OK) return st;
+  if (!indices || !out_w || !mf::aligned2(router_w)) return MF_ERR_INVALID_ARGUMENT;
+  auto s = static_cast<hipStream_t>(stream);
+  MF_HIP(ctx, mf::launch_router_logits(s, router_w, x, num_experts, d, t, x_stride, logits, nullptr));
+  MF_HIP(ctx, mf::launch_hash_weights(s, logits, indices, num_experts, top_k, t, route_scale, out_w));
+  return MF_OK;
+}
+
+mf_status mf_router_inkling(mf_ctx* ctx, mf_stream stream, const uint16_t* router_w, const uint16_t* x,
+                            uint32_t t, uint32_t x_stride, uint32_t n_routed, uint32_t n_shared, uint32_t d,
+                            uint32_t top_k, const float* gate_bias, const float* global_scale,
+                            float route_scale, float* logits, uint32_t* out_idx, float* out_w,
+                            float* out_gammas) {
+  if (n_shared > 8) return MF_ERR_INVALID_ARGUMENT;
+  const mf_status st = family_args_ok(ctx, router_w, x, t, x_stride, n_routed, d, top_k, logits);
+  if (st != MF_OK) return st;
+  if (!gate_bias || !global_scale || !out_idx || !out_w || (n_shared && !out_gammas) ||
+      !mf::aligned2(router_w))
+    return MF_ERR_INVALID_ARGUMENT;
+  auto s = static_cast<hipStream_t>(stream);
+  MF_HIP(ctx, mf::launch_router_logits(s, router_w, x, n_routed + n_shared, d, t, x_stride, logits, nullptr));
+  MF_HIP(ctx, mf::launch_select_inkling(s, logits, gate_bias, global_scale, n_routed, n_shared, top_k, t,
+                                        route_scale, out_idx, out_w, out_gammas));
+  return MF_OK;
+}
+
+mf_status mf_router_gemma4(mf_ctx* ctx, mf_stream stream, const uint8_t* router_codes,
+                           const uint16_t* router_scales, const uint16_t* router_biases, const uint16_t* x,
+                           uint32_t t, uint32_t x_stride, const uint16_t* effective_scale,
+                           const uint16_t* per_expert_scale, uint32_t num_experts, uint32_t d, uint32_t top_k,
+                           float* logits, uint32_t* out_idx, float* out_w) {
+  const mf_status st = family_args_ok(ctx, router_codes, x, t, x_stride, num_experts, d, top_k, logits);
+  if (st != MF_OK) return st;
+  if (d % MF_GROUP_SIZE != 0) return MF_ERR_DIMENSION_MISMATCH;
+  if (!router_scales || !router_biases || !effective_scale || !per_expert_scale || !out_idx || !out_w)
+    return MF_ERR_INVALID_ARGUMENT;
+  if (!mf::aligned2(router_scales) || !mf::aligned2(router_biases) || !mf::aligned2(effective_scale) ||
+      !mf::aligned2(per_expert_scale))
+    return MF_ERR_INVALID_ARGUMENT;
+  auto s = static_cast<hipStream_t>(stream);
+  MF_HIP(ctx, mf::launch_router_logits_int8(s, router_codes, router_scales, router_biases, x, effective_scale,
+                                            num_experts, d, t, x_stride, logits));
+  MF_HIP(ctx, mf::launch_select_scaled_softmax(s, logits, per_expert_scale, num_experts, top_k, t, out_idx,
+                                               out_w));
+  return MF_OK;
+}
+
 mf_status mf_moe_phase1(mf_moe* h, mf_stream stream, const void* expert_base,
                         size_t expert_stride, const mf_expert_offsets* offsets,
                         const uint32_t* idx, const uint16_t* x, uint32_t t, uint32_t x_stride,
@@ -321,7 +400,9 @@ mf_status mf_moe_decode_layer(mf_moe* h, mf_stream stream, const mf_moe_layer_we
   if (!h || !wts || !x || !y) return MF_ERR_INVALID_ARGUMENT;
   if (t == 0 || t > MF_MAX_TOKENS) return MF_ERR_INVALID_ARGUMENT;
   const mf_moe_config& c = h->cfg;
-  if (!wts->router_w || !wts->expert_base || !offsets_ok(wts->offsets, c.bits) ||
+  // no router weights: the routing in out_idx / out_w is the caller's (a family router wrote it)
+  const bool given = !wts->router_w;
+  if ((given && (!out_idx || !out_w)) || !wts->expert_base || !offsets_ok(wts->offsets, c.bits) ||
       !mf::aligned2(wts->expert_base) || (wts->expert_stride & 1) || !mf::aligned2(x) ||
       !mf::aligned2(y) || (hidden && !mf::aligned2(hidden)))
     return MF_ERR_INVALID_ARGUMENT;
@@ -330,15 +411,17 @@ mf_status mf_moe_decode_layer(mf_moe* h, mf_stream stream, const mf_moe_layer_we
                      !qtensor_ok(wts->shared_down, c.shared_bits)))
     return MF_ERR_INVALID_ARGUMENT;
   auto s = static_cast<hipStream_t>(stream);
-  if (h->fused && mf::fused_supported(*h, *wts, x, y, hidden)) {
+  if (!given && h->fused && mf::fused_supported(*h, *wts, x, y, hidden)) {
     MF_HIP(h->ctx, mf::launch_fused_decode(s, *h, *wts, x, t, y, hidden, out_idx, out_w));
     return MF_OK;
   }
-  uint32_t* idx = h->ws.idx;
-  float* w = h->ws.w;
-  MF_HIP(h->ctx, mf::launch_router_logits(s, wts->router_w, x, c.num_experts, c.d, t, c.d,
-                                          h->ws.logits, nullptr));
-  MF_HIP(h->ctx, mf::launch_topk(s, h->ws.logits, c.num_experts, c.top_k, t, c.router_mode, idx, w));
+  uint32_t* idx = given ? out_idx : h->ws.idx;
+  float* w = given ? out_w : h->ws.w;
+  if (!given) {
+    MF_HIP(h->ctx, mf::launch_router_logits(s, wts->router_w, x, c.num_experts, c.d, t, c.d,
+                                            h->ws.logits, nullptr));
+    MF_HIP(h->ctx, mf::launch_topk(s, h->ws.logits, c.num_experts, c.top_k, t, c.router_mode, idx, w));
+  }
   const uint16_t* residual = nullptr;
   if (c.shared_f) {
     // lane order of the fused kernel: both forms of the layer give the same bits
@@ -357,10 +440,10 @@ mf_status mf_moe_decode_layer(mf_moe* h, mf_stream stream, const mf_moe_layer_we
   MF_HIP(h->ctx, mf::launch_phase2(s, c, wts->expert_base, wts->expert_stride, wts->offsets, idx, w,
                                    h->ws.acts, residual, t, y));
   if (hidden) MF_HIP(h->ctx, mf::launch_residual_add(s, hidden, y, t * c.d));
-  if (out_idx)
+  if (out_idx && !given)
     MF_HIP(h->ctx, hipMemcpyAsync(out_idx, idx, sizeof(uint32_t) * t * c.top_k,
                                   hipMemcpyDeviceToDevice, s));
-  if (out_w)
+  if (out_w && !given)
     MF_HIP(h->ctx, hipMemcpyAsync(out_w, w, sizeof(float) * t * c.top_k, hipMemcpyDeviceToDevice, s));
   return MF_OK;
 }
@@ -447,7 +530,7 @@ mf_status mf_moe_prefill_layer(mf_moe* h, mf_stream stream, const mf_moe_layer_w
   if (!workspace) return MF_ERR_INVALID_ARGUMENT;
   if (workspace_bytes < mf::prefill_workspace_bytes(c, t)) return MF_ERR_SCRATCH_TOO_SMALL;
   const uint32_t offs = wts->offsets.gate_w | wts->offsets.up_w | wts->offsets.down_w;
-  if (!wts->router_w || !wts->expert_base || !offsets_ok(wts->offsets, c.bits) ||
+  if ((!wts->router_w && (!out_idx || !out_w)) || !wts->expert_base || !offsets_ok(wts->offsets, c.bits) ||
       !mf::aligned16(wts->expert_base) || wts->expert_stride % 16 || offs % 16 ||
       !mf::aligned16(wts->router_w) || !mf::aligned16(x) || !mf::aligned16(y) ||
       !mf::aligned16(workspace))

@@ -69,6 +69,29 @@ __device__ __forceinline__ float mf_exp(float x) {
   return p * __uint_as_float(static_cast<uint32_t>(e) << 23);
 }
 
+// log(t) for 1 <= t <= 2 (t = 1 + exp(-|x|) in the routers): 2*atanh((t-1)/(t+1)), odd series
+// through s^15; the same IEEE sequence as the CPU checker.
+__device__ __forceinline__ float mf_log_1to2(float t) {
+  const float s = (t - 1.0f) / (t + 1.0f);
+  const float z = s * s;
+  float p = 6.6666666667e-2f;
+  p = __builtin_fmaf(p, z, 7.6923076923e-2f);
+  p = __builtin_fmaf(p, z, 9.0909090909e-2f);
+  p = __builtin_fmaf(p, z, 1.1111111111e-1f);
+  p = __builtin_fmaf(p, z, 1.4285714286e-1f);
+  p = __builtin_fmaf(p, z, 2.0e-1f);
+  p = __builtin_fmaf(p, z, 3.3333333333e-1f);
+  float r = s * z;
+  r = __builtin_fmaf(r, p, s);
+  return r + r;
+}
+
+// moe.metal:736-740
+__device__ __forceinline__ float mf_sqrtsoftplus(float x) {
+  const float sp = (x > 0.0f ? x : 0.0f) + mf_log_1to2(1.0f + mf_exp(-__builtin_fabsf(x)));
+  return __builtin_sqrtf(sp);
+}
+
 // moe.metal:79-84
 __device__ __forceinline__ float mf_silu(float x) { return x / (1.0f + mf_exp(-x)); }
 

@@ -88,6 +88,20 @@ hipError_t launch_router_logits(hipStream_t s, const uint16_t* w, const uint16_t
 hipError_t launch_topk(hipStream_t s, const float* logits, uint32_t e, uint32_t k, uint32_t t,
                        int mode, uint32_t* idx, float* w);
 
+// router_family.hip
+hipError_t launch_router_logits_int8(hipStream_t s, const uint8_t* codes, const uint16_t* scales,
+                                     const uint16_t* biases, const uint16_t* x, const uint16_t* eff,
+                                     uint32_t e, uint32_t d, uint32_t t, uint32_t x_stride, float* logits);
+hipError_t launch_select_sqrtsoftplus(hipStream_t s, const float* logits, const float* bias, uint32_t e,
+                                      uint32_t k, uint32_t t, float route_scale, uint32_t* idx, float* w);
+hipError_t launch_hash_weights(hipStream_t s, const float* logits, const uint32_t* given, uint32_t e,
+                               uint32_t k, uint32_t t, float route_scale, float* w);
+hipError_t launch_select_inkling(hipStream_t s, const float* logits, const float* bias,
+                                 const float* global_scale, uint32_t n_routed, uint32_t n_shared, uint32_t k,
+                                 uint32_t t, float route_scale, uint32_t* idx, float* w, float* gammas);
+hipError_t launch_select_scaled_softmax(hipStream_t s, const float* logits, const uint16_t* expert_scale,
+                                        uint32_t e, uint32_t k, uint32_t t, uint32_t* idx, float* w);
+
 // moe_decode.hip
 hipError_t launch_phase1(hipStream_t s, const mf_moe_config& cfg, const void* base, size_t stride,
                          const mf_expert_offsets& off, const uint32_t* idx, const uint16_t* x,

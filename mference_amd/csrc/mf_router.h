@@ -55,7 +55,8 @@ constexpr uint32_t kNoWinner = 0xFFFFFFFFu;
 // lane r; weights are exp(s_r - s_0) / sum with the sum taken in rank order.
 // All 64 lanes call it.
 // MODE 1: lg holds probabilities of the full softmax; the weights are p_r / (sum + 1e-20)
-// with the sum in rank order (maple_moe.metal:100-118).
+// with the sum in rank order (maple_moe.metal:100-118).  MODE 2: lg holds selection scores of a
+// family router, only the indices are written.
 template <int PER, int MODE = 0>
 __device__ __forceinline__ void topk_select_sorted(const float* lg, uint32_t e, uint32_t k,
                                                    uint32_t* idx, float* w, uint32_t lane) {
@@ -107,6 +108,10 @@ __device__ __forceinline__ void topk_select_sorted(const float* lg, uint32_t e, 
       my_score = ws;
       my_idx = widx;
     }
+  }
+  if constexpr (MODE == 2) {  // indices only: the caller weighs them
+    if (lane < k) idx[lane] = my_idx;
+    return;
   }
   if constexpr (MODE == 1) {
     float sum = 0.0f;
@@ -206,6 +211,16 @@ __device__ __forceinline__ void topk_select_fast(const float* lg, uint32_t e, ui
   else if (per <= 2) topk_select_sorted<2>(lg, e, k, idx, w, lane);
   else if (per <= 4) topk_select_sorted<4>(lg, e, k, idx, w, lane);
   else topk_select_sorted<8>(lg, e, k, idx, w, lane);
+}
+
+// indices of the k best selection scores (same tie rule), for the family routers
+__device__ __forceinline__ void topk_select_indices(const float* score, uint32_t e, uint32_t k,
+                                                    uint32_t* idx, uint32_t lane) {
+  const uint32_t per = (e + kWave - 1) / kWave;
+  if (per <= 1) topk_select_sorted<1, 2>(score, e, k, idx, nullptr, lane);
+  else if (per <= 2) topk_select_sorted<2, 2>(score, e, k, idx, nullptr, lane);
+  else if (per <= 4) topk_select_sorted<4, 2>(score, e, k, idx, nullptr, lane);
+  else topk_select_sorted<8, 2>(score, e, k, idx, nullptr, lane);
 }
 
 }  // namespace mf

@@ -1398,8 +1398,10 @@ hipError_t launch_prefill_layer(hipStream_t s, const mf_moe& h, const mf_moe_lay
 #define MF_TRY(call) do { e = (call); if (e != hipSuccess) return e; } while (0)
   const size_t pairs = static_cast<size_t>(t) * c.top_k;
   const uint32_t max_tiles = prefill_tile_slots(c, t);
-  MF_TRY(launch_prefill_router(s, w.router_w, x, c.num_experts, c.d, t, c.d, ws.logits));
-  MF_TRY(launch_topk(s, ws.logits, c.num_experts, c.top_k, t, c.router_mode, ws.idx, ws.w));
+  if (w.router_w) {  // else the routing in out_idx / out_w is the caller's
+    MF_TRY(launch_prefill_router(s, w.router_w, x, c.num_experts, c.d, t, c.d, ws.logits));
+    MF_TRY(launch_topk(s, ws.logits, c.num_experts, c.top_k, t, c.router_mode, ws.idx, ws.w));
+  }
   MF_TRY(launch_group(s, ws.idx, ws.w, t, c.top_k, c.num_experts, ws.counts, ws.offsets, ws.starts,
                       ws.sorted, ws.tiles, max_tiles, ws.n_tiles, ws.status, h.ws.group_tmp + 2048));
 

@@ -21,7 +21,7 @@ from ._capi import (BITS_2, BITS_4, BITS_TERNARY, GROUP_SIZE, MAX_TOKENS, ROUTER
 
 __all__ = [
     "MetalContext", "QuantizedTensor", "Quantization", "DequantInt4GEMV", "DequantInt4GEMVMultiX",
-    "Elementwise", "SharedExpertInt4", "MoEExpertOffsets", "MoE", "MoELayerWeights",
+    "Elementwise", "FamilyRouters", "SharedExpertInt4", "MoEExpertOffsets", "MoE", "MoELayerWeights",
     "PrefillMoEGrouping", "PrefillTokenExpertPair", "MfError", "BITS_2", "BITS_4", "BITS_TERNARY",
     "ROUTER_TOPK_SOFTMAX", "ROUTER_FULL_SOFTMAX", "bf16_tensor", "bf16_bits",
 ]
@@ -205,6 +205,55 @@ class SharedExpertInt4:
             self.context.handle, _stream(stream), _ptr(x), gate.c(), up.c(), down.c(), gate.bits,
             gate.n, gate.rows, t, _ptr(y), _ptr(scratch_act),
             scratch_act.numel() * scratch_act.element_size()), self.context.handle)
+
+
+class FamilyRouters:
+    """The family-specific routers of the reference's operator classes, stand-alone: every call
+    runs the router GEMV into the caller's fp32 `logits` buffer [t, rows] and then the selection.
+    Routing weights are fp32 (the reference narrows them to fp16)."""
+
+    def __init__(self, context: MetalContext):
+        self.context = context
+
+    def encode_router_top_k(self, weights, hidden, correction_bias, out_indices, out_weights,
+                            num_experts: int, d: int, route_scale: float, logits, top_k: int = 6,
+                            t: int = 1, x_stride: Optional[int] = None, stream=None):
+        """MoEDeepseekV4.encodeRouterTopK (MoEDeepseekV4.swift:92-124): sqrtsoftplus selection."""
+        check(_capi.lib().mf_router_sqrtsoftplus(
+            self.context.handle, _stream(stream), _ptr(weights), _ptr(hidden), t,
+            d if x_stride is None else x_stride, num_experts, d, top_k, _ptr(correction_bias),
+            route_scale, _ptr(logits), _ptr(out_indices), _ptr(out_weights)), self.context.handle)
+
+    def encode_router_hash_weights(self, weights, hidden, indices, out_weights, num_experts: int,
+                                   d: int, route_scale: float, logits, top_k: int = 6, t: int = 1,
+                                   x_stride: Optional[int] = None, stream=None):
+        """MoEDeepseekV4.encodeRouterHashWeights (MoEDeepseekV4.swift:126-151)."""
+        check(_capi.lib().mf_router_hash_weights(
+            self.context.handle, _stream(stream), _ptr(weights), _ptr(hidden), t,
+            d if x_stride is None else x_stride, num_experts, d, top_k, _ptr(indices), route_scale,
+            _ptr(logits), _ptr(out_weights)), self.context.handle)
+
+    def encode_router_inkling(self, weights, hidden, gate_bias, global_scale, out_indices,
+                              out_weights, gammas_out, num_routed: int, num_shared: int, top_k: int,
+                              route_scale: float, d: int, logits, t: int = 1,
+                              x_stride: Optional[int] = None, stream=None):
+        """InklingKernels.encodeRouter / encodeRouterPrefill (InklingKernels.swift:377-476)."""
+        check(_capi.lib().mf_router_inkling(
+            self.context.handle, _stream(stream), _ptr(weights), _ptr(hidden), t,
+            d if x_stride is None else x_stride, num_routed, num_shared, d, top_k, _ptr(gate_bias),
+            _ptr(global_scale), route_scale, _ptr(logits), _ptr(out_indices), _ptr(out_weights),
+            _ptr(gammas_out)), self.context.handle)
+
+    def encode_router_gemma4(self, weights, scales, biases, hidden, effective_scale,
+                             per_expert_scale, out_indices, out_weights, num_experts: int, d: int,
+                             top_k: int, logits, t: int = 1, x_stride: Optional[int] = None,
+                             stream=None):
+        """MoE.encodeRouterGemma4 (MoE.swift:153-202): 8-bit affine router rows."""
+        check(_capi.lib().mf_router_gemma4(
+            self.context.handle, _stream(stream), _ptr(weights), _ptr(scales), _ptr(biases),
+            _ptr(hidden), t, d if x_stride is None else x_stride, _ptr(effective_scale),
+            _ptr(per_expert_scale), num_experts, d, top_k, _ptr(logits), _ptr(out_indices),
+            _ptr(out_weights)), self.context.handle)
 
 
 @dataclass

@@ -416,6 +416,158 @@ void mfo_topk_full_softmax(const float* logits, size_t e, size_t k, uint32_t* id
   free(scores);
 }
 
+/* ------------------------------------------------------- family routers */
+
+/* The selection rule every router of the reference shares (moe.metal:209-225,
+ * :764-780; inkling.metal:526-538): scan the experts in ascending order, a
+ * strictly greater score goes ahead, an equal score stays behind the earlier
+ * expert.  NaN and -inf are never taken; slots nobody filled keep index 0. */
+static void select_topk(const float* s, size_t e, size_t k, uint32_t* idx, float* score) {
+  for (size_t i = 0; i < k; ++i) {
+    idx[i] = 0;
+    score[i] = -INFINITY;
+  }
+  for (size_t x = 0; x < e; ++x) {
+    float v = s[x];
+    if (!(v > score[k - 1])) continue;
+    size_t pos = k - 1;
+    while (pos > 0 && score[pos - 1] < v) --pos;
+    for (size_t i = k - 1; i > pos; --i) {
+      idx[i] = idx[i - 1];
+      score[i] = score[i - 1];
+    }
+    idx[pos] = (uint32_t)x;
+    score[pos] = v;
+  }
+}
+
+/* log(t) for 1 <= t <= 2, the only range the routers need (t = 1 + exp(-|x|)):
+ * 2*atanh(s) with s = (t-1)/(t+1) <= 1/3, odd series through s^15 in fmaf
+ * form.  t-1 and t+1 are exact, the truncated tail is below 2e-9 relative.  The
+ * HIP kernels run the same IEEE sequence, so results agree bit for bit. */
+float mfo_log_1to2(float t) {
+  float s = (t - 1.0f) / (t + 1.0f);
+  float z = s * s;
+  float p = 6.6666666667e-2f;          /* 1/15 */
+  p = fmaf(p, z, 7.6923076923e-2f);    /* 1/13 */
+  p = fmaf(p, z, 9.0909090909e-2f);    /* 1/11 */
+  p = fmaf(p, z, 1.1111111111e-1f);    /* 1/9 */
+  p = fmaf(p, z, 1.4285714286e-1f);    /* 1/7 */
+  p = fmaf(p, z, 2.0e-1f);             /* 1/5 */
+  p = fmaf(p, z, 3.3333333333e-1f);    /* 1/3 */
+  float r = s * z;
+  r = fmaf(r, p, s);
+  return r + r;
+}
+
+/* moe.metal:736-740: sqrt(max(x,0) + log(1 + exp(-|x|))) */
+float mfo_sqrtsoftplus(float x) {
+  float sp = (x > 0.0f ? x : 0.0f) + mfo_log_1to2(1.0f + mfo_exp(-fabsf(x)));
+  return sqrtf(sp);
+}
+
+/* router_topk_select_sqrtsoftplus_k6 (moe.metal:744-786) for any k <= 8: the
+ * selection score carries the correction bias, the weights do not; weights are
+ * kept fp32 (the reference narrows them to fp16 at :784). */
+void mfo_router_sqrtsoftplus(const float* logits, const float* correction_bias, size_t e, size_t k,
+                             float route_scale, uint32_t* idx, float* w) {
+  float* sel = (float*)malloc(e * sizeof(float));
+  float score[8];
+  for (size_t x = 0; x < e; ++x) sel[x] = mfo_sqrtsoftplus(logits[x]) + correction_bias[x];
+  select_topk(sel, e, k, idx, score);
+  free(sel);
+  mfo_router_hash_weights(logits, idx, k, route_scale, w);
+}
+
+/* router_hash_weights_k6 (moe.metal:847-866): the experts are given. */
+void mfo_router_hash_weights(const float* logits, const uint32_t* idx, size_t k, float route_scale,
+                             float* w) {
+  float sum = 0.0f;
+  for (size_t i = 0; i < k; ++i) {
+    w[i] = mfo_sqrtsoftplus(logits[idx[i]]);
+    sum += w[i];
+  }
+  const float inv = route_scale / (sum + 1e-20f);
+  for (size_t i = 0; i < k; ++i) w[i] = w[i] * inv;
+}
+
+/* inkling_router_select (inkling.metal:503-566): selection on sigmoid(logit) +
+ * bias over the routed experts; weights are a softmax over the logsigmoid of
+ * the RAW logits of the selected experts and the n_shared sink rows that follow
+ * the routed ones, times route_scale * global_scale.  k <= 8, n_shared <= 8. */
+void mfo_router_inkling(const float* logits, const float* bias, float global_scale,
+                        size_t n_routed, size_t n_shared, size_t k, float route_scale,
+                        uint32_t* idx, float* w, float* gammas) {
+  float* sel = (float*)malloc(n_routed * sizeof(float));
+  float score[8], lp[16], ex[16];
+  for (size_t x = 0; x < n_routed; ++x) sel[x] = 1.0f / (1.0f + mfo_exp(-logits[x])) + bias[x];
+  select_topk(sel, n_routed, k, idx, score);
+  free(sel);
+  const size_t total = k + n_shared;
+  for (size_t i = 0; i < total; ++i) {
+    const float x = i < k ? logits[idx[i]] : logits[n_routed + (i - k)];
+    lp[i] = (x < 0.0f ? x : 0.0f) - mfo_log_1to2(1.0f + mfo_exp(-fabsf(x)));
+  }
+  float mx = -INFINITY;
+  for (size_t i = 0; i < total; ++i) mx = lp[i] > mx ? lp[i] : mx;
+  float denom = 0.0f;
+  for (size_t i = 0; i < total; ++i) {
+    ex[i] = mfo_exp(lp[i] - mx);
+    denom += ex[i];
+  }
+  const float s_all = route_scale * global_scale / denom;
+  for (size_t i = 0; i < k; ++i) w[i] = ex[i] * s_all;
+  for (size_t i = 0; i < n_shared; ++i) gammas[i] = ex[k + i] * s_all;
+}
+
+/* router_gemv_gemma4_body (moe.metal:102-139): 8-bit affine router rows, x
+ * scaled element-wise by effective_scale, per group acc = fma(s, sum q*x', acc);
+ * acc = fma(b, sum x', acc).  The summation order is this build's (the
+ * reference's is one 32-wide Metal SIMD's): 8-wide chunks dealt to 64 lanes as
+ * in mfo_dot_bf16_laneorder, a chunk's two sums by fmaf / add in ascending
+ * order from 0, then the two fmas into the lane's accumulator, then the
+ * neighbour-first butterfly. */
+float mfo_dot_int8_laneorder(const uint8_t* codes, const uint16_t* scales, const uint16_t* biases,
+                             const uint16_t* x, const uint16_t* effective_scale, size_t d) {
+  float p[64];
+  for (int l = 0; l < 64; ++l) p[l] = 0.0f;
+  for (size_t c = 0; c < d / 8; ++c) {
+    float dot = 0.0f, sum = 0.0f;
+    for (int j = 0; j < 8; ++j) {
+      const float xs = mfo_bf16_to_float(x[c * 8 + j]) * mfo_bf16_to_float(effective_scale[c * 8 + j]);
+      dot = fmaf((float)codes[c * 8 + j], xs, dot);
+      sum = sum + xs;
+    }
+    const size_t g = c * 8 / GROUP;
+    float acc = p[c % 64];
+    acc = fmaf(mfo_bf16_to_float(scales[g]), dot, acc);
+    acc = fmaf(mfo_bf16_to_float(biases[g]), sum, acc);
+    p[c % 64] = acc;
+  }
+  for (int s = 1; s <= 32; s <<= 1) {
+    float q[64];
+    for (int l = 0; l < 64; ++l) q[l] = p[l] + p[l ^ s];
+    memcpy(p, q, sizeof p);
+  }
+  return p[0];
+}
+
+void mfo_router_logits_int8(const uint8_t* codes, const uint16_t* scales, const uint16_t* biases,
+                            const uint16_t* x, const uint16_t* effective_scale, size_t e, size_t d,
+                            float* logits) {
+  for (size_t i = 0; i < e; ++i)
+    logits[i] = mfo_dot_int8_laneorder(codes + i * d, scales + i * (d / GROUP), biases + i * (d / GROUP), x,
+                                       effective_scale, d);
+}
+
+/* router_topk_select_k8 with its per-expert scale (moe.metal:190-240): the
+ * softmax weight over the selected, times bf16 per_expert_scale[expert]. */
+void mfo_topk_softmax_scaled(const float* logits, const uint16_t* per_expert_scale, size_t e, size_t k,
+                             uint32_t* idx, float* w) {
+  mfo_topk_softmax(logits, e, k, idx, w);
+  for (size_t i = 0; i < k; ++i) w[i] = w[i] * mfo_bf16_to_float(per_expert_scale[idx[i]]);
+}
+
 /* ------------------------------------------------------------------ GEMV */
 
 /* DequantInt4Gemv.swift:26-40 with the scalar loop of

@@ -86,6 +86,30 @@ void mfo_topk_softmax(const float* logits, size_t e, size_t k, uint32_t* idx, fl
 /* full softmax -> k x argmax -> renormalise (maple_moe.metal:62-119) */
 void mfo_topk_full_softmax(const float* logits, size_t e, size_t k, uint32_t* idx, float* w);
 
+/* ---- family routers (all share the tie rule of mfo_topk_softmax) -------- */
+/* log(t) on [1,2] and sqrt(softplus(x)) (moe.metal:736-740), IEEE sequences shared with the kernels */
+float mfo_log_1to2(float t);
+float mfo_sqrtsoftplus(float x);
+/* router_topk_select_sqrtsoftplus_k6 (moe.metal:744-786), k <= 8 */
+void mfo_router_sqrtsoftplus(const float* logits, const float* correction_bias, size_t e, size_t k,
+                             float route_scale, uint32_t* idx, float* w);
+/* router_hash_weights_k6 (moe.metal:847-866), k <= 8 */
+void mfo_router_hash_weights(const float* logits, const uint32_t* idx, size_t k, float route_scale,
+                             float* w);
+/* inkling_router_select (inkling.metal:503-566); logits [n_routed + n_shared] */
+void mfo_router_inkling(const float* logits, const float* bias, float global_scale,
+                        size_t n_routed, size_t n_shared, size_t k, float route_scale,
+                        uint32_t* idx, float* w, float* gammas);
+/* router_gemv_gemma4_body (moe.metal:102-139) in the build's fixed lane order */
+float mfo_dot_int8_laneorder(const uint8_t* codes, const uint16_t* scales, const uint16_t* biases,
+                             const uint16_t* x, const uint16_t* effective_scale, size_t d);
+void mfo_router_logits_int8(const uint8_t* codes, const uint16_t* scales, const uint16_t* biases,
+                            const uint16_t* x, const uint16_t* effective_scale, size_t e, size_t d,
+                            float* logits);
+/* router_topk_select_k8 incl. per_expert_scale (moe.metal:190-240) */
+void mfo_topk_softmax_scaled(const float* logits, const uint16_t* per_expert_scale, size_t e, size_t k,
+                             uint32_t* idx, float* w);
+
 /* ---- GEMV / expert FFN ------------------------------------------------- */
 /* y[m] = sum_n deq(W[m,n]) * x[n]; bulk dequant then sequential fp32 dot
  * (MferenceValidation/Support/Reference/Quant/DequantInt4Gemv.swift:26-40) */

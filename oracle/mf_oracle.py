@@ -90,6 +90,11 @@ def lib():
                                            C.c_size_t]
         L.mfo_exp.restype = C.c_float
         L.mfo_exp.argtypes = [C.c_float]
+        for fn in (L.mfo_log_1to2, L.mfo_sqrtsoftplus):
+            fn.restype = C.c_float
+            fn.argtypes = [C.c_float]
+        L.mfo_dot_int8_laneorder.restype = C.c_float
+        L.mfo_dot_int8_laneorder.argtypes = [C.c_void_p] * 5 + [C.c_size_t]
         L.mfo_silu.restype = C.c_float
         L.mfo_silu.argtypes = [C.c_float]
         L.mfo_dot_bf16_laneorder.restype = C.c_float
@@ -235,6 +240,72 @@ def topk_softmax(logits, k: int, full_softmax: bool = False):
     w = np.empty(k, np.float32)
     fn = lib().mfo_topk_full_softmax if full_softmax else lib().mfo_topk_softmax
     fn(_p(logits), C.c_size_t(logits.size), C.c_size_t(k), _p(idx), _p(w))
+    return idx, w
+
+
+def log_1to2(t: float) -> float:
+    return float(lib().mfo_log_1to2(C.c_float(t)))
+
+
+def sqrtsoftplus(x: float) -> float:
+    return float(lib().mfo_sqrtsoftplus(C.c_float(x)))
+
+
+def router_sqrtsoftplus(logits, correction_bias, k: int, route_scale: float):
+    """DeepSeek-V4 learned routing: (indices, weights)."""
+    logits = _c(logits, np.float32)
+    bias = _c(correction_bias, np.float32)
+    idx = np.empty(k, np.uint32)
+    w = np.empty(k, np.float32)
+    lib().mfo_router_sqrtsoftplus(_p(logits), _p(bias), C.c_size_t(logits.size), C.c_size_t(k),
+                                  C.c_float(route_scale), _p(idx), _p(w))
+    return idx, w
+
+
+def router_hash_weights(logits, indices, route_scale: float) -> np.ndarray:
+    """DeepSeek-V4 hash routing: weights of the given experts."""
+    logits = _c(logits, np.float32)
+    idx = _c(indices, np.uint32)
+    w = np.empty(idx.size, np.float32)
+    lib().mfo_router_hash_weights(_p(logits), _p(idx), C.c_size_t(idx.size), C.c_float(route_scale), _p(w))
+    return w
+
+
+def router_inkling(logits, bias, global_scale: float, n_routed: int, n_shared: int, k: int,
+                   route_scale: float):
+    """Inkling sigmoid router with shared sinks: (indices, weights, gammas)."""
+    logits = _c(logits, np.float32)
+    bias = _c(bias, np.float32)
+    assert logits.size == n_routed + n_shared and k <= 8 and n_shared <= 8
+    idx = np.empty(k, np.uint32)
+    w = np.empty(k, np.float32)
+    gam = np.empty(max(n_shared, 1), np.float32)
+    lib().mfo_router_inkling(_p(logits), _p(bias), C.c_float(global_scale), C.c_size_t(n_routed),
+                             C.c_size_t(n_shared), C.c_size_t(k), C.c_float(route_scale), _p(idx), _p(w),
+                             _p(gam))
+    return idx, w, gam[:n_shared]
+
+
+def router_logits_int8(codes, scales, biases, x, effective_scale) -> np.ndarray:
+    """Gemma's 8-bit affine router rows in the build's lane order."""
+    codes = _c(codes, np.uint8)
+    scales = _c(scales, np.uint16)
+    biases = _c(biases, np.uint16)
+    x = _c(x, np.uint16)
+    es = _c(effective_scale, np.uint16)
+    e, d = codes.shape
+    out = np.empty(e, np.float32)
+    lib().mfo_router_logits_int8(_p(codes), _p(scales), _p(biases), _p(x), _p(es), C.c_size_t(e),
+                                 C.c_size_t(d), _p(out))
+    return out
+
+
+def topk_softmax_scaled(logits, per_expert_scale, k: int):
+    logits = _c(logits, np.float32)
+    sc = _c(per_expert_scale, np.uint16)
+    idx = np.empty(k, np.uint32)
+    w = np.empty(k, np.float32)
+    lib().mfo_topk_softmax_scaled(_p(logits), _p(sc), C.c_size_t(logits.size), C.c_size_t(k), _p(idx), _p(w))
     return idx, w
 
 

@@ -291,6 +291,117 @@ def test_topk_fewer_experts_than_k_keeps_index_zero():
     assert list(idx[:3]) == [1, 2, 0] and list(idx[3:]) == [0] * 5 and not w[3:].any()
 
 
+# -------------------------------------------------------------- family routers
+
+def test_log_and_sqrtsoftplus_against_fp64():
+    for t in np.linspace(1.0, 2.0, 4097):
+        t = float(np.float32(t))
+        assert abs(O.log_1to2(t) - math.log(t)) <= 1.2e-7 * max(math.log(t), 0.5)
+    assert O.log_1to2(1.0) == 0.0
+    # closed forms: sqrt(ln 2) at 0; the log term vanishes in fp32 beyond |x| = 20
+    assert abs(O.sqrtsoftplus(0.0) - math.sqrt(math.log(2.0))) <= 1e-7
+    for x in (20.0, 33.5, 1000.0):
+        assert O.sqrtsoftplus(x) == float(np.sqrt(np.float32(x)))
+        assert O.sqrtsoftplus(-x) == 0.0
+    for x in np.linspace(-4.0, 12.0, 801):  # moe.metal:736-740 in fp64
+        x = float(np.float32(x))
+        want = math.sqrt(max(x, 0.0) + math.log1p(math.exp(-abs(x))))
+        assert abs(O.sqrtsoftplus(x) - want) <= 1e-5 * want
+
+
+@pytest.mark.parametrize("e", [8, 16, 24, 33, 100, 128, 168, 255, 256])
+def test_sqrtsoftplus_router_selection_and_weights(e):
+    # RouterTopKParityTests.swift:52-77: seeds, tie-heavy logits, duplicated correction biases
+    rng = O.Rng(0x5EED0002 + e)
+    k, route_scale = 6, 1.5
+    for trial in range(12):
+        logits = _tie_logits(e, trial, rng)
+        bias = np.array([np.float32((i // 7) % 4) * np.float32(0.25) if trial % 3 == 0
+                         else rng.uniform(-0.3, 0.3) for i in range(e)], np.float32)
+        idx, w = O.router_sqrtsoftplus(logits, bias, k, route_scale)
+        raw = np.array([O.sqrtsoftplus(float(v)) for v in logits], np.float32)
+        sel = raw + bias
+        assert list(idx) == sorted(range(e), key=lambda i: (-float(sel[i]), i))[:k]
+        # the bias picks, the raw scores weigh (moe.metal:773-785)
+        want = raw[idx].astype(np.float64)
+        want = route_scale * want / want.sum()
+        assert np.abs(w - want).max() <= 1e-6 and abs(float(w.sum()) - route_scale) <= 1e-6
+        assert np.array_equal(O.router_hash_weights(logits, idx, route_scale), w)
+
+
+def test_hash_router_weights_repeated_experts():
+    # RouterTopKParityTests.swift:81-104: a frozen row may repeat experts
+    rng = O.Rng(0x5EED0003)
+    for trial in range(12):
+        logits = _tie_logits(256, trial, rng)
+        idx = [(slot % 2) * 17 if trial % 4 == 0 else rng.next() % 256 for slot in range(6)]
+        w = O.router_hash_weights(logits, idx, 2.5)
+        s = np.array([math.sqrt(max(float(logits[i]), 0) + math.log1p(math.exp(-abs(float(logits[i])))))
+                      for i in idx])
+        assert np.abs(w - 2.5 * s / s.sum()).max() <= 2e-5
+        for a in range(6):
+            for b in range(6):
+                if idx[a] == idx[b]:
+                    assert w[a] == w[b]
+
+
+def test_inkling_router_is_sigmoid_share_with_sinks():
+    # softmax over logsigmoid(x) is sigmoid(x_i) / sum sigmoid(x_j): an independent closed form of
+    # inkling.metal:540-565 that a dropped sink, a wrong sign or a missing scale would break
+    rng = O.Rng(0x1A2B3C)
+    for trial in range(16):
+        n_routed, n_shared, k = (256, 2, 8) if trial % 2 == 0 else (100, 1, 6)
+        logits = _tie_logits(n_routed + n_shared, trial, rng)
+        bias = np.array([rng.uniform(-0.2, 0.2) for _ in range(n_routed)], np.float32)
+        if trial % 4 == 1:
+            bias[:] = 0.125
+        gs, rs = 0.75, 2.5
+        idx, w, gam = O.router_inkling(logits, bias, gs, n_routed, n_shared, k, rs)
+        sig = 1.0 / (1.0 + np.exp(-logits.astype(np.float64)))
+        sel = np.array([np.float32(1.0) / (np.float32(1.0) + np.float32(O.exp(-float(v)))) for v in logits[:n_routed]],
+                       np.float32) + bias
+        assert list(idx) == sorted(range(n_routed), key=lambda i: (-float(sel[i]), i))[:k]
+        members = list(idx) + list(range(n_routed, n_routed + n_shared))
+        want = rs * gs * sig[members] / sig[members].sum()
+        assert np.abs(np.concatenate([w, gam]) - want).max() <= 2e-6
+        assert abs(float(w.sum() + gam.sum()) - rs * gs) <= 2e-6
+
+
+def test_int8_router_rows_and_scaled_topk():
+    e, d = 24, 256
+    rng = O.Rng(0x6E44A)
+    codes = np.array([rng.next() % 256 for _ in range(e * d)], np.uint8).reshape(e, d)
+    scales = O.bf16_bits(rng.uniform_fill(0.001, 0.004, e * d // 64).reshape(e, d // 64))
+    biases = O.bf16_bits(rng.uniform_fill(-0.3, -0.1, e * d // 64).reshape(e, d // 64))
+    x = O.bf16_bits(rng.uniform_fill(-1.0, 1.0, d))
+    eff = O.bf16_bits(rng.uniform_fill(0.5, 1.5, d))
+    wf = (codes.astype(np.float64) * np.repeat(O.bf16_to_float(scales).astype(np.float64), 64, axis=1)
+          + np.repeat(O.bf16_to_float(biases).astype(np.float64), 64, axis=1))
+    ref = wf @ (O.bf16_to_float(x).astype(np.float64) * O.bf16_to_float(eff).astype(np.float64))
+    got = O.router_logits_int8(codes, scales, biases, x, eff)
+    assert np.abs(got - ref).max() <= 2e-6 * np.abs(wf).sum(axis=1).max()
+    one = np.full(d, 0x3F80, np.uint16)
+    for i in (0, 1, 63, 64, 200, 255):  # x = e_i: the dequantized weight, two roundings (Quantization.swift:104-119)
+        unit = np.zeros(d, np.uint16)
+        unit[i] = 0x3F80
+        s = O.bf16_to_float(scales[:, i // 64])
+        b = O.bf16_to_float(biases[:, i // 64])
+        assert np.array_equal(O.router_logits_int8(codes, scales, biases, unit, one),
+                              (s * codes[:, i].astype(np.float32)).astype(np.float32) + b)
+        twice = np.full(d, 0x4000, np.uint16)  # effective_scale = 2 doubles the row exactly
+        assert np.array_equal(O.router_logits_int8(codes, scales, biases, unit, twice),
+                              2 * O.router_logits_int8(codes, scales, biases, unit, one))
+    # RouterTopKParityTests.swift:30-47: per-expert scales in [0.6, 1.4] as bf16
+    r2 = O.Rng(0x5EED0001 + e)
+    for trial in range(12):
+        logits = _tie_logits(e, trial, r2)
+        scale = O.bf16_bits(np.array([r2.uniform(0.6, 1.4) for _ in range(e)], np.float32))
+        idx0, w0 = O.topk_softmax(logits, 8)
+        idx, w = O.topk_softmax_scaled(logits, scale, 8)
+        assert np.array_equal(idx, idx0)
+        assert np.array_equal(w, w0 * O.bf16_to_float(scale[idx]))
+
+
 # ------------------------------------------------------------------------ GEMV
 
 @pytest.mark.parametrize("bits", [4, 2])

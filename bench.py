@@ -331,6 +331,124 @@ def bench_dense_mlp(args, device) -> int:
     return 0
 
 
+def bench_family_routers(args, device) -> int:
+    """The four family routers at their reference shapes, T = 1 (decode) and T = 2048 (prefill): µs per
+    call from HIP-graph replays, the decode call against the HBM roofline of its router bytes, and the
+    routing of row 0 against the CPU checker bit for bit.  `sets` distinct weight sets rotate at T = 1."""
+    import numpy as np
+    import torch
+    from mference_amd import operators as ops
+    from oracle import mf_oracle as O
+
+    ctx = ops.MetalContext(0)
+    fam = ops.FamilyRouters(ctx)
+    gen = torch.Generator(device=device)
+    gen.manual_seed((ROOT_SEED + 0x600) & 0x7FFFFFFFFFFFFFFF)
+    sets = 64
+    shapes = {  # rows, shared sinks, D, K
+        "sqrtsoftplus (DeepSeek-V4)": (256, 0, 4096, 6), "hash weights (DeepSeek-V4)": (256, 0, 4096, 6),
+        "sigmoid + sinks (Inkling)": (256, 2, 2048, 8), "8-bit affine (Gemma)": (128, 0, 2816, 8)}
+    results = []
+    for name, (e, sh, d, k) in shapes.items():
+        rows = e + sh
+        int8 = name.startswith("8-bit")
+        for t in (1, 2048):
+            n_sets = sets if t == 1 else 1
+            if int8:
+                wr = torch.randint(0, 256, (n_sets, rows, d), generator=gen, device=device, dtype=torch.uint8)
+                sc = (torch.rand((n_sets, rows, d // 64), generator=gen, device=device) * 6e-4 + 2e-4).to(torch.bfloat16)
+                bi = (torch.rand((n_sets, rows, d // 64), generator=gen, device=device) * -0.04 - 0.04).to(torch.bfloat16)
+                eff = (torch.rand((d,), generator=gen, device=device) + 0.5).to(torch.bfloat16)
+                pes = (torch.rand((e,), generator=gen, device=device) * 0.8 + 0.6).to(torch.bfloat16)
+                nbytes = rows * d + 2 * 2 * rows * (d // 64)
+            else:
+                wr = (torch.randn((n_sets, rows, d), generator=gen, device=device) * 0.05).to(torch.bfloat16)
+                nbytes = rows * d * 2
+            x = torch.randn((t, d), generator=gen, device=device).to(torch.bfloat16)
+            bias = torch.rand((e,), generator=gen, device=device) * 0.6 - 0.3
+            gs = torch.full((1,), 0.75, device=device)
+            idx = torch.zeros((t, k), dtype=torch.int32, device=device)
+            given = torch.randint(0, e, (t, k), generator=gen, device=device, dtype=torch.int32)
+            wt = torch.zeros((t, k), dtype=torch.float32, device=device)
+            gam = torch.zeros((t, max(sh, 1)), dtype=torch.float32, device=device)
+            lg = torch.zeros((t, rows), dtype=torch.float32, device=device)
+
+            def call(i):
+                if int8:
+                    fam.encode_router_gemma4(wr[i], sc[i], bi[i], x, eff, pes, idx, wt, e, d, k, lg, t=t)
+                elif name.startswith("sqrt"):
+                    fam.encode_router_top_k(wr[i], x, bias, idx, wt, e, d, 1.5, lg, top_k=k, t=t)
+                elif name.startswith("hash"):
+                    fam.encode_router_hash_weights(wr[i], x, given, wt, e, d, 1.5, lg, top_k=k, t=t)
+                else:
+                    fam.encode_router_inkling(wr[i], x, bias, gs, idx, wt, gam, e, sh, k, 2.5, d, lg, t=t)
+
+            call(0)
+            torch.cuda.synchronize()
+            lg0 = lg[0].cpu().numpy()
+            if int8:
+                ref_lg = O.router_logits_int8(wr[0].cpu().numpy(), ops.bf16_bits(sc[0]), ops.bf16_bits(bi[0]),
+                                              ops.bf16_bits(x[0]), ops.bf16_bits(eff))
+                ri, rw = O.topk_softmax_scaled(ref_lg, ops.bf16_bits(pes), k)
+            else:
+                ref_lg = O.router_logits(ops.bf16_bits(wr[0]), ops.bf16_bits(x[0]))
+                if name.startswith("sqrt"):
+                    ri, rw = O.router_sqrtsoftplus(ref_lg, bias.cpu().numpy(), k, 1.5)
+                elif name.startswith("hash"):
+                    ri, rw = given[0].cpu().numpy().astype(np.uint32), O.router_hash_weights(
+                        ref_lg, given[0].cpu().numpy().astype(np.uint32), 1.5)
+                else:
+                    ri, rw, _ = O.router_inkling(ref_lg, bias.cpu().numpy(), 0.75, e, sh, k, 2.5)
+            exact = bool(np.array_equal(lg0.view(np.uint32), ref_lg.view(np.uint32))
+                         and (name.startswith("hash") or np.array_equal(idx[0].cpu().numpy().astype(np.uint32), ri))
+                         and np.array_equal(wt[0].cpu().numpy().view(np.uint32), rw.view(np.uint32)))
+            side = torch.cuda.Stream()
+            side.wait_stream(torch.cuda.current_stream())
+            with torch.cuda.stream(side):
+                for i in range(n_sets):
+                    call(i)
+            torch.cuda.current_stream().wait_stream(side)
+            torch.cuda.synchronize()
+            per_graph = n_sets if t == 1 else 10
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(graph):
+                for i in range(per_graph):
+                    call(i % n_sets)
+            reps = max(1, args.steps // 10)
+            for _ in range(max(1, args.warmup // 10)):
+                graph.replay()
+            torch.cuda.synchronize()
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            for _ in range(reps):
+                graph.replay()
+            e1.record()
+            torch.cuda.synchronize()
+            us = e0.elapsed_time(e1) / (reps * per_graph) * 1e3
+            run = {"router": name, "tokens": t, "rows": rows, "d": d, "top_k": k, "us_per_call": round(us, 2),
+                   "row0_bit_exact_vs_cpu_checker": exact}
+            if t == 1:
+                run.update(router_bytes=nbytes, gbps=round(nbytes / us / 1e3, 1),
+                           hbm_frac=round(nbytes / us / 1e3 / HBM_PEAK_GBPS, 4))
+            else:
+                run.update(tokens_per_s=round(t / us * 1e6))
+            results.append(run)
+    head = results[0]
+    print(json.dumps({
+        "metric": "us_per_router_call_T1", "value": head["us_per_call"], "unit": "us", "n_gpus": 1,
+        "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(head["us_per_call"] / 1e3, 5),
+        "higher_is_better": False, "scaling": "weak", "vs_baseline": None,
+        "dtype": "bf16 / u8 router rows x bf16 activations, fp32 accumulate and selection",
+        "data": "synthetic (N(0,0.05) router rows, N(0,1) activations)",
+        "config": {"workload": "family-routers", "launch": "hip_graph", "weight_sets_T1": sets},
+        "runs": results,
+        "roofline": {"bound": "hbm", "achieved": head["gbps"], "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+                     "frac": head["hbm_frac"], "traffic": None,
+                     "kernel": "mf::router_logits_kernel + mf::family_select_kernel (two launches per call)",
+                     "algorithmic_bytes": head["router_bytes"]}}))
+    return 0
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -338,7 +456,7 @@ def main() -> int:
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--layers", type=int, default=None)
     ap.add_argument("--workload", default="qwen-decode",
-                    choices=sorted(WORKLOADS) + ["dense-mlp"],
+                    choices=sorted(WORKLOADS) + ["dense-mlp", "family-routers"],
                     help="qwen-decode is the headline; the others measure the remaining "
                          "configurations of the same path")
     ap.add_argument("--tokens", type=int, default=None, help="token rows per step (decode: 1..8)")
@@ -366,6 +484,8 @@ def main() -> int:
     torch.cuda.set_device(device)
     if args.workload == "dense-mlp":
         return bench_dense_mlp(args, device)
+    if args.workload == "family-routers":
+        return bench_family_routers(args, device)
     w = dict(WORKLOADS[args.workload])
     if args.tokens:
         w["t"] = args.tokens

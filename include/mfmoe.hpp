@@ -134,6 +134,65 @@ class RMSNorm {
   mf_ctx* ctx_;
 };
 
+// The router calls of MoEDeepseekV4 (Kernels/MoE/MoEDeepseekV4.swift:92-151): learned top-k on
+// sqrt(softplus(logit)) + correction bias, and weighting of hash-routed experts.  routeScale is the
+// operator's constant as in the reference (:31-87); `logits` fp32 [tokens, numExperts] stands in for
+// its internal routerLogits buffer.
+class MoEDeepseekV4Router {
+ public:
+  MoEDeepseekV4Router(const MetalContext& context, float routeScale, uint32_t topK = 6)
+      : ctx_(context.raw()), routeScale_(routeScale), topK_(topK) {}
+  void encodeRouterTopK(mf_stream cb, const uint16_t* weights, const uint16_t* hidden,
+                        const float* correctionBias, uint32_t* outIndices, float* outWeights,
+                        uint32_t numExperts, uint32_t d, float* logits, uint32_t tokens = 1) const {
+    check(mf_router_sqrtsoftplus(ctx_, cb, weights, hidden, tokens, d, numExperts, d, topK_, correctionBias,
+                                 routeScale_, logits, outIndices, outWeights), ctx_);
+  }
+  void encodeRouterHashWeights(mf_stream cb, const uint16_t* weights, const uint16_t* hidden,
+                               const uint32_t* indices, float* outWeights, uint32_t numExperts, uint32_t d,
+                               float* logits, uint32_t tokens = 1) const {
+    check(mf_router_hash_weights(ctx_, cb, weights, hidden, tokens, d, numExperts, d, topK_, indices,
+                                 routeScale_, logits, outWeights), ctx_);
+  }
+
+ private:
+  mf_ctx* ctx_;
+  float routeScale_;
+  uint32_t topK_;
+};
+
+// InklingKernels.encodeRouter / encodeRouterPrefill (Kernels/Inkling/InklingKernels.swift:377-476)
+class InklingRouter {
+ public:
+  explicit InklingRouter(const MetalContext& context) : ctx_(context.raw()) {}
+  void encodeRouter(mf_stream cb, const uint16_t* weights, const uint16_t* hidden, const float* gateBias,
+                    const float* globalScale, uint32_t* outIndices, float* outWeights, float* gammasOut,
+                    uint32_t numRouted, uint32_t numShared, uint32_t topK, float routeScale, uint32_t d,
+                    float* logits, uint32_t tokens = 1) const {
+    check(mf_router_inkling(ctx_, cb, weights, hidden, tokens, d, numRouted, numShared, d, topK, gateBias,
+                            globalScale, routeScale, logits, outIndices, outWeights, gammasOut), ctx_);
+  }
+
+ private:
+  mf_ctx* ctx_;
+};
+
+// MoE.encodeRouterGemma4 (Kernels/MoE/MoE.swift:153-202): 8-bit affine router rows
+class Gemma4Router {
+ public:
+  explicit Gemma4Router(const MetalContext& context) : ctx_(context.raw()) {}
+  void encodeRouterGemma4(mf_stream cb, const uint8_t* weights, const uint16_t* scales, const uint16_t* biases,
+                          const uint16_t* hidden, const uint16_t* effectiveScale, const uint16_t* perExpertScale,
+                          uint32_t* outIndices, float* outWeights, uint32_t numExperts, uint32_t d, uint32_t topK,
+                          float* logits, uint32_t tokens = 1) const {
+    check(mf_router_gemma4(ctx_, cb, weights, scales, biases, hidden, tokens, d, effectiveScale, perExpertScale,
+                           numExperts, d, topK, logits, outIndices, outWeights), ctx_);
+  }
+
+ private:
+  mf_ctx* ctx_;
+};
+
 // SharedExpertInt4 (Kernels/MoE/SharedExpertInt4.swift:70-165), also the dense SwiGLU MLP.
 // Errors: MF_ERR_DIMENSION_MISMATCH / MF_ERR_SCRATCH_TOO_SMALL / MF_ERR_UNSUPPORTED_BITS are
 // SharedExpertError.dimensionMismatch / .scratchTooSmall / .unsupportedWeightBits (:4-19).

@@ -298,6 +298,15 @@ mf_status family_args_ok(const mf_ctx* ctx, const void* w, const uint16_t* x, ui
   if (!mf::aligned2(x) || (reinterpret_cast<uintptr_t>(logits) & 3u)) return MF_ERR_INVALID_ARGUMENT;
   return MF_OK;
 }
+// bf16 router rows for t tokens: the batched kernels of the prefill router from 16 tokens on (the same
+// bits: they keep the summation order of the one-row kernel), else one wave per (token, row)
+hipError_t family_logits(hipStream_t s, const uint16_t* w, const uint16_t* x, uint32_t rows, uint32_t d,
+                         uint32_t t, uint32_t x_stride, float* logits) {
+  const bool al = mf::aligned16(w) && mf::aligned16(x) && x_stride % 8 == 0;
+  if (t >= 16 && al && ((d % 512 == 0 && rows % 32 == 0) || d <= 4096))
+    return mf::launch_prefill_router(s, w, x, rows, d, t, x_stride, logits);
+  return mf::launch_router_logits(s, w, x, rows, d, t, x_stride, logits, nullptr);
+}
 }  // namespace
 
 mf_status mf_router_sqrtsoftplus(mf_ctx* ctx, mf_stream stream, const uint16_t* router_w, const uint16_t* x,
@@ -308,7 +317,7 @@ mf_status mf_router_sqrtsoftplus(mf_ctx* ctx, mf_stream stream, const uint16_t* 
   if (st != MF_OK) return st;
   if (!correction_bias || !out_idx || !out_w || !mf::aligned2(router_w)) return MF_ERR_INVALID_ARGUMENT;
   auto s = static_cast<hipStream_t>(stream);
-  MF_HIP(ctx, mf::launch_router_logits(s, router_w, x, num_experts, d, t, x_stride, logits, nullptr));
+  MF_HIP(ctx, family_logits(s, router_w, x, num_experts, d, t, x_stride, logits));
   MF_HIP(ctx, mf::launch_select_sqrtsoftplus(s, logits, correction_bias, num_experts, top_k, t, route_scale,
                                              out_idx, out_w));
   return MF_OK;
@@ -322,7 +331,7 @@ mf_status mf_router_hash_weights(mf_ctx* ctx, mf_stream stream, const uint16_t* 
   if (st != MF_OK) return st;
   if (!indices || !out_w || !mf::aligned2(router_w)) return MF_ERR_INVALID_ARGUMENT;
   auto s = static_cast<hipStream_t>(stream);
-  MF_HIP(ctx, mf::launch_router_logits(s, router_w, x, num_experts, d, t, x_stride, logits, nullptr));
+  MF_HIP(ctx, family_logits(s, router_w, x, num_experts, d, t, x_stride, logits));
   MF_HIP(ctx, mf::launch_hash_weights(s, logits, indices, num_experts, top_k, t, route_scale, out_w));
   return MF_OK;
 }
@@ -339,7 +348,7 @@ mf_status mf_router_inkling(mf_ctx* ctx, mf_stream stream, const uint16_t* route
       !mf::aligned2(router_w))
     return MF_ERR_INVALID_ARGUMENT;
   auto s = static_cast<hipStream_t>(stream);
-  MF_HIP(ctx, mf::launch_router_logits(s, router_w, x, n_routed + n_shared, d, t, x_stride, logits, nullptr));
+  MF_HIP(ctx, family_logits(s, router_w, x, n_routed + n_shared, d, t, x_stride, logits));
   MF_HIP(ctx, mf::launch_select_inkling(s, logits, gate_bias, global_scale, n_routed, n_shared, top_k, t,
                                         route_scale, out_idx, out_w, out_gammas));
   return MF_OK;

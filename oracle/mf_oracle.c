@@ -43,6 +43,25 @@
  *   mfo_topk_full_softmax         maple_moe.metal:62-119; checked on the
  *                                 reference's tied-score fixture
  *                                 (MapleMoETests.swift:24-40) and sentinels.
+ *   mfo_log_1to2,                 this build's own deterministic log on [1,2] (shared
+ *   mfo_sqrtsoftplus              bit for bit with the HIP kernels) and moe.metal:736-740;
+ *                                 checked against libm (1.2e-7), sqrt(ln 2) at 0, exactly
+ *                                 sqrt(x) / 0 beyond |x| = 20, fp64 on [-4, 12].
+ *   mfo_router_sqrtsoftplus,      moe.metal:744-786, :847-866; selection checked against
+ *   mfo_router_hash_weights       sort-by-(score desc, index asc) on the reference's
+ *                                 tie-heavy logits and duplicated biases
+ *                                 (RouterTopKParityTests.swift:52-104), weights against
+ *                                 fp64 and sum = route_scale; repeated experts.
+ *   mfo_router_inkling            inkling.metal:503-566; selection as above, weights against
+ *                                 the closed form sigmoid(x_i) / sum sigmoid(x_j) over the
+ *                                 picked experts and the sinks, sum = route * global scale.
+ *                                 A NaN logit is undefined behaviour in the reference
+ *                                 (writes past top_score); here it is never picked.
+ *   mfo_router_logits_int8,       moe.metal:102-139 with this build's summation order;
+ *   mfo_topk_softmax_scaled       checked against fp64, x = e_i (the two-rounding
+ *                                 dequantized weight), effective_scale = 2; the scaled
+ *                                 top-k on the reference's per-expert-scale draw
+ *                                 (RouterTopKParityTests.swift:30-47).
  *   mfo_gemv / mfo_gemv_multix    DequantInt4Gemv.swift:26-40; checked by
  *                                 x=e_i, x=1, linearity, fp64 brute force.
  *   mfo_expert_*, mfo_shared_*    Moe.swift:58-88 with the rounding points of

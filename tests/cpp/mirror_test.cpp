@@ -1,7 +1,8 @@
 // Drives libmfmoe through the C++ mirror of the reference's operator classes
 // (include/mfmoe.hpp) and checks the results against the CPU checker, the way the reference's
 // own XCTest cases drive its Swift operators: SeedTree-seeded inputs, one small layer,
-// decode == per-token checker, ragged prefill == per-token checker, grouping KATs and errors.
+// decode == per-token checker, ragged prefill == per-token checker, family routers bit for bit,
+// grouping KATs and errors.
 //
 //   mirror_test cpu   grouping KATs and error cases only (no GPU needed)
 //   mirror_test gpu   everything
@@ -263,10 +264,81 @@ static void test_layer() {
   EXPECT(thrown, "scratchTooSmall not thrown");
 }
 
+// ---------------------------------------------------------------- family routers (GPU)
+// The DeepSeek-V4 selector and the Inkling router through the mirror classes, bit for bit against
+// the checker on seeded inputs.
+static void test_family_routers(const mf::MetalContext& ctx) {
+  const uint32_t e = 64, shared = 2, d = 256, t = 3, k = 6;
+  mfo_rng rng = mfo_seed_tree_key(0x4D464D4F0000FA40ull, "family");
+  std::vector<float> wf((e + shared) * d), xf(t * d), bias(e);
+  mfo_rng_normal(&rng, 0.0f, 0.05f, wf.data(), wf.size());
+  mfo_rng_normal(&rng, 0.0f, 1.0f, xf.data(), xf.size());
+  mfo_rng_uniform_fill(&rng, -0.3f, 0.3f, bias.data(), bias.size());
+  std::vector<uint16_t> w(wf.size()), x(xf.size());
+  mfo_bf16_encode(wf.data(), wf.size(), w.data());
+  mfo_bf16_encode(xf.data(), xf.size(), x.data());
+  const std::vector<float> gs = {0.75f};
+  uint16_t* dw = to_device(w);
+  uint16_t* dx = to_device(x);
+  float* dbias = to_device(bias);
+  float* dgs = to_device(gs);
+  uint32_t* didx = to_device(std::vector<uint32_t>(t * 8));
+  float* dwt = to_device(std::vector<float>(t * 8));
+  float* dgam = to_device(std::vector<float>(t * shared));
+  float* dlg = to_device(std::vector<float>(t * (e + shared)));
+
+  mf::MoEDeepseekV4Router v4(ctx, 1.5f, k);
+  v4.encodeRouterTopK(nullptr, dw, dx, dbias, didx, dwt, e, d, dlg, t);
+  HIP_OK(hipDeviceSynchronize());
+  auto idx = to_host(didx, t * k);
+  auto wt = to_host(dwt, t * k);
+  for (uint32_t i = 0; i < t; ++i) {
+    std::vector<float> lg(e);
+    mfo_router_logits_bf16(w.data(), x.data() + i * d, e, d, lg.data());
+    uint32_t ri[8];
+    float rw[8];
+    mfo_router_sqrtsoftplus(lg.data(), bias.data(), e, k, 1.5f, ri, rw);
+    EXPECT(!std::memcmp(ri, idx.data() + i * k, k * 4) && !std::memcmp(rw, wt.data() + i * k, k * 4),
+           "sqrtsoftplus router row %u", i);
+  }
+  v4.encodeRouterHashWeights(nullptr, dw, dx, didx, dwt, e, d, dlg, t);
+  HIP_OK(hipDeviceSynchronize());
+  EXPECT(to_host(dwt, t * k) == wt, "hash weights of the selected experts");
+
+  mf::InklingRouter ink(ctx);
+  ink.encodeRouter(nullptr, dw, dx, dbias, dgs, didx, dwt, dgam, e, shared, 8, 2.5f, d, dlg, t);
+  HIP_OK(hipDeviceSynchronize());
+  idx = to_host(didx, t * 8);
+  wt = to_host(dwt, t * 8);
+  auto gam = to_host(dgam, t * shared);
+  for (uint32_t i = 0; i < t; ++i) {
+    std::vector<float> lg(e + shared);
+    mfo_router_logits_bf16(w.data(), x.data() + i * d, e + shared, d, lg.data());
+    uint32_t ri[8];
+    float rw[8], rg[8];
+    mfo_router_inkling(lg.data(), bias.data(), 0.75f, e, shared, 8, 2.5f, ri, rw, rg);
+    EXPECT(!std::memcmp(ri, idx.data() + i * 8, 32) && !std::memcmp(rw, wt.data() + i * 8, 32) &&
+               !std::memcmp(rg, gam.data() + i * shared, shared * 4), "inkling router row %u", i);
+  }
+  bool threw = false;
+  try {
+    mf::MoEDeepseekV4Router(ctx, 1.0f, 9).encodeRouterTopK(nullptr, dw, dx, dbias, didx, dwt, e, d, dlg, t);
+  } catch (const mf::Error& err) {
+    threw = err.status == MF_ERR_TOPK;
+  }
+  EXPECT(threw, "top-k above the maximum is MF_ERR_TOPK");
+  for (void* p : {(void*)dw, (void*)dx, (void*)dbias, (void*)dgs, (void*)didx, (void*)dwt, (void*)dgam, (void*)dlg})
+    HIP_OK(hipFree(p));
+}
+
 int main(int argc, char** argv) {
   const std::string mode = argc > 1 ? argv[1] : "cpu";
   test_grouping();
-  if (mode == "gpu") test_layer();
+  if (mode == "gpu") {
+    test_layer();
+    mf::MetalContext context(0);
+    test_family_routers(context);
+  }
   std::printf(g_fail ? "mirror_test: %d FAILED\n" : "mirror_test: ok\n", g_fail);
   return g_fail ? 1 : 0;
 }

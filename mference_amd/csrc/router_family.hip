@@ -6,6 +6,8 @@
 #include "mf_internal.h"
 #include "mf_router.h"
 
+#include <algorithm>
+
 #pragma clang fp contract(off)
 
 namespace mf {
@@ -63,6 +65,79 @@ __global__ __launch_bounds__(256) void router_logits_int8_kernel(
   }
   acc = wave_sum(acc);
   if (lane == 0) logits[static_cast<size_t>(tok) * e + row] = acc;
+}
+
+// The same rows for many tokens, bit-exact with the kernel above: a wave keeps R expert rows in
+// registers (lane l holds the chunks l, l+64, ... of each row as floats, with their group's scale and
+// bias) together with effective_scale, and streams token rows past them; sum x' of a chunk is the
+// same for every row and is built once per token.  Needs 16-byte aligned x and effective_scale, 8-byte
+// aligned code rows.
+template <int CPL, int R>
+__global__ __launch_bounds__(256) void router_logits_int8_tiled_kernel(
+    const uint8_t* __restrict__ codes, const uint16_t* __restrict__ scales,
+    const uint16_t* __restrict__ biases, const uint16_t* __restrict__ x,
+    const uint16_t* __restrict__ eff, uint32_t e, uint32_t d, uint32_t t, uint32_t x_stride,
+    float* __restrict__ logits, uint32_t tokens_per_block) {
+  const uint32_t lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
+  const uint32_t row0 = (blockIdx.x * 4 + wv) * R;
+  if (row0 >= e) return;
+  const uint32_t chunks = d / 8, groups = d / MF_GROUP_SIZE;
+  float qf[R][CPL][8], sf[R][CPL], bf[R][CPL], ef[CPL][8];
+#pragma unroll
+  for (int c = 0; c < CPL; ++c) {
+    const uint32_t ci = lane + 64 * c;
+    uint4 v = make_uint4(0, 0, 0, 0);
+    if (ci < chunks) v = load_x8<true>(eff + ci * 8);
+    ef[c][0] = bf16_lo(v.x); ef[c][1] = bf16_hi(v.x); ef[c][2] = bf16_lo(v.y); ef[c][3] = bf16_hi(v.y);
+    ef[c][4] = bf16_lo(v.z); ef[c][5] = bf16_hi(v.z); ef[c][6] = bf16_lo(v.w); ef[c][7] = bf16_hi(v.w);
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+      const bool live = ci < chunks && row0 + r < e;
+      uint2 q = make_uint2(0, 0);
+      if (live) q = *reinterpret_cast<const uint2*>(codes + static_cast<size_t>(row0 + r) * d + ci * 8);
+#pragma unroll
+      for (int j = 0; j < 8; ++j) qf[r][c][j] = static_cast<float>(((j < 4 ? q.x : q.y) >> (8 * (j & 3))) & 0xFFu);
+      const size_t g = static_cast<size_t>(row0 + r) * groups + ci * 8 / MF_GROUP_SIZE;
+      sf[r][c] = live ? bf16_to_f(scales[g]) : 0.0f;
+      bf[r][c] = live ? bf16_to_f(biases[g]) : 0.0f;
+    }
+  }
+  const uint32_t t0 = blockIdx.y * tokens_per_block;
+  const uint32_t t1 = min(t, t0 + tokens_per_block);
+  for (uint32_t tok = t0; tok < t1; ++tok) {
+    const uint16_t* xt = x + static_cast<size_t>(tok) * x_stride;
+    float xs[CPL][8], sum[CPL];
+#pragma unroll
+    for (int c = 0; c < CPL; ++c) {
+      const uint32_t ci = lane + 64 * c;
+      uint4 v = make_uint4(0, 0, 0, 0);
+      if (ci < chunks) v = load_x8<true>(xt + ci * 8);
+      const float xv[8] = {bf16_lo(v.x), bf16_hi(v.x), bf16_lo(v.y), bf16_hi(v.y),
+                           bf16_lo(v.z), bf16_hi(v.z), bf16_lo(v.w), bf16_hi(v.w)};
+      sum[c] = 0.0f;
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        xs[c][j] = xv[j] * ef[c][j];
+        sum[c] = sum[c] + xs[c][j];
+      }
+    }
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+      float acc = 0.0f;
+#pragma unroll
+      for (int c = 0; c < CPL; ++c) {
+        if (lane + 64 * c < chunks) {
+          float dot = 0.0f;
+#pragma unroll
+          for (int j = 0; j < 8; ++j) dot = __builtin_fmaf(qf[r][c][j], xs[c][j], dot);
+          acc = __builtin_fmaf(sf[r][c], dot, acc);
+          acc = __builtin_fmaf(bf[r][c], sum[c], acc);
+        }
+      }
+      acc = wave_sum(acc);
+      if (lane == 0 && row0 + r < e) logits[static_cast<size_t>(tok) * e + row0 + r] = acc;
+    }
+  }
 }
 
 enum Family { kSqrtSoftplus = 0, kHash = 1, kInkling = 2, kScaledSoftmax = 3 };
@@ -174,6 +249,19 @@ hipError_t launch_router_logits_int8(hipStream_t s, const uint8_t* codes, const 
   if (!waves) return hipSuccess;
   const int al = (reinterpret_cast<uintptr_t>(codes) % 8 == 0) && aligned16(x) && aligned16(eff) &&
                  x_stride % 8 == 0 && d % 8 == 0;
+  const uint32_t cpl = (d / 8 + 63) / 64;
+  if (al && t >= 16 && cpl <= 8) {  // many tokens: rows stay in registers
+    const uint32_t tpb = std::max(1u, std::min(64u, t / 64));
+#define MF_R8(CPL, R)                                                                                \
+  router_logits_int8_tiled_kernel<CPL, R><<<dim3((e + 4 * R - 1) / (4 * R), (t + tpb - 1) / tpb), dim3(256), 0, \
+                                            s>>>(codes, scales, biases, x, eff, e, d, t, x_stride, logits, tpb)
+    if (cpl <= 2) MF_R8(2, 4);
+    else if (cpl <= 4) MF_R8(4, 2);
+    else if (cpl <= 6) MF_R8(6, 2);
+    else MF_R8(8, 1);
+#undef MF_R8
+    return hipGetLastError();
+  }
   router_logits_int8_kernel<<<dim3((waves + 3) / 4), dim3(256), 0, s>>>(codes, scales, biases, x, eff, e, d, t,
                                                                        x_stride, logits, al);
   return hipGetLastError();

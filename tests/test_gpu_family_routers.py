@@ -195,7 +195,8 @@ def test_inkling_ties(gpu, oracle):
 
 
 @pytest.mark.parametrize("e,d,k,t,shift", [(128, 2816, 8, 1, 0), (128, 2816, 8, 3, 0), (24, 256, 8, 2, 0),
-                                           (128, 2816, 8, 2, 1), (256, 1024, 4, 150, 0)])
+                                           (128, 2816, 8, 2, 1), (256, 1024, 4, 150, 0), (128, 2816, 8, 40, 0),
+                                           (66, 4096, 8, 33, 0), (24, 256, 8, 20, 0), (128, 2816, 8, 20, 1)])
 def test_gemma4_router_bit_exact(gpu, oracle, e, d, k, t, shift):
     """8-bit affine router rows; shift = 1 hands over pointers that are only 1- / 2-byte aligned"""
     rng = oracle.Rng.key(ROOT_SEED + 0xFA32, f"gemma4-{e}-{d}-{k}-{t}")

@@ -270,6 +270,19 @@ mf_status mf_moe_phase1(mf_moe* h, mf_stream stream, const void* expert_base,
                         const uint32_t* idx, const uint16_t* x, uint32_t t, uint32_t x_stride,
                         uint16_t* acts);
 
+/* The same for a subset of the routed slots: MoE.encodeRoutedPersistentPhase1SubsetU16Load
+ * (MoE.swift:255-298), MoEDeepseekV4.encodeRoutedPhase1Subset (MoEDeepseekV4.swift:223-263),
+ * moe_phase1_gate_up_act_subset_u16load (moe.metal:531-565) -- the reference splits phase 1
+ * into cache hits and misses; with every expert resident nothing needs the split, but its
+ * invariant holds: the subsets together write the same bits as the full call.
+ * active_slots: device uint32 [active_count], entries token*top_k + slot; an entry past
+ * t*top_k does nothing (moe.metal:551); active_count == 0 launches nothing. */
+mf_status mf_moe_phase1_subset(mf_moe* h, mf_stream stream, const void* expert_base,
+                               size_t expert_stride, const mf_expert_offsets* offsets,
+                               const uint32_t* idx, const uint16_t* x, uint32_t t,
+                               uint32_t x_stride, uint16_t* acts, const uint32_t* active_slots,
+                               uint32_t active_count);
+
 /* Routed phase 2: y[t,d] = bf16(residual[t,d] + sum_k w[t,k] * (down_k . acts[t,k]))
  * in rank order.  MoE.encodeRoutedPersistentPhase2Reduce (MoE.swift:400-440),
  * MoEDeepseekV4.encodeRoutedPhase2Reduce (MoEDeepseekV4.swift:265-274).

@@ -249,6 +249,14 @@ class MoE {
     check(mf_moe_phase1(h_, cb, experts, expertStride, &routedOffsets, indices, x, tokens, cfg_.d, acts),
           ctx_);
   }
+  // encodeRoutedPersistentPhase1SubsetU16Load (MoE.swift:255-298): only the listed slots
+  void encodeRoutedPersistentPhase1SubsetU16Load(mf_stream cb, const void* experts, size_t expertStride,
+                                                 const MoEExpertOffsets& routedOffsets, const uint32_t* indices,
+                                                 const uint16_t* x, uint16_t* acts, const uint32_t* activeSlots,
+                                                 uint32_t activeCount, uint32_t tokens = 1) const {
+    check(mf_moe_phase1_subset(h_, cb, experts, expertStride, &routedOffsets, indices, x, tokens, cfg_.d, acts,
+                               activeSlots, activeCount), ctx_);
+  }
   // encodeRoutedPersistentPhase2Reduce (MoE.swift:400-440)
   void encodeRoutedPersistentPhase2Reduce(mf_stream cb, const void* experts, size_t expertStride,
                                           const MoEExpertOffsets& routedOffsets, const uint32_t* indices,

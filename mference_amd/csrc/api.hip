@@ -389,6 +389,22 @@ mf_status mf_moe_phase1(mf_moe* h, mf_stream stream, const void* expert_base,
   return MF_OK;
 }
 
+mf_status mf_moe_phase1_subset(mf_moe* h, mf_stream stream, const void* expert_base,
+                               size_t expert_stride, const mf_expert_offsets* offsets,
+                               const uint32_t* idx, const uint16_t* x, uint32_t t, uint32_t x_stride,
+                               uint16_t* acts, const uint32_t* active_slots, uint32_t active_count) {
+  if (active_count == 0) return MF_OK;  // MoE.swift:269
+  if (!active_slots || (reinterpret_cast<uintptr_t>(active_slots) & 3u)) return MF_ERR_INVALID_ARGUMENT;
+  if (!h || !expert_base || !offsets || !idx || !x || !acts) return MF_ERR_INVALID_ARGUMENT;
+  if (t == 0 || x_stride < h->cfg.d) return MF_ERR_INVALID_ARGUMENT;
+  if (!offsets_ok(*offsets, h->cfg.bits) || !mf::aligned2(expert_base) || (expert_stride & 1) ||
+      !mf::aligned2(x) || !mf::aligned2(acts))
+    return MF_ERR_INVALID_ARGUMENT;
+  MF_HIP(h->ctx, mf::launch_phase1(static_cast<hipStream_t>(stream), h->cfg, expert_base, expert_stride,
+                                   *offsets, idx, x, t, x_stride, acts, active_slots, active_count));
+  return MF_OK;
+}
+
 mf_status mf_moe_phase2(mf_moe* h, mf_stream stream, const void* expert_base,
                         size_t expert_stride, const mf_expert_offsets* offsets,
                         const uint32_t* idx, const float* w, const uint16_t* acts,

@@ -105,7 +105,8 @@ hipError_t launch_select_scaled_softmax(hipStream_t s, const float* logits, cons
 // moe_decode.hip
 hipError_t launch_phase1(hipStream_t s, const mf_moe_config& cfg, const void* base, size_t stride,
                          const mf_expert_offsets& off, const uint32_t* idx, const uint16_t* x,
-                         uint32_t t, uint32_t x_stride, uint16_t* acts);
+                         uint32_t t, uint32_t x_stride, uint16_t* acts, const uint32_t* subset = nullptr,
+                         uint32_t n_subset = 0);
 hipError_t launch_phase2(hipStream_t s, const mf_moe_config& cfg, const void* base, size_t stride,
                          const mf_expert_offsets& off, const uint32_t* idx, const float* w,
                          const uint16_t* acts, const uint16_t* residual, uint32_t t, uint16_t* y);

@@ -41,15 +41,21 @@ __global__ __launch_bounds__(256) void phase1_kernel(const uint8_t* __restrict__
                                                      uint16_t* __restrict__ acts, uint32_t D,
                                                      uint32_t F, uint32_t E, uint32_t pairs,
                                                      uint32_t K, float limit, int maple,
-                                                     uint32_t lpr_log2) {
+                                                     uint32_t lpr_log2,
+                                                     const uint32_t* __restrict__ subset,
+                                                     uint32_t all_pairs) {
   constexpr int EPL = Fmt<BITS>::kElemsPer16B;
   const uint32_t lane = threadIdx.x & 63;
   const uint32_t wave = (blockIdx.x * blockDim.x + threadIdx.x) >> 6;
   const uint32_t lpr = 1u << lpr_log2;
   const uint32_t rpw = 64u >> lpr_log2;
   const uint32_t waves_per_pair = (F + rpw - 1) / rpw;
-  const uint32_t pair = wave / waves_per_pair;
+  uint32_t pair = wave / waves_per_pair;
   if (pair >= pairs) return;
+  if (subset) {  // moe_phase1_gate_up_act_subset_u16load (moe.metal:531-565): only the listed slots
+    pair = subset[pair];
+    if (pair >= all_pairs) return;  // a slot past the table does nothing (:551)
+  }
   const uint32_t row = (wave % waves_per_pair) * rpw + (lane >> lpr_log2);
   const uint32_t sub = lane & (lpr - 1);
   const bool row_ok = row < F;
@@ -148,8 +154,10 @@ bool blob_aligned(const void* base, size_t stride, const mf_expert_offsets& o) {
 
 hipError_t launch_phase1(hipStream_t s, const mf_moe_config& cfg, const void* base, size_t stride,
                          const mf_expert_offsets& off, const uint32_t* idx, const uint16_t* x,
-                         uint32_t t, uint32_t x_stride, uint16_t* acts) {
-  const uint32_t pairs = t * cfg.top_k;
+                         uint32_t t, uint32_t x_stride, uint16_t* acts, const uint32_t* subset,
+                         uint32_t n_subset) {
+  const uint32_t all_pairs = t * cfg.top_k;
+  const uint32_t pairs = subset ? n_subset : all_pairs;
   if (!pairs) return hipSuccess;
   const bool al = blob_aligned(base, stride, off) && aligned16(x) && (x_stride % 8 == 0);
   const auto* b = static_cast<const uint8_t*>(base);
@@ -160,7 +168,7 @@ hipError_t launch_phase1(hipStream_t s, const mf_moe_config& cfg, const void* ba
     const uint32_t waves = pairs * ((cfg.f + rpw - 1) / rpw);                                    \
     phase1_kernel<BITS, AL><<<dim3((waves + 3) / 4), dim3(256), 0, s>>>(                         \
         b, stride, off, idx, x, x_stride, acts, cfg.d, cfg.f, cfg.num_experts, pairs, cfg.top_k, \
-        cfg.swiglu_limit, static_cast<int>(cfg.maple_rounding), lpr_log2);                       \
+        cfg.swiglu_limit, static_cast<int>(cfg.maple_rounding), lpr_log2, subset, all_pairs);    \
   }
   switch (cfg.bits) {
     case MF_BITS_4: if (al) MF_P1(kBits4, true) else MF_P1(kBits4, false) break;

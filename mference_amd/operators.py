@@ -335,6 +335,16 @@ class MoE:
                                         self.cfg.d if x_stride is None else x_stride, _ptr(acts)),
               self.context.handle)
 
+    def encode_routed_phase1_subset(self, experts: torch.Tensor, offsets: ExpertOffsets, indices, x, acts,
+                                    active_slots, active_count: int, t: int = 1,
+                                    x_stride: Optional[int] = None, stream=None):
+        """encodeRoutedPersistentPhase1SubsetU16Load (MoE.swift:255-298): only the listed slots."""
+        check(_capi.lib().mf_moe_phase1_subset(self._h, _stream(stream), _ptr(experts), experts.stride(0),
+                                               C.byref(offsets), _ptr(indices), _ptr(x), t,
+                                               self.cfg.d if x_stride is None else x_stride, _ptr(acts),
+                                               _ptr(active_slots), active_count),
+              self.context.handle)
+
     def encode_routed_phase2_reduce(self, experts: torch.Tensor, offsets: ExpertOffsets, indices,
                                     routing_weights, acts, residual, y, t: int = 1, stream=None):
         """encodeRoutedPersistentPhase2Reduce (MoE.swift:400-440)."""

@@ -338,6 +338,45 @@ def test_two_phase_matches_oracle_and_fused(gpu, oracle):
     assert_layer_close(oracle.bf16_to_float(ops.bf16_bits(y)), oracle.bf16_to_float(ref_y), "two-phase")
 
 
+@pytest.mark.parametrize("bits,t", [(4, 1), (2, 3), (1, 2)])
+def test_phase1_subsets_write_the_bits_of_the_full_call(gpu, oracle, bits, t):
+    """MoEFusedFFNTests.swift:126-186: phase 1 split into slot subsets (the reference's cache hits and
+    misses) followed by phase 2 gives the output of the full call bit for bit"""
+    d, f, e, k = 256, 128, 16, 8
+    root = ROOT_SEED + 0x2D4 + bits
+    layer = oracle.synth_layer(root, d, f, e, k, bits=bits, fs=0)
+    x = oracle.synth_x(root, t, d)
+    _, ref_idx, ref_w = oracle.moe_layer(layer, x)
+    moe = make_moe(gpu, layer)
+    wts = to_device_layer(layer)
+    xd = ops.bf16_tensor(x)
+    idx = torch.from_numpy(ref_idx.astype(np.int32)).cuda()
+    w = torch.from_numpy(ref_w).cuda()
+    full = torch.zeros((t, k, f), dtype=torch.bfloat16, device="cuda")
+    split = torch.full((t, k, f), 7.0, dtype=torch.bfloat16, device="cuda")
+    moe.encode_routed_phase1(wts.experts, wts.offsets, idx, xd, full, t=t)
+    slots = np.arange(t * k, dtype=np.int32)
+    parts = [slots[slots % 3 == 0], slots[slots % 3 == 1], np.concatenate([slots[slots % 3 == 2], [t * k + 5]])]
+    for part in parts:  # the last list also names a slot past the table, which must do nothing
+        moe.encode_routed_phase1_subset(wts.experts, wts.offsets, idx, xd, split,
+                                        torch.from_numpy(part.astype(np.int32)).cuda(), len(part), t=t)
+    moe.encode_routed_phase1_subset(wts.experts, wts.offsets, idx, xd, split, None, 0, t=t)  # no slots: no launch
+    y_full = torch.zeros((t, d), dtype=torch.bfloat16, device="cuda")
+    y_split = torch.zeros_like(y_full)
+    moe.encode_routed_phase2_reduce(wts.experts, wts.offsets, idx, w, full, None, y_full, t=t)
+    moe.encode_routed_phase2_reduce(wts.experts, wts.offsets, idx, w, split, None, y_split, t=t)
+    _sync()
+    assert torch.equal(full.view(torch.int16), split.view(torch.int16))
+    assert torch.equal(y_full.view(torch.int16), y_split.view(torch.int16))
+    # one subset alone leaves the other slots untouched
+    lone = torch.full((t, k, f), 7.0, dtype=torch.bfloat16, device="cuda")
+    moe.encode_routed_phase1_subset(wts.experts, wts.offsets, idx, xd, lone,
+                                    torch.tensor([1], dtype=torch.int32, device="cuda"), 1, t=t)
+    _sync()
+    assert torch.equal(lone[0, 1].view(torch.int16), full[0, 1].view(torch.int16))
+    assert bool((lone[0, 0] == 7.0).all()) and bool((lone[0, 2:] == 7.0).all())
+
+
 def test_qwen_shape_specialised_launch(gpu, oracle):
     """the full Qwen3.6-shaped layer (D 2048, F 512, E 256, K 8, shared 512) takes the
     shape-specialised fused kernel; weights drawn and quantized on the GPU as bench.py does"""

@@ -415,6 +415,49 @@ __global__ __launch_bounds__(256) void prep_rows_kernel(const PrepArgs a) {
   if ((c & 7) == 0) sums[c >> 3] = sum;
 }
 
+// The same for the layer's input rows and, in the same pass, the scalar shared gate's logit
+// w_sg . x of every row (prefill_qwen_shared_scalar_gate, prefill.metal:42-80) in the router's lane
+// order (dot_bf16_row: lane l takes the chunks l, l+64, ... of a row, neighbour-first butterfly), so
+// the gate has the bits of the stand-alone router-row launch it replaces.  One wave per row.
+__global__ __launch_bounds__(256) void prep_x_gate_kernel(const uint16_t* __restrict__ x,
+                                                          uint16_t* __restrict__ xp, float* __restrict__ sums,
+                                                          const uint16_t* __restrict__ w_sg,
+                                                          uint16_t* __restrict__ gate, uint32_t t, uint32_t d) {
+  const uint32_t lane = threadIdx.x & 63, row = blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (row >= t) return;
+  const uint32_t chunks = d / 8;  // a multiple of 8: the 8 lanes of a K group are live together
+  const size_t base = static_cast<size_t>(row) * chunks;
+  float acc = 0.0f;
+  for (uint32_t c0 = 0; c0 < chunks; c0 += kWave) {
+    const uint32_t c = c0 + lane;
+    const bool live = c < chunks;
+    uint4 v = make_uint4(0, 0, 0, 0), wv = make_uint4(0, 0, 0, 0);
+    if (live) {
+      v = *reinterpret_cast<const uint4*>(x + (base + c) * 8);
+      wv = *reinterpret_cast<const uint4*>(w_sg + static_cast<size_t>(c) * 8);
+    }
+    float sum = ((bf16_lo(v.x) + bf16_hi(v.x)) + (bf16_lo(v.y) + bf16_hi(v.y))) +
+                ((bf16_lo(v.z) + bf16_hi(v.z)) + (bf16_lo(v.w) + bf16_hi(v.w)));
+    sum = group_sum(sum, 8);
+    if (live) {
+      *reinterpret_cast<uint4*>(xp + (base + c) * 8) =
+          make_uint4(__builtin_amdgcn_perm(v.z, v.x, 0x05040100u), __builtin_amdgcn_perm(v.z, v.x, 0x07060302u),
+                     __builtin_amdgcn_perm(v.w, v.y, 0x05040100u), __builtin_amdgcn_perm(v.w, v.y, 0x07060302u));
+      if ((c & 7) == 0) sums[(base + c) >> 3] = sum;
+      acc = __builtin_fmaf(bf16_lo(wv.x), bf16_lo(v.x), acc);
+      acc = __builtin_fmaf(bf16_hi(wv.x), bf16_hi(v.x), acc);
+      acc = __builtin_fmaf(bf16_lo(wv.y), bf16_lo(v.y), acc);
+      acc = __builtin_fmaf(bf16_hi(wv.y), bf16_hi(v.y), acc);
+      acc = __builtin_fmaf(bf16_lo(wv.z), bf16_lo(v.z), acc);
+      acc = __builtin_fmaf(bf16_hi(wv.z), bf16_hi(v.z), acc);
+      acc = __builtin_fmaf(bf16_lo(wv.w), bf16_lo(v.w), acc);
+      acc = __builtin_fmaf(bf16_hi(wv.w), bf16_hi(v.w), acc);
+    }
+  }
+  acc = wave_sum(acc);
+  if (lane == 0) gate[row] = f_to_bf16(acc);
+}
+
 struct QmmArgs {
   // weights: routed = blobs of the expert pool, dense = one projection set
   const uint8_t* expert_base;
@@ -1405,7 +1448,13 @@ hipError_t launch_prefill_layer(hipStream_t s, const mf_moe& h, const mf_moe_lay
   MF_TRY(launch_group(s, ws.idx, ws.w, t, c.top_k, c.num_experts, ws.counts, ws.offsets, ws.starts,
                       ws.sorted, ws.tiles, max_tiles, ws.n_tiles, ws.status, h.ws.group_tmp + 2048));
 
-  MF_TRY(launch_prep_rows(s, x, ws.xp, ws.sum_x, static_cast<size_t>(t) * c.d));
+  const bool want_gate = c.shared_f && w.w_sg;
+  if (want_gate) {  // one pass over x: matmul order, group sums and the shared gate's logits
+    prep_x_gate_kernel<<<dim3((t + 3) / 4), dim3(256), 0, s>>>(x, ws.xp, ws.sum_x, w.w_sg, ws.gate, t, c.d);
+    MF_TRY(hipGetLastError());
+  } else {
+    MF_TRY(launch_prep_rows(s, x, ws.xp, ws.sum_x, static_cast<size_t>(t) * c.d));
+  }
 
   QmmArgs q{};
   q.expert_base = static_cast<const uint8_t*>(w.expert_base);
@@ -1480,10 +1529,7 @@ hipError_t launch_prefill_layer(hipStream_t s, const mf_moe& h, const mf_moe_lay
   const uint16_t* gate = nullptr;
   if (c.shared_f) {
     hs = ws.hs;
-    if (w.w_sg) {
-      MF_TRY(launch_router_logits(s, w.w_sg, x, 1, c.d, t, c.d, nullptr, ws.gate));
-      gate = ws.gate;
-    }
+    if (want_gate) gate = ws.gate;
   }
   const size_t n4 = static_cast<size_t>(t) * c.d / 4;
   prefill_reduce_kernel<<<dim3(static_cast<uint32_t>((n4 + 255) / 256)), dim3(256), 0, s>>>(

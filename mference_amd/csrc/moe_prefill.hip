@@ -1209,12 +1209,16 @@ __global__ __launch_bounds__(256) void prefill_reduce_kernel(const float* __rest
 
 hipError_t launch_prefill_router(hipStream_t s, const uint16_t* W, const uint16_t* x, uint32_t E,
                                  uint32_t D, uint32_t T, uint32_t x_stride, float* logits) {
-  if (D % 512 == 0 && E % 32 == 0 && aligned16(W) && aligned16(x) && x_stride % 8 == 0) {
+  // Up to 256 tokens the matrix-core kernel has too few workgroups (T/32 x E/32) to cover the chip: the
+  // register-tiled kernel is faster there (Qwen shape, layer time: 64 tokens 110 -> 100 us, 128 tokens
+  // 112 -> 103 us, 256 tokens 118 -> 116 us, equal at 384; it holds rows of up to 4096 elements).  Both give
+  // the same bits.
+  if ((T > 256 || D > 4096) && D % 512 == 0 && E % 32 == 0 && aligned16(W) && aligned16(x) && x_stride % 8 == 0) {
     prefill_router_mfma_kernel<<<dim3((T + 31) / 32, E / 32), dim3(256), 0, s>>>(W, x, E, D, T, x_stride, logits);
     return hipGetLastError();
   }
   const uint32_t cpl = (D / 8 + 63) / 64;
-  const uint32_t tpb = std::max(1u, std::min(64u, T / 64));  // about a thousand workgroups
+  const uint32_t tpb = std::max(4u, std::min(64u, T / 64));  // about a thousand workgroups, >= 4 tokens per row load
 #define MF_PR(CPL, R)                                                                              \
   prefill_router_kernel<CPL, R><<<dim3((E + 4 * R - 1) / (4 * R), (T + tpb - 1) / tpb), dim3(256), 0, s>>>( \
       W, x, E, D, T, x_stride, logits, tpb)

@@ -572,6 +572,17 @@ def main() -> int:
     gpu_ms = ev0.elapsed_time(ev1)
     ms_per_step = gpu_ms / K
     us_per_layer = ms_per_step * 1e3 / L
+    # spread over single steps (their own event pairs, after the timed region): p10 / median / p90
+    n_spread = min(K, 200)
+    evs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(n_spread)]
+    for a, b in evs:
+        a.record()
+        run()
+        b.record()
+    torch.cuda.synchronize()
+    per_step = np.sort(np.array([a.elapsed_time(b) for a, b in evs])) * 1e3 / L
+    spread = {"steps": n_spread, "p10": round(float(np.percentile(per_step, 10)), 3),
+              "median": round(float(np.median(per_step)), 3), "p90": round(float(np.percentile(per_step, 90)), 3)}
     for m in moes:
         m.status()
     finite = bool(torch.isfinite(ys.float()).all().item())
@@ -586,6 +597,7 @@ def main() -> int:
         "unit": "us",
         "n_gpus": 1, "steps": K, "warmup": W,
         "ms_per_step": round(ms_per_step, 5),
+        "us_per_layer_single_steps": spread,
         "higher_is_better": False,
         "scaling": "weak",
         "vs_baseline": None,

@@ -178,13 +178,18 @@ __device__ __forceinline__ void trace_mark(const FusedArgs& a, uint32_t slot) {
 // control flow -- the launch executes each instruction once per wave, so code
 // size is instruction-fetch latency.  RuntimeShape reads the dimensions from
 // the arguments and handles everything else.
-struct RuntimeShape {
-  static constexpr bool kStatic = false;
+// kGiven: the routing is the caller's (written by an earlier launch, e.g. a family router): the kernel
+// has no router rows, no logits exchange and no top-k, and reads indices and weights instead of
+// writing them.  A compile-time property, so the kernels that route keep their code as it is.
+template <bool GIVEN = false>
+struct RuntimeShapeT {
+  static constexpr bool kStatic = false, kGiven = GIVEN;
   static constexpr uint32_t D = 0, F = 0, E = 0, K = 0, T = 0, Fs = 0;
 };
-template <uint32_t D_, uint32_t F_, uint32_t E_, uint32_t K_, uint32_t T_, uint32_t Fs_>
+using RuntimeShape = RuntimeShapeT<false>;
+template <uint32_t D_, uint32_t F_, uint32_t E_, uint32_t K_, uint32_t T_, uint32_t Fs_, bool GIVEN = false>
 struct StaticShape {
-  static constexpr bool kStatic = true;
+  static constexpr bool kStatic = true, kGiven = GIVEN;
   static constexpr uint32_t D = D_, F = F_, E = E_, K = K_, T = T_, Fs = Fs_;
 };
 
@@ -228,7 +233,7 @@ __global__ __launch_bounds__(kFusedThreads) void fused_decode_kernel(const Fused
   {
     const uint32_t lpr_log2 = Fs ? lanes_per_row_log2_dev(D, Fmt<SBITS>::kElemsPer16B) : 0;
     const uint32_t lpr = 1u << lpr_log2, rpw = 64u >> lpr_log2;
-    const uint32_t n_router = E * T;
+    const uint32_t n_router = S::kGiven ? 0 : E * T;
     const uint32_t n_gate = (Fs && a.w_sg) ? T : 0;
     const uint32_t srg = Fs ? (Fs + rpw - 1) / rpw : 0;
     const uint32_t n_items = n_router + n_gate + T * srg;
@@ -284,19 +289,28 @@ __global__ __launch_bounds__(kFusedThreads) void fused_decode_kernel(const Fused
   trace_mark(a, 1);
 
   // ------------------------------------------------------- logits, top-k
-  if (wv < T)
-    poll_tagged_f32(a.t_logits + static_cast<size_t>(wv) * E, s_lg + wv * E, E, epoch, lane,
-                    a.status);
-  __syncthreads();
-  trace_mark(a, 2);
-  if (wv < T) {
-    if (a.router_mode == 0) topk_select_fast(s_lg + wv * E, E, K, s_idx + wv * K, s_w + wv * K, lane);
-    else topk_full_softmax_fast(s_lg + wv * E, s_lg + wv * E, E, K, s_idx + wv * K, s_w + wv * K, lane);
-  }
-  __syncthreads();
-  if (wg == 0 && threadIdx.x < T * K) {
-    if (a.out_idx) a.out_idx[threadIdx.x] = s_idx[threadIdx.x];
-    if (a.out_w) a.out_w[threadIdx.x] = s_w[threadIdx.x];
+  if constexpr (!S::kGiven) {
+    if (wv < T)
+      poll_tagged_f32(a.t_logits + static_cast<size_t>(wv) * E, s_lg + wv * E, E, epoch, lane,
+                      a.status);
+    __syncthreads();
+    trace_mark(a, 2);
+    if (wv < T) {
+      if (a.router_mode == 0) topk_select_fast(s_lg + wv * E, E, K, s_idx + wv * K, s_w + wv * K, lane);
+      else topk_full_softmax_fast(s_lg + wv * E, s_lg + wv * E, E, K, s_idx + wv * K, s_w + wv * K, lane);
+    }
+    __syncthreads();
+    if (wg == 0 && threadIdx.x < T * K) {
+      if (a.out_idx) a.out_idx[threadIdx.x] = s_idx[threadIdx.x];
+      if (a.out_w) a.out_w[threadIdx.x] = s_w[threadIdx.x];
+    }
+  } else {  // routing written by an earlier launch on the stream (a family router): read, never written
+    trace_mark(a, 2);
+    if (threadIdx.x < T * K) {
+      s_idx[threadIdx.x] = a.out_idx[threadIdx.x];
+      s_w[threadIdx.x] = a.out_w[threadIdx.x];
+    }
+    __syncthreads();
   }
   trace_mark(a, 3);
 
@@ -647,7 +661,15 @@ hipError_t launch_fused_decode(hipStream_t s, const mf_moe& h, const mf_moe_laye
   using TernT1 = StaticShape<2048, 1024, 64, 8, 1, 0>;
   const bool tern_t1 = c.bits == MF_BITS_TERNARY && c.d == 2048 && c.f == 1024 && c.num_experts == 64 &&
                        c.top_k == 8 && c.shared_f == 0 && t == 1;
-  if (qwen_t1) MF_FUSED(kBits4, kBits4, QwenT1);
+  using Given = RuntimeShapeT<true>;
+  using Big2T1Given = StaticShape<4096, 2048, 256, 6, 1, 2048, true>;
+  if (!w.router_w) {  // caller-given routing
+    if (big2 && t == 1) MF_FUSED(kBits2, kBits4, Big2T1Given);
+    else if (c.bits == MF_BITS_4) MF_FUSED(kBits4, kBits4, Given);
+    else if (c.bits == MF_BITS_2 && c.shared_f && c.shared_bits == MF_BITS_2) MF_FUSED(kBits2, kBits2, Given);
+    else if (c.bits == MF_BITS_2) MF_FUSED(kBits2, kBits4, Given);
+    else MF_FUSED(kBitsTernary, kBits4, Given);
+  } else if (qwen_t1) MF_FUSED(kBits4, kBits4, QwenT1);
   else if (big2 && t == 1) MF_FUSED(kBits2, kBits4, Big2T1);
   else if (big2 && t == 4) MF_FUSED(kBits2, kBits4, Big2T4);
   else if (tern_t1) MF_FUSED(kBitsTernary, kBits4, TernT1);

@@ -315,11 +315,17 @@ def test_decode_layer_with_given_routing_equals_own_routing(gpu, oracle):
     given = ops.MoELayerWeights(router_w=None, experts=wts.experts, offsets=wts.offsets, shared=wts.shared,
                                 w_sg=wts.w_sg)
     y1 = torch.zeros_like(y0)
-    moe.set_fused(True)  # the fused launch routes by itself, so given routing takes the chain
-    moe.encode_decode_layer(given, xd, y1, t=t, out_indices=idx, out_weights=w)
-    torch.cuda.synchronize()
+    for fused in (True, False):  # the fused launch skips its router rows and top-k; the chain its two launches
+        moe.set_fused(fused)
+        y1.zero_()
+        moe.encode_decode_layer(given, xd, y1, t=t, out_indices=idx, out_weights=w)
+        moe.status()
+        assert torch.equal(y0.view(torch.int16), y1.view(torch.int16)), fused
+        assert torch.equal(idx, idx_before) and torch.equal(w, w_before)
+    moe.set_fused(True)
+    moe.encode_decode_layer(wts, xd, y1, t=t)  # and the handle still routes by itself afterwards
+    moe.status()
     assert torch.equal(y0.view(torch.int16), y1.view(torch.int16))
-    assert torch.equal(idx, idx_before) and torch.equal(w, w_before)
     ref_y, _, _ = oracle.moe_layer(layer, x)
     assert_layer_close(oracle.bf16_to_float(ops.bf16_bits(y1)), oracle.bf16_to_float(ref_y), "given routing")
     with pytest.raises(ops.MfError) as err:  # no router and no routing

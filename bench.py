@@ -331,6 +331,78 @@ def bench_dense_mlp(args, device) -> int:
     return 0
 
 
+def measure_given_routing(ctx, device, layers=16, replays=50):
+    """Decode layers (T = 1) whose routing comes from a family router: the sqrtsoftplus router call followed
+    by the layer call with router_w = NULL, against the layer routing by itself; µs per layer from HIP-graph
+    replays over `layers` distinct weight sets."""
+    import torch
+    from mference_amd import operators as ops
+
+    out = []
+    fam = ops.FamilyRouters(ctx)
+    for name in ("qwen-decode", "dsv4-2bit"):
+        w = dict(WORKLOADS[name])
+        stack = build_stack(ctx, w, layers, device)
+        moes = [ops.MoE(ctx, w["d"], w["f"], w["e"], w["k"], bits=w["bits"], shared_f=w["fs"],
+                        shared_bits=w["shared_bits"]) for _ in range(layers)]
+        gen = torch.Generator(device=device)
+        gen.manual_seed(7)
+        xs = torch.randn((layers, 1, w["d"]), generator=gen, device=device).to(torch.bfloat16)
+        ys = torch.zeros_like(xs)
+        idx = torch.zeros((layers, 1, w["k"]), dtype=torch.int32, device=device)
+        wt = torch.zeros((layers, 1, w["k"]), dtype=torch.float32, device=device)
+        lg = torch.zeros((layers, 1, w["e"]), dtype=torch.float32, device=device)
+        bias = torch.zeros((w["e"],), device=device)
+        given = [ops.MoELayerWeights(router_w=None, experts=s.experts, offsets=s.offsets, shared=s.shared,
+                                     w_sg=s.w_sg) for s in stack]
+
+        def own():
+            for l in range(layers):
+                moes[l].encode_decode_layer(stack[l], xs[l], ys[l], t=1)
+
+        def routed(with_router, fused):
+            def f():
+                for l in range(layers):
+                    moes[l].set_fused(fused)
+                    if with_router:
+                        fam.encode_router_top_k(stack[l].router_w, xs[l], bias, idx[l], wt[l], w["e"], w["d"], 1.5,
+                                                lg[l], top_k=w["k"])
+                    moes[l].encode_decode_layer(given[l], xs[l], ys[l], t=1, out_indices=idx[l], out_weights=wt[l])
+            return f
+
+        run = {"layer": w["name"]}
+        for label, fn in (("routes_itself_us", own), ("router_call_plus_layer_us", routed(True, True)),
+                          ("layer_on_given_routing_us", routed(False, True)),
+                          ("router_call_plus_chain_of_launches_us", routed(True, False))):
+            fn()
+            torch.cuda.synchronize()
+            side = torch.cuda.Stream()
+            side.wait_stream(torch.cuda.current_stream())
+            with torch.cuda.stream(side):
+                fn()
+            torch.cuda.current_stream().wait_stream(side)
+            torch.cuda.synchronize()
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(graph):
+                fn()
+            for _ in range(10):
+                graph.replay()
+            torch.cuda.synchronize()
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            for _ in range(replays):
+                graph.replay()
+            e1.record()
+            torch.cuda.synchronize()
+            run[label] = round(e0.elapsed_time(e1) / replays / layers * 1e3, 2)
+        for m in moes:
+            m.set_fused(True)
+            m.status()
+        out.append(run)
+        del stack, moes, given
+    return out
+
+
 def bench_family_routers(args, device) -> int:
     """The four family routers at their reference shapes, T = 1 (decode) and T = 2048 (prefill): µs per
     call from HIP-graph replays, the decode call against the HBM roofline of its router bytes, and the
@@ -442,6 +514,7 @@ def bench_family_routers(args, device) -> int:
         "data": "synthetic (N(0,0.05) router rows, N(0,1) activations)",
         "config": {"workload": "family-routers", "launch": "hip_graph", "weight_sets_T1": sets},
         "runs": results,
+        "decode_layer_on_family_routing": measure_given_routing(ctx, device),
         "roofline": {"bound": "hbm", "achieved": head["gbps"], "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                      "frac": head["hbm_frac"], "traffic": None,
                      "kernel": "mf::router_logits_kernel + mf::family_select_kernel (two launches per call)",

@@ -48,7 +48,7 @@ __global__ __launch_bounds__(256) void prefill_router_kernel(const uint16_t* __r
                                                              uint32_t E, uint32_t D, uint32_t T,
                                                              uint32_t x_stride,
                                                              float* __restrict__ logits,
-                                                             uint32_t tokens_per_block) {
+                                                             uint32_t tokens_per_block, uint32_t ld) {
   const uint32_t lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
   const uint32_t row0 = (blockIdx.x * 4 + wv) * R;
   if (row0 >= E) return;
@@ -93,7 +93,7 @@ __global__ __launch_bounds__(256) void prefill_router_kernel(const uint16_t* __r
         }
       }
       const float v = wave_sum(acc);
-      if (lane == 0 && row0 + r < E) logits[static_cast<size_t>(t) * E + row0 + r] = v;
+      if (lane == 0 && row0 + r < E) logits[static_cast<size_t>(t) * ld + row0 + r] = v;
     }
   }
 }
@@ -113,7 +113,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
                                                                   const uint16_t* __restrict__ x,
                                                                   uint32_t E, uint32_t D, uint32_t T,
                                                                   uint32_t x_stride,
-                                                                  float* __restrict__ logits) {
+                                                                  float* __restrict__ logits, uint32_t ld) {
   __shared__ float s_part[3][16 * 64];
   const uint32_t lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
   const uint32_t m = lane & 31, b = lane >> 5;
@@ -213,7 +213,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
       const float s01 = total[r] + s_part[0][r * 64 + lane];
       const float s23 = s_part[1][r * 64 + lane] + s_part[2][r * 64 + lane];
       const uint32_t t = t0 + 8 * (r / 4) + 4 * b + (r % 4);
-      if (t < T) logits[static_cast<size_t>(t) * E + e0 + m] = s01 + s23;
+      if (t < T) logits[static_cast<size_t>(t) * ld + e0 + m] = s01 + s23;
     }
   }
 }
@@ -1212,16 +1212,25 @@ hipError_t launch_prefill_router(hipStream_t s, const uint16_t* W, const uint16_
   // Up to 256 tokens the matrix-core kernel has too few workgroups (T/32 x E/32) to cover the chip: the
   // register-tiled kernel is faster there (Qwen shape, layer time: 64 tokens 110 -> 100 us, 128 tokens
   // 112 -> 103 us, 256 tokens 118 -> 116 us, equal at 384; it holds rows of up to 4096 elements).  Both give
-  // the same bits.
-  if ((T > 256 || D > 4096) && D % 512 == 0 && E % 32 == 0 && aligned16(W) && aligned16(x) && x_stride % 8 == 0) {
-    prefill_router_mfma_kernel<<<dim3((T + 31) / 32, E / 32), dim3(256), 0, s>>>(W, x, E, D, T, x_stride, logits);
-    return hipGetLastError();
+  // the same bits.  The matrix-core kernel takes whole blocks of 32 rows; rows left over (the two sink rows
+  // of a 258-row Inkling router) go through the register-tiled kernel behind it.
+  const uint32_t e32 = (T > 256 || D > 4096) && D % 512 == 0 && aligned16(W) && aligned16(x) && x_stride % 8 == 0
+                           ? E & ~31u : 0u;
+  if (e32) {
+    prefill_router_mfma_kernel<<<dim3((T + 31) / 32, e32 / 32), dim3(256), 0, s>>>(W, x, e32, D, T, x_stride,
+                                                                                  logits, E);
+    if (e32 == E) return hipGetLastError();
   }
+  const uint32_t rest = E - e32;
+  const uint16_t* Wr = W + static_cast<size_t>(e32) * D;
+  float* lr = logits + e32;
   const uint32_t cpl = (D / 8 + 63) / 64;
-  const uint32_t tpb = std::max(4u, std::min(64u, T / 64));  // about a thousand workgroups, >= 4 tokens per row load
+  // about a thousand workgroups, >= 4 tokens per row load; the few rows left over by the matrix-core kernel
+  // fill one workgroup column only, so they take the shortest token runs
+  const uint32_t tpb = e32 ? 4u : std::max(4u, std::min(64u, T / 64));
 #define MF_PR(CPL, R)                                                                              \
-  prefill_router_kernel<CPL, R><<<dim3((E + 4 * R - 1) / (4 * R), (T + tpb - 1) / tpb), dim3(256), 0, s>>>( \
-      W, x, E, D, T, x_stride, logits, tpb)
+  prefill_router_kernel<CPL, R><<<dim3((rest + 4 * R - 1) / (4 * R), (T + tpb - 1) / tpb), dim3(256), 0, s>>>( \
+      Wr, x, rest, D, T, x_stride, lr, tpb, E)
   if (cpl <= 1) MF_PR(1, 4);
   else if (cpl <= 2) MF_PR(2, 4);
   else if (cpl <= 4) MF_PR(4, 4);

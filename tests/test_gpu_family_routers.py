@@ -148,7 +148,8 @@ def test_hash_router_repeats_and_out_of_range(gpu, oracle):
 
 
 @pytest.mark.parametrize("n_routed,n_shared,d,k,t", [(256, 2, 1024, 8, 1), (256, 2, 2048, 8, 5), (100, 1, 512, 6, 3),
-                                                     (64, 0, 256, 4, 2), (256, 2, 1024, 8, 200)])
+                                                     (64, 0, 256, 4, 2), (256, 2, 1024, 8, 200), (256, 2, 2048, 8, 300),
+                                                     (100, 1, 512, 6, 290)])
 def test_inkling_router_bit_exact(gpu, oracle, n_routed, n_shared, d, k, t):
     rows = n_routed + n_shared
     rng, wr, x = _draw(oracle, f"inkling-{rows}-{d}-{k}-{t}", rows, d, t, 0.05)
@@ -163,8 +164,10 @@ def test_inkling_router_bit_exact(gpu, oracle, n_routed, n_shared, d, k, t):
                               gam if n_shared else None, n_routed, n_shared, k, 2.5, d, lg, t=t)
     torch.cuda.synchronize()
     idx_h, w_h, gam_h = idx.cpu().numpy().astype(np.uint32), w.cpu().numpy(), gam.cpu().numpy()
-    for i in list(range(min(t, 8))) + ([t - 1] if t > 8 else []):
+    lg_h = lg.cpu().numpy()
+    for i in list(range(min(t, 8))) + ([t - 1, t // 2, 33] if t > 40 else []):
         ref_lg = oracle.router_logits(wr, x[i])
+        assert np.array_equal(_bits(lg_h[i]), _bits(ref_lg))
         ri, rw, rg = oracle.router_inkling(ref_lg, bias, 0.75, n_routed, n_shared, k, 2.5)
         assert np.array_equal(idx_h[i], ri)
         assert np.array_equal(_bits(w_h[i]), _bits(rw))

@@ -113,3 +113,59 @@ def test_grouping_matches_the_oracle_on_random_routes(oracle):
         assert np.array_equal(g.per_expert_offsets, ref["offsets"][:e])
         assert np.array_equal(g.per_expert_counts, ref["counts"][:e])
         assert np.array_equal(g.groups, ref["groups"]) and np.array_equal(g.tiles, ref["tiles"])
+
+
+def _c_layout(tmp_path):
+    """sizeof / offsetof of every struct in include/mfmoe.h, printed by a gcc-built probe."""
+    import subprocess
+    structs = {
+        "mf_expert_offsets": ["gate_w", "gate_s", "gate_b", "up_w", "up_s", "up_b",
+                              "down_w", "down_s", "down_b"],
+        "mf_qtensor": ["weights", "scales", "biases"],
+        "mf_pair": ["token", "expert", "rank", "weight_bits"],
+        "mf_moe_config": ["d", "f", "num_experts", "top_k", "bits", "router_mode", "swiglu_limit",
+                          "shared_f", "shared_bits", "maple_rounding"],
+        "mf_moe_layer_weights": ["router_w", "expert_base", "expert_stride", "offsets",
+                                 "shared_gate", "shared_up", "shared_down", "w_sg"],
+    }
+    lines = ['#include <stdio.h>', '#include <stddef.h>', '#include "mfmoe.h"', 'int main(void){']
+    for s, fields in structs.items():
+        lines.append(f'printf("{s} size %zu\\n", sizeof({s}));')
+        for f in fields:
+            lines.append(f'printf("{s} {f} %zu\\n", offsetof({s}, {f}));')
+    lines.append('return 0;}')
+    src = tmp_path / "layout_probe.c"
+    src.write_text("\n".join(lines))
+    exe = tmp_path / "layout_probe"
+    subprocess.run(["gcc", "-std=c11", "-I", os.path.join(ROOT, "include"), str(src), "-o", str(exe)],
+                   check=True)
+    out = subprocess.run([str(exe)], check=True, capture_output=True, text=True).stdout
+    table = {}
+    for line in out.splitlines():
+        s, f, v = line.split()
+        table[(s, f)] = int(v)
+    return structs, table
+
+
+def test_struct_layouts_of_header_and_ctypes_mirror_agree(tmp_path):
+    """The header compiles as plain C, and the ctypes structures the Python host side passes
+    have the sizes and field offsets the C compiler gives the header's.  The route record keeps
+    the reference's pinned layout: 16 bytes, stride 16, token / expert / rank / weight bits at
+    0 / 4 / 8 / 12 (PrefillRouterTests.swift:12-19); the offset table is nine uint32
+    (MoEExpertOffsets, Kernels/MoE/MoE.swift:4-29)."""
+    structs, table = _c_layout(tmp_path)
+    mirror = {"mf_expert_offsets": _capi.ExpertOffsets, "mf_qtensor": _capi.QTensor,
+              "mf_pair": _capi.Pair, "mf_moe_config": _capi.MoEConfig,
+              "mf_moe_layer_weights": _capi.LayerWeights}
+    for s, fields in structs.items():
+        cls = mirror[s]
+        assert C.sizeof(cls) == table[(s, "size")], s
+        assert [n for n, _ in cls._fields_] == fields, s
+        for f in fields:
+            assert getattr(cls, f).offset == table[(s, f)], (s, f)
+    assert table[("mf_pair", "size")] == 16
+    assert [table[("mf_pair", f)] for f in ("token", "expert", "rank", "weight_bits")] == [0, 4, 8, 12]
+    assert table[("mf_expert_offsets", "size")] == 36
+    assert [table[("mf_expert_offsets", f)] for f in structs["mf_expert_offsets"]] == list(range(0, 36, 4))
+    pairs = (_capi.Pair * 3)()
+    assert C.addressof(pairs[1]) - C.addressof(pairs[0]) == 16

@@ -10,7 +10,7 @@ checks, same error cases), `Model.routedExpertOffsets` / `routedExpertPhysicalOf
 pool the operators address as `expert_base + expert * stride`.
 
 What it does not do: the group-32 gate projection of the DeepSeek conversion is detected
-(`routed_gate_group_size`) but the kernels take group 64 only; Maple's per-row alpha tables
+(`routed_gate_group_size`) and refused (`require_group64_gate`): the kernels take group 64 only; Maple's per-row alpha tables
 are expected already expanded to per-group scale / bias entries, which is how the reference's
 repacker stores them.
 """
@@ -188,18 +188,35 @@ def routed_gate_group_size(layout: PackedExpertsLayout, layer: int, moe_intermed
     return hidden // groups
 
 
-def load_layer_experts(directory: str, layout: PackedExpertsLayout, layer: int, device="cuda"):
+def require_group64_gate(layout: PackedExpertsLayout, layer: int, moe_intermediate: int, hidden: int) -> None:
+    """Raises when the layer's gate projection is quantized in groups other than 64 (the
+    group-32 gate of the DeepSeek conversion, ModelExpertIO.swift:122-135): the operators read
+    one scale / bias entry per 64 columns and would compute wrong activations from such a
+    blob without noticing."""
+    g = routed_gate_group_size(layout, layer, moe_intermediate, hidden)
+    if g != GROUP_SIZE:
+        raise ModelError.index_corrupt(
+            f"layer {layer}: gate projection uses quantization group {g}; "
+            f"the resident operators take group {GROUP_SIZE} only")
+
+
+def load_layer_experts(directory: str, layout: PackedExpertsLayout, layer: int, device="cuda",
+                       moe_intermediate: Optional[int] = None, hidden: Optional[int] = None):
     """Read `packed_experts/<layer file>` into one resident uint8 tensor of
     experts_per_layer * expert_stride bytes in LOGICAL expert order (the operators address
     expert e at e * stride; the file may hold the blobs in any physical order).  Returns
     (tensor, stride).  The read goes through a pinned staging buffer in chunks, so a 453 MB
-    layer never needs a second full copy in host memory."""
+    layer never needs a second full copy in host memory.  With `moe_intermediate` and `hidden`
+    given, a layer whose gate projection is not quantized in groups of 64 is refused
+    (`require_group64_gate`) before anything is read."""
     import numpy as np
     import torch
 
     entry = layout.layers[layer]
     if not entry.experts:
         raise ModelError.index_corrupt(f"layer {layer} has no routed experts")
+    if moe_intermediate is not None and hidden is not None:
+        require_group64_gate(layout, layer, moe_intermediate, hidden)
     path = os.path.join(directory, "packed_experts", entry.file)
     if not os.path.isfile(path):
         raise ModelError.missing_file(entry.file)

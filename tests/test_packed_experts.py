@@ -131,6 +131,13 @@ def test_gate_group_size_from_the_scale_slice(tmp_path, oracle):
     layout = pe.PackedExpertsLayoutReader.load(str(tmp_path))
     assert pe.routed_gate_group_size(layout, 0, 128, 256) == 32
     assert pe.routed_gate_group_size(layout, 0, 0, 256) == 64
+    # such a layer is refused before its file is read: the operators take group 64 only
+    with pytest.raises(pe.ModelError, match="group 32") as err:
+        pe.load_layer_experts(str(tmp_path), layout, 0, device="cpu", moe_intermediate=128, hidden=256)
+    assert err.value.kind == "indexCorrupt"
+    with pytest.raises(pe.ModelError):
+        pe.require_group64_gate(layout, 0, 128, 256)
+    pe.require_group64_gate(layout, 0, 0, 256)   # unknown intermediate size: falls back to 64
 
 
 def test_layer_file_checks(tmp_path, oracle):

@@ -4,14 +4,17 @@ from __future__ import annotations
 import os
 import subprocess
 import sys
+from concurrent.futures import ThreadPoolExecutor
 
 HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
+OBJ = os.path.join(HERE, "build")
 LIB = os.path.join(HERE, "libmfmoe.so")
-SOURCES = ["format.hip", "gemv.hip", "router.hip", "router_family.hip", "moe_decode.hip", "moe_fused.hip", "moe_prefill.hip", "api.hip"]
+SOURCES = ["format.hip", "gemv.hip", "router.hip", "router_family.hip", "moe_decode.hip", "moe_fused.hip",
+           "moe_prefill.hip", "api.hip"]
 
 FLAGS = [
-    "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-shared",
+    "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC",
     "-ffp-contract=off",
     # packed-FP32 instructions are switched off for all device code
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
@@ -19,37 +22,31 @@ FLAGS = [
 ]
 
 
-def build(verbose: bool = False) -> str:
-    hipcc = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
-    cmd = [hipcc, *FLAGS, "-o", LIB, *[os.path.join(CSRC, s) for s in SOURCES]]
+def _run(cmd: list[str], verbose: bool) -> None:
     if verbose:
         print(" ".join(cmd), flush=True)
     proc = subprocess.run(cmd, capture_output=True, text=True)
     if proc.returncode != 0:
         sys.stderr.write(proc.stdout + proc.stderr)
-        raise RuntimeError("hipcc failed building libmfmoe.so")
+        raise RuntimeError("hipcc failed: " + " ".join(cmd[-3:]))
     if verbose and proc.stderr:
         sys.stderr.write(proc.stderr)
-    build_microbench(verbose)
+
+
+def build(verbose: bool = False, only: list[str] | None = None) -> str:
+    """Compiles every source to an object of its own (in parallel) and links them.  `only` names the
+    sources to recompile when the other objects are already there (a developer's shortcut; the build
+    check compiles everything)."""
+    hipcc = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
+    os.makedirs(OBJ, exist_ok=True)
+    objs = [os.path.join(OBJ, s.replace(".hip", ".o")) for s in SOURCES]
+    todo = [(s, o) for s, o in zip(SOURCES, objs) if only is None or s in only or not os.path.exists(o)]
+    jobs = min(8, max(1, (os.cpu_count() or 2) // 2))
+    with ThreadPoolExecutor(jobs) as pool:
+        list(pool.map(lambda so: _run([hipcc, *FLAGS, "-c", "-o", so[1], os.path.join(CSRC, so[0])], verbose), todo))
+    _run([hipcc, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", LIB, *objs], verbose)
     return LIB
 
 
-def build_microbench(verbose: bool = False) -> str:
-    """The stand-alone issue-port measurement (csrc/microbench/issue_port.hip): a program of its own,
-    not part of libmfmoe.so."""
-    hipcc = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
-    src = os.path.join(CSRC, "microbench", "issue_port.hip")
-    exe = os.path.join(CSRC, "microbench", "issue_port")
-    cmd = [hipcc, "--offload-arch=gfx950", "-O3", "-std=c++17", "-Xclang", "-target-feature", "-Xclang",
-           "-packed-fp32-ops", "-o", exe, src]
-    if verbose:
-        print(" ".join(cmd), flush=True)
-    proc = subprocess.run(cmd, capture_output=True, text=True)
-    if proc.returncode != 0:
-        sys.stderr.write(proc.stdout + proc.stderr)
-        raise RuntimeError("hipcc failed building microbench/issue_port")
-    return exe
-
-
 if __name__ == "__main__":
-    print(build(verbose=True))
+    print(build(verbose=True, only=sys.argv[1:] or None))

@@ -436,7 +436,7 @@ mf_status mf_moe_decode_layer(mf_moe* h, mf_stream stream, const mf_moe_layer_we
                      !qtensor_ok(wts->shared_down, c.shared_bits)))
     return MF_ERR_INVALID_ARGUMENT;
   auto s = static_cast<hipStream_t>(stream);
-  if (h->fused && mf::fused_supported(*h, *wts, x, y, hidden)) {
+  if (h->fused && mf::fused_supported(*h, *wts, x, y, hidden, t)) {
     MF_HIP(h->ctx, mf::launch_fused_decode(s, *h, *wts, x, t, y, hidden, out_idx, out_w));
     return MF_OK;
   }

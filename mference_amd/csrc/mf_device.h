@@ -178,6 +178,14 @@ __device__ __forceinline__ uint16_t load_u16_agent(const uint16_t* p) {
 __device__ __forceinline__ void store_u32_agent(uint32_t* p, uint32_t v) {
   __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
+// 16 bytes (16-byte aligned) written through as one request; readers rely on nothing wider than
+// the 4-byte words being whole
+__device__ __forceinline__ void store_u32x4_agent(uint32_t* p, uint32_t a, uint32_t b, uint32_t c, uint32_t d) {
+  typedef __attribute__((ext_vector_type(4))) unsigned int u32x4;
+  const u32x4 v = {a, b, c, d};
+  asm volatile("global_store_dwordx4 %0, %1, off sc1" : : "v"(p), "v"(v) : "memory");
+}
+__device__ __forceinline__ void store_u32x4_agent(uint32_t* p, uint32_t a) { store_u32x4_agent(p, a, a, a, a); }
 __device__ __forceinline__ void store_f32_agent(float* p, float v) {
   __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
@@ -205,6 +213,11 @@ __device__ __forceinline__ uint4 load_u32x4_agentbuf(const AgentBuf& b, uint32_t
                                                            16 /* sc1 */);
   return make_uint4(v.x, v.y, v.z, v.w);
 }
+
+// Nothing is moved across this point by the compiler: placed behind a group of loads it keeps
+// them one batch of requests (the compiler otherwise sinks some of them below the arithmetic on
+// the others, which turns one memory round trip into several).
+__device__ __forceinline__ void issue_fence() { asm volatile("" ::: "memory"); }
 
 // every store this wave has issued is acknowledged at its scope
 __device__ __forceinline__ void wait_stores() { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); }
@@ -463,6 +476,28 @@ __device__ __forceinline__ XSlice<BITS> load_xslice(const uint16_t* x) {
       const uint4 a = load_x8<MODE == kXAligned>(x + 8 * q);
       raw[4 * q] = a.x; raw[4 * q + 1] = a.y; raw[4 * q + 2] = a.z; raw[4 * q + 3] = a.w;
     }
+  }
+  XSlice<BITS> xs;
+  permute_x<BITS>(raw, xs);
+  return xs;
+}
+
+// the same in two steps: request the lane's slice (16-byte aligned), permute it later
+template <int BITS> struct XRaw { uint4 q[Fmt<BITS>::kElemsPer16B / 8]; };
+template <int BITS>
+__device__ __forceinline__ XRaw<BITS> load_xraw(const uint16_t* x) {
+  XRaw<BITS> r;
+#pragma unroll
+  for (int q = 0; q < Fmt<BITS>::kElemsPer16B / 8; ++q) r.q[q] = load_x8<true>(x + 8 * q);
+  return r;
+}
+template <int BITS>
+__device__ __forceinline__ XSlice<BITS> make_xslice(const XRaw<BITS>& r) {
+  constexpr int kQuads = Fmt<BITS>::kElemsPer16B / 8;
+  uint32_t raw[kQuads * 4];
+#pragma unroll
+  for (int q = 0; q < kQuads; ++q) {
+    raw[4 * q] = r.q[q].x; raw[4 * q + 1] = r.q[q].y; raw[4 * q + 2] = r.q[q].z; raw[4 * q + 3] = r.q[q].w;
   }
   XSlice<BITS> xs;
   permute_x<BITS>(raw, xs);

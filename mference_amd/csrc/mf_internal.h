@@ -114,7 +114,7 @@ hipError_t launch_phase2(hipStream_t s, const mf_moe_config& cfg, const void* ba
 
 // moe_fused.hip
 bool fused_supported(const mf_moe& h, const mf_moe_layer_weights& w, const void* x, const void* y,
-                     const void* hidden);
+                     const void* hidden, uint32_t t);
 hipError_t launch_fused_decode(hipStream_t s, const mf_moe& h, const mf_moe_layer_weights& w,
                                const uint16_t* x, uint32_t t, uint16_t* y, uint16_t* hidden,
                                uint32_t* out_idx, float* out_w);

@@ -20,23 +20,36 @@ __device__ __forceinline__ float dot_bf16_row(const uint16_t* __restrict__ w,
                                               uint32_t lane, bool aligned) {
   float acc = 0.0f;
   const uint32_t chunks = d / 8;
-  for (uint32_t c = lane; c < chunks; c += kWave) {
-    uint4 wv, xv;
-    if (aligned) {
-      wv = load_x8<true>(w + c * 8);
-      xv = load_x8<true>(x + c * 8);
-    } else {
-      wv = load_x8<false>(w + c * 8);
-      xv = load_x8<false>(x + c * 8);
+  // four steps' loads are requested before the first product is taken: a lane's chunks are one
+  // memory round trip, not one per step (the order of the fmaf chain is unchanged)
+  for (uint32_t c0 = lane; c0 < chunks; c0 += 4 * kWave) {
+    uint4 wv[4], xv[4];
+#pragma unroll
+    for (int s = 0; s < 4; ++s) {
+      const uint32_t c = c0 + s * kWave;
+      if (c < chunks) {
+        if (aligned) {
+          wv[s] = load_x8<true>(w + c * 8);
+          xv[s] = load_x8<true>(x + c * 8);
+        } else {
+          wv[s] = load_x8<false>(w + c * 8);
+          xv[s] = load_x8<false>(x + c * 8);
+        }
+      }
     }
-    acc = __builtin_fmaf(bf16_lo(wv.x), bf16_lo(xv.x), acc);
-    acc = __builtin_fmaf(bf16_hi(wv.x), bf16_hi(xv.x), acc);
-    acc = __builtin_fmaf(bf16_lo(wv.y), bf16_lo(xv.y), acc);
-    acc = __builtin_fmaf(bf16_hi(wv.y), bf16_hi(xv.y), acc);
-    acc = __builtin_fmaf(bf16_lo(wv.z), bf16_lo(xv.z), acc);
-    acc = __builtin_fmaf(bf16_hi(wv.z), bf16_hi(xv.z), acc);
-    acc = __builtin_fmaf(bf16_lo(wv.w), bf16_lo(xv.w), acc);
-    acc = __builtin_fmaf(bf16_hi(wv.w), bf16_hi(xv.w), acc);
+#pragma unroll
+    for (int s = 0; s < 4; ++s) {
+      if (c0 + s * kWave < chunks) {
+        acc = __builtin_fmaf(bf16_lo(wv[s].x), bf16_lo(xv[s].x), acc);
+        acc = __builtin_fmaf(bf16_hi(wv[s].x), bf16_hi(xv[s].x), acc);
+        acc = __builtin_fmaf(bf16_lo(wv[s].y), bf16_lo(xv[s].y), acc);
+        acc = __builtin_fmaf(bf16_hi(wv[s].y), bf16_hi(xv[s].y), acc);
+        acc = __builtin_fmaf(bf16_lo(wv[s].z), bf16_lo(xv[s].z), acc);
+        acc = __builtin_fmaf(bf16_hi(wv[s].z), bf16_hi(xv[s].z), acc);
+        acc = __builtin_fmaf(bf16_lo(wv[s].w), bf16_lo(xv[s].w), acc);
+        acc = __builtin_fmaf(bf16_hi(wv[s].w), bf16_hi(xv[s].w), acc);
+      }
+    }
   }
   return wave_sum(acc);
 }
@@ -211,6 +224,181 @@ __device__ __forceinline__ void topk_select_fast(const float* lg, uint32_t e, ui
   else if (per <= 2) topk_select_sorted<2>(lg, e, k, idx, w, lane);
   else if (per <= 4) topk_select_sorted<4>(lg, e, k, idx, w, lane);
   else topk_select_sorted<8>(lg, e, k, idx, w, lane);
+}
+
+// ---- workgroup-collective selection (the fused decode launch)
+//
+// The rank of expert i is the number of experts that beat it under the selectors' total order
+// (higher score first, equal scores: lower index first; NaN counts as -inf), so the expert of
+// rank r is exactly what round r of the serial selector picks.
+__device__ __forceinline__ float score_or_ninf(float x) {
+  const float ninf = -__builtin_inff();
+  return (x > ninf) ? x : ninf;
+}
+// does (q, j) beat (v, i)?  q, v hold no NaN
+__device__ __forceinline__ uint32_t beats(float q, uint32_t j, float v, uint32_t i) {
+  return (q > v || (q == v && j < i)) ? 1u : 0u;
+}
+
+// Full rank count: every wave takes a block of 64 candidates (one per lane) and a slice of the
+// experts to compare them with, read from LDS four at a time as broadcasts, and adds its count to
+// rank[] with an LDS atomic.  vals, rank: LDS [t_count][e], vals without NaN, e a multiple of 4,
+// rank zero on entry.  A workgroup barrier has to follow before topk_rank_emit.
+template <int ORDER>  // -1: every j < i (an equal score beats), +1: every j > i, 0: mixed
+__device__ __forceinline__ uint32_t count_beats(const float* lg, uint32_t j0, uint32_t j1, float v, uint32_t i) {
+  uint32_t cnt = 0;
+  for (uint32_t j = j0; j + 4 <= j1; j += 4) {
+    const float4 q = *reinterpret_cast<const float4*>(lg + j);
+    if constexpr (ORDER < 0) cnt += (q.x >= v) + (q.y >= v) + (q.z >= v) + (q.w >= v);
+    else if constexpr (ORDER > 0) cnt += (q.x > v) + (q.y > v) + (q.z > v) + (q.w > v);
+    else cnt += beats(q.x, j, v, i) + beats(q.y, j + 1, v, i) + beats(q.z, j + 2, v, i) + beats(q.w, j + 3, v, i);
+  }
+  return cnt;
+}
+__device__ __forceinline__ void topk_rank_count(const float* vals, uint32_t* rank, uint32_t t_count,
+                                                uint32_t e, uint32_t wv, uint32_t lane, uint32_t nwaves) {
+  const uint32_t eb = (e + kWave - 1) / kWave;  // candidate blocks per token
+  const uint32_t blocks = t_count * eb;
+  uint32_t split = 1;  // slices of the comparison range, each a multiple of 4 long
+  while (blocks * split * 2 <= nwaves && e % (8 * split) == 0) split *= 2;
+  const uint32_t jr = e / split;
+  for (uint32_t item = wv; item < blocks * split; item += nwaves) {
+    const uint32_t b = item / split, js = item % split;
+    const uint32_t t = b / eb, i0 = (b % eb) * kWave, i = i0 + lane;
+    const float* lg = vals + t * e;
+    const float v = i < e ? lg[i] : 0.0f;
+    const uint32_t j0 = js * jr, j1 = j0 + jr;
+    uint32_t cnt;
+    if (j1 <= i0) cnt = count_beats<-1>(lg, j0, j1, v, i);
+    else if (j0 >= i0 + kWave) cnt = count_beats<1>(lg, j0, j1, v, i);
+    else cnt = count_beats<0>(lg, j0, j1, v, i);
+    if (i < e) atomicAdd(&rank[t * e + i], cnt);
+  }
+}
+// Every expert whose rank is below k writes itself to idx / sc [t_count][k] (a value that is not a
+// candidate -- -inf -- gives index 0, score -inf, like a round without a winner).  idx / sc
+// entries of ranks that no expert takes (k > e) must have been set to 0 / -inf by the caller.
+__device__ __forceinline__ void topk_rank_emit(const float* vals, const uint32_t* rank, uint32_t t_count,
+                                               uint32_t e, uint32_t k, uint32_t* idx, float* sc,
+                                               uint32_t tid, uint32_t nthreads) {
+  const float ninf = -__builtin_inff();
+  for (uint32_t p = tid; p < t_count * e; p += nthreads) {
+    const uint32_t r = rank[p];
+    if (r < k) {
+      const uint32_t t = p / e, i = p % e;
+      const float x = vals[p];
+      const bool valid = x > ninf;
+      idx[t * k + r] = valid ? i : 0u;
+      sc[t * k + r] = valid ? x : ninf;
+    }
+  }
+}
+
+// Selection with a prefilter, for e a multiple of 64 with e / 16 >= k and one wave per block of 64
+// experts (t_count * e / 64 <= nwaves).  The k-th largest of the maxima of the 16-expert
+// sub-blocks, L, is a lower bound of the k-th largest score: k distinct experts reach it.  So
+// every selected expert has a score >= L, and so has everything that beats such an expert: the
+// ranks of the experts with score >= L among themselves are their ranks among all.  There are
+// usually a dozen of them; they are compacted into a list and one wave per token ranks the list.
+// More than 64 of them (many equal scores, or fewer than k finite ones) raise *fallback and the
+// caller counts ranks over everything instead.
+// scr: LDS words, zero on entry: [0, 256) sub-block maxima, [256, 264) list lengths per token,
+// [512, 512 + t_count * 128) the lists of (score bits, index).  Contains workgroup barriers: all
+// threads call it.
+constexpr uint32_t kPrefilterScratchWords = 512 + MF_MAX_TOKENS * 128;
+__device__ __forceinline__ bool topk_prefilter_fits(uint32_t t_count, uint32_t e, uint32_t k, uint32_t nwaves) {
+  return e % 64 == 0 && e / 16 >= k && t_count * (e / 64) <= nwaves && t_count * (e / 16) <= 256;
+}
+__device__ __forceinline__ void topk_prefilter(const float* vals, uint32_t* scr, uint32_t* fallback,
+                                               uint32_t t_count, uint32_t e, uint32_t k, uint32_t* idx,
+                                               float* sc, uint32_t wv, uint32_t lane) {
+  const float ninf = -__builtin_inff();
+  float* smax = reinterpret_cast<float*>(scr);
+  uint32_t* n_list = scr + 256;
+  uint32_t* lists = scr + 512;
+  const uint32_t eb = e / kWave, nsb = e / 16;
+  const bool mine = wv < t_count * eb;  // this wave has a block
+  const uint32_t t = mine ? wv / eb : 0, b = mine ? wv % eb : 0;
+  const uint32_t i = b * kWave + lane;
+  const float v = mine ? vals[t * e + i] : ninf;
+  if (mine) {  // maximum of each row of 16 lanes
+    float m = v;
+    m = fmaxf(m, dpp_f<0xB1>(m));
+    m = fmaxf(m, dpp_f<0x4E>(m));
+    m = fmaxf(m, dpp_f<0x141>(m));
+    m = fmaxf(m, dpp_f<0x140>(m));
+    if ((lane & 15) == 0) smax[t * nsb + b * 4 + lane / 16] = m;
+  }
+  __syncthreads();
+  if (mine) {
+    // L: the sub-block maximum of rank k - 1 (ranked like the scores, so exactly one lane has it)
+    const float* sm = smax + t * nsb;
+    const float ml = lane < nsb ? sm[lane] : ninf;
+    uint32_t r = 0;
+    for (uint32_t j = 0; j < nsb; j += 4) {
+      const float4 q = *reinterpret_cast<const float4*>(sm + j);
+      r += beats(q.x, j, ml, lane) + beats(q.y, j + 1, ml, lane) + beats(q.z, j + 2, ml, lane) + beats(q.w, j + 3, ml, lane);
+    }
+    const unsigned long long km = __ballot(lane < nsb && r == k - 1);
+    const float L = readlane_f(ml, __ffsll(static_cast<long long>(km)) - 1);
+    // the experts that reach L join their token's list (in any order: the list is ranked below)
+    const bool c = v >= L;
+    const unsigned long long cm = __ballot(c);
+    const uint32_t n = static_cast<uint32_t>(__popcll(cm));
+    uint32_t base = 0;
+    if (lane == 0) base = atomicAdd(&n_list[t], n);
+    base = static_cast<uint32_t>(__builtin_amdgcn_readfirstlane(static_cast<int>(base)));
+    const uint32_t pos = base + __builtin_amdgcn_mbcnt_hi(static_cast<uint32_t>(cm >> 32),
+                                                          __builtin_amdgcn_mbcnt_lo(static_cast<uint32_t>(cm), 0u));
+    if (c && pos < kWave) {
+      lists[t * 128 + 2 * pos] = __float_as_uint(v);
+      lists[t * 128 + 2 * pos + 1] = i;
+    }
+  }
+  __syncthreads();
+  if (wv < t_count) {  // wave t ranks the list of token t
+    const uint32_t n = n_list[wv];
+    if (n > kWave) {
+      if (lane == 0) *fallback = 1u;
+    } else {
+      const uint2* lst = reinterpret_cast<const uint2*>(lists + wv * 128);
+      const uint2 me = lane < n ? lst[lane] : make_uint2(0u, 0u);
+      const float vc = __uint_as_float(me.x);
+      uint32_t r = 0;
+      for (uint32_t j = 0; j < n; ++j) {
+        const uint2 o = lst[j];
+        r += beats(__uint_as_float(o.x), o.y, vc, me.y);
+      }
+      if (lane < n && r < k) {
+        const bool valid = vc > ninf;
+        idx[wv * k + r] = valid ? me.y : 0u;
+        sc[wv * k + r] = valid ? vc : ninf;
+      }
+    }
+  }
+  __syncthreads();
+}
+
+// Routing weight of rank `lane` from the selected scores (my_score in lanes < k): MODE 0
+// exp(s_r - s_0) / sum, MODE 1 p_r / (sum + 1e-20); sums in rank order -- the tails of
+// topk_select_sorted.  All 64 lanes call it.
+template <int MODE>
+__device__ __forceinline__ float topk_weight_of_rank(float my_score, uint32_t k) {
+  if constexpr (MODE == 1) {
+    float sum = 0.0f;
+#pragma unroll
+    for (int i = 0; i < MF_MAX_TOPK; ++i)
+      if (static_cast<uint32_t>(i) < k) sum += readlane_f(my_score, i);
+    return my_score / (sum + 1.0e-20f);
+  } else {
+    const float s0 = readlane_f(my_score, 0);
+    const float my_e = mf_exp(my_score - s0);
+    float sum = 0.0f;
+#pragma unroll
+    for (int i = 0; i < MF_MAX_TOPK; ++i)
+      if (static_cast<uint32_t>(i) < k) sum += readlane_f(my_e, i);
+    return my_e / sum;
+  }
 }
 
 // indices of the k best selection scores (same tie rule), for the family routers

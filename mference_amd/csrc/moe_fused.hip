@@ -4,8 +4,8 @@
 //
 //   A  router logits (one wave per expert row), the scalar shared gate w_sg.x,
 //      shared-expert gate/up/activation rows
-//      -> every workgroup gathers the logits and recomputes the (cheap,
-//         deterministic) top-k itself
+//      -> every workgroup gathers the logits and selects the top-k itself (cheap and
+//         deterministic: rank counting over the logits in LDS, all waves)
 //   B  routed gate/up/activation rows of the K selected experts of every token
 //   C  per token: the shared expert's down rows of this workgroup's output rows
 //      (-> gated h1, kept in LDS), then the routed down rows: K waves take the K
@@ -18,16 +18,22 @@
 // value; bf16 activations: a 16-bit tag above the value), producers write them
 // with device-coherent stores and go on, consumers poll the data itself with
 // device-coherent loads into LDS until every tag they need is current.  This
-// costs one store propagation plus about one load round trip per exchange;
+// costs one store propagation plus about one load round trip per exchange
+// (0.55 - 0.65 us between two workgroups, on the same XCD or not);
 // a barrier built on a flag or counter costs a store acknowledgement, the flag's
-// own propagation, a poll and then the data load (measured: 4-5 us against
-// about 2 us, two exchanges per layer).  The epoch is a per-workgroup counter
+// own propagation, a poll and then the data load.  The epoch is a per-workgroup counter
 // in the workspace that every workgroup raises by one per launch, so all
 // workgroups agree on it without talking, nothing is reset between launches
 // and a captured HIP graph can replay the launch.  One token slot of the
 // activation buffers (epoch mod 8, if unused by this launch) is re-tagged per
 // launch so that no stale word is ever older than 8 launches: a 16-bit tag can
 // never alias.
+//
+// Producers write whole 64-byte pieces.  Work is dealt in chunks of consecutive rows, one chunk
+// per workgroup, the waves' results meet in LDS and one store instruction writes the chunk:
+// when neighbouring words of a line are written through by different workgroups (different
+// XCDs), the partial-line writes serialise in the memory system and the gather of a 16 KiB
+// vector by all workgroups takes 3.3 us instead of 1.4 us (2 KiB: 2.4 against 1.2 us).
 //
 // Nothing but the router decides which weights are read, so stage C's packed
 // codes are requested before the routed activations are polled: their HBM
@@ -37,7 +43,7 @@
 // grid has to be resident at once: the launcher never asks for more workgroups
 // than CUs and the kernel needs a whole CU (1024 threads, <= 128 VGPRs).  Waits
 // are bounded: a poll that does not complete within kSpinLimit tries sets the
-// status word and lets the grid drain.
+// status word, the workgroup writes NaN to the output rows it owns and the grid drains.
 #include "mf_device.h"
 #include "mf_internal.h"
 #include "mf_router.h"
@@ -48,7 +54,10 @@ namespace mf {
 
 constexpr uint32_t kFusedThreads = 1024;
 constexpr uint32_t kFusedWaves = kFusedThreads / kWave;
-constexpr uint32_t kSpinLimit = 1u << 20;  // x ~1 us per poll
+constexpr uint32_t kSpinLimit = 1u << 17;  // x ~0.6 us per poll
+constexpr uint32_t kRouterChunk = 8;       // router rows per workgroup chunk: 8 tagged logits = 64 bytes
+constexpr uint32_t kRankCountLimit = 1u << 18;  // T * E * E up to which the top-k counts ranks
+constexpr uint32_t kRankWords = 2048;      // ... and T * E it may have then
 constexpr uint32_t kMaxH1 = 2048;          // output rows of one token a workgroup may own
 
 template <int BITS> struct Chunk {
@@ -101,13 +110,42 @@ __device__ __forceinline__ void gate_up_partial(const uint8_t* gw, const uint16_
   for (uint32_t e0 = sub * EPL; e0 < N; e0 += lpr * EPL) {
     const Chunk<BITS> g = load_chunk<BITS>(gw, gs, gb, e0);
     const Chunk<BITS> u = load_chunk<BITS>(uw, us, ub, e0);
-    const XSlice<BITS> xs = load_xslice<BITS, kXAligned>(x + e0);
+    const XRaw<BITS> xr = load_xraw<BITS>(x + e0);
+    issue_fence();
+    const XSlice<BITS> xs = make_xslice<BITS>(xr);
     const float gd = codes_dot<BITS>(g.codes, xs), ud = codes_dot<BITS>(u.codes, xs);
     ga = __builtin_fmaf(g.s, gd, ga);
     ga = __builtin_fmaf(g.b, xs.sum, ga);
     ua = __builtin_fmaf(u.s, ud, ua);
     ua = __builtin_fmaf(u.b, xs.sum, ua);
   }
+}
+
+// The lane slices of x a routed row meets (XSlice: permuted pairs + their sum) depend on the token
+// only, so a workgroup builds them once in LDS instead of once per row: slice sl of token t keeps
+// its pairs as 16-byte blocks xq[(t * kQ + q) * n_sl + sl] (neighbouring lanes read neighbouring
+// blocks) and its sum at xsum[t * n_sl + sl].
+template <int BITS>
+__device__ __forceinline__ void store_xslice_lds(uint4* xq, float* xsum, uint32_t t, uint32_t n_sl, uint32_t sl,
+                                                 const XSlice<BITS>& xs) {
+  constexpr uint32_t kQ = XSlice<BITS>::kPairs / 4;
+#pragma unroll
+  for (uint32_t q = 0; q < kQ; ++q)
+    xq[(t * kQ + q) * n_sl + sl] = make_uint4(xs.p[4 * q], xs.p[4 * q + 1], xs.p[4 * q + 2], xs.p[4 * q + 3]);
+  xsum[t * n_sl + sl] = xs.sum;
+}
+template <int BITS>
+__device__ __forceinline__ XSlice<BITS> load_xslice_lds(const uint4* xq, const float* xsum, uint32_t t, uint32_t n_sl,
+                                                        uint32_t sl) {
+  constexpr uint32_t kQ = XSlice<BITS>::kPairs / 4;
+  XSlice<BITS> xs;
+#pragma unroll
+  for (uint32_t q = 0; q < kQ; ++q) {
+    const uint4 v = xq[(t * kQ + q) * n_sl + sl];
+    xs.p[4 * q] = v.x; xs.p[4 * q + 1] = v.y; xs.p[4 * q + 2] = v.z; xs.p[4 * q + 3] = v.w;
+  }
+  xs.sum = xsum[t * n_sl + sl];
+  return xs;
 }
 
 struct FusedArgs {
@@ -133,37 +171,20 @@ struct FusedArgs {
   int router_mode;
   float limit;
   int maple;  // MapleMoE's rounding points (mf_moe_config::maple_rounding)
+  uint32_t stage_words;  // words of the LDS staging area
+  int xprep;             // the routed rows read x from LDS, permuted and summed once per workgroup
 };
 
 __device__ __forceinline__ void store_u64_agent(unsigned long long* p, unsigned long long v) {
   __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
-__device__ __forceinline__ void give_up(uint32_t* status, uint32_t lane) {
-  if (lane == 0) store_u32_agent(status, 1u);
-}
-
-// One wave gathers n tagged fp32 entries (n % 2 == 0) into dst (LDS).
-__device__ __forceinline__ void poll_tagged_f32(const unsigned long long* src, float* dst,
-                                                uint32_t n, uint32_t epoch, uint32_t lane,
-                                                uint32_t* status) {
-  for (uint32_t base = 0; base < n; base += 2 * kWave) {
-    const uint32_t e0 = base + 2 * lane;
-    const bool in = e0 < n;
-    uint4 v = make_uint4(0, epoch, 0, epoch);
-    for (uint32_t spins = 0;; ++spins) {
-      if (in) v = load_u32x4_agent(src + e0);
-      if (__all(!in || (v.y == epoch && v.w == epoch))) break;
-      if (spins > kSpinLimit) {
-        give_up(status, lane);
-        break;
-      }
-      __builtin_amdgcn_s_sleep(1);
-    }
-    if (in) {
-      dst[e0] = __uint_as_float(v.x);
-      dst[e0 + 1] = __uint_as_float(v.z);
-    }
+// a bounded wait ran out: the status word tells the host, the LDS flag makes this workgroup
+// write NaN instead of a result
+__device__ __forceinline__ void give_up(uint32_t* status, uint32_t* s_fail, uint32_t lane) {
+  if (lane == 0) {
+    store_u32_agent(status, 1u);
+    *s_fail = 1u;
   }
 }
 
@@ -210,47 +231,92 @@ __global__ __launch_bounds__(kFusedThreads) void fused_decode_kernel(const Fused
   // LDS carve-up (the launcher sizes it with fused_lds_bytes)
   uint32_t* s_idx = reinterpret_cast<uint32_t*>(smem);                 // [8*8]
   float* s_w = reinterpret_cast<float*>(smem + 256);                    // [8*8]
+  float* s_sc = reinterpret_cast<float*>(smem + 512);                   // [8*8] selected scores
+  uint32_t* s_flag = reinterpret_cast<uint32_t*>(smem + 768);           // [8] token has a non-finite logit
+  uint32_t* s_fail = reinterpret_cast<uint32_t*>(smem + 800);           // a bounded wait gave up; [1]: selection fallback
   float* s_v = reinterpret_cast<float*>(smem + 1024);                   // [16][64]
   float* s_h1 = reinterpret_cast<float*>(smem + 1024 + 4096);           // [kMaxH1]
-  uint8_t* dyn = smem + 1024 + 4096 + kMaxH1 * 4;
+  uint32_t* s_rank = reinterpret_cast<uint32_t*>(smem + 1024 + 4096 + kMaxH1 * 4);  // [kRankWords]
+  uint8_t* dyn = smem + 1024 + 4096 + kMaxH1 * 4 + kRankWords * 4;
   float* s_lg = reinterpret_cast<float*>(dyn);                          // [MF_MAX_TOKENS][E]
   uint32_t* s_sact = reinterpret_cast<uint32_t*>(dyn + MF_MAX_TOKENS * E * 4);  // [(Fs+4)/2]
   uint32_t* s_acts = s_sact + (((Fs + 4) / 2 + 3) & ~3u);               // [K*F/2], 16-byte aligned
+  uint32_t* s_stage = s_acts + ((K * F / 2 + 3) & ~3u);                 // chunk staging, a.stage_words
   const uint32_t sact_stride = Fs + 4;  // words per token in t_sact
 
-  const uint32_t lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
+  const uint32_t lane = threadIdx.x & 63;
+  // the wave index as a scalar: what derives from it (rows, experts, base addresses) is then
+  // computed once per wave by the scalar unit instead of per lane
+  const uint32_t wv = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const uint32_t G = gridDim.x, wg = blockIdx.x;
-  const uint32_t gw = wv * G + wg;  // consecutive work items land on different CUs
-  const uint32_t total_waves = kFusedWaves * G;
+  // x slices of the routed rows, built once per workgroup (when a.xprep)
+  constexpr uint32_t kEPL = Fmt<BITS>::kElemsPer16B;
+  const uint32_t n_sl = D / kEPL;  // slices per token (the last partial slice, if any, is not kept)
+  uint4* s_xq = reinterpret_cast<uint4*>(s_stage + a.stage_words);
+  float* s_xsum = reinterpret_cast<float*>(s_xq + T * (XSlice<BITS>::kPairs / 4) * n_sl);
 
-  const uint32_t epoch =
-      __hip_atomic_load(&a.epoch[wg], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) + 1u;
-  const uint32_t tag16 = epoch & 0xFFFFu;
-  const unsigned long long etag = static_cast<unsigned long long>(epoch) << 32;
+  // The launch epoch comes out of device memory (a captured graph replays the launch with the same
+  // arguments) and is first needed when a result is tagged.  The load is requested here; every
+  // user takes the value through epoch_now(), whose empty asm statement keeps the compiler from
+  // waiting for it any earlier -- in particular not before the first rows' loads are out.
+  uint32_t epoch_lane_off = 0;
+  asm volatile("" : "+v"(epoch_lane_off));
+  const uint32_t epoch_raw =
+      __hip_atomic_load(&a.epoch[wg] + epoch_lane_off, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  auto epoch_now = [&]() __attribute__((always_inline)) {
+    uint32_t e = epoch_raw;
+    asm volatile("" : "+v"(e));
+    return e + 1u;
+  };
   trace_mark(a, 0);
+  // rank counting selects the top-k when it is cheap enough, else one wave per token sorts
+  const bool rank_count = !S::kGiven && T * E * E <= kRankCountLimit && T * E <= kRankWords;
+  // Who does what while the logits are on their way: the top waves poll for them (n_poll waves),
+  // the waves below those build the x slices, the bottom waves have the rows of stage A.
+  const uint32_t n2 = S::kGiven ? 0 : T * E / 2;  // 16-byte pieces of tagged logits (E % 4 == 0)
+  const uint32_t n_poll = n2 ? ((n2 + kWave - 1) / kWave < 8 ? (n2 + kWave - 1) / kWave : 8) : 0;
+  const uint32_t n_xw = (T * n_sl + kWave - 1) / kWave < kFusedWaves - n_poll - 4
+                            ? (T * n_sl + kWave - 1) / kWave : kFusedWaves - n_poll - 4;
 
   // ------------------------------------------------------------- stage A
+  // Router rows are on the critical path and their logits are gathered by everybody: they go in
+  // chunks of kRouterChunk consecutive rows to the first workgroups (a wave each; the chunk
+  // leaves as one 64-byte store).  The shared expert's rows and the scalar-gate rows are needed
+  // much later; they are dealt one at a time over the waves of the other workgroups (their
+  // dot products are vector-ALU work: spread thin, they cost no workgroup more than a row or two).
   {
     const uint32_t lpr_log2 = Fs ? lanes_per_row_log2_dev(D, Fmt<SBITS>::kElemsPer16B) : 0;
     const uint32_t lpr = 1u << lpr_log2, rpw = 64u >> lpr_log2;
-    const uint32_t n_router = S::kGiven ? 0 : E * T;
+    const uint32_t n_rows_r = S::kGiven ? 0 : E * T;
+    const uint32_t n_rc = (n_rows_r + kRouterChunk - 1) / kRouterChunk;
+    unsigned long long* s_stage64 = reinterpret_cast<unsigned long long*>(s_stage);
+    for (uint32_t ci = wg; ci < n_rc; ci += G) {
+      const uint32_t row = ci * kRouterChunk + wv;
+      if (wv < kRouterChunk && row < n_rows_r) {
+        const uint32_t tok = row / E, e = row % E;
+        const float v = dot_bf16_row(a.router_w + static_cast<size_t>(e) * D,
+                                     a.x + static_cast<size_t>(tok) * D, D, lane, true);
+        if (lane == 0) s_stage64[wv] = (static_cast<unsigned long long>(epoch_now()) << 32) | __float_as_uint(v);
+      }
+      __syncthreads();
+      if (wv == 0 && lane < kRouterChunk && ci * kRouterChunk + lane < n_rows_r)
+        store_u64_agent(&a.t_logits[ci * kRouterChunk + lane], s_stage64[lane]);
+      if (ci + G < n_rc) __syncthreads();  // the staging words are reused
+    }
+    const uint32_t skip = n_rc < G ? n_rc : 0;  // workgroups [0, skip) had router rows
     const uint32_t n_gate = (Fs && a.w_sg) ? T : 0;
     const uint32_t srg = Fs ? (Fs + rpw - 1) / rpw : 0;
-    const uint32_t n_items = n_router + n_gate + T * srg;
-    for (uint32_t item = gw; item < n_items; item += total_waves) {
-      if (item < n_router) {
-        const uint32_t tok = item / E, row = item % E;
-        const float v = dot_bf16_row(a.router_w + static_cast<size_t>(row) * D,
-                                     a.x + static_cast<size_t>(tok) * D, D, lane, true);
-        if (lane == 0) store_u64_agent(&a.t_logits[item], etag | __float_as_uint(v));
-      } else if (item < n_router + n_gate) {
-        const uint32_t tok = item - n_router;
+    const uint32_t n_items = n_gate + T * srg;
+    const uint32_t Gs = G - skip;
+    for (uint32_t item = wg >= skip ? wv * Gs + (wg - skip) : n_items; item < n_items; item += kFusedWaves * Gs) {
+      if (item < n_gate) {
+        const uint32_t tok = item;
         const float v = dot_bf16_row(a.w_sg, a.x + static_cast<size_t>(tok) * D, D, lane, true);
         if (lane < 4)  // the gate rides behind the token's shared activations
           store_u32_agent(&a.t_sact[static_cast<size_t>(tok) * sact_stride + Fs + lane],
-                          (lane == 0 ? static_cast<uint32_t>(f_to_bf16(v)) : 0u) | (tag16 << 16));
+                          (lane == 0 ? static_cast<uint32_t>(f_to_bf16(v)) : 0u) | (epoch_now() << 16));
       } else {
-        const uint32_t it = item - n_router - n_gate;
+        const uint32_t it = item - n_gate;
         const uint32_t srg1 = srg ? srg : 1u;  // no shared expert: this branch is never taken
         const uint32_t tok = it / srg1;
         const uint32_t row = (it % srg1) * rpw + (lane >> lpr_log2);
@@ -272,16 +338,34 @@ __global__ __launch_bounds__(kFusedThreads) void fused_decode_kernel(const Fused
           // dequant_int4.metal:240-245: gate and up narrowed before the activation
           const float rg = round_bf16(g), ru = round_bf16(u);
           store_u32_agent(&a.t_sact[static_cast<size_t>(tok) * sact_stride + row],
-                          static_cast<uint32_t>(f_to_bf16(mf_silu(rg) * ru)) | (tag16 << 16));
+                          static_cast<uint32_t>(f_to_bf16(mf_silu(rg) * ru)) | (epoch_now() << 16));
         }
       }
     }
+    // the x slices of the routed rows
+    if (a.xprep && wv + n_poll + n_xw >= kFusedWaves && wv + n_poll < kFusedWaves) {
+      for (uint32_t q = (wv + n_poll + n_xw - kFusedWaves) * kWave + lane; q < T * n_sl; q += n_xw * kWave) {
+        const uint32_t tok = q / n_sl, sl = q % n_sl;
+        store_xslice_lds<BITS>(s_xq, s_xsum, tok, n_sl, sl,
+                               load_xslice<BITS, kXAligned>(a.x + static_cast<size_t>(tok) * D + sl * kEPL));
+      }
+    }
+  }
+  const uint32_t epoch = epoch_now();
+  const uint32_t tag16 = epoch & 0xFFFFu;
+  for (uint32_t i = threadIdx.x; i < kRankWords; i += kFusedThreads) s_rank[i] = 0u;
+  if (threadIdx.x < MF_MAX_TOKENS * MF_MAX_TOPK) {
+    s_idx[threadIdx.x] = 0u;
+    s_sc[threadIdx.x] = -__builtin_inff();
+  }
+  if (threadIdx.x < MF_MAX_TOKENS + 2) s_flag[threadIdx.x] = 0u;  // + s_fail and the selection's fallback flag behind it
+  {
     // keep every word of the activation buffers recently tagged (see the top)
     const uint32_t ts = epoch % MF_MAX_TOKENS;
     if (ts >= T) {
       const uint32_t gtid = wg * kFusedThreads + threadIdx.x, gthreads = G * kFusedThreads;
-      for (uint32_t i = gtid; i < K * F; i += gthreads)
-        store_u32_agent(&a.t_acts[static_cast<size_t>(ts) * K * F + i], tag16 << 16);
+      for (uint32_t i = gtid * 4; i < K * F; i += gthreads * 4)  // K * F is a multiple of 64
+        store_u32x4_agent(&a.t_acts[static_cast<size_t>(ts) * K * F + i], tag16 << 16);
       for (uint32_t i = gtid; i < (Fs ? sact_stride : 0); i += gthreads)
         store_u32_agent(&a.t_sact[static_cast<size_t>(ts) * sact_stride + i], tag16 << 16);
     }
@@ -290,20 +374,63 @@ __global__ __launch_bounds__(kFusedThreads) void fused_decode_kernel(const Fused
 
   // ------------------------------------------------------- logits, top-k
   if constexpr (!S::kGiven) {
-    if (wv < T)
-      poll_tagged_f32(a.t_logits + static_cast<size_t>(wv) * E, s_lg + wv * E, E, epoch, lane,
-                      a.status);
+    // every lane takes two tagged logits
+    if (wv + n_poll >= kFusedWaves) {
+      for (uint32_t p0 = (kFusedWaves - 1 - wv) * kWave; p0 < n2; p0 += n_poll * kWave) {
+        const uint32_t p = p0 + lane;
+        const bool in = p < n2;
+        uint4 v = make_uint4(0, epoch, 0, epoch);
+        for (uint32_t spins = 0;; ++spins) {
+          if (in) v = load_u32x4_agent(a.t_logits + 2 * p);
+          if (__all(!in || (v.y == epoch && v.w == epoch))) break;
+          if (spins > kSpinLimit) {
+            give_up(a.status, s_fail, lane);
+            break;
+          }
+          __builtin_amdgcn_s_sleep(1);
+        }
+        if (in) {  // rank counting wants no NaN among the scores it compares
+          const bool clean = rank_count && a.router_mode == 0;
+          s_lg[2 * p] = clean ? score_or_ninf(__uint_as_float(v.x)) : __uint_as_float(v.x);
+          s_lg[2 * p + 1] = clean ? score_or_ninf(__uint_as_float(v.z)) : __uint_as_float(v.z);
+        }
+      }
+    }
     __syncthreads();
     trace_mark(a, 2);
-    if (wv < T) {
+    if (rank_count) {
+      if (a.router_mode != 0) {  // full softmax first: the probabilities replace the logits
+        if (wv < T && !full_softmax_probs(s_lg + wv * E, s_lg + wv * E, E, lane)) {
+          if (lane == 0) s_flag[wv] = 1u;  // the token routes nowhere; its scores only have to be comparable
+          for (uint32_t i = lane; i < E; i += kWave) s_lg[wv * E + i] = 0.0f;
+        }
+        __syncthreads();
+      }
+      bool counted = false;
+      if (topk_prefilter_fits(T, E, K, kFusedWaves)) {
+        topk_prefilter(s_lg, s_rank, s_fail + 1, T, E, K, s_idx, s_sc, wv, lane);
+        counted = s_fail[1] == 0u;  // else too many experts passed the prefilter: rank everything
+        if (!counted) {
+          __syncthreads();
+          for (uint32_t i = threadIdx.x; i < kRankWords; i += kFusedThreads) s_rank[i] = 0u;
+          __syncthreads();
+        }
+      }
+      if (!counted) {
+        topk_rank_count(s_lg, s_rank, T, E, wv, lane, kFusedWaves);
+        __syncthreads();
+        topk_rank_emit(s_lg, s_rank, T, E, K, s_idx, s_sc, threadIdx.x, kFusedThreads);
+      }
+      if (a.router_mode != 0) {  // a token with a non-finite logit routes nowhere (maple_moe.metal:62-119)
+        __syncthreads();
+        if (threadIdx.x < T * K && s_flag[threadIdx.x / K]) s_idx[threadIdx.x] = E;
+      }
+      // the routing weights follow after stage B: nothing needs them before stage C
+    } else if (wv < T) {
       if (a.router_mode == 0) topk_select_fast(s_lg + wv * E, E, K, s_idx + wv * K, s_w + wv * K, lane);
       else topk_full_softmax_fast(s_lg + wv * E, s_lg + wv * E, E, K, s_idx + wv * K, s_w + wv * K, lane);
     }
     __syncthreads();
-    if (wg == 0 && threadIdx.x < T * K) {
-      if (a.out_idx) a.out_idx[threadIdx.x] = s_idx[threadIdx.x];
-      if (a.out_w) a.out_w[threadIdx.x] = s_w[threadIdx.x];
-    }
   } else {  // routing written by an earlier launch on the stream (a family router): read, never written
     trace_mark(a, 2);
     if (threadIdx.x < T * K) {
@@ -315,74 +442,79 @@ __global__ __launch_bounds__(kFusedThreads) void fused_decode_kernel(const Fused
   trace_mark(a, 3);
 
   // ------------------------------------------------------------- stage B
+  // Every workgroup takes a run of consecutive units (rpw rows of one routed slot), its waves
+  // take them in turn; gate and up sums meet in LDS, the first threads turn them into
+  // activations (one exp and one division per thread instead of per wave) and the run leaves as
+  // one contiguous piece.
   {
-    const uint32_t lpr_log2 = lanes_per_row_log2_dev(D, Fmt<BITS>::kElemsPer16B);
+    const uint32_t lpr_log2 = lanes_per_row_log2_dev(D, kEPL);
     const uint32_t lpr = 1u << lpr_log2, rpw = 64u >> lpr_log2;
-    const uint32_t rgf = (F + rpw - 1) / rpw;
+    const uint32_t rgf = (F + rpw - 1) / rpw;   // units per (token, slot)
     const uint32_t n_items = T * K * rgf;
-    // a row is one 16-byte step per lane and waves have more than one item.  A shape-specialised
-    // kernel compiles the path in only when a full grid of 256 workgroups would have such waves
-    // (on a smaller grid it then simply takes the general path).
-    constexpr uint32_t kStaticRpw = static_rows_per_wave(S::kStatic ? S::D : 64u, Fmt<BITS>::kElemsPer16B);
-    constexpr bool kMayHoist =
-        !S::kStatic || S::T * S::K * ((S::F + kStaticRpw - 1) / kStaticRpw) > kFusedWaves * 256u;
-    const bool one_step = kMayHoist && lpr * Fmt<BITS>::kElemsPer16B >= D && n_items > total_waves;
-    XSlice<BITS> xs_cur{};
-    uint32_t xs_tok = 0xFFFFFFFFu;
-    for (uint32_t item = gw; item < n_items; item += total_waves) {
+    uint32_t per_wg = (n_items + G - 1) / G;
+    per_wg = (per_wg + kFusedWaves - 1) / kFusedWaves * kFusedWaves;
+    const uint32_t first = wg * per_wg;
+    const uint32_t last = first + per_wg < n_items ? first + per_wg : n_items;
+    float* s_gu = reinterpret_cast<float*>(s_stage);  // (gate sum, up sum) per staged row
+    const uint32_t sub = lane & (lpr - 1), rloc = lane >> lpr_log2;
+    const uint32_t ng = D / kGroup;
+    const size_t rb = static_cast<size_t>(D) * Store<BITS>::kBits / 8;
+    for (uint32_t item = first + wv; item < last; item += kFusedWaves) {
       const uint32_t pair = item / rgf;
-      const uint32_t row = (item % rgf) * rpw + (lane >> lpr_log2);
-      const uint32_t sub = lane & (lpr - 1);
+      const uint32_t row = (item % rgf) * rpw + rloc;
       const bool ok = row < F;
-      const uint32_t expert = s_idx[pair];
-      uint32_t* dst = &a.t_acts[static_cast<size_t>(pair) * F + (ok ? row : 0)];
-      if (expert >= E) {  // router sentinel: the slot contributes nothing
-        if (ok && sub == 0) store_u32_agent(dst, tag16 << 16);
-        continue;
-      }
-      const uint8_t* blob = a.expert_base + static_cast<size_t>(expert) * a.expert_stride;
-      const size_t r = ok ? row : 0;
-      const uint32_t ng = D / kGroup;
-      const size_t rb = static_cast<size_t>(D) * Store<BITS>::kBits / 8;
+      const uint32_t expert = __builtin_amdgcn_readfirstlane(s_idx[pair]);
       float ga = 0.0f, ua = 0.0f;
-      if (one_step) {
-        // the lane's slice of x depends on the token only: a wave with several items of one
-        // token builds it once (same operations as gate_up_partial, one step)
-        const uint32_t e0 = sub * Fmt<BITS>::kElemsPer16B, tok = pair / K;
-        if (tok != xs_tok) {
-          if (e0 < D) xs_cur = load_xslice<BITS, kXAligned>(a.x + static_cast<size_t>(tok) * D + e0);
-          xs_tok = tok;
-        }
-        if (ok && e0 < D) {
-          const Chunk<BITS> gc = load_chunk<BITS>(blob + a.off.gate_w + r * rb,
-                                                  reinterpret_cast<const uint16_t*>(blob + a.off.gate_s) + r * ng,
-                                                  reinterpret_cast<const uint16_t*>(blob + a.off.gate_b) + r * ng, e0);
-          const Chunk<BITS> uc = load_chunk<BITS>(blob + a.off.up_w + r * rb,
-                                                  reinterpret_cast<const uint16_t*>(blob + a.off.up_s) + r * ng,
-                                                  reinterpret_cast<const uint16_t*>(blob + a.off.up_b) + r * ng, e0);
-          const float gd = codes_dot<BITS>(gc.codes, xs_cur), ud = codes_dot<BITS>(uc.codes, xs_cur);
+      if (expert < E && ok) {  // a router sentinel contributes nothing: its sums stay 0
+        const uint8_t* blob = a.expert_base + static_cast<size_t>(expert) * a.expert_stride;
+        const uint8_t* gw = blob + a.off.gate_w + row * rb;
+        const uint8_t* uw = blob + a.off.up_w + row * rb;
+        const uint16_t* gs = reinterpret_cast<const uint16_t*>(blob + a.off.gate_s) + static_cast<size_t>(row) * ng;
+        const uint16_t* gb = reinterpret_cast<const uint16_t*>(blob + a.off.gate_b) + static_cast<size_t>(row) * ng;
+        const uint16_t* us = reinterpret_cast<const uint16_t*>(blob + a.off.up_s) + static_cast<size_t>(row) * ng;
+        const uint16_t* ub = reinterpret_cast<const uint16_t*>(blob + a.off.up_b) + static_cast<size_t>(row) * ng;
+        const uint32_t tok = pair / K;
+        for (uint32_t e0 = sub * kEPL; e0 < D; e0 += lpr * kEPL) {  // the steps of gate_up_partial
+          const Chunk<BITS> gc = load_chunk<BITS>(gw, gs, gb, e0);
+          const Chunk<BITS> uc = load_chunk<BITS>(uw, us, ub, e0);
+          issue_fence();
+          const XSlice<BITS> xs = a.xprep ? load_xslice_lds<BITS>(s_xq, s_xsum, tok, n_sl, e0 / kEPL)
+                                          : load_xslice<BITS, kXAligned>(a.x + static_cast<size_t>(tok) * D + e0);
+          const float gd = codes_dot<BITS>(gc.codes, xs), ud = codes_dot<BITS>(uc.codes, xs);
           ga = __builtin_fmaf(gc.s, gd, ga);
-          ga = __builtin_fmaf(gc.b, xs_cur.sum, ga);
+          ga = __builtin_fmaf(gc.b, xs.sum, ga);
           ua = __builtin_fmaf(uc.s, ud, ua);
-          ua = __builtin_fmaf(uc.b, xs_cur.sum, ua);
+          ua = __builtin_fmaf(uc.b, xs.sum, ua);
         }
-      } else if (ok)
-        gate_up_partial<BITS>(blob + a.off.gate_w + r * rb,
-                              reinterpret_cast<const uint16_t*>(blob + a.off.gate_s) + r * ng,
-                              reinterpret_cast<const uint16_t*>(blob + a.off.gate_b) + r * ng,
-                              blob + a.off.up_w + r * rb,
-                              reinterpret_cast<const uint16_t*>(blob + a.off.up_s) + r * ng,
-                              reinterpret_cast<const uint16_t*>(blob + a.off.up_b) + r * ng,
-                              a.x + static_cast<size_t>(pair / K) * D, D, sub, lpr, ga, ua);
-      float g = group_sum(ga, static_cast<int>(lpr));
-      float u = group_sum(ua, static_cast<int>(lpr));
-      if (ok && sub == 0) {
-        // moe.metal:27-34, 528; maple_moe.metal:153-164
-        store_u32_agent(dst, static_cast<uint32_t>(routed_activation(g, u, a.limit, a.maple != 0)) | (tag16 << 16));
       }
+      const float g = group_sum(ga, static_cast<int>(lpr));
+      const float u = group_sum(ua, static_cast<int>(lpr));
+      if (sub == 0) {
+        float* dst = s_gu + 2 * ((item - first) * rpw + rloc);
+        dst[0] = g;
+        dst[1] = u;
+      }
+    }
+    __syncthreads();
+    // staged row (item - first) * rpw + r is activation (item % rgf) * rpw + r of pair item / rgf
+    const uint32_t n_words = first < last ? (last - first) * rpw : 0;
+    for (uint32_t i = threadIdx.x; i < n_words; i += kFusedThreads) {
+      const uint32_t item = first + i / rpw, row = (item % rgf) * rpw + i % rpw;
+      // moe.metal:27-34, 528; maple_moe.metal:153-164
+      const uint32_t word =
+          static_cast<uint32_t>(routed_activation(s_gu[2 * i], s_gu[2 * i + 1], a.limit, a.maple != 0)) | (tag16 << 16);
+      if (row < F) store_u32_agent(&a.t_acts[static_cast<size_t>(item / rgf) * F + row], word);
     }
   }
   trace_mark(a, 4);
+  // routing weights of token t by the wave 15 - t (rank counting left scores, not weights)
+  if (rank_count && wv + T >= kFusedWaves) {
+    const uint32_t tok = kFusedWaves - 1 - wv;
+    const float my_score = lane < K ? s_sc[tok * K + lane] : -__builtin_inff();
+    float wgt = a.router_mode == 0 ? topk_weight_of_rank<0>(my_score, K) : topk_weight_of_rank<1>(my_score, K);
+    if (s_flag[tok]) wgt = 0.0f;  // maple_moe.metal:62-119: a non-finite logit routes nowhere
+    if (lane < K) s_w[tok * K + lane] = wgt;
+  }
 
   // ------------------------------------------------------------- stage C
   const uint32_t lpr_log2 = lanes_per_row_log2_dev(F, Fmt<BITS>::kElemsPer16B);
@@ -407,7 +539,7 @@ __global__ __launch_bounds__(kFusedThreads) void fused_decode_kernel(const Fused
       const uint32_t unit = wg * ub + unit_local;
       if (unit_local < ub && unit < rg_per_tok) {
         const uint32_t row = unit * rpw + (lane >> lpr_log2);
-        const uint32_t expert = s_idx[tok * K + slot];
+        const uint32_t expert = __builtin_amdgcn_readfirstlane(s_idx[tok * K + slot]);
         if (row < D && expert < E && sub * Fmt<BITS>::kElemsPer16B < F) {
           const uint8_t* blob = a.expert_base + static_cast<size_t>(expert) * a.expert_stride;
           pre = load_chunk<BITS>(blob + a.off.down_w + row * rb,
@@ -463,7 +595,7 @@ __global__ __launch_bounds__(kFusedThreads) void fused_decode_kernel(const Fused
                                 (v1.x ^ want) | (v1.y ^ want) | (v1.z ^ want) | (v1.w ^ want);
           if (__all((diff >> 16) == 0)) break;
           if (spins > kSpinLimit) {
-            give_up(a.status, lane);
+            give_up(a.status, s_fail, lane);
             break;
           }
           __builtin_amdgcn_s_sleep(1);
@@ -528,7 +660,7 @@ __global__ __launch_bounds__(kFusedThreads) void fused_decode_kernel(const Fused
       if (active) {
         const uint32_t row = unit * rpw + (lane >> lpr_log2);
         const uint32_t pair = tok * K + slot;
-        const uint32_t expert = s_idx[pair];
+        const uint32_t expert = __builtin_amdgcn_readfirstlane(s_idx[pair]);
         float part = 0.0f;
         if (row < D && expert < E) {
           const uint8_t* blob = a.expert_base + static_cast<size_t>(expert) * a.expert_stride;
@@ -552,26 +684,60 @@ __global__ __launch_bounds__(kFusedThreads) void fused_decode_kernel(const Fused
           float acc = Fs ? s_h1[round * rows_per_round + threadIdx.x] : 0.0f;  // residual first
           for (uint32_t k = 0; k < K; ++k)
             if (s_idx[tok * K + k] < E) acc = acc + s_v[(ul * K + k) * kWave + rr];
-          const uint16_t yb = f_to_bf16(acc);
+          const bool failed = *s_fail != 0u;  // a wait gave up: no result, and hidden stays as it is
+          const uint16_t yb = failed ? static_cast<uint16_t>(0x7FC0u) : f_to_bf16(acc);
           a.y[o] = yb;
-          if (a.hidden)  // residual_add_fp16, utility.metal:83-92
+          if (a.hidden && !failed)  // residual_add_fp16, utility.metal:83-92
             a.hidden[o] = f_to_bf16(bf16_to_f(a.hidden[o]) + bf16_to_f(yb));
         }
       }
       __syncthreads();
     }
   }
+  if constexpr (!S::kGiven) {
+    if (wg == 0 && threadIdx.x < T * K) {  // s_w was complete before stage C's first barrier
+      if (a.out_idx) a.out_idx[threadIdx.x] = s_idx[threadIdx.x];
+      if (a.out_w) a.out_w[threadIdx.x] = s_w[threadIdx.x];
+    }
+  }
   if (threadIdx.x == 0) a.epoch[wg] = epoch;
   trace_mark(a, 6);
 }
 
-size_t fused_lds_bytes(const mf_moe_config& c) {
-  return 1024 + 4096 + kMaxH1 * 4 + static_cast<size_t>(MF_MAX_TOKENS) * c.num_experts * 4 +
-         2 * static_cast<size_t>(c.shared_f) + 128 + 2 * static_cast<size_t>(c.top_k) * c.f;
+// words of the LDS staging area: a chunk of router logits in stage A, the (gate, up) sums of a
+// workgroup's run of routed rows in stage B
+static uint32_t fused_stage_words(const mf_moe_config& c, uint32_t num_cu, uint32_t t) {
+  const uint32_t epl = c.bits == MF_BITS_4 ? 32 : 64;
+  const uint32_t rpw = 64u >> lanes_per_row_log2_dev(c.d, epl);
+  const uint32_t rgf = (c.f + rpw - 1) / rpw;
+  uint32_t per_wg = (t * c.top_k * rgf + num_cu - 1) / num_cu;
+  per_wg = (per_wg + kFusedWaves - 1) / kFusedWaves * kFusedWaves;
+  const uint32_t words = 2 * per_wg * rpw;
+  return words < 64 ? 64 : (words + 3) & ~3u;
+}
+// words of the x slices of the routed rows (permuted pairs + sum per slice)
+static uint32_t fused_xprep_words(const mf_moe_config& c, uint32_t t) {
+  const uint32_t epl = c.bits == MF_BITS_4 ? 32 : 64;
+  return t * (c.d / epl) * (epl / 2 + 1);
+}
+static size_t fused_lds_base(const mf_moe_config& c, uint32_t num_cu, uint32_t t) {
+  const size_t sact_words = ((c.shared_f + 4) / 2 + 3) & ~size_t(3);
+  const size_t acts_words = (static_cast<size_t>(c.top_k) * c.f / 2 + 3) & ~size_t(3);
+  return 1024 + 4096 + kMaxH1 * 4 + kRankWords * 4 + static_cast<size_t>(MF_MAX_TOKENS) * c.num_experts * 4 +
+         4 * (sact_words + acts_words + fused_stage_words(c, num_cu, t));
+}
+constexpr size_t kFusedLdsLimit = 150 * 1024;
+// the x slices are kept in LDS when they fit beside everything else
+static bool fused_xprep(const mf_moe_config& c, uint32_t num_cu, uint32_t t) {
+  return fused_lds_base(c, num_cu, t) + 4 * static_cast<size_t>(fused_xprep_words(c, t)) <= kFusedLdsLimit;
+}
+size_t fused_lds_bytes(const mf_moe_config& c, uint32_t num_cu, uint32_t t) {
+  const size_t base = fused_lds_base(c, num_cu, t);
+  return fused_xprep(c, num_cu, t) ? base + 4 * static_cast<size_t>(fused_xprep_words(c, t)) : base;
 }
 
 bool fused_supported(const mf_moe& h, const mf_moe_layer_weights& w, const void* x, const void* y,
-                     const void* hidden) {
+                     const void* hidden, uint32_t t) {
   const mf_moe_config& c = h.cfg;
   if (c.num_experts % 4 != 0) return false;  // tagged logits are read two entries per lane
   const bool combo = (c.bits == MF_BITS_4 && (!c.shared_f || c.shared_bits == MF_BITS_4)) ||
@@ -579,7 +745,7 @@ bool fused_supported(const mf_moe& h, const mf_moe_layer_weights& w, const void*
                                               c.shared_bits == MF_BITS_2)) ||
                      (c.bits == MF_BITS_TERNARY && (!c.shared_f || c.shared_bits == MF_BITS_4));
   if (!combo || c.d % 8 != 0) return false;
-  if (fused_lds_bytes(c) > 150 * 1024) return false;
+  if (fused_lds_base(c, static_cast<uint32_t>(h.ctx->num_cu), t) > kFusedLdsLimit) return false;
   {  // rows of one token a workgroup owns must fit the h1 array
     const uint32_t epl = c.bits == MF_BITS_4 ? 32 : 64;
     const uint32_t rpw = 64u >> lanes_per_row_log2_dev(c.f, epl);
@@ -635,7 +801,10 @@ hipError_t launch_fused_decode(hipStream_t s, const mf_moe& h, const mf_moe_laye
   a.limit = c.swiglu_limit;
   a.maple = static_cast<int>(c.maple_rounding);
   const dim3 grid(static_cast<uint32_t>(h.ctx->num_cu)), block(kFusedThreads);
-  const size_t lds = fused_lds_bytes(c);
+  const uint32_t num_cu = static_cast<uint32_t>(h.ctx->num_cu);
+  const size_t lds = fused_lds_bytes(c, num_cu, t);
+  a.stage_words = fused_stage_words(c, num_cu, t);
+  a.xprep = fused_xprep(c, num_cu, t) ? 1 : 0;
 #define MF_FUSED(B, SB, SHAPE)                                                                 \
   do {                                                                                         \
     auto kern = fused_decode_kernel<B, SB, SHAPE>;                                             \

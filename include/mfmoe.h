@@ -163,6 +163,20 @@ mf_status mf_shared_expert(mf_ctx* ctx, mf_stream stream, const uint16_t* x, mf_
                            uint32_t t, uint16_t* y, uint16_t* scratch_act,
                            size_t scratch_act_bytes);
 
+/* mf_shared_expert for callers that cannot allocate device memory and bring no scratch buffer:
+ * code under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc.  It has no
+ * counterpart in the reference (SharedExpertInt4.encode takes the caller's scratch buffer,
+ * SharedExpertInt4.swift:76-78).  The activation vector act[t,f] lives in a device array that is
+ * part of the library image (MF_STATIC_ACT_ELEMS bf16 = 512 KiB, held on every GPU the library
+ * runs on until the process ends); the call launches the kernels of mf_shared_expert and calls no
+ * hipMalloc / hipFree.  Same arguments, checks and results (bit for bit) as mf_shared_expert;
+ * t * f > MF_STATIC_ACT_ELEMS returns MF_ERR_SCRATCH_TOO_SMALL and launches nothing.  All calls on
+ * one GPU share the array: calls that overlap on one GPU (two streams, two threads) race. */
+#define MF_STATIC_ACT_ELEMS (MF_MAX_TOKENS * 32768u)
+mf_status mf_shared_expert_static(mf_ctx* ctx, mf_stream stream, const uint16_t* x, mf_qtensor gate,
+                                  mf_qtensor up, mf_qtensor down, mf_bits bits, uint32_t d, uint32_t f,
+                                  uint32_t t, uint16_t* y);
+
 /* ---------------------------------------------------------- MoE operator */
 
 /* Shape/activation specialisation of one operator instance: MoE.init

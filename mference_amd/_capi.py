@@ -15,6 +15,7 @@ GROUP_SIZE = 64
 MAX_TOKENS = 8
 MAX_TOPK = 8
 MAX_EXPERTS = 512
+STATIC_ACT_ELEMS = MAX_TOKENS * 32768  # MF_STATIC_ACT_ELEMS
 
 BITS_TERNARY, BITS_2, BITS_4 = 1, 2, 4
 ROUTER_TOPK_SOFTMAX, ROUTER_FULL_SOFTMAX = 0, 1
@@ -79,6 +80,7 @@ SIGNATURES = {
     "mf_residual_rmsnorm": (_I, [_P, _P, _P, _P, _P, _P, _U32, _U32, C.c_float]),
     "mf_shared_expert": (_I, [_P, _P, _P, QTensor, QTensor, QTensor, _I, _U32, _U32, _U32, _P, _P,
                               _SZ]),
+    "mf_shared_expert_static": (_I, [_P, _P, _P, QTensor, QTensor, QTensor, _I, _U32, _U32, _U32, _P]),
     "mf_moe_create": (_I, [_P, C.POINTER(MoEConfig), C.POINTER(_P)]),
     "mf_moe_destroy": (None, [_P]),
     "mf_moe_router": (_I, [_P, _P, _P, _P, _U32, _U32, _P, _P, _P]),

@@ -11,7 +11,7 @@ CSRC = os.path.join(HERE, "csrc")
 OBJ = os.path.join(HERE, "build")
 LIB = os.path.join(HERE, "libmfmoe.so")
 SOURCES = ["format.hip", "gemv.hip", "router.hip", "router_family.hip", "moe_decode.hip", "moe_fused.hip",
-           "moe_prefill.hip", "api.hip"]
+           "moe_prefill.hip", "static_scratch.hip", "api.hip"]
 
 FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC",

@@ -83,6 +83,10 @@ mf_status mf_ctx_create(int device, mf_ctx** out) {
   if (!ctx) return MF_ERR_OUT_OF_MEMORY;
   ctx->device = device;
   ctx->num_cu = prop.multiProcessorCount;
+  if (mf::static_scratch_init(device) != hipSuccess) {  // mf_shared_expert_static's array on this GPU
+    delete ctx;
+    return MF_ERR_NO_DEVICE;
+  }
   *out = ctx;
   return MF_OK;
 }

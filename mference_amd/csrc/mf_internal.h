@@ -102,6 +102,9 @@ hipError_t launch_select_inkling(hipStream_t s, const float* logits, const float
 hipError_t launch_select_scaled_softmax(hipStream_t s, const float* logits, const uint16_t* expert_scale,
                                         uint32_t e, uint32_t k, uint32_t t, uint32_t* idx, float* w);
 
+// static_scratch.hip: this device's address of the library's built-in scratch array (device = current device)
+hipError_t static_scratch_init(int device);
+
 // moe_decode.hip
 hipError_t launch_phase1(hipStream_t s, const mf_moe_config& cfg, const void* base, size_t stride,
                          const mf_expert_offsets& off, const uint32_t* idx, const uint16_t* x,

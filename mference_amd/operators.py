@@ -207,6 +207,20 @@ class SharedExpertInt4:
             scratch_act.numel() * scratch_act.element_size()), self.context.handle)
 
 
+    def encode_static(self, x: torch.Tensor, gate: QuantizedTensor, up: QuantizedTensor,
+                      down: QuantizedTensor, y: torch.Tensor, t: int = 1, stream=None) -> None:
+        """The same operator for callers that cannot allocate and bring no scratch: the
+        activations go through the library's built-in device array (mf_shared_expert_static;
+        t * f <= STATIC_ACT_ELEMS, calls on one GPU must not overlap)."""
+        if not (gate.rows == up.rows and gate.n == up.n and down.rows == gate.n
+                and down.n == gate.rows):
+            raise MfError(-2, f"gate=({gate.rows},{gate.n}) up=({up.rows},{up.n}) "
+                              f"down=({down.rows},{down.n})")
+        check(_capi.lib().mf_shared_expert_static(
+            self.context.handle, _stream(stream), _ptr(x), gate.c(), up.c(), down.c(), gate.bits,
+            gate.n, gate.rows, t, _ptr(y)), self.context.handle)
+
+
 class FamilyRouters:
     """The family-specific routers of the reference's operator classes, stand-alone: every call
     runs the router GEMV into the caller's fp32 `logits` buffer [t, rows] and then the selection.

@@ -235,6 +235,14 @@ __device__ __forceinline__ float score_or_ninf(float x) {
   const float ninf = -__builtin_inff();
   return (x > ninf) ? x : ninf;
 }
+// a score (no NaN) as an unsigned number that orders like the score; -0 and +0 get one key
+__device__ __forceinline__ uint32_t score_key(float x) {
+  const uint32_t b = __float_as_uint(x + 0.0f);
+  return b ^ ((b >> 31) ? 0xFFFFFFFFu : 0x80000000u);
+}
+__device__ __forceinline__ float key_score(uint32_t k) {
+  return __uint_as_float(k ^ ((k >> 31) ? 0x80000000u : 0xFFFFFFFFu));
+}
 // does (q, j) beat (v, i)?  q, v hold no NaN
 __device__ __forceinline__ uint32_t beats(float q, uint32_t j, float v, uint32_t i) {
   return (q > v || (q == v && j < i)) ? 1u : 0u;
@@ -303,7 +311,7 @@ __device__ __forceinline__ void topk_rank_emit(const float* vals, const uint32_t
 // More than 64 of them (many equal scores, or fewer than k finite ones) raise *fallback and the
 // caller counts ranks over everything instead.
 // scr: LDS words, zero on entry: [0, 256) sub-block maxima, [256, 264) list lengths per token,
-// [512, 512 + t_count * 128) the lists of (score bits, index).  Contains workgroup barriers: all
+// [512, 512 + t_count * 128) the lists of (~index, score key).  Contains workgroup barriers: all
 // threads call it.
 constexpr uint32_t kPrefilterScratchWords = 512 + MF_MAX_TOKENS * 128;
 __device__ __forceinline__ bool topk_prefilter_fits(uint32_t t_count, uint32_t e, uint32_t k, uint32_t nwaves) {
@@ -331,16 +339,22 @@ __device__ __forceinline__ void topk_prefilter(const float* vals, uint32_t* scr,
   }
   __syncthreads();
   if (mine) {
-    // L: the sub-block maximum of rank k - 1 (ranked like the scores, so exactly one lane has it)
+    // L: the k-th largest sub-block maximum = the largest maximum that at least k maxima reach
+    // (equal maxima need no tie rule here: only the value matters)
     const float* sm = smax + t * nsb;
     const float ml = lane < nsb ? sm[lane] : ninf;
-    uint32_t r = 0;
-    for (uint32_t j = 0; j < nsb; j += 4) {
-      const float4 q = *reinterpret_cast<const float4*>(sm + j);
-      r += beats(q.x, j, ml, lane) + beats(q.y, j + 1, ml, lane) + beats(q.z, j + 2, ml, lane) + beats(q.w, j + 3, ml, lane);
+    uint32_t ge = 0;
+    for (uint32_t j0 = 0; j0 < nsb; j0 += 16) {  // four LDS reads in flight; maxima past nsb read as -inf
+      float4 q[4];
+#pragma unroll
+      for (uint32_t u = 0; u < 4; ++u)
+        q[u] = j0 + 4 * u < nsb ? *reinterpret_cast<const float4*>(sm + j0 + 4 * u) : make_float4(ninf, ninf, ninf, ninf);
+#pragma unroll
+      for (uint32_t u = 0; u < 4; ++u) ge += (q[u].x >= ml) + (q[u].y >= ml) + (q[u].z >= ml) + (q[u].w >= ml);
     }
-    const unsigned long long km = __ballot(lane < nsb && r == k - 1);
-    const float L = readlane_f(ml, __ffsll(static_cast<long long>(km)) - 1);
+    // lanes past nsb hold -inf and count the -inf padding: they never raise the maximum below
+    float L = (lane < nsb && ge >= k) ? ml : ninf;
+    L = wave_max(L);
     // the experts that reach L join their token's list (in any order: the list is ranked below)
     const bool c = v >= L;
     const unsigned long long cm = __ballot(c);
@@ -350,9 +364,10 @@ __device__ __forceinline__ void topk_prefilter(const float* vals, uint32_t* scr,
     base = static_cast<uint32_t>(__builtin_amdgcn_readfirstlane(static_cast<int>(base)));
     const uint32_t pos = base + __builtin_amdgcn_mbcnt_hi(static_cast<uint32_t>(cm >> 32),
                                                           __builtin_amdgcn_mbcnt_lo(static_cast<uint32_t>(cm), 0u));
-    if (c && pos < kWave) {
-      lists[t * 128 + 2 * pos] = __float_as_uint(v);
-      lists[t * 128 + 2 * pos + 1] = i;
+    if (c && pos < kWave) {  // (score as an unsigned key that sorts like the score, ~index): one 64-bit
+                             // comparison then says "beats", ties to the lower index included
+      lists[t * 128 + 2 * pos] = ~i;
+      lists[t * 128 + 2 * pos + 1] = score_key(v);
     }
   }
   __syncthreads();
@@ -361,17 +376,26 @@ __device__ __forceinline__ void topk_prefilter(const float* vals, uint32_t* scr,
     if (n > kWave) {
       if (lane == 0) *fallback = 1u;
     } else {
-      const uint2* lst = reinterpret_cast<const uint2*>(lists + wv * 128);
-      const uint2 me = lane < n ? lst[lane] : make_uint2(0u, 0u);
-      const float vc = __uint_as_float(me.x);
+      const unsigned long long* lst = reinterpret_cast<const unsigned long long*>(lists + wv * 128);
+      const unsigned long long me = lane < n ? lst[lane] : 0ull;
       uint32_t r = 0;
-      for (uint32_t j = 0; j < n; ++j) {
-        const uint2 o = lst[j];
-        r += beats(__uint_as_float(o.x), o.y, vc, me.y);
+      for (uint32_t j0 = 0; j0 < n; j0 += 8) {  // eight entries per step, their LDS reads in flight together
+        uint4 o[4];
+#pragma unroll
+        for (uint32_t u = 0; u < 4; ++u) o[u] = *reinterpret_cast<const uint4*>(lists + wv * 128 + 2 * (j0 + 2 * u));
+#pragma unroll
+        for (uint32_t u = 0; u < 4; ++u) {  // entries past the list's end beat nothing
+          const uint32_t j = j0 + 2 * u;
+          const unsigned long long k0 = (static_cast<unsigned long long>(o[u].y) << 32) | o[u].x;
+          const unsigned long long k1 = (static_cast<unsigned long long>(o[u].w) << 32) | o[u].z;
+          r += (j < n && k0 > me ? 1u : 0u) + (j + 1 < n && k1 > me ? 1u : 0u);
+        }
       }
+      const float vc = key_score(static_cast<uint32_t>(me >> 32));
+      const uint32_t ic = ~static_cast<uint32_t>(me);
       if (lane < n && r < k) {
         const bool valid = vc > ninf;
-        idx[wv * k + r] = valid ? me.y : 0u;
+        idx[wv * k + r] = valid ? ic : 0u;
         sc[wv * k + r] = valid ? vc : ninf;
       }
     }

@@ -681,9 +681,19 @@ __global__ __launch_bounds__(kFusedThreads) void fused_decode_kernel(const Fused
         const uint32_t row = u2 * rpw + rr;
         if (u2 < rg_per_tok && row < D) {
           const size_t o = static_cast<size_t>(tok) * D + row;
-          float acc = Fs ? s_h1[round * rows_per_round + threadIdx.x] : 0.0f;  // residual first
-          for (uint32_t k = 0; k < K; ++k)
-            if (s_idx[tok * K + k] < E) acc = acc + s_v[(ul * K + k) * kWave + rr];
+          // the K weighted values first (independent LDS reads: one round of latency, not K),
+          // then the sum in rank order, residual first
+          float vk[MF_MAX_TOPK];
+          bool live[MF_MAX_TOPK];
+#pragma unroll
+          for (uint32_t k = 0; k < MF_MAX_TOPK; ++k) {
+            live[k] = k < K && s_idx[tok * K + (k < K ? k : 0)] < E;
+            vk[k] = s_v[(ul * K + (k < K ? k : 0)) * kWave + rr];
+          }
+          float acc = Fs ? s_h1[round * rows_per_round + threadIdx.x] : 0.0f;
+#pragma unroll
+          for (uint32_t k = 0; k < MF_MAX_TOPK; ++k)
+            if (live[k]) acc = acc + vk[k];
           const bool failed = *s_fail != 0u;  // a wait gave up: no result, and hidden stays as it is
           const uint16_t yb = failed ? static_cast<uint16_t>(0x7FC0u) : f_to_bf16(acc);
           a.y[o] = yb;

@@ -64,13 +64,9 @@ def build_stack(ctx, w, layers, device):
     quantizer into resident expert blobs."""
     import torch
     from mference_amd import operators as ops
-    from oracle import mf_oracle as O  # blob layout helper only (host arithmetic)
 
     quant = ops.Quantization(ctx)
-    off_h, _, stride = O.blob_layout(w["d"], w["f"], w["bits"])
-    off = ops.MoEExpertOffsets()
-    for name, _ in off._fields_:
-        setattr(off, name, getattr(off_h, name))
+    off, _, stride = ops.expert_blob_layout(w["d"], w["f"], w["bits"])
     stack = []
     E, D, F = w["e"], w["d"], w["f"]
     for l in range(layers):

@@ -306,6 +306,16 @@ mf_status mf_moe_phase2(mf_moe* h, mf_stream stream, const void* expert_base,
                         const uint32_t* idx, const float* w, const uint16_t* acts,
                         const uint16_t* residual, uint32_t t, uint16_t* y);
 
+/* Byte offsets of the nine sub-tensors of one routed expert of hidden size d and intermediate
+ * size f, laid out back to back in the order the reference's repacker writes them -- gate
+ * {codes, scales, biases}, up {...}, down {...} (MferenceRepack/Core/Planning/RepackPlanner.swift:
+ * 544-712; read back by Model.routedExpertOffsets, Runtime/Inference/ModelExpertIO.swift:20-35);
+ * ternary experts store no biases (their bias offsets read 0).  blob_bytes: size of one expert;
+ * stride: that size rounded up to `align` (the reference rounds to a 16 KiB page).  Host
+ * arithmetic only; for callers that build a resident pool themselves (synthetic weights, tests). */
+mf_status mf_expert_blob_layout(uint32_t d, uint32_t f, mf_bits bits, uint32_t align, mf_expert_offsets* offsets,
+                                size_t* blob_bytes, size_t* stride);
+
 /* Everything one layer reads. */
 typedef struct {
   const uint16_t* router_w;   /* bf16 [num_experts, d]; NULL: the routing is the caller's -- the layer

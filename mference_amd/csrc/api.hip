@@ -186,6 +186,33 @@ mf_status mf_shared_expert(mf_ctx* ctx, mf_stream stream, const uint16_t* x, mf_
   return MF_OK;
 }
 
+mf_status mf_expert_blob_layout(uint32_t d, uint32_t f, mf_bits bits, uint32_t align, mf_expert_offsets* offsets,
+                                size_t* blob_bytes, size_t* stride) {
+  if (!offsets) return MF_ERR_INVALID_ARGUMENT;
+  if (!bits_ok(bits)) return MF_ERR_UNSUPPORTED_BITS;
+  if (d == 0 || f == 0 || d % MF_GROUP_SIZE != 0 || f % MF_GROUP_SIZE != 0) return MF_ERR_DIMENSION_MISMATCH;
+  if (align == 0) return MF_ERR_INVALID_ARGUMENT;
+  const uint64_t code_bits = bits == MF_BITS_4 ? 4 : 2;
+  const uint64_t gu_w = static_cast<uint64_t>(f) * d * code_bits / 8, gu_s = static_cast<uint64_t>(f) * (d / MF_GROUP_SIZE) * 2;
+  const uint64_t dn_w = static_cast<uint64_t>(d) * f * code_bits / 8, dn_s = static_cast<uint64_t>(d) * (f / MF_GROUP_SIZE) * 2;
+  const bool has_bias = bits != MF_BITS_TERNARY;
+  const uint64_t sizes[3][2] = {{gu_w, gu_s}, {gu_w, gu_s}, {dn_w, dn_s}};
+  uint32_t* out[3][3] = {{&offsets->gate_w, &offsets->gate_s, &offsets->gate_b},
+                         {&offsets->up_w, &offsets->up_s, &offsets->up_b},
+                         {&offsets->down_w, &offsets->down_s, &offsets->down_b}};
+  uint64_t pos = 0;
+  for (int p = 0; p < 3; ++p) {
+    *out[p][0] = static_cast<uint32_t>(pos); pos += sizes[p][0];
+    *out[p][1] = static_cast<uint32_t>(pos); pos += sizes[p][1];
+    *out[p][2] = has_bias ? static_cast<uint32_t>(pos) : 0u;
+    if (has_bias) pos += sizes[p][1];
+    if (pos > 0xFFFFFFFFull) return MF_ERR_DIMENSION_MISMATCH;  // MoEExpertOffsets holds 32-bit offsets
+  }
+  if (blob_bytes) *blob_bytes = static_cast<size_t>(pos);
+  if (stride) *stride = static_cast<size_t>((pos + align - 1) / align * align);
+  return MF_OK;
+}
+
 /* ---------------------------------------------------------- MoE operator */
 
 mf_status mf_moe_create(mf_ctx* ctx, const mf_moe_config* cfg, mf_moe** out) {
@@ -512,9 +539,16 @@ mf_status mf_moe_status(mf_moe* h, mf_stream stream) {
 
 mf_status mf_moe_group(mf_moe* h, mf_stream stream, const uint32_t* idx, const float* w, uint32_t t,
                        mf_pair* sorted_pairs, uint32_t* expert_offsets, uint32_t* expert_counts) {
-  if (!h || !idx || !w || !sorted_pairs || !expert_offsets || !expert_counts)
-    return MF_ERR_INVALID_ARGUMENT;
+  if (!h || !expert_offsets || !expert_counts) return MF_ERR_INVALID_ARGUMENT;
   auto s = static_cast<hipStream_t>(stream);
+  if (t == 0) {  // queryCount == 0 is valid (PrefillMoEGrouping.swift:99-104): no pairs, every expert empty
+    MF_HIP(h->ctx, hipMemsetAsync(expert_counts, 0, sizeof(uint32_t) * h->cfg.num_experts, s));
+    MF_HIP(h->ctx, hipMemsetAsync(expert_offsets, 0xFF, sizeof(uint32_t) * h->cfg.num_experts, s));
+    MF_HIP(h->ctx, hipMemsetAsync(h->ws.group_tmp + 3 * 512, 0, sizeof(uint32_t), s));
+    return MF_OK;
+  }
+  if (!idx || !w || !sorted_pairs) return MF_ERR_INVALID_ARGUMENT;
+  if (t > (1u << 20)) return MF_ERR_QUERY_COUNT;  // t * top_k stays far inside 32 bits, as in the prefill call
   uint32_t* starts = h->ws.group_tmp + 512;
   uint32_t* status = h->ws.group_tmp + 3 * 512;
   MF_HIP(h->ctx, mf::launch_group(s, idx, w, t, h->cfg.top_k, h->cfg.num_experts, expert_counts,

@@ -1216,6 +1216,10 @@ hipError_t launch_prefill_router(hipStream_t s, const uint16_t* W, const uint16_
   // of a 258-row Inkling router) go through the register-tiled kernel behind it.
   const uint32_t e32 = (T > 256 || D > 4096) && D % 512 == 0 && aligned16(W) && aligned16(x) && x_stride % 8 == 0
                            ? E & ~31u : 0u;
+  // rows of more than 4096 elements that the matrix-core kernel does not take (a width that is no
+  // multiple of 512, rows left over by the blocks of 32, unaligned operands): the register-tiled
+  // kernel cannot hold them, so the whole call goes one wave per (token, row) -- the same bits
+  if ((D / 8 + 63) / 64 > 8 && e32 != E) return launch_router_logits(s, W, x, E, D, T, x_stride, logits, nullptr);
   if (e32) {
     prefill_router_mfma_kernel<<<dim3((T + 31) / 32, e32 / 32), dim3(256), 0, s>>>(W, x, e32, D, T, x_stride,
                                                                                   logits, E);

@@ -270,6 +270,15 @@ class FamilyRouters:
             _ptr(out_weights)), self.context.handle)
 
 
+def expert_blob_layout(d: int, f: int, bits: int = BITS_4, align: int = 256):
+    """(offsets, blob_bytes, stride) of one routed expert in the reference's blob order
+    (RepackPlanner.swift:544-712, ModelExpertIO.swift:20-35): mf_expert_blob_layout."""
+    off = ExpertOffsets()
+    blob, stride = C.c_size_t(0), C.c_size_t(0)
+    check(_capi.lib().mf_expert_blob_layout(d, f, bits, align, C.byref(off), C.byref(blob), C.byref(stride)))
+    return off, blob.value, stride.value
+
+
 @dataclass
 class MoELayerWeights:
     """Everything one MoE layer reads, resident in device memory."""
@@ -280,6 +289,9 @@ class MoELayerWeights:
     w_sg: Optional[torch.Tensor] = None    # bf16 [d]
 
     def c(self) -> _capi.LayerWeights:
+        if self.experts.ndim != 2 or self.experts.stride(1) != 1:
+            # a 1-D pool would make stride(0) one byte: every expert would read expert 0's bytes
+            raise MfError(-1, "experts must be a [num_experts, stride] byte tensor")
         L = _capi.LayerWeights()
         L.router_w = _ptr(self.router_w)
         L.expert_base = _ptr(self.experts)

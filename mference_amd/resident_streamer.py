@@ -100,6 +100,8 @@ class ResidentExpertStreamer:
     def expert_buffer(self, layer: int, expert: int) -> Tuple["object", int, int]:
         """(buffer, offset, size) of one expert (`expertBuffer(layer:expert:)`): the buffer is the
         expert's row of the pool, the offset inside it 0."""
+        if layer != 0:  # the pool holds the one layer of the file the layout names
+            raise StreamerError.offset_out_of_range(layer)
         if not 0 <= expert < self.layout.experts_per_layer:
             raise StreamerError.slot_out_of_range(expert)
         return self.pool[expert], 0, self.layout.expert_stride

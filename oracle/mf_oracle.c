@@ -18,11 +18,14 @@
  *                                 by the reference's invariants (nibble order,
  *                                 constant group, codebook ends, error bound,
  *                                 edge list) and by brute-force nearest-code.
- *   mfo_quantize_affine bits 2    PARITY UNPINNED: the reference has no 2-bit
- *                                 quantizer (only random-code fixtures,
+ *   mfo_quantize_affine bits 2    PARITY UNPINNED against the reference, which
+ *                                 has no 2-bit quantizer to compare with (only
+ *                                 random-code fixtures,
  *                                 DSV4ToySynthetic.swift:319-337).  Defined by
- *                                 analogy (scale=(max-min)/3); only the 2-bit
- *                                 DEQUANT / element order is pinned.
+ *                                 analogy (scale=(max-min)/3) and checked the
+ *                                 way the 4-bit one is: brute-force nearest of
+ *                                 the four levels.  The 2-bit DEQUANT / element
+ *                                 order is pinned.
  *   mfo_dequantize                closed form q*s+b, two roundings
  *                                 (Quantization.swift:104-119); element order
  *                                 pinned by hand-built byte KATs

@@ -169,3 +169,24 @@ def test_struct_layouts_of_header_and_ctypes_mirror_agree(tmp_path):
     assert [table[("mf_expert_offsets", f)] for f in structs["mf_expert_offsets"]] == list(range(0, 36, 4))
     pairs = (_capi.Pair * 3)()
     assert C.addressof(pairs[1]) - C.addressof(pairs[0]) == 16
+
+
+@pytest.mark.parametrize("d,f,bits", [(2048, 512, 4), (4096, 2048, 2), (2048, 1024, 1), (128, 64, 4)])
+def test_expert_blob_layout_matches_checker(d, f, bits):
+    """mf_expert_blob_layout (the product's own helper) against the checker's restatement of the
+    repacker's blob order; the Qwen expert is 1 769 472 bytes = 108 pages of 16 KiB exactly."""
+    from mference_amd import operators as ops
+    from oracle import mf_oracle as O
+    off, blob, stride = ops.expert_blob_layout(d, f, bits, 16384)
+    ref_off, ref_blob, ref_stride = O.blob_layout(d, f, bits, 16384)
+    for name, _ in off._fields_:
+        assert getattr(off, name) == getattr(ref_off, name), name
+    assert (blob, stride) == (ref_blob, ref_stride)
+    if (d, f, bits) == (2048, 512, 4):
+        assert blob == 1769472 == 108 * 16384 == stride
+    lib = _capi.lib()
+    o = _capi.ExpertOffsets()
+    assert lib.mf_expert_blob_layout(100, 64, 4, 256, C.byref(o), None, None) == -2
+    assert lib.mf_expert_blob_layout(128, 64, 3, 256, C.byref(o), None, None) == -3
+    assert lib.mf_expert_blob_layout(128, 64, 4, 0, C.byref(o), None, None) == -1
+    assert lib.mf_expert_blob_layout(128, 64, 4, 256, None, None, None) == -1

@@ -531,3 +531,23 @@ def test_residual_rmsnorm_matches_oracle(gpu, oracle, d, t, with_delta):
     step = np.maximum(np.abs(ref), 2.0 ** -126) * 2.0 ** -7
     assert (np.abs(got - ref) <= step).all()
     assert (ops.bf16_bits(out) != ref_out).mean() < 0.01
+
+
+@pytest.mark.parametrize("count", [1, 63, 512, 4099])
+def test_silu_mul_matches_oracle(gpu, oracle, count):
+    """silu_mul_fp16 (utility.metal:21-33): out = narrow(silu(gate) * up), one rounding, bit for bit
+    against the checker's silu on every element (incl. large |gate|, zeros and negative zero)."""
+    rng = oracle.Rng.key(0x51, f"silu-mul-{count}")
+    g = rng.normal(0.0, 3.0, count).astype(np.float32)
+    u = rng.normal(0.0, 2.0, count).astype(np.float32)
+    g[: min(count, 6)] = np.array([0.0, -0.0, 40.0, -40.0, 88.5, -100.0], np.float32)[: min(count, 6)]
+    gb, ub = oracle.bf16_bits(g), oracle.bf16_bits(u)
+    gf, uf = oracle.bf16_to_float(gb), oracle.bf16_to_float(ub)
+    ref = oracle.bf16_bits(np.array([np.float32(oracle.silu(float(a))) * np.float32(b) for a, b in zip(gf, uf)],
+                                    np.float32))
+    out = torch.full((count + 8,), 1.0, dtype=torch.bfloat16, device="cuda")  # 8 sentinels behind
+    ops.Elementwise(gpu).encode_silu_mul(ops.bf16_tensor(gb), ops.bf16_tensor(ub), out, count)
+    _sync()
+    got = ops.bf16_bits(out)
+    assert np.array_equal(got[:count], ref)
+    assert np.all(got[count:] == 0x3F80)  # nothing written past count

@@ -43,6 +43,26 @@ def test_device_grouping_matches_oracle(gpu, oracle, t, k, e, live):
     assert np.array_equal(counts.cpu().numpy().view(np.uint32), ref["counts"])
 
 
+def test_device_grouping_of_no_tokens(gpu):
+    """queryCount == 0 is a valid call (PrefillMoEGrouping.swift:99-104): no pairs, every expert
+    empty (count 0, offset 0xFFFFFFFF), status clean; an absurd token count is refused."""
+    e, k = 24, 4
+    moe = ops.MoE(gpu, 128, 64, e, k)
+    offsets = torch.full((e,), 7, dtype=torch.int32, device="cuda")
+    counts = torch.full((e,), 7, dtype=torch.int32, device="cuda")
+    lib = _capi.lib()
+    assert lib.mf_moe_group(moe._h, None, None, None, 0, None, offsets.data_ptr(), counts.data_ptr()) == 0
+    moe.group_status()
+    assert np.all(offsets.cpu().numpy().view(np.uint32) == 0xFFFFFFFF)
+    assert np.all(counts.cpu().numpy() == 0)
+    idx = torch.zeros((1, k), dtype=torch.int32, device="cuda")
+    w = torch.zeros((1, k), dtype=torch.float32, device="cuda")
+    sp = torch.zeros((k, 4), dtype=torch.int32, device="cuda")
+    assert lib.mf_moe_group(moe._h, None, idx.data_ptr(), w.data_ptr(), (1 << 20) + 1, sp.data_ptr(),
+                            offsets.data_ptr(), counts.data_ptr()) == -10
+    torch.cuda.synchronize()
+
+
 def test_device_grouping_flags_expert_out_of_range(gpu):
     t, k, e = 9, 4, 16
     idx = np.tile(np.arange(k, dtype=np.uint32), (t, 1))

@@ -124,7 +124,7 @@ def test_roundtrip_bounds():
         assert np.all(np.abs(rec - raw) <= bound)
 
 
-@pytest.mark.parametrize("bits", [4, 8])
+@pytest.mark.parametrize("bits", [2, 4, 8])
 def test_codes_are_nearest_levels(bits):
     """brute force: every stored code is the nearest of the 2^bits levels q*s+b"""
     raw = O.Rng.key(0x51A71001, "int4-affine-round-trip").uniform_fill(-1.0, 1.0, 4 * 256).reshape(4, 256)

@@ -154,10 +154,32 @@ mf_status mf_residual_add(mf_ctx* ctx, mf_stream stream, uint16_t* hidden,
 mf_status mf_residual_rmsnorm(mf_ctx* ctx, mf_stream stream, uint16_t* hidden, const uint16_t* delta,
                               const uint16_t* weight, uint16_t* out, uint32_t d, uint32_t t, float eps);
 
+/* MPPPrefillInt4QMM.encode (Kernels/TensorCore/MPPPrefillInt4QMM.swift:34-78; kernel
+ * mpp_prefill_affine_threadgroup_f16, Metal/TensorCore/tensorops.metal:13-105) and its scalar twin
+ * PrefillInt4QMM (prefill_dequant_int4_qmm_f16_block, Metal/Prefill/prefill.metal:822-859): the
+ * dense projection of many rows, y[m, n] = x[m, k] . deq(W[n, k])^T with fp32 accumulation, x bf16
+ * [m, k], y bf16 [m, n] (fp32 when out_f32 != 0), k a multiple of 64, any m and n.  With n and k
+ * multiples of 128, 16-byte aligned w.weights / x / y and a 16-byte aligned workspace of at least
+ * mf_qmm_workspace_bytes(m, n, k) the call runs on the matrix cores (codes expanded to exact bf16 in
+ * registers, one fp32 scale multiply per 64-wide K group -- the kernel of mf_moe_prefill_layer; a K
+ * beyond 4096 is cut into windows whose fp32 results are added in order); every other shape,
+ * alignment or workspace runs row by row through the kernels of mf_gemv, bit-identical to
+ * mf_gemv.  Where the reference returns .unavailable (bad sizes or offsets) the call returns a
+ * negative status and launches nothing.  Replaces the 4-bit, 2-bit and ternary projections alike. */
+size_t mf_qmm_workspace_bytes(uint32_t m, uint32_t n, uint32_t k);
+mf_status mf_qmm(mf_ctx* ctx, mf_stream stream, mf_qtensor w, mf_bits bits, const uint16_t* x, void* y, uint32_t m,
+                 uint32_t n, uint32_t k, int out_f32, void* workspace, size_t workspace_bytes);
+
 /* SharedExpertInt4.encode (Kernels/MoE/SharedExpertInt4.swift:70-165) /
  * SharedExpertRuntime.encode (:193-202): y[t,d] = bf16(down . act),
- * act = bf16(silu(bf16(gate.x)) * bf16(up.x)).  scratch_act holds t*f bf16.
- * Also the dense SwiGLU MLP of Qwen38ForwardRunner (mlp.encode, :1094). */
+ * act = bf16(silu(bf16(gate.x)) * bf16(up.x)).  Also the dense SwiGLU MLP of Qwen38ForwardRunner
+ * (mlp.encode, :1094) and, for any t, PrefillSharedExpert.encodeBlock (Kernels/Prefill/MoE/
+ * PrefillSharedExpert.swift:81-190) / encodeDenseMLPPrefill (Qwen38ForwardRunner.swift:862-913):
+ * from 32 rows on the projections run on the matrix cores when d and f are multiples of 128,
+ * d <= 7168, the operands are 16-byte aligned and scratch_act holds
+ * mf_shared_expert_scratch_bytes(d, f, t) bytes; otherwise row by row, MF_MAX_TOKENS rows per pair
+ * of launches, for which t*f bf16 of scratch suffice (all that t <= MF_MAX_TOKENS ever needs). */
+size_t mf_shared_expert_scratch_bytes(uint32_t d, uint32_t f, uint32_t t);
 mf_status mf_shared_expert(mf_ctx* ctx, mf_stream stream, const uint16_t* x, mf_qtensor gate,
                            mf_qtensor up, mf_qtensor down, mf_bits bits, uint32_t d, uint32_t f,
                            uint32_t t, uint16_t* y, uint16_t* scratch_act,

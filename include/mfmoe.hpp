@@ -206,6 +206,37 @@ class SharedExpertInt4 {
     check(mf_shared_expert(ctx_, commandBuffer, x, gate, up, down, bits_, d, f, tokens, y, scratchAct,
                            scratchActBytes), ctx_);
   }
+  // scratch the block form (PrefillSharedExpert.encodeBlock, from 32 rows on) can use
+  static size_t scratchBytes(uint32_t d, uint32_t f, uint32_t tokens) { return mf_shared_expert_scratch_bytes(d, f, tokens); }
+  // the same operator without a scratch argument and without device allocation (the activations go
+  // through a device array inside the library; tokens * f <= MF_STATIC_ACT_ELEMS, calls must not overlap)
+  void encodeStatic(mf_stream commandBuffer, const uint16_t* x, mf_qtensor gate, mf_qtensor up, mf_qtensor down,
+                    uint32_t d, uint32_t f, uint16_t* y, uint32_t tokens = 1) const {
+    check(mf_shared_expert_static(ctx_, commandBuffer, x, gate, up, down, bits_, d, f, tokens, y), ctx_);
+  }
+
+ private:
+  mf_ctx* ctx_;
+  mf_bits bits_;
+};
+
+// MPPPrefillInt4QMM (Kernels/TensorCore/MPPPrefillInt4QMM.swift:34-78): y[m, n] = x[m, k] . deq(W[n, k])^T.
+// encode returns the path like the reference: Unavailable for sizes or offsets it rejects.
+class MPPPrefillInt4QMM {
+ public:
+  enum class Path { AffineMatrixCoreBF16, Unavailable };
+  static constexpr int tileM = 64, tileN = 32, tileK = MF_GROUP_SIZE;
+  explicit MPPPrefillInt4QMM(const MetalContext& context, mf_bits bits = MF_BITS_4) : ctx_(context.raw()), bits_(bits) {}
+  static size_t workspaceBytes(uint32_t m, uint32_t n, uint32_t k) { return mf_qmm_workspace_bytes(m, n, k); }
+  Path encode(mf_stream commandBuffer, mf_qtensor weights, const uint16_t* x, void* y, uint32_t m, uint32_t n,
+              uint32_t k, void* workspace, size_t workspaceBytes, bool outputFloat32 = false) const {
+    const mf_status st = mf_qmm(ctx_, commandBuffer, weights, bits_, x, y, m, n, k, outputFloat32 ? 1 : 0, workspace,
+                                workspaceBytes);
+    if (st == MF_ERR_INVALID_ARGUMENT || st == MF_ERR_DIMENSION_MISMATCH || st == MF_ERR_UNSUPPORTED_BITS)
+      return Path::Unavailable;
+    check(st, ctx_);
+    return Path::AffineMatrixCoreBF16;
+  }
 
  private:
   mf_ctx* ctx_;
@@ -213,6 +244,14 @@ class SharedExpertInt4 {
 };
 
 using MoEExpertOffsets = mf_expert_offsets;  // Kernels/MoE/MoE.swift:4-29
+// offsets, blob size and page-rounded stride of one routed expert in the repacker's blob order
+// (RepackPlanner.swift:544-712, ModelExpertIO.swift:20-35)
+inline MoEExpertOffsets expertBlobLayout(uint32_t d, uint32_t f, mf_bits bits, uint32_t align, size_t* blobBytes,
+                                         size_t* stride) {
+  MoEExpertOffsets off{};
+  check(mf_expert_blob_layout(d, f, bits, align, &off, blobBytes, stride), nullptr);
+  return off;
+}
 
 // MoE (Kernels/MoE/MoE.swift), MoEDeepseekV4 (2-bit, top-6) and MapleMoE (ternary, full-softmax
 // router) in one class, selected by the configuration — the specialisation arguments of

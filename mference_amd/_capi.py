@@ -80,6 +80,9 @@ SIGNATURES = {
     "mf_residual_rmsnorm": (_I, [_P, _P, _P, _P, _P, _P, _U32, _U32, C.c_float]),
     "mf_shared_expert": (_I, [_P, _P, _P, QTensor, QTensor, QTensor, _I, _U32, _U32, _U32, _P, _P,
                               _SZ]),
+    "mf_shared_expert_scratch_bytes": (_SZ, [_U32, _U32, _U32]),
+    "mf_qmm_workspace_bytes": (_SZ, [_U32, _U32, _U32]),
+    "mf_qmm": (_I, [_P, _P, QTensor, _I, _P, _P, _U32, _U32, _U32, _I, _P, _SZ]),
     "mf_shared_expert_static": (_I, [_P, _P, _P, QTensor, QTensor, QTensor, _I, _U32, _U32, _U32, _P]),
     "mf_expert_blob_layout": (_I, [_U32, _U32, _I, _U32, C.POINTER(ExpertOffsets), C.POINTER(_SZ), C.POINTER(_SZ)]),
     "mf_moe_create": (_I, [_P, C.POINTER(MoEConfig), C.POINTER(_P)]),

@@ -165,6 +165,11 @@ mf_status mf_residual_rmsnorm(mf_ctx* ctx, mf_stream stream, uint16_t* hidden, c
   return MF_OK;
 }
 
+size_t mf_shared_expert_scratch_bytes(uint32_t d, uint32_t f, uint32_t t) {
+  if (t <= MF_MAX_TOKENS || d % MF_GROUP_SIZE || f % MF_GROUP_SIZE) return static_cast<size_t>(t) * f * sizeof(uint16_t);
+  return mf::dense_mlp_scratch_bytes(d, f, t);
+}
+
 mf_status mf_shared_expert(mf_ctx* ctx, mf_stream stream, const uint16_t* x, mf_qtensor gate,
                            mf_qtensor up, mf_qtensor down, mf_bits bits, uint32_t d, uint32_t f,
                            uint32_t t, uint16_t* y, uint16_t* scratch_act,
@@ -173,7 +178,7 @@ mf_status mf_shared_expert(mf_ctx* ctx, mf_stream stream, const uint16_t* x, mf_
   if (!bits_ok(bits)) return MF_ERR_UNSUPPORTED_BITS;
   if (d == 0 || f == 0 || d % MF_GROUP_SIZE != 0 || f % MF_GROUP_SIZE != 0)
     return MF_ERR_DIMENSION_MISMATCH;
-  if (t == 0 || t > MF_MAX_TOKENS) return MF_ERR_INVALID_ARGUMENT;
+  if (t == 0 || t > (1u << 20)) return MF_ERR_INVALID_ARGUMENT;
   if (!qtensor_ok(gate, bits) || !qtensor_ok(up, bits) || !qtensor_ok(down, bits))
     return MF_ERR_INVALID_ARGUMENT;
   if (!mf::aligned2(x) || !mf::aligned2(y) || !mf::aligned2(scratch_act))
@@ -181,8 +186,48 @@ mf_status mf_shared_expert(mf_ctx* ctx, mf_stream stream, const uint16_t* x, mf_
   if (scratch_act_bytes < static_cast<size_t>(t) * f * sizeof(uint16_t))
     return MF_ERR_SCRATCH_TOO_SMALL;
   auto s = static_cast<hipStream_t>(stream);
-  MF_HIP(ctx, mf::launch_gate_up_act(s, gate, up, bits, x, scratch_act, f, d, t));
-  MF_HIP(ctx, mf::launch_gemv(s, down, bits, scratch_act, y, d, f, t, false));
+  // PrefillSharedExpert.encodeBlock (PrefillSharedExpert.swift:114-172): from 32 rows on the projections
+  // go through the matrix-core matmul when the shape allows and the scratch holds its staging rows
+  if (t >= 32 && mf::dense_mlp_takes(gate, up, down, x, y, scratch_act, d, f, t) &&
+      scratch_act_bytes >= mf::dense_mlp_scratch_bytes(d, f, t)) {
+    MF_HIP(ctx, mf::launch_dense_mlp(s, gate, up, down, bits, x, y, d, f, t, scratch_act));
+    return MF_OK;
+  }
+  // row by row otherwise (PrefillSharedExpert.swift:174-190), MF_MAX_TOKENS rows per pair of launches
+  for (uint32_t t0 = 0; t0 < t; t0 += MF_MAX_TOKENS) {
+    const uint32_t tc = std::min<uint32_t>(t - t0, MF_MAX_TOKENS);
+    uint16_t* act = scratch_act + static_cast<size_t>(t0) * f;
+    MF_HIP(ctx, mf::launch_gate_up_act(s, gate, up, bits, x + static_cast<size_t>(t0) * d, act, f, d, tc));
+    MF_HIP(ctx, mf::launch_gemv(s, down, bits, act, y + static_cast<size_t>(t0) * d, d, f, tc, false));
+  }
+  return MF_OK;
+}
+
+size_t mf_qmm_workspace_bytes(uint32_t m, uint32_t n, uint32_t k) {
+  if (m == 0 || n == 0 || k == 0 || k % MF_GROUP_SIZE) return 0;
+  return mf::dense_qmm_workspace_bytes(m, n, k);
+}
+
+mf_status mf_qmm(mf_ctx* ctx, mf_stream stream, mf_qtensor w, mf_bits bits, const uint16_t* x, void* y, uint32_t m,
+                 uint32_t n, uint32_t k, int out_f32, void* workspace, size_t workspace_bytes) {
+  // the conditions under which MPPPrefillInt4QMM.encode returns .unavailable (MPPPrefillInt4QMM.swift:43-55)
+  if (!ctx || !x || !y) return MF_ERR_INVALID_ARGUMENT;
+  if (!bits_ok(bits)) return MF_ERR_UNSUPPORTED_BITS;
+  if (m == 0 || n == 0 || k == 0 || k % MF_GROUP_SIZE != 0 || m > (1u << 20)) return MF_ERR_DIMENSION_MISMATCH;
+  if (!qtensor_ok(w, bits) || !mf::aligned2(x) || !mf::aligned2(y)) return MF_ERR_INVALID_ARGUMENT;
+  auto s = static_cast<hipStream_t>(stream);
+  if (workspace && mf::aligned16(workspace) && mf::dense_qmm_takes(w, bits, x, y, m, n, k) &&
+      workspace_bytes >= mf::dense_qmm_workspace_bytes(m, n, k)) {
+    MF_HIP(ctx, mf::launch_dense_qmm(s, w, bits, x, y, m, n, k, out_f32 != 0, workspace));
+    return MF_OK;
+  }
+  // any other shape or alignment: the rows MF_MAX_TOKENS at a time through the GEMV kernels
+  const size_t ybytes = out_f32 ? sizeof(float) : sizeof(uint16_t);
+  for (uint32_t m0 = 0; m0 < m; m0 += MF_MAX_TOKENS) {
+    const uint32_t mc = std::min<uint32_t>(m - m0, MF_MAX_TOKENS);
+    MF_HIP(ctx, mf::launch_gemv(s, w, bits, x + static_cast<size_t>(m0) * k,
+                                static_cast<uint8_t*>(y) + static_cast<size_t>(m0) * n * ybytes, n, k, mc, out_f32 != 0));
+  }
   return MF_OK;
 }
 

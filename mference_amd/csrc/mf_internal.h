@@ -136,6 +136,16 @@ bool prefill_supported(const mf_moe_config& c);
 hipError_t launch_prefill_layer(hipStream_t s, const mf_moe& h, const mf_moe_layer_weights& w,
                                 const uint16_t* x, uint32_t t, uint16_t* y, void* workspace,
                                 uint32_t* out_idx, float* out_w);
+// dense projections over many rows through the matrix-core matmul (moe_prefill.hip)
+bool dense_qmm_takes(const mf_qtensor& w, int bits, const void* x, const void* y, uint32_t m, uint32_t n, uint32_t k);
+size_t dense_qmm_workspace_bytes(uint32_t m, uint32_t n, uint32_t k);
+hipError_t launch_dense_qmm(hipStream_t s, const mf_qtensor& w, int bits, const uint16_t* x, void* y, uint32_t m,
+                            uint32_t n, uint32_t k, bool out_f32, void* workspace);
+bool dense_mlp_takes(const mf_qtensor& gate, const mf_qtensor& up, const mf_qtensor& down, const void* x,
+                     const void* y, const void* scratch, uint32_t d, uint32_t f, uint32_t t);
+size_t dense_mlp_scratch_bytes(uint32_t d, uint32_t f, uint32_t t);
+hipError_t launch_dense_mlp(hipStream_t s, const mf_qtensor& gate, const mf_qtensor& up, const mf_qtensor& down,
+                            int bits, const uint16_t* x, uint16_t* y, uint32_t d, uint32_t f, uint32_t t, void* scratch);
 hipError_t launch_prefill_router(hipStream_t s, const uint16_t* W, const uint16_t* x, uint32_t E,
                                  uint32_t D, uint32_t T, uint32_t x_stride, float* logits);
 }  // namespace mf

@@ -476,6 +476,15 @@ struct QmmArgs {
   const Tile* tiles;
   const uint32_t* n_tiles;
   uint32_t rows, kdim;  // weight rows (output width) and contraction length
+  // a launch may take a window of the contraction (long K is cut into windows whose fp32 results are
+  // added afterwards): rows of weights, tables and group sums are ng_ld groups apart (0: kdim / 64)
+  // and the window starts at group g_off (a multiple of 8)
+  uint32_t ng_ld, g_off;
+  // several windows in one launch (dense mode): tile slots [w * win_tiles, (w + 1) * win_tiles) belong to
+  // window w, which covers the groups from dense_window_start(ng_ld, n_win, w) on and writes its fp32
+  // result out_win_stride elements behind the previous window's
+  uint32_t n_win, win_tiles;
+  size_t out_win_stride;
   // epilogue
   int epi;              // 0 swiglu -> bf16 [pair, rows] in prep order; 1 fp32 [token*K+rank, rows]; 2 bf16 [pair, rows]
   int narrow;           // shared-expert rounding points (dequant_int4.metal:240-245)
@@ -490,6 +499,12 @@ struct QmmArgs {
   unsigned long long* trace;
   uint32_t trace_items;
 };
+
+// first K group of window wdx when ng groups are cut into n_win windows (multiples of 8 groups)
+__host__ __device__ __forceinline__ uint32_t dense_window_start(uint32_t ng, uint32_t n_win, uint32_t wdx) {
+  if (wdx >= n_win) return ng;
+  return static_cast<uint32_t>(static_cast<uint64_t>(ng) * wdx / n_win) & ~7u;
+}
 
 __device__ __forceinline__ void qmm_trace(const QmmArgs& a, uint32_t work, uint32_t k) {
   if (a.trace && threadIdx.x == 0 && work < a.trace_items) a.trace[work * 8 + k] = wall_clock64();
@@ -537,8 +552,17 @@ void qmm_kernel(const QmmLaunch launch) {
   const uint32_t work = (blockIdx.x & 7u) * launch.per_xcd[second ? 1 : 0] + (xcd_slot - (second ? launch.per_xcd[0] : 0u));
   const uint32_t wave_rows = a.pair_rows ? 32u * NPROJ : 32u;  // weight rows of one wave
   const uint32_t n_slices = a.rows / (kQmmWaves * wave_rows);
-  const uint32_t tile_id = work / n_slices, slice = work % n_slices;
-  const uint32_t ng = a.kdim / kGroup;
+  uint32_t tile_id = work / n_slices;
+  const uint32_t slice = work % n_slices;
+  uint32_t ng = a.kdim / kGroup, g_off = a.g_off;
+  uint8_t* out_base = static_cast<uint8_t*>(a.out);
+  if (a.n_win > 1) {  // this work item's window of the contraction
+    const uint32_t win = tile_id / a.win_tiles;
+    tile_id -= win * a.win_tiles;
+    g_off = dense_window_start(a.ng_ld, a.n_win, win);
+    ng = dense_window_start(a.ng_ld, a.n_win, win + 1) - g_off;
+    out_base += win * a.out_win_stride * sizeof(float);
+  }
   qmm_trace(a, work, 0);
 
   uint32_t expert = 0, pair_start, count;
@@ -578,7 +602,8 @@ void qmm_kernel(const QmmLaunch launch) {
     }
     row_base[p] = (slice * kQmmWaves + wv) * wave_rows + (a.pair_rows ? 32u * p : 0u);
   }
-  const size_t row_bytes = static_cast<size_t>(ng) * kGB;
+  const uint32_t ng_ld = a.ng_ld ? a.ng_ld : ng;
+  const size_t row_bytes = static_cast<size_t>(ng_ld) * kGB;
 
   // ---- everything the tile needs that depends only on the tile: issued back to back.
   // Routes past `count` read the tile's last route instead (finite data, results discarded).
@@ -600,12 +625,12 @@ void qmm_kernel(const QmmLaunch launch) {
   QmmCodes<BITS> cur[NPROJ][4];
 #pragma unroll
   for (int p = 0; p < NPROJ; ++p) {
-    wrow[p] = Wp[p] + (row_base[p] + m) * row_bytes + h * (kGB / 2);
+    wrow[p] = Wp[p] + (row_base[p] + m) * row_bytes + static_cast<size_t>(g_off) * kGB + h * (kGB / 2);
 #pragma unroll
     for (int u = 0; u < 4; ++u) cur[p][u].load(wrow[p] + min(static_cast<uint32_t>(u), ng - 1) * kGB);
   }
   // x rows of groups 0..2 and, for the bias terms, the group sums of the lane's two routes
-  const uint16_t* st_src = a.x + static_cast<size_t>(st_row) * a.x_stride + st_q * 16;
+  const uint16_t* st_src = a.x + static_cast<size_t>(st_row) * a.x_stride + static_cast<size_t>(g_off) * kGroup + st_q * 16;
   // K groups travel in pairs (ng is even: kdim is a multiple of 128)
   // (arrays of a native vector type: arrays of the uint4 struct were kept in scratch memory)
   typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
@@ -634,7 +659,7 @@ void qmm_kernel(const QmmLaunch launch) {
     const uint32_t gc = gl < ng ? gl : 0;  // a lane without groups reads group 0 and drops it
 #pragma unroll
     for (int p = 0; p < NPROJ; ++p) {
-      const size_t at = static_cast<size_t>(row_base[p] + m) * ng + gc;
+      const size_t at = static_cast<size_t>(row_base[p] + m) * ng_ld + g_off + gc;
       t.B[p] = NG8 ? (a.tab_aligned ? load_x8<true>(Bp[p] + at) : load_x8<false>(Bp[p] + at))
                    : load_bf16x8_guarded(Bp[p] + at, ng - gc);
       t.S[p] = NG8 ? (a.tab_aligned ? load_x8<true>(Sp[p] + at) : load_x8<false>(Sp[p] + at))
@@ -642,7 +667,7 @@ void qmm_kernel(const QmmLaunch launch) {
     }
 #pragma unroll
     for (int nt = 0; nt < 2; ++nt) {
-      const float* sp = a.sumx + static_cast<size_t>(xrow[nt]) * ng + gc;
+      const float* sp = a.sumx + static_cast<size_t>(xrow[nt]) * ng_ld + g_off + gc;
       if (NG8) {
         const float4 s0 = *reinterpret_cast<const float4*>(sp), s1 = *reinterpret_cast<const float4*>(sp + 4);
         t.sx[nt][0] = s0.x; t.sx[nt][1] = s0.y; t.sx[nt][2] = s0.z; t.sx[nt][3] = s0.w;
@@ -854,7 +879,7 @@ void qmm_kernel(const QmmLaunch launch) {
       const uint32_t sl = s_slot[tok];
       const uint4 v = reinterpret_cast<const uint4*>(so)[c];
       if (sl != 0xFFFFFFFFu)
-        *reinterpret_cast<uint4*>(static_cast<uint16_t*>(a.out) + static_cast<size_t>(sl) * a.rows + row_base[0] +
+        *reinterpret_cast<uint4*>(reinterpret_cast<uint16_t*>(out_base) + static_cast<size_t>(sl) * a.rows + row_base[0] +
                                   part * 8) = v;
     }
   } else {
@@ -871,8 +896,8 @@ void qmm_kernel(const QmmLaunch launch) {
 #pragma unroll
           for (int p = 0; p < NPROJ; ++p) {
             if (p > 0 && !a.pair_rows) break;
-            if (a.epi == 1) static_cast<float*>(a.out)[at + row_base[p] + m] = acc[p][nt][4 * j + i];
-            else static_cast<uint16_t*>(a.out)[at + row_base[p] + m] = f_to_bf16(acc[p][nt][4 * j + i]);
+            if (a.epi == 1) reinterpret_cast<float*>(out_base)[at + row_base[p] + m] = acc[p][nt][4 * j + i];
+            else reinterpret_cast<uint16_t*>(out_base)[at + row_base[p] + m] = f_to_bf16(acc[p][nt][4 * j + i]);
           }
         }
       }
@@ -1349,6 +1374,10 @@ hipError_t launch_qmm(hipStream_t s, int bits, QmmArgs a, int nproj, uint32_t ti
     if (q.dense_mode) {
       q.dense_tiles = slots;
       slots = (slots + 7) / 8 * 8;
+      if (q.n_win > 1) {  // every window of the contraction has its own run of tile slots
+        q.win_tiles = slots;
+        slots *= q.n_win;
+      }
     }
     launch.per_xcd[part] = slots / 8 * n_slices;
     q.tab_aligned = q.dense_mode
@@ -1356,8 +1385,8 @@ hipError_t launch_qmm(hipStream_t s, int bits, QmmArgs a, int nproj, uint32_t ti
               aligned16(q.dense[1].biases)
         : aligned16(q.expert_base) && q.expert_stride % 16 == 0 &&
               (q.s_off[0] | q.b_off[0] | q.s_off[1] | q.b_off[1]) % 16 == 0;
-    lds = std::max(lds, qmm_lds_bytes(q.kdim, nproj));
-    ng8 = ng8 && (q.kdim / kGroup) % 8 == 0;
+    lds = std::max(lds, qmm_lds_bytes(q.kdim, nproj));  // with windows: kdim is the longest window
+    ng8 = ng8 && (q.n_win > 1 ? q.ng_ld : q.kdim / kGroup) % 8 == 0;
   }
   const dim3 grid(8 * (launch.per_xcd[0] + launch.per_xcd[1])), block(256);
   if (grid.x == 0) return hipSuccess;
@@ -1384,6 +1413,141 @@ hipError_t launch_qmm(hipStream_t s, int bits, QmmArgs a, int nproj, uint32_t ti
 namespace {
 size_t up256(size_t v) { return (v + 255) / 256 * 256; }
 }  // namespace
+
+// ---- dense projections over many rows: MPPPrefillInt4QMM.encode (MPPPrefillInt4QMM.swift:34-78) and the
+// block form of the shared expert / dense MLP (PrefillSharedExpert.encodeBlock, PrefillSharedExpert.swift:81-172)
+//
+// y[m, n] = x[m, k] . W[n, k]^T through qmm_kernel in dense mode.  The kernel keeps the scales of a
+// workgroup's rows for the whole contraction in LDS, so a long K is cut into windows of at most
+// kDenseWindow groups (multiples of 8 groups, the last takes the rest): every window is a launch that
+// writes fp32 [m, n], and dense_combine_kernel adds the windows in order and narrows the sum.
+constexpr uint32_t kDenseWindow = 64;   // K groups per launch (4096 values)
+constexpr uint32_t kDenseFusedMax = 112;  // K groups a gate/up + SwiGLU launch can hold (both projections' scales in LDS)
+
+__global__ __launch_bounds__(256) void dense_combine_kernel(const float* __restrict__ parts, uint32_t n_parts,
+                                                            size_t part_stride, void* __restrict__ y, size_t count,
+                                                            int out_f32) {
+  const size_t i = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+  if (i >= count) return;
+  float acc = parts[i];
+  for (uint32_t p = 1; p < n_parts; ++p) acc = acc + parts[p * part_stride + i];
+  if (out_f32) static_cast<float*>(y)[i] = acc;
+  else static_cast<uint16_t*>(y)[i] = f_to_bf16(acc);
+}
+
+static uint32_t dense_windows(uint32_t ng) { return (ng + kDenseWindow - 1) / kDenseWindow; }
+
+// bytes of fp32 window results a projection of n rows over m tokens needs (0: one window, written directly)
+static size_t dense_parts_bytes(uint32_t m, uint32_t n, uint32_t k) {
+  const uint32_t n_win = dense_windows(k / kGroup);
+  return n_win > 1 ? up256(sizeof(float) * static_cast<size_t>(m) * n) * n_win : 0;
+}
+
+bool dense_qmm_takes(const mf_qtensor& w, int bits, const void* x, const void* y, uint32_t m, uint32_t n, uint32_t k) {
+  if (n % kQmmRows || k % (2 * kGroup) || m == 0) return false;
+  if (!aligned16(w.weights) || !aligned16(x) || !aligned16(y)) return false;
+  if (static_cast<uint64_t>(m) * n >= (1ull << 31)) return false;
+  return true;
+}
+
+size_t dense_qmm_workspace_bytes(uint32_t m, uint32_t n, uint32_t k) {
+  return up256(sizeof(uint16_t) * static_cast<size_t>(m) * k) + up256(sizeof(float) * static_cast<size_t>(m) * (k / kGroup)) +
+         dense_parts_bytes(m, n, k);
+}
+
+// x_prepared: rows already in the matmul's order with their group sums in sumx (x is then ignored)
+static hipError_t dense_project(hipStream_t s, const mf_qtensor& w, int bits, const uint16_t* xp, const float* sumx,
+                                void* y, uint32_t m, uint32_t n, uint32_t k, bool out_f32, void* parts) {
+  const uint32_t ng = k / kGroup, n_win = dense_windows(ng);
+  const int code_bits = bits == MF_BITS_4 ? 4 : 2;
+  QmmArgs d{};
+  d.dense_mode = 1; d.dense_rows = m; d.top_k = 1;
+  d.dense[0] = d.dense[1] = w;
+  if (bits == MF_BITS_TERNARY) {  // bias = -scale: the kernel reads the scale table as bias table
+    d.ternary = 1;
+    d.dense[0].biases = d.dense[1].biases = w.scales;
+  }
+  d.x = xp; d.sumx = sumx; d.x_stride = k; d.rows = n;
+  d.pair_rows = n % (2 * kQmmRows) == 0;
+  const uint32_t tiles = (m + kTileTokens - 1) / kTileTokens;
+  const size_t part_stride = up256(sizeof(float) * static_cast<size_t>(m) * n) / sizeof(float);
+  d.ng_ld = ng;
+  if (n_win == 1) {
+    d.kdim = k; d.epi = out_f32 ? 1 : 2; d.out = y;
+  } else {  // all windows in one launch, each writing fp32 into its own buffer
+    uint32_t longest = 0;
+    for (uint32_t wdx = 0; wdx < n_win; ++wdx)
+      longest = std::max(longest, dense_window_start(ng, n_win, wdx + 1) - dense_window_start(ng, n_win, wdx));
+    d.kdim = longest * kGroup; d.n_win = n_win; d.out_win_stride = part_stride; d.epi = 1; d.out = parts;
+  }
+  {
+    const hipError_t e = launch_qmm(s, code_bits, d, d.pair_rows ? 2 : 1, tiles, nullptr, 0);
+    if (e != hipSuccess) return e;
+  }
+  if (n_win > 1) {
+    const size_t count = static_cast<size_t>(m) * n;
+    dense_combine_kernel<<<dim3(static_cast<uint32_t>((count + 255) / 256)), dim3(256), 0, s>>>(
+        static_cast<const float*>(parts), n_win, part_stride, y, count, out_f32 ? 1 : 0);
+    return hipGetLastError();
+  }
+  return hipSuccess;
+}
+
+hipError_t launch_dense_qmm(hipStream_t s, const mf_qtensor& w, int bits, const uint16_t* x, void* y, uint32_t m,
+                            uint32_t n, uint32_t k, bool out_f32, void* workspace) {
+  uint8_t* base = static_cast<uint8_t*>(workspace);
+  uint16_t* xp = reinterpret_cast<uint16_t*>(base);
+  float* sumx = reinterpret_cast<float*>(base + up256(sizeof(uint16_t) * static_cast<size_t>(m) * k));
+  void* parts = reinterpret_cast<uint8_t*>(sumx) + up256(sizeof(float) * static_cast<size_t>(m) * (k / kGroup));
+  const hipError_t e = launch_prep_rows(s, x, xp, sumx, static_cast<size_t>(m) * k);
+  if (e != hipSuccess) return e;
+  return dense_project(s, w, bits, xp, sumx, y, m, n, k, out_f32, parts);
+}
+
+// The block form of the shared expert / dense SwiGLU MLP: gate and up in one launch with the SwiGLU epilogue
+// (gate and up narrowed first, dequant_int4.metal:240-245), then the down projection.
+bool dense_mlp_takes(const mf_qtensor& gate, const mf_qtensor& up, const mf_qtensor& down, const void* x,
+                     const void* y, const void* scratch, uint32_t d, uint32_t f, uint32_t t) {
+  if (d % kQmmRows || f % kQmmRows || d / kGroup > kDenseFusedMax || t == 0) return false;
+  return aligned16(gate.weights) && aligned16(up.weights) && aligned16(down.weights) && aligned16(x) && aligned16(y) &&
+         aligned16(scratch) && static_cast<uint64_t>(t) * std::max(d, f) < (1ull << 31);
+}
+
+size_t dense_mlp_scratch_bytes(uint32_t d, uint32_t f, uint32_t t) {
+  return up256(sizeof(uint16_t) * static_cast<size_t>(t) * f) + up256(sizeof(uint16_t) * static_cast<size_t>(t) * d) +
+         up256(sizeof(float) * static_cast<size_t>(t) * (d / kGroup)) + up256(sizeof(float) * static_cast<size_t>(t) * (f / kGroup)) +
+         dense_parts_bytes(t, d, f);
+}
+
+hipError_t launch_dense_mlp(hipStream_t s, const mf_qtensor& gate, const mf_qtensor& up, const mf_qtensor& down,
+                            int bits, const uint16_t* x, uint16_t* y, uint32_t d, uint32_t f, uint32_t t, void* scratch) {
+  uint8_t* base = static_cast<uint8_t*>(scratch);
+  uint16_t* act = reinterpret_cast<uint16_t*>(base);
+  base += up256(sizeof(uint16_t) * static_cast<size_t>(t) * f);
+  uint16_t* xp = reinterpret_cast<uint16_t*>(base);
+  base += up256(sizeof(uint16_t) * static_cast<size_t>(t) * d);
+  float* sumx = reinterpret_cast<float*>(base);
+  base += up256(sizeof(float) * static_cast<size_t>(t) * (d / kGroup));
+  float* sum_act = reinterpret_cast<float*>(base);
+  base += up256(sizeof(float) * static_cast<size_t>(t) * (f / kGroup));
+  hipError_t e = launch_prep_rows(s, x, xp, sumx, static_cast<size_t>(t) * d);
+  if (e != hipSuccess) return e;
+  const int code_bits = bits == MF_BITS_4 ? 4 : 2;
+  QmmArgs q{};
+  q.dense_mode = 1; q.dense_rows = t; q.top_k = 1; q.narrow = 1;
+  q.dense[0] = gate; q.dense[1] = up;
+  if (bits == MF_BITS_TERNARY) {
+    q.ternary = 1;
+    q.dense[0].biases = gate.scales;
+    q.dense[1].biases = up.scales;
+  }
+  q.x = xp; q.sumx = sumx; q.x_stride = d; q.rows = f; q.kdim = d; q.epi = 0; q.out = act;
+  e = launch_qmm(s, code_bits, q, 2, (t + kTileTokens - 1) / kTileTokens, nullptr, 0);
+  if (e != hipSuccess) return e;
+  e = launch_prep_rows(s, act, nullptr, sum_act, static_cast<size_t>(t) * f);  // the activations are in matmul order already
+  if (e != hipSuccess) return e;
+  return dense_project(s, down, bits, act, sum_act, y, t, d, f, false, base);
+}
 
 // entries of the tile list: every live expert may end in a partial tile; a multiple of 8
 uint32_t prefill_tile_slots(const mf_moe_config& c, uint32_t t) {

@@ -21,7 +21,7 @@ from ._capi import (BITS_2, BITS_4, BITS_TERNARY, GROUP_SIZE, MAX_TOKENS, ROUTER
 
 __all__ = [
     "MetalContext", "QuantizedTensor", "Quantization", "DequantInt4GEMV", "DequantInt4GEMVMultiX",
-    "Elementwise", "FamilyRouters", "SharedExpertInt4", "MoEExpertOffsets", "MoE", "MoELayerWeights",
+    "Elementwise", "FamilyRouters", "SharedExpertInt4", "MPPPrefillInt4QMM", "MoEExpertOffsets", "MoE", "MoELayerWeights",
     "PrefillMoEGrouping", "PrefillTokenExpertPair", "MfError", "BITS_2", "BITS_4", "BITS_TERNARY",
     "ROUTER_TOPK_SOFTMAX", "ROUTER_FULL_SOFTMAX", "bf16_tensor", "bf16_bits",
 ]
@@ -155,6 +155,34 @@ class DequantInt4GEMVMultiX(DequantInt4GEMV):
         super().encode(weights, x, y, m, n, output_float32, stream, t)
 
 
+class MPPPrefillInt4QMM:
+    """Kernels/TensorCore/MPPPrefillInt4QMM.swift:34-78: y[m, n] = x[m, k] . deq(W[n, k])^T for many
+    rows.  `encode` returns the path taken, like the reference's `Path`."""
+    tile_m, tile_n, tile_k = 64, 32, GROUP_SIZE
+
+    def __init__(self, context: MetalContext):
+        self.context = context
+        self._ws = None
+
+    def workspace_bytes(self, m: int, n: int, k: int) -> int:
+        return int(_capi.lib().mf_qmm_workspace_bytes(m, n, k))
+
+    def encode(self, weights: QuantizedTensor, x: torch.Tensor, y: torch.Tensor, m: int, n: int, k: int,
+               workspace: Optional[torch.Tensor] = None, stream=None) -> str:
+        if workspace is None:
+            need = self.workspace_bytes(m, n, k)
+            if self._ws is None or self._ws.numel() < need:
+                self._ws = torch.empty(max(need, 256), dtype=torch.uint8, device=x.device)
+            workspace = self._ws
+        st = _capi.lib().mf_qmm(self.context.handle, _stream(stream), weights.c(), weights.bits, _ptr(x), _ptr(y),
+                                m, n, k, 1 if y.dtype == torch.float32 else 0, _ptr(workspace),
+                                workspace.numel() * workspace.element_size())
+        if st in (-1, -2, -3):
+            return "unavailable"
+        check(st, self.context.handle)
+        return "affine-matrix-core-bf16"
+
+
 class Elementwise:
     """Kernels/Primitives/Elementwise.swift:60-87."""
 
@@ -206,6 +234,11 @@ class SharedExpertInt4:
             gate.n, gate.rows, t, _ptr(y), _ptr(scratch_act),
             scratch_act.numel() * scratch_act.element_size()), self.context.handle)
 
+
+    @staticmethod
+    def scratch_bytes(d: int, f: int, t: int) -> int:
+        """bytes of scratch the call can use for t rows (the matrix-core path from 32 rows on)"""
+        return int(_capi.lib().mf_shared_expert_scratch_bytes(d, f, t))
 
     def encode_static(self, x: torch.Tensor, gate: QuantizedTensor, up: QuantizedTensor,
                       down: QuantizedTensor, y: torch.Tensor, t: int = 1, stream=None) -> None:

@@ -249,6 +249,112 @@ def measure_prefill(ctx, w, layer, device, tokens=(128, 512, 2048), steps=100, w
     return out
 
 
+def _omp_threads(n):
+    """thread count of the CPU checker's OpenMP loops (libgomp of this process); None = leave"""
+    import ctypes
+    try:
+        gomp = ctypes.CDLL("libgomp.so.1")
+        prev = gomp.omp_get_max_threads()
+        if n:
+            gomp.omp_set_num_threads(int(n))
+        return prev
+    except OSError:
+        return None
+
+
+def bench_single_expert(args, device) -> int:
+    """One SwiGLU expert FFN at batch 1 (hidden 2048, intermediate 512, 4-bit g64): the shared-expert
+    operator on one expert's projections, `layers` distinct experts in rotation; beside it the CPU checker
+    (a restatement of the reference's CPU path) single-threaded and on all cores."""
+    import numpy as np
+    import torch
+    from mference_amd import operators as ops
+    from oracle import mf_oracle as O
+
+    D, F = 2048, 512
+    L = args.layers or 256  # 256 experts = 453 MB: more than the 256 MB last-level cache holds
+    ctx = ops.MetalContext(0)
+    quant = ops.Quantization(ctx)
+    gen = torch.Generator(device=device)
+    gen.manual_seed((ROOT_SEED + 0x000) & 0x7FFFFFFFFFFFFFFF)
+    big = [quant.quantize_affine(torch.randn((L * r, c), generator=gen, device=device) * 0.02, 4)
+           for r, c in ((F, D), (F, D), (D, F))]
+
+    def view(q, i, rows):
+        return ops.QuantizedTensor(q.packed[i * rows:(i + 1) * rows], q.scales[i * rows:(i + 1) * rows],
+                                   q.biases[i * rows:(i + 1) * rows], 4, rows, q.n)
+    sets = [[view(big[0], i, F), view(big[1], i, F), view(big[2], i, D)] for i in range(L)]
+    mlp = ops.SharedExpertInt4(ctx)
+    x = torch.randn((1, D), generator=gen, device=device).to(torch.bfloat16)
+    y = torch.zeros((L, 1, D), dtype=torch.bfloat16, device=device)
+    scratch = torch.zeros((1, F), dtype=torch.bfloat16, device=device)
+
+    def step():
+        for l in range(L):
+            mlp.encode(x, sets[l][0], sets[l][1], sets[l][2], y[l], scratch, t=1)
+
+    def hq(q):
+        return O.QTensor(q.packed.cpu().numpy(), ops.bf16_bits(q.scales), ops.bf16_bits(q.biases), 4, q.rows, q.n)
+    step()
+    torch.cuda.synchronize()
+    h0 = [hq(q) for q in sets[0]]
+    xb = ops.bf16_bits(x[0])
+    ref = O.bf16_to_float(O.shared_expert(h0[0], h0[1], h0[2], xb)).astype(np.float64)
+    got = O.bf16_to_float(ops.bf16_bits(y[0][0])).astype(np.float64)
+    parity = dict(max_abs=float(np.abs(got - ref).max()), rel_l2=float(np.linalg.norm(got - ref) / np.linalg.norm(ref)))
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        step()
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        step()
+    for _ in range(args.warmup):
+        graph.replay()
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    for _ in range(args.steps):
+        graph.replay()
+    e1.record()
+    torch.cuda.synchronize()
+    us = e0.elapsed_time(e1) / args.steps / L * 1e3
+    nbytes = 3 * (D * F // 2 + 2 * 2 * (D * F // 64))  # 1 769 472
+    achieved = nbytes / (us * 1e-6) / 1e9
+    out = {
+        "metric": "us_per_expert_ffn_T1", "value": round(us, 3), "unit": "us", "n_gpus": 1,
+        "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(us * L / 1e3, 5),
+        "higher_is_better": False, "scaling": "weak", "vs_baseline": None,
+        "dtype": "u4 codes x bf16 activations, fp32 accumulate", "data": "synthetic (N(0,0.02) weights, 4-bit g64; x ~ N(0,1))",
+        "config": {"workload": "single-swiglu-expert-ffn-D2048-F512-T1", "weight_sets": L, "tokens": 1, "launch": "hip_graph"},
+        "parity_set0": parity,
+        "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+                     "frac": round(achieved / HBM_PEAK_GBPS, 4), "traffic": None,
+                     "kernel": "mf::gate_up_act_kernel + mf::gemv_kernel (two launches per expert)",
+                     "algorithmic_bytes": nbytes}}
+    if not args.no_cpu_baseline:
+        all_cores = int(os.environ.get("OMP_NUM_THREADS") or min(16, os.cpu_count() or 1))
+        res = []
+        for threads in (1, all_cores):
+            prev = _omp_threads(threads)
+            n, t0 = 0, time.perf_counter()
+            while True:
+                O.shared_expert(h0[0], h0[1], h0[2], xb)
+                n += 1
+                el = time.perf_counter() - t0
+                if el >= args.cpu_seconds / 2 or n >= 20000:
+                    break
+            _omp_threads(prev)
+            res.append({"value": round(el / n * 1e6, 1), "unit": "us", "cores": threads if prev else 1, "kind": "port",
+                        "sample": f"{n} repetitions of the same expert FFN"})
+        out["cpu_baseline"] = res[1]
+        out["cpu_baseline_single_thread"] = res[0]
+    print(json.dumps(out))
+    return 0
+
+
 def bench_dense_mlp(args, device) -> int:
     """Dense 4-bit SwiGLU MLP (hidden 5120, intermediate 17408) at T token rows: the shared-expert
     operator on a dense layer; `layers` distinct weight sets rotate so HBM is read every step."""
@@ -543,7 +649,7 @@ def main() -> int:
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--layers", type=int, default=None)
     ap.add_argument("--workload", default="qwen-decode",
-                    choices=sorted(WORKLOADS) + ["dense-mlp", "family-routers"],
+                    choices=sorted(WORKLOADS) + ["dense-mlp", "family-routers", "single-expert"],
                     help="qwen-decode is the headline; the others measure the remaining "
                          "configurations of the same path")
     ap.add_argument("--tokens", type=int, default=None, help="token rows per step (decode: 1..8)")
@@ -571,6 +677,8 @@ def main() -> int:
     torch.cuda.set_device(device)
     if args.workload == "dense-mlp":
         return bench_dense_mlp(args, device)
+    if args.workload == "single-expert":
+        return bench_single_expert(args, device)
     if args.workload == "family-routers":
         return bench_family_routers(args, device)
     w = dict(WORKLOADS[args.workload])
@@ -727,6 +835,18 @@ def main() -> int:
                                "kind": "port",
                                "sample": f"{n} repetitions of layer 0 of the same workload "
                                          f"(OpenMP over weight rows, {cores} threads)"}
+        prev = _omp_threads(1)  # the same on one core
+        if prev:
+            n1, t1 = 0, time.perf_counter()
+            while True:
+                O.moe_layer(host0, xb)
+                n1 += 1
+                el1 = time.perf_counter() - t1
+                if el1 >= args.cpu_seconds / 3 or n1 >= 2000:
+                    break
+            _omp_threads(prev)
+            out["cpu_baseline_single_thread"] = {"value": round(el1 / n1 * 1e6, 1), "unit": "us", "cores": 1,
+                                                 "kind": "port", "sample": f"{n1} repetitions of layer 0, one thread"}
     if args.pmc_calibration:
         out["pmc_calibration"] = pmc_calibration(device)
     print(json.dumps(out))

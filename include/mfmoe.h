@@ -130,7 +130,13 @@ mf_status mf_dequantize(mf_ctx* ctx, mf_stream stream, mf_qtensor q, size_t rows
  * DequantInt4GEMVMultiX.encode (Kernels/Quant/DequantInt4GEMVMultiX.swift:48-82)
  * for 1 < t <= 8, MapleTernaryGEMV.encode (Kernels/Quant/MapleTernaryGEMV.swift:
  * 29-45) for ternary.  x bf16 [t, n], y [t, m] bf16 or fp32 (out_f32 != 0,
- * the _f32out kernels).  Each weight row is read once for all t tokens. */
+ * the _f32out kernels).  Each weight row is read once for all t tokens.
+ * Two storages of ternary weights exist in the reference.  Routed experts pack four 2-bit codes
+ * per byte with a scale table only (RepackPlanner.swift:560-651): MF_BITS_TERNARY.  The resident
+ * projections MapleTernaryGEMV reads keep the same codes widened to nibbles, with a scale (alpha)
+ * and a bias (-alpha) table repeated over each source group of 128 (RepackPlanner.swift:414-470,
+ * Metal/Quant/maple_ternary.metal:12-15, 59-69): that is a 4-bit affine tensor whose codes happen
+ * to be 0, 1, 2 -- pass it as MF_BITS_4. */
 mf_status mf_gemv(mf_ctx* ctx, mf_stream stream, mf_qtensor w, mf_bits bits, const uint16_t* x,
                   void* y, uint32_t m, uint32_t n, uint32_t t, int out_f32);
 

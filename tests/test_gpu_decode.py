@@ -551,3 +551,91 @@ def test_silu_mul_matches_oracle(gpu, oracle, count):
     got = ops.bf16_bits(out)
     assert np.array_equal(got[:count], ref)
     assert np.all(got[count:] == 0x3F80)  # nothing written past count
+
+
+def test_nibble_widened_ternary_gemv_exact_bits(gpu, oracle):
+    """MapleTernaryGEMV.encode on the resident projections' storage (maple_ternary.metal:12-81): ternary
+    codes widened to nibbles with scale (alpha) and bias (-alpha) tables repeated over each source group
+    of 128 -- a 4-bit affine tensor, so mf_gemv reads it as MF_BITS_4.  The reference's own vector
+    (MapleTernaryGEMVTests.swift:61-134): codes (row*5 + index*3) & 3, alpha = (row+1)(source+1)/8,
+    x = (index*7) % 13 - 6, nine rows (a tail of one past two blocks of four), every buffer entered at an
+    offset; all values are small exact numbers, so the expected bf16 bits do not depend on summation order."""
+    d, rows, groups = 2048, 9, 2048 // 64
+    idx = np.arange(d)
+    codes = ((np.arange(rows)[:, None] * 5 + idx[None, :] * 3) & 3).astype(np.uint8)
+    packed = (codes[:, 0::2] | (codes[:, 1::2] << 4)).astype(np.uint8)
+    alpha = ((np.arange(rows)[:, None] + 1) * (np.arange(groups // 2)[None, :] + 1) / 8.0).astype(np.float32)
+    scales = np.repeat(oracle.bf16_bits(alpha), 2, axis=1)
+    biases = np.repeat(oracle.bf16_bits(-alpha), 2, axis=1)
+    x = ((idx * 7) % 13 - 6).astype(np.float32)
+    xb = oracle.bf16_bits(x)
+    # ternaryReference (:357-378) in exact arithmetic
+    xs = oracle.bf16_to_float(xb).astype(np.float64)
+    s = np.repeat(oracle.bf16_to_float(scales), 64, axis=1).astype(np.float64)
+    b = np.repeat(oracle.bf16_to_float(biases), 64, axis=1).astype(np.float64)
+    total = ((codes.astype(np.float64) * s + b) * xs[None, :]).sum(axis=1)
+    assert np.all(total == total.astype(np.float32))  # exactly representable: any order gives these bits
+    expected = oracle.bf16_bits(total.astype(np.float32))
+
+    def at_offset(arr, prefix_bytes, fill):
+        raw = np.ascontiguousarray(arr).view(np.uint8).reshape(-1)
+        buf = torch.full((prefix_bytes + raw.size + 6,), fill, dtype=torch.uint8, device="cuda")
+        buf[prefix_bytes:prefix_bytes + raw.size] = torch.from_numpy(raw.copy()).cuda()
+        return buf, buf[prefix_bytes:prefix_bytes + raw.size]
+
+    kw, wd = at_offset(packed, 1, 0xA5)        # weightsOffset 1
+    ks, sd = at_offset(scales, 6, 0xA5)        # 3 parameters in
+    kb, bd = at_offset(biases, 6, 0xA5)
+    kx, xd = at_offset(xb, 8, 0xA5)            # 4 activations in
+    y = torch.full((5 + rows + 3,), 0, dtype=torch.int16, device="cuda")
+    y[:] = 0x7BAD
+    q = ops.QuantizedTensor(wd, sd.view(torch.bfloat16), bd.view(torch.bfloat16), ops.BITS_4, rows, d)
+    ops.DequantInt4GEMV(gpu).encode(q, xd.view(torch.bfloat16), y[5:5 + rows].view(torch.bfloat16), rows, d)
+    _sync()
+    got = y.cpu().numpy().view(np.uint16)
+    assert np.all(got[:5] == 0x7BAD) and np.all(got[5 + rows:] == 0x7BAD)
+    assert np.array_equal(got[5:5 + rows], expected)
+
+
+def test_single_expert_ffn_at_full_size(gpu, oracle):
+    """One SwiGLU expert FFN at batch 1, hidden 2048 / intermediate 512, weights N(0, 0.02) quantized
+    4-bit g64, x ~ N(0, 1) (the CPU-runnable configuration): as the shared-expert operator
+    (gate and up narrowed before the activation, dequant_int4.metal:240-245) against the checker's
+    shared expert, and as a routed expert through the two phases with K = 1, weight 1, no residual
+    (gate and up kept fp32, moe.metal:526-528, 1262-1270) against the checker's phase functions."""
+    d, f = 2048, 512
+    rng = oracle.Rng.key(ROOT_SEED + 0x000, "single-expert")
+    gq = oracle.quantize(rng.normal(0.0, 0.02, f * d).reshape(f, d), 4)
+    uq = oracle.quantize(rng.normal(0.0, 0.02, f * d).reshape(f, d), 4)
+    dq = oracle.quantize(rng.normal(0.0, 0.02, d * f).reshape(d, f), 4)
+    xb = oracle.bf16_bits(rng.normal(0.0, 1.0, d))
+    x = ops.bf16_tensor(xb.reshape(1, d))
+    # shared-expert form
+    y = torch.zeros((1, d), dtype=torch.bfloat16, device="cuda")
+    scratch = torch.zeros((1, f), dtype=torch.bfloat16, device="cuda")
+    ops.SharedExpertInt4(gpu).encode(x, to_device_q(gq), to_device_q(uq), to_device_q(dq), y, scratch, t=1)
+    _sync()
+    assert_layer_close(oracle.bf16_to_float(ops.bf16_bits(y)[0]), oracle.bf16_to_float(oracle.shared_expert(gq, uq, dq, xb)),
+                       "single expert, shared form")
+    # routed form: one blob in the reference's order, K = 1
+    off, blob_bytes, stride = ops.expert_blob_layout(d, f, 4, 16384)
+    assert blob_bytes == 1769472
+    blob = np.zeros(stride, np.uint8)
+    ooff = oracle.ExpertOffsets()
+    for name, _ in off._fields_:
+        setattr(ooff, name, getattr(off, name))
+    oracle.pack_expert_blob(gq, uq, dq, ooff, blob)
+    moe = ops.MoE(gpu, d, f, 1, 1, bits=4)
+    experts = torch.from_numpy(blob.reshape(1, stride)).cuda()
+    idx = torch.zeros((1, 1), dtype=torch.int32, device="cuda")
+    w = torch.ones((1, 1), dtype=torch.float32, device="cuda")
+    acts = torch.zeros((1, 1, f), dtype=torch.bfloat16, device="cuda")
+    y2 = torch.zeros((1, d), dtype=torch.bfloat16, device="cuda")
+    moe.encode_routed_phase1(experts, off, idx, x, acts)
+    moe.encode_routed_phase2_reduce(experts, off, idx, w, acts, None, y2)
+    _sync()
+    ref_acts = oracle.expert_phase1(blob, ooff, 4, d, f, xb)
+    assert np.array_equal(ops.bf16_bits(acts).reshape(-1), ref_acts) or \
+        np.abs(oracle.bf16_to_float(ops.bf16_bits(acts).reshape(-1)) - oracle.bf16_to_float(ref_acts)).max() <= 2e-2
+    ref_y = oracle.bf16_bits(oracle.expert_down(blob, ooff, 4, d, f, ref_acts))
+    assert_layer_close(oracle.bf16_to_float(ops.bf16_bits(y2)[0]), oracle.bf16_to_float(ref_y), "single expert, routed form")

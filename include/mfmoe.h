@@ -451,6 +451,35 @@ mf_status mf_moe_prefill_layer(mf_moe* h, mf_stream stream, const mf_moe_layer_w
                                const uint16_t* x, uint32_t t, uint16_t* y, void* workspace,
                                size_t workspace_bytes, uint32_t* out_idx, float* out_w);
 
+
+/* The two halves of the ragged layer on their own, for callers that hold a grouping already.
+ *
+ * mf_moe_ragged_qmm: PrefillGroupedRoutedMoE.encodeStreamedBatched (Kernels/Prefill/MoE/
+ * PrefillGroupedRoutedMoE.swift:392-466): for every route of `sorted_pairs` (mf_moe_group's output:
+ * the routes of expert 0, then expert 1, ..., expert_counts[e] of them each, starting at 0) the routed
+ * expert's gate/up -> SwiGLU -> down result as fp32 in route_partials[(token * top_k + rank), d], the
+ * row order the reference's down kernel writes (prefill.metal route_partials).  Rows of routes that are
+ * not in the grouping are left untouched.  The reference walks the pairs in micro-batches of 32 rows
+ * per dispatch pair; here one launch per projection covers every tile of every expert.  The counts
+ * and pairs are checked on the device before they are trusted (sum of counts <= t * top_k, token < t,
+ * rank < top_k): a grouping that fails computes nothing and mf_moe_group_status returns
+ * MF_ERR_EXPERT_RANGE.  Needs the matrix-core configuration (mf_moe_prefill_workspace_bytes(h, t) != 0),
+ * else MF_ERR_DIMENSION_MISMATCH; workspace as for mf_moe_prefill_layer.
+ *
+ * mf_moe_unpermute: PrefillMoE.encodeReduceTokenMajor (Kernels/Prefill/MoE/PrefillMoE.swift:11-38,
+ * Metal/Prefill/prefill.metal:631-652): y[token, :] = sum over ranks of route_weights[token, rank] *
+ * route_partials[token * top_k + rank, :], accumulated in fp32 in rank order, stored as bf16.
+ * idx (nullable) [t, top_k]: routes whose expert index is >= num_experts are skipped, as the layer call
+ * skips them; residual (nullable) [t, d] bf16 is the value the sum starts from (the shared expert's
+ * output in the layer call). */
+mf_status mf_moe_ragged_qmm(mf_moe* h, mf_stream stream, const void* expert_base, size_t expert_stride,
+                            const mf_expert_offsets* offsets, const uint16_t* x,
+                            const mf_pair* sorted_pairs, const uint32_t* expert_counts, uint32_t t,
+                            float* route_partials, void* workspace, size_t workspace_bytes);
+mf_status mf_moe_unpermute(mf_moe* h, mf_stream stream, const float* route_partials,
+                           const float* route_weights, const uint32_t* idx, const uint16_t* residual,
+                           uint32_t t, uint16_t* y);
+
 #ifdef __cplusplus
 }
 #endif

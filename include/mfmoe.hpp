@@ -327,6 +327,21 @@ class MoE {
           ctx_);
   }
   void groupStatus(mf_stream cb) const { check(mf_moe_group_status(h_, cb), ctx_); }
+  // PrefillGroupedRoutedMoE.encodeStreamedBatched (PrefillGroupedRoutedMoE.swift:392-466) over a
+  // grouping the caller holds; routePartials is fp32 [tokens * topK, d], row token * topK + rank
+  void encodeStreamedBatched(mf_stream cb, const void* expertBase, size_t expertStride,
+                             const mf_expert_offsets& offsets, const uint16_t* hidden,
+                             const mf_pair* sortedPairs, const uint32_t* expertCounts, uint32_t tokens,
+                             float* routePartials, void* workspace, size_t workspaceBytes) const {
+    check(mf_moe_ragged_qmm(h_, cb, expertBase, expertStride, &offsets, hidden, sortedPairs, expertCounts,
+                            tokens, routePartials, workspace, workspaceBytes), ctx_);
+  }
+  // PrefillMoE.encodeReduceTokenMajor (PrefillMoE.swift:11-38)
+  void encodeReduceTokenMajor(mf_stream cb, const float* routePartials, const float* routeWeights,
+                              uint16_t* h2, uint32_t tokens, const uint32_t* indices = nullptr,
+                              const uint16_t* residual = nullptr) const {
+    check(mf_moe_unpermute(h_, cb, routePartials, routeWeights, indices, residual, tokens, h2), ctx_);
+  }
   void setFused(bool enabled) const { check(mf_moe_set_fused(h_, enabled ? 1 : 0), ctx_); }
   void status(mf_stream cb) const { check(mf_moe_status(h_, cb), ctx_); }
 

@@ -40,6 +40,11 @@ def build(verbose: bool = False, only: list[str] | None = None) -> str:
     hipcc = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
     os.makedirs(OBJ, exist_ok=True)
     objs = [os.path.join(OBJ, s.replace(".hip", ".o")) for s in SOURCES]
+    if only is not None:
+        only = [s if s.endswith(".hip") else s + ".hip" for s in only]
+        unknown = [s for s in only if s not in SOURCES]
+        if unknown:
+            raise ValueError(f"not a source of the library: {unknown}")
     todo = [(s, o) for s, o in zip(SOURCES, objs) if only is None or s in only or not os.path.exists(o)]
     jobs = min(8, max(1, (os.cpu_count() or 2) // 2))
     with ThreadPoolExecutor(jobs) as pool:

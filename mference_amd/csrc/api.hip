@@ -654,6 +654,41 @@ mf_status mf_moe_prefill_layer(mf_moe* h, mf_stream stream, const mf_moe_layer_w
   return MF_OK;
 }
 
+mf_status mf_moe_ragged_qmm(mf_moe* h, mf_stream stream, const void* expert_base, size_t expert_stride,
+                            const mf_expert_offsets* offsets, const uint16_t* x, const mf_pair* sorted_pairs,
+                            const uint32_t* expert_counts, uint32_t t, float* route_partials, void* workspace,
+                            size_t workspace_bytes) {
+  if (!h || !offsets || !x || !sorted_pairs || !expert_counts || !route_partials || !expert_base)
+    return MF_ERR_INVALID_ARGUMENT;
+  if (t == 0 || t > (1u << 20)) return MF_ERR_QUERY_COUNT;
+  const mf_moe_config& c = h->cfg;
+  if (!mf::prefill_supported(c)) return MF_ERR_DIMENSION_MISMATCH;
+  if (!workspace) return MF_ERR_INVALID_ARGUMENT;
+  if (workspace_bytes < mf::prefill_workspace_bytes(c, t)) return MF_ERR_SCRATCH_TOO_SMALL;
+  const uint32_t offs = offsets->gate_w | offsets->up_w | offsets->down_w;
+  if (!offsets_ok(*offsets, c.bits) || !mf::aligned16(expert_base) || expert_stride % 16 || offs % 16 ||
+      !mf::aligned16(x) || !mf::aligned16(route_partials) || !mf::aligned16(workspace) ||
+      reinterpret_cast<uintptr_t>(sorted_pairs) % 16)
+    return MF_ERR_INVALID_ARGUMENT;
+  MF_HIP(h->ctx, mf::launch_ragged_qmm(static_cast<hipStream_t>(stream), *h, expert_base, expert_stride, *offsets,
+                                       x, sorted_pairs, expert_counts, t, route_partials, workspace));
+  return MF_OK;
+}
+
+mf_status mf_moe_unpermute(mf_moe* h, mf_stream stream, const float* route_partials, const float* route_weights,
+                           const uint32_t* idx, const uint16_t* residual, uint32_t t, uint16_t* y) {
+  if (!h || !route_partials || !route_weights || !y) return MF_ERR_INVALID_ARGUMENT;
+  if (t == 0 || t > (1u << 20)) return MF_ERR_QUERY_COUNT;
+  const mf_moe_config& c = h->cfg;
+  if (c.d % 4) return MF_ERR_DIMENSION_MISMATCH;
+  if (!mf::aligned16(route_partials) || reinterpret_cast<uintptr_t>(y) % 8 ||
+      (residual && reinterpret_cast<uintptr_t>(residual) % 8))
+    return MF_ERR_INVALID_ARGUMENT;
+  MF_HIP(h->ctx, mf::launch_unpermute(static_cast<hipStream_t>(stream), c, route_partials, route_weights, idx,
+                                      residual, t, y));
+  return MF_OK;
+}
+
 mf_status mf_group_pairs_host(const mf_pair* pairs, size_t n_pairs, int query_count, int top_k,
                               int num_experts, int tile_expert_count,
                               const uint64_t* sort_keys, size_t n_sort_keys, mf_pair* sorted,

@@ -136,6 +136,11 @@ bool prefill_supported(const mf_moe_config& c);
 hipError_t launch_prefill_layer(hipStream_t s, const mf_moe& h, const mf_moe_layer_weights& w,
                                 const uint16_t* x, uint32_t t, uint16_t* y, void* workspace,
                                 uint32_t* out_idx, float* out_w);
+hipError_t launch_ragged_qmm(hipStream_t s, const mf_moe& h, const void* expert_base, size_t expert_stride,
+                             const mf_expert_offsets& off, const uint16_t* x, const mf_pair* sorted,
+                             const uint32_t* counts, uint32_t t, float* partials, void* workspace);
+hipError_t launch_unpermute(hipStream_t s, const mf_moe_config& c, const float* partials, const float* w,
+                            const uint32_t* idx, const uint16_t* residual, uint32_t t, uint16_t* y);
 // dense projections over many rows through the matrix-core matmul (moe_prefill.hip)
 bool dense_qmm_takes(const mf_qtensor& w, int bits, const void* x, const void* y, uint32_t m, uint32_t n, uint32_t k);
 size_t dense_qmm_workspace_bytes(uint32_t m, uint32_t n, uint32_t k);

@@ -263,15 +263,15 @@ __global__ __launch_bounds__(512) void group_scan_kernel(uint32_t* __restrict__ 
                                                          uint32_t tile_slots,
                                                          uint32_t* __restrict__ n_tiles,
                                                          const uint32_t* __restrict__ chunk_bad,
-                                                         uint32_t* __restrict__ status) {
+                                                         uint32_t* __restrict__ status,
+                                                         int drop_if_bad = 0) {
   __shared__ uint32_t s_cnt[MF_MAX_EXPERTS], s_tile[MF_MAX_EXPERTS];
   const uint32_t e = threadIdx.x;
-  {  // status word: 2 when any chunk met an expert index out of range (n_chunks <= blockDim)
-    const int any_bad = __syncthreads_or(e < n_chunks && chunk_bad[e] ? 1 : 0);
-    if (e == 0) *status = any_bad ? 2u : 0u;
-  }
+  // status word: 2 when any chunk met an expert index out of range (n_chunks <= blockDim)
+  const int any_bad = __syncthreads_or(e < n_chunks && chunk_bad[e] ? 1 : 0);
+  if (e == 0) *status = any_bad ? 2u : 0u;
   uint32_t c = 0;
-  if (e < E) {
+  if (e < E && !(any_bad && drop_if_bad)) {  // a caller's grouping that failed its check yields no tiles
     uint32_t k = 0;
     for (; k + 32 <= n_chunks; k += 32) {  // 32 independent loads in flight: the loop is all latency
       uint32_t v[32];
@@ -288,8 +288,8 @@ __global__ __launch_bounds__(512) void group_scan_kernel(uint32_t* __restrict__ 
       chunk_hist[k * E + e] = c;
       c += v;
     }
-    counts[e] = c;
   }
+  if (e < E) counts[e] = c;
   s_cnt[e] = c;
   s_tile[e] = (c + kTileTokens - 1) / kTileTokens;
   __syncthreads();
@@ -1215,7 +1215,7 @@ __global__ __launch_bounds__(256) void prefill_reduce_kernel(const float* __rest
     }
   }
   for (uint32_t r = 0; r < K; ++r) {
-    if (idx[t * K + r] >= E) continue;
+    if (idx && idx[t * K + r] >= E) continue;  // a route without an expert adds nothing
     const float wt = w[t * K + r];
     float4 v = *reinterpret_cast<const float4*>(partials + (static_cast<size_t>(t) * K + r) * D + d);
     if (maple) {  // maple_moe.metal:258: the down output is a bf16 number before its weight
@@ -1228,6 +1228,33 @@ __global__ __launch_bounds__(256) void prefill_reduce_kernel(const float* __rest
   o.x = static_cast<uint32_t>(f_to_bf16(acc[0])) | (static_cast<uint32_t>(f_to_bf16(acc[1])) << 16);
   o.y = static_cast<uint32_t>(f_to_bf16(acc[2])) | (static_cast<uint32_t>(f_to_bf16(acc[3])) << 16);
   *reinterpret_cast<uint2*>(y + i4) = o;
+}
+
+// A caller's grouping before the matmuls trust it: the counts cover at most T*K routes, and every
+// route the counts cover names a token below T and a rank below K.  Sets *bad otherwise.
+__global__ __launch_bounds__(256) void ragged_check_kernel(const mf_pair* __restrict__ sorted,
+                                                           const uint32_t* __restrict__ counts,
+                                                           uint32_t E, uint32_t T, uint32_t K,
+                                                           uint32_t* __restrict__ bad) {
+  __shared__ unsigned long long s_total;
+  if (threadIdx.x == 0) s_total = 0;
+  __syncthreads();
+  unsigned long long part = 0;
+  for (uint32_t e = threadIdx.x; e < E; e += blockDim.x) part += counts[e];
+  if (part) atomicAdd(&s_total, part);
+  __syncthreads();
+  const unsigned long long total = s_total, pairs = static_cast<unsigned long long>(T) * K;
+  if (total > pairs) {
+    if (blockIdx.x == 0 && threadIdx.x == 0) atomicOr(bad, 1u);
+    return;
+  }
+  bool wrong = false;
+  for (size_t i = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x; i < total;
+       i += static_cast<size_t>(gridDim.x) * blockDim.x) {
+    const mf_pair p = sorted[i];
+    wrong |= p.token >= T || p.rank >= K;
+  }
+  if (wrong) atomicOr(bad, 1u);
 }
 
 // ------------------------------------------------------------------ launchers
@@ -1610,11 +1637,45 @@ bool prefill_supported(const mf_moe_config& c) {
   return true;
 }
 
+struct RaggedOnly {
+  const mf_pair* sorted;    // [t * top_k] by (expert, token, rank)
+  const uint32_t* counts;   // [num_experts]
+  float* partials;          // [t * top_k, d] fp32, row token * top_k + rank
+};
 hipError_t launch_prefill_layer(hipStream_t s, const mf_moe& h, const mf_moe_layer_weights& w,
                                 const uint16_t* x, uint32_t t, uint16_t* y, void* workspace,
-                                uint32_t* out_idx, float* out_w) {
-  const mf_moe_config& c = h.cfg;
-  PrefillWs ws = prefill_carve(c, t, workspace);
+                                uint32_t* out_idx, float* out_w, const RaggedOnly* ragged);
+
+// The routed experts alone over a grouping the caller holds (sorted pairs + per-expert counts):
+// PrefillGroupedRoutedMoE.encodeStreamedBatched.  Runs the layer call's matmul launches and stops
+// before the un-permute; the per-route results go to the caller's fp32 buffer.
+hipError_t launch_ragged_qmm(hipStream_t s, const mf_moe& h, const void* expert_base, size_t expert_stride,
+                             const mf_expert_offsets& off, const uint16_t* x, const mf_pair* sorted,
+                             const uint32_t* counts, uint32_t t, float* partials, void* workspace) {
+  RaggedOnly r{sorted, counts, partials};
+  mf_moe_layer_weights w{};
+  w.expert_base = expert_base;
+  w.expert_stride = expert_stride;
+  w.offsets = off;
+  return launch_prefill_layer(s, h, w, x, t, nullptr, workspace, nullptr, nullptr, &r);
+}
+
+hipError_t launch_unpermute(hipStream_t s, const mf_moe_config& c, const float* partials, const float* w,
+                            const uint32_t* idx, const uint16_t* residual, uint32_t t, uint16_t* y) {
+  const size_t n4 = static_cast<size_t>(t) * c.d / 4;
+  if (!n4) return hipSuccess;
+  prefill_reduce_kernel<<<dim3(static_cast<uint32_t>((n4 + 255) / 256)), dim3(256), 0, s>>>(
+      partials, w, idx, residual, nullptr, y, t, c.top_k, c.d, c.num_experts, static_cast<int>(c.maple_rounding));
+  return hipGetLastError();
+}
+
+hipError_t launch_prefill_layer(hipStream_t s, const mf_moe& h, const mf_moe_layer_weights& w,
+                                const uint16_t* x, uint32_t t, uint16_t* y, void* workspace,
+                                uint32_t* out_idx, float* out_w, const RaggedOnly* ragged) {
+  const mf_moe_config& cfg_in = h.cfg;
+  mf_moe_config c = cfg_in;
+  if (ragged) c.shared_f = 0;  // the routed experts only
+  PrefillWs ws = prefill_carve(cfg_in, t, workspace);
   // the caller's routing outputs, when given, are the routing buffers of the whole call
   if (out_idx) ws.idx = out_idx;
   if (out_w) ws.w = out_w;
@@ -1622,12 +1683,31 @@ hipError_t launch_prefill_layer(hipStream_t s, const mf_moe& h, const mf_moe_lay
 #define MF_TRY(call) do { e = (call); if (e != hipSuccess) return e; } while (0)
   const size_t pairs = static_cast<size_t>(t) * c.top_k;
   const uint32_t max_tiles = prefill_tile_slots(c, t);
-  if (w.router_w) {  // else the routing in out_idx / out_w is the caller's
-    MF_TRY(launch_prefill_router(s, w.router_w, x, c.num_experts, c.d, t, c.d, ws.logits));
-    MF_TRY(launch_topk(s, ws.logits, c.num_experts, c.top_k, t, c.router_mode, ws.idx, ws.w));
+  if (ragged) {
+    // the caller's grouping: its per-expert counts are a one-chunk histogram for the scan that lays
+    // out the tile list (the runs start at 0 in expert order, as mf_moe_group writes them)
+    uint32_t* hist = h.ws.group_tmp + 2048;
+    uint32_t* bad = hist + static_cast<size_t>(kGroupChunks) * MF_MAX_EXPERTS;
+    ws.status = h.ws.group_tmp + 3 * 512;  // the word mf_moe_group_status reads
+    MF_TRY(hipMemcpyAsync(hist, ragged->counts, sizeof(uint32_t) * c.num_experts, hipMemcpyDeviceToDevice, s));
+    MF_TRY(hipMemsetAsync(bad, 0, sizeof(uint32_t), s));
+    const uint32_t check_wgs = static_cast<uint32_t>(std::min<size_t>((pairs + 255) / 256, 2048));
+    ragged_check_kernel<<<dim3(std::max(check_wgs, 1u)), dim3(256), 0, s>>>(ragged->sorted, ragged->counts, c.num_experts,
+                                                                           t, c.top_k, bad);
+    MF_TRY(hipGetLastError());
+    group_scan_kernel<<<dim3(1), dim3(MF_MAX_EXPERTS), 0, s>>>(hist, 1, c.num_experts, ws.counts, ws.offsets, ws.starts,
+                                                               ws.tiles, max_tiles, ws.n_tiles, bad, ws.status, 1);
+    MF_TRY(hipGetLastError());
+    ws.sorted = const_cast<mf_pair*>(ragged->sorted);
+    ws.partials = ragged->partials;
+  } else {
+    if (w.router_w) {  // else the routing in out_idx / out_w is the caller's
+      MF_TRY(launch_prefill_router(s, w.router_w, x, c.num_experts, c.d, t, c.d, ws.logits));
+      MF_TRY(launch_topk(s, ws.logits, c.num_experts, c.top_k, t, c.router_mode, ws.idx, ws.w));
+    }
+    MF_TRY(launch_group(s, ws.idx, ws.w, t, c.top_k, c.num_experts, ws.counts, ws.offsets, ws.starts,
+                        ws.sorted, ws.tiles, max_tiles, ws.n_tiles, ws.status, h.ws.group_tmp + 2048));
   }
-  MF_TRY(launch_group(s, ws.idx, ws.w, t, c.top_k, c.num_experts, ws.counts, ws.offsets, ws.starts,
-                      ws.sorted, ws.tiles, max_tiles, ws.n_tiles, ws.status, h.ws.group_tmp + 2048));
 
   const bool want_gate = c.shared_f && w.w_sg;
   if (want_gate) {  // one pass over x: matmul order, group sums and the shared gate's logits
@@ -1706,6 +1786,7 @@ hipError_t launch_prefill_layer(hipStream_t s, const mf_moe& h, const mf_moe_lay
       else MF_TRY(launch_qmm(s, 4, d, d.pair_rows ? 2 : 1, dense_tiles, nullptr, 0));
     }
   }
+  if (ragged) return hipSuccess;  // the per-route results are the caller's: mf_moe_unpermute reduces them
   const uint16_t* hs = nullptr;
   const uint16_t* gate = nullptr;
   if (c.shared_f) {
@@ -1718,6 +1799,12 @@ hipError_t launch_prefill_layer(hipStream_t s, const mf_moe& h, const mf_moe_lay
   MF_TRY(hipGetLastError());
 #undef MF_TRY
   return hipSuccess;
+}
+
+hipError_t launch_prefill_layer(hipStream_t s, const mf_moe& h, const mf_moe_layer_weights& w,
+                                const uint16_t* x, uint32_t t, uint16_t* y, void* workspace,
+                                uint32_t* out_idx, float* out_w) {
+  return launch_prefill_layer(s, h, w, x, t, y, workspace, out_idx, out_w, nullptr);
 }
 
 }  // namespace mf

@@ -454,6 +454,32 @@ class MoE:
         return workspace
 
 
+    def encode_streamed_batched(self, experts: torch.Tensor, offsets: ExpertOffsets, hidden, sorted_pairs,
+                                expert_counts, route_partials, t: int, workspace=None, stream=None):
+        """PrefillGroupedRoutedMoE.encodeStreamedBatched (PrefillGroupedRoutedMoE.swift:392-466): the
+        routed experts over a grouping the caller holds (encode_group's sorted pairs and counts).
+        route_partials: float32 [t * top_k, d], row token * top_k + rank.  A grouping that fails the
+        device check computes nothing and group_status() raises."""
+        if experts.dim() != 2:
+            raise ValueError("experts must be a 2-D uint8 pool [num_experts, blob_stride]")
+        if workspace is None:
+            workspace = torch.empty(max(self.prefill_workspace_bytes(t), 16), dtype=torch.uint8,
+                                    device=hidden.device)
+        check(_capi.lib().mf_moe_ragged_qmm(self._h, _stream(stream), _ptr(experts), experts.stride(0),
+                                            C.byref(offsets), _ptr(hidden), _ptr(sorted_pairs),
+                                            _ptr(expert_counts), t, _ptr(route_partials),
+                                            _ptr(workspace), workspace.numel()), self.context.handle)
+        return workspace
+
+    def encode_reduce_token_major(self, route_partials, route_weights, h2, t: int, indices=None,
+                                  residual=None, stream=None):
+        """PrefillMoE.encodeReduceTokenMajor (PrefillMoE.swift:11-38): h2[token] = sum over ranks of
+        route_weights[token, rank] * route_partials[token * top_k + rank] (+ residual), bf16."""
+        check(_capi.lib().mf_moe_unpermute(self._h, _stream(stream), _ptr(route_partials),
+                                           _ptr(route_weights), _ptr(indices), _ptr(residual), t,
+                                           _ptr(h2)), self.context.handle)
+
+
 PAIR_DTYPE = np.dtype([("token", "<u4"), ("expert", "<u4"), ("rank", "<u4"),
                        ("weight_bits", "<u4")])
 GROUP_DTYPE = np.dtype([("expert", "<u4"), ("pair_start", "<u4"), ("pair_count", "<u4")])

@@ -366,7 +366,20 @@ typedef struct {
  * phases) with no host readback between router and experts.
  * x, y bf16 [t, d], t <= MF_MAX_TOKENS; out_idx / out_w may be NULL.
  * If `hidden` is not NULL, hidden[t,d] = bf16(hidden + y) is applied in the same
- * launch (residual_add_fp16, utility.metal:83-92). */
+ * launch (residual_add_fp16, utility.metal:83-92).
+ *
+ * What the caller owes the fused launch.  It is one workgroup per compute unit, and the workgroups
+ * hand each other the router logits and the routed activations through device memory while they
+ * run, so all of them must be on the device at the same time: while it runs, nothing else may
+ * occupy compute units of this device -- no kernel on another stream, no other process on the
+ * card.  Launches on ONE stream (or one captured graph) keep the contract by themselves.  A
+ * workgroup that waits for a neighbour that never started gives up after a bounded spin (about
+ * 0.1 s), writes NaN to every element of y it owns, leaves `hidden` untouched and records the
+ * event; mf_moe_status then returns MF_ERR_LAUNCH.  So a y of NaN with a finite x means: check
+ * mf_moe_status.  An engine that overlaps this layer with kernels on other streams (attention,
+ * copies done by kernels) calls mf_moe_set_fused(h, 0) once and gets the chain of ordinary
+ * launches, which have no such requirement and give the same bits.  Two handles used at the same
+ * time on two streams of one device fall under the same rule. */
 mf_status mf_moe_decode_layer(mf_moe* h, mf_stream stream, const mf_moe_layer_weights* wts,
                               const uint16_t* x, uint32_t t, uint16_t* y, uint16_t* hidden,
                               uint32_t* out_idx, float* out_w);
@@ -391,7 +404,9 @@ mf_status mf_moe_set_phase_trace(mf_moe* h, uint64_t* device_buffer, size_t byte
 int mf_ctx_num_cu(const mf_ctx* ctx);
 
 /* Synchronises `stream` and reports whether any fused launch of this handle
- * gave up waiting for data of another workgroup (MF_ERR_LAUNCH) since the handle was created.
+ * gave up waiting for data of another workgroup (MF_ERR_LAUNCH) since the handle was created
+ * (the outputs of such a launch are NaN, see mf_moe_decode_layer; mf_last_hip_error names the
+ * status word).  MF_OK means every fused launch so far ran to the end.
  * No counterpart in the reference (Metal reports this through
  * MTLCommandBuffer.error). */
 mf_status mf_moe_status(mf_moe* h, mf_stream stream);

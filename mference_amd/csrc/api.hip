@@ -587,9 +587,9 @@ mf_status mf_moe_group(mf_moe* h, mf_stream stream, const uint32_t* idx, const f
   if (!h || !expert_offsets || !expert_counts) return MF_ERR_INVALID_ARGUMENT;
   auto s = static_cast<hipStream_t>(stream);
   if (t == 0) {  // queryCount == 0 is valid (PrefillMoEGrouping.swift:99-104): no pairs, every expert empty
-    MF_HIP(h->ctx, hipMemsetAsync(expert_counts, 0, sizeof(uint32_t) * h->cfg.num_experts, s));
-    MF_HIP(h->ctx, hipMemsetAsync(expert_offsets, 0xFF, sizeof(uint32_t) * h->cfg.num_experts, s));
-    MF_HIP(h->ctx, hipMemsetAsync(h->ws.group_tmp + 3 * 512, 0, sizeof(uint32_t), s));
+    MF_HIP(h->ctx, mf::launch_group(s, nullptr, nullptr, 0, h->cfg.top_k, h->cfg.num_experts, expert_counts,
+                                    expert_offsets, h->ws.group_tmp + 512, nullptr, nullptr, 0, nullptr,
+                                    h->ws.group_tmp + 3 * 512, h->ws.group_tmp + 2048));
     return MF_OK;
   }
   if (!idx || !w || !sorted_pairs) return MF_ERR_INVALID_ARGUMENT;

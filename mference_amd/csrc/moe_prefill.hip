@@ -1230,6 +1230,14 @@ __global__ __launch_bounds__(256) void prefill_reduce_kernel(const float* __rest
   *reinterpret_cast<uint2*>(y + i4) = o;
 }
 
+// The caller's counts as the one-chunk histogram of the scan, and the check's flag cleared (a kernel,
+// not a memset or a copy node, so that the call can be captured into a graph).
+__global__ __launch_bounds__(512) void ragged_begin_kernel(const uint32_t* __restrict__ counts, uint32_t E,
+                                                           uint32_t* __restrict__ hist, uint32_t* __restrict__ bad) {
+  if (threadIdx.x < E) hist[threadIdx.x] = counts[threadIdx.x];
+  if (threadIdx.x == 0) *bad = 0;
+}
+
 // A caller's grouping before the matmuls trust it: the counts cover at most T*K routes, and every
 // route the counts cover names a token below T and a rank below K.  Sets *bad otherwise.
 __global__ __launch_bounds__(256) void ragged_check_kernel(const mf_pair* __restrict__ sorted,
@@ -1301,6 +1309,12 @@ hipError_t launch_group(hipStream_t s, const uint32_t* idx, const float* w, uint
                         mf_pair* sorted, void* tiles, uint32_t tile_slots, uint32_t* n_tiles,
                         uint32_t* status, uint32_t* chunk_hist) {
   const uint32_t n_pairs = t * K;
+  if (n_pairs == 0) {  // no routes: the scan over no chunks writes empty experts and a clean status word
+    group_scan_kernel<<<dim3(1), dim3(MF_MAX_EXPERTS), 0, s>>>(chunk_hist, 0, E, counts, offsets, starts,
+                                                               static_cast<Tile*>(tiles), tile_slots, n_tiles,
+                                                               chunk_hist, status);
+    return hipGetLastError();
+  }
   // at most kGroupChunks chunks, each a whole number of kGroupBlock-pair steps
   const uint32_t steps = (n_pairs + kGroupBlock - 1) / kGroupBlock;
   const uint32_t chunk_pairs = (steps + kGroupChunks - 1) / kGroupChunks * kGroupBlock;
@@ -1689,8 +1703,7 @@ hipError_t launch_prefill_layer(hipStream_t s, const mf_moe& h, const mf_moe_lay
     uint32_t* hist = h.ws.group_tmp + 2048;
     uint32_t* bad = hist + static_cast<size_t>(kGroupChunks) * MF_MAX_EXPERTS;
     ws.status = h.ws.group_tmp + 3 * 512;  // the word mf_moe_group_status reads
-    MF_TRY(hipMemcpyAsync(hist, ragged->counts, sizeof(uint32_t) * c.num_experts, hipMemcpyDeviceToDevice, s));
-    MF_TRY(hipMemsetAsync(bad, 0, sizeof(uint32_t), s));
+    ragged_begin_kernel<<<dim3(1), dim3(MF_MAX_EXPERTS), 0, s>>>(ragged->counts, c.num_experts, hist, bad);
     const uint32_t check_wgs = static_cast<uint32_t>(std::min<size_t>((pairs + 255) / 256, 2048));
     ragged_check_kernel<<<dim3(std::max(check_wgs, 1u)), dim3(256), 0, s>>>(ragged->sorted, ragged->counts, c.num_experts,
                                                                            t, c.top_k, bad);

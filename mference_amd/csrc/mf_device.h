@@ -379,7 +379,8 @@ template <> struct QmmCodes<2> {
 
 // tmp[token block] += x * codes over one group: 8 MFMAs; `after(s)` runs once both token blocks have
 // issued theirs on operand s (the caller may then overwrite bx[.][s])
-template <int BITS, typename After>
+// (NTA = 1: only the first token block holds routes, the second is left alone)
+template <int BITS, int NTA = 2, typename After>
 __device__ __forceinline__ void group_products(const QmmCodes<BITS>& c, const uint4 (&bx)[2][4], f32x16_t (&tmp)[2],
                                                After after) {
   if constexpr (BITS == 4) {
@@ -387,7 +388,7 @@ __device__ __forceinline__ void group_products(const QmmCodes<BITS>& c, const ui
     for (int s = 0; s < 4; ++s) {
       const uint4 av = expand_q4(c.w[s]);
       tmp[0] = mfma_bf16(bx[0][s], av, tmp[0]);
-      tmp[1] = mfma_bf16(bx[1][s], av, tmp[1]);
+      if constexpr (NTA > 1) tmp[1] = mfma_bf16(bx[1][s], av, tmp[1]);
       after(s);
     }
   } else {
@@ -396,10 +397,10 @@ __device__ __forceinline__ void group_products(const QmmCodes<BITS>& c, const ui
       uint4 a, b;
       expand_q2(c.w[j], a, b);
       tmp[0] = mfma_bf16(bx[0][2 * j], a, tmp[0]);
-      tmp[1] = mfma_bf16(bx[1][2 * j], a, tmp[1]);
+      if constexpr (NTA > 1) tmp[1] = mfma_bf16(bx[1][2 * j], a, tmp[1]);
       after(2 * j);
       tmp[0] = mfma_bf16(bx[0][2 * j + 1], b, tmp[0]);
-      tmp[1] = mfma_bf16(bx[1][2 * j + 1], b, tmp[1]);
+      if constexpr (NTA > 1) tmp[1] = mfma_bf16(bx[1][2 * j + 1], b, tmp[1]);
       after(2 * j + 1);
     }
   }

@@ -20,6 +20,8 @@
 // (Metal/Prefill/prefill.metal:748-820), prefill_moe_reduce_token_major
 // (:631-652) and the staged-affine tensor-core QMM
 // mpp_prefill_affine_threadgroup_f16 (Metal/TensorCore/tensorops.metal:13-105).
+#include <type_traits>
+
 #include "mf_device.h"
 #include "mf_internal.h"
 #include "mf_router.h"
@@ -698,6 +700,11 @@ void qmm_kernel(const QmmLaunch launch) {
   // -offset * S is formed in place (exponent + 4 or + 2, sign flipped: exact; a zero scale becomes 2^-123 / 2^-125).
   // sumx enters as three bf16 terms, which hold all 24 bits: the -offset * S * sumx term cancels the
   // offset * sum(x) the matrix core accumulated with the codes, so it has to be exact.
+  // A tile of at most 32 routes fills only the first token block: the second block's matrix
+  // instructions and scale multiplies are left out (NTA = 1); its accumulators stay zero and its
+  // output slots are empty.
+  auto tile_body = [&](auto nta_c) {
+  constexpr int NTA = decltype(nta_c)::value;
   for (uint32_t g0 = 0; g0 < ng; g0 += 16) {
     const TabStep t = tab_cur;
     tab_cur = tab_fetch(g0 + 16 < ng ? g0 + 16 : g0);  // past the end: the same step again, unused
@@ -723,7 +730,7 @@ void qmm_kernel(const QmmLaunch launch) {
       if (!have) ab[p] = as[p] = make_uint4(0, 0, 0, 0);
     }
 #pragma unroll
-    for (int nt = 0; nt < 2; ++nt) {
+    for (int nt = 0; nt < NTA; ++nt) {
       uint32_t hi[8], mid[8], lo[8];
 #pragma unroll
       for (int e = 0; e < 8; ++e) {
@@ -778,21 +785,26 @@ void qmm_kernel(const QmmLaunch launch) {
 #pragma unroll
     for (int uu = 0; uu < 2; ++uu) {  // pair of K groups g0 + 2uu, g0 + 2uu + 1 in stage uu
       const uint32_t gu = g0 + 2 * uu;
-      if (gu >= ng) break;
+      if (!NG8 && gu >= ng) break;
       __syncthreads();  // stage uu is complete, stage uu ^ 1 is no longer read
-      // ---- the next pair into the other stage, fetch the pair after it into the freed registers
-      if (gu + 2 < ng) {
+      // ---- the next pair into the other stage, fetch the pair after it into the freed registers.
+      // With whole steps of 8 groups the body has no branch (past the end the last pair is fetched
+      // again and the write goes to the stage nobody reads any more): every pass issues the same
+      // loads in the same order, so a wait for the codes of this pass never covers the x rows
+      // requested a moment before it.
+      if (NG8 || gu + 2 < ng) {
         uint4* wbuf = s_x + (uu ^ 1) * 1024;
 #pragma unroll
         for (int gi = 0; gi < 2; ++gi) {
           *reinterpret_cast<u32x4_t*>(wbuf + gi * 512 + st_slot0) = xs[gi][0];
           *reinterpret_cast<u32x4_t*>(wbuf + gi * 512 + st_slot1) = xs[gi][1];
         }
-        if (gu + 4 < ng) {
+        if (NG8 || gu + 4 < ng) {
+          const uint32_t gx = NG8 ? min(gu + 4, ng - 2) : gu + 4;
 #pragma unroll
           for (int gi = 0; gi < 2; ++gi) {
-            xs[gi][0] = *reinterpret_cast<const u32x4_t*>(st_src + (gu + 4 + gi) * kGroup);
-            xs[gi][1] = *reinterpret_cast<const u32x4_t*>(st_src + (gu + 4 + gi) * kGroup + 8);
+            xs[gi][0] = *reinterpret_cast<const u32x4_t*>(st_src + (gx + gi) * kGroup);
+            xs[gi][1] = *reinterpret_cast<const u32x4_t*>(st_src + (gx + gi) * kGroup + 8);
           }
         }
       }
@@ -803,7 +815,7 @@ void qmm_kernel(const QmmLaunch launch) {
         const uint4* buf = s_x + uu * 1024 + gi * 512;
         uint4 bx[2][4];
 #pragma unroll
-        for (int nt = 0; nt < 2; ++nt)
+        for (int nt = 0; nt < NTA; ++nt)
 #pragma unroll
           for (int s = 0; s < 4; ++s) bx[nt][s] = buf[((nt * 4 + s) * 2 + h) * 32 + rd_col[s]];
 #pragma unroll
@@ -811,21 +823,25 @@ void qmm_kernel(const QmmLaunch launch) {
           const float sc = s_scale[((p * kQmmWaves + wv) * ng + g) * 32 + m];
           f32x16_t tmp[2];
 #pragma unroll
-          for (int nt = 0; nt < 2; ++nt)
+          for (int nt = 0; nt < NTA; ++nt)
 #pragma unroll
             for (int r = 0; r < 16; ++r) tmp[nt][r] = 0.0f;
-          group_products<BITS>(cur[p][2 * uu + gi], bx, tmp, [](int) {});
+          group_products<BITS, NTA>(cur[p][2 * uu + gi], bx, tmp, [](int) {});
           // the register that held this group's codes takes those of the group four ahead
           // (past the end the last group is read again: no branch inside the unrolled body)
           cur[p][2 * uu + gi].load(wrow[p] + min(g + 4, ng - 1) * kGB);
 #pragma unroll
-          for (int nt = 0; nt < 2; ++nt)
+          for (int nt = 0; nt < NTA; ++nt)
 #pragma unroll
             for (int r = 0; r < 16; ++r) acc[p][nt][r] = __builtin_fmaf(sc, tmp[nt][r], acc[p][nt][r]);
         }
       }
     }
   }
+  };  // tile_body
+  // (the one-projection form keeps to its budget of 168 registers, three waves per SIMD, with one body only)
+  if (NPROJ == 1 || count > 32) tile_body(std::integral_constant<int, 2>{});
+  else tile_body(std::integral_constant<int, 1>{});
 
   qmm_trace(a, work, 3);
   // ---- epilogue: the lane holds weight row row_base[p] + m for tokens 8j + 4h + i of each 32-token block
@@ -839,6 +855,7 @@ void qmm_kernel(const QmmLaunch launch) {
     const uint32_t dw = ((m & ~7u) >> 1) + (m & 3u);  // word of the row pair (r, r + 4)
 #pragma unroll
     for (int nt = 0; nt < 2; ++nt) {
+      if (nt == 1 && count <= 32) break;  // no route in the second block: its slots are empty
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
         uint32_t bits[4];
@@ -875,6 +892,7 @@ void qmm_kernel(const QmmLaunch launch) {
     const uint32_t lane = threadIdx.x & 63u;
 #pragma unroll
     for (int it = 0; it < 4; ++it) {
+      if (it == 2 && count <= 32) break;
       const uint32_t c = it * 64 + lane, tok = c >> 2, part = c & 3u;
       const uint32_t sl = s_slot[tok];
       const uint4 v = reinterpret_cast<const uint4*>(so)[c];
@@ -885,6 +903,7 @@ void qmm_kernel(const QmmLaunch launch) {
   } else {
 #pragma unroll
     for (int nt = 0; nt < 2; ++nt) {
+      if (nt == 1 && count <= 32) break;
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
         const uint4 sl = *reinterpret_cast<const uint4*>(s_slot + nt * 32 + 8 * j + 4 * h);
@@ -1051,9 +1070,13 @@ void qmm_kres_kernel(const KresLaunch launch) {
   // sum(x) of a group as three bf16 terms (all 24 bits), see qmm_kernel.  Both halves of the wave hold
   // the sums of groups 0..7 of the lane's two routes: K slots 8h..8h+7 of the bias product are those
   // groups again, multiplied by the biases for h = 0 and by -offset * scale for h = 1.
+  // A tile of at most 32 routes fills only the first route block (NTA = 1): the second block, whose routes
+  // would all repeat the last route, is left out of the products, the scale multiplies and the stores.
+  auto tile_body = [&](auto nta_c) {
+  constexpr int NTA = decltype(nta_c)::value;
   uint4 b_term[2][3];
 #pragma unroll
-  for (int nt = 0; nt < 2; ++nt) {
+  for (int nt = 0; nt < NTA; ++nt) {
     float sx[8];
 #pragma unroll
     for (int e = 0; e < 8; ++e) sx[e] = e < NG ? s_sum[(nt * 32 + m) * NG + e] : 0.0f;
@@ -1093,7 +1116,7 @@ void qmm_kres_kernel(const KresLaunch launch) {
 #pragma unroll
     for (int p = 0; p < 2; ++p)
 #pragma unroll
-      for (int nt = 0; nt < 2; ++nt) {
+      for (int nt = 0; nt < NTA; ++nt) {
 #pragma unroll
         for (int r = 0; r < 16; ++r) acc[p][nt][r] = 0.0f;
 #pragma unroll
@@ -1111,7 +1134,7 @@ void qmm_kres_kernel(const KresLaunch launch) {
     uint4 bx[2][4];
     if (w == 0) {
 #pragma unroll
-      for (int nt = 0; nt < 2; ++nt)
+      for (int nt = 0; nt < NTA; ++nt)
 #pragma unroll
         for (int s = 0; s < 4; ++s) bx[nt][s] = s_x[((nt * 4 + s) * 2 + h) * 32 + rd_col[s]];
     }
@@ -1124,13 +1147,13 @@ void qmm_kres_kernel(const KresLaunch launch) {
         const float sc = QmmCodes<BITS>::kScaleMul * ((g & 1) ? bf16_hi(sw[g >> 1]) : bf16_lo(sw[g >> 1]));
         f32x16_t tmp[2];
 #pragma unroll
-        for (int nt = 0; nt < 2; ++nt)
+        for (int nt = 0; nt < NTA; ++nt)
 #pragma unroll
           for (int r = 0; r < 16; ++r) tmp[nt][r] = 0.0f;
-        group_products<BITS>(cur[p][g % kRing], bx, tmp, [&](int s) {
+        group_products<BITS, NTA>(cur[p][g % kRing], bx, tmp, [&](int s) {
           if (p == 1) {  // both row blocks have read x slot s of this group
             bx[0][s] = nbuf[((0 * 4 + s) * 2 + h) * 32 + rd_col[s]];
-            bx[1][s] = nbuf[((1 * 4 + s) * 2 + h) * 32 + rd_col[s]];
+            if (NTA > 1) bx[1][s] = nbuf[((1 * 4 + s) * 2 + h) * 32 + rd_col[s]];
           }
         });
         // the register takes the codes kRing groups on: of this slice, or of the next one
@@ -1138,12 +1161,13 @@ void qmm_kres_kernel(const KresLaunch launch) {
         cur[p][g % kRing].load(ahead < NG ? wrow + p * 32 * kRowBytes + ahead * kGB
                                           : wnext + p * 32 * kRowBytes + (ahead - NG) * kGB);
 #pragma unroll
-        for (int nt = 0; nt < 2; ++nt)
+        for (int nt = 0; nt < NTA; ++nt)
 #pragma unroll
           for (int r = 0; r < 16; ++r) acc[p][nt][r] = __builtin_fmaf(sc, tmp[nt][r], acc[p][nt][r]);
         // the sums are wanted here, not after the last group: without this the compiler keeps every
         // group's products and adds them up at the end of the slice, out of scratch memory
-        asm volatile("" : "+v"(acc[p][0]), "+v"(acc[p][1]));
+        if constexpr (NTA > 1) asm volatile("" : "+v"(acc[p][0]), "+v"(acc[p][1]));
+        else asm volatile("" : "+v"(acc[p][0]));
         __builtin_amdgcn_sched_barrier(0);  // one unit at a time: hoisted loads would cost more registers than exist
       }
     }
@@ -1155,7 +1179,7 @@ void qmm_kres_kernel(const KresLaunch launch) {
       uint8_t* out = static_cast<uint8_t*>(a.out);
       const uint32_t pitch = a.rows * 4, col = row * 4;
 #pragma unroll
-      for (int nt = 0; nt < 2; ++nt) {
+      for (int nt = 0; nt < NTA; ++nt) {
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
           const uint4 sl = *reinterpret_cast<const uint4*>(s_slot + nt * 32 + 8 * j + 4 * h);
@@ -1172,7 +1196,7 @@ void qmm_kres_kernel(const KresLaunch launch) {
       uint8_t* out = static_cast<uint8_t*>(a.out);
       const uint32_t pitch = a.rows * 2, col = row * 2;
 #pragma unroll
-      for (int nt = 0; nt < 2; ++nt) {
+      for (int nt = 0; nt < NTA; ++nt) {
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
           const uint4 sl = *reinterpret_cast<const uint4*>(s_slot + nt * 32 + 8 * j + 4 * h);
@@ -1188,6 +1212,9 @@ void qmm_kres_kernel(const KresLaunch launch) {
     }
     wrow = wnext;
   }
+  };  // tile_body
+  if (count > 32) tile_body(std::integral_constant<int, 2>{});
+  else tile_body(std::integral_constant<int, 1>{});
   qmm_trace(a, work, 4);
 }
 
@@ -1763,7 +1790,11 @@ hipError_t launch_prefill_layer(hipStream_t s, const mf_moe& h, const mf_moe_lay
   q.w_off[1] = w.offsets.up_w; q.s_off[1] = w.offsets.up_s; q.b_off[1] = ternary ? w.offsets.up_s : w.offsets.up_b;
   q.x = ws.xp; q.sumx = ws.sum_x; q.x_stride = c.d; q.gather = 1; q.rows = c.f; q.kdim = c.d; q.epi = 0;
   q.out = ws.acts;
-  MF_TRY(launch_qmm(s, code_bits, q, 2, max_tiles, shared_rides ? &d : nullptr, dense_tiles));
+  // Short batches leave workgroup slots over: the shared expert's work items (whole 64-row tiles, the
+  // longest of the launch) go first there; in a long batch they go last and fill the holes of the last round.
+  const bool dense_first = shared_rides && pairs <= 4096;
+  if (dense_first) MF_TRY(launch_qmm(s, code_bits, d, 2, dense_tiles, &q, max_tiles));
+  else MF_TRY(launch_qmm(s, code_bits, q, 2, max_tiles, shared_rides ? &d : nullptr, dense_tiles));
   if (c.shared_f && !shared_rides) MF_TRY(launch_qmm(s, 4, d, 2, dense_tiles, nullptr, 0));
   // phase 2: routed down -> fp32 partials [token*K+rank, D]; shared down -> hs [token, D]
   q.w_off[0] = w.offsets.down_w; q.s_off[0] = w.offsets.down_s; q.b_off[0] = ternary ? w.offsets.down_s : w.offsets.down_b;
@@ -1789,7 +1820,10 @@ hipError_t launch_prefill_layer(hipStream_t s, const mf_moe& h, const mf_moe_lay
                               d_ring ? static_cast<size_t>(t) * c.shared_f : 0));
   }
   if (shared_rides) {
-    if (kres_q && kres_d && d.kdim == q.kdim) MF_TRY(launch_qmm_kres(s, 4, q, max_tiles, &d, dense_tiles));
+    if (kres_q && kres_d && d.kdim == q.kdim) {
+      if (dense_first) MF_TRY(launch_qmm_kres(s, 4, d, dense_tiles, &q, max_tiles));
+      else MF_TRY(launch_qmm_kres(s, 4, q, max_tiles, &d, dense_tiles));
+    } else if (dense_first) MF_TRY(launch_qmm(s, 4, d, q.pair_rows ? 2 : 1, dense_tiles, &q, max_tiles));
     else MF_TRY(launch_qmm(s, 4, q, q.pair_rows ? 2 : 1, max_tiles, &d, dense_tiles));
   } else {
     if (kres_q) MF_TRY(launch_qmm_kres(s, code_bits, q, max_tiles, nullptr, 0));

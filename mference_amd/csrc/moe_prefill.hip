@@ -45,13 +45,49 @@ struct Tile {
 // expert rows in registers (lane l holds the chunks l, l+64, ... of each row)
 // and streams token rows past them.
 template <int CPL, int R>
+__device__ __forceinline__ void router_rows(const uint16_t* __restrict__ W, const uint16_t* __restrict__ x,
+                                            uint32_t E, uint32_t D, uint32_t T, uint32_t x_stride,
+                                            float* __restrict__ logits, uint32_t tokens_per_block, uint32_t ld,
+                                            uint32_t lane, uint32_t wv);
+
+// What a short batch hangs on the router launch so that it needs no launch of its own: the x
+// preparation (matmul order, group sums, scalar shared gate) in extra workgroup columns.  (The top-k of
+// a token block by the last workgroup to finish that block's logits was tried and lost: the
+// device-wide fence every workgroup needs for it costs more than the launch it saves.)
+struct RouterTail {
+  uint16_t* xp;          // null: none of this
+  uint32_t router_cols;  // workgroup columns that compute logits; the columns behind them prepare x
+  const uint16_t* w_sg;  // null: no scalar gate
+  float* sums;
+  uint16_t* gate;
+};
+
+__device__ __forceinline__ void prep_x_row(const uint16_t* __restrict__ x, uint16_t* __restrict__ xp,
+                                           float* __restrict__ sums, const uint16_t* __restrict__ w_sg,
+                                           uint16_t* __restrict__ gate, uint32_t row, uint32_t d, uint32_t lane);
+
+template <int CPL, int R>
 __global__ __launch_bounds__(256) void prefill_router_kernel(const uint16_t* __restrict__ W,
                                                              const uint16_t* __restrict__ x,
                                                              uint32_t E, uint32_t D, uint32_t T,
                                                              uint32_t x_stride,
                                                              float* __restrict__ logits,
-                                                             uint32_t tokens_per_block, uint32_t ld) {
+                                                             uint32_t tokens_per_block, uint32_t ld,
+                                                             const RouterTail tail) {
   const uint32_t lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
+  if (tail.xp && blockIdx.x >= tail.router_cols) {  // an x-preparation workgroup: one row per wave
+    const uint32_t row = ((blockIdx.x - tail.router_cols) * gridDim.y + blockIdx.y) * 4 + wv;
+    if (row < T) prep_x_row(x + static_cast<size_t>(row) * x_stride, tail.xp, tail.sums, tail.w_sg, tail.gate, row, D, lane);
+    return;
+  }
+  router_rows<CPL, R>(W, x, E, D, T, x_stride, logits, tokens_per_block, ld, lane, wv);
+}
+
+template <int CPL, int R>
+__device__ __forceinline__ void router_rows(const uint16_t* __restrict__ W, const uint16_t* __restrict__ x,
+                                            uint32_t E, uint32_t D, uint32_t T, uint32_t x_stride,
+                                            float* __restrict__ logits, uint32_t tokens_per_block, uint32_t ld,
+                                            uint32_t lane, uint32_t wv) {
   const uint32_t row0 = (blockIdx.x * 4 + wv) * R;
   if (row0 >= E) return;
   const uint32_t chunks = D / 8;
@@ -253,6 +289,54 @@ __global__ __launch_bounds__(256) void group_count_kernel(const uint32_t* __rest
   for (uint32_t e = threadIdx.x; e < E; e += blockDim.x) chunk_hist[blockIdx.x * E + e] = s_hist[e];
 }
 
+// From every expert's count (thread e holds c; threads past MF_MAX_EXPERTS only keep the barriers
+// company): counts, offsets (0xFFFFFFFF for an empty expert), the start of every expert's run and
+// the tile list of the matmul (runs of kTileTokens routes).
+__device__ __forceinline__ void group_layout(uint32_t c, uint32_t E, uint32_t* __restrict__ counts,
+                                             uint32_t* __restrict__ offsets, uint32_t* __restrict__ starts,
+                                             Tile* __restrict__ tiles, uint32_t tile_slots,
+                                             uint32_t* __restrict__ n_tiles, uint32_t* s_cnt, uint32_t* s_tile) {
+  const uint32_t e = threadIdx.x;
+  const bool act = e < MF_MAX_EXPERTS;
+  if (e < E) counts[e] = c;
+  if (act) {
+    s_cnt[e] = c;
+    s_tile[e] = (c + kTileTokens - 1) / kTileTokens;
+  }
+  __syncthreads();
+  for (uint32_t o = 1; o < MF_MAX_EXPERTS; o <<= 1) {  // inclusive scans
+    const uint32_t a = act && e >= o ? s_cnt[e - o] : 0, b = act && e >= o ? s_tile[e - o] : 0;
+    __syncthreads();
+    if (act) {
+      s_cnt[e] += a;
+      s_tile[e] += b;
+    }
+    __syncthreads();
+  }
+  // The tile list has tile_slots entries (a multiple of 8).  The matmul sends the workgroups of
+  // slot range k * tile_slots/8 .. to XCD k, so every eighth of the list gets an eighth of the
+  // live tiles, in expert order; the rest of each eighth stays empty (count 0).
+  if (tiles) {
+    for (uint32_t i = e; i < tile_slots; i += blockDim.x) tiles[i] = Tile{0, 0, 0, 0};
+    __syncthreads();
+  }
+  if (e < E) {
+    const uint32_t start = s_cnt[e] - c;
+    starts[e] = start;
+    offsets[e] = c ? start : 0xFFFFFFFFu;
+    if (tiles) {
+      const uint32_t total = s_tile[MF_MAX_EXPERTS - 1], per_live = (total + 7) / 8, per_slot = tile_slots / 8;
+      const uint32_t nt = (c + kTileTokens - 1) / kTileTokens, t0 = s_tile[e] - nt;
+      for (uint32_t j = 0; j < nt; ++j) {
+        const uint32_t id = t0 + j;
+        tiles[(id / per_live) * per_slot + id % per_live] =
+            Tile{e, start + j * kTileTokens, min(kTileTokens, c - j * kTileTokens), 0};
+      }
+    }
+  }
+  if (n_tiles && e == MF_MAX_EXPERTS - 1) *n_tiles = s_tile[e];
+}
+
 // counts, offsets (0xFFFFFFFF for an empty expert), the start of every expert's
 // run, chunk_hist turned into each chunk's first position inside its expert's
 // run, and the tile list of the matmul (runs of kTileTokens routes).
@@ -291,39 +375,7 @@ __global__ __launch_bounds__(512) void group_scan_kernel(uint32_t* __restrict__ 
       c += v;
     }
   }
-  if (e < E) counts[e] = c;
-  s_cnt[e] = c;
-  s_tile[e] = (c + kTileTokens - 1) / kTileTokens;
-  __syncthreads();
-  for (uint32_t o = 1; o < MF_MAX_EXPERTS; o <<= 1) {  // inclusive scans
-    const uint32_t a = e >= o ? s_cnt[e - o] : 0, b = e >= o ? s_tile[e - o] : 0;
-    __syncthreads();
-    s_cnt[e] += a;
-    s_tile[e] += b;
-    __syncthreads();
-  }
-  // The tile list has tile_slots entries (a multiple of 8).  The matmul sends the workgroups of
-  // slot range k * tile_slots/8 .. to XCD k, so every eighth of the list gets an eighth of the
-  // live tiles, in expert order; the rest of each eighth stays empty (count 0).
-  if (tiles) {
-    for (uint32_t i = e; i < tile_slots; i += MF_MAX_EXPERTS) tiles[i] = Tile{0, 0, 0, 0};
-    __syncthreads();
-  }
-  if (e < E) {
-    const uint32_t start = s_cnt[e] - c;
-    starts[e] = start;
-    offsets[e] = c ? start : 0xFFFFFFFFu;
-    if (tiles) {
-      const uint32_t total = s_tile[MF_MAX_EXPERTS - 1], per_live = (total + 7) / 8, per_slot = tile_slots / 8;
-      const uint32_t nt = (c + kTileTokens - 1) / kTileTokens, t0 = s_tile[e] - nt;
-      for (uint32_t j = 0; j < nt; ++j) {
-        const uint32_t id = t0 + j;
-        tiles[(id / per_live) * per_slot + id % per_live] =
-            Tile{e, start + j * kTileTokens, min(kTileTokens, c - j * kTileTokens), 0};
-      }
-    }
-  }
-  if (n_tiles && e == MF_MAX_EXPERTS - 1) *n_tiles = s_tile[e];
+  group_layout(c, E, counts, offsets, starts, tiles, tile_slots, n_tiles, s_cnt, s_tile);
 }
 
 __global__ __launch_bounds__(256) void group_emit_kernel(const uint32_t* __restrict__ idx,
@@ -383,6 +435,79 @@ __global__ __launch_bounds__(256) void group_emit_kernel(const uint32_t* __restr
   }
 }
 
+// The three steps above in one workgroup, for a pair list short enough that one workgroup is not
+// the slower way: each of the 16 waves is a "chunk" (a contiguous run of the pair list), the per-chunk
+// counts live in LDS, and the result is the same stable order.
+constexpr uint32_t kGroupSmallPairs = 2048;
+
+__global__ __launch_bounds__(1024) void group_small_kernel(const uint32_t* __restrict__ idx,
+                                                           const float* __restrict__ w, uint32_t n_pairs,
+                                                           uint32_t K, uint32_t E, uint32_t* __restrict__ counts,
+                                                           uint32_t* __restrict__ offsets,
+                                                           uint32_t* __restrict__ starts,
+                                                           mf_pair* __restrict__ sorted, Tile* __restrict__ tiles,
+                                                           uint32_t tile_slots, uint32_t* __restrict__ n_tiles,
+                                                           uint32_t* __restrict__ status) {
+  __shared__ uint32_t s_hist[16][MF_MAX_EXPERTS];  // routes per expert of each wave, then its running base
+  __shared__ uint32_t s_cnt[MF_MAX_EXPERTS], s_tile[MF_MAX_EXPERTS];
+  const uint32_t lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
+  for (uint32_t i = threadIdx.x; i < 16 * MF_MAX_EXPERTS; i += blockDim.x) (&s_hist[0][0])[i] = 0;
+  __syncthreads();
+  const uint32_t chunk = ((n_pairs + 15) / 16 + 63) / 64 * 64;
+  const uint32_t p0 = min(n_pairs, wv * chunk), p1 = min(n_pairs, p0 + chunk);
+  bool bad = false;
+  for (uint32_t p = p0 + lane; p < p1; p += 64) {
+    const uint32_t e = idx[p];
+    if (e < E) atomicAdd(&s_hist[wv][e], 1u);
+    else bad = true;
+  }
+  const int any_bad = __syncthreads_or(bad ? 1 : 0);
+  if (threadIdx.x == 0) *status = any_bad ? 2u : 0u;
+  uint32_t c = 0;
+  if (threadIdx.x < E) {
+#pragma unroll
+    for (int v = 0; v < 16; ++v) {
+      const uint32_t n = s_hist[v][threadIdx.x];
+      s_hist[v][threadIdx.x] = c;
+      c += n;
+    }
+  }
+  group_layout(c, E, counts, offsets, starts, tiles, tile_slots, n_tiles, s_cnt, s_tile);
+  __syncthreads();
+  // s_cnt holds the inclusive scan: an expert's run starts at s_cnt[e] - (its count); the waves' bases are
+  // relative to that start
+  for (uint32_t q0 = p0; q0 < p1; q0 += 64) {
+    const uint32_t p = q0 + lane;
+    const bool valid = p < p1;
+    const uint32_t e = valid ? idx[p] : 0xFFFFFFFFu;
+    bool open = valid && e < E;
+    const bool mine = open;
+    uint32_t pos = 0;
+    unsigned long long todo = __ballot(open);
+    while (todo) {  // rank of this route among the routes of its expert in this step, in pair order
+      const int leader = __ffsll(static_cast<long long>(todo)) - 1;
+      const uint32_t e0 = static_cast<uint32_t>(__builtin_amdgcn_readlane(static_cast<int>(e), leader));
+      const unsigned long long same = __ballot(open && e == e0);
+      const uint32_t base = s_hist[wv][e0];
+      if (open && e == e0) {
+        pos = base + __popcll(same & ((1ull << lane) - 1ull));
+        open = false;
+      }
+      if (lane == static_cast<uint32_t>(leader)) s_hist[wv][e0] = base + __popcll(same);
+      todo &= ~same;
+    }
+    if (mine) {
+      const uint32_t run = (e ? s_cnt[e - 1] : 0u);  // exclusive scan = start of the expert's run
+      mf_pair r;
+      r.token = p / K;
+      r.expert = e;
+      r.rank = p % K;
+      r.weight_bits = __float_as_uint(w[p]);
+      sorted[run + pos] = r;
+    }
+  }
+}
+
 // --------------------------------------------------------------- the matmul
 
 // Activation rows as the matmul wants them: inside every run of 8 K values the
@@ -421,12 +546,9 @@ __global__ __launch_bounds__(256) void prep_rows_kernel(const PrepArgs a) {
 // w_sg . x of every row (prefill_qwen_shared_scalar_gate, prefill.metal:42-80) in the router's lane
 // order (dot_bf16_row: lane l takes the chunks l, l+64, ... of a row, neighbour-first butterfly), so
 // the gate has the bits of the stand-alone router-row launch it replaces.  One wave per row.
-__global__ __launch_bounds__(256) void prep_x_gate_kernel(const uint16_t* __restrict__ x,
-                                                          uint16_t* __restrict__ xp, float* __restrict__ sums,
-                                                          const uint16_t* __restrict__ w_sg,
-                                                          uint16_t* __restrict__ gate, uint32_t t, uint32_t d) {
-  const uint32_t lane = threadIdx.x & 63, row = blockIdx.x * 4 + (threadIdx.x >> 6);
-  if (row >= t) return;
+__device__ __forceinline__ void prep_x_row(const uint16_t* __restrict__ xr, uint16_t* __restrict__ xp,
+                                           float* __restrict__ sums, const uint16_t* __restrict__ w_sg,
+                                           uint16_t* __restrict__ gate, uint32_t row, uint32_t d, uint32_t lane) {
   const uint32_t chunks = d / 8;  // a multiple of 8: the 8 lanes of a K group are live together
   const size_t base = static_cast<size_t>(row) * chunks;
   float acc = 0.0f;
@@ -435,8 +557,8 @@ __global__ __launch_bounds__(256) void prep_x_gate_kernel(const uint16_t* __rest
     const bool live = c < chunks;
     uint4 v = make_uint4(0, 0, 0, 0), wv = make_uint4(0, 0, 0, 0);
     if (live) {
-      v = *reinterpret_cast<const uint4*>(x + (base + c) * 8);
-      wv = *reinterpret_cast<const uint4*>(w_sg + static_cast<size_t>(c) * 8);
+      v = *reinterpret_cast<const uint4*>(xr + static_cast<size_t>(c) * 8);
+      if (w_sg) wv = *reinterpret_cast<const uint4*>(w_sg + static_cast<size_t>(c) * 8);
     }
     float sum = ((bf16_lo(v.x) + bf16_hi(v.x)) + (bf16_lo(v.y) + bf16_hi(v.y))) +
                 ((bf16_lo(v.z) + bf16_hi(v.z)) + (bf16_lo(v.w) + bf16_hi(v.w)));
@@ -457,7 +579,16 @@ __global__ __launch_bounds__(256) void prep_x_gate_kernel(const uint16_t* __rest
     }
   }
   acc = wave_sum(acc);
-  if (lane == 0) gate[row] = f_to_bf16(acc);
+  if (w_sg && lane == 0) gate[row] = f_to_bf16(acc);
+}
+
+__global__ __launch_bounds__(256) void prep_x_gate_kernel(const uint16_t* __restrict__ x,
+                                                          uint16_t* __restrict__ xp, float* __restrict__ sums,
+                                                          const uint16_t* __restrict__ w_sg,
+                                                          uint16_t* __restrict__ gate, uint32_t t, uint32_t d) {
+  const uint32_t lane = threadIdx.x & 63, row = blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (row >= t) return;
+  prep_x_row(x + static_cast<size_t>(row) * d, xp, sums, w_sg, gate, row, d, lane);
 }
 
 struct QmmArgs {
@@ -1294,8 +1425,15 @@ __global__ __launch_bounds__(256) void ragged_check_kernel(const mf_pair* __rest
 
 // ------------------------------------------------------------------ launchers
 
+// `tail` (optional): the x preparation a short batch wants done in the same launch; on return
+// tail->xp is null when the launch did not take it on (the caller then launches it).
 hipError_t launch_prefill_router(hipStream_t s, const uint16_t* W, const uint16_t* x, uint32_t E,
-                                 uint32_t D, uint32_t T, uint32_t x_stride, float* logits) {
+                                 uint32_t D, uint32_t T, uint32_t x_stride, float* logits, RouterTail* tail) {
+  RouterTail fused{};
+  if (tail) {
+    fused = *tail;
+    tail->xp = nullptr;
+  }
   // Up to 256 tokens the matrix-core kernel has too few workgroups (T/32 x E/32) to cover the chip: the
   // register-tiled kernel is faster there (Qwen shape, layer time: 64 tokens 110 -> 100 us, 128 tokens
   // 112 -> 103 us, 256 tokens 118 -> 116 us, equal at 384; it holds rows of up to 4096 elements).  Both give
@@ -1319,16 +1457,31 @@ hipError_t launch_prefill_router(hipStream_t s, const uint16_t* W, const uint16_
   // about a thousand workgroups, >= 4 tokens per row load; the few rows left over by the matrix-core kernel
   // fill one workgroup column only, so they take the shortest token runs
   const uint32_t tpb = e32 ? 4u : std::max(4u, std::min(64u, T / 64));
+  const uint32_t token_blocks = (T + tpb - 1) / tpb;
+  // the whole call in this kernel, x rows as the preparation reads them: the launch takes the tail on
+  const bool take_tail = fused.xp && !e32 && cpl <= 8 && x_stride == D && D % 64 == 0 && aligned16(x) &&
+                         aligned16(fused.xp) && (!fused.w_sg || aligned16(fused.w_sg));
+  if (!take_tail) fused = RouterTail{};
+  const uint32_t prep_cols = take_tail ? ((T + 3) / 4 + token_blocks - 1) / token_blocks : 0u;
 #define MF_PR(CPL, R)                                                                              \
-  prefill_router_kernel<CPL, R><<<dim3((rest + 4 * R - 1) / (4 * R), (T + tpb - 1) / tpb), dim3(256), 0, s>>>( \
-      Wr, x, rest, D, T, x_stride, lr, tpb, E)
+  do {                                                                                             \
+    fused.router_cols = (rest + 4 * R - 1) / (4 * R);                                              \
+    prefill_router_kernel<CPL, R><<<dim3(fused.router_cols + prep_cols, token_blocks), dim3(256), 0, s>>>( \
+        Wr, x, rest, D, T, x_stride, lr, tpb, E, fused);                                           \
+  } while (0)
   if (cpl <= 1) MF_PR(1, 4);
   else if (cpl <= 2) MF_PR(2, 4);
   else if (cpl <= 4) MF_PR(4, 4);
   else if (cpl <= 8) MF_PR(8, 2);
   else return hipErrorInvalidValue;
 #undef MF_PR
+  if (take_tail) tail->xp = fused.xp;
   return hipGetLastError();
+}
+
+hipError_t launch_prefill_router(hipStream_t s, const uint16_t* W, const uint16_t* x, uint32_t E,
+                                 uint32_t D, uint32_t T, uint32_t x_stride, float* logits) {
+  return launch_prefill_router(s, W, x, E, D, T, x_stride, logits, nullptr);
 }
 
 hipError_t launch_group(hipStream_t s, const uint32_t* idx, const float* w, uint32_t t, uint32_t K,
@@ -1336,6 +1489,11 @@ hipError_t launch_group(hipStream_t s, const uint32_t* idx, const float* w, uint
                         mf_pair* sorted, void* tiles, uint32_t tile_slots, uint32_t* n_tiles,
                         uint32_t* status, uint32_t* chunk_hist) {
   const uint32_t n_pairs = t * K;
+  if (n_pairs && n_pairs <= kGroupSmallPairs) {
+    group_small_kernel<<<dim3(1), dim3(1024), 0, s>>>(idx, w, n_pairs, K, E, counts, offsets, starts, sorted,
+                                                      static_cast<Tile*>(tiles), tile_slots, n_tiles, status);
+    return hipGetLastError();
+  }
   if (n_pairs == 0) {  // no routes: the scan over no chunks writes empty experts and a clean status word
     group_scan_kernel<<<dim3(1), dim3(MF_MAX_EXPERTS), 0, s>>>(chunk_hist, 0, E, counts, offsets, starts,
                                                                static_cast<Tile*>(tiles), tile_slots, n_tiles,
@@ -1724,6 +1882,7 @@ hipError_t launch_prefill_layer(hipStream_t s, const mf_moe& h, const mf_moe_lay
 #define MF_TRY(call) do { e = (call); if (e != hipSuccess) return e; } while (0)
   const size_t pairs = static_cast<size_t>(t) * c.top_k;
   const uint32_t max_tiles = prefill_tile_slots(c, t);
+  bool x_prepared = false;
   if (ragged) {
     // the caller's grouping: its per-expert counts are a one-chunk histogram for the scan that lays
     // out the tile list (the runs start at 0 in expert order, as mf_moe_group writes them)
@@ -1742,7 +1901,13 @@ hipError_t launch_prefill_layer(hipStream_t s, const mf_moe& h, const mf_moe_lay
     ws.partials = ragged->partials;
   } else {
     if (w.router_w) {  // else the routing in out_idx / out_w is the caller's
-      MF_TRY(launch_prefill_router(s, w.router_w, x, c.num_experts, c.d, t, c.d, ws.logits));
+      RouterTail tail{};
+      tail.xp = ws.xp;
+      tail.w_sg = c.shared_f ? w.w_sg : nullptr;
+      tail.sums = ws.sum_x;
+      tail.gate = ws.gate;
+      MF_TRY(launch_prefill_router(s, w.router_w, x, c.num_experts, c.d, t, c.d, ws.logits, &tail));
+      x_prepared = tail.xp != nullptr;
       MF_TRY(launch_topk(s, ws.logits, c.num_experts, c.top_k, t, c.router_mode, ws.idx, ws.w));
     }
     MF_TRY(launch_group(s, ws.idx, ws.w, t, c.top_k, c.num_experts, ws.counts, ws.offsets, ws.starts,
@@ -1750,7 +1915,9 @@ hipError_t launch_prefill_layer(hipStream_t s, const mf_moe& h, const mf_moe_lay
   }
 
   const bool want_gate = c.shared_f && w.w_sg;
-  if (want_gate) {  // one pass over x: matmul order, group sums and the shared gate's logits
+  if (x_prepared) {
+    // the router launch has prepared x (and the gate's logits) on the side
+  } else if (want_gate) {  // one pass over x: matmul order, group sums and the shared gate's logits
     prep_x_gate_kernel<<<dim3((t + 3) / 4), dim3(256), 0, s>>>(x, ws.xp, ws.sum_x, w.w_sg, ws.gate, t, c.d);
     MF_TRY(hipGetLastError());
   } else {

@@ -191,6 +191,28 @@ def test_prefill_other_widths_take_the_decode_launch(gpu, oracle):
         assert np.array_equal(y, ops.bf16_bits(yd))
 
 
+@pytest.mark.parametrize("d,e,t", [(5120, 32, 40), (5120, 32, 300), (4224, 32, 40), (4224, 48, 290),
+                                   (5120, 48, 290)])
+def test_prefill_rows_wider_than_4096(gpu, oracle, d, e, t):
+    """Hidden sizes past 4096: a multiple of 512 takes the matrix-core router for whole blocks of 32
+    router rows (rows left over -- e = 48 -- and widths that are no multiple of 512 -- 4224 -- go one wave
+    per (token, row)); the matmuls take any multiple of 128 up to 8192.  Routing bit-exact, layer within
+    the tolerance."""
+    f, k, fs = 128, 4, 128
+    root = ROOT_SEED + 0xA300 + d + e + t
+    layer = oracle.synth_layer(root, d, f, e, k, bits=4, fs=fs)
+    x = oracle.synth_x(root, t, d)
+    moe = make_moe(gpu, layer)
+    assert moe.prefill_workspace_bytes(t) > 0
+    wts = to_device_layer(layer)
+    y, idx, w = _run_prefill(moe, wts, x, t, d, k)
+    rows = np.arange(t) if t <= 64 else np.random.default_rng(t).choice(t, size=48, replace=False)
+    ref_y, ref_idx, ref_w = oracle.moe_layer(layer, x[rows])
+    assert np.array_equal(idx[rows], ref_idx)
+    assert np.array_equal(w[rows].view(np.uint32), ref_w.view(np.uint32))
+    assert_layer_close(oracle.bf16_to_float(y[rows]), oracle.bf16_to_float(ref_y), f"prefill d={d} e={e} t={t}")
+
+
 @pytest.mark.parametrize("workload,t", [("dsv4-2bit", 300), ("maple-ternary", 300)])
 def test_prefill_other_formats_full_size(gpu, oracle, workload, t):
     """the large 2-bit layer (D 4096, F 2048, E 256, K 6, 4-bit shared 2048) and the ternary layer

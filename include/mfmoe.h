@@ -227,6 +227,14 @@ typedef struct {
                             * (maple_moe_phase2, maple_moe.metal:243-264); swiglu_limit is
                             * ignored.  0: the MoE / MoEDeepseekV4 rule (moe.metal:27-34, 528,
                             * 1262-1270) */
+  uint32_t gate_group_size; /* quantization group of the routed GATE projection: 0 or 64 = like every other
+                             * table; 32 = the DeepSeek-V4 conversion's gate_proj (two scale / bias entries
+                             * per 64 weights: moe_int2_gate_up_rows_simd_dev_vec's gate_group_size,
+                             * Metal/MoE/moe.metal:962-1060; MoEDeepseekV4.encodeRoutedPhase1(gateGroupSize:),
+                             * MoEDeepseekV4.swift:199-263; Model.routedGateGroupSize,
+                             * Runtime/Inference/ModelExpertIO.swift:118-135).  2-bit experts only.  Such a
+                             * layer runs on the chain of launches (the fused launch and the matrix-core
+                             * prefill take group 64); up and down stay at 64. */
 } mf_moe_config;
 
 /* MoE.init (Kernels/MoE/MoE.swift:65-151): one operator instance per shape; owns the

@@ -262,11 +262,12 @@ class MoE {
   MoE(const MetalContext& context, uint32_t specializedD, uint32_t specializedF,
       uint32_t specializedNumExperts, uint32_t specializedTopK = 8, mf_bits bits = MF_BITS_4,
       mf_router_mode routerMode = MF_ROUTER_TOPK_SOFTMAX, float swigluLimit = 0.0f,
-      uint32_t sharedF = 0, mf_bits sharedBits = MF_BITS_4, bool mapleRounding = false)
+      uint32_t sharedF = 0, mf_bits sharedBits = MF_BITS_4, bool mapleRounding = false,
+      uint32_t gateGroupSize = 0)  // 32: MoEDeepseekV4.encodeRoutedPhase1(gateGroupSize:), MoEDeepseekV4.swift:199
       : ctx_(context.raw()) {
     cfg_ = mf_moe_config{specializedD, specializedF, specializedNumExperts, specializedTopK, bits,
                          routerMode,   swigluLimit,  sharedF,               sharedBits,
-                         mapleRounding ? 1u : 0u};
+                         mapleRounding ? 1u : 0u, gateGroupSize};
     check(mf_moe_create(ctx_, &cfg_, &h_), ctx_);
   }
   ~MoE() { mf_moe_destroy(h_); }

@@ -46,6 +46,7 @@ class MoEConfig(C.Structure):
         ("d", C.c_uint32), ("f", C.c_uint32), ("num_experts", C.c_uint32), ("top_k", C.c_uint32),
         ("bits", C.c_int), ("router_mode", C.c_int), ("swiglu_limit", C.c_float),
         ("shared_f", C.c_uint32), ("shared_bits", C.c_int), ("maple_rounding", C.c_uint32),
+        ("gate_group_size", C.c_uint32),
     ]
 
 

@@ -11,7 +11,7 @@
 
 namespace {
 
-constexpr int kAbiVersion = 1;
+constexpr int kAbiVersion = 2;  // 2: mf_moe_config.gate_group_size
 
 mf_status fail_hip(mf_ctx* ctx, hipError_t e, const char* what) {
   if (ctx) snprintf(ctx->hip_error, sizeof ctx->hip_error, "%s: %s", what, hipGetErrorString(e));
@@ -275,6 +275,9 @@ mf_status mf_moe_create(mf_ctx* ctx, const mf_moe_config* cfg, mf_moe** out) {
   if (cfg->router_mode == MF_ROUTER_FULL_SOFTMAX && cfg->num_experts % 32 != 0)
     return MF_ERR_INVALID_ARGUMENT;
   if (cfg->maple_rounding > 1) return MF_ERR_INVALID_ARGUMENT;
+  if (cfg->gate_group_size != 0 && cfg->gate_group_size != 64 &&
+      !(cfg->gate_group_size == 32 && cfg->bits == MF_BITS_2))
+    return MF_ERR_INVALID_ARGUMENT;
 
   auto* h = new (std::nothrow) mf_moe();
   if (!h) return MF_ERR_OUT_OF_MEMORY;

@@ -544,6 +544,40 @@ __device__ __forceinline__ void lane_dot(const uint4& codes, const uint16_t* x, 
   sum = xs.sum;
 }
 
+// A lane's 64 two-bit codes as two runs of 32 (a gate projection quantized at group 32 has a
+// scale / bias entry for each): sum(q x) and sum(x) of either run.
+template <bool ALIGNED>
+__device__ __forceinline__ void lane_dot_halves_q2(const uint4& codes, const uint16_t* x, float (&dot)[2],
+                                                   float (&sum)[2]) {
+  uint32_t raw[32];
+#pragma unroll
+  for (int q = 0; q < 8; ++q) {
+    const uint4 a = load_x8<ALIGNED>(x + 8 * q);
+    raw[4 * q] = a.x; raw[4 * q + 1] = a.y; raw[4 * q + 2] = a.z; raw[4 * q + 3] = a.w;
+  }
+  const uint32_t ws[4] = {codes.x, codes.y, codes.z, codes.w};
+#pragma unroll
+  for (int half = 0; half < 2; ++half) {
+    float s = 0.0f, d = 0.0f;
+#pragma unroll
+    for (int i = 0; i < 16; ++i) s = dot2_bf16(raw[16 * half + i], kOnes, s);
+#pragma unroll
+    for (int j = 2 * half; j < 2 * half + 2; ++j) {
+      const uint32_t w = ws[j];
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {
+        // code i of the word pairs with code i + 8: raw pairs (x_2i', x_2i'+1) regrouped as (x_i, x_i+8)
+        const uint32_t lo = raw[8 * j + (i >> 1)], hi = raw[8 * j + 4 + (i >> 1)];
+        const uint32_t xp = (i & 1) ? __builtin_amdgcn_perm(hi, lo, 0x07060302u) : __builtin_amdgcn_perm(hi, lo, 0x05040100u);
+        const uint32_t cw = i < 3 ? w << (5 - 2 * i) : w >> (2 * i - 5);
+        d = dot2_bf16(and_or(cw, 0x00600060u, kMagic4), xp, d);
+      }
+    }
+    sum[half] = s;
+    dot[half] = __builtin_fmaf(-4.0f, s, d);  // sum((4 + q) x) -> sum(q x)
+  }
+}
+
 // scale / bias of the group that holds element e0 of a row whose tables start
 // at srow / brow; ternary rows carry no bias table (bias = -scale).
 template <int BITS>

@@ -32,7 +32,9 @@ __device__ __forceinline__ BlobView view_blob(const uint8_t* blob, const mf_expe
 // gate and up rows share the x loads (moe_phase1_gate_up_act_u16load,
 // moe.metal:499-583; 2-bit twin :966-1116; ternary maple_moe_phase1,
 // maple_moe.metal:190-221; `maple` selects its bf16-stepped activation, :153-164).
-template <int BITS, bool ALIGNED>
+// G32 (2-bit experts only): the gate projection's tables hold an entry per 32 weights
+// (moe_int2_gate_up_rows_simd_dev_vec with gate_group_size 32, moe.metal:962-1060); up stays at 64.
+template <int BITS, bool ALIGNED, bool G32 = false>
 __global__ __launch_bounds__(256) void phase1_kernel(const uint8_t* __restrict__ base,
                                                      size_t stride, mf_expert_offsets off,
                                                      const uint32_t* __restrict__ idx,
@@ -76,14 +78,28 @@ __global__ __launch_bounds__(256) void phase1_kernel(const uint8_t* __restrict__
     const uint4 gc = load_codes16<ALIGNED>(bv.gw + boff);
     const uint4 uc = load_codes16<ALIGNED>(bv.uw + boff);
     float gs, gb, us, ub, gd, ud, sum, sum2;
-    load_scale_bias<BITS>(bv.gs + r * n_groups, bv.gb + r * n_groups, e0, gs, gb);
     load_scale_bias<BITS>(bv.us + r * n_groups, bv.ub + r * n_groups, e0, us, ub);
-    lane_dot<BITS, ALIGNED>(gc, xt + e0, gd, sum);
     lane_dot<BITS, ALIGNED>(uc, xt + e0, ud, sum2);
-    ga = __builtin_fmaf(gs, gd, ga);
-    ga = __builtin_fmaf(gb, sum, ga);
+    if constexpr (G32 && BITS == kBits2) {
+      // the lane's 64 weights are two gate groups: entries e0 / 32 and e0 / 32 + 1 of a row of D / 32
+      const uint16_t* gsr = bv.gs + r * (2 * n_groups) + e0 / 32;
+      const uint16_t* gbr = bv.gb + r * (2 * n_groups) + e0 / 32;
+      float hd[2], hs[2];
+      lane_dot_halves_q2<ALIGNED>(gc, xt + e0, hd, hs);
+#pragma unroll
+      for (int half = 0; half < 2; ++half) {
+        ga = __builtin_fmaf(bf16_to_f(gsr[half]), hd[half], ga);
+        ga = __builtin_fmaf(bf16_to_f(gbr[half]), hs[half], ga);
+      }
+      (void)gs; (void)gb; (void)gd; (void)sum;
+    } else {
+      load_scale_bias<BITS>(bv.gs + r * n_groups, bv.gb + r * n_groups, e0, gs, gb);
+      lane_dot<BITS, ALIGNED>(gc, xt + e0, gd, sum);
+      ga = __builtin_fmaf(gs, gd, ga);
+      ga = __builtin_fmaf(gb, sum, ga);
+    }
     ua = __builtin_fmaf(us, ud, ua);
-    ua = __builtin_fmaf(ub, sum, ua);
+    ua = __builtin_fmaf(ub, sum2, ua);
   }
   const float g = group_sum(ga, static_cast<int>(lpr));
   const float u = group_sum(ua, static_cast<int>(lpr));
@@ -172,7 +188,20 @@ hipError_t launch_phase1(hipStream_t s, const mf_moe_config& cfg, const void* ba
   }
   switch (cfg.bits) {
     case MF_BITS_4: if (al) MF_P1(kBits4, true) else MF_P1(kBits4, false) break;
-    case MF_BITS_2: if (al) MF_P1(kBits2, true) else MF_P1(kBits2, false) break;
+    case MF_BITS_2:
+      if (cfg.gate_group_size == 32) {
+        const uint32_t lpr_log2 = lanes_per_row_log2(cfg.d, Fmt<kBits2>::kElemsPer16B);
+        const uint32_t rpw = 64u >> lpr_log2;
+        const uint32_t waves = pairs * ((cfg.f + rpw - 1) / rpw);
+#define MF_P1G(AL)                                                                                  \
+  phase1_kernel<kBits2, AL, true><<<dim3((waves + 3) / 4), dim3(256), 0, s>>>(                      \
+      b, stride, off, idx, x, x_stride, acts, cfg.d, cfg.f, cfg.num_experts, pairs, cfg.top_k,      \
+      cfg.swiglu_limit, static_cast<int>(cfg.maple_rounding), lpr_log2, subset, all_pairs)
+        if (al) MF_P1G(true); else MF_P1G(false);
+#undef MF_P1G
+        break;
+      }
+      if (al) MF_P1(kBits2, true) else MF_P1(kBits2, false) break;
     case MF_BITS_TERNARY: if (al) MF_P1(kBitsTernary, true) else MF_P1(kBitsTernary, false) break;
     default: return hipErrorInvalidValue;
   }

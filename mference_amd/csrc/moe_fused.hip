@@ -750,6 +750,7 @@ bool fused_supported(const mf_moe& h, const mf_moe_layer_weights& w, const void*
                      const void* hidden, uint32_t t) {
   const mf_moe_config& c = h.cfg;
   if (c.num_experts % 4 != 0) return false;  // tagged logits are read two entries per lane
+  if (c.gate_group_size == 32) return false;  // a gate projection at group 32 runs on the chain of launches
   const bool combo = (c.bits == MF_BITS_4 && (!c.shared_f || c.shared_bits == MF_BITS_4)) ||
                      (c.bits == MF_BITS_2 && (!c.shared_f || c.shared_bits == MF_BITS_4 ||
                                               c.shared_bits == MF_BITS_2)) ||

@@ -1831,6 +1831,7 @@ size_t prefill_workspace_bytes(const mf_moe_config& c, uint32_t t) {
 bool prefill_supported(const mf_moe_config& c) {
   if (c.bits != MF_BITS_4 && c.bits != MF_BITS_2 && c.bits != MF_BITS_TERNARY) return false;
   if (c.shared_f && c.shared_bits != MF_BITS_4) return false;
+  if (c.gate_group_size == 32) return false;  // the matmul's tables hold one entry per 64 weights
   if (c.d % kQmmRows || c.f % kQmmRows || (c.shared_f % kQmmRows)) return false;
   if (c.d > 8192 || c.f > 8192 || c.shared_f > 8192) return false;
   return true;

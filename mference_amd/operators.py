@@ -344,10 +344,12 @@ class MoE:
     def __init__(self, context: MetalContext, d: int, f: int, num_experts: int, top_k: int,
                  bits: int = BITS_4, router_mode: int = ROUTER_TOPK_SOFTMAX,
                  swiglu_limit: float = 0.0, shared_f: int = 0, shared_bits: int = BITS_4,
-                 maple_rounding: bool = False):
+                 maple_rounding: bool = False, gate_group_size: int = 0):
+        """gate_group_size 32: MoEDeepseekV4.encodeRoutedPhase1(gateGroupSize:) -- the routed gate
+        projection's tables hold an entry per 32 weights (2-bit experts only)."""
         self.context = context
         self.cfg = _capi.MoEConfig(d, f, num_experts, top_k, bits, router_mode, swiglu_limit,
-                                   shared_f, shared_bits, 1 if maple_rounding else 0)
+                                   shared_f, shared_bits, 1 if maple_rounding else 0, gate_group_size)
         self._h = C.c_void_p()
         check(_capi.lib().mf_moe_create(context.handle, C.byref(self.cfg), C.byref(self._h)),
               context.handle)

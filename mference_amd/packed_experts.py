@@ -9,10 +9,10 @@ checks, same error cases), `Model.routedExpertOffsets` / `routedExpertPhysicalOf
 (ModelExpertIO.swift:118-135), and loads a layer file straight into the resident HBM expert
 pool the operators address as `expert_base + expert * stride`.
 
-What it does not do: the group-32 gate projection of the DeepSeek conversion is detected
-(`routed_gate_group_size`) and refused (`require_group64_gate`): the kernels take group 64 only; Maple's per-row alpha tables
-are expected already expanded to per-group scale / bias entries, which is how the reference's
-repacker stores them.
+The group-32 gate projection of the DeepSeek conversion is detected (`routed_gate_group_size`) and,
+for 2-bit codes, accepted (`require_supported_gate_group` returns the group to hand to
+`MoE(gate_group_size=...)`); other groupings are refused.  Maple's per-row alpha tables: see
+`expand_row_alpha`.
 """
 from __future__ import annotations
 
@@ -188,16 +188,29 @@ def routed_gate_group_size(layout: PackedExpertsLayout, layer: int, moe_intermed
     return hidden // groups
 
 
-def require_group64_gate(layout: PackedExpertsLayout, layer: int, moe_intermediate: int, hidden: int) -> None:
-    """Raises when the layer's gate projection is quantized in groups other than 64 (the
-    group-32 gate of the DeepSeek conversion, ModelExpertIO.swift:122-135): the operators read
-    one scale / bias entry per 64 columns and would compute wrong activations from such a
-    blob without noticing."""
+def gate_code_bits(layout: PackedExpertsLayout, layer: int, moe_intermediate: int, hidden: int) -> int:
+    """Bits per weight of the gate projection's packed codes, from the byte size of its slice
+    (0 when the slice or the shape is unknown)."""
+    gate = layout.expert(layer, 0).sub_tensors.get("gate")
+    if gate is None or moe_intermediate <= 0 or hidden <= 0:
+        return 0
+    return gate.size * 8 // (moe_intermediate * hidden)
+
+
+def require_supported_gate_group(layout: PackedExpertsLayout, layer: int, moe_intermediate: int, hidden: int) -> int:
+    """The layer's gate quantization group, for `MoE(gate_group_size=...)`: 64, or 32 with 2-bit codes
+    (the DeepSeek conversion's gate_proj, ModelExpertIO.swift:122-135, which the operators run on their
+    chain of launches).  Any other combination raises: the operators would compute wrong activations
+    from such a blob without noticing."""
     g = routed_gate_group_size(layout, layer, moe_intermediate, hidden)
-    if g != GROUP_SIZE:
-        raise ModelError.index_corrupt(
-            f"layer {layer}: gate projection uses quantization group {g}; "
-            f"the resident operators take group {GROUP_SIZE} only")
+    if g == GROUP_SIZE:
+        return g
+    bits = gate_code_bits(layout, layer, moe_intermediate, hidden)
+    if g == 32 and bits == 2:
+        return g
+    raise ModelError.index_corrupt(
+        f"layer {layer}: gate projection uses quantization group {g} with {bits}-bit codes; "
+        f"the resident operators take group {GROUP_SIZE}, or group 32 with 2-bit codes")
 
 
 def load_layer_experts(directory: str, layout: PackedExpertsLayout, layer: int, device="cuda",
@@ -207,8 +220,8 @@ def load_layer_experts(directory: str, layout: PackedExpertsLayout, layer: int, 
     expert e at e * stride; the file may hold the blobs in any physical order).  Returns
     (tensor, stride).  The read goes through a pinned staging buffer in chunks, so a 453 MB
     layer never needs a second full copy in host memory.  With `moe_intermediate` and `hidden`
-    given, a layer whose gate projection is not quantized in groups of 64 is refused
-    (`require_group64_gate`) before anything is read."""
+    given, a layer whose gate projection's quantization group the operators do not take is refused
+    (`require_supported_gate_group`) before anything is read."""
     import numpy as np
     import torch
 
@@ -216,7 +229,7 @@ def load_layer_experts(directory: str, layout: PackedExpertsLayout, layer: int, 
     if not entry.experts:
         raise ModelError.index_corrupt(f"layer {layer} has no routed experts")
     if moe_intermediate is not None and hidden is not None:
-        require_group64_gate(layout, layer, moe_intermediate, hidden)
+        require_supported_gate_group(layout, layer, moe_intermediate, hidden)
     path = os.path.join(directory, "packed_experts", entry.file)
     if not os.path.isfile(path):
         raise ModelError.missing_file(entry.file)

@@ -270,18 +270,23 @@ int mfo_pack_codes(const uint8_t* codes, size_t rows, size_t n, int bits, uint8_
 
 /* Quantization.swift:104-119: Float(q) * scale + bias, two roundings.
  * Ternary: bias = -scale (RepackPlanner.swift:629,640; MapleMoETests.swift:327-332) */
-static void dequant_row(const uint8_t* prow, const uint16_t* s, const uint16_t* b, size_t n,
-                        int bits, float* out) {
-  const size_t ngroups = n / GROUP;
+static void dequant_row_group(const uint8_t* prow, const uint16_t* s, const uint16_t* b, size_t n,
+                              int bits, size_t group, float* out) {
+  const size_t ngroups = n / group;
   for (size_t g = 0; g < ngroups; ++g) {
     float scale = mfo_bf16_to_float(s[g]);
     float bias = bits == MFO_BITS_TERNARY ? -scale : mfo_bf16_to_float(b[g]);
-    for (size_t k = 0; k < GROUP; ++k) {
-      float q = (float)get_code(prow, g * GROUP + k, bits);
+    for (size_t k = 0; k < group; ++k) {
+      float q = (float)get_code(prow, g * group + k, bits);
       float prod = q * scale;
-      out[g * GROUP + k] = prod + bias;
+      out[g * group + k] = prod + bias;
     }
   }
+}
+
+static void dequant_row(const uint8_t* prow, const uint16_t* s, const uint16_t* b, size_t n,
+                        int bits, float* out) {
+  dequant_row_group(prow, s, b, n, bits, GROUP, out);
 }
 
 int mfo_dequantize(const uint8_t* packed, const uint16_t* scales, const uint16_t* biases,
@@ -596,15 +601,23 @@ void mfo_topk_softmax_scaled(const float* logits, const uint16_t* per_expert_sca
  * DequantInt4GEMVReferenceTests.swift:17-30 in place of vDSP_dotpr. */
 int mfo_gemv(const uint8_t* packed, const uint16_t* scales, const uint16_t* biases,
              int bits, size_t m, size_t n, const float* x, float* y) {
-  if (n % GROUP != 0 || !codes_per_byte(bits)) return MFO_ERR_ARG;
-  const size_t ngroups = n / GROUP, row_bytes = mfo_packed_row_bytes(bits, n);
+  return mfo_gemv_group(packed, scales, biases, bits, m, n, GROUP, x, y);
+}
+
+/* The same with a scale / bias entry per `group` weights (32 or 64): the gate projection of the
+ * DeepSeek-V4 conversion, whose kernel derives the table entry of an element as elem / gate_group_size
+ * (moe_int2_gate_up_rows_simd_dev_vec, moe.metal:962-1060); the packed codes do not depend on the group. */
+int mfo_gemv_group(const uint8_t* packed, const uint16_t* scales, const uint16_t* biases,
+                   int bits, size_t m, size_t n, size_t group, const float* x, float* y) {
+  if ((group != 32 && group != GROUP) || n % GROUP != 0 || !codes_per_byte(bits)) return MFO_ERR_ARG;
+  const size_t ngroups = n / group, row_bytes = mfo_packed_row_bytes(bits, n);
 #pragma omp parallel
   {
     float* wrow = (float*)malloc(n * sizeof(float));
 #pragma omp for schedule(static)
     for (size_t r = 0; r < m; ++r) {
-      dequant_row(packed + r * row_bytes, scales + r * ngroups,
-                  biases ? biases + r * ngroups : NULL, n, bits, wrow);
+      dequant_row_group(packed + r * row_bytes, scales + r * ngroups,
+                        biases ? biases + r * ngroups : NULL, n, bits, group, wrow);
       float sum = 0.0f;
       for (size_t i = 0; i < n; ++i) {
         float prod = wrow[i] * x[i];
@@ -653,14 +666,20 @@ static const uint16_t* u16_at(const uint8_t* base, uint32_t off) {
 
 int mfo_expert_phase1(const uint8_t* blob, const mfo_expert_offsets* off, int bits,
                       size_t d, size_t f, float limit, int maple, const uint16_t* x, uint16_t* acts) {
+  return mfo_expert_phase1_gate(blob, off, bits, d, f, GROUP, limit, maple, x, acts);
+}
+
+int mfo_expert_phase1_gate(const uint8_t* blob, const mfo_expert_offsets* off, int bits,
+                           size_t d, size_t f, size_t gate_group, float limit, int maple,
+                           const uint16_t* x, uint16_t* acts) {
   if ((off->gate_s | off->gate_b | off->up_s | off->up_b) & 1u) return MFO_ERR_ARG;
   float* xf = (float*)malloc(d * sizeof(float));
   float* g = (float*)malloc(f * sizeof(float));
   float* u = (float*)malloc(f * sizeof(float));
   mfo_bf16_decode(x, d, xf);
   const int tern = bits == MFO_BITS_TERNARY;
-  int rc = mfo_gemv(blob + off->gate_w, u16_at(blob, off->gate_s),
-                    tern ? NULL : u16_at(blob, off->gate_b), bits, f, d, xf, g);
+  int rc = mfo_gemv_group(blob + off->gate_w, u16_at(blob, off->gate_s),
+                          tern ? NULL : u16_at(blob, off->gate_b), bits, f, d, gate_group, xf, g);
   if (!rc)
     rc = mfo_gemv(blob + off->up_w, u16_at(blob, off->up_s),
                   tern ? NULL : u16_at(blob, off->up_b), bits, f, d, xf, u);
@@ -789,7 +808,8 @@ int mfo_moe_layer(const mfo_layer* L, const uint16_t* x, uint16_t* y, uint32_t* 
   for (size_t s = 0; s < k && !rc; ++s) {
     if (idx[s] >= e) continue; /* sentinel route: contributes nothing */
     const uint8_t* blob = L->experts + (size_t)idx[s] * L->expert_stride;
-    rc = mfo_expert_phase1(blob, &L->off, L->bits, d, f, L->swiglu_limit, L->maple_rounding, x, acts);
+    rc = mfo_expert_phase1_gate(blob, &L->off, L->bits, d, f, L->gate_group ? (size_t)L->gate_group : GROUP,
+                                L->swiglu_limit, L->maple_rounding, x, acts);
     if (!rc) rc = mfo_expert_down(blob, &L->off, L->bits, d, f, acts, v);
     if (!rc)
       for (size_t i = 0; i < d; ++i) {

@@ -121,6 +121,11 @@ int mfo_gemv_multix(const uint8_t* packed, const uint16_t* scales, const uint16_
 float mfo_silu(float x);
 /* routed phase 1: acts[f] = bf16(silu(clamp(gate.x)) * clamp(up.x)), fp32 gate/up
  * (moe.metal:499-529, clamp :27-34).  limit <= 0 disables the clamp. */
+int mfo_gemv_group(const uint8_t* packed, const uint16_t* scales, const uint16_t* biases,
+                   int bits, size_t m, size_t n, size_t group, const float* x, float* y);
+int mfo_expert_phase1_gate(const uint8_t* blob, const mfo_expert_offsets* off, int bits,
+                           size_t d, size_t f, size_t gate_group, float limit, int maple,
+                           const uint16_t* x, uint16_t* acts);
 int mfo_expert_phase1(const uint8_t* blob, const mfo_expert_offsets* off, int bits,
                       size_t d, size_t f, float swiglu_limit, int maple, const uint16_t* x,
                       uint16_t* acts);
@@ -161,6 +166,7 @@ typedef struct {
   const uint8_t* sdw; const uint16_t* sds; const uint16_t* sdb; /* shared down */
   const uint16_t* w_sg;      /* [d] bf16 scalar shared gate, may be NULL    */
   int maple_rounding;        /* MapleMoE's activation and bf16 down outputs */
+  int gate_group;            /* group of the routed gate tables: 0 / 64, or 32 */
 } mfo_layer;
 
 /* one token through router -> routed experts -> shared expert -> combine.

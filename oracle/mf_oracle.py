@@ -52,7 +52,7 @@ class _Layer(C.Structure):
         ("sgw", C.c_void_p), ("sgs", C.c_void_p), ("sgb", C.c_void_p),
         ("suw", C.c_void_p), ("sus", C.c_void_p), ("sub", C.c_void_p),
         ("sdw", C.c_void_p), ("sds", C.c_void_p), ("sdb", C.c_void_p),
-        ("w_sg", C.c_void_p), ("maple_rounding", C.c_int),
+        ("w_sg", C.c_void_p), ("maple_rounding", C.c_int), ("gate_group", C.c_int),
     ]
 
 
@@ -334,12 +334,13 @@ def gemv_multix(q: QTensor, x_bits) -> np.ndarray:
 
 
 def expert_phase1(blob, off: ExpertOffsets, bits: int, d: int, f: int, x_bits,
-                  swiglu_limit: float = 0.0, maple: bool = False) -> np.ndarray:
+                  swiglu_limit: float = 0.0, maple: bool = False, gate_group: int = GROUP) -> np.ndarray:
     blob = _c(blob, np.uint8)
     x_bits = _c(x_bits, np.uint16)
     acts = np.empty(f, np.uint16)
-    rc = lib().mfo_expert_phase1(_p(blob), C.byref(off), bits, C.c_size_t(d), C.c_size_t(f),
-                                 C.c_float(swiglu_limit), C.c_int(1 if maple else 0), _p(x_bits), _p(acts))
+    rc = lib().mfo_expert_phase1_gate(_p(blob), C.byref(off), bits, C.c_size_t(d), C.c_size_t(f),
+                                      C.c_size_t(gate_group), C.c_float(swiglu_limit),
+                                      C.c_int(1 if maple else 0), _p(x_bits), _p(acts))
     if rc:
         raise ValueError("mfo_expert_phase1")
     return acts
@@ -414,6 +415,7 @@ class Layer:
     router_mode: int = 0
     swiglu_limit: float = 0.0
     maple_rounding: bool = False    # MapleMoE's activation and bf16 down outputs
+    gate_group: int = GROUP         # group of the routed gate tables (32: the DeepSeek-V4 conversion)
 
     def _struct(self) -> _Layer:
         L = _Layer()
@@ -421,6 +423,7 @@ class Layer:
         L.bits, L.shared_bits = self.bits, self.shared_bits
         L.router_mode, L.swiglu_limit = self.router_mode, self.swiglu_limit
         L.maple_rounding = 1 if self.maple_rounding else 0
+        L.gate_group = self.gate_group
         L.router_w = self.router_w.ctypes.data
         L.experts = self.experts.ctypes.data
         L.expert_stride = self.experts.strides[0]
@@ -510,10 +513,11 @@ def reduce_token_major(partials, w) -> np.ndarray:
 
 # ---------------------------------------------------------------- layer builder
 
-def blob_layout(d: int, f: int, bits: int, align: int = 256):
+def blob_layout(d: int, f: int, bits: int, align: int = 256, gate_group: int = GROUP):
     """Sub-tensor byte offsets inside one expert blob, in the reference's order
     gate{W,s,b}, up{W,s,b}, down{W,s,b} (RepackPlanner.swift:544-712), and the
-    blob stride rounded up to `align`.  Ternary stores no biases."""
+    blob stride rounded up to `align`.  Ternary stores no biases.  `gate_group` 32: the gate
+    tables hold an entry per 32 weights (ModelExpertIO.swift:118-135)."""
     gu_w = f * packed_row_bytes(bits, d)
     gu_s = f * (d // GROUP) * 2
     dn_w = d * packed_row_bytes(bits, f)
@@ -521,7 +525,7 @@ def blob_layout(d: int, f: int, bits: int, align: int = 256):
     has_b = bits != BITS_TERNARY
     off = ExpertOffsets()
     pos = 0
-    for name, wsz, ssz in (("gate", gu_w, gu_s), ("up", gu_w, gu_s), ("down", dn_w, dn_s)):
+    for name, wsz, ssz in (("gate", gu_w, f * (d // gate_group) * 2), ("up", gu_w, gu_s), ("down", dn_w, dn_s)):
         setattr(off, f"{name}_w", pos)
         pos += wsz
         setattr(off, f"{name}_s", pos)
@@ -543,9 +547,24 @@ def pack_expert_blob(gate: QTensor, up: QTensor, down: QTensor, off: ExpertOffse
             out[bo:bo + q.biases.size * 2] = q.biases.reshape(-1).view(np.uint8)
 
 
+def quantize_group32_q2(w) -> QTensor:
+    """2-bit affine quantization with a scale / bias entry per 32 weights, out of the group-64
+    quantizer: every run of 32 is laid out twice in a row of twice the length, so each group of 64
+    there has the run's own minimum and maximum; its table entry is the run's, its first 32 codes
+    are the run's codes."""
+    w = _c(w, np.float32)
+    rows, n = w.shape
+    runs = w.reshape(rows, n // 32, 32)
+    q = quantize(np.concatenate([runs, runs], axis=2).reshape(rows, 2 * n), BITS_2)
+    codes = ((q.packed[:, :, None] >> (2 * np.arange(4, dtype=np.uint8))) & 3).reshape(rows, n // 32, 64)
+    packed = pack_codes(np.ascontiguousarray(codes[:, :, :32]).reshape(rows, n), BITS_2)
+    return QTensor(packed, q.scales, q.biases, BITS_2, rows, n)
+
+
 def synth_layer(root: int, d: int, f: int, e: int, k: int, bits: int = BITS_4, fs: int = 0,
                 shared_bits: int = BITS_4, sigma: float = 0.02, router_mode: int = 0,
-                swiglu_limit: float = 0.0, with_w_sg: bool = True, maple_rounding: bool = False) -> Layer:
+                swiglu_limit: float = 0.0, with_w_sg: bool = True, maple_rounding: bool = False,
+                gate_group: int = GROUP) -> Layer:
     """Seeded synthetic layer: one SeedTree stream per tensor (labels "router",
     "shared.gate|up|down", "w_sg", "expert<i>.gate|up|down"), N(0, sigma)
     weights by Box-Muller, quantized per group of 64."""
@@ -553,7 +572,7 @@ def synth_layer(root: int, d: int, f: int, e: int, k: int, bits: int = BITS_4, f
         return Rng.key(root, label).normal(0.0, sigma, rows * cols).reshape(rows, cols)
 
     router_w = bf16_bits(nrm("router", e, d))
-    off, _, stride = blob_layout(d, f, bits)
+    off, _, stride = blob_layout(d, f, bits, gate_group=gate_group)
     experts = np.zeros((e, stride), np.uint8)
     for i in range(e):
         if bits == BITS_TERNARY:
@@ -568,7 +587,8 @@ def synth_layer(root: int, d: int, f: int, e: int, k: int, bits: int = BITS_4, f
                                   BITS_TERNARY, rows, cols))
             pack_expert_blob(qs[0], qs[1], qs[2], off, experts[i])
         else:
-            g = quantize(nrm(f"expert{i}.gate", f, d), bits)
+            gate_w = nrm(f"expert{i}.gate", f, d)
+            g = quantize_group32_q2(gate_w) if gate_group == 32 else quantize(gate_w, bits)
             u = quantize(nrm(f"expert{i}.up", f, d), bits)
             dn = quantize(nrm(f"expert{i}.down", d, f), bits)
             pack_expert_blob(g, u, dn, off, experts[i])
@@ -582,7 +602,8 @@ def synth_layer(root: int, d: int, f: int, e: int, k: int, bits: int = BITS_4, f
             w_sg = bf16_bits(nrm("w_sg", 1, d).reshape(d))
     return Layer(d=d, f=f, e=e, k=k, bits=bits, router_w=router_w, experts=experts, off=off,
                  fs=fs, shared_bits=shared_bits, shared=shared, w_sg=w_sg,
-                 router_mode=router_mode, swiglu_limit=swiglu_limit, maple_rounding=maple_rounding)
+                 router_mode=router_mode, swiglu_limit=swiglu_limit, maple_rounding=maple_rounding,
+                 gate_group=gate_group)
 
 
 def synth_x(root: int, t: int, d: int, label: str = "x") -> np.ndarray:

@@ -35,7 +35,8 @@ def make_moe(ctx, layer) -> ops.MoE:
     return ops.MoE(ctx, layer.d, layer.f, layer.e, layer.k, bits=layer.bits,
                    router_mode=layer.router_mode, swiglu_limit=layer.swiglu_limit,
                    shared_f=layer.fs, shared_bits=layer.shared_bits,
-                   maple_rounding=getattr(layer, "maple_rounding", False))
+                   maple_rounding=getattr(layer, "maple_rounding", False),
+                   gate_group_size=getattr(layer, "gate_group", 64))
 
 
 def errors(actual: np.ndarray, ref: np.ndarray):
@@ -67,17 +68,19 @@ def write_packed_experts(directory, layer, physical_order=None, page=16384):
     pack_bits = 2 if bits == 1 else bits
     gu_w, gu_s = f * d * pack_bits // 8, f * (d // 64) * 2
     dn_w, dn_s = d * f * pack_bits // 8, d * (f // 64) * 2
+    gg = getattr(layer, "gate_group", 64)
+    g_s = f * (d // gg) * 2
     off = layer.off
     tensors = {
         "gate": dict(offset=off.gate_w, size=gu_w, dtype="U32", shape=[f, d * pack_bits // 32], bits=pack_bits),
-        "gate_scales": dict(offset=off.gate_s, size=gu_s, dtype="BF16", shape=[f, d // 64]),
+        "gate_scales": dict(offset=off.gate_s, size=g_s, dtype="BF16", shape=[f, d // gg]),
         "up": dict(offset=off.up_w, size=gu_w, dtype="U32", shape=[f, d * pack_bits // 32], bits=pack_bits),
         "up_scales": dict(offset=off.up_s, size=gu_s, dtype="BF16", shape=[f, d // 64]),
         "down": dict(offset=off.down_w, size=dn_w, dtype="U32", shape=[d, f * pack_bits // 32], bits=pack_bits),
         "down_scales": dict(offset=off.down_s, size=dn_s, dtype="BF16", shape=[d, f // 64]),
     }
     if bits != 1:
-        tensors["gate_biases"] = dict(offset=off.gate_b, size=gu_s, dtype="BF16", shape=[f, d // 64])
+        tensors["gate_biases"] = dict(offset=off.gate_b, size=g_s, dtype="BF16", shape=[f, d // gg])
         tensors["up_biases"] = dict(offset=off.up_b, size=gu_s, dtype="BF16", shape=[f, d // 64])
         tensors["down_biases"] = dict(offset=off.down_b, size=dn_s, dtype="BF16", shape=[d, f // 64])
     experts = [dict(expert=ex, physicalRank=rank_of[ex], offset=rank_of[ex] * stride, size=stride,

@@ -124,7 +124,7 @@ def _c_layout(tmp_path):
         "mf_qtensor": ["weights", "scales", "biases"],
         "mf_pair": ["token", "expert", "rank", "weight_bits"],
         "mf_moe_config": ["d", "f", "num_experts", "top_k", "bits", "router_mode", "swiglu_limit",
-                          "shared_f", "shared_bits", "maple_rounding"],
+                          "shared_f", "shared_bits", "maple_rounding", "gate_group_size"],
         "mf_moe_layer_weights": ["router_w", "expert_base", "expert_stride", "offsets",
                                  "shared_gate", "shared_up", "shared_down", "w_sg"],
     }

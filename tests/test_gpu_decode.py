@@ -3,6 +3,7 @@ import numpy as np
 import pytest
 import torch
 
+from mference_amd import _capi
 from mference_amd import operators as ops
 from helpers import ROOT_SEED, assert_layer_close, errors, make_moe, to_device_layer, to_device_q
 
@@ -336,6 +337,55 @@ def test_two_phase_matches_oracle_and_fused(gpu, oracle):
         ma, rl = errors(oracle.bf16_to_float(ops.bf16_bits(acts[0, s])), oracle.bf16_to_float(ref_act))
         assert rl < 1e-3
     assert_layer_close(oracle.bf16_to_float(ops.bf16_bits(y)), oracle.bf16_to_float(ref_y), "two-phase")
+
+
+@pytest.mark.parametrize("d,f,e,k,fs,t", [(256, 128, 16, 6, 128, 3), (1024, 256, 32, 6, 0, 8), (4096, 128, 8, 2, 0, 1)])
+def test_gate_projection_at_group_32(gpu, oracle, d, f, e, k, fs, t):
+    """DeepSeek-V4's 2-bit experts with the gate tables per 32 weights
+    (moe_int2_gate_up_rows_simd_dev_vec's gate_group_size, moe.metal:962-1060): phase 1 against the
+    oracle row by row, the layer call (which runs the chain of launches for such a layer) against the
+    per-token oracle, and the prefill call, which hands the rows to the decode launch.  A handle made
+    for group 64 reads the same blob differently -- the tables are really used per 32."""
+    root = ROOT_SEED + 0x2E0 + d
+    layer = oracle.synth_layer(root, d, f, e, k, bits=2, fs=fs, gate_group=32, swiglu_limit=7.0)
+    x = oracle.synth_x(root, t, d)
+    ref_y, ref_idx, ref_w = oracle.moe_layer(layer, x)
+    moe = make_moe(gpu, layer)
+    assert moe.cfg.gate_group_size == 32
+    wts = to_device_layer(layer)
+    xd = ops.bf16_tensor(x)
+    idx = torch.from_numpy(ref_idx.astype(np.int32)).cuda()
+    acts = torch.zeros((t, k, f), dtype=torch.bfloat16, device="cuda")
+    moe.encode_routed_phase1(wts.experts, wts.offsets, idx, xd, acts, t=t)
+    _sync()
+    worst = 0.0
+    for tok in range(t):
+        for s in range(k):
+            ref_act = oracle.expert_phase1(layer.experts[ref_idx[tok, s]], layer.off, 2, d, f, x[tok],
+                                           swiglu_limit=7.0, gate_group=32)
+            _, rl = errors(oracle.bf16_to_float(ops.bf16_bits(acts[tok, s])), oracle.bf16_to_float(ref_act))
+            worst = max(worst, rl)
+    assert worst < 2e-3, worst
+    y = torch.zeros((t, d), dtype=torch.bfloat16, device="cuda")
+    out_idx = torch.zeros((t, k), dtype=torch.int32, device="cuda")
+    moe.encode_decode_layer(wts, xd, y, t=t, out_indices=out_idx)
+    moe.status()
+    assert np.array_equal(out_idx.cpu().numpy().astype(np.uint32), ref_idx)
+    assert_layer_close(oracle.bf16_to_float(ops.bf16_bits(y)), oracle.bf16_to_float(ref_y), "group-32 gate layer")
+    assert moe.prefill_workspace_bytes(t) == 0
+    y2 = torch.zeros_like(y)
+    moe.encode_prefill_layer(wts, xd, y2, t)
+    _sync()
+    assert np.array_equal(ops.bf16_bits(y2), ops.bf16_bits(y))
+    # the same bytes through a group-64 handle: other activations
+    other = ops.MoE(gpu, d, f, e, k, bits=2, swiglu_limit=7.0)
+    acts64 = torch.zeros_like(acts)
+    other.encode_routed_phase1(wts.experts, wts.offsets, idx, xd, acts64, t=t)
+    _sync()
+    assert not np.array_equal(ops.bf16_bits(acts64), ops.bf16_bits(acts))
+    # group 32 goes with 2-bit codes only
+    with pytest.raises(_capi.MfError):
+        ops.MoE(gpu, d, f, e, k, bits=4, gate_group_size=32)
 
 
 @pytest.mark.parametrize("bits,t", [(4, 1), (2, 3), (1, 2)])

@@ -6,6 +6,7 @@ repository root).  None of these checks re-types the oracle's formula: they are
 published constants, literal integer KATs, invariants, or an independent fp64
 numpy composition.
 """
+import ctypes as C
 import math
 
 import numpy as np
@@ -643,3 +644,42 @@ def test_reduce_token_major_closed_form():
     got = O.reduce_token_major(part, w)
     ref = (part.astype(np.float64) * w.astype(np.float64)[..., None]).sum(axis=1)
     assert np.abs(got - ref).max() < 2e-6
+
+
+def test_gate_projection_at_group_32_against_float64(oracle):
+    """The group-32 form of the GEMV (the DeepSeek conversion's gate projection: a table entry per 32
+    weights, entry = element / 32, moe.metal:996-1041) against float64 arithmetic on codes and tables
+    taken apart by hand; group 64 through the same entry point is the ordinary GEMV bit for bit; and the
+    helper that quantizes at group 32 gives, per run of 32, the levels nearest to the weights."""
+    rng = np.random.default_rng(32)
+    rows, n = 24, 256
+    w = (rng.standard_normal((rows, n)) * 0.05).astype(np.float32)
+    q = oracle.quantize_group32_q2(w)
+    assert q.scales.shape == (rows, n // 32) and q.packed.shape == (rows, n // 4)
+    codes = ((q.packed[:, :, None] >> (2 * np.arange(4, dtype=np.uint8))) & 3).reshape(rows, n).astype(np.float64)
+    s = np.repeat(oracle.bf16_to_float(q.scales).astype(np.float64), 32, axis=1)
+    b = np.repeat(oracle.bf16_to_float(q.biases).astype(np.float64), 32, axis=1)
+    deq = codes * s + b
+    # nearest level of the run's own four levels, up to the rounding of the tables to bf16
+    levels = (np.arange(4)[None, None, :] * s[:, :, None] + b[:, :, None])
+    best = np.abs(levels - w[:, :, None].astype(np.float64)).min(axis=2)
+    assert np.all(np.abs(deq - w) <= best + 1e-3 * np.abs(s))
+    x = (rng.standard_normal(n)).astype(np.float32)
+    y = np.empty(rows, np.float32)
+    lib = oracle.lib()
+    rc = lib.mfo_gemv_group(oracle._p(q.packed), oracle._p(q.scales), oracle._p(q.biases), 2,
+                            C.c_size_t(rows), C.c_size_t(n), C.c_size_t(32), oracle._p(x), oracle._p(y))
+    assert rc == 0
+    want = deq @ x.astype(np.float64)
+    assert np.allclose(y, want, rtol=0, atol=2e-5 * np.abs(deq).sum(axis=1).max())
+    # a wrong table index (entry = element / 64, or the second half reading the first entry) moves the result
+    wrong = (codes * np.repeat(oracle.bf16_to_float(q.scales)[:, ::2].astype(np.float64), 64, axis=1)
+             + np.repeat(oracle.bf16_to_float(q.biases)[:, ::2].astype(np.float64), 64, axis=1)) @ x.astype(np.float64)
+    assert np.abs(wrong - want).max() > 100 * np.abs(y - want).max()
+    q64 = oracle.quantize(w, 2)
+    y64 = np.empty(rows, np.float32)
+    rc = lib.mfo_gemv_group(oracle._p(q64.packed), oracle._p(q64.scales), oracle._p(q64.biases), 2,
+                            C.c_size_t(rows), C.c_size_t(n), C.c_size_t(64), oracle._p(x), oracle._p(y64))
+    assert rc == 0 and np.array_equal(y64.view(np.uint32), oracle.gemv(q64, x).view(np.uint32))
+    assert lib.mfo_gemv_group(oracle._p(q.packed), oracle._p(q.scales), oracle._p(q.biases), 2,
+                              C.c_size_t(rows), C.c_size_t(n), C.c_size_t(16), oracle._p(x), oracle._p(y)) != 0

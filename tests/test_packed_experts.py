@@ -131,13 +131,31 @@ def test_gate_group_size_from_the_scale_slice(tmp_path, oracle):
     layout = pe.PackedExpertsLayoutReader.load(str(tmp_path))
     assert pe.routed_gate_group_size(layout, 0, 128, 256) == 32
     assert pe.routed_gate_group_size(layout, 0, 0, 256) == 64
-    # such a layer is refused before its file is read: the operators take group 64 only
+    # a 4-bit gate at group 32 is refused before its file is read: group 32 goes with 2-bit codes only
+    assert pe.gate_code_bits(layout, 0, 128, 256) == 4
     with pytest.raises(pe.ModelError, match="group 32") as err:
         pe.load_layer_experts(str(tmp_path), layout, 0, device="cpu", moe_intermediate=128, hidden=256)
     assert err.value.kind == "indexCorrupt"
     with pytest.raises(pe.ModelError):
-        pe.require_group64_gate(layout, 0, 128, 256)
-    pe.require_group64_gate(layout, 0, 0, 256)   # unknown intermediate size: falls back to 64
+        pe.require_supported_gate_group(layout, 0, 128, 256)
+    assert pe.require_supported_gate_group(layout, 0, 0, 256) == 64   # unknown intermediate size: falls back to 64
+
+
+def test_group32_gate_of_2bit_experts_is_accepted(tmp_path, oracle):
+    """the DeepSeek conversion's layers: 2-bit codes, gate tables per 32 weights (ModelExpertIO.swift:118-135)"""
+    d, f, e, k = 256, 128, 4, 2
+    layer = oracle.synth_layer(ROOT_SEED + 0xB110, d, f, e, k, bits=2, gate_group=32)
+    write_packed_experts(str(tmp_path), layer)
+    layout = pe.PackedExpertsLayoutReader.load(str(tmp_path))
+    assert pe.routed_gate_group_size(layout, 0, f, d) == 32
+    assert pe.gate_code_bits(layout, 0, f, d) == 2
+    assert pe.require_supported_gate_group(layout, 0, f, d) == 32
+    off = pe.routed_expert_offsets(layout, 0)
+    for name, _ in layer.off._fields_:
+        assert getattr(off, name) == getattr(layer.off, name), name
+    pool, stride = pe.load_layer_experts(str(tmp_path), layout, 0, device="cpu", moe_intermediate=f, hidden=d)
+    blob = layer.experts.shape[1]
+    assert np.array_equal(pool.numpy().reshape(e, stride)[:, :blob], layer.experts)
 
 
 def test_layer_file_checks(tmp_path, oracle):

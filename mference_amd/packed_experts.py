@@ -261,3 +261,56 @@ def load_layer_experts(directory: str, layout: PackedExpertsLayout, layer: int, 
             pool[e0 * stride:(e0 + cnt) * stride].copy_(stage[:cnt * stride], non_blocking=False)
     del src
     return pool, stride
+
+
+# ---- Maple's routed tensors: per-row alpha instead of per-group tables
+
+def expand_row_alpha(row_alpha, input_width: int):
+    """A Maple routed tensor ships 2-bit codes {0, 1, 2} and ONE bf16 `row_alpha` per output row;
+    the expert blob the kernels read holds a scale and a bias entry per row and group of 64 inputs.
+    The reference's repacker makes them by repeating every alpha input_width / 64 times, the bias
+    copy with the sign bit flipped (RepackPlanner.swift:596-640, the `.repeatBF16(count:negated:)`
+    transform of SourceByteProvider.swift:369-393): weight = (q - 1) * alpha.
+    row_alpha: uint16 bf16 bit patterns, shape [rows] (or [experts, rows]).  Returns
+    (scales, biases), uint16 arrays of shape [..., rows, input_width // 64]."""
+    import numpy as np
+    a = np.asarray(row_alpha)
+    if a.dtype != np.uint16:
+        raise ModelError.index_corrupt(f"row_alpha must be bf16 bit patterns (uint16), got {a.dtype}")
+    if input_width <= 0 or input_width % GROUP_SIZE:
+        raise ModelError.index_corrupt(f"row_alpha: input width {input_width} is no positive multiple of {GROUP_SIZE}")
+    reps = input_width // GROUP_SIZE
+    scales = np.repeat(a[..., None], reps, axis=-1)
+    return scales, scales ^ np.uint16(0x8000)
+
+
+def maple_expert_blob(gate, up, down, align: int = 16384):
+    """One routed expert's blob from Maple source tensors, in the repacker's order
+    gate {codes, scales, biases}, up {...}, down {...} (RepackPlanner.swift:544-651).
+    Each of gate / up / down is (packed 2-bit codes uint8 [rows, input / 4], row_alpha uint16 [rows]).
+    Returns (blob uint8 [stride], MoEExpertOffsets, stride); the ternary operators read the codes and
+    the scale tables (their bias is -scale by construction; the bias tables are carried for
+    byte-compatibility with the reference's layout)."""
+    import numpy as np
+    from .operators import MoEExpertOffsets
+    off = MoEExpertOffsets()
+    chunks = []
+    pos = 0
+    for role, (codes, alpha) in (("gate", gate), ("up", up), ("down", down)):
+        codes = np.ascontiguousarray(codes, dtype=np.uint8)
+        rows, row_bytes = codes.shape
+        width = row_bytes * 4
+        alpha = np.asarray(alpha)
+        if alpha.shape != (rows,):
+            raise ModelError.index_corrupt(
+                f"{role}: row_alpha shape {alpha.shape} does not match the {rows} output rows")
+        scales, biases = expand_row_alpha(alpha, width)
+        for suffix, arr in (("w", codes), ("s", scales), ("b", biases)):
+            setattr(off, f"{role}_{suffix}", pos)
+            raw = np.ascontiguousarray(arr).reshape(-1).view(np.uint8)
+            chunks.append(raw)
+            pos += raw.size
+    stride = (pos + align - 1) // align * align
+    blob = np.zeros(stride, np.uint8)
+    blob[:pos] = np.concatenate(chunks)
+    return blob, off, stride

@@ -271,3 +271,60 @@ def test_resident_streamer_pool_runs_a_layer(tmp_path, gpu, oracle):
     moe.status()
     assert np.array_equal(idx.cpu().numpy().astype(np.uint32), ref_idx)
     assert_layer_close(oracle.bf16_to_float(ops.bf16_bits(y)), oracle.bf16_to_float(ref_y), "layer from the streamer's pool")
+
+
+def test_row_alpha_expansion(oracle):
+    """RepackPlanner.swift:596-640 / SourceByteProvider.swift:369-393: every alpha repeated once per
+    group of 64 inputs, the bias copy with the sign bit flipped"""
+    alpha = oracle.bf16_bits(np.array([0.5, 0.0, 0.0123, 3.0], np.float32))
+    scales, biases = pe.expand_row_alpha(alpha, 256)
+    assert scales.shape == biases.shape == (4, 4) and scales.dtype == np.uint16
+    assert np.array_equal(scales, np.tile(alpha[:, None], (1, 4)))
+    assert np.array_equal(oracle.bf16_to_float(biases), -oracle.bf16_to_float(scales))
+    assert biases[1, 0] == 0x8000  # -0.0: the sign bit is flipped, nothing is computed
+    s3, _ = pe.expand_row_alpha(np.stack([alpha, alpha]), 128)
+    assert s3.shape == (2, 4, 2)
+    with pytest.raises(pe.ModelError):
+        pe.expand_row_alpha(alpha, 96)
+    with pytest.raises(pe.ModelError):
+        pe.expand_row_alpha(alpha.astype(np.float32), 128)
+
+
+@pytest.mark.gpu
+def test_maple_layer_from_row_alpha(gpu, oracle):
+    """A Maple layer whose experts come as codes + row_alpha: the blobs built by `maple_expert_blob`
+    (scale and bias tables per group, the repacker's order) run to the result of the per-token oracle
+    on the same weights written as scale-only ternary tables."""
+    import torch
+    from mference_amd import operators as ops
+    from helpers import assert_layer_close
+    d, f, e, k, t = 256, 128, 32, 8, 3
+    rng = np.random.default_rng(ROOT_SEED + 0xB300)
+    router_w = oracle.bf16_bits((rng.standard_normal((e, d)) * 0.02).astype(np.float32))
+    off_o, _, stride_o = oracle.blob_layout(d, f, 1)
+    experts_o = np.zeros((e, stride_o), np.uint8)
+    blobs = []
+    for ex in range(e):
+        parts, q = [], []
+        for rows, cols in ((f, d), (f, d), (d, f)):
+            codes = rng.integers(0, 3, size=(rows, cols)).astype(np.uint8)
+            alpha = oracle.bf16_bits((np.abs(rng.standard_normal(rows)) * 0.02 + 1e-3).astype(np.float32))
+            packed = oracle.pack_codes(codes, 1)
+            parts.append((packed, alpha))
+            q.append(oracle.QTensor(packed, np.repeat(alpha[:, None], cols // 64, axis=1), None, 1, rows, cols))
+        oracle.pack_expert_blob(q[0], q[1], q[2], off_o, experts_o[ex])
+        blob, off, stride = pe.maple_expert_blob(*parts)
+        blobs.append(blob)
+    assert stride % 16384 == 0 and off.gate_b > off.gate_s > off.gate_w == 0
+    layer = oracle.Layer(d=d, f=f, e=e, k=k, bits=1, router_w=router_w, experts=experts_o, off=off_o,
+                         router_mode=1, maple_rounding=True)
+    x = oracle.synth_x(ROOT_SEED + 0xB300, t, d)
+    ref_y, ref_idx, _ = oracle.moe_layer(layer, x)
+    moe = ops.MoE(gpu, d, f, e, k, bits=ops.BITS_TERNARY, router_mode=ops.ROUTER_FULL_SOFTMAX, maple_rounding=True)
+    wts = ops.MoELayerWeights(ops.bf16_tensor(router_w), torch.from_numpy(np.stack(blobs)).cuda(), off)
+    y = torch.zeros((t, d), dtype=torch.bfloat16, device="cuda")
+    idx = torch.zeros((t, k), dtype=torch.int32, device="cuda")
+    moe.encode_decode_layer(wts, ops.bf16_tensor(x), y, t=t, out_indices=idx)
+    moe.status()
+    assert np.array_equal(idx.cpu().numpy().astype(np.uint32), ref_idx)
+    assert_layer_close(oracle.bf16_to_float(ops.bf16_bits(y)), oracle.bf16_to_float(ref_y), "maple from row_alpha")

@@ -74,17 +74,82 @@ class PackedExpertsLayout:     # PackedExpertsLayout.swift:36-46
         return self.layers[layer].experts[expert]
 
 
+# ---- layout.json as a schema: a kind per field, one checker for every level of the document.
+# The reference walks the document with a guard per level (PackedExpertsLayout.swift:75-141); the
+# error a level reports when any of its fields has the wrong kind is that level's `what`.
+
 def _is_int(v) -> bool:
     return isinstance(v, int) and not isinstance(v, bool)
 
 
-def _uint(v) -> Optional[int]:
+def _as_uint(v) -> Optional[int]:
     """NSNumber.uint64Value of a JSON number: integers, and floats holding one"""
     if _is_int(v) and v >= 0:
         return v
     if isinstance(v, float) and v >= 0 and v == int(v):
         return int(v)
     return None
+
+
+_KINDS = {
+    "uint": _as_uint,
+    "int": lambda v: v if _is_int(v) else None,
+    "str": lambda v: v if isinstance(v, str) else None,
+    "objects": lambda v: v if isinstance(v, list) and all(isinstance(x, dict) for x in v) else None,
+    "object_map": lambda v: v if isinstance(v, dict) and all(isinstance(x, dict) for x in v.values()) else None,
+    "ints": lambda v: v if isinstance(v, list) and all(_is_int(x) for x in v) else None,
+}
+_TOP = (("expertStride", "uint"), ("numLayers", "int"), ("expertsPerLayer", "int"), ("layers", "objects"))
+_LAYER = (("layer", "int"), ("file", "str"), ("experts", "objects"))
+_EXPERT = (("offset", "uint"), ("size", "uint"), ("tensors", "object_map"))
+_TENSOR = (("offset", "uint"), ("size", "uint"), ("dtype", "str"), ("shape", "ints"))
+
+
+def _take(obj, schema, what: str) -> list:
+    """The schema's fields of `obj`, each converted by its kind; `what` names the level in the error."""
+    out = []
+    for key, kind in schema:
+        v = _KINDS[kind](obj.get(key)) if isinstance(obj, dict) else None
+        if v is None:
+            raise ModelError.index_corrupt(f"layout.json: {what}")
+        out.append(v)
+    return out
+
+
+def _optional_int(obj, key) -> Optional[int]:
+    v = obj.get(key)
+    return v if _is_int(v) else None
+
+
+def _sub_tensors(tensors: dict) -> Dict[str, SubTensorEntry]:
+    subs: Dict[str, SubTensorEntry] = {}
+    for role, t in tensors.items():
+        off, size, _, _ = _take(t, _TENSOR, f"malformed tensor {role}")
+        if "bits" in t and not _is_int(t["bits"]):
+            raise ModelError.index_corrupt(f"layout.json: malformed tensor bits {role}")
+        subs[role] = SubTensorEntry(off, size)
+    return subs
+
+
+def _layer_experts(entries: list, per_layer: int) -> List[ExpertEntry]:
+    """The experts of one layer by LOGICAL id; an entry without an id takes the next free position in
+    file order; every id of the layer has to be there."""
+    by_id: Dict[int, ExpertEntry] = {}
+    for obj in entries:
+        off, size, tensors = _take(obj, _EXPERT, "malformed expert entry")
+        subs = _sub_tensors(tensors)
+        expert_id = _optional_int(obj, "expert")
+        if expert_id is None:
+            expert_id = len(by_id)
+        if not 0 <= expert_id < per_layer:
+            raise ModelError.index_corrupt("layout.json: expert id out of range")
+        rank = _optional_int(obj, "physicalRank")
+        if rank is not None and not 0 <= rank < per_layer:
+            raise ModelError.index_corrupt("layout.json: physicalRank out of range")
+        by_id[expert_id] = ExpertEntry(expert_id, off, size, subs)
+    if len(by_id) != per_layer:
+        raise ModelError.index_corrupt("layout.json: missing expert entries")
+    return [by_id[i] for i in range(per_layer)]
 
 
 class PackedExpertsLayoutReader:
@@ -105,53 +170,12 @@ class PackedExpertsLayoutReader:
                 root = json.loads(fh.read().decode("utf-8"))
         except (ValueError, UnicodeDecodeError) as exc:
             raise ModelError.index_corrupt(f"layout.json: {exc}") from None
-        if not isinstance(root, dict):
-            root = {}
-        stride = _uint(root.get("expertStride"))
-        n_layers = root.get("numLayers")
-        per_layer = root.get("expertsPerLayer")
-        layers_arr = root.get("layers")
-        if (stride is None or not _is_int(n_layers) or not _is_int(per_layer)
-                or not isinstance(layers_arr, list) or not all(isinstance(x, dict) for x in layers_arr)):
-            raise ModelError.index_corrupt("layout.json: missing top-level keys")
-
+        stride, n_layers, per_layer, layer_objs = _take(root, _TOP, "missing top-level keys")
         layers: List[LayerLayout] = []
-        for obj in layers_arr:
-            layer_idx, file, experts_arr = obj.get("layer"), obj.get("file"), obj.get("experts")
-            if (not _is_int(layer_idx) or not isinstance(file, str) or not isinstance(experts_arr, list)
-                    or not all(isinstance(x, dict) for x in experts_arr)):
-                raise ModelError.index_corrupt("layout.json: malformed layer entry")
-            if not experts_arr:   # leading dense-FFN layers: an empty entry, no blob file
-                layers.append(LayerLayout(layer_idx, file, []))
-                continue
-            experts: List[Optional[ExpertEntry]] = [None] * per_layer
-            for eobj in experts_arr:
-                off, esize, tensors = _uint(eobj.get("offset")), _uint(eobj.get("size")), eobj.get("tensors")
-                if (off is None or esize is None or not isinstance(tensors, dict)
-                        or not all(isinstance(t, dict) for t in tensors.values())):
-                    raise ModelError.index_corrupt("layout.json: malformed expert entry")
-                subs: Dict[str, SubTensorEntry] = {}
-                for role, t in tensors.items():
-                    toff, tsize = _uint(t.get("offset")), _uint(t.get("size"))
-                    shape = t.get("shape")
-                    if (toff is None or tsize is None or not isinstance(t.get("dtype"), str)
-                            or not isinstance(shape, list) or not all(_is_int(s) for s in shape)):
-                        raise ModelError.index_corrupt(f"layout.json: malformed tensor {role}")
-                    if "bits" in t and not _is_int(t["bits"]):
-                        raise ModelError.index_corrupt(f"layout.json: malformed tensor bits {role}")
-                    subs[role] = SubTensorEntry(toff, tsize)
-                expert_id = eobj.get("expert")
-                if not _is_int(expert_id):   # absent id: the next free position in file order
-                    expert_id = sum(1 for x in experts if x is not None)
-                if expert_id < 0 or expert_id >= per_layer:
-                    raise ModelError.index_corrupt("layout.json: expert id out of range")
-                rank = eobj.get("physicalRank")
-                if _is_int(rank) and (rank < 0 or rank >= per_layer):
-                    raise ModelError.index_corrupt("layout.json: physicalRank out of range")
-                experts[expert_id] = ExpertEntry(expert_id, off, esize, subs)
-            if any(x is None for x in experts):
-                raise ModelError.index_corrupt("layout.json: missing expert entries")
-            layers.append(LayerLayout(layer_idx, file, list(experts)))   # type: ignore[arg-type]
+        for obj in layer_objs:
+            index, file, entries = _take(obj, _LAYER, "malformed layer entry")
+            # a leading dense-FFN layer is an entry without experts and without a blob file
+            layers.append(LayerLayout(index, file, _layer_experts(entries, per_layer) if entries else []))
         return PackedExpertsLayout(stride, n_layers, per_layer, layers)
 
 

@@ -642,6 +642,42 @@ def bench_family_routers(args, device) -> int:
     return 0
 
 
+def phase_trace(ctx, w, stack, moes, device) -> int:
+    """Stage stamps every workgroup of the fused decode launch writes (100 MHz wall clock): per stamp
+    the median over the layers of the earliest / median / latest workgroup, in us from the start of the
+    layer's first workgroup, and the time from the end of one launch to the start of the next."""
+    import numpy as np
+    import torch
+    from mference_amd import _capi
+    L = len(moes)
+    ncu = _capi.lib().mf_ctx_num_cu(ctx.handle)
+    xs = torch.randn((L, w["t"], w["d"]), device=device).to(torch.bfloat16)
+    ys = torch.zeros_like(xs)
+    stamps = torch.zeros((L, ncu * 8), dtype=torch.int64, device=device)
+    for l in range(L):
+        moes[l].set_phase_trace(stamps[l])
+    for _ in range(6):
+        for l in range(L):
+            moes[l].encode_decode_layer(stack[l], xs[l], ys[l], t=w["t"])
+    torch.cuda.synchronize()
+    for m in moes:
+        m.status()
+        m.set_phase_trace(None)
+    t = stamps.cpu().numpy().reshape(L, ncu, 8).astype(np.float64)
+    names = ["start", "stage_a_done", "logits_gathered", "topk_done", "stage_b_done", "activations_gathered", "end"]
+    skip = min(8, L // 2)   # the first layers of a pass start behind an idle device
+    rel = (t[:, :, :7] - t[:, :, 0].min(axis=1)[:, None, None]) / 100.0
+    out = {"workload": w["name"], "layers": L, "workgroups": int(ncu), "unit": "us from the layer's first workgroup start",
+           "stamps": {n: {"earliest": round(float(np.median(rel[skip:, :, i].min(axis=1))), 2),
+                          "median": round(float(np.median(np.median(rel[skip:, :, i], axis=1))), 2),
+                          "latest": round(float(np.median(rel[skip:, :, i].max(axis=1))), 2)}
+                      for i, n in enumerate(names)},
+           "gap_end_to_next_start_us": round(float(np.median(
+               [(t[l, :, 0].min() - t[l - 1, :, 6].max()) / 100.0 for l in range(skip + 1, L)])), 2)}
+    print(json.dumps(out))
+    return 0
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -662,6 +698,9 @@ def main() -> int:
     ap.add_argument("--no-prefill", action="store_true", help="skip the ragged prefill section")
     ap.add_argument("--prefill-only", action="store_true",
                     help="one layer, the ragged prefill section only (for profiling)")
+    ap.add_argument("--phase-trace", action="store_true",
+                    help="stage stamps of the fused decode launch (eager launches, the layer stack six "
+                         "times over, the last pass reported) instead of the timed run")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build measures one GPU only (--gpus 1); no multi-GPU path exists",
@@ -704,6 +743,9 @@ def main() -> int:
                     shared_bits=w["shared_bits"], maple_rounding=bool(w.get("maple")),
                     router_mode=ops.ROUTER_FULL_SOFTMAX if w["bits"] == 1 else ops.ROUTER_TOPK_SOFTMAX)
             for _ in range(L)]
+
+    if args.phase_trace:
+        return phase_trace(ctx, w, stack, moes, device)
 
     gen = torch.Generator(device=device)
     gen.manual_seed(ROOT_SEED + 0x100 * w["config"] + 0xFF)
@@ -811,6 +853,9 @@ def main() -> int:
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS,
                      "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBPS, 4),
                      "traffic": profiled_traffic_bytes() if args.workload == "qwen-decode" else None,
+                     "traffic_source": "rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE summary committed as "
+                                       "profiles/fused_decode_qwen_t1.md (a constant of that profile run, not "
+                                       "measured by this run)" if args.workload == "qwen-decode" else None,
                      "kernel": "mf::fused_decode_kernel (one launch per layer)",
                      "algorithmic_bytes_per_layer": ab["expert_bytes"]},
     }

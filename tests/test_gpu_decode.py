@@ -603,6 +603,23 @@ def test_silu_mul_matches_oracle(gpu, oracle, count):
     assert np.all(got[count:] == 0x3F80)  # nothing written past count
 
 
+@pytest.mark.parametrize("count", [1, 7, 64, 2048, 5001])
+def test_residual_add_matches_oracle(gpu, oracle, count):
+    """residual_add_fp16 (utility.metal:83-92): hidden = narrow(hidden + delta), one rounding, in place,
+    nothing written past count"""
+    rng = oracle.Rng.key(0x52, f"residual-add-{count}")
+    hb = oracle.bf16_bits(rng.normal(0.0, 2.0, count).astype(np.float32))
+    db = oracle.bf16_bits(rng.normal(0.0, 0.5, count).astype(np.float32))
+    ref = oracle.bf16_bits(oracle.bf16_to_float(hb) + oracle.bf16_to_float(db))
+    hidden = torch.full((count + 8,), 1.0, dtype=torch.bfloat16, device="cuda")
+    hidden[:count] = ops.bf16_tensor(hb)
+    ops.Elementwise(gpu).encode_residual_add(hidden, ops.bf16_tensor(db), count)
+    _sync()
+    got = ops.bf16_bits(hidden)
+    assert np.array_equal(got[:count], ref)
+    assert np.all(got[count:] == 0x3F80)
+
+
 def test_nibble_widened_ternary_gemv_exact_bits(gpu, oracle):
     """MapleTernaryGEMV.encode on the resident projections' storage (maple_ternary.metal:12-81): ternary
     codes widened to nibbles with scale (alpha) and bias (-alpha) tables repeated over each source group

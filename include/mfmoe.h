@@ -352,6 +352,30 @@ mf_status mf_moe_phase2(mf_moe* h, mf_stream stream, const void* expert_base,
 mf_status mf_expert_blob_layout(uint32_t d, uint32_t f, mf_bits bits, uint32_t align, mf_expert_offsets* offsets,
                                 size_t* blob_bytes, size_t* stride);
 
+/* The routed phases over slots named directly, for a caller that holds its experts in slots of its
+ * own (a streaming cache) instead of one pool indexed by expert id.  Slot s = token * top_k + rank
+ * reads the blob at (uint8*)slab + slot_offsets[s]:
+ *  - slab + per-slot byte offsets: MoE.encodeSlotMapGuardedFFN (Kernels/MoE/MoE.swift:333-407; kernels
+ *    moe_phase1_gate_up_act_slotmap / moe_phase2_down_reduce_slotmap, Metal/MoE/moe.metal:619-708);
+ *  - slab == NULL and the table holding device ADDRESSES: the routed argument buffer of K
+ *    (buffer, offset) pairs, MoE.makeRoutedArgumentBuffer + encodeRoutedPersistentPhase1U16Load /
+ *    encodeRoutedPersistentPhase2Reduce(routedArgBuffer:routedBlobs:) (MoE.swift:205-253, 409-440).
+ * slot_offsets: device, uint64 [t * top_k] (the reference's are 32-bit: its slab is below 4 GiB); every
+ * blob starts on a 16-byte boundary.  all_hit (nullable): a device word; the launches do nothing while it
+ * reads 0 -- the guard of the reference's slot-map form, whose lookup kernel writes it.
+ * mf_moe_slot_lookup is that kernel, router_slot_lookup_k8 (moe.metal:594-617): slot_of is the caller's
+ * device table int16 [num_experts] (negative: not in a slot); out_slot_offsets[s] = slot * slot_stride,
+ * out_all_hit = 1 when every routed expert of the call has a slot. */
+mf_status mf_moe_slot_lookup(mf_moe* h, mf_stream stream, const uint32_t* idx, uint32_t t,
+                             const int16_t* slot_of, uint64_t slot_stride, uint64_t* out_slot_offsets,
+                             uint32_t* out_all_hit);
+mf_status mf_moe_phase1_slots(mf_moe* h, mf_stream stream, const void* slab, const uint64_t* slot_offsets,
+                              const uint32_t* all_hit, const mf_expert_offsets* offsets, const uint16_t* x,
+                              uint32_t t, uint32_t x_stride, uint16_t* acts);
+mf_status mf_moe_phase2_slots(mf_moe* h, mf_stream stream, const void* slab, const uint64_t* slot_offsets,
+                              const uint32_t* all_hit, const mf_expert_offsets* offsets, const float* w,
+                              const uint16_t* acts, const uint16_t* residual, uint32_t t, uint16_t* y);
+
 /* Everything one layer reads. */
 typedef struct {
   const uint16_t* router_w;   /* bf16 [num_experts, d]; NULL: the routing is the caller's -- the layer

@@ -311,6 +311,24 @@ class MoE {
                          uint32_t* outIndices = nullptr, float* outWeights = nullptr) const {
     check(mf_moe_decode_layer(h_, cb, &weights, x, tokens, y, hidden, outIndices, outWeights), ctx_);
   }
+  // router_slot_lookup_k8 + encodeSlotMapGuardedFFN's two routed launches (MoE.swift:333-407), and the
+  // routed-argument-buffer forms (MoE.swift:205-253, 409-440: slab == nullptr, the table holds addresses)
+  void encodeSlotLookup(mf_stream cb, const uint32_t* indices, const int16_t* slotOf, uint64_t slotStride,
+                        uint64_t* outSlotOffsets, uint32_t* outAllHit, uint32_t tokens = 1) const {
+    check(mf_moe_slot_lookup(h_, cb, indices, tokens, slotOf, slotStride, outSlotOffsets, outAllHit), ctx_);
+  }
+  void encodeRoutedPhase1Slots(mf_stream cb, const void* slab, const uint64_t* slotOffsets, const uint32_t* allHit,
+                               const MoEExpertOffsets& routedOffsets, const uint16_t* x, uint16_t* acts,
+                               uint32_t tokens = 1) const {
+    check(mf_moe_phase1_slots(h_, cb, slab, slotOffsets, allHit, &routedOffsets, x, tokens, cfg_.d, acts), ctx_);
+  }
+  void encodeRoutedPhase2ReduceSlots(mf_stream cb, const void* slab, const uint64_t* slotOffsets,
+                                     const uint32_t* allHit, const MoEExpertOffsets& routedOffsets,
+                                     const float* routingWeights, const uint16_t* acts, const uint16_t* residual,
+                                     uint16_t* y, uint32_t tokens = 1) const {
+    check(mf_moe_phase2_slots(h_, cb, slab, slotOffsets, allHit, &routedOffsets, routingWeights, acts, residual,
+                              tokens, y), ctx_);
+  }
   // PrefillGroupedRoutedMoE.encodeStreamedBatched + PrefillMoE.encodeReduceTokenMajor +
   // PrefillSharedExpert.encodeBlock (PrefillGroupedRoutedMoE.swift:392-466, PrefillMoE.swift:11-38,
   // PrefillSharedExpert.swift:81-99) for `tokens` rows

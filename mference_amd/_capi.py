@@ -106,6 +106,9 @@ SIGNATURES = {
     "mf_moe_group_status": (_I, [_P, _P]),
     "mf_moe_prefill_workspace_bytes": (_SZ, [_P, _U32]),
     "mf_moe_prefill_layer": (_I, [_P, _P, C.POINTER(LayerWeights), _P, _U32, _P, _P, _SZ, _P, _P]),
+    "mf_moe_slot_lookup": (_I, [_P, _P, _P, _U32, _P, C.c_uint64, _P, _P]),
+    "mf_moe_phase1_slots": (_I, [_P, _P, _P, _P, _P, C.POINTER(ExpertOffsets), _P, _U32, _U32, _P]),
+    "mf_moe_phase2_slots": (_I, [_P, _P, _P, _P, _P, C.POINTER(ExpertOffsets), _P, _P, _P, _U32, _P]),
     "mf_moe_ragged_qmm": (_I, [_P, _P, _P, _SZ, C.POINTER(ExpertOffsets), _P, _P, _P, _U32, _P, _P, _SZ]),
     "mf_moe_unpermute": (_I, [_P, _P, _P, _P, _P, _P, _U32, _P]),
     "mf_group_pairs_host": (_I, [_P, _SZ, _I, _I, _I, _I, _P, _SZ, _P, _P, _P, _P,

@@ -484,6 +484,44 @@ mf_status mf_moe_phase1_subset(mf_moe* h, mf_stream stream, const void* expert_b
   return MF_OK;
 }
 
+mf_status mf_moe_slot_lookup(mf_moe* h, mf_stream stream, const uint32_t* idx, uint32_t t,
+                             const int16_t* slot_of, uint64_t slot_stride, uint64_t* out_slot_offsets,
+                             uint32_t* out_all_hit) {
+  if (!h || !idx || !slot_of || !out_slot_offsets || !out_all_hit) return MF_ERR_INVALID_ARGUMENT;
+  if (t == 0 || t > MF_MAX_TOKENS) return MF_ERR_INVALID_ARGUMENT;
+  if ((reinterpret_cast<uintptr_t>(out_slot_offsets) & 7u) || (reinterpret_cast<uintptr_t>(slot_of) & 1u))
+    return MF_ERR_INVALID_ARGUMENT;
+  MF_HIP(h->ctx, mf::launch_slot_lookup(static_cast<hipStream_t>(stream), idx, slot_of, t * h->cfg.top_k,
+                                        h->cfg.num_experts, slot_stride, out_slot_offsets, out_all_hit));
+  return MF_OK;
+}
+
+mf_status mf_moe_phase1_slots(mf_moe* h, mf_stream stream, const void* slab, const uint64_t* slot_offsets,
+                              const uint32_t* all_hit, const mf_expert_offsets* offsets, const uint16_t* x,
+                              uint32_t t, uint32_t x_stride, uint16_t* acts) {
+  if (!h || !slot_offsets || !offsets || !x || !acts) return MF_ERR_INVALID_ARGUMENT;
+  if (t == 0 || x_stride < h->cfg.d) return MF_ERR_INVALID_ARGUMENT;
+  if (!offsets_ok(*offsets, h->cfg.bits) || !mf::aligned2(slab) || !mf::aligned2(x) || !mf::aligned2(acts) ||
+      (reinterpret_cast<uintptr_t>(slot_offsets) & 7u))
+    return MF_ERR_INVALID_ARGUMENT;
+  MF_HIP(h->ctx, mf::launch_phase1(static_cast<hipStream_t>(stream), h->cfg, slab, 0, *offsets, nullptr, x, t,
+                                   x_stride, acts, nullptr, 0, slot_offsets, all_hit));
+  return MF_OK;
+}
+
+mf_status mf_moe_phase2_slots(mf_moe* h, mf_stream stream, const void* slab, const uint64_t* slot_offsets,
+                              const uint32_t* all_hit, const mf_expert_offsets* offsets, const float* w,
+                              const uint16_t* acts, const uint16_t* residual, uint32_t t, uint16_t* y) {
+  if (!h || !slot_offsets || !offsets || !w || !acts || !y) return MF_ERR_INVALID_ARGUMENT;
+  if (t == 0) return MF_ERR_INVALID_ARGUMENT;
+  if (!offsets_ok(*offsets, h->cfg.bits) || !mf::aligned2(slab) || !mf::aligned2(acts) || !mf::aligned2(y) ||
+      (residual && !mf::aligned2(residual)) || (reinterpret_cast<uintptr_t>(slot_offsets) & 7u))
+    return MF_ERR_INVALID_ARGUMENT;
+  MF_HIP(h->ctx, mf::launch_phase2(static_cast<hipStream_t>(stream), h->cfg, slab, 0, *offsets, nullptr, w, acts,
+                                   residual, t, y, slot_offsets, all_hit));
+  return MF_OK;
+}
+
 mf_status mf_moe_phase2(mf_moe* h, mf_stream stream, const void* expert_base,
                         size_t expert_stride, const mf_expert_offsets* offsets,
                         const uint32_t* idx, const float* w, const uint16_t* acts,

@@ -109,10 +109,15 @@ hipError_t static_scratch_init(int device);
 hipError_t launch_phase1(hipStream_t s, const mf_moe_config& cfg, const void* base, size_t stride,
                          const mf_expert_offsets& off, const uint32_t* idx, const uint16_t* x,
                          uint32_t t, uint32_t x_stride, uint16_t* acts, const uint32_t* subset = nullptr,
-                         uint32_t n_subset = 0);
+                         uint32_t n_subset = 0, const uint64_t* slot_offsets = nullptr,
+                         const uint32_t* all_hit = nullptr);
 hipError_t launch_phase2(hipStream_t s, const mf_moe_config& cfg, const void* base, size_t stride,
                          const mf_expert_offsets& off, const uint32_t* idx, const float* w,
-                         const uint16_t* acts, const uint16_t* residual, uint32_t t, uint16_t* y);
+                         const uint16_t* acts, const uint16_t* residual, uint32_t t, uint16_t* y,
+                         const uint64_t* slot_offsets = nullptr, const uint32_t* all_hit = nullptr);
+hipError_t launch_slot_lookup(hipStream_t s, const uint32_t* idx, const int16_t* slot_of, uint32_t n_slots_in,
+                              uint32_t num_experts, uint64_t slot_stride, uint64_t* out_offsets,
+                              uint32_t* out_all_hit);
 
 
 // moe_fused.hip

@@ -8,6 +8,15 @@
 
 namespace mf {
 
+// Slots named directly instead of through expert indices: slot s of the call reads the blob at
+// base + offsets[s] (base null: the table holds device addresses).  all_hit (optional): a device word
+// that switches the launch off when zero (the reference's slot-map lookup found a routed expert
+// missing from its slots, router_slot_lookup_k8, moe.metal:594-617).
+struct SlotMap {
+  const uint64_t* offsets;
+  const uint32_t* all_hit;
+};
+
 struct BlobView {
   const uint8_t* gw; const uint16_t* gs; const uint16_t* gb;
   const uint8_t* uw; const uint16_t* us; const uint16_t* ub;
@@ -45,7 +54,7 @@ __global__ __launch_bounds__(256) void phase1_kernel(const uint8_t* __restrict__
                                                      uint32_t K, float limit, int maple,
                                                      uint32_t lpr_log2,
                                                      const uint32_t* __restrict__ subset,
-                                                     uint32_t all_pairs) {
+                                                     uint32_t all_pairs, const SlotMap slots) {
   constexpr int EPL = Fmt<BITS>::kElemsPer16B;
   const uint32_t lane = threadIdx.x & 63;
   const uint32_t wave = (blockIdx.x * blockDim.x + threadIdx.x) >> 6;
@@ -61,12 +70,19 @@ __global__ __launch_bounds__(256) void phase1_kernel(const uint8_t* __restrict__
   const uint32_t row = (wave % waves_per_pair) * rpw + (lane >> lpr_log2);
   const uint32_t sub = lane & (lpr - 1);
   const bool row_ok = row < F;
-  const uint32_t expert = idx[pair];
-  if (expert >= E) {  // router sentinel: the slot contributes nothing
-    if (row_ok && sub == 0) acts[static_cast<size_t>(pair) * F + row] = 0;
-    return;
+  if (slots.all_hit && *slots.all_hit == 0u) return;  // guarded form: nothing unless every slot was found
+  const uint8_t* blob;
+  if (slots.offsets) {  // the slot's blob is named directly (moe_phase1_gate_up_act_slotmap, moe.metal:619-708)
+    blob = base + slots.offsets[pair];
+  } else {
+    const uint32_t expert = idx[pair];
+    if (expert >= E) {  // router sentinel: the slot contributes nothing
+      if (row_ok && sub == 0) acts[static_cast<size_t>(pair) * F + row] = 0;
+      return;
+    }
+    blob = base + static_cast<size_t>(expert) * stride;
   }
-  const BlobView bv = view_blob(base + static_cast<size_t>(expert) * stride, off);
+  const BlobView bv = view_blob(blob, off);
   const uint16_t* xt = x + static_cast<size_t>(pair / K) * x_stride;
   const uint32_t n_groups = D / kGroup;
   const size_t row_bytes = static_cast<size_t>(D) * Store<BITS>::kBits / 8;
@@ -119,8 +135,10 @@ __global__ __launch_bounds__(256) void phase2_kernel(const uint8_t* __restrict__
                                                      const uint16_t* __restrict__ residual,
                                                      uint16_t* __restrict__ y, uint32_t D,
                                                      uint32_t F, uint32_t E, uint32_t T,
-                                                     uint32_t K, int maple, uint32_t lpr_log2) {
+                                                     uint32_t K, int maple, uint32_t lpr_log2,
+                                                     const SlotMap slots) {
   constexpr int EPL = Fmt<BITS>::kElemsPer16B;
+  if (slots.all_hit && *slots.all_hit == 0u) return;
   const uint32_t lane = threadIdx.x & 63;
   const uint32_t wave = (blockIdx.x * blockDim.x + threadIdx.x) >> 6;
   const uint32_t lpr = 1u << lpr_log2;
@@ -137,9 +155,15 @@ __global__ __launch_bounds__(256) void phase2_kernel(const uint8_t* __restrict__
   float acc = residual ? bf16_to_f(residual[static_cast<size_t>(tok) * D + r]) : 0.0f;
   for (uint32_t k = 0; k < K; ++k) {
     const uint32_t pair = tok * K + k;
-    const uint32_t expert = idx[pair];
-    if (expert >= E) continue;
-    const BlobView bv = view_blob(base + static_cast<size_t>(expert) * stride, off);
+    const uint8_t* blob;
+    if (slots.offsets) {
+      blob = base + slots.offsets[pair];
+    } else {
+      const uint32_t expert = idx[pair];
+      if (expert >= E) continue;
+      blob = base + static_cast<size_t>(expert) * stride;
+    }
+    const BlobView bv = view_blob(blob, off);
     const uint16_t* a = acts + static_cast<size_t>(pair) * F;
     float part = 0.0f;
     for (uint32_t e0 = sub * EPL; e0 < F; e0 += lpr * EPL) {
@@ -159,6 +183,25 @@ __global__ __launch_bounds__(256) void phase2_kernel(const uint8_t* __restrict__
   if (row_ok && sub == 0) y[static_cast<size_t>(tok) * D + row] = f_to_bf16(acc);
 }
 
+// router_slot_lookup_k8 (moe.metal:594-617): the slot of every routed expert from the caller's
+// expert -> slot table (negative: not resident), as a byte offset into the slab, and whether all of
+// them were found.  One workgroup; n routes.
+__global__ __launch_bounds__(256) void slot_lookup_kernel(const uint32_t* __restrict__ idx,
+                                                          const int16_t* __restrict__ slot_of, uint32_t n,
+                                                          uint32_t E, uint64_t slot_stride,
+                                                          uint64_t* __restrict__ out_offsets,
+                                                          uint32_t* __restrict__ out_all_hit) {
+  bool miss = false;
+  for (uint32_t i = threadIdx.x; i < n; i += blockDim.x) {
+    const uint32_t e = min(idx[i], E - 1u);
+    const int slot = slot_of[e];
+    miss |= slot < 0;
+    out_offsets[i] = slot < 0 ? 0ull : static_cast<uint64_t>(slot) * slot_stride;
+  }
+  const int any_miss = __syncthreads_or(miss ? 1 : 0);
+  if (threadIdx.x == 0) *out_all_hit = any_miss ? 0u : 1u;
+}
+
 namespace {
 
 bool blob_aligned(const void* base, size_t stride, const mf_expert_offsets& o) {
@@ -171,11 +214,11 @@ bool blob_aligned(const void* base, size_t stride, const mf_expert_offsets& o) {
 hipError_t launch_phase1(hipStream_t s, const mf_moe_config& cfg, const void* base, size_t stride,
                          const mf_expert_offsets& off, const uint32_t* idx, const uint16_t* x,
                          uint32_t t, uint32_t x_stride, uint16_t* acts, const uint32_t* subset,
-                         uint32_t n_subset) {
+                         uint32_t n_subset, const uint64_t* slot_offsets, const uint32_t* all_hit) {
   const uint32_t all_pairs = t * cfg.top_k;
   const uint32_t pairs = subset ? n_subset : all_pairs;
   if (!pairs) return hipSuccess;
-  const bool al = blob_aligned(base, stride, off) && aligned16(x) && (x_stride % 8 == 0);
+  const bool al = blob_aligned(base, slot_offsets ? 0 : stride, off) && aligned16(x) && (x_stride % 8 == 0);
   const auto* b = static_cast<const uint8_t*>(base);
 #define MF_P1(BITS, AL)                                                                          \
   {                                                                                              \
@@ -184,7 +227,8 @@ hipError_t launch_phase1(hipStream_t s, const mf_moe_config& cfg, const void* ba
     const uint32_t waves = pairs * ((cfg.f + rpw - 1) / rpw);                                    \
     phase1_kernel<BITS, AL><<<dim3((waves + 3) / 4), dim3(256), 0, s>>>(                         \
         b, stride, off, idx, x, x_stride, acts, cfg.d, cfg.f, cfg.num_experts, pairs, cfg.top_k, \
-        cfg.swiglu_limit, static_cast<int>(cfg.maple_rounding), lpr_log2, subset, all_pairs);    \
+        cfg.swiglu_limit, static_cast<int>(cfg.maple_rounding), lpr_log2, subset, all_pairs,     \
+        SlotMap{slot_offsets, all_hit});                                                         \
   }
   switch (cfg.bits) {
     case MF_BITS_4: if (al) MF_P1(kBits4, true) else MF_P1(kBits4, false) break;
@@ -196,7 +240,8 @@ hipError_t launch_phase1(hipStream_t s, const mf_moe_config& cfg, const void* ba
 #define MF_P1G(AL)                                                                                  \
   phase1_kernel<kBits2, AL, true><<<dim3((waves + 3) / 4), dim3(256), 0, s>>>(                      \
       b, stride, off, idx, x, x_stride, acts, cfg.d, cfg.f, cfg.num_experts, pairs, cfg.top_k,      \
-      cfg.swiglu_limit, static_cast<int>(cfg.maple_rounding), lpr_log2, subset, all_pairs)
+      cfg.swiglu_limit, static_cast<int>(cfg.maple_rounding), lpr_log2, subset, all_pairs,          \
+      SlotMap{slot_offsets, all_hit})
         if (al) MF_P1G(true); else MF_P1G(false);
 #undef MF_P1G
         break;
@@ -209,11 +254,21 @@ hipError_t launch_phase1(hipStream_t s, const mf_moe_config& cfg, const void* ba
   return hipGetLastError();
 }
 
+hipError_t launch_slot_lookup(hipStream_t s, const uint32_t* idx, const int16_t* slot_of, uint32_t n_slots_in,
+                              uint32_t num_experts, uint64_t slot_stride, uint64_t* out_offsets,
+                              uint32_t* out_all_hit) {
+  slot_lookup_kernel<<<dim3(1), dim3(256), 0, s>>>(idx, slot_of, n_slots_in, num_experts, slot_stride, out_offsets,
+                                                   out_all_hit);
+  return hipGetLastError();
+}
+
 hipError_t launch_phase2(hipStream_t s, const mf_moe_config& cfg, const void* base, size_t stride,
                          const mf_expert_offsets& off, const uint32_t* idx, const float* w,
-                         const uint16_t* acts, const uint16_t* residual, uint32_t t, uint16_t* y) {
+                         const uint16_t* acts, const uint16_t* residual, uint32_t t, uint16_t* y,
+                         const uint64_t* slot_offsets, const uint32_t* all_hit) {
   if (!t) return hipSuccess;
-  const bool al = blob_aligned(base, stride, off) && aligned16(acts);
+  // (with a slot table the caller promises blobs on 16-byte boundaries; `stride` is not used)
+  const bool al = blob_aligned(base, slot_offsets ? 0 : stride, off) && aligned16(acts);
   const auto* b = static_cast<const uint8_t*>(base);
 #define MF_P2(BITS, AL)                                                                      \
   {                                                                                          \
@@ -222,7 +277,8 @@ hipError_t launch_phase2(hipStream_t s, const mf_moe_config& cfg, const void* ba
     const uint32_t waves = t * ((cfg.d + rpw - 1) / rpw);                                    \
     phase2_kernel<BITS, AL><<<dim3((waves + 3) / 4), dim3(256), 0, s>>>(                     \
         b, stride, off, idx, w, acts, residual, y, cfg.d, cfg.f, cfg.num_experts, t,         \
-        cfg.top_k, static_cast<int>(cfg.maple_rounding), lpr_log2);                          \
+        cfg.top_k, static_cast<int>(cfg.maple_rounding), lpr_log2,                           \
+        SlotMap{slot_offsets, all_hit});                                                     \
   }
   switch (cfg.bits) {
     case MF_BITS_4: if (al) MF_P2(kBits4, true) else MF_P2(kBits4, false) break;

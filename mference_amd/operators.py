@@ -414,6 +414,29 @@ class MoE:
                                         _ptr(acts), _ptr(residual), t, _ptr(y)),
               self.context.handle)
 
+    def encode_slot_lookup(self, indices, slot_of, slot_stride: int, out_slot_offsets, out_all_hit,
+                           t: int = 1, stream=None):
+        """router_slot_lookup_k8 (moe.metal:594-617): slot byte offsets of the routed experts from the
+        caller's expert -> slot table (int16, negative = not resident), and the all-hit word."""
+        check(_capi.lib().mf_moe_slot_lookup(self._h, _stream(stream), _ptr(indices), t, _ptr(slot_of),
+                                             slot_stride, _ptr(out_slot_offsets), _ptr(out_all_hit)),
+              self.context.handle)
+
+    def encode_routed_phase1_slots(self, slab, slot_offsets, offsets: ExpertOffsets, x, acts, t: int = 1,
+                                   all_hit=None, stream=None):
+        """Phase 1 over slots named directly (MoE.swift:205-253 with `slab=None` and a table of device
+        addresses; MoE.swift:333-407 with a slab and byte offsets, guarded by `all_hit`)."""
+        check(_capi.lib().mf_moe_phase1_slots(self._h, _stream(stream), _ptr(slab), _ptr(slot_offsets),
+                                              _ptr(all_hit), C.byref(offsets), _ptr(x), t, x.stride(0) if x.dim() > 1 else self.cfg.d,
+                                              _ptr(acts)), self.context.handle)
+
+    def encode_routed_phase2_reduce_slots(self, slab, slot_offsets, offsets: ExpertOffsets, routing_weights,
+                                          acts, residual, y, t: int = 1, all_hit=None, stream=None):
+        """Phase 2 + rank-ordered reduce over slots named directly (MoE.swift:409-440, 333-407)."""
+        check(_capi.lib().mf_moe_phase2_slots(self._h, _stream(stream), _ptr(slab), _ptr(slot_offsets),
+                                              _ptr(all_hit), C.byref(offsets), _ptr(routing_weights),
+                                              _ptr(acts), _ptr(residual), t, _ptr(y)), self.context.handle)
+
     def encode_decode_layer(self, weights: MoELayerWeights, x, y, t: int = 1, hidden=None,
                             out_indices=None, out_weights=None, stream=None):
         """The fused decode layer (router -> experts -> shared add), one call."""

@@ -388,6 +388,78 @@ def test_gate_projection_at_group_32(gpu, oracle, d, f, e, k, fs, t):
         ops.MoE(gpu, d, f, e, k, bits=4, gate_group_size=32)
 
 
+@pytest.mark.parametrize("bits,t", [(4, 1), (2, 2), (1, 1)])
+def test_routed_phases_over_slots_named_directly(gpu, oracle, bits, t):
+    """The slot-map form (MoE.encodeSlotMapGuardedFFN, MoE.swift:333-407; router_slot_lookup_k8,
+    moe.metal:594-617) and the routed-argument-buffer form (K (buffer, offset) pairs, MoE.swift:205-253,
+    409-440): experts copied into slots of a slab in another order -- or left in two separate buffers and
+    named by address -- give the bits of the pool-indexed calls; with a routed expert missing from the
+    slots the lookup clears the all-hit word and the guarded launches write nothing."""
+    d, f, e, k = 256, 128, 32, 4
+    root = ROOT_SEED + 0x2F0 + bits
+    layer = oracle.synth_layer(root, d, f, e, k, bits=bits, fs=0, router_mode=1 if bits == 1 else 0)
+    x = oracle.synth_x(root, t, d)
+    _, ref_idx, ref_w = oracle.moe_layer(layer, x)
+    moe = make_moe(gpu, layer)
+    wts = to_device_layer(layer)
+    xd = ops.bf16_tensor(x)
+    idx = torch.from_numpy(ref_idx.astype(np.int32)).cuda()
+    w = torch.from_numpy(ref_w).cuda()
+    acts0 = torch.zeros((t, k, f), dtype=torch.bfloat16, device="cuda")
+    y0 = torch.zeros((t, d), dtype=torch.bfloat16, device="cuda")
+    moe.encode_routed_phase1(wts.experts, wts.offsets, idx, xd, acts0, t=t)
+    moe.encode_routed_phase2_reduce(wts.experts, wts.offsets, idx, w, acts0, None, y0, t=t)
+    # a slab of 24 slots, 16-byte aligned stride larger than the blob; the routed experts get slots in
+    # descending order, the others none
+    stride = (layer.experts.shape[1] + 255) // 256 * 256 + 16
+    used = sorted(set(ref_idx.reshape(-1).tolist()))
+    slot_of = np.full(e, -1, np.int16)
+    slab_h = np.full((24, stride), 0xEE, np.uint8)
+    for n, ex in enumerate(reversed(used)):
+        slot_of[ex] = 23 - 2 * n if 23 - 2 * n >= 0 else n
+        slab_h[slot_of[ex], :layer.experts.shape[1]] = layer.experts[ex]
+    slab = torch.from_numpy(slab_h).cuda()
+    so = torch.zeros(t * k, dtype=torch.int64, device="cuda")
+    hit = torch.zeros(1, dtype=torch.int32, device="cuda")
+    moe.encode_slot_lookup(idx, torch.from_numpy(slot_of).cuda(), stride, so, hit, t=t)
+    _sync()
+    assert hit.item() == 1
+    assert np.array_equal(so.cpu().numpy(), slot_of[ref_idx.reshape(-1)].astype(np.int64) * stride)
+    acts1 = torch.zeros_like(acts0)
+    y1 = torch.zeros_like(y0)
+    moe.encode_routed_phase1_slots(slab, so, wts.offsets, xd, acts1, t=t, all_hit=hit)
+    moe.encode_routed_phase2_reduce_slots(slab, so, wts.offsets, w, acts1, None, y1, t=t, all_hit=hit)
+    _sync()
+    assert np.array_equal(ops.bf16_bits(acts1), ops.bf16_bits(acts0))
+    assert np.array_equal(ops.bf16_bits(y1), ops.bf16_bits(y0))
+    # one routed expert loses its slot: the word reads 0 and the guarded launches leave their outputs alone
+    gone = slot_of.copy()
+    gone[used[0]] = -1
+    moe.encode_slot_lookup(idx, torch.from_numpy(gone).cuda(), stride, so, hit, t=t)
+    acts2 = torch.full_like(acts0, 3.0)
+    y2 = torch.full_like(y0, 5.0)
+    moe.encode_routed_phase1_slots(slab, so, wts.offsets, xd, acts2, t=t, all_hit=hit)
+    moe.encode_routed_phase2_reduce_slots(slab, so, wts.offsets, w, acts2, None, y2, t=t, all_hit=hit)
+    _sync()
+    assert hit.item() == 0 and torch.all(acts2 == 3.0).item() and torch.all(y2 == 5.0).item()
+    # the argument-buffer form: no slab, the table holds the device address of every slot's blob; the
+    # blobs sit in two separate allocations
+    half = [ex for n, ex in enumerate(used) if n % 2 == 0]
+    buf_a = torch.from_numpy(np.ascontiguousarray(layer.experts[half])).cuda()
+    rest = [ex for ex in used if ex not in half]
+    buf_b = torch.from_numpy(np.ascontiguousarray(layer.experts[rest])).cuda() if rest else buf_a
+    addr = {ex: buf_a.data_ptr() + n * buf_a.stride(0) for n, ex in enumerate(half)}
+    addr.update({ex: buf_b.data_ptr() + n * buf_b.stride(0) for n, ex in enumerate(rest)})
+    table = torch.from_numpy(np.array([addr[int(ex)] for ex in ref_idx.reshape(-1)], np.int64)).cuda()
+    acts3 = torch.zeros_like(acts0)
+    y3 = torch.zeros_like(y0)
+    moe.encode_routed_phase1_slots(None, table, wts.offsets, xd, acts3, t=t)
+    moe.encode_routed_phase2_reduce_slots(None, table, wts.offsets, w, acts3, None, y3, t=t)
+    _sync()
+    assert np.array_equal(ops.bf16_bits(acts3), ops.bf16_bits(acts0))
+    assert np.array_equal(ops.bf16_bits(y3), ops.bf16_bits(y0))
+
+
 @pytest.mark.parametrize("bits,t", [(4, 1), (2, 3), (1, 2)])
 def test_phase1_subsets_write_the_bits_of_the_full_call(gpu, oracle, bits, t):
     """MoEFusedFFNTests.swift:126-186: phase 1 split into slot subsets (the reference's cache hits and

@@ -299,20 +299,33 @@ __device__ __forceinline__ void group_layout(uint32_t c, uint32_t E, uint32_t* _
   const uint32_t e = threadIdx.x;
   const bool act = e < MF_MAX_EXPERTS;
   if (e < E) counts[e] = c;
-  if (act) {
-    s_cnt[e] = c;
-    s_tile[e] = (c + kTileTokens - 1) / kTileTokens;
+  // inclusive scans of the counts and of the tile counts over the MF_MAX_EXPERTS entries: inside a wave
+  // by shuffles, the eight wave totals through the last slots of the two arrays' neighbours
+  __shared__ uint32_t s_wave_cnt[MF_MAX_EXPERTS / 64], s_wave_tile[MF_MAX_EXPERTS / 64];
+  uint32_t run_c = act ? c : 0u, run_t = act ? (c + kTileTokens - 1) / kTileTokens : 0u;
+  const uint32_t lane = e & 63u;
+  for (uint32_t o = 1; o < 64; o <<= 1) {
+    const uint32_t a = static_cast<uint32_t>(__shfl_up(static_cast<int>(run_c), o, 64));
+    const uint32_t b = static_cast<uint32_t>(__shfl_up(static_cast<int>(run_t), o, 64));
+    if (lane >= o) {
+      run_c += a;
+      run_t += b;
+    }
+  }
+  if (act && lane == 63) {
+    s_wave_cnt[e >> 6] = run_c;
+    s_wave_tile[e >> 6] = run_t;
   }
   __syncthreads();
-  for (uint32_t o = 1; o < MF_MAX_EXPERTS; o <<= 1) {  // inclusive scans
-    const uint32_t a = act && e >= o ? s_cnt[e - o] : 0, b = act && e >= o ? s_tile[e - o] : 0;
-    __syncthreads();
-    if (act) {
-      s_cnt[e] += a;
-      s_tile[e] += b;
+  if (act) {
+    for (uint32_t v = 0; v < (e >> 6); ++v) {
+      run_c += s_wave_cnt[v];
+      run_t += s_wave_tile[v];
     }
-    __syncthreads();
+    s_cnt[e] = run_c;
+    s_tile[e] = run_t;
   }
+  __syncthreads();
   // The tile list has tile_slots entries (a multiple of 8).  The matmul sends the workgroups of
   // slot range k * tile_slots/8 .. to XCD k, so every eighth of the list gets an eighth of the
   // live tiles, in expert order; the rest of each eighth stays empty (count 0).
@@ -435,34 +448,27 @@ __global__ __launch_bounds__(256) void group_emit_kernel(const uint32_t* __restr
   }
 }
 
-// The three steps above in one workgroup, for a pair list short enough that one workgroup is not
-// the slower way: each of the 16 waves is a "chunk" (a contiguous run of the pair list), the per-chunk
-// counts live in LDS, and the result is the same stable order.
-constexpr uint32_t kGroupSmallPairs = 2048;
-
-__global__ __launch_bounds__(1024) void group_small_kernel(const uint32_t* __restrict__ idx,
-                                                           const float* __restrict__ w, uint32_t n_pairs,
-                                                           uint32_t K, uint32_t E, uint32_t* __restrict__ counts,
-                                                           uint32_t* __restrict__ offsets,
-                                                           uint32_t* __restrict__ starts,
-                                                           mf_pair* __restrict__ sorted, Tile* __restrict__ tiles,
-                                                           uint32_t tile_slots, uint32_t* __restrict__ n_tiles,
-                                                           uint32_t* __restrict__ status) {
-  __shared__ uint32_t s_hist[16][MF_MAX_EXPERTS];  // routes per expert of each wave, then its running base
-  __shared__ uint32_t s_cnt[MF_MAX_EXPERTS], s_tile[MF_MAX_EXPERTS];
+// The stable counting sort by ballots, in one workgroup of 16 waves: each wave is a "chunk" (a contiguous
+// run of the pair list) with its per-expert counts in LDS (s_hist: [16][MF_MAX_EXPERTS]).
+__device__ __forceinline__ void group_serial(const uint32_t* __restrict__ idx, const float* __restrict__ w,
+                                             uint32_t n_pairs, uint32_t K, uint32_t E,
+                                             uint32_t* __restrict__ counts, uint32_t* __restrict__ offsets,
+                                             uint32_t* __restrict__ starts, mf_pair* __restrict__ sorted,
+                                             Tile* __restrict__ tiles, uint32_t tile_slots,
+                                             uint32_t* __restrict__ n_tiles, uint32_t* s_hist_flat,
+                                             uint32_t* s_cnt, uint32_t* s_tile) {
+  uint32_t (*s_hist)[MF_MAX_EXPERTS] = reinterpret_cast<uint32_t (*)[MF_MAX_EXPERTS]>(s_hist_flat);
   const uint32_t lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
-  for (uint32_t i = threadIdx.x; i < 16 * MF_MAX_EXPERTS; i += blockDim.x) (&s_hist[0][0])[i] = 0;
+  __syncthreads();
+  for (uint32_t i = threadIdx.x; i < 16 * MF_MAX_EXPERTS; i += blockDim.x) s_hist_flat[i] = 0;
   __syncthreads();
   const uint32_t chunk = ((n_pairs + 15) / 16 + 63) / 64 * 64;
   const uint32_t p0 = min(n_pairs, wv * chunk), p1 = min(n_pairs, p0 + chunk);
-  bool bad = false;
   for (uint32_t p = p0 + lane; p < p1; p += 64) {
     const uint32_t e = idx[p];
     if (e < E) atomicAdd(&s_hist[wv][e], 1u);
-    else bad = true;
   }
-  const int any_bad = __syncthreads_or(bad ? 1 : 0);
-  if (threadIdx.x == 0) *status = any_bad ? 2u : 0u;
+  __syncthreads();
   uint32_t c = 0;
   if (threadIdx.x < E) {
 #pragma unroll
@@ -474,7 +480,7 @@ __global__ __launch_bounds__(1024) void group_small_kernel(const uint32_t* __res
   }
   group_layout(c, E, counts, offsets, starts, tiles, tile_slots, n_tiles, s_cnt, s_tile);
   __syncthreads();
-  // s_cnt holds the inclusive scan: an expert's run starts at s_cnt[e] - (its count); the waves' bases are
+  // s_cnt holds the inclusive scan: an expert's run starts at s_cnt[e - 1]; the waves' bases are
   // relative to that start
   for (uint32_t q0 = p0; q0 < p1; q0 += 64) {
     const uint32_t p = q0 + lane;
@@ -497,7 +503,7 @@ __global__ __launch_bounds__(1024) void group_small_kernel(const uint32_t* __res
       todo &= ~same;
     }
     if (mine) {
-      const uint32_t run = (e ? s_cnt[e - 1] : 0u);  // exclusive scan = start of the expert's run
+      const uint32_t run = (e ? s_cnt[e - 1] : 0u);
       mf_pair r;
       r.token = p / K;
       r.expert = e;
@@ -505,6 +511,100 @@ __global__ __launch_bounds__(1024) void group_small_kernel(const uint32_t* __res
       r.weight_bits = __float_as_uint(w[p]);
       sorted[run + pos] = r;
     }
+  }
+}
+
+// The three steps above in one workgroup, for token counts whose (expert x token) bit matrix fits LDS.
+// A token names an expert at most once (a top-k does), so "the routes of expert e in token order" is row
+// e of that matrix: a route's place in its expert's run is the number of set bits before its token's, i.e.
+// a per-word prefix count plus a popcount -- no serial ranking at all.  Every thread marks its routes
+// (LDS atomic OR), the rows are prefix-counted (several threads per row), the expert counts go through the
+// same layout step as the three-launch form, and every thread places its routes.  Input that does name
+// an expert twice in one token (legal for the reference's grouping, never produced by a router) is
+// noticed when the bit is already set; the workgroup then does the stable ranking the slow way (each of
+// its 16 waves a chunk of the pair list, ballots per step) -- same result, same launch.
+constexpr uint32_t kGroupOnePairs = 8192;  // beyond this the pair list is worth several workgroups (T=2048, K=8: 31 us in one, 20 us in three launches)
+constexpr uint32_t kGroupOneMaxBytes = 112 * 1024;  // bit matrix + prefix counts the single workgroup may hold
+
+__host__ __device__ __forceinline__ uint32_t group_one_row_words(uint32_t t) { return ((t + 31) / 32) | 1u; }  // odd: rows fall on different banks
+__host__ __device__ __forceinline__ size_t group_one_lds_bytes(uint32_t t, uint32_t E) {
+  const size_t bits = static_cast<size_t>(E) * group_one_row_words(t) * 6;  // u32 words + u16 prefix counts
+  const size_t serial = 16 * MF_MAX_EXPERTS * 4;                            // the slow path's per-wave counts
+  return (bits > serial ? bits : serial) + 16;
+}
+
+__global__ __launch_bounds__(1024) void group_one_kernel(const uint32_t* __restrict__ idx,
+                                                         const float* __restrict__ w, uint32_t n_pairs,
+                                                         uint32_t K, uint32_t E, uint32_t tpe_log2,
+                                                         uint32_t* __restrict__ counts,
+                                                         uint32_t* __restrict__ offsets,
+                                                         uint32_t* __restrict__ starts,
+                                                         mf_pair* __restrict__ sorted, Tile* __restrict__ tiles,
+                                                         uint32_t tile_slots, uint32_t* __restrict__ n_tiles,
+                                                         uint32_t* __restrict__ status) {
+  extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
+  __shared__ uint32_t s_cnt[MF_MAX_EXPERTS], s_tile[MF_MAX_EXPERTS];
+  const uint32_t T = n_pairs / K, W = group_one_row_words(T);
+  uint32_t* bm = reinterpret_cast<uint32_t*>(smem);                 // [E][W] bits: token t of row e
+  uint16_t* pref = reinterpret_cast<uint16_t*>(smem + static_cast<size_t>(E) * W * 4);  // [E][W] set bits before word
+  for (uint32_t i = threadIdx.x; i < E * W; i += blockDim.x) bm[i] = 0;
+  __syncthreads();
+  bool bad = false, dup = false;
+  for (uint32_t p = threadIdx.x; p < n_pairs; p += blockDim.x) {
+    const uint32_t e = idx[p], t = p / K;
+    if (e < E) {
+      const uint32_t bit = 1u << (t & 31u);
+      dup |= (atomicOr(&bm[e * W + (t >> 5)], bit) & bit) != 0u;
+    } else {
+      bad = true;
+    }
+  }
+  const int any_bad = __syncthreads_or(bad ? 1 : 0);
+  const int any_dup = __syncthreads_or(dup ? 1 : 0);
+  if (threadIdx.x == 0) *status = any_bad ? 2u : 0u;
+  if (any_dup) {
+    group_serial(idx, w, n_pairs, K, E, counts, offsets, starts, sorted, tiles, tile_slots, n_tiles,
+                 reinterpret_cast<uint32_t*>(smem), s_cnt, s_tile);
+    return;
+  }
+  // prefix counts of every row: 2^tpe_log2 threads per row, each a run of words
+  const uint32_t tpe = 1u << tpe_log2, row = threadIdx.x >> tpe_log2, part = threadIdx.x & (tpe - 1u);
+  const uint32_t per = (W + tpe - 1) / tpe, w0 = min(W, part * per), w1 = min(W, w0 + per);
+  uint32_t mine = 0;
+  if (row < E)
+    for (uint32_t j = w0; j < w1; ++j) mine += __popc(bm[row * W + j]);
+  // exclusive scan of `mine` over the row's threads (they are neighbours in one wave: tpe <= 16)
+  uint32_t before = 0, total = mine;
+  for (uint32_t o = 1; o < tpe; o <<= 1) {
+    const uint32_t v = static_cast<uint32_t>(__shfl_up(static_cast<int>(total), o, 64));
+    if (part >= o) total += v;
+  }
+  before = total - mine;
+  const uint32_t row_total = static_cast<uint32_t>(__shfl(static_cast<int>(total), (threadIdx.x & 63u) | (tpe - 1u), 64));
+  if (row < E) {
+    uint32_t c = before;
+    for (uint32_t j = w0; j < w1; ++j) {
+      pref[row * W + j] = static_cast<uint16_t>(c);
+      c += __popc(bm[row * W + j]);
+    }
+    if (part == 0) s_tile[row] = row_total;  // parked for the layout step below
+  }
+  __syncthreads();
+  const uint32_t c = threadIdx.x < E ? s_tile[threadIdx.x] : 0u;
+  __syncthreads();
+  group_layout(c, E, counts, offsets, starts, tiles, tile_slots, n_tiles, s_cnt, s_tile);
+  __syncthreads();
+  for (uint32_t p = threadIdx.x; p < n_pairs; p += blockDim.x) {
+    const uint32_t e = idx[p];
+    if (e >= E) continue;
+    const uint32_t t = p / K, at = e * W + (t >> 5);
+    const uint32_t pos = (e ? s_cnt[e - 1] : 0u) + pref[at] + __popc(bm[at] & ((1u << (t & 31u)) - 1u));
+    mf_pair r;
+    r.token = t;
+    r.expert = e;
+    r.rank = p - t * K;
+    r.weight_bits = __float_as_uint(w[p]);
+    sorted[pos] = r;
   }
 }
 
@@ -1489,8 +1589,14 @@ hipError_t launch_group(hipStream_t s, const uint32_t* idx, const float* w, uint
                         mf_pair* sorted, void* tiles, uint32_t tile_slots, uint32_t* n_tiles,
                         uint32_t* status, uint32_t* chunk_hist) {
   const uint32_t n_pairs = t * K;
-  if (n_pairs && n_pairs <= kGroupSmallPairs) {
-    group_small_kernel<<<dim3(1), dim3(1024), 0, s>>>(idx, w, n_pairs, K, E, counts, offsets, starts, sorted,
+  if (n_pairs && n_pairs <= kGroupOnePairs && group_one_lds_bytes(t, E) <= kGroupOneMaxBytes) {
+    const size_t lds = group_one_lds_bytes(t, E);
+    uint32_t tpe_log2 = 0;  // threads per row of the bit matrix: as many as 1024 threads give, at most 16
+    while (tpe_log2 < 4 && (E << (tpe_log2 + 1)) <= 1024) ++tpe_log2;
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(group_one_kernel),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(kGroupOneMaxBytes));
+    if (e != hipSuccess) return e;
+    group_one_kernel<<<dim3(1), dim3(1024), lds, s>>>(idx, w, n_pairs, K, E, tpe_log2, counts, offsets, starts, sorted,
                                                       static_cast<Tile*>(tiles), tile_slots, n_tiles, status);
     return hipGetLastError();
   }

@@ -23,7 +23,8 @@ def _group_on_device(moe, idx, w, t, k, e):
 
 
 @pytest.mark.parametrize("t,k,e,live", [(1, 8, 16, 16), (37, 4, 16, 16), (300, 8, 256, 256),
-                                        (129, 8, 64, 9), (64, 2, 512, 40)])
+                                        (129, 8, 64, 9), (64, 2, 512, 40), (2048, 8, 256, 200),
+                                        (1500, 8, 512, 512), (6000, 4, 128, 128)])
 def test_device_grouping_matches_oracle(gpu, oracle, t, k, e, live):
     """`live` < e leaves experts without a token: their offset is 0xFFFFFFFF
     (PrefillMoEGrouping.swift:151-160)."""
@@ -39,6 +40,26 @@ def test_device_grouping_matches_oracle(gpu, oracle, t, k, e, live):
     assert np.array_equal(got[:, 1], ref["sorted"]["expert"])
     assert np.array_equal(got[:, 2], ref["sorted"]["rank"])
     assert np.array_equal(got[:, 3], ref["sorted"]["weight_bits"])
+    assert np.array_equal(offsets.cpu().numpy().view(np.uint32), ref["offsets"])
+    assert np.array_equal(counts.cpu().numpy().view(np.uint32), ref["counts"])
+
+
+@pytest.mark.parametrize("t,k,e", [(40, 4, 16), (700, 8, 64), (2048, 8, 256), (5000, 6, 64)])
+def test_device_grouping_with_an_expert_named_twice_in_a_token(gpu, oracle, t, k, e):
+    """The reference's grouping takes any pair list; a token may name one expert under two ranks
+    (PrefillMoEGrouping.swift:91-192 orders such routes by rank).  The device form -- one workgroup with a
+    bit per (expert, token) up to a few thousand tokens, several launches beyond -- keeps that order."""
+    rng = np.random.default_rng(t + e)
+    idx = rng.integers(0, e, size=(t, k)).astype(np.uint32)   # with replacement: plenty of repeats
+    idx[t // 2, :] = 3
+    w = rng.random((t, k), dtype=np.float32)
+    moe = ops.MoE(gpu, 128, 64, e, k)
+    sorted_pairs, offsets, counts = _group_on_device(moe, idx, w, t, k, e)
+    moe.group_status()
+    ref = oracle.group_pairs(oracle.make_pairs(idx, w.view(np.uint32)), t, k, e)
+    got = sorted_pairs.cpu().numpy().view(np.uint32)
+    for col, name in enumerate(("token", "expert", "rank", "weight_bits")):
+        assert np.array_equal(got[:, col], ref["sorted"][name]), name
     assert np.array_equal(offsets.cpu().numpy().view(np.uint32), ref["offsets"])
     assert np.array_equal(counts.cpu().numpy().view(np.uint32), ref["counts"])
 

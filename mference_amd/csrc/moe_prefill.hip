@@ -151,9 +151,15 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
                                                                   const uint16_t* __restrict__ x,
                                                                   uint32_t E, uint32_t D, uint32_t T,
                                                                   uint32_t x_stride,
-                                                                  float* __restrict__ logits, uint32_t ld) {
+                                                                  float* __restrict__ logits, uint32_t ld,
+                                                                  const RouterTail tail) {
   __shared__ float s_part[3][16 * 64];
   const uint32_t lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
+  if (tail.xp && blockIdx.y >= tail.router_cols) {  // an x-preparation workgroup (rows behind the expert blocks)
+    const uint32_t row = ((blockIdx.y - tail.router_cols) * gridDim.x + blockIdx.x) * 4 + wv;
+    if (row < T) prep_x_row(x + static_cast<size_t>(row) * x_stride, tail.xp, tail.sums, tail.w_sg, tail.gate, row, D, lane);
+    return;
+  }
   const uint32_t m = lane & 31, b = lane >> 5;
   // token tiles vary fastest: workgroups go to the XCDs round-robin, so each XCD's L2 sees an
   // eighth of the token rows (and all of the small router matrix)
@@ -1545,9 +1551,20 @@ hipError_t launch_prefill_router(hipStream_t s, const uint16_t* W, const uint16_
   // multiple of 512, rows left over by the blocks of 32, unaligned operands): the register-tiled
   // kernel cannot hold them, so the whole call goes one wave per (token, row) -- the same bits
   if ((D / 8 + 63) / 64 > 8 && e32 != E) return launch_router_logits(s, W, x, E, D, T, x_stride, logits, nullptr);
+  const bool tail_ok = fused.xp && x_stride == D && D % 64 == 0 && aligned16(x) && aligned16(fused.xp) &&
+                       (!fused.w_sg || aligned16(fused.w_sg));
   if (e32) {
-    prefill_router_mfma_kernel<<<dim3((T + 31) / 32, e32 / 32), dim3(256), 0, s>>>(W, x, e32, D, T, x_stride,
-                                                                                  logits, E);
+    RouterTail mt{};
+    uint32_t prep_rows = 0;
+    if (tail_ok) {  // the x preparation rides in this launch: workgroup rows behind the expert blocks
+      mt = fused;
+      mt.router_cols = e32 / 32;
+      prep_rows = ((T + 3) / 4 + (T + 31) / 32 - 1) / ((T + 31) / 32);
+      fused.xp = nullptr;  // done here: the register-tiled launch for left-over rows does not repeat it
+      tail->xp = mt.xp;
+    }
+    prefill_router_mfma_kernel<<<dim3((T + 31) / 32, e32 / 32 + prep_rows), dim3(256), 0, s>>>(W, x, e32, D, T, x_stride,
+                                                                                              logits, E, mt);
     if (e32 == E) return hipGetLastError();
   }
   const uint32_t rest = E - e32;
@@ -1559,8 +1576,7 @@ hipError_t launch_prefill_router(hipStream_t s, const uint16_t* W, const uint16_
   const uint32_t tpb = e32 ? 4u : std::max(4u, std::min(64u, T / 64));
   const uint32_t token_blocks = (T + tpb - 1) / tpb;
   // the whole call in this kernel, x rows as the preparation reads them: the launch takes the tail on
-  const bool take_tail = fused.xp && !e32 && cpl <= 8 && x_stride == D && D % 64 == 0 && aligned16(x) &&
-                         aligned16(fused.xp) && (!fused.w_sg || aligned16(fused.w_sg));
+  const bool take_tail = tail_ok && fused.xp && !e32 && cpl <= 8;
   if (!take_tail) fused = RouterTail{};
   const uint32_t prep_cols = take_tail ? ((T + 3) / 4 + token_blocks - 1) / token_blocks : 0u;
 #define MF_PR(CPL, R)                                                                              \

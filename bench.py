@@ -642,6 +642,45 @@ def bench_family_routers(args, device) -> int:
     return 0
 
 
+def prefill_phase_trace(ctx, w, layer, device, tokens) -> int:
+    """Stage stamps of the work items (tile x row slice) of the routed gate/up matmul of the ragged prefill
+    layer: 0 start, 1 loads issued, 2 tables and bias terms done, 3 main loop done, 4 end (100 MHz clock)."""
+    import numpy as np
+    import torch
+    from mference_amd import operators as ops
+    gen = torch.Generator(device=device)
+    gen.manual_seed((ROOT_SEED + 0x100 * 2 + 0x7F) & 0x7FFFFFFFFFFFFFFF)
+    router = layer.router_w.clone()
+    router[:, -1] = (torch.randn((w["e"],), generator=gen, device=device) * 1.5).to(torch.bfloat16)
+    lw = ops.MoELayerWeights(router, layer.experts, layer.offsets, layer.shared, layer.w_sg)
+    moe = ops.MoE(ctx, w["d"], w["f"], w["e"], w["k"], bits=w["bits"], shared_f=w["fs"], shared_bits=w["shared_bits"],
+                  maple_rounding=bool(w.get("maple")),
+                  router_mode=ops.ROUTER_FULL_SOFTMAX if w["bits"] == 1 else ops.ROUTER_TOPK_SOFTMAX)
+    out = {"workload": w["name"], "unit": "us", "runs": []}
+    for t in tokens:
+        x = torch.randn((t, w["d"]), generator=gen, device=device).to(torch.bfloat16)
+        x[:, -1] = 1.0
+        y = torch.zeros_like(x)
+        ws = moe.encode_prefill_layer(lw, x, y, t)
+        stamps = torch.zeros((32768, 8), dtype=torch.int64, device=device)
+        moe.set_phase_trace(stamps)
+        for _ in range(3):
+            stamps.zero_()
+            moe.encode_prefill_layer(lw, x, y, t, workspace=ws)
+        torch.cuda.synchronize()
+        moe.set_phase_trace(None)
+        s = stamps.cpu().numpy().astype(np.float64)
+        s = s[s[:, 4] > 0]
+        d = np.diff(s[:, :5], axis=1).mean(axis=0) / 100.0
+        out["runs"].append({"tokens": t, "live_work_items": int(s.shape[0]),
+                            "loads_issued": round(float(d[0]), 2), "tables_and_bias_terms": round(float(d[1]), 2),
+                            "main_loop": round(float(d[2]), 2), "stores": round(float(d[3]), 2),
+                            "per_item": round(float((s[:, 4] - s[:, 0]).mean() / 100.0), 2),
+                            "span_first_start_to_last_end": round(float((s[:, 4].max() - s[:, 0].min()) / 100.0), 1)})
+    print(json.dumps(out))
+    return 0
+
+
 def phase_trace(ctx, w, stack, moes, device) -> int:
     """Stage stamps every workgroup of the fused decode launch writes (100 MHz wall clock): per stamp
     the median over the layers of the earliest / median / latest workgroup, in us from the start of the
@@ -731,6 +770,8 @@ def main() -> int:
         L = 1
     ctx = ops.MetalContext(0)
     stack = build_stack(ctx, w, L, device)
+    if args.prefill_only and args.phase_trace:
+        return prefill_phase_trace(ctx, w, stack[0], device, (args.tokens,) if args.tokens else (128, 512, 2048))
     if args.prefill_only:
         tokens = (args.tokens,) if args.tokens else (128, 512, 2048)
         res = {"prefill": measure_prefill(ctx, w, stack[0], device, tokens=tokens, steps=min(args.steps, 100),

@@ -144,6 +144,32 @@ def test_prefill_layer_matches_per_token_oracle(gpu, oracle, bits, d, f, e, k, f
     assert np.array_equal(y, y2)
 
 
+@pytest.mark.parametrize("bits,d,f,e,k,fs,t,mode", [
+    (4, 512, 256, 32, 8, 256, 1100, 0),    # 8800 routes, the shared expert rides along
+    (4, 1024, 128, 16, 8, 0, 1031, 0),     # few experts: long runs, an odd tile out at the end of every run
+    (2, 512, 256, 16, 6, 128, 1500, 0),    # 2-bit codes; the 4-bit shared expert is a launch of its own
+    (1, 512, 128, 32, 8, 0, 1030, 1),      # ternary rows, full-softmax router
+])
+def test_prefill_long_batches_against_the_per_token_oracle(gpu, oracle, bits, d, f, e, k, fs, t, mode):
+    """More than a thousand tokens on small layers (long runs per expert, many full tiles, an odd tile at
+    the end of every run), checked directly against the per-token checker: routing bit-exact, sampled rows
+    within the layer tolerance; and the rows do not depend on their neighbours (the first 300 tokens alone
+    give the same bits)."""
+    root = ROOT_SEED + 0xA400 + d + t
+    layer = oracle.synth_layer(root, d, f, e, k, bits=bits, fs=fs, router_mode=mode)
+    x = oracle.synth_x(root, t, d)
+    moe = make_moe(gpu, layer)
+    wts = to_device_layer(layer)
+    y, idx, w = _run_prefill(moe, wts, x, t, d, k)
+    rows = np.random.default_rng(t).choice(t, size=64, replace=False)
+    ref_y, ref_idx, ref_w = oracle.moe_layer(layer, x[rows])
+    assert np.array_equal(idx[rows], ref_idx)
+    assert np.array_equal(w[rows].view(np.uint32), ref_w.view(np.uint32))
+    assert_layer_close(oracle.bf16_to_float(y[rows]), oracle.bf16_to_float(ref_y), f"long batch bits={bits} t={t}")
+    y_short, _, _ = _run_prefill(moe, wts, x[:300], 300, d, k)
+    assert np.array_equal(y_short, y[:300])
+
+
 @pytest.mark.parametrize("bits,d,f,e,k,t", [(1, 512, 256, 32, 8, 150), (4, 256, 128, 32, 4, 70)])
 def test_prefill_layer_with_maple_rounding(gpu, oracle, bits, d, f, e, k, t):
     """MapleMoE's rounding points in the prefill call: the SwiGLU epilogue takes maple_swiglu,

@@ -343,6 +343,18 @@ void mf_moe_destroy(mf_moe* h) {
   delete h;
 }
 
+namespace {
+// bf16 router rows for t tokens: the batched kernels of the prefill router from 16 tokens on (the same
+// bits: they keep the summation order of the one-row kernel), else one wave per (token, row)
+hipError_t family_logits(hipStream_t s, const uint16_t* w, const uint16_t* x, uint32_t rows, uint32_t d,
+                         uint32_t t, uint32_t x_stride, float* logits) {
+  const bool al = mf::aligned16(w) && mf::aligned16(x) && x_stride % 8 == 0;
+  if (t >= 16 && al && ((d % 512 == 0 && rows % 32 == 0) || d <= 4096))
+    return mf::launch_prefill_router(s, w, x, rows, d, t, x_stride, logits);
+  return mf::launch_router_logits(s, w, x, rows, d, t, x_stride, logits, nullptr);
+}
+}  // namespace
+
 mf_status mf_moe_router(mf_moe* h, mf_stream stream, const uint16_t* router_w, const uint16_t* x,
                         uint32_t t, uint32_t x_stride, uint32_t* out_idx, float* out_w,
                         float* out_logits) {
@@ -356,8 +368,7 @@ mf_status mf_moe_router(mf_moe* h, mf_stream stream, const uint16_t* router_w, c
   for (uint32_t t0 = 0; t0 < t;) {
     const uint32_t tc = out_logits ? t - t0 : std::min<uint32_t>(t - t0, MF_MAX_TOKENS);
     float* lg = out_logits ? out_logits + static_cast<size_t>(t0) * e : h->ws.logits;
-    MF_HIP(h->ctx, mf::launch_router_logits(s, router_w, x + static_cast<size_t>(t0) * x_stride, e,
-                                            h->cfg.d, tc, x_stride, lg, nullptr));
+    MF_HIP(h->ctx, family_logits(s, router_w, x + static_cast<size_t>(t0) * x_stride, e, h->cfg.d, tc, x_stride, lg));
     MF_HIP(h->ctx, mf::launch_topk(s, lg, e, h->cfg.top_k, tc, h->cfg.router_mode,
                                    out_idx + static_cast<size_t>(t0) * h->cfg.top_k,
                                    out_w + static_cast<size_t>(t0) * h->cfg.top_k));
@@ -376,15 +387,6 @@ mf_status family_args_ok(const mf_ctx* ctx, const void* w, const uint16_t* x, ui
   if (top_k == 0 || top_k > MF_MAX_TOPK) return MF_ERR_TOPK;
   if (!mf::aligned2(x) || (reinterpret_cast<uintptr_t>(logits) & 3u)) return MF_ERR_INVALID_ARGUMENT;
   return MF_OK;
-}
-// bf16 router rows for t tokens: the batched kernels of the prefill router from 16 tokens on (the same
-// bits: they keep the summation order of the one-row kernel), else one wave per (token, row)
-hipError_t family_logits(hipStream_t s, const uint16_t* w, const uint16_t* x, uint32_t rows, uint32_t d,
-                         uint32_t t, uint32_t x_stride, float* logits) {
-  const bool al = mf::aligned16(w) && mf::aligned16(x) && x_stride % 8 == 0;
-  if (t >= 16 && al && ((d % 512 == 0 && rows % 32 == 0) || d <= 4096))
-    return mf::launch_prefill_router(s, w, x, rows, d, t, x_stride, logits);
-  return mf::launch_router_logits(s, w, x, rows, d, t, x_stride, logits, nullptr);
 }
 }  // namespace
 

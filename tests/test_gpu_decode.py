@@ -195,7 +195,10 @@ def test_gemv_misaligned_pointers(gpu, oracle):
 
 
 @pytest.mark.parametrize("e,d,k,t", [(256, 2048, 8, 1), (16, 128, 8, 3), (64, 2048, 8, 5),
-                                     (256, 4096, 6, 2), (100, 192, 4, 9), (8, 64, 8, 1)])
+                                     (256, 4096, 6, 2), (100, 192, 4, 9), (8, 64, 8, 1),
+                                     # the block form (PrefillRouter.encodeGemma4Block): from 16 tokens on the
+                                     # batched kernels take the logits -- register-tiled, then matrix-core
+                                     (100, 192, 4, 33), (64, 512, 8, 40), (64, 1024, 8, 300)])
 @pytest.mark.parametrize("mode", [0, 1])
 def test_router_bit_exact(gpu, oracle, e, d, k, t, mode):
     if mode == 1 and e % 32:

@@ -1,0 +1,78 @@
+"""Seeded sweeps over layer shapes nobody picked by hand: the decode call (fused launch and chain of
+launches) and the prefill call against the per-token CPU oracle.  Shapes are drawn from what
+mf_moe_create accepts (widths in multiples of the group size, up to 8 routes per token), so the sweep
+crosses the boundaries between the specialised kernels and their fall-backs: widths that are and are not
+multiples of 128 or 512, expert counts that are no multiple of 32, tiles that are empty, partial and full."""
+import numpy as np
+import pytest
+import torch
+
+from mference_amd import operators as ops
+from helpers import ROOT_SEED, assert_layer_close, make_moe, to_device_layer
+
+pytestmark = pytest.mark.gpu
+
+
+def _draw(seed, prefill):
+    rng = np.random.default_rng(seed)
+    bits = int(rng.choice([4, 4, 2, 1]))
+    d = int(rng.choice([64, 128, 192, 256, 384, 512, 1024]))
+    f = int(rng.choice([64, 128, 192, 256, 512]))
+    e = int(rng.choice([8, 12, 16, 24, 32, 64, 100]))
+    k = int(rng.choice([1, 2, 4, 6, 8]))
+    k = min(k, e)
+    fs = int(rng.choice([0, 0, 64, 128, f]))
+    if bits != 4 and rng.integers(2):
+        fs = 0
+    mode = int(rng.integers(2)) if e % 32 == 0 else 0
+    limit = float(rng.choice([0.0, 0.0, 7.0]))
+    t = int(rng.integers(9, 420)) if prefill else int(rng.integers(1, 9))
+    return bits, d, f, e, k, fs, t, mode, limit
+
+
+@pytest.mark.parametrize("seed", range(40))
+def test_decode_sweep(gpu, oracle, seed):
+    bits, d, f, e, k, fs, t, mode, limit = _draw(0xD0C0 + seed, prefill=False)
+    root = ROOT_SEED + 0xB000 + seed
+    layer = oracle.synth_layer(root, d, f, e, k, bits=bits, fs=fs, router_mode=mode, swiglu_limit=limit)
+    x = oracle.synth_x(root, t, d)
+    ref_y, ref_idx, ref_w = oracle.moe_layer(layer, x)
+    moe = make_moe(gpu, layer)
+    wts = to_device_layer(layer)
+    xd = ops.bf16_tensor(x)
+    what = f"seed {seed}: bits={bits} d={d} f={f} e={e} k={k} fs={fs} t={t} mode={mode} limit={limit}"
+    results = {}
+    for fused in (True, False):
+        moe.set_fused(fused)
+        y = torch.zeros((t, d), dtype=torch.bfloat16, device="cuda")
+        idx = torch.zeros((t, k), dtype=torch.int32, device="cuda")
+        w = torch.zeros((t, k), dtype=torch.float32, device="cuda")
+        for _ in range(2):
+            y.zero_()
+            moe.encode_decode_layer(wts, xd, y, t=t, out_indices=idx, out_weights=w)
+            moe.status()
+        assert np.array_equal(idx.cpu().numpy().astype(np.uint32), ref_idx), what
+        assert np.array_equal(w.cpu().numpy().view(np.uint32), ref_w.view(np.uint32)), what
+        assert_layer_close(oracle.bf16_to_float(ops.bf16_bits(y)), oracle.bf16_to_float(ref_y), what)
+        results[fused] = ops.bf16_bits(y)
+    assert np.array_equal(results[True], results[False]), what
+
+
+@pytest.mark.parametrize("seed", range(28))
+def test_prefill_sweep(gpu, oracle, seed):
+    bits, d, f, e, k, fs, t, mode, limit = _draw(0xF111 + seed, prefill=True)
+    root = ROOT_SEED + 0xB800 + seed
+    layer = oracle.synth_layer(root, d, f, e, k, bits=bits, fs=fs, router_mode=mode, swiglu_limit=limit)
+    x = oracle.synth_x(root, t, d)
+    ref_y, ref_idx, ref_w = oracle.moe_layer(layer, x)
+    moe = make_moe(gpu, layer)
+    wts = to_device_layer(layer)
+    y = torch.zeros((t, d), dtype=torch.bfloat16, device="cuda")
+    idx = torch.zeros((t, k), dtype=torch.int32, device="cuda")
+    w = torch.zeros((t, k), dtype=torch.float32, device="cuda")
+    moe.encode_prefill_layer(wts, ops.bf16_tensor(x), y, t, out_indices=idx, out_weights=w)
+    torch.cuda.synchronize()
+    what = f"seed {seed}: bits={bits} d={d} f={f} e={e} k={k} fs={fs} t={t} mode={mode} limit={limit}"
+    assert np.array_equal(idx.cpu().numpy().astype(np.uint32), ref_idx), what
+    assert np.array_equal(w.cpu().numpy().view(np.uint32), ref_w.view(np.uint32)), what
+    assert_layer_close(oracle.bf16_to_float(ops.bf16_bits(y)), oracle.bf16_to_float(ref_y), what)

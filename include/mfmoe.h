@@ -251,8 +251,7 @@ void mf_moe_destroy(mf_moe* h);
  * out_idx uint32 [t, top_k]; out_w fp32 [t, top_k]; out_logits fp32
  * [t, num_experts] or NULL.  Any t >= 1.  From 16 tokens on the logits of a call are
  * computed by the batched kernels of the prefill layer (the same bits); without
- * out_logits the call works through the handle's own buffer MF_MAX_TOKENS rows at a
- * time, so a caller with many tokens should pass out_logits. */
+ * out_logits the call works through the handle's own buffer 256 rows at a time. */
 mf_status mf_moe_router(mf_moe* h, mf_stream stream, const uint16_t* router_w,
                         const uint16_t* x, uint32_t t, uint32_t x_stride, uint32_t* out_idx,
                         float* out_w, float* out_logits);

@@ -12,6 +12,8 @@
 namespace {
 
 constexpr int kAbiVersion = 2;  // 2: mf_moe_config.gate_group_size
+// rows of router logits a handle holds for mf_moe_router calls that bring no logits buffer
+constexpr uint32_t kRouterRows = 256;
 
 mf_status fail_hip(mf_ctx* ctx, hipError_t e, const char* what) {
   if (ctx) snprintf(ctx->hip_error, sizeof ctx->hip_error, "%s: %s", what, hipGetErrorString(e));
@@ -290,7 +292,7 @@ mf_status mf_moe_create(mf_ctx* ctx, const mf_moe_config* cfg, mf_moe** out) {
     pos = round_up(pos + bytes, 256);
     return at;
   };
-  const size_t o_logits = take(T * cfg->num_experts * sizeof(float));
+  const size_t o_logits = take(kRouterRows * cfg->num_experts * sizeof(float));
   const size_t o_idx = take(T * cfg->top_k * sizeof(uint32_t));
   const size_t o_w = take(T * cfg->top_k * sizeof(float));
   const size_t o_acts = take(T * cfg->top_k * cfg->f * sizeof(uint16_t));
@@ -363,10 +365,9 @@ mf_status mf_moe_router(mf_moe* h, mf_stream stream, const uint16_t* router_w, c
   if (!mf::aligned2(router_w) || !mf::aligned2(x)) return MF_ERR_INVALID_ARGUMENT;
   auto s = static_cast<hipStream_t>(stream);
   const uint32_t e = h->cfg.num_experts;
-  // logits go to the caller's buffer when given, else through the handle's
-  // workspace in chunks of MF_MAX_TOKENS rows
+  // logits go to the caller's buffer when given, else through the handle's (kRouterRows rows at a time)
   for (uint32_t t0 = 0; t0 < t;) {
-    const uint32_t tc = out_logits ? t - t0 : std::min<uint32_t>(t - t0, MF_MAX_TOKENS);
+    const uint32_t tc = out_logits ? t - t0 : std::min<uint32_t>(t - t0, kRouterRows);
     float* lg = out_logits ? out_logits + static_cast<size_t>(t0) * e : h->ws.logits;
     MF_HIP(h->ctx, family_logits(s, router_w, x + static_cast<size_t>(t0) * x_stride, e, h->cfg.d, tc, x_stride, lg));
     MF_HIP(h->ctx, mf::launch_topk(s, lg, e, h->cfg.top_k, tc, h->cfg.router_mode,

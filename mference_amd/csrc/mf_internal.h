@@ -16,7 +16,7 @@ struct mf_ctx {
 // Per-operator device workspace (the routerLogits buffer and argument table the
 // reference's MoE class owns, MoE.swift:136-150).
 struct mf_moe_workspace {
-  float* logits;        // [MF_MAX_TOKENS, num_experts]
+  float* logits;        // [256, num_experts]: MF_MAX_TOKENS rows for the decode calls, 256 for mf_moe_router
   uint32_t* idx;        // [MF_MAX_TOKENS, top_k]
   float* w;             // [MF_MAX_TOKENS, top_k]
   uint16_t* acts;       // [MF_MAX_TOKENS, top_k, f]

@@ -218,6 +218,11 @@ def test_router_bit_exact(gpu, oracle, e, d, k, t, mode):
         ri, rw = oracle.topk_softmax(ref_lg, k, full_softmax=bool(mode))
         assert np.array_equal(idx[i].cpu().numpy().astype(np.uint32), ri)
         assert np.array_equal(w[i].cpu().numpy().view(np.uint32), rw.view(np.uint32))
+    # without a logits buffer the call goes through the handle's own, 256 rows at a time: the same routes
+    idx2, w2 = torch.zeros_like(idx), torch.zeros_like(w)
+    moe.encode_router(ops.bf16_tensor(wr), ops.bf16_tensor(x), idx2, w2, t=t)
+    _sync()
+    assert torch.equal(idx2, idx) and torch.equal(w2, w)
 
 
 def _tie_logits(oracle, count, trial, rng):

@@ -690,6 +690,16 @@ __global__ __launch_bounds__(kFusedThreads) void fused_decode_kernel(const Fused
       have_next = request_round0(tok + 1 < T ? tok + 1 : tok, pre_next);
       issue_fence();
     }
+    // When a lane's share of a row is one 16-byte step, its slice of the slot's activations is the same in
+    // every round: it is built once per token (with several rounds of rows that is a third of the round's
+    // vector work).
+    // (2-bit codes only: their slices are the longest to build and their layers the ones with several rounds;
+    // the 4-bit and ternary launches measured slower with the extra path compiled in)
+    const bool one_step = BITS == kBits2 && lpr * Fmt<BITS>::kElemsPer16B >= F && rounds > 1 && unit_local < ub;
+    XSlice<BITS> xs_slot{};
+    if (one_step && sub * Fmt<BITS>::kElemsPer16B < F)
+      xs_slot = load_xslice<BITS, kXAligned>(reinterpret_cast<const uint16_t*>(s_acts) + slot * F +
+                                             sub * Fmt<BITS>::kElemsPer16B);
     for (uint32_t round = 0; round < rounds; ++round) {
       const uint32_t unit = (round * G + wg) * ub + unit_local;
       const bool active = unit_local < ub && unit < rg_per_tok;
@@ -700,11 +710,25 @@ __global__ __launch_bounds__(kFusedThreads) void fused_decode_kernel(const Fused
         float part = 0.0f;
         if (row < D && expert < E) {
           const uint8_t* blob = a.expert_base + static_cast<size_t>(expert) * a.expert_stride;
-          part = row_partial<BITS>(blob + a.off.down_w + row * rb,
-                                   reinterpret_cast<const uint16_t*>(blob + a.off.down_s) + row * ng,
-                                   reinterpret_cast<const uint16_t*>(blob + a.off.down_b) + row * ng,
-                                   reinterpret_cast<const uint16_t*>(s_acts) + slot * F, F, sub, lpr,
-                                   have_pre && round == 0, pre);
+          const uint8_t* wrow = blob + a.off.down_w + row * rb;
+          const uint16_t* srow = reinterpret_cast<const uint16_t*>(blob + a.off.down_s) + row * ng;
+          const uint16_t* brow = reinterpret_cast<const uint16_t*>(blob + a.off.down_b) + row * ng;
+          if (one_step) {
+            const uint32_t e0 = sub * Fmt<BITS>::kElemsPer16B;
+            if (e0 < F) {  // the one step of row_partial over the slice at hand
+              uint4 codes = pre.codes;
+              float sc = pre.s, bi = pre.b;
+              if (!(have_pre && round == 0)) {
+                codes = load_codes16<true>(wrow + static_cast<size_t>(e0) * Store<BITS>::kBits / 8);
+                load_scale_bias<BITS>(srow, brow, e0, sc, bi);
+              }
+              part = __builtin_fmaf(sc, codes_dot<BITS>(codes, xs_slot), 0.0f);
+              part = __builtin_fmaf(bi, xs_slot.sum, part);
+            }
+          } else {
+            part = row_partial<BITS>(wrow, srow, brow, reinterpret_cast<const uint16_t*>(s_acts) + slot * F, F, sub,
+                                     lpr, have_pre && round == 0, pre);
+          }
         }
         const float v = group_sum(part, static_cast<int>(lpr));
         // moe.metal:1262; maple_moe.metal:258 (the down output is a bf16 number first)

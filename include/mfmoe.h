@@ -37,6 +37,10 @@ extern "C" {
 #define MF_MAX_TOKENS 8  /* kMultiXMaxT, dequant_int4.metal:356 */
 #define MF_MAX_TOPK 8    /* kMaxStreamedExperts, moe.metal:5 */
 #define MF_MAX_EXPERTS 512
+/* rows (tokens) one batched call takes: row * top_k and the byte offsets derived from it stay inside
+ * 32 bits; a larger t is refused (MF_ERR_INVALID_ARGUMENT, MF_ERR_QUERY_COUNT where the reference
+ * names the query count) */
+#define MF_MAX_ROWS (1u << 20)
 
 typedef enum {
   MF_OK = 0,

@@ -180,7 +180,7 @@ mf_status mf_shared_expert(mf_ctx* ctx, mf_stream stream, const uint16_t* x, mf_
   if (!bits_ok(bits)) return MF_ERR_UNSUPPORTED_BITS;
   if (d == 0 || f == 0 || d % MF_GROUP_SIZE != 0 || f % MF_GROUP_SIZE != 0)
     return MF_ERR_DIMENSION_MISMATCH;
-  if (t == 0 || t > (1u << 20)) return MF_ERR_INVALID_ARGUMENT;
+  if (t == 0 || t > MF_MAX_ROWS) return MF_ERR_INVALID_ARGUMENT;
   if (!qtensor_ok(gate, bits) || !qtensor_ok(up, bits) || !qtensor_ok(down, bits))
     return MF_ERR_INVALID_ARGUMENT;
   if (!mf::aligned2(x) || !mf::aligned2(y) || !mf::aligned2(scratch_act))
@@ -215,7 +215,7 @@ mf_status mf_qmm(mf_ctx* ctx, mf_stream stream, mf_qtensor w, mf_bits bits, cons
   // the conditions under which MPPPrefillInt4QMM.encode returns .unavailable (MPPPrefillInt4QMM.swift:43-55)
   if (!ctx || !x || !y) return MF_ERR_INVALID_ARGUMENT;
   if (!bits_ok(bits)) return MF_ERR_UNSUPPORTED_BITS;
-  if (m == 0 || n == 0 || k == 0 || k % MF_GROUP_SIZE != 0 || m > (1u << 20)) return MF_ERR_DIMENSION_MISMATCH;
+  if (m == 0 || n == 0 || k == 0 || k % MF_GROUP_SIZE != 0 || m > MF_MAX_ROWS) return MF_ERR_DIMENSION_MISMATCH;
   if (!qtensor_ok(w, bits) || !mf::aligned2(x) || !mf::aligned2(y)) return MF_ERR_INVALID_ARGUMENT;
   auto s = static_cast<hipStream_t>(stream);
   if (workspace && mf::aligned16(workspace) && mf::dense_qmm_takes(w, bits, x, y, m, n, k) &&
@@ -361,7 +361,7 @@ mf_status mf_moe_router(mf_moe* h, mf_stream stream, const uint16_t* router_w, c
                         uint32_t t, uint32_t x_stride, uint32_t* out_idx, float* out_w,
                         float* out_logits) {
   if (!h || !router_w || !x || !out_idx || !out_w) return MF_ERR_INVALID_ARGUMENT;
-  if (t == 0 || x_stride < h->cfg.d) return MF_ERR_INVALID_ARGUMENT;
+  if (t == 0 || t > MF_MAX_ROWS || x_stride < h->cfg.d) return MF_ERR_INVALID_ARGUMENT;
   if (!mf::aligned2(router_w) || !mf::aligned2(x)) return MF_ERR_INVALID_ARGUMENT;
   auto s = static_cast<hipStream_t>(stream);
   const uint32_t e = h->cfg.num_experts;
@@ -383,7 +383,7 @@ namespace {
 mf_status family_args_ok(const mf_ctx* ctx, const void* w, const uint16_t* x, uint32_t t, uint32_t x_stride,
                          uint32_t rows, uint32_t d, uint32_t top_k, const float* logits) {
   if (!ctx || !w || !x || !logits) return MF_ERR_INVALID_ARGUMENT;
-  if (t == 0 || d == 0 || d % 8 != 0 || x_stride < d) return MF_ERR_INVALID_ARGUMENT;
+  if (t == 0 || t > MF_MAX_ROWS || d == 0 || d % 8 != 0 || x_stride < d) return MF_ERR_INVALID_ARGUMENT;
   if (rows == 0 || rows > MF_MAX_EXPERTS) return MF_ERR_NUM_EXPERTS;
   if (top_k == 0 || top_k > MF_MAX_TOPK) return MF_ERR_TOPK;
   if (!mf::aligned2(x) || (reinterpret_cast<uintptr_t>(logits) & 3u)) return MF_ERR_INVALID_ARGUMENT;
@@ -462,7 +462,7 @@ mf_status mf_moe_phase1(mf_moe* h, mf_stream stream, const void* expert_base,
                         const uint32_t* idx, const uint16_t* x, uint32_t t, uint32_t x_stride,
                         uint16_t* acts) {
   if (!h || !expert_base || !offsets || !idx || !x || !acts) return MF_ERR_INVALID_ARGUMENT;
-  if (t == 0 || x_stride < h->cfg.d) return MF_ERR_INVALID_ARGUMENT;
+  if (t == 0 || t > MF_MAX_ROWS || x_stride < h->cfg.d) return MF_ERR_INVALID_ARGUMENT;
   if (!offsets_ok(*offsets, h->cfg.bits) || !mf::aligned2(expert_base) || (expert_stride & 1) ||
       !mf::aligned2(x) || !mf::aligned2(acts))
     return MF_ERR_INVALID_ARGUMENT;
@@ -478,7 +478,7 @@ mf_status mf_moe_phase1_subset(mf_moe* h, mf_stream stream, const void* expert_b
   if (active_count == 0) return MF_OK;  // MoE.swift:269
   if (!active_slots || (reinterpret_cast<uintptr_t>(active_slots) & 3u)) return MF_ERR_INVALID_ARGUMENT;
   if (!h || !expert_base || !offsets || !idx || !x || !acts) return MF_ERR_INVALID_ARGUMENT;
-  if (t == 0 || x_stride < h->cfg.d) return MF_ERR_INVALID_ARGUMENT;
+  if (t == 0 || t > MF_MAX_ROWS || x_stride < h->cfg.d) return MF_ERR_INVALID_ARGUMENT;
   if (!offsets_ok(*offsets, h->cfg.bits) || !mf::aligned2(expert_base) || (expert_stride & 1) ||
       !mf::aligned2(x) || !mf::aligned2(acts))
     return MF_ERR_INVALID_ARGUMENT;
@@ -503,7 +503,7 @@ mf_status mf_moe_phase1_slots(mf_moe* h, mf_stream stream, const void* slab, con
                               const uint32_t* all_hit, const mf_expert_offsets* offsets, const uint16_t* x,
                               uint32_t t, uint32_t x_stride, uint16_t* acts) {
   if (!h || !slot_offsets || !offsets || !x || !acts) return MF_ERR_INVALID_ARGUMENT;
-  if (t == 0 || x_stride < h->cfg.d) return MF_ERR_INVALID_ARGUMENT;
+  if (t == 0 || t > MF_MAX_ROWS || x_stride < h->cfg.d) return MF_ERR_INVALID_ARGUMENT;
   if (!offsets_ok(*offsets, h->cfg.bits) || !mf::aligned2(slab) || !mf::aligned2(x) || !mf::aligned2(acts) ||
       (reinterpret_cast<uintptr_t>(slot_offsets) & 7u))
     return MF_ERR_INVALID_ARGUMENT;
@@ -516,7 +516,7 @@ mf_status mf_moe_phase2_slots(mf_moe* h, mf_stream stream, const void* slab, con
                               const uint32_t* all_hit, const mf_expert_offsets* offsets, const float* w,
                               const uint16_t* acts, const uint16_t* residual, uint32_t t, uint16_t* y) {
   if (!h || !slot_offsets || !offsets || !w || !acts || !y) return MF_ERR_INVALID_ARGUMENT;
-  if (t == 0) return MF_ERR_INVALID_ARGUMENT;
+  if (t == 0 || t > MF_MAX_ROWS) return MF_ERR_INVALID_ARGUMENT;
   if (!offsets_ok(*offsets, h->cfg.bits) || !mf::aligned2(slab) || !mf::aligned2(acts) || !mf::aligned2(y) ||
       (residual && !mf::aligned2(residual)) || (reinterpret_cast<uintptr_t>(slot_offsets) & 7u))
     return MF_ERR_INVALID_ARGUMENT;
@@ -530,7 +530,7 @@ mf_status mf_moe_phase2(mf_moe* h, mf_stream stream, const void* expert_base,
                         const uint32_t* idx, const float* w, const uint16_t* acts,
                         const uint16_t* residual, uint32_t t, uint16_t* y) {
   if (!h || !expert_base || !offsets || !idx || !w || !acts || !y) return MF_ERR_INVALID_ARGUMENT;
-  if (t == 0) return MF_ERR_INVALID_ARGUMENT;
+  if (t == 0 || t > MF_MAX_ROWS) return MF_ERR_INVALID_ARGUMENT;
   if (!offsets_ok(*offsets, h->cfg.bits) || !mf::aligned2(expert_base) || (expert_stride & 1) ||
       !mf::aligned2(acts) || !mf::aligned2(y) || (residual && !mf::aligned2(residual)))
     return MF_ERR_INVALID_ARGUMENT;
@@ -637,7 +637,7 @@ mf_status mf_moe_group(mf_moe* h, mf_stream stream, const uint32_t* idx, const f
     return MF_OK;
   }
   if (!idx || !w || !sorted_pairs) return MF_ERR_INVALID_ARGUMENT;
-  if (t > (1u << 20)) return MF_ERR_QUERY_COUNT;  // t * top_k stays far inside 32 bits, as in the prefill call
+  if (t > MF_MAX_ROWS) return MF_ERR_QUERY_COUNT;  // t * top_k stays far inside 32 bits, as in the prefill call
   uint32_t* starts = h->ws.group_tmp + 512;
   uint32_t* status = h->ws.group_tmp + 3 * 512;
   MF_HIP(h->ctx, mf::launch_group(s, idx, w, t, h->cfg.top_k, h->cfg.num_experts, expert_counts,
@@ -664,7 +664,7 @@ mf_status mf_moe_prefill_layer(mf_moe* h, mf_stream stream, const mf_moe_layer_w
                                const uint16_t* x, uint32_t t, uint16_t* y, void* workspace,
                                size_t workspace_bytes, uint32_t* out_idx, float* out_w) {
   if (!h || !wts || !x || !y) return MF_ERR_INVALID_ARGUMENT;
-  if (t == 0 || t > (1u << 20)) return MF_ERR_INVALID_ARGUMENT;
+  if (t == 0 || t > MF_MAX_ROWS) return MF_ERR_INVALID_ARGUMENT;
   const mf_moe_config& c = h->cfg;
   if (!mf::prefill_supported(c)) {
     // 2-bit / ternary experts, or widths the matmul tiles do not divide: the same rows through
@@ -704,7 +704,7 @@ mf_status mf_moe_ragged_qmm(mf_moe* h, mf_stream stream, const void* expert_base
                             size_t workspace_bytes) {
   if (!h || !offsets || !x || !sorted_pairs || !expert_counts || !route_partials || !expert_base)
     return MF_ERR_INVALID_ARGUMENT;
-  if (t == 0 || t > (1u << 20)) return MF_ERR_QUERY_COUNT;
+  if (t == 0 || t > MF_MAX_ROWS) return MF_ERR_QUERY_COUNT;
   const mf_moe_config& c = h->cfg;
   if (!mf::prefill_supported(c)) return MF_ERR_DIMENSION_MISMATCH;
   if (!workspace) return MF_ERR_INVALID_ARGUMENT;
@@ -722,7 +722,7 @@ mf_status mf_moe_ragged_qmm(mf_moe* h, mf_stream stream, const void* expert_base
 mf_status mf_moe_unpermute(mf_moe* h, mf_stream stream, const float* route_partials, const float* route_weights,
                            const uint32_t* idx, const uint16_t* residual, uint32_t t, uint16_t* y) {
   if (!h || !route_partials || !route_weights || !y) return MF_ERR_INVALID_ARGUMENT;
-  if (t == 0 || t > (1u << 20)) return MF_ERR_QUERY_COUNT;
+  if (t == 0 || t > MF_MAX_ROWS) return MF_ERR_QUERY_COUNT;
   const mf_moe_config& c = h->cfg;
   if (c.d % 4) return MF_ERR_DIMENSION_MISMATCH;
   if (!mf::aligned16(route_partials) || reinterpret_cast<uintptr_t>(y) % 8 ||

@@ -218,6 +218,8 @@ hipError_t launch_phase1(hipStream_t s, const mf_moe_config& cfg, const void* ba
   const uint32_t all_pairs = t * cfg.top_k;
   const uint32_t pairs = subset ? n_subset : all_pairs;
   if (!pairs) return hipSuccess;
+  // one wave per group of rows of a route: the count has to fit the 32-bit indexing of the kernel
+  if (static_cast<uint64_t>(pairs) * cfg.f >= (1ull << 31)) return hipErrorInvalidValue;
   const bool al = blob_aligned(base, slot_offsets ? 0 : stride, off) && aligned16(x) && (x_stride % 8 == 0);
   const auto* b = static_cast<const uint8_t*>(base);
 #define MF_P1(BITS, AL)                                                                          \
@@ -267,6 +269,7 @@ hipError_t launch_phase2(hipStream_t s, const mf_moe_config& cfg, const void* ba
                          const uint16_t* acts, const uint16_t* residual, uint32_t t, uint16_t* y,
                          const uint64_t* slot_offsets, const uint32_t* all_hit) {
   if (!t) return hipSuccess;
+  if (static_cast<uint64_t>(t) * cfg.d >= (1ull << 31)) return hipErrorInvalidValue;  // 32-bit wave and row indices
   // (with a slot table the caller promises blobs on 16-byte boundaries; `stride` is not used)
   const bool al = blob_aligned(base, slot_offsets ? 0 : stride, off) && aligned16(acts);
   const auto* b = static_cast<const uint8_t*>(base);

@@ -262,6 +262,32 @@ def test_family_router_argument_errors(gpu):
     assert e6.value.status == -1
 
 
+def test_row_counts_beyond_the_limit_are_refused(gpu):
+    """MF_MAX_ROWS (2^20) bounds t in every batched call: a larger count is an argument error and nothing
+    is launched (the buffers here are far too small for such a call)."""
+    too_many = (1 << 20) + 1
+    fam = ops.FamilyRouters(gpu)
+    z16 = torch.zeros(4096, dtype=torch.bfloat16, device="cuda")
+    zf = torch.zeros(4096, dtype=torch.float32, device="cuda")
+    zi = torch.zeros(64, dtype=torch.int32, device="cuda")
+    with pytest.raises(ops.MfError) as err:
+        fam.encode_router_top_k(z16, z16, zf, zi, zf, 16, 64, 1.0, zf, t=too_many)
+    assert err.value.status == -1
+    moe = ops.MoE(gpu, 64, 64, 16, 2, bits=4)
+    offsets, blob_bytes, stride = ops.expert_blob_layout(64, 64, 4)
+    experts = torch.zeros((16, stride), dtype=torch.uint8, device="cuda")
+    calls = [
+        lambda: moe.encode_router(z16, z16, zi, zf, t=too_many),
+        lambda: moe.encode_routed_phase1(experts, offsets, zi, z16, z16, t=too_many),
+        lambda: moe.encode_routed_phase2_reduce(experts, offsets, zi, zf, z16, None, z16, t=too_many),
+    ]
+    for call in calls:
+        with pytest.raises(ops.MfError) as err:
+            call()
+        assert err.value.status == -1
+    torch.cuda.synchronize()
+
+
 def test_sqrtsoftplus_routing_feeds_the_two_phase_layer(gpu, oracle):
     """a 2-bit layer routed by the DeepSeek-V4 selector: router -> phase 1 -> phase 2 through the ABI
     against the checker's composition of the same parts"""

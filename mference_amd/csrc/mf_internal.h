@@ -29,7 +29,8 @@ struct mf_moe_workspace {
   uint32_t* t_acts;              // [MF_MAX_TOKENS, top_k, f]
   uint32_t* epoch;               // [512] one launch counter per workgroup
   uint32_t* status;              // non-zero once a bounded wait gave up
-  uint32_t* group_tmp;           // grouping scratch: [512, 1024) starts, [1536] status word, [2048, ...) per-chunk counts
+  uint32_t* group_tmp;           // grouping scratch: [512, 1024) starts, [1536] status word, [2048, ...) per-chunk counts,
+                                 // flags, and the per-chunk route words and count bytes of the prefill layer call
 };
 
 struct mf_moe {

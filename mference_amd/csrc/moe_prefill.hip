@@ -301,10 +301,12 @@ __global__ __launch_bounds__(256) void group_count_kernel(const uint32_t* __rest
 __device__ __forceinline__ void group_layout(uint32_t c, uint32_t E, uint32_t* __restrict__ counts,
                                              uint32_t* __restrict__ offsets, uint32_t* __restrict__ starts,
                                              Tile* __restrict__ tiles, uint32_t tile_slots,
-                                             uint32_t* __restrict__ n_tiles, uint32_t* s_cnt, uint32_t* s_tile) {
+                                             uint32_t* __restrict__ n_tiles, uint32_t* s_cnt, uint32_t* s_tile,
+                                             bool publish = true) {
   const uint32_t e = threadIdx.x;
   const bool act = e < MF_MAX_EXPERTS;
-  if (e < E) counts[e] = c;
+  if (!publish) tiles = nullptr, n_tiles = nullptr;  // the scans only (s_cnt, s_tile): another workgroup writes
+  if (publish && e < E) counts[e] = c;
   // inclusive scans of the counts and of the tile counts over the MF_MAX_EXPERTS entries: inside a wave
   // by shuffles, the eight wave totals through the last slots of the two arrays' neighbours
   __shared__ uint32_t s_wave_cnt[MF_MAX_EXPERTS / 64], s_wave_tile[MF_MAX_EXPERTS / 64];
@@ -339,7 +341,7 @@ __device__ __forceinline__ void group_layout(uint32_t c, uint32_t E, uint32_t* _
     for (uint32_t i = e; i < tile_slots; i += blockDim.x) tiles[i] = Tile{0, 0, 0, 0};
     __syncthreads();
   }
-  if (e < E) {
+  if (publish && e < E) {
     const uint32_t start = s_cnt[e] - c;
     starts[e] = start;
     offsets[e] = c ? start : 0xFFFFFFFFu;
@@ -611,6 +613,133 @@ __global__ __launch_bounds__(1024) void group_one_kernel(const uint32_t* __restr
     r.rank = p - t * K;
     r.weight_bits = __float_as_uint(w[p]);
     sorted[pos] = r;
+  }
+}
+
+// The layer call selects the routes itself, so selection and grouping share launches: two instead of the
+// selector's one plus the grouping's one or three.  A top-k names an expert at most once per token, so the
+// routes of expert e inside a chunk of up to 64 consecutive tokens are a 64-bit word (bit i: token i of
+// the chunk routes to e) and "how many routes of e come before mine" is a popcount.
+//
+// First launch: a workgroup selects the routes of one chunk (a wave a token at a time, the selectors of
+// topk_kernel), stores them, and leaves the chunk's word per expert and, in a byte matrix [expert][chunk],
+// its number of routes per expert.
+constexpr uint32_t kSelectWaves = 16;
+constexpr uint32_t kChunkTokensMax = 64;
+static_assert(kChunkTokensMax * MF_MAX_TOPK <= MF_MAX_EXPERTS, "a chunk's routes are placed by one workgroup in one step");
+static_assert(kGroupChunks % 16 == 0, "an expert's row of per-chunk counts is read 16 bytes at a time");
+
+__global__ __launch_bounds__(kSelectWaves * 64) void topk_chunk_kernel(const float* __restrict__ logits, uint32_t T,
+                                                                       uint32_t E, uint32_t K, int mode,
+                                                                       uint32_t chunk_tokens,
+                                                                       uint32_t* __restrict__ idx,
+                                                                       float* __restrict__ w,
+                                                                       unsigned long long* __restrict__ chunk_bits,
+                                                                       uint8_t* __restrict__ chunk_cnt,
+                                                                       uint32_t* __restrict__ chunk_bad) {
+  __shared__ uint32_t s_bits[2][MF_MAX_EXPERTS];
+  __shared__ float s_p[kSelectWaves][MF_MAX_EXPERTS];  // the full softmax's probabilities, a row per wave
+  __shared__ uint32_t s_i[kSelectWaves][MF_MAX_TOPK];
+  __shared__ float s_wt[kSelectWaves][MF_MAX_TOPK];
+  const uint32_t lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
+  for (uint32_t e = threadIdx.x; e < E; e += blockDim.x) s_bits[0][e] = s_bits[1][e] = 0u;
+  __syncthreads();
+  const uint32_t t0 = blockIdx.x * chunk_tokens, t1 = min(T, t0 + chunk_tokens);
+  bool bad = false;
+  for (uint32_t t = t0 + wv; t < t1; t += kSelectWaves) {
+    const float* lg = logits + static_cast<size_t>(t) * E;
+    if (mode == 0) topk_select_fast(lg, E, K, s_i[wv], s_wt[wv], lane);
+    else topk_full_softmax_fast(lg, s_p[wv], E, K, s_i[wv], s_wt[wv], lane);
+    if (lane < K) {
+      const uint32_t e = s_i[wv][lane];
+      idx[static_cast<size_t>(t) * K + lane] = e;
+      w[static_cast<size_t>(t) * K + lane] = s_wt[wv][lane];
+      const uint32_t i = t - t0;
+      if (e < E) atomicOr(&s_bits[i >> 5][e], 1u << (i & 31u));
+      else bad = true;  // the full softmax's "routes nowhere"
+    }
+  }
+  // one flag per chunk, always written: nothing has to be cleared before the launch
+  const int any_bad = __syncthreads_or(bad ? 1 : 0);
+  if (threadIdx.x == 0) chunk_bad[blockIdx.x] = any_bad ? 1u : 0u;
+  for (uint32_t e = threadIdx.x; e < E; e += blockDim.x) {
+    const uint32_t lo = s_bits[0][e], hi = s_bits[1][e];
+    chunk_bits[static_cast<size_t>(blockIdx.x) * E + e] =
+        static_cast<unsigned long long>(lo) | (static_cast<unsigned long long>(hi) << 32);
+    chunk_cnt[static_cast<size_t>(e) * kGroupChunks + blockIdx.x] = static_cast<uint8_t>(__popc(lo) + __popc(hi));
+  }
+}
+
+// the bytes of word j (chunks 4j .. 4j+3) that belong to chunks below `limit`
+__device__ __forceinline__ uint32_t chunk_bytes_below(uint32_t limit, uint32_t j) {
+  if (limit >= 4 * j + 4) return 0xFFFFFFFFu;
+  if (limit <= 4 * j) return 0u;
+  return (1u << (8 * (limit - 4 * j))) - 1u;
+}
+
+// Second launch: every workgroup adds up its experts' rows of per-chunk counts (an expert's total, and its
+// routes in the chunks before the workgroup's own), repeats the layout scans for itself, and places the
+// routes of its chunk; the first workgroup also publishes counts, offsets, starts, the tile list and the
+// status word.
+__global__ __launch_bounds__(MF_MAX_EXPERTS) void group_place_kernel(const uint32_t* __restrict__ idx,
+                                                                    const float* __restrict__ w, uint32_t T,
+                                                                    uint32_t K, uint32_t E, uint32_t chunk_tokens,
+                                                                    uint32_t n_chunks,
+                                                                    const unsigned long long* __restrict__ chunk_bits,
+                                                                    const uint8_t* __restrict__ chunk_cnt,
+                                                                    const uint32_t* __restrict__ chunk_bad,
+                                                                    uint32_t* __restrict__ counts,
+                                                                    uint32_t* __restrict__ offsets,
+                                                                    uint32_t* __restrict__ starts,
+                                                                    mf_pair* __restrict__ sorted,
+                                                                    Tile* __restrict__ tiles, uint32_t tile_slots,
+                                                                    uint32_t* __restrict__ n_tiles,
+                                                                    uint32_t* __restrict__ status) {
+  __shared__ uint32_t s_cnt[MF_MAX_EXPERTS], s_tile[MF_MAX_EXPERTS], s_base[MF_MAX_EXPERTS];
+  __shared__ unsigned long long s_mine[MF_MAX_EXPERTS];
+  const uint32_t e = threadIdx.x, me = blockIdx.x;
+  const bool first = me == 0;
+  // this workgroup's routes, requested before anything is waited for
+  const uint32_t t0 = me * chunk_tokens, t1 = min(T, t0 + chunk_tokens);
+  const uint32_t n = (t1 - t0) * K;  // <= kChunkTokensMax * MF_MAX_TOPK <= blockDim
+  const size_t p = static_cast<size_t>(t0) * K + threadIdx.x;
+  uint32_t ex = 0xFFFFFFFFu, wbits = 0u;
+  if (threadIdx.x < n) {
+    ex = idx[p];
+    wbits = __float_as_uint(w[p]);
+  }
+  uint32_t c = 0, before = 0;
+  if (e < E) {
+    const uint4* row = reinterpret_cast<const uint4*>(chunk_cnt + static_cast<size_t>(e) * kGroupChunks);
+    uint4 v[kGroupChunks / 16];
+#pragma unroll
+    for (uint32_t j = 0; j < kGroupChunks / 16; ++j)
+      v[j] = 16 * j < n_chunks ? row[j] : make_uint4(0, 0, 0, 0);
+    s_mine[e] = chunk_bits[static_cast<size_t>(me) * E + e];
+#pragma unroll
+    for (uint32_t j = 0; j < kGroupChunks / 16; ++j) {
+      const uint32_t q[4] = {v[j].x, v[j].y, v[j].z, v[j].w};
+#pragma unroll
+      for (uint32_t u = 0; u < 4; ++u) {
+        const uint32_t word = 4 * j + u;
+        c = __builtin_amdgcn_sad_u8(q[u] & chunk_bytes_below(n_chunks, word), 0u, c);
+        before = __builtin_amdgcn_sad_u8(q[u] & chunk_bytes_below(me, word), 0u, before);
+      }
+    }
+  }
+  const int any_bad = __syncthreads_or(e < n_chunks && chunk_bad[e] ? 1 : 0);  // n_chunks <= blockDim
+  if (first && e == 0) *status = any_bad ? 2u : 0u;
+  group_layout(c, E, counts, offsets, starts, tiles, tile_slots, n_tiles, s_cnt, s_tile, first);
+  if (e < E) s_base[e] = s_cnt[e] - c + before;  // s_cnt is the inclusive scan of the counts
+  __syncthreads();
+  if (ex < E) {
+    const uint32_t i = threadIdx.x / K;
+    mf_pair r;
+    r.token = t0 + i;
+    r.expert = ex;
+    r.rank = threadIdx.x - i * K;
+    r.weight_bits = wbits;
+    sorted[s_base[ex] + __popcll(s_mine[ex] & ((1ull << i) - 1ull))] = r;
   }
 }
 
@@ -1636,7 +1765,36 @@ hipError_t launch_group(hipStream_t s, const uint32_t* idx, const float* w, uint
   return hipGetLastError();
 }
 
-size_t group_scratch_words() { return 2048 + static_cast<size_t>(kGroupChunks) * MF_MAX_EXPERTS + kGroupChunks; }
+// words of the handle's grouping scratch: 2048 of small tables, the per-chunk counts and flags of the
+// three-launch grouping, and behind them the per-chunk 64-bit words and the [expert][chunk] count bytes of
+// the layer call's own grouping
+constexpr size_t kGroupBitsAt = 2048 + static_cast<size_t>(kGroupChunks) * MF_MAX_EXPERTS + kGroupChunks;  // even
+constexpr size_t kGroupCntAt = kGroupBitsAt + 2 * static_cast<size_t>(kGroupChunks) * MF_MAX_EXPERTS;
+size_t group_scratch_words() { return kGroupCntAt + static_cast<size_t>(kGroupChunks) * MF_MAX_EXPERTS / 4; }
+
+// Selection and grouping of the layer call's own routes in two launches (topk_chunk_kernel,
+// group_place_kernel); false when the batch is too long for chunks of 64 tokens.
+bool topk_group_takes(uint32_t t) { return t != 0 && t <= kGroupChunks * kChunkTokensMax; }
+
+hipError_t launch_topk_group(hipStream_t s, const float* logits, uint32_t t, uint32_t K, uint32_t E, int mode,
+                             uint32_t* idx, float* w, uint32_t* counts, uint32_t* offsets, uint32_t* starts,
+                             mf_pair* sorted, void* tiles, uint32_t tile_slots, uint32_t* n_tiles, uint32_t* status,
+                             uint32_t* group_tmp) {
+  // a token per wave while that gives at most 128 chunks, then longer chunks, then more of them
+  uint32_t chunk_tokens = ((t + 127) / 128 + kSelectWaves - 1) / kSelectWaves * kSelectWaves;
+  chunk_tokens = std::min(std::max(chunk_tokens, kSelectWaves), kChunkTokensMax);
+  const uint32_t n_chunks = (t + chunk_tokens - 1) / chunk_tokens;
+  auto* bits = reinterpret_cast<unsigned long long*>(group_tmp + kGroupBitsAt);
+  auto* cnt = reinterpret_cast<uint8_t*>(group_tmp + kGroupCntAt);
+  uint32_t* bad = group_tmp + 2048 + static_cast<size_t>(kGroupChunks) * MF_MAX_EXPERTS;
+  topk_chunk_kernel<<<dim3(n_chunks), dim3(kSelectWaves * 64), 0, s>>>(logits, t, E, K, mode, chunk_tokens, idx, w, bits,
+                                                                       cnt, bad);
+  group_place_kernel<<<dim3(n_chunks), dim3(MF_MAX_EXPERTS), 0, s>>>(idx, w, t, K, E, chunk_tokens, n_chunks, bits, cnt,
+                                                                    bad, counts, offsets, starts, sorted,
+                                                                    static_cast<Tile*>(tiles), tile_slots, n_tiles,
+                                                                    status);
+  return hipGetLastError();
+}
 
 size_t qmm_lds_bytes(uint32_t kdim, int nproj) {
   const uint32_t ng = kdim / kGroup;
@@ -2005,7 +2163,7 @@ hipError_t launch_prefill_layer(hipStream_t s, const mf_moe& h, const mf_moe_lay
 #define MF_TRY(call) do { e = (call); if (e != hipSuccess) return e; } while (0)
   const size_t pairs = static_cast<size_t>(t) * c.top_k;
   const uint32_t max_tiles = prefill_tile_slots(c, t);
-  bool x_prepared = false;
+  bool x_prepared = false, fused_group = false;
   if (ragged) {
     // the caller's grouping: its per-expert counts are a one-chunk histogram for the scan that lays
     // out the tile list (the runs start at 0 in expert order, as mf_moe_group writes them)
@@ -2031,10 +2189,16 @@ hipError_t launch_prefill_layer(hipStream_t s, const mf_moe& h, const mf_moe_lay
       tail.gate = ws.gate;
       MF_TRY(launch_prefill_router(s, w.router_w, x, c.num_experts, c.d, t, c.d, ws.logits, &tail));
       x_prepared = tail.xp != nullptr;
-      MF_TRY(launch_topk(s, ws.logits, c.num_experts, c.top_k, t, c.router_mode, ws.idx, ws.w));
+      fused_group = topk_group_takes(t) && pairs > kGroupOnePairs;
+      if (fused_group)
+        MF_TRY(launch_topk_group(s, ws.logits, t, c.top_k, c.num_experts, c.router_mode, ws.idx, ws.w, ws.counts,
+                                 ws.offsets, ws.starts, ws.sorted, ws.tiles, max_tiles, ws.n_tiles, ws.status,
+                                 h.ws.group_tmp));
+      else MF_TRY(launch_topk(s, ws.logits, c.num_experts, c.top_k, t, c.router_mode, ws.idx, ws.w));
     }
-    MF_TRY(launch_group(s, ws.idx, ws.w, t, c.top_k, c.num_experts, ws.counts, ws.offsets, ws.starts,
-                        ws.sorted, ws.tiles, max_tiles, ws.n_tiles, ws.status, h.ws.group_tmp + 2048));
+    if (!fused_group)
+      MF_TRY(launch_group(s, ws.idx, ws.w, t, c.top_k, c.num_experts, ws.counts, ws.offsets, ws.starts,
+                          ws.sorted, ws.tiles, max_tiles, ws.n_tiles, ws.status, h.ws.group_tmp + 2048));
   }
 
   const bool want_gate = c.shared_f && w.w_sg;

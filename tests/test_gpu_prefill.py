@@ -149,12 +149,16 @@ def test_prefill_layer_matches_per_token_oracle(gpu, oracle, bits, d, f, e, k, f
     (4, 1024, 128, 16, 8, 0, 1031, 0),     # few experts: long runs, an odd tile out at the end of every run
     (2, 512, 256, 16, 6, 128, 1500, 0),    # 2-bit codes; the 4-bit shared expert is a launch of its own
     (1, 512, 128, 32, 8, 0, 1030, 1),      # ternary rows, full-softmax router
+    (4, 128, 128, 100, 3, 0, 3000, 0),     # 94 chunks of 32 tokens (two per wave of the selecting launch), 3 routes each
+    (4, 128, 128, 24, 1, 128, 8500, 0),    # 133 chunks of 64 tokens, one route per token
 ])
 def test_prefill_long_batches_against_the_per_token_oracle(gpu, oracle, bits, d, f, e, k, fs, t, mode):
     """More than a thousand tokens on small layers (long runs per expert, many full tiles, an odd tile at
     the end of every run), checked directly against the per-token checker: routing bit-exact, sampled rows
     within the layer tolerance; and the rows do not depend on their neighbours (the first 300 tokens alone
-    give the same bits)."""
+    give the same bits).  Beyond 8192 routes the layer call selects and groups its routes in two launches
+    of its own (chunks of up to 64 tokens, an expert's routes of a chunk as a 64-bit word); the 300-token
+    call groups them in one workgroup: the same rows from both."""
     root = ROOT_SEED + 0xA400 + d + t
     layer = oracle.synth_layer(root, d, f, e, k, bits=bits, fs=fs, router_mode=mode)
     x = oracle.synth_x(root, t, d)
@@ -393,29 +397,36 @@ def test_prefill_16k_tokens_repeat_the_2048_token_rows(gpu):
     assert torch.equal(yb.view(torch.int16).view(reps, t, d), y.view(torch.int16).expand(reps, t, d))
 
 
-def test_non_finite_token_takes_sentinel_routes(gpu, oracle):
+@pytest.mark.parametrize("d,f,t", [(512, 256, 100), (128, 128, 1100)])
+def test_non_finite_token_takes_sentinel_routes(gpu, oracle, d, f, t):
     """full-softmax router: a token whose logits are not finite gets indices = num_experts and
     weights 0 (maple_moe.metal:73-79); its routes contribute nothing, in the decode launch and in
-    the prefill call, and the other tokens of the batch are untouched"""
-    d, f, e, k, t = 512, 256, 32, 8, 100
-    root = ROOT_SEED + 0xAB00
+    the prefill call (short batch: grouped by one workgroup; long batch: selected and grouped chunk by
+    chunk), and the other tokens of the batch are untouched"""
+    e, k = 32, 8
+    root = ROOT_SEED + 0xAB00 + t
     layer = oracle.synth_layer(root, d, f, e, k, bits=1, router_mode=1)
     x = oracle.synth_x(root, t, d)
-    bad = [3, 64, 99]
+    bad = [3, 64, t - 1]
     x[bad, 7] = 0x7FC0   # bf16 NaN
-    ref_y, ref_idx, ref_w = oracle.moe_layer(layer, x)
-    assert (ref_idx[bad] == e).all() and (ref_w[bad] == 0).all() and (ref_y[bad] == 0).all()
+    rows = sorted(set(bad) | set(range(0, 8)) | set(range(60, 70)) | set(range(t - 10, t)))
+    ref_y, ref_idx, ref_w = oracle.moe_layer(layer, x[rows])
+    at = {r: i for i, r in enumerate(rows)}
+    ref_bad = [at[r] for r in bad]
+    assert (ref_idx[ref_bad] == e).all() and (ref_w[ref_bad] == 0).all() and (ref_y[ref_bad] == 0).all()
     moe = make_moe(gpu, layer)
     wts = to_device_layer(layer)
     y, idx, w = _run_prefill(moe, wts, x, t, d, k)
-    assert np.array_equal(idx, ref_idx)
-    assert np.array_equal(w.view(np.uint32), ref_w.view(np.uint32))
+    assert np.array_equal(idx[rows], ref_idx)
+    assert np.array_equal(w[rows].view(np.uint32), ref_w.view(np.uint32))
     assert (y[bad] == 0).all()
-    good = [i for i in range(t) if i not in bad]
-    assert_layer_close(oracle.bf16_to_float(y[good]), oracle.bf16_to_float(ref_y[good]), "tokens next to a NaN token")
+    good = [r for r in rows if r not in bad]
+    assert_layer_close(oracle.bf16_to_float(y[good]), oracle.bf16_to_float(ref_y[[at[r] for r in good]]),
+                       "tokens next to a NaN token")
+    ref_idx = {r: ref_idx[at[r]] for r in (2, 3, 4)}
     yd = torch.zeros((3, d), dtype=torch.bfloat16, device="cuda")
     idd = torch.zeros((3, k), dtype=torch.int32, device="cuda")
     moe.encode_decode_layer(wts, ops.bf16_tensor(x[[2, 3, 4]]), yd, t=3, out_indices=idd)
     moe.status()
-    assert np.array_equal(idd.cpu().numpy().astype(np.uint32), ref_idx[[2, 3, 4]])
+    assert np.array_equal(idd.cpu().numpy().astype(np.uint32), np.stack([ref_idx[r] for r in (2, 3, 4)]))
     assert (ops.bf16_bits(yd)[1] == 0).all()

@@ -79,6 +79,31 @@ def test_prefill_sweep(gpu, oracle, seed):
     assert_layer_close(oracle.bf16_to_float(ops.bf16_bits(y)), oracle.bf16_to_float(ref_y), what)
 
 
+@pytest.mark.parametrize("seed", range(8))
+def test_prefill_long_sweep(gpu, oracle, seed):
+    """the same draw with 2200 to 4400 tokens (beyond 8192 routes the layer call selects and groups its
+    routes chunk by chunk): routing bit-exact on every row, 48 sampled rows against the per-token checker"""
+    bits, d, f, e, k, fs, _, mode, limit = _draw(0xF1A0 + seed, prefill=True)
+    d, f = min(d, 512), min(f, 256)   # the checker walks every sampled row's experts in numpy
+    t = int(np.random.default_rng(0xF1A1 + seed).integers(2200, 4400))
+    root = ROOT_SEED + 0xBC00 + seed
+    layer = oracle.synth_layer(root, d, f, e, k, bits=bits, fs=min(fs, f), router_mode=mode, swiglu_limit=limit)
+    x = oracle.synth_x(root, t, d)
+    moe = make_moe(gpu, layer)
+    wts = to_device_layer(layer)
+    y = torch.zeros((t, d), dtype=torch.bfloat16, device="cuda")
+    idx = torch.zeros((t, k), dtype=torch.int32, device="cuda")
+    w = torch.zeros((t, k), dtype=torch.float32, device="cuda")
+    moe.encode_prefill_layer(wts, ops.bf16_tensor(x), y, t, out_indices=idx, out_weights=w)
+    torch.cuda.synchronize()
+    what = f"seed {seed}: bits={bits} d={d} f={f} e={e} k={k} fs={min(fs, f)} t={t} mode={mode} limit={limit}"
+    rows = np.sort(np.random.default_rng(seed).choice(t, size=48, replace=False))
+    ref_y, ref_idx, ref_w = oracle.moe_layer(layer, x[rows])
+    assert np.array_equal(idx.cpu().numpy().astype(np.uint32)[rows], ref_idx), what
+    assert np.array_equal(w.cpu().numpy().view(np.uint32)[rows], ref_w.view(np.uint32)), what
+    assert_layer_close(oracle.bf16_to_float(ops.bf16_bits(y)[rows]), oracle.bf16_to_float(ref_y), what)
+
+
 @pytest.mark.parametrize("seed", range(20))
 def test_qmm_sweep(gpu, oracle, seed):
     """the dense projection of many rows (mf_qmm) over drawn (bits, m, n, k): one, two and three windows of

@@ -622,12 +622,11 @@ __global__ __launch_bounds__(1024) void group_one_kernel(const uint32_t* __restr
 // the chunk routes to e) and "how many routes of e come before mine" is a popcount.
 //
 // First launch: a workgroup selects the routes of one chunk (a wave a token at a time, the selectors of
-// topk_kernel), stores them, and leaves the chunk's word per expert and, in a byte matrix [expert][chunk],
-// its number of routes per expert.
+// topk_kernel), stores them, and leaves the chunk's word per expert and, as a row of bytes, its number of
+// routes per expert.
 constexpr uint32_t kSelectWaves = 16;
 constexpr uint32_t kChunkTokensMax = 64;
 static_assert(kChunkTokensMax * MF_MAX_TOPK <= MF_MAX_EXPERTS, "a chunk's routes are placed by one workgroup in one step");
-static_assert(kGroupChunks % 16 == 0, "an expert's row of per-chunk counts is read 16 bytes at a time");
 
 __global__ __launch_bounds__(kSelectWaves * 64) void topk_chunk_kernel(const float* __restrict__ logits, uint32_t T,
                                                                        uint32_t E, uint32_t K, int mode,
@@ -666,21 +665,13 @@ __global__ __launch_bounds__(kSelectWaves * 64) void topk_chunk_kernel(const flo
     const uint32_t lo = s_bits[0][e], hi = s_bits[1][e];
     chunk_bits[static_cast<size_t>(blockIdx.x) * E + e] =
         static_cast<unsigned long long>(lo) | (static_cast<unsigned long long>(hi) << 32);
-    chunk_cnt[static_cast<size_t>(e) * kGroupChunks + blockIdx.x] = static_cast<uint8_t>(__popc(lo) + __popc(hi));
+    chunk_cnt[static_cast<size_t>(blockIdx.x) * E + e] = static_cast<uint8_t>(__popc(lo) + __popc(hi));
   }
 }
 
-// the bytes of word j (chunks 4j .. 4j+3) that belong to chunks below `limit`
-__device__ __forceinline__ uint32_t chunk_bytes_below(uint32_t limit, uint32_t j) {
-  if (limit >= 4 * j + 4) return 0xFFFFFFFFu;
-  if (limit <= 4 * j) return 0u;
-  return (1u << (8 * (limit - 4 * j))) - 1u;
-}
-
-// Second launch: every workgroup adds up its experts' rows of per-chunk counts (an expert's total, and its
-// routes in the chunks before the workgroup's own), repeats the layout scans for itself, and places the
-// routes of its chunk; the first workgroup also publishes counts, offsets, starts, the tile list and the
-// status word.
+// Second launch: every workgroup adds up the chunks' counts per expert (an expert's total, and its routes
+// in the chunks before the workgroup's own), repeats the layout scans for itself, and places the routes of
+// its chunk; the first workgroup also publishes counts, offsets, starts, the tile list and the status word.
 __global__ __launch_bounds__(MF_MAX_EXPERTS) void group_place_kernel(const uint32_t* __restrict__ idx,
                                                                     const float* __restrict__ w, uint32_t T,
                                                                     uint32_t K, uint32_t E, uint32_t chunk_tokens,
@@ -710,21 +701,22 @@ __global__ __launch_bounds__(MF_MAX_EXPERTS) void group_place_kernel(const uint3
   }
   uint32_t c = 0, before = 0;
   if (e < E) {
-    const uint4* row = reinterpret_cast<const uint4*>(chunk_cnt + static_cast<size_t>(e) * kGroupChunks);
-    uint4 v[kGroupChunks / 16];
-#pragma unroll
-    for (uint32_t j = 0; j < kGroupChunks / 16; ++j)
-      v[j] = 16 * j < n_chunks ? row[j] : make_uint4(0, 0, 0, 0);
     s_mine[e] = chunk_bits[static_cast<size_t>(me) * E + e];
+    uint32_t k = 0;
+    for (; k + 32 <= n_chunks; k += 32) {  // 32 independent byte loads in flight
+      uint32_t v[32];
 #pragma unroll
-    for (uint32_t j = 0; j < kGroupChunks / 16; ++j) {
-      const uint32_t q[4] = {v[j].x, v[j].y, v[j].z, v[j].w};
+      for (int u = 0; u < 32; ++u) v[u] = chunk_cnt[static_cast<size_t>(k + u) * E + e];
 #pragma unroll
-      for (uint32_t u = 0; u < 4; ++u) {
-        const uint32_t word = 4 * j + u;
-        c = __builtin_amdgcn_sad_u8(q[u] & chunk_bytes_below(n_chunks, word), 0u, c);
-        before = __builtin_amdgcn_sad_u8(q[u] & chunk_bytes_below(me, word), 0u, before);
+      for (int u = 0; u < 32; ++u) {
+        c += v[u];
+        before += k + u < me ? v[u] : 0u;
       }
+    }
+    for (; k < n_chunks; ++k) {
+      const uint32_t v = chunk_cnt[static_cast<size_t>(k) * E + e];
+      c += v;
+      before += k < me ? v : 0u;
     }
   }
   const int any_bad = __syncthreads_or(e < n_chunks && chunk_bad[e] ? 1 : 0);  // n_chunks <= blockDim
@@ -1766,7 +1758,7 @@ hipError_t launch_group(hipStream_t s, const uint32_t* idx, const float* w, uint
 }
 
 // words of the handle's grouping scratch: 2048 of small tables, the per-chunk counts and flags of the
-// three-launch grouping, and behind them the per-chunk 64-bit words and the [expert][chunk] count bytes of
+// three-launch grouping, and behind them the per-chunk 64-bit words and the [chunk][expert] count bytes of
 // the layer call's own grouping
 constexpr size_t kGroupBitsAt = 2048 + static_cast<size_t>(kGroupChunks) * MF_MAX_EXPERTS + kGroupChunks;  // even
 constexpr size_t kGroupCntAt = kGroupBitsAt + 2 * static_cast<size_t>(kGroupChunks) * MF_MAX_EXPERTS;

@@ -147,16 +147,26 @@ __device__ __forceinline__ void router_rows(const uint16_t* __restrict__ W, cons
 // Needs D % 512 == 0 (all 64 chains the same length) and E % 32 == 0.
 typedef __attribute__((ext_vector_type(32))) float f32x32_t;
 
-__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) void prefill_router_mfma_kernel(const uint16_t* __restrict__ W,
+// N_I = D / 512 as a compile-time constant unrolls the whole walk (a wave's 8 chain pairs x N_I runs): the
+// operand offsets, the ring slots and the levels of the binary counter are then literals, the operand ring
+// needs no register moves and a chain's first instruction takes the constant 0 as its accumulator -- 3.9
+// vector instructions per matrix instruction where the loop for any width (N_I = 0) issues 10.6, and the
+// matrix instructions of a SIMD wait for its vector instructions (T=2048: 38.6 -> 34.1 us, T=512: 18.5 ->
+// 14.8 us).  (The unrolled form needs 123 registers; eight waves of 8 chains per block, four to a SIMD,
+// measured no faster than these four of 16 chains: 34.7 / 15.8 us.)
+template <int N_I>
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2)))
+void prefill_router_mfma_kernel(const uint16_t* __restrict__ W,
                                                                   const uint16_t* __restrict__ x,
                                                                   uint32_t E, uint32_t D, uint32_t T,
                                                                   uint32_t x_stride,
                                                                   float* __restrict__ logits, uint32_t ld,
                                                                   const RouterTail tail) {
-  __shared__ float s_part[3][16 * 64];
+  constexpr int WAVES = 4, kPairs = 32 / WAVES;  // waves of a workgroup, chain pairs of one wave
+  __shared__ float s_part[WAVES - 1][16 * 64];
   const uint32_t lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
   if (tail.xp && blockIdx.y >= tail.router_cols) {  // an x-preparation workgroup (rows behind the expert blocks)
-    const uint32_t row = ((blockIdx.y - tail.router_cols) * gridDim.x + blockIdx.x) * 4 + wv;
+    const uint32_t row = ((blockIdx.y - tail.router_cols) * gridDim.x + blockIdx.x) * WAVES + wv;
     if (row < T) prep_x_row(x + static_cast<size_t>(row) * x_stride, tail.xp, tail.sums, tail.w_sg, tail.gate, row, D, lane);
     return;
   }
@@ -165,12 +175,69 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
   // eighth of the token rows (and all of the small router matrix)
   const uint32_t t0 = blockIdx.x * 32, e0 = blockIdx.y * 32;
   const uint32_t n_i = D / 512;
-  const uint16_t* xrow = x + static_cast<size_t>(min(t0 + m, T - 1)) * x_stride + 8 * (16 * wv + b);
-  const uint16_t* wrow = W + static_cast<size_t>(e0 + m) * D + 8 * (16 * wv + b);
+  const uint16_t* xrow = x + static_cast<size_t>(min(t0 + m, T - 1)) * x_stride + 8 * (2 * kPairs * wv + b);
+  const uint16_t* wrow = W + static_cast<size_t>(e0 + m) * D + 8 * (2 * kPairs * wv + b);
 
   float lev0[16], lev1[16], lev2[16], total[16];
 #pragma unroll
   for (int r = 0; r < 16; ++r) lev0[r] = lev1[r] = lev2[r] = total[r] = 0.0f;
+  if constexpr (N_I > 0) {
+    // step q = pp * N_I + i, operands 4 steps ahead in a ring of 8 slots
+    constexpr int kSteps = kPairs * N_I, kAhead = 4;
+    uint4 rx[2 * kAhead], rw[2 * kAhead];
+#pragma unroll
+    for (int q = 0; q < kAhead && q < kSteps; ++q) {
+      rx[q] = *reinterpret_cast<const uint4*>(xrow + 16 * (q / N_I) + 512 * (q % N_I));
+      rw[q] = *reinterpret_cast<const uint4*>(wrow + 16 * (q / N_I) + 512 * (q % N_I));
+    }
+    f32x32_t acc;
+#pragma unroll
+    for (int q = 0; q < kSteps; ++q) {
+      if (q + kAhead < kSteps) {
+        const int qa = q + kAhead;
+        rx[qa % (2 * kAhead)] = *reinterpret_cast<const uint4*>(xrow + 16 * (qa / N_I) + 512 * (qa % N_I));
+        rw[qa % (2 * kAhead)] = *reinterpret_cast<const uint4*>(wrow + 16 * (qa / N_I) + 512 * (qa % N_I));
+      }
+      const uint4 cxq = rx[q % (2 * kAhead)], cwq = rw[q % (2 * kAhead)];
+      const uint32_t xw[4] = {cxq.x, cxq.y, cxq.z, cxq.w}, ww[4] = {cwq.x, cwq.y, cwq.z, cwq.w};
+      float xa[8], wa[8];
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        xa[2 * j] = bf16_lo(xw[j]); xa[2 * j + 1] = bf16_hi(xw[j]);
+        wa[2 * j] = bf16_lo(ww[j]); wa[2 * j + 1] = bf16_hi(ww[j]);
+      }
+      // all 16 operands in registers of their own before the step's first matrix instruction (see below)
+      asm volatile("" : "+v"(xa[0]), "+v"(xa[1]), "+v"(xa[2]), "+v"(xa[3]), "+v"(xa[4]), "+v"(xa[5]), "+v"(xa[6]), "+v"(xa[7]),
+                        "+v"(wa[0]), "+v"(wa[1]), "+v"(wa[2]), "+v"(wa[3]), "+v"(wa[4]), "+v"(wa[5]), "+v"(wa[6]), "+v"(wa[7]));
+      if (q % N_I == 0) {  // a chain's first product lands on 0
+        f32x32_t zero;
+#pragma unroll
+        for (int r = 0; r < 32; ++r) zero[r] = 0.0f;
+        acc = __builtin_amdgcn_mfma_f32_32x32x1f32(xa[0], wa[0], zero, 0, 0, 0);
+      } else {
+        acc = __builtin_amdgcn_mfma_f32_32x32x1f32(xa[0], wa[0], acc, 0, 0, 0);
+      }
+#pragma unroll
+      for (int j = 1; j < 8; ++j) acc = __builtin_amdgcn_mfma_f32_32x32x1f32(xa[j], wa[j], acc, 0, 0, 0);
+      if (q % N_I == N_I - 1) {  // the pair of chains is complete: stride-1 level, then the binary counter
+        constexpr int kLevels = kPairs == 8 ? 3 : 2;
+        const int pp = q / N_I;
+        float carry[16];
+#pragma unroll
+        for (int r = 0; r < 16; ++r) carry[r] = acc[r] + acc[16 + r];
+        int level = 0;
+#pragma unroll
+        for (; level < kLevels && ((pp >> level) & 1); ++level) {
+          float* lv = level == 0 ? lev0 : level == 1 ? lev1 : lev2;
+#pragma unroll
+          for (int r = 0; r < 16; ++r) carry[r] = lv[r] + carry[r];
+        }
+        float* dst = level == kLevels ? total : level == 0 ? lev0 : level == 1 ? lev1 : lev2;
+#pragma unroll
+        for (int r = 0; r < 16; ++r) dst[r] = carry[r];
+      }
+    }
+  } else {
   // step q = pp * n_i + i: chain pair pp (chains 16 wv + 2 pp + b), K run i; operands run 4 steps ahead
   const uint32_t steps = 8 * n_i;
   uint4 cx[4], cw[4], nx[4], nw[4];
@@ -246,18 +313,25 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
       cw[u] = nw[u];
     }
   }
+  }  // the loop for any width
   if (wv > 0) {
 #pragma unroll
     for (int r = 0; r < 16; ++r) s_part[wv - 1][r * 64 + lane] = total[r];
   }
   __syncthreads();
-  if (wv == 0) {
+  if (wv == 0) {  // the last levels of the tree: neighbouring waves first
 #pragma unroll
     for (int r = 0; r < 16; ++r) {
-      const float s01 = total[r] + s_part[0][r * 64 + lane];
-      const float s23 = s_part[1][r * 64 + lane] + s_part[2][r * 64 + lane];
+      float v[WAVES];
+      v[0] = total[r];
+#pragma unroll
+      for (int u = 1; u < WAVES; ++u) v[u] = s_part[u - 1][r * 64 + lane];
+#pragma unroll
+      for (int stride = 1; stride < WAVES; stride *= 2)
+#pragma unroll
+        for (int u = 0; u < WAVES; u += 2 * stride) v[u] = v[u] + v[u + stride];
       const uint32_t t = t0 + 8 * (r / 4) + 4 * b + (r % 4);
-      if (t < T) logits[static_cast<size_t>(t) * ld + e0 + m] = s01 + s23;
+      if (t < T) logits[static_cast<size_t>(t) * ld + e0 + m] = v[0];
     }
   }
 }
@@ -1680,12 +1754,15 @@ hipError_t launch_prefill_router(hipStream_t s, const uint16_t* W, const uint16_
     if (tail_ok) {  // the x preparation rides in this launch: workgroup rows behind the expert blocks
       mt = fused;
       mt.router_cols = e32 / 32;
-      prep_rows = ((T + 3) / 4 + (T + 31) / 32 - 1) / ((T + 31) / 32);
       fused.xp = nullptr;  // done here: the register-tiled launch for left-over rows does not repeat it
       tail->xp = mt.xp;
     }
-    prefill_router_mfma_kernel<<<dim3((T + 31) / 32, e32 / 32 + prep_rows), dim3(256), 0, s>>>(W, x, e32, D, T, x_stride,
-                                                                                              logits, E, mt);
+    if (tail_ok) prep_rows = ((T + 3) / 4 + (T + 31) / 32 - 1) / ((T + 31) / 32);
+    const dim3 grid((T + 31) / 32, e32 / 32 + prep_rows);
+    if (D == 1024) prefill_router_mfma_kernel<2><<<grid, dim3(256), 0, s>>>(W, x, e32, D, T, x_stride, logits, E, mt);
+    else if (D == 2048) prefill_router_mfma_kernel<4><<<grid, dim3(256), 0, s>>>(W, x, e32, D, T, x_stride, logits, E, mt);
+    else if (D == 4096) prefill_router_mfma_kernel<8><<<grid, dim3(256), 0, s>>>(W, x, e32, D, T, x_stride, logits, E, mt);
+    else prefill_router_mfma_kernel<0><<<grid, dim3(256), 0, s>>>(W, x, e32, D, T, x_stride, logits, E, mt);
     if (e32 == E) return hipGetLastError();
   }
   const uint32_t rest = E - e32;

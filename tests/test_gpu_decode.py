@@ -507,9 +507,11 @@ def test_phase1_subsets_write_the_bits_of_the_full_call(gpu, oracle, bits, t):
     assert bool((lone[0, 0] == 7.0).all()) and bool((lone[0, 2:] == 7.0).all())
 
 
-def test_qwen_shape_specialised_launch(gpu, oracle):
+@pytest.mark.parametrize("t", [1, 2, 5, 8])
+def test_qwen_shape_specialised_launch(gpu, oracle, t):
     """the full Qwen3.6-shaped layer (D 2048, F 512, E 256, K 8, shared 512) takes the
-    shape-specialised fused kernel; weights drawn and quantized on the GPU as bench.py does"""
+    shape-specialised fused kernels (one for a single token row, one for any other count); weights drawn
+    and quantized on the GPU as bench.py does"""
     import bench
     w = dict(bench.QWEN)
     stack = bench.build_stack(gpu, w, 1, torch.device("cuda", 0))
@@ -519,14 +521,14 @@ def test_qwen_shape_specialised_launch(gpu, oracle):
     gen.manual_seed(1234)
     outs = {}
     for rep in range(3):
-        x = torch.randn((1, w["d"]), generator=gen, device="cuda").to(torch.bfloat16)
+        x = torch.randn((t, w["d"]), generator=gen, device="cuda").to(torch.bfloat16)
         ref_y, ref_idx, ref_w = oracle.moe_layer(host, ops.bf16_bits(x))
         for fused in (True, False):
             moe.set_fused(fused)
             y = torch.zeros_like(x)
-            idx = torch.zeros((1, w["k"]), dtype=torch.int32, device="cuda")
-            rw = torch.zeros((1, w["k"]), dtype=torch.float32, device="cuda")
-            moe.encode_decode_layer(stack[0], x, y, out_indices=idx, out_weights=rw)
+            idx = torch.zeros((t, w["k"]), dtype=torch.int32, device="cuda")
+            rw = torch.zeros((t, w["k"]), dtype=torch.float32, device="cuda")
+            moe.encode_decode_layer(stack[0], x, y, t=t, out_indices=idx, out_weights=rw)
             moe.status()
             assert np.array_equal(idx.cpu().numpy().astype(np.uint32), ref_idx)
             assert np.array_equal(rw.cpu().numpy().view(np.uint32), ref_w.view(np.uint32))
@@ -536,11 +538,12 @@ def test_qwen_shape_specialised_launch(gpu, oracle):
         assert np.array_equal(outs[True], outs[False])
 
 
-@pytest.mark.parametrize("workload,t", [("dsv4-2bit", 1), ("dsv4-2bit", 4), ("maple-ternary", 1)])
+@pytest.mark.parametrize("workload,t", [("dsv4-2bit", 1), ("dsv4-2bit", 4), ("dsv4-2bit", 7), ("maple-ternary", 1),
+                                        ("maple-ternary", 3), ("maple-ternary", 8)])
 def test_other_shape_specialised_launches(gpu, oracle, workload, t):
-    """the large 2-bit layer (D 4096, F 2048, E 256, K 6, 4-bit shared 2048; T = 1 and 4) and the
-    ternary layer (D 2048, F 1024, E 64, K 8, full-softmax router) at full size take their own
-    shape-specialised fused kernels; weights drawn and quantized on the GPU as bench.py does,
+    """the large 2-bit layer (D 4096, F 2048, E 256, K 6, 4-bit shared 2048) and the ternary layer
+    (D 2048, F 1024, E 64, K 8, full-softmax router) at full size take their own shape-specialised fused
+    kernels (one for a single token row, one for any other count); weights drawn and quantized on the GPU as bench.py does,
     checked against the CPU checker and against the chain of separate launches"""
     import bench
     w = dict(bench.WORKLOADS[workload])

@@ -38,6 +38,9 @@ WORKLOADS = {
                       e=256, k=6, fs=2048, bits=2, shared_bits=4, t=1, layers=4),
     "maple-ternary": dict(name="ternary-moe-layer-decode-D2048-F1024-E64-K8", config=4, d=2048, f=1024,
                           e=64, k=8, fs=0, bits=1, shared_bits=4, t=1, layers=40, maple=True),
+    # the reference's MaplePreview architecture (ModelTypes.swift:515-560): 256 ternary experts of 512, top-8
+    "maple-preview": dict(name="ternary-moe-layer-decode-D2048-F512-E256-K8", config=4, d=2048, f=512,
+                          e=256, k=8, fs=0, bits=1, shared_bits=4, t=1, layers=40, maple=True),
 }
 DENSE_MLP = dict(name="dense-4bit-swiglu-mlp-D5120-F17408", d=5120, f=17408, bits=4, layers=8)
 

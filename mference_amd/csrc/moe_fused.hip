@@ -910,6 +910,11 @@ hipError_t launch_fused_decode(hipStream_t s, const mf_moe& h, const mf_moe_laye
   using TernTn = StaticShape<2048, 1024, 64, 8, kDyn, 0>;
   const bool tern = c.bits == MF_BITS_TERNARY && c.d == 2048 && c.f == 1024 && c.num_experts == 64 &&
                     c.top_k == 8 && c.shared_f == 0;
+  // MaplePreview's ternary layer (ModelTypes.swift:515-560: hidden 2048, 256 experts of 512, top-8, no shared expert)
+  using MapleT1 = StaticShape<2048, 512, 256, 8, 1, 0>;
+  using MapleTn = StaticShape<2048, 512, 256, 8, kDyn, 0>;
+  const bool maple = c.bits == MF_BITS_TERNARY && c.d == 2048 && c.f == 512 && c.num_experts == 256 &&
+                     c.top_k == 8 && c.shared_f == 0;
   using Given = RuntimeShapeT<true>;
   using Big2T1Given = StaticShape<4096, 2048, 256, 6, 1, 2048, true>;
   if (!w.router_w) {  // caller-given routing
@@ -924,6 +929,8 @@ hipError_t launch_fused_decode(hipStream_t s, const mf_moe& h, const mf_moe_laye
   else if (big2) MF_FUSED(kBits2, kBits4, Big2Tn);
   else if (tern && t == 1) MF_FUSED(kBitsTernary, kBits4, TernT1);
   else if (tern) MF_FUSED(kBitsTernary, kBits4, TernTn);
+  else if (maple && t == 1) MF_FUSED(kBitsTernary, kBits4, MapleT1);
+  else if (maple) MF_FUSED(kBitsTernary, kBits4, MapleTn);
   else if (c.bits == MF_BITS_4) MF_FUSED(kBits4, kBits4, RuntimeShape);
   else if (c.bits == MF_BITS_2 && c.shared_f && c.shared_bits == MF_BITS_2)
     MF_FUSED(kBits2, kBits2, RuntimeShape);

@@ -539,7 +539,8 @@ def test_qwen_shape_specialised_launch(gpu, oracle, t):
 
 
 @pytest.mark.parametrize("workload,t", [("dsv4-2bit", 1), ("dsv4-2bit", 4), ("dsv4-2bit", 7), ("maple-ternary", 1),
-                                        ("maple-ternary", 3), ("maple-ternary", 8)])
+                                        ("maple-ternary", 3), ("maple-ternary", 8), ("maple-preview", 1),
+                                        ("maple-preview", 6)])
 def test_other_shape_specialised_launches(gpu, oracle, workload, t):
     """the large 2-bit layer (D 4096, F 2048, E 256, K 6, 4-bit shared 2048) and the ternary layer
     (D 2048, F 1024, E 64, K 8, full-softmax router) at full size take their own shape-specialised fused

@@ -207,13 +207,18 @@ template <bool GIVEN = false>
 struct RuntimeShapeT {
   static constexpr bool kStatic = false, kGiven = GIVEN;
   static constexpr uint32_t D = kDyn, F = kDyn, E = kDyn, K = kDyn, T = kDyn, Fs = kDyn;
+  static constexpr uint32_t Mode = kDyn, Maple = kDyn, NoLimit = 0, XPrep = kDyn;
 };
 using RuntimeShape = RuntimeShapeT<false>;
-template <uint32_t D_, uint32_t F_, uint32_t E_, uint32_t K_, uint32_t T_, uint32_t Fs_, bool GIVEN = false>
+// MODE_ / MAPLE_: the router mode and the Maple rounding flag as literals (kDyn: from the arguments);
+// NOLIMIT_ = 1: the layer has no SwiGLU clamp; XPREP_ = 1: the x slices are kept in LDS.
+template <uint32_t D_, uint32_t F_, uint32_t E_, uint32_t K_, uint32_t T_, uint32_t Fs_, bool GIVEN = false,
+          uint32_t MODE_ = kDyn, uint32_t MAPLE_ = kDyn, uint32_t NOLIMIT_ = 0, uint32_t XPREP_ = kDyn>
 struct StaticShape {
   static constexpr bool kStatic = D_ != kDyn && F_ != kDyn && E_ != kDyn && K_ != kDyn && T_ != kDyn && Fs_ != kDyn;
   static constexpr bool kGiven = GIVEN;
   static constexpr uint32_t D = D_, F = F_, E = E_, K = K_, T = T_, Fs = Fs_;
+  static constexpr uint32_t Mode = MODE_, Maple = MAPLE_, NoLimit = NOLIMIT_, XPrep = XPREP_;
 };
 
 // rows one wave takes per step when a row has n elements (compile-time twin of
@@ -230,6 +235,10 @@ __global__ __launch_bounds__(kFusedThreads) void fused_decode_kernel(const Fused
   const uint32_t D = S::D != kDyn ? S::D : a.D, F = S::F != kDyn ? S::F : a.F;
   const uint32_t E = S::E != kDyn ? S::E : a.E, K = S::K != kDyn ? S::K : a.K;
   const uint32_t T = S::T != kDyn ? S::T : a.T, Fs = S::Fs != kDyn ? S::Fs : a.Fs;
+  const int router_mode = S::Mode != kDyn ? static_cast<int>(S::Mode) : a.router_mode;
+  const bool maple = S::Maple != kDyn ? S::Maple != 0u : a.maple != 0;
+  const float limit = S::NoLimit ? 0.0f : a.limit;
+  const bool xprep = S::XPrep != kDyn ? S::XPrep != 0u : a.xprep != 0;
   // LDS carve-up (the launcher sizes it with fused_lds_bytes)
   uint32_t* s_idx = reinterpret_cast<uint32_t*>(smem);                 // [8*8]
   float* s_w = reinterpret_cast<float*>(smem + 256);                    // [8*8]
@@ -345,7 +354,7 @@ __global__ __launch_bounds__(kFusedThreads) void fused_decode_kernel(const Fused
       }
     }
     // the x slices of the routed rows
-    if (a.xprep && wv + n_poll + n_xw >= kFusedWaves && wv + n_poll < kFusedWaves) {
+    if (xprep && wv + n_poll + n_xw >= kFusedWaves && wv + n_poll < kFusedWaves) {
       for (uint32_t q = (wv + n_poll + n_xw - kFusedWaves) * kWave + lane; q < T * n_sl; q += n_xw * kWave) {
         const uint32_t tok = q / n_sl, sl = q % n_sl;
         store_xslice_lds<BITS>(s_xq, s_xsum, tok, n_sl, sl,
@@ -392,7 +401,7 @@ __global__ __launch_bounds__(kFusedThreads) void fused_decode_kernel(const Fused
           __builtin_amdgcn_s_sleep(1);
         }
         if (in) {  // rank counting wants no NaN among the scores it compares
-          const bool clean = rank_count && a.router_mode == 0;
+          const bool clean = rank_count && router_mode == 0;
           s_lg[2 * p] = clean ? score_or_ninf(__uint_as_float(v.x)) : __uint_as_float(v.x);
           s_lg[2 * p + 1] = clean ? score_or_ninf(__uint_as_float(v.z)) : __uint_as_float(v.z);
         }
@@ -401,7 +410,7 @@ __global__ __launch_bounds__(kFusedThreads) void fused_decode_kernel(const Fused
     __syncthreads();
     trace_mark(a, 2);
     if (rank_count) {
-      if (a.router_mode != 0) {  // full softmax first: the probabilities replace the logits
+      if (router_mode != 0) {  // full softmax first: the probabilities replace the logits
         if (wv < T && !full_softmax_probs(s_lg + wv * E, s_lg + wv * E, E, lane)) {
           if (lane == 0) s_flag[wv] = 1u;  // the token routes nowhere; its scores only have to be comparable
           for (uint32_t i = lane; i < E; i += kWave) s_lg[wv * E + i] = 0.0f;
@@ -423,13 +432,13 @@ __global__ __launch_bounds__(kFusedThreads) void fused_decode_kernel(const Fused
         __syncthreads();
         topk_rank_emit(s_lg, s_rank, T, E, K, s_idx, s_sc, threadIdx.x, kFusedThreads);
       }
-      if (a.router_mode != 0) {  // a token with a non-finite logit routes nowhere (maple_moe.metal:62-119)
+      if (router_mode != 0) {  // a token with a non-finite logit routes nowhere (maple_moe.metal:62-119)
         __syncthreads();
         if (threadIdx.x < T * K && s_flag[threadIdx.x / K]) s_idx[threadIdx.x] = E;
       }
       // the routing weights follow after stage B: nothing needs them before stage C
     } else if (wv < T) {
-      if (a.router_mode == 0) topk_select_fast(s_lg + wv * E, E, K, s_idx + wv * K, s_w + wv * K, lane);
+      if (router_mode == 0) topk_select_fast(s_lg + wv * E, E, K, s_idx + wv * K, s_w + wv * K, lane);
       else topk_full_softmax_fast(s_lg + wv * E, s_lg + wv * E, E, K, s_idx + wv * K, s_w + wv * K, lane);
     }
     __syncthreads();
@@ -485,7 +494,7 @@ __global__ __launch_bounds__(kFusedThreads) void fused_decode_kernel(const Fused
           const Chunk<BITS> gc = load_chunk<BITS>(gw, gs, gb, e0);
           const Chunk<BITS> uc = load_chunk<BITS>(uw, us, ub, e0);
           issue_fence();
-          const XSlice<BITS> xs = a.xprep ? load_xslice_lds<BITS>(s_xq, s_xsum, tok, n_sl, e0 / kEPL)
+          const XSlice<BITS> xs = xprep ? load_xslice_lds<BITS>(s_xq, s_xsum, tok, n_sl, e0 / kEPL)
                                           : load_xslice<BITS, kXAligned>(a.x + static_cast<size_t>(tok) * D + e0);
           const float gd = codes_dot<BITS>(gc.codes, xs), ud = codes_dot<BITS>(uc.codes, xs);
           if (ok) {
@@ -511,7 +520,7 @@ __global__ __launch_bounds__(kFusedThreads) void fused_decode_kernel(const Fused
       const uint32_t item = first + i / rpw, row = (item % rgf) * rpw + i % rpw;
       // moe.metal:27-34, 528; maple_moe.metal:153-164
       const uint32_t word =
-          static_cast<uint32_t>(routed_activation(s_gu[2 * i], s_gu[2 * i + 1], a.limit, a.maple != 0)) | (tag16 << 16);
+          static_cast<uint32_t>(routed_activation(s_gu[2 * i], s_gu[2 * i + 1], limit, maple)) | (tag16 << 16);
       if (row < F) store_u32_agent(&a.t_acts[static_cast<size_t>(item / rgf) * F + row], word);
     }
   }
@@ -520,7 +529,7 @@ __global__ __launch_bounds__(kFusedThreads) void fused_decode_kernel(const Fused
   if (rank_count && wv + T >= kFusedWaves) {
     const uint32_t tok = kFusedWaves - 1 - wv;
     const float my_score = lane < K ? s_sc[tok * K + lane] : -__builtin_inff();
-    float wgt = a.router_mode == 0 ? topk_weight_of_rank<0>(my_score, K) : topk_weight_of_rank<1>(my_score, K);
+    float wgt = router_mode == 0 ? topk_weight_of_rank<0>(my_score, K) : topk_weight_of_rank<1>(my_score, K);
     if (s_flag[tok]) wgt = 0.0f;  // maple_moe.metal:62-119: a non-finite logit routes nowhere
     if (lane < K) s_w[tok * K + lane] = wgt;
   }
@@ -734,7 +743,7 @@ __global__ __launch_bounds__(kFusedThreads) void fused_decode_kernel(const Fused
         }
         const float v = group_sum(part, static_cast<int>(lpr));
         // moe.metal:1262; maple_moe.metal:258 (the down output is a bf16 number first)
-        if (sub == 0) s_v[wv * kWave + (lane >> lpr_log2)] = s_w[pair] * (a.maple ? round_bf16(v) : v);
+        if (sub == 0) s_v[wv * kWave + (lane >> lpr_log2)] = s_w[pair] * (maple ? round_bf16(v) : v);
       }
       __syncthreads();
       if (threadIdx.x < rows_per_round) {
@@ -894,27 +903,28 @@ hipError_t launch_fused_decode(hipStream_t s, const mf_moe& h, const mf_moe_laye
   // token loop; Qwen shape 12.3 us against 13.5 us through Tn).  Which literal buys what, Qwen shape, 4
   // token rows: none 40.2 us, T alone 39.8, top_k 37.5, top_k + experts 36.5, d + f 35.1, d + f + top_k 33.9,
   // those + shared_f 29.1, all but T 27.2, all 27.1.
-  using QwenT1 = StaticShape<2048, 512, 256, 8, 1, 512>;
-  using QwenTn = StaticShape<2048, 512, 256, 8, kDyn, 512>;
+  using QwenT1 = StaticShape<2048, 512, 256, 8, 1, 512, false, 0, 0, 1, 1>;
+  using QwenTn = StaticShape<2048, 512, 256, 8, kDyn, 512, false, 0>;
   const bool qwen = c.bits == MF_BITS_4 && c.shared_bits == MF_BITS_4 && c.d == 2048 &&
                     c.f == 512 && c.num_experts == 256 && c.top_k == 8 && c.shared_f == 512 &&
                     c.router_mode == MF_ROUTER_TOPK_SOFTMAX;
   // the large 2-bit layer (hidden 4096, 256 experts of 2048, top-6, 4-bit shared expert of 2048)
-  using Big2T1 = StaticShape<4096, 2048, 256, 6, 1, 2048>;
-  using Big2Tn = StaticShape<4096, 2048, 256, 6, kDyn, 2048>;
+  using Big2T1 = StaticShape<4096, 2048, 256, 6, 1, 2048, false, 0, 0, 0, 1>;
+  using Big2Tn = StaticShape<4096, 2048, 256, 6, kDyn, 2048, false, 0>;
   const bool big2 = c.bits == MF_BITS_2 && c.shared_bits == MF_BITS_4 && c.d == 4096 && c.f == 2048 &&
                     c.num_experts == 256 && c.top_k == 6 && c.shared_f == 2048 &&
                     c.router_mode == MF_ROUTER_TOPK_SOFTMAX;
   // the ternary layer (hidden 2048, 64 experts of 1024, top-8, no shared expert)
-  using TernT1 = StaticShape<2048, 1024, 64, 8, 1, 0>;
+  using TernT1 = StaticShape<2048, 1024, 64, 8, 1, 0, false, 1, 1, 1, 1>;
   using TernTn = StaticShape<2048, 1024, 64, 8, kDyn, 0>;
   const bool tern = c.bits == MF_BITS_TERNARY && c.d == 2048 && c.f == 1024 && c.num_experts == 64 &&
                     c.top_k == 8 && c.shared_f == 0;
   // MaplePreview's ternary layer (ModelTypes.swift:515-560: hidden 2048, 256 experts of 512, top-8, no shared expert)
-  using MapleT1 = StaticShape<2048, 512, 256, 8, 1, 0>;
+  using MapleT1 = StaticShape<2048, 512, 256, 8, 1, 0, false, 1, 1, 1, 1>;
   using MapleTn = StaticShape<2048, 512, 256, 8, kDyn, 0>;
   const bool maple = c.bits == MF_BITS_TERNARY && c.d == 2048 && c.f == 512 && c.num_experts == 256 &&
                      c.top_k == 8 && c.shared_f == 0;
+  const bool no_limit = c.swiglu_limit == 0.0f;  // the one-token instances of the benchmark shapes have these flags as literals
   using Given = RuntimeShapeT<true>;
   using Big2T1Given = StaticShape<4096, 2048, 256, 6, 1, 2048, true>;
   if (!w.router_w) {  // caller-given routing
@@ -923,13 +933,15 @@ hipError_t launch_fused_decode(hipStream_t s, const mf_moe& h, const mf_moe_laye
     else if (c.bits == MF_BITS_2 && c.shared_f && c.shared_bits == MF_BITS_2) MF_FUSED(kBits2, kBits2, Given);
     else if (c.bits == MF_BITS_2) MF_FUSED(kBits2, kBits4, Given);
     else MF_FUSED(kBitsTernary, kBits4, Given);
-  } else if (qwen && t == 1) MF_FUSED(kBits4, kBits4, QwenT1);
+  } else if (qwen && t == 1 && !c.maple_rounding && no_limit && a.xprep) MF_FUSED(kBits4, kBits4, QwenT1);
   else if (qwen) MF_FUSED(kBits4, kBits4, QwenTn);
-  else if (big2 && t == 1) MF_FUSED(kBits2, kBits4, Big2T1);
+  else if (big2 && t == 1 && !c.maple_rounding && a.xprep) MF_FUSED(kBits2, kBits4, Big2T1);
   else if (big2) MF_FUSED(kBits2, kBits4, Big2Tn);
-  else if (tern && t == 1) MF_FUSED(kBitsTernary, kBits4, TernT1);
+  else if (tern && t == 1 && c.router_mode == MF_ROUTER_FULL_SOFTMAX && c.maple_rounding && no_limit && a.xprep)
+    MF_FUSED(kBitsTernary, kBits4, TernT1);
   else if (tern) MF_FUSED(kBitsTernary, kBits4, TernTn);
-  else if (maple && t == 1) MF_FUSED(kBitsTernary, kBits4, MapleT1);
+  else if (maple && t == 1 && c.router_mode == MF_ROUTER_FULL_SOFTMAX && c.maple_rounding && no_limit && a.xprep)
+    MF_FUSED(kBitsTernary, kBits4, MapleT1);
   else if (maple) MF_FUSED(kBitsTernary, kBits4, MapleTn);
   else if (c.bits == MF_BITS_4) MF_FUSED(kBits4, kBits4, RuntimeShape);
   else if (c.bits == MF_BITS_2 && c.shared_f && c.shared_bits == MF_BITS_2)

@@ -1285,41 +1285,47 @@ void qmm_kernel(const QmmLaunch launch) {
     uint32_t* so = reinterpret_cast<uint32_t*>(s_x) + wv * 1024;
     const bool upper = (m >> 2) & 1u;
     const uint32_t dw = ((m & ~7u) >> 1) + (m & 3u);  // word of the row pair (r, r + 4)
+    // The activation's variants are chosen outside the element loops (one uniform branch: Maple's or the
+    // ordinary one) and, for the ordinary one, by selects -- narrowed or not, clamped or not -- so that the
+    // 64 exponentials and reciprocals of a lane are one block of code the compiler can interleave (with
+    // the three tests inside the loops every element was a block of its own).
+    const bool clamp = a.limit > 0.0f, narrow = a.narrow != 0;
+    auto swiglu_block = [&](auto maple_tag) __attribute__((always_inline)) {
+      constexpr bool kMaple = decltype(maple_tag)::value;
 #pragma unroll
-    for (int nt = 0; nt < 2; ++nt) {
-      if (nt == 1 && count <= 32) break;  // no route in the second block: its slots are empty
+      for (int nt = 0; nt < 2; ++nt) {
+        if (nt == 1 && count <= 32) break;  // no route in the second block: its slots are empty
 #pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        uint32_t bits[4];
+        for (int j = 0; j < 4; ++j) {
+          uint32_t bits[4];
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-          float gv = acc[0][nt][4 * j + i], uv = acc[NPROJ - 1][nt][4 * j + i];
-          if (a.maple) {  // maple_moe.metal:153-164
-            bits[i] = f_to_bf16(maple_swiglu(gv, uv));
-            continue;
+          for (int i = 0; i < 4; ++i) {
+            float gv = acc[0][nt][4 * j + i], uv = acc[NPROJ - 1][nt][4 * j + i];
+            if constexpr (kMaple) {  // maple_moe.metal:153-164
+              bits[i] = f_to_bf16(maple_swiglu(gv, uv));
+            } else {
+              const float gr = round_bf16(gv), ur = round_bf16(uv);
+              const float g0 = narrow ? gr : gv, u0 = narrow ? ur : uv;
+              gv = clamp ? fminf(g0, a.limit) : g0;  // (selects, so that a NaN stays one without a clamp)
+              uv = clamp ? fminf(fmaxf(u0, -a.limit), a.limit) : u0;
+              bits[i] = f_to_bf16(fast_silu(gv) * uv);
+            }
           }
-          if (a.narrow) {
-            gv = round_bf16(gv);
-            uv = round_bf16(uv);
-          }
-          if (a.limit > 0.0f) {
-            gv = fminf(gv, a.limit);
-            uv = fminf(fmaxf(uv, -a.limit), a.limit);
-          }
-          bits[i] = f_to_bf16(fast_silu(gv) * uv);
+          // lanes m and m ^ 4 trade halves: the lower lane ends with tokens i = 0, 1 of both rows,
+          // the upper lane with tokens i = 2, 3
+          const uint32_t t01 = bits[0] | (bits[1] << 16), t23 = bits[2] | (bits[3] << 16);
+          const uint32_t keep = upper ? t23 : t01;
+          const uint32_t got = static_cast<uint32_t>(
+              __builtin_amdgcn_ds_swizzle(static_cast<int>(upper ? t01 : t23), 0x101F));  // lane ^ 4
+          const uint32_t lo_row = upper ? got : keep, hi_row = upper ? keep : got;
+          const uint32_t tok = nt * 32 + 8 * j + 4 * h + (upper ? 2u : 0u);
+          so[tok * 16 + dw] = __builtin_amdgcn_perm(hi_row, lo_row, 0x05040100u);
+          so[(tok + 1) * 16 + dw] = __builtin_amdgcn_perm(hi_row, lo_row, 0x07060302u);
         }
-        // lanes m and m ^ 4 trade halves: the lower lane ends with tokens i = 0, 1 of both rows,
-        // the upper lane with tokens i = 2, 3
-        const uint32_t t01 = bits[0] | (bits[1] << 16), t23 = bits[2] | (bits[3] << 16);
-        const uint32_t keep = upper ? t23 : t01;
-        const uint32_t got = static_cast<uint32_t>(
-            __builtin_amdgcn_ds_swizzle(static_cast<int>(upper ? t01 : t23), 0x101F));  // lane ^ 4
-        const uint32_t lo_row = upper ? got : keep, hi_row = upper ? keep : got;
-        const uint32_t tok = nt * 32 + 8 * j + 4 * h + (upper ? 2u : 0u);
-        so[tok * 16 + dw] = __builtin_amdgcn_perm(hi_row, lo_row, 0x05040100u);
-        so[(tok + 1) * 16 + dw] = __builtin_amdgcn_perm(hi_row, lo_row, 0x07060302u);
       }
-    }
+    };
+    if (a.maple) swiglu_block(std::true_type{});
+    else swiglu_block(std::false_type{});
     __builtin_amdgcn_wave_barrier();  // the wave reads back only what it wrote itself
     const uint32_t lane = threadIdx.x & 63u;
 #pragma unroll

@@ -1679,15 +1679,30 @@ __global__ __launch_bounds__(256) void prefill_reduce_kernel(const float* __rest
       for (int i = 0; i < 4; ++i) acc[i] = round_bf16(acc[i] / den);
     }
   }
-  for (uint32_t r = 0; r < K; ++r) {
-    if (idx && idx[t * K + r] >= E) continue;  // a route without an expert adds nothing
-    const float wt = w[t * K + r];
-    float4 v = *reinterpret_cast<const float4*>(partials + (static_cast<size_t>(t) * K + r) * D + d);
-    if (maple) {  // maple_moe.metal:258: the down output is a bf16 number before its weight
-      v.x = round_bf16(v.x); v.y = round_bf16(v.y); v.z = round_bf16(v.z); v.w = round_bf16(v.w);
+  // all of a token's routes are requested before the first is used (a short batch has few waves: a loop
+  // that tests a route's expert before it asks for the route's row walks K round trips one after another);
+  // the row of a route without an expert is read and dropped
+  uint32_t ex[MF_MAX_TOPK];
+  float wt[MF_MAX_TOPK];
+  float4 v[MF_MAX_TOPK];
+#pragma unroll
+  for (uint32_t r = 0; r < MF_MAX_TOPK; ++r) {
+    if (r < K) {
+      ex[r] = idx ? idx[t * K + r] : 0u;
+      wt[r] = w[t * K + r];
+      v[r] = *reinterpret_cast<const float4*>(partials + (static_cast<size_t>(t) * K + r) * D + d);
     }
-    const float p0 = wt * v.x, p1 = wt * v.y, p2 = wt * v.z, p3 = wt * v.w;
-    acc[0] = acc[0] + p0; acc[1] = acc[1] + p1; acc[2] = acc[2] + p2; acc[3] = acc[3] + p3;
+  }
+#pragma unroll
+  for (uint32_t r = 0; r < MF_MAX_TOPK; ++r) {
+    if (r < K && ex[r] < E) {  // a route without an expert adds nothing
+      float4 q = v[r];
+      if (maple) {  // maple_moe.metal:258: the down output is a bf16 number before its weight
+        q.x = round_bf16(q.x); q.y = round_bf16(q.y); q.z = round_bf16(q.z); q.w = round_bf16(q.w);
+      }
+      const float p0 = wt[r] * q.x, p1 = wt[r] * q.y, p2 = wt[r] * q.z, p3 = wt[r] * q.w;
+      acc[0] = acc[0] + p0; acc[1] = acc[1] + p1; acc[2] = acc[2] + p2; acc[3] = acc[3] + p3;
+    }
   }
   uint2 o;
   o.x = static_cast<uint32_t>(f_to_bf16(acc[0])) | (static_cast<uint32_t>(f_to_bf16(acc[1])) << 16);

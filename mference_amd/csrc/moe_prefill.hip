@@ -629,11 +629,25 @@ __global__ __launch_bounds__(1024) void group_one_kernel(const uint32_t* __restr
   const uint32_t T = n_pairs / K, W = group_one_row_words(T);
   uint32_t* bm = reinterpret_cast<uint32_t*>(smem);                 // [E][W] bits: token t of row e
   uint16_t* pref = reinterpret_cast<uint16_t*>(smem + static_cast<size_t>(E) * W * 4);  // [E][W] set bits before word
+  // a thread's routes (at most kGroupOnePairs / 1024 = 8) stay in registers from the marking pass to the
+  // placing pass: one round trip to memory instead of two
+  constexpr uint32_t kMine = kGroupOnePairs / 1024;
+  static_assert(kGroupOnePairs % 1024 == 0, "the launch has 1024 threads");
+  uint32_t my_e[kMine], my_w[kMine];
+#pragma unroll
+  for (uint32_t u = 0; u < kMine; ++u) {
+    const uint32_t p = threadIdx.x + u * 1024;
+    my_e[u] = p < n_pairs ? idx[p] : 0xFFFFFFFFu;
+    my_w[u] = p < n_pairs ? __float_as_uint(w[p]) : 0u;
+  }
   for (uint32_t i = threadIdx.x; i < E * W; i += blockDim.x) bm[i] = 0;
   __syncthreads();
   bool bad = false, dup = false;
-  for (uint32_t p = threadIdx.x; p < n_pairs; p += blockDim.x) {
-    const uint32_t e = idx[p], t = p / K;
+#pragma unroll
+  for (uint32_t u = 0; u < kMine; ++u) {
+    const uint32_t p = threadIdx.x + u * 1024;
+    if (p >= n_pairs) break;
+    const uint32_t e = my_e[u], t = p / K;
     if (e < E) {
       const uint32_t bit = 1u << (t & 31u);
       dup |= (atomicOr(&bm[e * W + (t >> 5)], bit) & bit) != 0u;
@@ -676,16 +690,17 @@ __global__ __launch_bounds__(1024) void group_one_kernel(const uint32_t* __restr
   __syncthreads();
   group_layout(c, E, counts, offsets, starts, tiles, tile_slots, n_tiles, s_cnt, s_tile);
   __syncthreads();
-  for (uint32_t p = threadIdx.x; p < n_pairs; p += blockDim.x) {
-    const uint32_t e = idx[p];
-    if (e >= E) continue;
+#pragma unroll
+  for (uint32_t u = 0; u < kMine; ++u) {
+    const uint32_t p = threadIdx.x + u * 1024, e = my_e[u];
+    if (p >= n_pairs || e >= E) continue;
     const uint32_t t = p / K, at = e * W + (t >> 5);
     const uint32_t pos = (e ? s_cnt[e - 1] : 0u) + pref[at] + __popc(bm[at] & ((1u << (t & 31u)) - 1u));
     mf_pair r;
     r.token = t;
     r.expert = e;
     r.rank = p - t * K;
-    r.weight_bits = __float_as_uint(w[p]);
+    r.weight_bits = my_w[u];
     sorted[pos] = r;
   }
 }

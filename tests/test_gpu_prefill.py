@@ -151,6 +151,7 @@ def test_prefill_layer_matches_per_token_oracle(gpu, oracle, bits, d, f, e, k, f
     (1, 512, 128, 32, 8, 0, 1030, 1),      # ternary rows, full-softmax router
     (4, 128, 128, 100, 3, 0, 3000, 0),     # 94 chunks of 32 tokens (two per wave of the selecting launch), 3 routes each
     (4, 128, 128, 24, 1, 128, 8500, 0),    # 133 chunks of 64 tokens, one route per token
+    (4, 128, 128, 512, 2, 0, 16000, 0),    # 250 chunks of 64 tokens, the largest expert count
 ])
 def test_prefill_long_batches_against_the_per_token_oracle(gpu, oracle, bits, d, f, e, k, fs, t, mode):
     """More than a thousand tokens on small layers (long runs per expert, many full tiles, an odd tile at

@@ -931,8 +931,15 @@ hipError_t launch_fused_decode(hipStream_t s, const mf_moe& h, const mf_moe_laye
   const bool no_limit = c.swiglu_limit == 0.0f;  // the one-token instances of the benchmark shapes have these flags as literals
   using Given = RuntimeShapeT<true>;
   using Big2T1Given = StaticShape<4096, 2048, 256, 6, 1, 2048, true>;
+  using QwenT1Given = StaticShape<2048, 512, 256, 8, 1, 512, true, kDyn, 0, 1, 1>;
+  using QwenTnGiven = StaticShape<2048, 512, 256, 8, kDyn, 512, true>;
+  // (with the routing given the router mode plays no part: the shapes are recognised without it)
+  const bool qwen_dims = c.bits == MF_BITS_4 && c.shared_bits == MF_BITS_4 && c.d == 2048 && c.f == 512 &&
+                         c.num_experts == 256 && c.top_k == 8 && c.shared_f == 512;
   if (!w.router_w) {  // caller-given routing
     if (big2 && t == 1) MF_FUSED(kBits2, kBits4, Big2T1Given);
+    else if (qwen_dims && t == 1 && !c.maple_rounding && no_limit && a.xprep) MF_FUSED(kBits4, kBits4, QwenT1Given);
+    else if (qwen_dims) MF_FUSED(kBits4, kBits4, QwenTnGiven);
     else if (c.bits == MF_BITS_4) MF_FUSED(kBits4, kBits4, Given);
     else if (c.bits == MF_BITS_2 && c.shared_f && c.shared_bits == MF_BITS_2) MF_FUSED(kBits2, kBits2, Given);
     else if (c.bits == MF_BITS_2) MF_FUSED(kBits2, kBits4, Given);

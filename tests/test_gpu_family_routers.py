@@ -79,6 +79,36 @@ def test_sqrtsoftplus_router_bit_exact(gpu, oracle, e, d, k, t):
     assert torch.equal(w, w2)
 
 
+@pytest.mark.parametrize("seed", range(14))
+def test_router_logits_sweep(gpu, oracle, seed):
+    """drawn (experts, width, tokens) across the batched router's kernels: the register-tiled one (up to 256
+    tokens, widths that are no multiple of 512), the matrix-core walk as a loop (1536, 2560, 3072) and unrolled
+    (1024, 2048, 4096), expert counts that leave rows over after the blocks of 32 (100, 258) -- logits bit for
+    bit against the one-row order of the checker on sampled tokens, and the selection on top of them"""
+    rng0 = np.random.default_rng(0x60A7 + seed)
+    e = int(rng0.choice([32, 64, 100, 128, 256, 258, 512]))
+    d = int(rng0.choice([512, 1024, 1536, 2048, 2560, 3072, 4096]))
+    t = int(rng0.choice([17, 200, 257, 300, 700, 1500]))
+    k = int(rng0.choice([2, 6, 8]))
+    rng, wr, x = _draw(oracle, f"sweep-{seed}", e, d, t, 0.05)
+    bias = rng.uniform_fill(-0.3, 0.3, e)
+    fam = ops.FamilyRouters(gpu)
+    idx = torch.zeros((t, k), dtype=torch.int32, device="cuda")
+    w = torch.zeros((t, k), dtype=torch.float32, device="cuda")
+    lg = torch.zeros((t, e), dtype=torch.float32, device="cuda")
+    fam.encode_router_top_k(ops.bf16_tensor(wr), ops.bf16_tensor(x), _f32(bias), idx, w, e, d, 1.5, lg,
+                            top_k=k, t=t)
+    torch.cuda.synchronize()
+    lg_h, idx_h, w_h = lg.cpu().numpy(), idx.cpu().numpy().astype(np.uint32), w.cpu().numpy()
+    what = f"seed {seed}: e={e} d={d} t={t} k={k}"
+    for i in sorted(set([0, 1, 31, 32, t // 2, t - 2, t - 1]) & set(range(t))):
+        ref_lg = oracle.router_logits(wr, x[i])
+        assert np.array_equal(_bits(lg_h[i]), _bits(ref_lg)), (what, i)
+        ri, rw = oracle.router_sqrtsoftplus(ref_lg, bias, k, 1.5)
+        assert np.array_equal(idx_h[i], ri), (what, i)
+        assert np.array_equal(_bits(w_h[i]), _bits(rw)), (what, i)
+
+
 @pytest.mark.parametrize("e", [8, 16, 24, 33, 100, 128, 168, 255, 256])
 def test_sqrtsoftplus_ties_match_serial(gpu, oracle, e):
     """RouterTopKParityTests.swift:52-77: tie-heavy logits and duplicated correction biases"""

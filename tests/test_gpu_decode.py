@@ -538,6 +538,37 @@ def test_qwen_shape_specialised_launch(gpu, oracle, t):
         assert np.array_equal(outs[True], outs[False])
 
 
+@pytest.mark.parametrize("limit,maple", [(7.0, False), (0.0, True), (3.0, True)])
+def test_qwen_shape_with_other_flags(gpu, oracle, limit, maple):
+    """the Qwen-shaped layer with a SwiGLU clamp or Maple rounding: the one-token instance has "no clamp, no
+    Maple rounding" as literals, so these calls take the instance that reads the flags from the arguments --
+    one token row and three, against the checker and against the chain of launches"""
+    import bench
+    w = dict(bench.QWEN)
+    stack = bench.build_stack(gpu, w, 1, torch.device("cuda", 0))
+    host = bench.layer_to_host(stack[0], w)
+    host.swiglu_limit, host.maple_rounding = limit, maple
+    moe = ops.MoE(gpu, w["d"], w["f"], w["e"], w["k"], bits=4, shared_f=w["fs"], swiglu_limit=limit,
+                  maple_rounding=maple)
+    gen = torch.Generator(device="cuda")
+    gen.manual_seed(99)
+    for t in (1, 3):
+        x = torch.randn((t, w["d"]), generator=gen, device="cuda").to(torch.bfloat16)
+        ref_y, ref_idx, ref_w = oracle.moe_layer(host, ops.bf16_bits(x))
+        outs = {}
+        for fused in (True, False):
+            moe.set_fused(fused)
+            y = torch.zeros_like(x)
+            idx = torch.zeros((t, w["k"]), dtype=torch.int32, device="cuda")
+            moe.encode_decode_layer(stack[0], x, y, t=t, out_indices=idx)
+            moe.status()
+            assert np.array_equal(idx.cpu().numpy().astype(np.uint32), ref_idx)
+            assert_layer_close(oracle.bf16_to_float(ops.bf16_bits(y)), oracle.bf16_to_float(ref_y),
+                               f"qwen shape limit={limit} maple={maple} t={t} fused={fused}")
+            outs[fused] = ops.bf16_bits(y)
+        assert np.array_equal(outs[True], outs[False])
+
+
 @pytest.mark.parametrize("workload,t", [("dsv4-2bit", 1), ("dsv4-2bit", 4), ("dsv4-2bit", 7), ("maple-ternary", 1),
                                         ("maple-ternary", 3), ("maple-ternary", 8), ("maple-preview", 1),
                                         ("maple-preview", 6)])

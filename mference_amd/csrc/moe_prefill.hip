@@ -1771,12 +1771,12 @@ hipError_t launch_prefill_router(hipStream_t s, const uint16_t* W, const uint16_
     fused = *tail;
     tail->xp = nullptr;
   }
-  // Up to 256 tokens the matrix-core kernel has too few workgroups (T/32 x E/32) to cover the chip: the
-  // register-tiled kernel is faster there (Qwen shape, layer time: 64 tokens 110 -> 100 us, 128 tokens
-  // 112 -> 103 us, 256 tokens 118 -> 116 us, equal at 384; it holds rows of up to 4096 elements).  Both give
-  // the same bits.  The matrix-core kernel takes whole blocks of 32 rows; rows left over (the two sink rows
-  // of a 258-row Inkling router) go through the register-tiled kernel behind it.
-  const uint32_t e32 = (T > 256 || D > 4096) && D % 512 == 0 && aligned16(W) && aligned16(x) && x_stride % 8 == 0
+  // Up to 192 tokens the matrix-core kernel has too few workgroups (T/32 x E/32) to cover the chip: the
+  // register-tiled kernel is faster there (Qwen shape, layer time: 128 tokens 79 against 82 us, equal at 192,
+  // 256 tokens 98.4 against 96.4 us; it holds rows of up to 4096 elements).  Both give the same bits.  The
+  // matrix-core kernel takes whole blocks of 32 rows; rows left over (the two sink rows of a 258-row
+  // Inkling router) go through the register-tiled kernel behind it.
+  const uint32_t e32 = (T > 192 || D > 4096) && D % 512 == 0 && aligned16(W) && aligned16(x) && x_stride % 8 == 0
                            ? E & ~31u : 0u;
   // rows of more than 4096 elements that the matrix-core kernel does not take (a width that is no
   // multiple of 512, rows left over by the blocks of 32, unaligned operands): the register-tiled

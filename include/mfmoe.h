@@ -179,6 +179,14 @@ mf_status mf_residual_rmsnorm(mf_ctx* ctx, mf_stream stream, uint16_t* hidden, c
 size_t mf_qmm_workspace_bytes(uint32_t m, uint32_t n, uint32_t k);
 mf_status mf_qmm(mf_ctx* ctx, mf_stream stream, mf_qtensor w, mf_bits bits, const uint16_t* x, void* y, uint32_t m,
                  uint32_t n, uint32_t k, int out_f32, void* workspace, size_t workspace_bytes);
+/* The `Path` MPPPrefillInt4QMM.encode returns (MPPPrefillInt4QMM.swift:5-8, 43-55): which kernel mf_qmm
+ * takes for these arguments -- MF_QMM_PATH_MATRIX_CORE or MF_QMM_PATH_ROWS (row by row through the
+ * kernels of mf_gemv) -- or the negative status with which mf_qmm would refuse them (the reference's
+ * .unavailable).  Launches nothing and touches no device memory. */
+#define MF_QMM_PATH_MATRIX_CORE 1
+#define MF_QMM_PATH_ROWS 2
+int mf_qmm_path(mf_qtensor w, mf_bits bits, const uint16_t* x, const void* y, uint32_t m, uint32_t n, uint32_t k,
+                const void* workspace, size_t workspace_bytes);
 
 /* SharedExpertInt4.encode (Kernels/MoE/SharedExpertInt4.swift:70-165) /
  * SharedExpertRuntime.encode (:193-202): y[t,d] = bf16(down . act),
@@ -196,9 +204,9 @@ mf_status mf_shared_expert(mf_ctx* ctx, mf_stream stream, const uint16_t* x, mf_
                            size_t scratch_act_bytes);
 
 /* mf_shared_expert for callers that cannot allocate device memory and bring no scratch buffer:
- * code under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc.  It has no
- * counterpart in the reference (SharedExpertInt4.encode takes the caller's scratch buffer,
- * SharedExpertInt4.swift:76-78).  The activation vector act[t,f] lives in a device array that is
+ * code under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc.
+ * It has no counterpart in the reference, whose operators always take the caller's scratch buffer.
+ * The activation vector act[t,f] lives in a device array that is
  * part of the library image (MF_STATIC_ACT_ELEMS bf16 = 512 KiB, held on every GPU the library
  * runs on until the process ends); the call launches the kernels of mf_shared_expert and calls no
  * hipMalloc / hipFree.  Same arguments, checks and results (bit for bit) as mf_shared_expert;
@@ -240,6 +248,14 @@ typedef struct {
                              * layer runs on the chain of launches (the fused launch and the matrix-core
                              * prefill take group 64); up and down stay at 64. */
 } mf_moe_config;
+
+/* The preconditions of MoE.init / MoEDeepseekV4.init / MapleMoE.init (MoE.swift:65-151, 165-167;
+ * MoEDeepseekV4.swift:31-87) as a status instead of a trap: MF_OK when mf_moe_create would accept the
+ * shape.  Host arithmetic only, no device.  Refused: sizes that are no multiples of 64, more than
+ * MF_MAX_EXPERTS experts or MF_MAX_TOPK routes, an unknown format, the full-softmax router
+ * (MF_ROUTER_FULL_SOFTMAX) with an expert count that is no multiple of 32, a gate group of 32 on
+ * anything but 2-bit experts. */
+mf_status mf_moe_config_check(const mf_moe_config* cfg);
 
 /* MoE.init (Kernels/MoE/MoE.swift:65-151): one operator instance per shape; owns the
  * router-logit and activation workspace (MoE.swift:136-150). */
@@ -352,11 +368,19 @@ mf_status mf_moe_phase2(mf_moe* h, mf_stream stream, const void* expert_base,
  * size f, laid out back to back in the order the reference's repacker writes them -- gate
  * {codes, scales, biases}, up {...}, down {...} (MferenceRepack/Core/Planning/RepackPlanner.swift:
  * 544-712; read back by Model.routedExpertOffsets, Runtime/Inference/ModelExpertIO.swift:20-35);
- * ternary experts store no biases (their bias offsets read 0).  blob_bytes: size of one expert;
- * stride: that size rounded up to `align` (the reference rounds to a 16 KiB page).  Host
- * arithmetic only; for callers that build a resident pool themselves (synthetic weights, tests). */
+ * blob_bytes: size of one expert; stride: that size rounded up to `align` (the reference rounds to a
+ * 16 KiB page).  Host arithmetic only; for callers that build a resident pool themselves (synthetic
+ * weights, tests).
+ * Ternary experts, mf_expert_blob_layout: a COMPACT form private to this library -- codes and scale tables
+ * only, bias offsets 0 (the kernels take bias = -scale) -- which is NOT the byte layout of a Maple
+ * packed_experts file.  mf_expert_blob_layout_repacked gives the layout the reference's repacker writes for
+ * every format: ternary tensors carry their negated-scale bias tables there too (RepackPlanner.swift:619-640),
+ * so offsets, blob size and stride equal those of a real file; for 4-bit and 2-bit experts the two calls
+ * agree.  The ternary operators accept either layout (they read the scale tables only). */
 mf_status mf_expert_blob_layout(uint32_t d, uint32_t f, mf_bits bits, uint32_t align, mf_expert_offsets* offsets,
                                 size_t* blob_bytes, size_t* stride);
+mf_status mf_expert_blob_layout_repacked(uint32_t d, uint32_t f, mf_bits bits, uint32_t align,
+                                         mf_expert_offsets* offsets, size_t* blob_bytes, size_t* stride);
 
 /* The routed phases over slots named directly, for a caller that holds its experts in slots of its
  * own (a streaming cache) instead of one pool indexed by expert id.  Slot s = token * top_k + rank
@@ -371,7 +395,12 @@ mf_status mf_expert_blob_layout(uint32_t d, uint32_t f, mf_bits bits, uint32_t a
  * reads 0 -- the guard of the reference's slot-map form, whose lookup kernel writes it.
  * mf_moe_slot_lookup is that kernel, router_slot_lookup_k8 (moe.metal:594-617): slot_of is the caller's
  * device table int16 [num_experts] (negative: not in a slot); out_slot_offsets[s] = slot * slot_stride,
- * out_all_hit = 1 when every routed expert of the call has a slot. */
+ * out_all_hit = 1 when every routed expert of the call has a slot.
+ * Limits: t <= MF_MAX_TOKENS in all three calls (one guard word covers one lookup; longer batches go in
+ * chunks, each with its own lookup and guard word).  slot_stride has to be a multiple of 16 (anything else
+ * is refused with MF_ERR_INVALID_ARGUMENT); a slab that is not 16-byte aligned is read through the byte-wise
+ * kernels.  In the table-of-addresses form (slab == NULL) the host cannot see the addresses: the 16-byte
+ * alignment of every blob is the caller's promise there, as the header of this comment states. */
 mf_status mf_moe_slot_lookup(mf_moe* h, mf_stream stream, const uint32_t* idx, uint32_t t,
                              const int16_t* slot_of, uint64_t slot_stride, uint64_t* out_slot_offsets,
                              uint32_t* out_all_hit);

@@ -224,18 +224,17 @@ class SharedExpertInt4 {
 // encode returns the path like the reference: Unavailable for sizes or offsets it rejects.
 class MPPPrefillInt4QMM {
  public:
-  enum class Path { AffineMatrixCoreBF16, Unavailable };
+  enum class Path { AffineMatrixCoreBF16, AffineRowsGEMV, Unavailable };
   static constexpr int tileM = 64, tileN = 32, tileK = MF_GROUP_SIZE;
   explicit MPPPrefillInt4QMM(const MetalContext& context, mf_bits bits = MF_BITS_4) : ctx_(context.raw()), bits_(bits) {}
   static size_t workspaceBytes(uint32_t m, uint32_t n, uint32_t k) { return mf_qmm_workspace_bytes(m, n, k); }
   Path encode(mf_stream commandBuffer, mf_qtensor weights, const uint16_t* x, void* y, uint32_t m, uint32_t n,
               uint32_t k, void* workspace, size_t workspaceBytes, bool outputFloat32 = false) const {
-    const mf_status st = mf_qmm(ctx_, commandBuffer, weights, bits_, x, y, m, n, k, outputFloat32 ? 1 : 0, workspace,
-                                workspaceBytes);
-    if (st == MF_ERR_INVALID_ARGUMENT || st == MF_ERR_DIMENSION_MISMATCH || st == MF_ERR_UNSUPPORTED_BITS)
-      return Path::Unavailable;
-    check(st, ctx_);
-    return Path::AffineMatrixCoreBF16;
+    const int path = mf_qmm_path(weights, bits_, x, y, m, n, k, workspace, workspaceBytes);
+    if (path < 0) return Path::Unavailable;
+    check(mf_qmm(ctx_, commandBuffer, weights, bits_, x, y, m, n, k, outputFloat32 ? 1 : 0, workspace, workspaceBytes),
+          ctx_);
+    return path == MF_QMM_PATH_MATRIX_CORE ? Path::AffineMatrixCoreBF16 : Path::AffineRowsGEMV;
   }
 
  private:

@@ -84,8 +84,11 @@ SIGNATURES = {
     "mf_shared_expert_scratch_bytes": (_SZ, [_U32, _U32, _U32]),
     "mf_qmm_workspace_bytes": (_SZ, [_U32, _U32, _U32]),
     "mf_qmm": (_I, [_P, _P, QTensor, _I, _P, _P, _U32, _U32, _U32, _I, _P, _SZ]),
+    "mf_qmm_path": (_I, [QTensor, _I, _P, _P, _U32, _U32, _U32, _P, _SZ]),
     "mf_shared_expert_static": (_I, [_P, _P, _P, QTensor, QTensor, QTensor, _I, _U32, _U32, _U32, _P]),
     "mf_expert_blob_layout": (_I, [_U32, _U32, _I, _U32, C.POINTER(ExpertOffsets), C.POINTER(_SZ), C.POINTER(_SZ)]),
+    "mf_expert_blob_layout_repacked": (_I, [_U32, _U32, _I, _U32, C.POINTER(ExpertOffsets), C.POINTER(_SZ), C.POINTER(_SZ)]),
+    "mf_moe_config_check": (_I, [C.POINTER(MoEConfig)]),
     "mf_moe_create": (_I, [_P, C.POINTER(MoEConfig), C.POINTER(_P)]),
     "mf_moe_destroy": (None, [_P]),
     "mf_moe_router": (_I, [_P, _P, _P, _P, _U32, _U32, _P, _P, _P]),

@@ -210,16 +210,32 @@ size_t mf_qmm_workspace_bytes(uint32_t m, uint32_t n, uint32_t k) {
   return mf::dense_qmm_workspace_bytes(m, n, k);
 }
 
-mf_status mf_qmm(mf_ctx* ctx, mf_stream stream, mf_qtensor w, mf_bits bits, const uint16_t* x, void* y, uint32_t m,
-                 uint32_t n, uint32_t k, int out_f32, void* workspace, size_t workspace_bytes) {
-  // the conditions under which MPPPrefillInt4QMM.encode returns .unavailable (MPPPrefillInt4QMM.swift:43-55)
-  if (!ctx || !x || !y) return MF_ERR_INVALID_ARGUMENT;
+// the conditions under which MPPPrefillInt4QMM.encode returns .unavailable (MPPPrefillInt4QMM.swift:43-55),
+// then the kernel the call takes
+static int qmm_path(mf_qtensor w, mf_bits bits, const uint16_t* x, const void* y, uint32_t m, uint32_t n, uint32_t k,
+                    const void* workspace, size_t workspace_bytes) {
+  if (!x || !y) return MF_ERR_INVALID_ARGUMENT;
   if (!bits_ok(bits)) return MF_ERR_UNSUPPORTED_BITS;
   if (m == 0 || n == 0 || k == 0 || k % MF_GROUP_SIZE != 0 || m > MF_MAX_ROWS) return MF_ERR_DIMENSION_MISMATCH;
   if (!qtensor_ok(w, bits) || !mf::aligned2(x) || !mf::aligned2(y)) return MF_ERR_INVALID_ARGUMENT;
-  auto s = static_cast<hipStream_t>(stream);
   if (workspace && mf::aligned16(workspace) && mf::dense_qmm_takes(w, bits, x, y, m, n, k) &&
-      workspace_bytes >= mf::dense_qmm_workspace_bytes(m, n, k)) {
+      workspace_bytes >= mf::dense_qmm_workspace_bytes(m, n, k))
+    return MF_QMM_PATH_MATRIX_CORE;
+  return MF_QMM_PATH_ROWS;
+}
+
+int mf_qmm_path(mf_qtensor w, mf_bits bits, const uint16_t* x, const void* y, uint32_t m, uint32_t n, uint32_t k,
+                const void* workspace, size_t workspace_bytes) {
+  return qmm_path(w, bits, x, y, m, n, k, workspace, workspace_bytes);
+}
+
+mf_status mf_qmm(mf_ctx* ctx, mf_stream stream, mf_qtensor w, mf_bits bits, const uint16_t* x, void* y, uint32_t m,
+                 uint32_t n, uint32_t k, int out_f32, void* workspace, size_t workspace_bytes) {
+  if (!ctx) return MF_ERR_INVALID_ARGUMENT;
+  const int path = qmm_path(w, bits, x, y, m, n, k, workspace, workspace_bytes);
+  if (path < 0) return static_cast<mf_status>(path);
+  auto s = static_cast<hipStream_t>(stream);
+  if (path == MF_QMM_PATH_MATRIX_CORE) {
     MF_HIP(ctx, mf::launch_dense_qmm(s, w, bits, x, y, m, n, k, out_f32 != 0, workspace));
     return MF_OK;
   }
@@ -233,8 +249,21 @@ mf_status mf_qmm(mf_ctx* ctx, mf_stream stream, mf_qtensor w, mf_bits bits, cons
   return MF_OK;
 }
 
+static mf_status blob_layout(uint32_t d, uint32_t f, mf_bits bits, uint32_t align, bool ternary_bias_tables,
+                             mf_expert_offsets* offsets, size_t* blob_bytes, size_t* stride);
+
 mf_status mf_expert_blob_layout(uint32_t d, uint32_t f, mf_bits bits, uint32_t align, mf_expert_offsets* offsets,
                                 size_t* blob_bytes, size_t* stride) {
+  return blob_layout(d, f, bits, align, false, offsets, blob_bytes, stride);
+}
+
+mf_status mf_expert_blob_layout_repacked(uint32_t d, uint32_t f, mf_bits bits, uint32_t align,
+                                         mf_expert_offsets* offsets, size_t* blob_bytes, size_t* stride) {
+  return blob_layout(d, f, bits, align, true, offsets, blob_bytes, stride);
+}
+
+static mf_status blob_layout(uint32_t d, uint32_t f, mf_bits bits, uint32_t align, bool ternary_bias_tables,
+                             mf_expert_offsets* offsets, size_t* blob_bytes, size_t* stride) {
   if (!offsets) return MF_ERR_INVALID_ARGUMENT;
   if (!bits_ok(bits)) return MF_ERR_UNSUPPORTED_BITS;
   if (d == 0 || f == 0 || d % MF_GROUP_SIZE != 0 || f % MF_GROUP_SIZE != 0) return MF_ERR_DIMENSION_MISMATCH;
@@ -242,7 +271,7 @@ mf_status mf_expert_blob_layout(uint32_t d, uint32_t f, mf_bits bits, uint32_t a
   const uint64_t code_bits = bits == MF_BITS_4 ? 4 : 2;
   const uint64_t gu_w = static_cast<uint64_t>(f) * d * code_bits / 8, gu_s = static_cast<uint64_t>(f) * (d / MF_GROUP_SIZE) * 2;
   const uint64_t dn_w = static_cast<uint64_t>(d) * f * code_bits / 8, dn_s = static_cast<uint64_t>(d) * (f / MF_GROUP_SIZE) * 2;
-  const bool has_bias = bits != MF_BITS_TERNARY;
+  const bool has_bias = bits != MF_BITS_TERNARY || ternary_bias_tables;
   const uint64_t sizes[3][2] = {{gu_w, gu_s}, {gu_w, gu_s}, {dn_w, dn_s}};
   uint32_t* out[3][3] = {{&offsets->gate_w, &offsets->gate_s, &offsets->gate_b},
                          {&offsets->up_w, &offsets->up_s, &offsets->up_b},
@@ -262,9 +291,8 @@ mf_status mf_expert_blob_layout(uint32_t d, uint32_t f, mf_bits bits, uint32_t a
 
 /* ---------------------------------------------------------- MoE operator */
 
-mf_status mf_moe_create(mf_ctx* ctx, const mf_moe_config* cfg, mf_moe** out) {
-  if (!ctx || !cfg || !out) return MF_ERR_INVALID_ARGUMENT;
-  *out = nullptr;
+mf_status mf_moe_config_check(const mf_moe_config* cfg) {
+  if (!cfg) return MF_ERR_INVALID_ARGUMENT;
   if (!bits_ok(cfg->bits)) return MF_ERR_UNSUPPORTED_BITS;
   if (cfg->shared_f && !bits_ok(cfg->shared_bits)) return MF_ERR_UNSUPPORTED_BITS;
   if (cfg->d == 0 || cfg->d % MF_GROUP_SIZE != 0 || cfg->f == 0 || cfg->f % MF_GROUP_SIZE != 0 ||
@@ -280,6 +308,14 @@ mf_status mf_moe_create(mf_ctx* ctx, const mf_moe_config* cfg, mf_moe** out) {
   if (cfg->gate_group_size != 0 && cfg->gate_group_size != 64 &&
       !(cfg->gate_group_size == 32 && cfg->bits == MF_BITS_2))
     return MF_ERR_INVALID_ARGUMENT;
+  return MF_OK;
+}
+
+mf_status mf_moe_create(mf_ctx* ctx, const mf_moe_config* cfg, mf_moe** out) {
+  if (!ctx || !cfg || !out) return MF_ERR_INVALID_ARGUMENT;
+  *out = nullptr;
+  const mf_status cfg_status = mf_moe_config_check(cfg);
+  if (cfg_status != MF_OK) return cfg_status;
 
   auto* h = new (std::nothrow) mf_moe();
   if (!h) return MF_ERR_OUT_OF_MEMORY;
@@ -494,6 +530,9 @@ mf_status mf_moe_slot_lookup(mf_moe* h, mf_stream stream, const uint32_t* idx, u
   if (t == 0 || t > MF_MAX_TOKENS) return MF_ERR_INVALID_ARGUMENT;
   if ((reinterpret_cast<uintptr_t>(out_slot_offsets) & 7u) || (reinterpret_cast<uintptr_t>(slot_of) & 1u))
     return MF_ERR_INVALID_ARGUMENT;
+  // the routed phases read every blob with 16-byte loads when the slab is 16-byte aligned: the offsets
+  // this call writes have to keep that alignment
+  if (slot_stride % 16 != 0) return MF_ERR_INVALID_ARGUMENT;
   MF_HIP(h->ctx, mf::launch_slot_lookup(static_cast<hipStream_t>(stream), idx, slot_of, t * h->cfg.top_k,
                                         h->cfg.num_experts, slot_stride, out_slot_offsets, out_all_hit));
   return MF_OK;
@@ -503,7 +542,8 @@ mf_status mf_moe_phase1_slots(mf_moe* h, mf_stream stream, const void* slab, con
                               const uint32_t* all_hit, const mf_expert_offsets* offsets, const uint16_t* x,
                               uint32_t t, uint32_t x_stride, uint16_t* acts) {
   if (!h || !slot_offsets || !offsets || !x || !acts) return MF_ERR_INVALID_ARGUMENT;
-  if (t == 0 || t > MF_MAX_ROWS || x_stride < h->cfg.d) return MF_ERR_INVALID_ARGUMENT;
+  // (one guard word covers one lookup, and a lookup covers at most MF_MAX_TOKENS rows)
+  if (t == 0 || t > MF_MAX_TOKENS || x_stride < h->cfg.d) return MF_ERR_INVALID_ARGUMENT;
   if (!offsets_ok(*offsets, h->cfg.bits) || !mf::aligned2(slab) || !mf::aligned2(x) || !mf::aligned2(acts) ||
       (reinterpret_cast<uintptr_t>(slot_offsets) & 7u))
     return MF_ERR_INVALID_ARGUMENT;
@@ -516,7 +556,7 @@ mf_status mf_moe_phase2_slots(mf_moe* h, mf_stream stream, const void* slab, con
                               const uint32_t* all_hit, const mf_expert_offsets* offsets, const float* w,
                               const uint16_t* acts, const uint16_t* residual, uint32_t t, uint16_t* y) {
   if (!h || !slot_offsets || !offsets || !w || !acts || !y) return MF_ERR_INVALID_ARGUMENT;
-  if (t == 0 || t > MF_MAX_ROWS) return MF_ERR_INVALID_ARGUMENT;
+  if (t == 0 || t > MF_MAX_TOKENS) return MF_ERR_INVALID_ARGUMENT;
   if (!offsets_ok(*offsets, h->cfg.bits) || !mf::aligned2(slab) || !mf::aligned2(acts) || !mf::aligned2(y) ||
       (residual && !mf::aligned2(residual)) || (reinterpret_cast<uintptr_t>(slot_offsets) & 7u))
     return MF_ERR_INVALID_ARGUMENT;

@@ -889,6 +889,23 @@ hipError_t launch_gemv(hipStream_t s, const mf_qtensor& w, int bits, const uint1
     qa.W[0] = ma.W[0]; qa.S[0] = ma.S[0]; qa.B[0] = ma.B[0];
     qa.x = x; qa.y = y; qa.M = m; qa.N = n; qa.T = t; qa.out_f32 = ma.out_f32;
     if (rows_quad_try<1>(s, qa, device_cu_count(), err)) return err;
+    // Five to eight token rows of a matrix the quad kernel takes: two launches, rows 0..3 and the
+    // rest.  The quad kernel runs the same instructions for a token whatever rides along, so every row
+    // keeps the bits of a single-token call (MultiXKernelParityTests.swift:50-77); the weights stream
+    // twice.  (y rows are m elements apart, 2 or 4 bytes each: 16-byte aligned since m % 4 == 0 and t > 4
+    // only reaches here with m >= 1024.)
+    if (t > 4 && t <= 8) {
+      RowsQuadArgs q0 = qa, q1 = qa;
+      q0.T = 4;
+      q1.T = t - 4;
+      q1.x = x + static_cast<size_t>(4) * n;
+      q1.y = static_cast<uint8_t*>(y) + static_cast<size_t>(4) * m * (out_f32 ? 4 : 2);
+      if (rows_quad_try<1>(s, q0, device_cu_count(), err)) {
+        if (err != hipSuccess) return err;
+        if (rows_quad_try<1>(s, q1, device_cu_count(), err)) return err;
+        return hipErrorUnknown;  // (not reached: the second launch has the shape of the first)
+      }
+    }
     if (rows_mfma_try<1>(s, ma, device_cu_count(), err)) return err;
   }
   if (!lane_order && al && (bits == kBits4 || bits == kBits2)) {
@@ -929,6 +946,18 @@ hipError_t launch_gate_up_act(hipStream_t s, const mf_qtensor& gate, const mf_qt
     for (int p = 0; p < 2; ++p) { qa.W[p] = ma.W[p]; qa.S[p] = ma.S[p]; qa.B[p] = ma.B[p]; }
     qa.x = x; qa.y = act; qa.M = f; qa.N = d; qa.T = t;
     if (rows_quad_try<2>(s, qa, device_cu_count(), err)) return err;
+    if (t > 4 && t <= 8) {  // as in launch_gemv: rows 0..3, then the rest, same bits as single-token calls
+      RowsQuadArgs q0 = qa, q1 = qa;
+      q0.T = 4;
+      q1.T = t - 4;
+      q1.x = x + static_cast<size_t>(4) * d;
+      q1.y = act + static_cast<size_t>(4) * f;
+      if (rows_quad_try<2>(s, q0, device_cu_count(), err)) {
+        if (err != hipSuccess) return err;
+        if (rows_quad_try<2>(s, q1, device_cu_count(), err)) return err;
+        return hipErrorUnknown;
+      }
+    }
     if (rows_mfma_try<2>(s, ma, device_cu_count(), err)) return err;
   }
   if (!lane_order && al && (bits == kBits4 || bits == kBits2)) {

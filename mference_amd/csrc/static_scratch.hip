@@ -11,6 +11,8 @@
 // gate/up launch writes every element the down launch reads -- so nothing is cleared.
 #include <stdio.h>
 
+#include <atomic>
+
 #include "mf_internal.h"
 
 namespace {
@@ -19,7 +21,9 @@ constexpr size_t kStaticActBytes = MF_STATIC_ACT_ELEMS * sizeof(uint16_t);  // 5
 static __device__ __align__(256) unsigned char scratch[kStaticActBytes];
 
 constexpr int kMaxDevices = 64;
-void* g_scratch_ptr[kMaxDevices] = {nullptr};  // device address of `scratch` on each GPU
+// device address of `scratch` on each GPU.  Atomic: contexts may be created from several host threads;
+// every thread that looks the address up on a device gets the same value, so the last store wins harmlessly.
+std::atomic<void*> g_scratch_ptr[kMaxDevices];
 
 }  // namespace
 
@@ -28,12 +32,12 @@ namespace mf {
 // Looks up this device's address of the scratch array; `device` must be the current device.
 hipError_t static_scratch_init(int device) {
   if (device < 0 || device >= kMaxDevices) return hipErrorInvalidDevice;
-  if (g_scratch_ptr[device]) return hipSuccess;
+  if (g_scratch_ptr[device].load(std::memory_order_acquire)) return hipSuccess;
   void* ptr = nullptr;
   const hipError_t e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
   if (e != hipSuccess) return e;
   if (!ptr) return hipErrorInvalidSymbol;
-  g_scratch_ptr[device] = ptr;
+  g_scratch_ptr[device].store(ptr, std::memory_order_release);
   return hipSuccess;
 }
 
@@ -60,12 +64,14 @@ extern "C" mf_status mf_shared_expert_static(mf_ctx* ctx, mf_stream stream, cons
              static_cast<size_t>(t) * f, static_cast<unsigned>(MF_STATIC_ACT_ELEMS));
     return MF_ERR_SCRATCH_TOO_SMALL;
   }
-  if (ctx->device < 0 || ctx->device >= kMaxDevices || !g_scratch_ptr[ctx->device]) {
+  void* const scratch_ptr =
+      ctx->device >= 0 && ctx->device < kMaxDevices ? g_scratch_ptr[ctx->device].load(std::memory_order_acquire) : nullptr;
+  if (!scratch_ptr) {
     snprintf(ctx->hip_error, sizeof ctx->hip_error,
              "mf_shared_expert_static: the scratch array's address is unknown on device %d", ctx->device);
     return MF_ERR_LAUNCH;
   }
-  auto* act = static_cast<uint16_t*>(g_scratch_ptr[ctx->device]);
+  auto* act = static_cast<uint16_t*>(scratch_ptr);
   auto s = static_cast<hipStream_t>(stream);
   hipError_t e = mf::launch_gate_up_act(s, gate, up, bits, x, act, f, d, t);
   if (e == hipSuccess) e = mf::launch_gemv(s, down, bits, act, y, d, f, t, false);

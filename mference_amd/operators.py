@@ -174,13 +174,18 @@ class MPPPrefillInt4QMM:
             if self._ws is None or self._ws.numel() < need:
                 self._ws = torch.empty(max(need, 256), dtype=torch.uint8, device=x.device)
             workspace = self._ws
-        st = _capi.lib().mf_qmm(self.context.handle, _stream(stream), weights.c(), weights.bits, _ptr(x), _ptr(y),
-                                m, n, k, 1 if y.dtype == torch.float32 else 0, _ptr(workspace),
-                                workspace.numel() * workspace.element_size())
-        if st in (-1, -2, -3):
+        ws_bytes = workspace.numel() * workspace.element_size()
+        # the reference's guard conditions (MPPPrefillInt4QMM.swift:43-55) give "unavailable"; a path that
+        # ran is named for the kernel that ran it
+        path = _capi.lib().mf_qmm_path(weights.c(), weights.bits, _ptr(x), _ptr(y), m, n, k, _ptr(workspace), ws_bytes)
+        if path < 0:
             return "unavailable"
-        check(st, self.context.handle)
-        return "affine-matrix-core-bf16"
+        check(_capi.lib().mf_qmm(self.context.handle, _stream(stream), weights.c(), weights.bits, _ptr(x), _ptr(y),
+                                 m, n, k, 1 if y.dtype == torch.float32 else 0, _ptr(workspace), ws_bytes),
+              self.context.handle)
+        return self.PATHS[path]
+
+    PATHS = {1: "affine-matrix-core-bf16", 2: "affine-rows-gemv"}
 
 
 class Elementwise:
@@ -303,12 +308,15 @@ class FamilyRouters:
             _ptr(out_weights)), self.context.handle)
 
 
-def expert_blob_layout(d: int, f: int, bits: int = BITS_4, align: int = 256):
+def expert_blob_layout(d: int, f: int, bits: int = BITS_4, align: int = 256, repacked: bool = False):
     """(offsets, blob_bytes, stride) of one routed expert in the reference's blob order
-    (RepackPlanner.swift:544-712, ModelExpertIO.swift:20-35): mf_expert_blob_layout."""
+    (RepackPlanner.swift:544-712, ModelExpertIO.swift:20-35): mf_expert_blob_layout, or with
+    `repacked` mf_expert_blob_layout_repacked -- the byte layout of a packed_experts file, which for
+    ternary experts also carries the negated-scale bias tables (RepackPlanner.swift:619-640)."""
     off = ExpertOffsets()
     blob, stride = C.c_size_t(0), C.c_size_t(0)
-    check(_capi.lib().mf_expert_blob_layout(d, f, bits, align, C.byref(off), C.byref(blob), C.byref(stride)))
+    fn = _capi.lib().mf_expert_blob_layout_repacked if repacked else _capi.lib().mf_expert_blob_layout
+    check(fn(d, f, bits, align, C.byref(off), C.byref(blob), C.byref(stride)))
     return off, blob.value, stride.value
 
 

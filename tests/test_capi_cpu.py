@@ -59,6 +59,34 @@ def test_status_strings_and_bad_arguments():
     assert ei.value.name == "MF_ERR_DIMENSION_MISMATCH"
 
 
+def test_operator_shapes_are_checked_without_a_device():
+    """mf_moe_config_check: what mf_moe_create refuses, as a status (MoE.swift:165-167 traps instead).  The
+    full-softmax router ranks 32 experts per lane step, so an expert count that is no multiple of 32 is refused
+    in that mode -- the GPU tie tests skip exactly those parameters -- and accepted in the top-k softmax mode."""
+    lib = _capi.lib()
+
+    def status(**kw):
+        base = dict(d=256, f=128, num_experts=64, top_k=8, bits=4, router_mode=0, swiglu_limit=0.0, shared_f=0,
+                    shared_bits=4, maple_rounding=0, gate_group_size=0)
+        base.update(kw)
+        return lib.mf_moe_config_check(C.byref(_capi.MoEConfig(**base)))
+
+    assert status() == 0
+    assert lib.mf_moe_config_check(None) == -1
+    for e in (8, 16, 24, 33, 100, 168, 255):          # RouterTopKParityTests.swift:34 expert counts
+        assert status(num_experts=e, router_mode=0) == 0
+        assert status(num_experts=e, router_mode=1) == (0 if e % 32 == 0 else -1), e
+    for e in (32, 64, 128, 256):
+        assert status(num_experts=e, router_mode=1) == 0
+    assert status(d=100) == -2 and status(f=96) == -2 and status(shared_f=100) == -2
+    assert status(bits=3) == -3 and status(shared_f=64, shared_bits=8) == -3
+    assert status(num_experts=0) == -1 and status(num_experts=513) == -1
+    assert status(top_k=0) == -1 and status(top_k=9) == -1
+    assert status(router_mode=2) == -1 and status(maple_rounding=2) == -1
+    assert status(gate_group_size=32, bits=4) == -1 and status(gate_group_size=32, bits=2) == 0
+    assert status(gate_group_size=16, bits=2) == -1
+
+
 KAT_PAIRS = [(0, 3, 0, 10), (0, 1, 1, 11), (0, 4, 2, 12), (1, 1, 0, 13), (1, 3, 1, 14), (1, 2, 2, 15),
              (2, 4, 0, 16), (2, 3, 1, 17), (2, 1, 2, 18), (3, 5, 0, 19), (3, 1, 1, 20), (3, 4, 2, 21)]
 G = ops.PrefillMoEGrouping
@@ -190,3 +218,26 @@ def test_expert_blob_layout_matches_checker(d, f, bits):
     assert lib.mf_expert_blob_layout(128, 64, 3, 256, C.byref(o), None, None) == -3
     assert lib.mf_expert_blob_layout(128, 64, 4, 0, C.byref(o), None, None) == -1
     assert lib.mf_expert_blob_layout(128, 64, 4, 256, None, None, None) == -1
+
+
+@pytest.mark.parametrize("d,f", [(2048, 1024), (2048, 512), (256, 128)])
+def test_repacked_ternary_layout_is_the_file_layout(d, f):
+    """mf_expert_blob_layout_repacked against the blob a Maple packed_experts file holds (codes, scales and
+    the negated-scale bias tables of all three projections, RepackPlanner.swift:544-651), as
+    packed_experts.maple_expert_blob builds it from source tensors; 4-bit and 2-bit experts: both helpers agree."""
+    from mference_amd import packed_experts as pe
+    rng = np.random.default_rng(d + f)
+    mk = lambda rows, width: (rng.integers(0, 256, size=(rows, width // 4), dtype=np.uint8),
+                              rng.integers(0x3C00, 0x3E00, size=rows).astype(np.uint16))
+    blob, off_file, stride_file = pe.maple_expert_blob(mk(f, d), mk(f, d), mk(d, f), align=16384)
+    off, blob_bytes, stride = ops.expert_blob_layout(d, f, ops.BITS_TERNARY, 16384, repacked=True)
+    for name, _ in off._fields_:
+        assert getattr(off, name) == getattr(off_file, name), name
+    assert stride == stride_file == blob.size
+    assert blob_bytes == 3 * (d * f // 4) + 2 * 2 * (2 * f * (d // 64) + d * (f // 64))
+    compact = ops.expert_blob_layout(d, f, ops.BITS_TERNARY, 16384)
+    assert compact[1] < blob_bytes and compact[0].gate_b == 0
+    for bits in (ops.BITS_4, ops.BITS_2):
+        a, b = ops.expert_blob_layout(d, f, bits, 16384), ops.expert_blob_layout(d, f, bits, 16384, repacked=True)
+        assert (a[1], a[2]) == (b[1], b[2])
+        assert all(getattr(a[0], n) == getattr(b[0], n) for n, _ in a[0]._fields_)

@@ -94,8 +94,11 @@ def test_gemv_matches_oracle(gpu, oracle, bits, m, n, t):
     (4, 1280, 17408, 1),   # nine steps, split over waves when there are few rows
     (2, 1024, 8192, 1),    # 2-bit: 64 elements per 16 bytes
     (2, 1024, 4096, 4),
-    (4, 1056, 5120, 5),    # three or more token rows of a 4-bit matrix: the matrix-core kernel
-    (4, 1024, 17408, 8),   # ... with 16 K-splits per row block
+    (4, 1056, 5120, 5),    # five to eight token rows of a 4-bit matrix the quad kernel takes: rows 0..3, then the rest
+    (4, 1024, 17408, 8),
+    (4, 1056, 5184, 5),    # K not a multiple of 512: the 32x32x16 matrix-core kernel (K split over waves)
+    (4, 17408, 5120, 8),   # the dense MLP's projections at full size, the widest multi-token call
+    (4, 5120, 17408, 8),
 ])
 def test_gemv_streaming_rows_kernel(gpu, oracle, bits, m, n, t):
     """wide matrices take the streaming form (x slices resident in registers, rows walked by
@@ -112,11 +115,23 @@ def test_gemv_streaming_rows_kernel(gpu, oracle, bits, m, n, t):
     _sync()
     got = y32.cpu().numpy()
     assert np.abs(got - ref).max() / max(np.abs(ref).max(), 1e-6) < 2e-5
-    if t > 1:  # multi-token rows == single-token calls, bit for bit, when the row split is the same
+    # Multi-token rows against single-token calls (MultiXKernelParityTests.swift:50-77).  4-bit matrices with
+    # K a multiple of 512 run the quad kernel for every token count (five to eight rows as 4 + the rest), where
+    # a token's instructions do not depend on the others: bit for bit, every row.  The other wide shapes
+    # (2-bit, K not a multiple of 512) pick their split of a row over waves by the token count, so their
+    # rows agree with single-token calls to fp32 summation order only.
+    quad = bits == 4 and n % 512 == 0 and m % 4 == 0 and m >= 1024
+    for i in (range(t) if quad else range(min(t, 2))):
+        if t == 1:
+            break
         yi = torch.zeros((1, m), dtype=torch.float32, device="cuda")
-        g.encode(dq, xd[0:1].contiguous(), yi, m, n, 1, output_float32=True)
+        g.encode(dq, xd[i:i + 1].contiguous(), yi, m, n, 1, output_float32=True)
         _sync()
-        assert np.abs(yi.cpu().numpy()[0] - got[0]).max() / max(np.abs(ref).max(), 1e-6) < 2e-6
+        one = yi.cpu().numpy()[0]
+        if quad:
+            assert np.array_equal(one.view(np.uint32), got[i].view(np.uint32)), f"row {i} of {t}"
+        else:
+            assert np.abs(one - got[i]).max() / max(np.abs(ref).max(), 1e-6) < 2e-6
 
 
 @pytest.mark.parametrize("m,n,t", [
@@ -407,7 +422,7 @@ def test_routed_phases_over_slots_named_directly(gpu, oracle, bits, t):
     root = ROOT_SEED + 0x2F0 + bits
     layer = oracle.synth_layer(root, d, f, e, k, bits=bits, fs=0, router_mode=1 if bits == 1 else 0)
     x = oracle.synth_x(root, t, d)
-    _, ref_idx, ref_w = oracle.moe_layer(layer, x)
+    ref_y, ref_idx, ref_w = oracle.moe_layer(layer, x)
     moe = make_moe(gpu, layer)
     wts = to_device_layer(layer)
     xd = ops.bf16_tensor(x)
@@ -440,6 +455,24 @@ def test_routed_phases_over_slots_named_directly(gpu, oracle, bits, t):
     _sync()
     assert np.array_equal(ops.bf16_bits(acts1), ops.bf16_bits(acts0))
     assert np.array_equal(ops.bf16_bits(y1), ops.bf16_bits(y0))
+    # ... and, directly, the checker's layer (no shared expert, no residual: y = sum of the weighted routes)
+    assert_layer_close(oracle.bf16_to_float(ops.bf16_bits(y1)), oracle.bf16_to_float(ref_y), f"slots bits={bits}")
+    # a slab that starts 2 bytes into its allocation (all the reference promises) takes the byte-wise kernels
+    raw = torch.zeros(slab.numel() + 32, dtype=torch.uint8, device="cuda")
+    odd_slab = raw[2:2 + slab.numel()]
+    odd_slab.copy_(slab.reshape(-1))
+    acts_o = torch.zeros_like(acts0)
+    y_o = torch.zeros_like(y0)
+    moe.encode_routed_phase1_slots(odd_slab, so, wts.offsets, xd, acts_o, t=t, all_hit=hit)
+    moe.encode_routed_phase2_reduce_slots(odd_slab, so, wts.offsets, w, acts_o, None, y_o, t=t, all_hit=hit)
+    _sync()
+    assert np.array_equal(ops.bf16_bits(y_o), ops.bf16_bits(y0))
+    # refused without a launch: a slot stride that would break the 16-byte alignment of the blobs, and more
+    # rows than one lookup (one guard word) covers
+    with pytest.raises(_capi.MfError):
+        moe.encode_slot_lookup(idx, torch.from_numpy(slot_of).cuda(), stride + 8, so, hit, t=t)
+    with pytest.raises(_capi.MfError):
+        moe.encode_routed_phase1_slots(slab, so, wts.offsets, xd, acts1, t=ops.MAX_TOKENS + 1, all_hit=hit)
     # one routed expert loses its slot: the word reads 0 and the guarded launches leave their outputs alone
     gone = slot_of.copy()
     gone[used[0]] = -1
@@ -821,3 +854,60 @@ def test_single_expert_ffn_at_full_size(gpu, oracle):
         np.abs(oracle.bf16_to_float(ops.bf16_bits(acts).reshape(-1)) - oracle.bf16_to_float(ref_acts)).max() <= 2e-2
     ref_y = oracle.bf16_bits(oracle.expert_down(blob, ooff, 4, d, f, ref_acts))
     assert_layer_close(oracle.bf16_to_float(ops.bf16_bits(y2)[0]), oracle.bf16_to_float(ref_y), "single expert, routed form")
+
+
+@pytest.mark.parametrize("e", [64, 256])
+def test_fused_topk_on_non_finite_logits(gpu, oracle, e):
+    """top-k softmax router (mode 0) on logits that are NaN, +inf, -inf, mostly -inf (fewer finite ones than
+    routes) or all equal: NaN counts as -inf and is never picked, ranks nobody wins keep index 0 (the serial
+    selector of moe.metal:190-240).  The fused launch -- threshold prefilter, its fallback to a rank count over
+    all experts when more than 64 candidates tie, and the rank count itself -- gives the indices of the checker
+    and the indices AND weight bits of the chain of launches, for the four rows in one call and one at a time."""
+    d, f, k, t = 2 * e, 64, 8, 4
+    root = ROOT_SEED + 0x9A0 + e
+    layer = oracle.synth_layer(root, d, f, e, k, bits=4, fs=0)
+    rng = oracle.Rng.key(root, "taps")
+    a = oracle.bf16_bits(rng.normal(0.0, 1.0, e))
+    b = np.full(e, 0xFF80, np.uint16)                      # -inf ...
+    b[[1, e // 2, e - 2, 7, 11, 30, 40]] = oracle.bf16_bits(rng.normal(0.0, 1.0, 7))  # ... but k - 1 finite ones
+    a[3], a[5], a[9], a[e - 1] = 0x7FC0, 0x7F80, 0xFF80, 0x7F80   # NaN, +inf, -inf, +inf
+    rw = np.zeros((e, d), np.uint16)
+    rw[np.arange(e), np.arange(e)] = a                     # logit[e] = a[e] x[e] + b[e] x[E + e]
+    rw[np.arange(e), e + np.arange(e)] = b
+    layer.router_w = rw
+    one, zero = 0x3F80, 0
+    x = np.zeros((t, d), np.uint16)
+    x[0, :e] = one          # logits a: NaN and both infinities among ordinary scores
+    x[1, e:] = one          # logits b (+ 0 * a: NaN where a is not finite): k - 1 finite scores
+    x[2, :] = one           # a + b
+    x[3, :] = zero          # all logits 0 (NaN where a tap is not finite): every expert ties
+    ref_idx = np.stack([oracle.moe_layer(layer, x[i:i + 1])[1][0] for i in range(t)])
+    ref_w = np.stack([oracle.moe_layer(layer, x[i:i + 1])[2][0] for i in range(t)])
+    moe = make_moe(gpu, layer)
+    wts = to_device_layer(layer)
+    xd = ops.bf16_tensor(x)
+
+    def run(fused, rows):
+        moe.set_fused(fused)
+        n = len(rows)
+        y = torch.zeros((n, d), dtype=torch.bfloat16, device="cuda")
+        idx = torch.zeros((n, k), dtype=torch.int32, device="cuda")
+        w = torch.zeros((n, k), dtype=torch.float32, device="cuda")
+        moe.encode_decode_layer(wts, xd[rows].contiguous(), y, t=n, out_indices=idx, out_weights=w)
+        moe.status()
+        return idx.cpu().numpy().astype(np.uint32), w.cpu().numpy().view(np.uint32), ops.bf16_bits(y)
+
+    try:
+        chain = run(False, list(range(t)))
+        fused = run(True, list(range(t)))
+        assert np.array_equal(chain[0], ref_idx) and np.array_equal(fused[0], ref_idx)
+        finite = np.isfinite(ref_w)
+        assert np.array_equal(chain[1][finite], ref_w.view(np.uint32)[finite])
+        assert np.isnan(chain[1].view(np.float32)[~finite]).all()
+        for part in range(3):
+            assert np.array_equal(fused[part], chain[part]), ("indices", "weights", "outputs")[part]
+        for i in range(t):
+            one_row = run(True, [i])
+            assert np.array_equal(one_row[0][0], ref_idx[i]) and np.array_equal(one_row[1][0], fused[1][i])
+    finally:
+        moe.set_fused(True)

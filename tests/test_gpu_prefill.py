@@ -144,6 +144,46 @@ def test_prefill_layer_matches_per_token_oracle(gpu, oracle, bits, d, f, e, k, f
     assert np.array_equal(y, y2)
 
 
+_SKEWED = {}
+
+
+def _skewed_qwen_layer(oracle):
+    """the benchmark's layer: Qwen3.6-shaped, and a per-expert router bias ~ N(0, 1.5) carried by the last
+    router column against a constant-one last feature of x, so that expert loads are uneven and many experts
+    get no token"""
+    if not _SKEWED:
+        root = ROOT_SEED + 0xA000 + 0x5CE
+        layer = oracle.synth_layer(root, 2048, 512, 256, 8, bits=4, fs=512)
+        bias = oracle.Rng.key(root, "router.bias").normal(0.0, 1.5, 256)
+        layer.router_w[:, -1] = oracle.bf16_bits(bias)
+        _SKEWED["layer"] = layer
+        _SKEWED["root"] = root
+    return _SKEWED["layer"], _SKEWED["root"]
+
+
+@pytest.mark.parametrize("t", [128, 512, 2048])
+def test_skewed_qwen_prefill_against_the_checker(gpu, oracle, t):
+    """The headline prefill configuration at its three token counts, directly against the per-token checker:
+    routing indices and weights bit for bit on every row, the layer output within tolerance on 64 sampled rows
+    (the busiest expert takes most tokens here, so full 64-route tiles, ragged tails and experts without
+    tokens all occur in one call)."""
+    layer, root = _skewed_qwen_layer(oracle)
+    d, k = layer.d, layer.k
+    x = oracle.synth_x(root + t, t, d)
+    x[:, -1] = 0x3F80
+    moe = make_moe(gpu, layer)
+    wts = to_device_layer(layer)
+    y, idx, w = _run_prefill(moe, wts, x, t, d, k)
+    rows = np.unique(np.concatenate([np.arange(8), np.arange(t - 8, t),
+                                     np.random.default_rng(t).choice(t, size=48, replace=False)]))
+    ref_y, ref_idx, ref_w = oracle.moe_layer(layer, x[rows])
+    assert np.array_equal(idx[rows], ref_idx)
+    assert np.array_equal(w[rows].view(np.uint32), ref_w.view(np.uint32))
+    assert_layer_close(oracle.bf16_to_float(y[rows]), oracle.bf16_to_float(ref_y), f"skewed qwen prefill t={t}")
+    counts = np.bincount(idx.reshape(-1), minlength=layer.e)
+    assert (counts == 0).sum() > 0 and counts.max() > t // 2, "the routing of this case is meant to be skewed"
+
+
 @pytest.mark.parametrize("bits,d,f,e,k,fs,t,mode", [
     (4, 512, 256, 32, 8, 256, 1100, 0),    # 8800 routes, the shared expert rides along
     (4, 1024, 128, 16, 8, 0, 1031, 0),     # few experts: long runs, an odd tile out at the end of every run

@@ -13,11 +13,21 @@ from helpers import to_device_q
 pytestmark = pytest.mark.gpu
 
 
+def _ternary(oracle, rng, rows, cols):
+    u = rng.uniform_fill(0.0, 1.0, rows * cols).reshape(rows, cols)
+    codes = np.where(u < 0.25, 0, np.where(u < 0.75, 1, 2)).astype(np.uint8)
+    scales = oracle.bf16_bits(np.abs(rng.normal(0.0, 0.02, rows * (cols // 64))).reshape(rows, cols // 64) + 1e-3)
+    return oracle.QTensor(oracle.pack_codes(codes, 1), scales, None, 1, rows, cols)
+
+
 def _case(oracle, label, d, f, t, bits=4):
     rng = oracle.Rng.key(0xA110C, label)
-    gq = oracle.quantize(rng.normal(0.0, 0.02, f * d).reshape(f, d), bits)
-    uq = oracle.quantize(rng.normal(0.0, 0.02, f * d).reshape(f, d), bits)
-    dq = oracle.quantize(rng.normal(0.0, 0.02, d * f).reshape(d, f), bits)
+    if bits == 1:
+        gq, uq, dq = _ternary(oracle, rng, f, d), _ternary(oracle, rng, f, d), _ternary(oracle, rng, d, f)
+    else:
+        gq = oracle.quantize(rng.normal(0.0, 0.02, f * d).reshape(f, d), bits)
+        uq = oracle.quantize(rng.normal(0.0, 0.02, f * d).reshape(f, d), bits)
+        dq = oracle.quantize(rng.normal(0.0, 0.02, d * f).reshape(d, f), bits)
     x = oracle.bf16_bits(rng.normal(0.0, 1.0, t * d).reshape(t, d))
     return gq, uq, dq, x
 
@@ -45,6 +55,24 @@ def test_static_scratch_matches_shared_expert_twice(gpu, oracle):
     _run_both(gpu, oracle, "first-large", 2048, 1024, 4)
     _run_both(gpu, oracle, "second-small", 512, 256, 1)
     _run_both(gpu, oracle, "third-2bit", 1024, 512, 2, bits=2)
+    _run_both(gpu, oracle, "fourth-ternary", 512, 1024, 3, bits=1)
+
+
+def test_static_scratch_allocates_nothing(gpu, oracle):
+    """a run of calls leaves the device's free memory where it was: no hipMalloc / hipFree behind the entry point
+    (operands and outputs are allocated before the first reading)"""
+    gq, uq, dq, x = _case(oracle, "no-alloc", 1024, 512, 4)
+    g, u, dn, xd = to_device_q(gq), to_device_q(uq), to_device_q(dq), ops.bf16_tensor(x)
+    op = ops.SharedExpertInt4(gpu)
+    y = torch.zeros((4, 1024), dtype=torch.bfloat16, device="cuda")
+    op.encode_static(xd, g, u, dn, y, t=4)   # (first call on the device: whatever the runtime sets up lazily)
+    torch.cuda.synchronize()
+    free_before, _ = torch.cuda.mem_get_info()
+    for n in range(20):
+        op.encode_static(xd[:1 + n % 4], g, u, dn, y[:1 + n % 4], t=1 + n % 4)
+    torch.cuda.synchronize()
+    free_after, _ = torch.cuda.mem_get_info()
+    assert free_after == free_before, (free_before, free_after)
 
 
 def test_static_scratch_rejects_what_does_not_fit(gpu, oracle):

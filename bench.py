@@ -138,13 +138,13 @@ def layer_to_host(wts, w):
                    router_mode=1 if w["bits"] == 1 else 0, maple_rounding=bool(w.get("maple")))
 
 
-def profiled_traffic_bytes():
-    """HBM bytes per launch of the fused kernel from the committed rocprofv3 --pmc
-    summary (FETCH_SIZE + WRITE_SIZE, scaled by a copy kernel of known size)."""
+def profiled_traffic_bytes(name="fused_decode_qwen_t1.md", unit="launch"):
+    """HBM bytes per launch of the fused kernel (per layer call of the prefill) from the committed
+    rocprofv3 --pmc summary (FETCH_SIZE + WRITE_SIZE, scaled by a copy kernel of known size)."""
     import re
-    path = os.path.join(ROOT, "profiles", "fused_decode_qwen_t1.md")
+    path = os.path.join(ROOT, "profiles", name)
     try:
-        m = re.search(r"Traffic per launch = \*\*([0-9,]+) B\*\*", open(path).read())
+        m = re.search(r"Traffic per %s = \*\*([0-9,]+) B\*\*" % unit, open(path).read())
         return int(m.group(1).replace(",", "")) if m else None
     except OSError:
         return None
@@ -239,14 +239,24 @@ def measure_prefill(ctx, w, layer, device, tokens=(128, 512, 2048), steps=100, w
         us = e0.elapsed_time(e1) / (reps * per_graph) * 1e3
         flops = 2.0 * 3 * w["d"] * (t * w["k"] * w["f"] + t * w["fs"])
         tflops = flops / us / 1e6
+        # algorithmic bytes of the call: the experts that got a token + the shared expert + router, once each,
+        # the token rows in and out (the short batches are bound by these, not by the matrix cores)
+        ab = algorithmic_bytes(dict(w, experts_touched=int((counts > 0).sum()), t=t))
+        hbm_gbps = ab["total"] / us / 1e3
         run.update(us_per_layer=round(us, 1), tokens_per_s=round(t / us * 1e6, 1),
                    tflops=round(tflops, 1), mfma_frac=round(tflops / MFMA_BF16_PEAK_TFLOPS, 4),
+                   algorithmic_bytes=int(ab["total"]), hbm_gbps=round(hbm_gbps, 1),
+                   hbm_frac=round(hbm_gbps / HBM_PEAK_GBPS, 4),
                    experts_without_tokens=int((counts == 0).sum()), max_expert_load=int(counts.max()),
                    output_finite=bool(torch.isfinite(y.float()).all().item()))
         out["runs"].append(run)
     last = out["runs"][-1]
     out["roofline"] = {"bound": "mfma", "achieved": last["tflops"], "peak": MFMA_BF16_PEAK_TFLOPS,
-                       "unit": "TFLOP/s", "frac": last["mfma_frac"], "traffic": None,
+                       "unit": "TFLOP/s", "frac": last["mfma_frac"],
+                       "traffic": profiled_traffic_bytes("prefill_qmm_qwen_t2048.md", "layer") if qwen and last["tokens"] == 2048 else None,
+                       "traffic_source": "rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE summary committed as "
+                                         "profiles/prefill_qmm_qwen_t2048.md (all launches of one layer call at T=2048; a "
+                                         "constant of that profile run, not measured by this run)",
                        "kernel": "whole layer at T=%d (router, grouping, mf::qmm_kernel, mf::qmm_kres_kernel, reduce); "
                                  "algorithmic flops = 2*3*D*(T*K*F + T*Fs)" % last["tokens"]}
     return out
@@ -398,8 +408,13 @@ def bench_dense_mlp(args, device) -> int:
     step()
     torch.cuda.synchronize()
     rows = list(range(t)) if t <= 8 else sorted({0, 1, t // 2, t - 1})  # the checker takes ~1 s per row
-    ref = np.stack([O.shared_expert(hq(sets[0][0]), hq(sets[0][1]), hq(sets[0][2]), ops.bf16_bits(x[i]))
-                    for i in rows])
+    h0 = [hq(q) for q in sets[0]]
+    t_cpu = time.perf_counter()
+    ref = np.stack([O.shared_expert(h0[0], h0[1], h0[2], ops.bf16_bits(x[i])) for i in rows])
+    cpu_us_per_row = (time.perf_counter() - t_cpu) / len(rows) * 1e6
+    cores = int(os.environ.get("OMP_NUM_THREADS") or min(16, os.cpu_count() or 1))
+    cpu_baseline = {"value": round(cpu_us_per_row * t, 1), "unit": "us", "cores": cores, "kind": "port",
+                    "sample": f"{len(rows)} token rows of weight set 0 through the CPU checker, scaled to {t} rows"}
     got = O.bf16_to_float(ops.bf16_bits(y[0][rows])).astype(np.float64)
     reff = O.bf16_to_float(ref).astype(np.float64)
     parity = dict(max_abs=float(np.abs(got - reff).max()),
@@ -435,6 +450,7 @@ def bench_dense_mlp(args, device) -> int:
             "dtype": "u4 codes x bf16 activations, fp32 accumulate", "data": "synthetic (N(0,0.02) weights, 4-bit g64)",
             "config": {"workload": w["name"] + "-T%d" % t, "weight_sets": L, "tokens": t, "launch": "hip_graph"},
             "tokens_per_s": round(t / (us * 1e-6), 1), "parity_set0_rows": rows, "parity_set0": parity,
+            "cpu_baseline": cpu_baseline,
             "hbm_gbps_weight_bytes": round(achieved, 1),
             "roofline": {"bound": "mfma", "achieved": round(tflops, 1), "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
                          "frac": round(tflops / MFMA_BF16_PEAK_TFLOPS, 4), "traffic": None,
@@ -447,10 +463,10 @@ def bench_dense_mlp(args, device) -> int:
         "higher_is_better": False, "scaling": "weak", "vs_baseline": None,
         "dtype": "u4 codes x bf16 activations, fp32 accumulate", "data": "synthetic (N(0,0.02) weights, 4-bit g64)",
         "config": {"workload": w["name"] + "-T%d" % t, "weight_sets": L, "tokens": t, "launch": "hip_graph"},
-        "parity_set0": parity,
+        "parity_set0": parity, "cpu_baseline": cpu_baseline,
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                      "frac": round(achieved / HBM_PEAK_GBPS, 4), "traffic": None,
-                     "kernel": "mf::gate_up_act_kernel + mf::gemv_kernel", "algorithmic_bytes": nbytes}}))
+                     "kernel": "mf::rows_quad_kernel (gate/up + activation, then down)", "algorithmic_bytes": nbytes}}))
     return 0
 
 
@@ -720,6 +736,49 @@ def phase_trace(ctx, w, stack, moes, device) -> int:
     return 0
 
 
+OTHER_CONFIGS = [
+    # (key, BASELINE.json configuration, extra arguments of this script)
+    ("single_expert_ffn_T1", 0, ["--workload", "single-expert", "--steps", "20", "--warmup", "5"]),
+    ("large_2bit_layer_T1", 3, ["--workload", "dsv4-2bit", "--steps", "100", "--warmup", "10"]),
+    ("large_2bit_layer_T4", 3, ["--workload", "dsv4-2bit", "--tokens", "4", "--steps", "100", "--warmup", "10"]),
+    ("ternary_layer_T1", 4, ["--workload", "maple-ternary", "--steps", "100", "--warmup", "10"]),
+    ("dense_mlp_T1", 4, ["--workload", "dense-mlp", "--steps", "50", "--warmup", "10"]),
+    ("dense_mlp_T4", 4, ["--workload", "dense-mlp", "--tokens", "4", "--steps", "50", "--warmup", "10"]),
+]
+
+
+def measure_other_configs(cpu_seconds: float, budget_s: float = 400.0) -> dict:
+    """The remaining BASELINE.json configurations, each measured by this script in a child process of its
+    own (one GPU, one after the other, after the headline's timed region) and reduced to a few fields:
+    time, algorithmic bytes, achieved rate and fraction of the HBM peak, parity against the CPU checker
+    and the checker's own time."""
+    import subprocess
+    out, t_start = {}, time.perf_counter()
+    for key, cfg, extra in OTHER_CONFIGS:
+        if time.perf_counter() - t_start > budget_s:
+            out[key] = {"skipped": "time budget of the default run"}
+            continue
+        cmd = [sys.executable, os.path.abspath(__file__), "--gpus", "1", "--no-prefill", "--no-other-configs",
+               "--cpu-seconds", str(cpu_seconds)] + extra
+        try:
+            proc = subprocess.run(cmd, capture_output=True, text=True, timeout=240)
+            line = [l for l in proc.stdout.splitlines() if l.startswith("{")][-1]
+            r = json.loads(line)
+        except Exception as exc:  # a configuration that fails says so and does not take the headline down
+            out[key] = {"error": repr(exc)[:200]}
+            continue
+        roof = r.get("roofline", {})
+        entry = {"baseline_config": cfg, "workload": r["config"]["workload"], "us": r["value"],
+                 "algorithmic_bytes": roof.get("algorithmic_bytes_per_layer", roof.get("algorithmic_bytes")),
+                 "achieved_gbps": roof.get("achieved"), "hbm_frac": roof.get("frac"),
+                 "parity": r.get("parity_layer0", r.get("parity_set0")), "kernel": roof.get("kernel")}
+        for k in ("cpu_baseline", "cpu_baseline_single_thread"):
+            if k in r:
+                entry[k] = {f: r[k][f] for f in ("value", "unit", "cores")}
+        out[key] = entry
+    return out
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -738,6 +797,8 @@ def main() -> int:
                          "traffic) so that FETCH_SIZE / WRITE_SIZE counters can be scaled")
     ap.add_argument("--cpu-seconds", type=float, default=12.0)
     ap.add_argument("--no-prefill", action="store_true", help="skip the ragged prefill section")
+    ap.add_argument("--no-other-configs", action="store_true",
+                    help="skip the short runs of the other BASELINE configurations that the default run appends")
     ap.add_argument("--prefill-only", action="store_true",
                     help="one layer, the ragged prefill section only (for profiling)")
     ap.add_argument("--phase-trace", action="store_true",
@@ -938,6 +999,11 @@ def main() -> int:
                                                  "kind": "port", "sample": f"{n1} repetitions of layer 0, one thread"}
     if args.pmc_calibration:
         out["pmc_calibration"] = pmc_calibration(device)
+    if args.workload == "qwen-decode" and not args.tokens and not args.no_other_configs and not args.layers:
+        # free the stack first: the children build their own weights on the same GPU
+        del stack, moes, graph, run
+        torch.cuda.empty_cache()
+        out["other_configs"] = measure_other_configs(cpu_seconds=min(args.cpu_seconds, 2.0))
     print(json.dumps(out))
     return 0
 

@@ -16,7 +16,8 @@ __global__ __launch_bounds__(256) void quantize_kernel(const float* __restrict__
                                                        uint8_t* __restrict__ packed,
                                                        uint16_t* __restrict__ scales,
                                                        uint16_t* __restrict__ biases) {
-  constexpr int kQMax = (BITS == kBits4) ? 15 : 3;
+  constexpr int kQMax = (BITS == kBits8) ? 255 : (BITS == kBits4) ? 15 : 3;  // 8-bit: Quantization.swift:135-176
+  constexpr int kCodeBits = (BITS == kBits8) ? 8 : Store<BITS>::kBits;
   const size_t g = (static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x) >> 4;
   const int l16 = threadIdx.x & 15;
   const bool live = g < n_groups;
@@ -56,14 +57,18 @@ __global__ __launch_bounds__(256) void quantize_kernel(const float* __restrict__
     const float t = (v[i] - bias) * inv;
     const float rq = __builtin_roundf(t);  // Swift .rounded(): half away from zero
     const int q = rq >= static_cast<float>(kQMax) ? kQMax : (rq <= 0.0f ? 0 : static_cast<int>(rq));
-    code |= static_cast<uint32_t>(q) << (Store<BITS>::kBits * i);
+    code |= static_cast<uint32_t>(q) << (kCodeBits * i);
   }
   if (!live) return;
   if (l16 == 0) {
     scales[g] = sb;
     biases[g] = bb;
   }
-  if constexpr (BITS == kBits4) {
+  if constexpr (BITS == kBits8) {
+    uint8_t* o = packed + g * 64 + l16 * 4;  // (2-byte aligned at least: written as two halves)
+    *reinterpret_cast<uint16_t*>(o) = static_cast<uint16_t>(code);
+    *reinterpret_cast<uint16_t*>(o + 2) = static_cast<uint16_t>(code >> 16);
+  } else if constexpr (BITS == kBits4) {
     *reinterpret_cast<uint16_t*>(packed + g * 32 + l16 * 2) = static_cast<uint16_t>(code);
   } else {
     packed[g * 16 + l16] = static_cast<uint8_t>(code);
@@ -84,13 +89,20 @@ __global__ __launch_bounds__(256) void dequantize_kernel(const uint8_t* __restri
   const float s = bf16_to_f(scales[g]);
   const float b = (BITS == kBitsTernary) ? -s : bf16_to_f(biases[g]);
   uint32_t w;
-  if constexpr (BITS == kBits4) {
+  if constexpr (BITS == kBits8) {  // a byte per code (Quantization.swift:179-190)
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      const float prod = static_cast<float>(packed[e0 + i]) * s;
+      out[e0 + i] = prod + b;
+    }
+    return;
+  } else if constexpr (BITS == kBits4) {
     w = load_u32_bytes(packed + e0 / 2);
   } else {
     const uint8_t* p = packed + e0 / 4;
     w = static_cast<uint32_t>(p[0]) | (static_cast<uint32_t>(p[1]) << 8);
   }
-  constexpr int kW = Store<BITS>::kBits;
+  constexpr int kW = BITS == kBits8 ? 8 : Store<BITS>::kBits;
   constexpr uint32_t kMask = (1u << kW) - 1u;
 #pragma unroll
   for (int i = 0; i < 8; ++i) {
@@ -106,7 +118,10 @@ hipError_t launch_quantize(hipStream_t s, const float* w, size_t rows, size_t n,
   if (n_groups == 0) return hipSuccess;
   const size_t blocks = (n_groups * 16 + 255) / 256;
   auto* p = static_cast<uint8_t*>(packed);
-  if (bits == kBits4)
+  if (bits == kBits8)
+    quantize_kernel<kBits8><<<dim3(static_cast<uint32_t>(blocks)), dim3(256), 0, s>>>(
+        w, n_groups, p, scales, biases);
+  else if (bits == kBits4)
     quantize_kernel<kBits4><<<dim3(static_cast<uint32_t>(blocks)), dim3(256), 0, s>>>(
         w, n_groups, p, scales, biases);
   else
@@ -122,7 +137,9 @@ hipError_t launch_dequantize(hipStream_t s, const mf_qtensor& q, size_t rows, si
   const size_t blocks = (n_elems / 8 + 255) / 256;
   const auto* p = static_cast<const uint8_t*>(q.weights);
   const dim3 grid(static_cast<uint32_t>(blocks)), block(256);
-  if (bits == kBits4)
+  if (bits == kBits8)
+    dequantize_kernel<kBits8><<<grid, block, 0, s>>>(p, q.scales, q.biases, n_elems, out);
+  else if (bits == kBits4)
     dequantize_kernel<kBits4><<<grid, block, 0, s>>>(p, q.scales, q.biases, n_elems, out);
   else if (bits == kBits2)
     dequantize_kernel<kBits2><<<grid, block, 0, s>>>(p, q.scales, q.biases, n_elems, out);

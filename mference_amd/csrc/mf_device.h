@@ -14,7 +14,7 @@ namespace mf {
 constexpr int kWave = 64;    // gfx950 wavefront
 constexpr int kGroup = 64;   // quantization group (Quantization.swift:5)
 
-enum : int { kBitsTernary = 1, kBits2 = 2, kBits4 = 4 };
+enum : int { kBitsTernary = 1, kBits2 = 2, kBits4 = 4, kBits8 = 8 };  // 8: GEMV, quantizer and scalar gate only
 
 // elements covered by one 16-byte load of packed codes
 template <int BITS> struct Fmt { static constexpr int kElemsPer16B = (BITS == kBits4) ? 32 : 64; };

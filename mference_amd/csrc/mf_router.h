@@ -54,6 +54,45 @@ __device__ __forceinline__ float dot_bf16_row(const uint16_t* __restrict__ w,
   return wave_sum(acc);
 }
 
+// The same for a row of 8-bit affine codes (dequant_int8_gemv_simd, Metal/Quant/dequant_int8.metal:66-107:
+// w = q * scale + bias per group of 64, fma(s, sum q x, acc), fma(b, sum x, acc)): chunk c of 8 codes
+// belongs to lane c % 64 and lies inside one group; its sum q*x and sum x are built in ascending order
+// from 0 and enter the lane's accumulator as the two fmas; lanes combine neighbours first.
+__device__ __forceinline__ float dot_q8_row(const uint8_t* __restrict__ q_row, const uint16_t* __restrict__ s_row,
+                                            const uint16_t* __restrict__ b_row, const uint16_t* __restrict__ x,
+                                            uint32_t d, uint32_t lane, bool aligned) {
+  float acc = 0.0f;
+  for (uint32_t c = lane; c < d / 8; c += kWave) {
+    uint32_t q[2];
+    uint4 xv;
+    if (aligned) {
+      const uint2 qq = *reinterpret_cast<const uint2*>(q_row + c * 8);
+      q[0] = qq.x; q[1] = qq.y;
+      xv = load_x8<true>(x + c * 8);
+    } else {
+      const uint8_t* p = q_row + c * 8;
+      q[0] = p[0] | (p[1] << 8) | (p[2] << 16) | (static_cast<uint32_t>(p[3]) << 24);
+      q[1] = p[4] | (p[5] << 8) | (p[6] << 16) | (static_cast<uint32_t>(p[7]) << 24);
+      xv = load_x8<false>(x + c * 8);
+    }
+    const uint32_t xs[4] = {xv.x, xv.y, xv.z, xv.w};
+    float dot = 0.0f, sum = 0.0f;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const float x0 = bf16_lo(xs[j]), x1 = bf16_hi(xs[j]);
+      const uint32_t word = q[j >> 1] >> ((j & 1) * 16);
+      dot = __builtin_fmaf(static_cast<float>(word & 0xFFu), x0, dot);
+      sum = sum + x0;
+      dot = __builtin_fmaf(static_cast<float>((word >> 8) & 0xFFu), x1, dot);
+      sum = sum + x1;
+    }
+    const uint32_t g = c * 8 / MF_GROUP_SIZE;
+    acc = __builtin_fmaf(bf16_to_f(s_row[g]), dot, acc);
+    acc = __builtin_fmaf(bf16_to_f(b_row[g]), sum, acc);
+  }
+  return wave_sum(acc);
+}
+
 constexpr int kMaxPerLane = MF_MAX_EXPERTS / kWave;  // 8
 constexpr uint32_t kNoWinner = 0xFFFFFFFFu;
 

@@ -68,7 +68,11 @@ typedef enum {
 typedef enum {
   MF_BITS_TERNARY = 1, /* 2-bit codes {0,1,2}, bf16 scale per 64, bias = -scale */
   MF_BITS_2 = 2,       /* 2-bit affine: 16 codes per uint32, element j at bit 2*(j%16) */
-  MF_BITS_4 = 4        /* 4-bit affine: 8 codes per uint32, element j at bit 4*(j%8)   */
+  MF_BITS_4 = 4,       /* 4-bit affine: 8 codes per uint32, element j at bit 4*(j%8)   */
+  MF_BITS_8 = 8        /* 8-bit affine, a byte per code (Metal/Quant/dequant_int8.metal:5-13): accepted by
+                          mf_quantize_affine, mf_dequantize and mf_gemv, and as the format of the scalar
+                          shared gate (mf_moe_layer_weights.w_sg_q8); the experts, the shared expert and
+                          mf_qmm take the three formats above */
 } mf_bits;
 
 typedef enum {
@@ -424,6 +428,12 @@ typedef struct {
   mf_expert_offsets offsets;
   mf_qtensor shared_gate, shared_up, shared_down; /* used when shared_f > 0 */
   const uint16_t* w_sg;       /* bf16 [d] scalar shared gate, or NULL */
+  mf_qtensor w_sg_q8;         /* the scalar shared gate as the reference's model files store it: 8-bit affine
+                               * [1, d] with bf16 scale / bias per 64 (DequantInt8GEMV on sharedProj.scalarGate,
+                               * Runtime/Inference/RealForwardRunner.swift:2925-2941; dequant_int8_gemv_simd,
+                               * Metal/Quant/dequant_int8.metal:66-107).  Used when w_sg_q8.weights != NULL
+                               * (w_sg is then ignored); all three pointers zero: w_sg decides.  The gate
+                               * logit is the mf_gemv(MF_BITS_8) value of that row, narrowed to bf16. */
 } mf_moe_layer_weights;
 
 /* The fused decode layer, one launch: router -> top-k -> routed gate/up/act ->

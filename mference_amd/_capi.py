@@ -17,7 +17,7 @@ MAX_TOPK = 8
 MAX_EXPERTS = 512
 STATIC_ACT_ELEMS = MAX_TOKENS * 32768  # MF_STATIC_ACT_ELEMS
 
-BITS_TERNARY, BITS_2, BITS_4 = 1, 2, 4
+BITS_TERNARY, BITS_2, BITS_4, BITS_8 = 1, 2, 4, 8
 ROUTER_TOPK_SOFTMAX, ROUTER_FULL_SOFTMAX = 0, 1
 
 STATUS_NAMES = {
@@ -56,6 +56,7 @@ class LayerWeights(C.Structure):
         ("offsets", ExpertOffsets),
         ("shared_gate", QTensor), ("shared_up", QTensor), ("shared_down", QTensor),
         ("w_sg", C.c_void_p),
+        ("w_sg_q8", QTensor),
     ]
 
 

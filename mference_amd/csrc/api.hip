@@ -27,6 +27,8 @@ mf_status fail_hip(mf_ctx* ctx, hipError_t e, const char* what) {
   } while (0)
 
 bool bits_ok(int bits) { return bits == MF_BITS_4 || bits == MF_BITS_2 || bits == MF_BITS_TERNARY; }
+// the calls that also take 8-bit affine tensors: quantizer, dequantizer, GEMV
+bool bits_ok_rows(int bits) { return bits_ok(bits) || bits == MF_BITS_8; }
 
 bool qtensor_ok(const mf_qtensor& q, int bits) {
   if (!q.weights || !q.scales || !mf::aligned2(q.scales)) return false;
@@ -103,7 +105,7 @@ mf_status mf_quantize_affine(mf_ctx* ctx, mf_stream stream, const float* w, size
                              size_t n, mf_bits bits, void* packed, uint16_t* scales,
                              uint16_t* biases) {
   if (!ctx || !w || !packed || !scales || !biases) return MF_ERR_INVALID_ARGUMENT;
-  if (bits != MF_BITS_4 && bits != MF_BITS_2) return MF_ERR_UNSUPPORTED_BITS;
+  if (bits != MF_BITS_4 && bits != MF_BITS_2 && bits != MF_BITS_8) return MF_ERR_UNSUPPORTED_BITS;
   if (n % MF_GROUP_SIZE != 0) return MF_ERR_INVALID_ARGUMENT;
   if (!mf::aligned16(w) || !mf::aligned2(packed) || !mf::aligned2(scales) || !mf::aligned2(biases))
     return MF_ERR_INVALID_ARGUMENT;
@@ -115,7 +117,7 @@ mf_status mf_quantize_affine(mf_ctx* ctx, mf_stream stream, const float* w, size
 mf_status mf_dequantize(mf_ctx* ctx, mf_stream stream, mf_qtensor q, size_t rows, size_t n,
                         mf_bits bits, float* out) {
   if (!ctx || !out) return MF_ERR_INVALID_ARGUMENT;
-  if (!bits_ok(bits)) return MF_ERR_UNSUPPORTED_BITS;
+  if (!bits_ok_rows(bits)) return MF_ERR_UNSUPPORTED_BITS;
   if (!qtensor_ok(q, bits) || n % MF_GROUP_SIZE != 0) return MF_ERR_INVALID_ARGUMENT;
   MF_HIP(ctx, mf::launch_dequantize(static_cast<hipStream_t>(stream), q, rows, n, bits, out));
   return MF_OK;
@@ -126,7 +128,7 @@ mf_status mf_dequantize(mf_ctx* ctx, mf_stream stream, mf_qtensor q, size_t rows
 mf_status mf_gemv(mf_ctx* ctx, mf_stream stream, mf_qtensor w, mf_bits bits, const uint16_t* x,
                   void* y, uint32_t m, uint32_t n, uint32_t t, int out_f32) {
   if (!ctx || !x || !y) return MF_ERR_INVALID_ARGUMENT;
-  if (!bits_ok(bits)) return MF_ERR_UNSUPPORTED_BITS;
+  if (!bits_ok_rows(bits)) return MF_ERR_UNSUPPORTED_BITS;
   if (!qtensor_ok(w, bits) || !mf::aligned2(x) || !mf::aligned2(y)) return MF_ERR_INVALID_ARGUMENT;
   if (n == 0 || n % MF_GROUP_SIZE != 0 || t == 0 || t > MF_MAX_TOKENS)
     return MF_ERR_INVALID_ARGUMENT;
@@ -595,6 +597,7 @@ mf_status mf_moe_decode_layer(mf_moe* h, mf_stream stream, const mf_moe_layer_we
                      !qtensor_ok(wts->shared_up, c.shared_bits) ||
                      !qtensor_ok(wts->shared_down, c.shared_bits)))
     return MF_ERR_INVALID_ARGUMENT;
+  if (c.shared_f && wts->w_sg_q8.weights && !qtensor_ok(wts->w_sg_q8, MF_BITS_8)) return MF_ERR_INVALID_ARGUMENT;
   auto s = static_cast<hipStream_t>(stream);
   if (h->fused && mf::fused_supported(*h, *wts, x, y, hidden, t)) {
     MF_HIP(h->ctx, mf::launch_fused_decode(s, *h, *wts, x, t, y, hidden, out_idx, out_w));
@@ -614,7 +617,10 @@ mf_status mf_moe_decode_layer(mf_moe* h, mf_stream stream, const mf_moe_layer_we
                                           h->ws.shared_act, c.shared_f, c.d, t, true));
     MF_HIP(h->ctx, mf::launch_gemv(s, wts->shared_down, c.shared_bits, h->ws.shared_act,
                                    h->ws.shared_y, c.d, c.shared_f, t, false, true));
-    if (wts->w_sg) {
+    if (wts->w_sg_q8.weights) {  // the gate as the model files store it: an 8-bit row (RealForwardRunner.swift:2925-2941)
+      MF_HIP(h->ctx, mf::launch_gemv(s, wts->w_sg_q8, MF_BITS_8, x, h->ws.gate, 1, c.d, t, false));
+      MF_HIP(h->ctx, mf::launch_sigmoid_scalar_mul(s, h->ws.shared_y, h->ws.gate, c.d, t));
+    } else if (wts->w_sg) {
       MF_HIP(h->ctx, mf::launch_router_logits(s, wts->w_sg, x, 1, c.d, t, c.d, nullptr, h->ws.gate));
       MF_HIP(h->ctx, mf::launch_sigmoid_scalar_mul(s, h->ws.shared_y, h->ws.gate, c.d, t));
     }
@@ -731,8 +737,10 @@ mf_status mf_moe_prefill_layer(mf_moe* h, mf_stream stream, const mf_moe_layer_w
                      !qtensor_ok(wts->shared_up, c.shared_bits) ||
                      !qtensor_ok(wts->shared_down, c.shared_bits) ||
                      !mf::aligned16(wts->shared_gate.weights) || !mf::aligned16(wts->shared_up.weights) ||
-                     !mf::aligned16(wts->shared_down.weights) || (wts->w_sg && !mf::aligned16(wts->w_sg))))
+                     !mf::aligned16(wts->shared_down.weights) ||
+                     (wts->w_sg && !wts->w_sg_q8.weights && !mf::aligned16(wts->w_sg))))
     return MF_ERR_INVALID_ARGUMENT;
+  if (c.shared_f && wts->w_sg_q8.weights && !qtensor_ok(wts->w_sg_q8, MF_BITS_8)) return MF_ERR_INVALID_ARGUMENT;
   MF_HIP(h->ctx, mf::launch_prefill_layer(static_cast<hipStream_t>(stream), *h, *wts, x, t, y, workspace,
                                           out_idx, out_w));
   return MF_OK;

@@ -7,6 +7,7 @@
 // butterfly.
 #include "mf_device.h"
 #include "mf_internal.h"
+#include "mf_router.h"
 
 #pragma clang fp contract(off)
 
@@ -715,6 +716,26 @@ __global__ void residual_add_kernel(uint16_t* hidden, const uint16_t* delta, uin
   hidden[i] = f_to_bf16(bf16_to_f(hidden[i]) + bf16_to_f(delta[i]));
 }
 
+// 8-bit affine rows (dequant_int8_gemv_simd, Metal/Quant/dequant_int8.metal:66-107): one wave per
+// (token, row) in the lane order of dot_q8_row, so a token's value does not depend on how many tokens ride along.
+__global__ __launch_bounds__(256) void gemv_q8_kernel(const uint8_t* __restrict__ W, const uint16_t* __restrict__ S,
+                                                      const uint16_t* __restrict__ B, const uint16_t* __restrict__ x,
+                                                      void* __restrict__ y, uint32_t m, uint32_t n, uint32_t t,
+                                                      int out_f32, int aligned) {
+  const uint32_t lane = threadIdx.x & 63;
+  const uint32_t wave = (blockIdx.x * blockDim.x + threadIdx.x) >> 6;
+  if (wave >= m * t) return;
+  const uint32_t tok = wave / m, row = wave % m;
+  const uint32_t ng = n / kGroup;
+  const float v = dot_q8_row(W + static_cast<size_t>(row) * n, S + static_cast<size_t>(row) * ng,
+                             B + static_cast<size_t>(row) * ng, x + static_cast<size_t>(tok) * n, n, lane, aligned != 0);
+  if (lane == 0) {
+    const size_t at = static_cast<size_t>(tok) * m + row;
+    if (out_f32) static_cast<float*>(y)[at] = v;
+    else static_cast<uint16_t*>(y)[at] = f_to_bf16(v);
+  }
+}
+
 namespace {
 
 template <int BITS, bool ALIGNED>
@@ -879,6 +900,15 @@ bool rows_quad_try(hipStream_t s, const RowsQuadArgs& a, uint32_t num_cu, hipErr
 
 hipError_t launch_gemv(hipStream_t s, const mf_qtensor& w, int bits, const uint16_t* x, void* y,
                        uint32_t m, uint32_t n, uint32_t t, bool out_f32, bool lane_order) {
+  if (bits == kBits8) {  // one wave per (token, row); any number of token rows
+    const uint64_t waves = static_cast<uint64_t>(m) * t;
+    if (!waves) return hipSuccess;
+    if (waves >= (1ull << 30)) return hipErrorInvalidValue;
+    const int al8 = (reinterpret_cast<uintptr_t>(w.weights) % 8 == 0) && n % 8 == 0 && aligned16(x);
+    gemv_q8_kernel<<<dim3(static_cast<uint32_t>((waves + 3) / 4)), dim3(256), 0, s>>>(
+        static_cast<const uint8_t*>(w.weights), w.scales, w.biases, x, y, m, n, t, out_f32 ? 1 : 0, al8);
+    return hipGetLastError();
+  }
   const bool al = aligned16(w.weights) && aligned16(x);
   if (!lane_order && al && bits == kBits4 && aligned16(w.scales) && aligned16(w.biases)) {
     RowsMfmaArgs ma{};

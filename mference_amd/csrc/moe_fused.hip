@@ -155,6 +155,10 @@ struct FusedArgs {
   mf_expert_offsets off;
   mf_qtensor sg, su, sd;
   const uint16_t* w_sg;
+  // the scalar gate as 8-bit affine codes [1, D] with its scale / bias tables (null: w_sg, or no gate)
+  const uint8_t* gq_w;
+  const uint16_t* gq_s;
+  const uint16_t* gq_b;
   const uint16_t* x;
   uint16_t* y;
   uint16_t* hidden;
@@ -315,14 +319,15 @@ __global__ __launch_bounds__(kFusedThreads) void fused_decode_kernel(const Fused
       if (ci + G < n_rc) __syncthreads();  // the staging words are reused
     }
     const uint32_t skip = n_rc < G ? n_rc : 0;  // workgroups [0, skip) had router rows
-    const uint32_t n_gate = (Fs && a.w_sg) ? T : 0;
+    const uint32_t n_gate = (Fs && (a.w_sg || a.gq_w)) ? T : 0;
     const uint32_t srg = Fs ? (Fs + rpw - 1) / rpw : 0;
     const uint32_t n_items = n_gate + T * srg;
     const uint32_t Gs = G - skip;
     for (uint32_t item = wg >= skip ? wv * Gs + (wg - skip) : n_items; item < n_items; item += kFusedWaves * Gs) {
       if (item < n_gate) {
         const uint32_t tok = item;
-        const float v = dot_bf16_row(a.w_sg, a.x + static_cast<size_t>(tok) * D, D, lane, true);
+        const float v = a.gq_w ? dot_q8_row(a.gq_w, a.gq_s, a.gq_b, a.x + static_cast<size_t>(tok) * D, D, lane, true)
+                               : dot_bf16_row(a.w_sg, a.x + static_cast<size_t>(tok) * D, D, lane, true);
         if (lane < 4)  // the gate rides behind the token's shared activations
           store_u32_agent(&a.t_sact[static_cast<size_t>(tok) * sact_stride + Fs + lane],
                           (lane == 0 ? static_cast<uint32_t>(f_to_bf16(v)) : 0u) | (epoch_now() << 16));
@@ -620,7 +625,8 @@ __global__ __launch_bounds__(kFusedThreads) void fused_decode_kernel(const Fused
     // one round trip, during which the routed words are still on their way anyway) and the few
     // waves that own the shared-expert down rows compute the gated shared output h1 while the
     // rest of the workgroup polls for the routed words -- h1 leaves the critical path.
-    const uint32_t n_a = K * F, n_s = Fs ? (a.w_sg ? Fs + 4 : Fs) : 0;
+    const bool gated = a.w_sg || a.gq_w;
+    const uint32_t n_a = K * F, n_s = Fs ? (gated ? Fs + 4 : Fs) : 0;
     const AgentBuf ba = make_agent_buf(a.t_acts + static_cast<size_t>(tok) * n_a);
     const AgentBuf bs = make_agent_buf(a.t_sact + static_cast<size_t>(tok) * sact_stride);
     const uint32_t want = tag16 << 16;
@@ -658,7 +664,7 @@ __global__ __launch_bounds__(kFusedThreads) void fused_decode_kernel(const Fused
     // gated shared output h1 of the output rows this workgroup owns for this token; waves
     // [0, nw) share the rows
     auto shared_rows = [&](uint32_t nw) __attribute__((always_inline)) {
-      const float gate = a.w_sg ? bf16_lo(s_sact[Fs / 2]) : 0.0f;
+      const float gate = gated ? bf16_lo(s_sact[Fs / 2]) : 0.0f;
       for (uint32_t s0 = wv * srpw; s0 < n_slots; s0 += nw * srpw) {
         const uint32_t i = s0 + (lane >> slpr_log2);  // slot of (round, unit_local, row in unit)
         const uint32_t round = i / rows_per_round, in_round = i % rows_per_round;
@@ -675,7 +681,7 @@ __global__ __launch_bounds__(kFusedThreads) void fused_decode_kernel(const Fused
         const float v = group_sum(part, static_cast<int>(slpr));
         if (ok && ssub == 0) {
           float h = round_bf16(v);  // dequant_int4.metal:177-180
-          if (a.w_sg) h = round_bf16(h / (1.0f + mf_exp(-gate)));  // utility.metal:49-59
+          if (gated) h = round_bf16(h / (1.0f + mf_exp(-gate)));  // utility.metal:49-59
           s_h1[i] = h;
         }
       }
@@ -848,7 +854,8 @@ bool fused_supported(const mf_moe& h, const mf_moe_layer_weights& w, const void*
     if (!aligned16(w.shared_gate.weights) || !aligned16(w.shared_up.weights) ||
         !aligned16(w.shared_down.weights))
       return false;
-    if (w.w_sg && !aligned16(w.w_sg)) return false;
+    if (w.w_sg && !w.w_sg_q8.weights && !aligned16(w.w_sg)) return false;
+    if (w.w_sg_q8.weights && (reinterpret_cast<uintptr_t>(w.w_sg_q8.weights) & 7u)) return false;
   }
   return true;
 }
@@ -865,7 +872,11 @@ hipError_t launch_fused_decode(hipStream_t s, const mf_moe& h, const mf_moe_laye
   a.sg = w.shared_gate;
   a.su = w.shared_up;
   a.sd = w.shared_down;
-  a.w_sg = c.shared_f ? w.w_sg : nullptr;
+  const bool gate_q8 = c.shared_f && w.w_sg_q8.weights;
+  a.w_sg = c.shared_f && !gate_q8 ? w.w_sg : nullptr;
+  a.gq_w = gate_q8 ? static_cast<const uint8_t*>(w.w_sg_q8.weights) : nullptr;
+  a.gq_s = gate_q8 ? w.w_sg_q8.scales : nullptr;
+  a.gq_b = gate_q8 ? w.w_sg_q8.biases : nullptr;
   a.x = x;
   a.y = y;
   a.hidden = hidden;

@@ -2289,7 +2289,7 @@ hipError_t launch_prefill_layer(hipStream_t s, const mf_moe& h, const mf_moe_lay
     if (w.router_w) {  // else the routing in out_idx / out_w is the caller's
       RouterTail tail{};
       tail.xp = ws.xp;
-      tail.w_sg = c.shared_f ? w.w_sg : nullptr;
+      tail.w_sg = c.shared_f && !w.w_sg_q8.weights ? w.w_sg : nullptr;  // (an 8-bit gate row: its own launch below)
       tail.sums = ws.sum_x;
       tail.gate = ws.gate;
       MF_TRY(launch_prefill_router(s, w.router_w, x, c.num_experts, c.d, t, c.d, ws.logits, &tail));
@@ -2306,15 +2306,19 @@ hipError_t launch_prefill_layer(hipStream_t s, const mf_moe& h, const mf_moe_lay
                           ws.sorted, ws.tiles, max_tiles, ws.n_tiles, ws.status, h.ws.group_tmp + 2048));
   }
 
-  const bool want_gate = c.shared_f && w.w_sg;
+  const bool gate_q8 = c.shared_f && w.w_sg_q8.weights;
+  const bool want_gate = c.shared_f && (w.w_sg || gate_q8);
   if (x_prepared) {
     // the router launch has prepared x (and the gate's logits) on the side
-  } else if (want_gate) {  // one pass over x: matmul order, group sums and the shared gate's logits
+  } else if (want_gate && !gate_q8) {  // one pass over x: matmul order, group sums and the shared gate's logits
     prep_x_gate_kernel<<<dim3((t + 3) / 4), dim3(256), 0, s>>>(x, ws.xp, ws.sum_x, w.w_sg, ws.gate, t, c.d);
     MF_TRY(hipGetLastError());
   } else {
     MF_TRY(launch_prep_rows(s, x, ws.xp, ws.sum_x, static_cast<size_t>(t) * c.d));
   }
+  // the scalar gate stored as an 8-bit row (RealForwardRunner.swift:2925-2941): one wave per token, the
+  // bits of mf_gemv(MF_BITS_8) -- and of the decode launch
+  if (gate_q8) MF_TRY(launch_gemv(s, w.w_sg_q8, MF_BITS_8, x, ws.gate, 1, c.d, t, false));
 
   QmmArgs q{};
   q.expert_base = static_cast<const uint8_t*>(w.expert_base);

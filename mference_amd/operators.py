@@ -16,7 +16,7 @@ import numpy as np
 import torch
 
 from . import _capi
-from ._capi import (BITS_2, BITS_4, BITS_TERNARY, GROUP_SIZE, MAX_TOKENS, ROUTER_FULL_SOFTMAX,
+from ._capi import (BITS_2, BITS_4, BITS_8, BITS_TERNARY, GROUP_SIZE, MAX_TOKENS, ROUTER_FULL_SOFTMAX,
                     ROUTER_TOPK_SOFTMAX, ExpertOffsets, MfError, check)
 
 __all__ = [
@@ -116,7 +116,7 @@ class Quantization:
             raise ValueError("w must be a 2-D float32 tensor")
         w = w.contiguous()
         rows, n = w.shape
-        store = 4 if bits == BITS_4 else 2
+        store = {BITS_8: 8, BITS_4: 4}.get(bits, 2)   # 8-bit: quantizeInt8Affine (Quantization.swift:135-176)
         packed = torch.empty((rows, n * store // 8), dtype=torch.uint8, device=w.device)
         scales = torch.empty((rows, n // GROUP_SIZE), dtype=torch.bfloat16, device=w.device)
         biases = torch.empty_like(scales)
@@ -328,6 +328,7 @@ class MoELayerWeights:
     offsets: ExpertOffsets
     shared: Optional[Sequence[QuantizedTensor]] = None  # gate, up, down
     w_sg: Optional[torch.Tensor] = None    # bf16 [d]
+    w_sg_q8: Optional[QuantizedTensor] = None  # the scalar gate as an 8-bit affine row [1, d] (replaces w_sg)
 
     def c(self) -> _capi.LayerWeights:
         if self.experts.ndim != 2 or self.experts.stride(1) != 1:
@@ -341,6 +342,8 @@ class MoELayerWeights:
         if self.shared is not None:
             L.shared_gate, L.shared_up, L.shared_down = (q.c() for q in self.shared)
         L.w_sg = _ptr(self.w_sg)
+        if self.w_sg_q8 is not None:
+            L.w_sg_q8 = self.w_sg_q8.c()
         return L
 
 

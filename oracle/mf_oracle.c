@@ -799,7 +799,14 @@ int mfo_moe_layer(const mfo_layer* L, const uint16_t* x, uint16_t* y, uint32_t* 
   if (L->fs > 0) {
     rc = mfo_shared_expert(L->sgw, L->sgs, L->sgb, L->suw, L->sus, L->sub, L->sdw, L->sds,
                            L->sdb, L->shared_bits, d, L->fs, x, h1);
-    if (!rc && L->w_sg) {
+    if (!rc && L->gqw) {
+      /* the 8-bit row in the lane order of mfo_router_logits_int8, x unscaled (effective scale 1) */
+      uint16_t* ones = (uint16_t*)malloc(d * sizeof(uint16_t));
+      for (size_t i = 0; i < d; ++i) ones[i] = 0x3F80;
+      uint16_t gate = mfo_bf16_bits(mfo_dot_int8_laneorder(L->gqw, L->gqs, L->gqb, x, ones, d));
+      free(ones);
+      mfo_sigmoid_scalar_mul(h1, d, gate);
+    } else if (!rc && L->w_sg) {
       uint16_t gate = mfo_bf16_bits(mfo_dot_bf16_laneorder(L->w_sg, x, d));
       mfo_sigmoid_scalar_mul(h1, d, gate);
     }

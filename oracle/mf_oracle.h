@@ -167,6 +167,9 @@ typedef struct {
   const uint16_t* w_sg;      /* [d] bf16 scalar shared gate, may be NULL    */
   int maple_rounding;        /* MapleMoE's activation and bf16 down outputs */
   int gate_group;            /* group of the routed gate tables: 0 / 64, or 32 */
+  /* the scalar shared gate as an 8-bit affine row [1,d] (RealForwardRunner.swift:2925-2941,
+   * dequant_int8.metal:66-107); used instead of w_sg when gqw != NULL */
+  const uint8_t* gqw; const uint16_t* gqs; const uint16_t* gqb;
 } mfo_layer;
 
 /* one token through router -> routed experts -> shared expert -> combine.

@@ -53,6 +53,7 @@ class _Layer(C.Structure):
         ("suw", C.c_void_p), ("sus", C.c_void_p), ("sub", C.c_void_p),
         ("sdw", C.c_void_p), ("sds", C.c_void_p), ("sdb", C.c_void_p),
         ("w_sg", C.c_void_p), ("maple_rounding", C.c_int), ("gate_group", C.c_int),
+        ("gqw", C.c_void_p), ("gqs", C.c_void_p), ("gqb", C.c_void_p),
     ]
 
 
@@ -416,6 +417,7 @@ class Layer:
     swiglu_limit: float = 0.0
     maple_rounding: bool = False    # MapleMoE's activation and bf16 down outputs
     gate_group: int = GROUP         # group of the routed gate tables (32: the DeepSeek-V4 conversion)
+    w_sg_q8: Optional["QTensor"] = None  # the scalar gate as an 8-bit affine row [1, d] (replaces w_sg)
 
     def _struct(self) -> _Layer:
         L = _Layer()
@@ -435,6 +437,9 @@ class Layer:
             L.sdw, L.sds, L.sdb = dn.packed.ctypes.data, dn.scales.ctypes.data, dn.biases.ctypes.data
         if self.w_sg is not None:
             L.w_sg = self.w_sg.ctypes.data
+        if self.w_sg_q8 is not None:
+            q = self.w_sg_q8
+            L.gqw, L.gqs, L.gqb = q.packed.ctypes.data, q.scales.ctypes.data, q.biases.ctypes.data
         return L
 
 

@@ -28,7 +28,8 @@ def to_device_layer(layer, device="cuda") -> ops.MoELayerWeights:
         router_w=ops.bf16_tensor(layer.router_w, device),
         experts=torch.from_numpy(layer.experts).to(device),
         offsets=off, shared=shared,
-        w_sg=None if layer.w_sg is None else ops.bf16_tensor(layer.w_sg, device))
+        w_sg=None if layer.w_sg is None else ops.bf16_tensor(layer.w_sg, device),
+        w_sg_q8=None if getattr(layer, "w_sg_q8", None) is None else to_device_q(layer.w_sg_q8, device))
 
 
 def make_moe(ctx, layer) -> ops.MoE:

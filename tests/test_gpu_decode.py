@@ -14,7 +14,7 @@ def _sync():
     torch.cuda.synchronize()
 
 
-@pytest.mark.parametrize("bits", [4, 2])
+@pytest.mark.parametrize("bits", [4, 2, 8])
 @pytest.mark.parametrize("rows,n", [(7, 64), (16, 256), (33, 2048), (5, 4096)])
 def test_quantize_bit_exact(gpu, oracle, bits, rows, n):
     rng = oracle.Rng.key(0x51A71001, f"quant-{bits}-{rows}-{n}")
@@ -30,7 +30,7 @@ def test_quantize_bit_exact(gpu, oracle, bits, rows, n):
     assert np.array_equal(ops.bf16_bits(q.biases), ref.biases)
 
 
-@pytest.mark.parametrize("bits", [4, 2, 1])
+@pytest.mark.parametrize("bits", [4, 2, 1, 8])
 def test_dequantize_bit_exact(gpu, oracle, bits):
     rows, n = 9, 512
     rng = oracle.Rng.key(0xF5, f"dequant-{bits}")
@@ -911,3 +911,85 @@ def test_fused_topk_on_non_finite_logits(gpu, oracle, e):
             assert np.array_equal(one_row[0][0], ref_idx[i]) and np.array_equal(one_row[1][0], fused[1][i])
     finally:
         moe.set_fused(True)
+
+
+@pytest.mark.parametrize("m,n,t", [(1, 2048, 1), (1, 2048, 8), (64, 64, 3), (65, 192, 2), (130, 2816, 1), (8, 5120, 8)])
+def test_int8_gemv(gpu, oracle, m, n, t):
+    """8-bit affine rows (DequantInt8GEMV.encode, Kernels/Quant/DequantInt8GEMV.swift:53; dequant_int8_gemv_simd,
+    dequant_int8.metal:66-107): the value of every (token, row) has the bits of the checker's lane-order row dot
+    (x unscaled), agrees with the reference's CPU path (bulk dequantize, scalar dot) to fp32 summation order, and
+    does not depend on how many token rows ride along; weights two bytes into their allocation take the
+    byte-wise loads."""
+    rng = oracle.Rng.key(0x18, f"gemv8-{m}-{n}-{t}")
+    q = oracle.quantize(rng.normal(0.0, 0.02, m * n).reshape(m, n), 8)
+    x = oracle.bf16_bits(rng.normal(0.0, 1.0, t * n).reshape(t, n))
+    ones = np.full(n, 0x3F80, np.uint16)
+    exact = np.stack([oracle.router_logits_int8(q.packed, q.scales, q.biases, x[i], ones) for i in range(t)])
+    ref = oracle.gemv_multix(q, x)
+    g = ops.DequantInt4GEMVMultiX(gpu)
+    dq = to_device_q(q)
+    xd = ops.bf16_tensor(x)
+    y32 = torch.full((t, m), 7.0, dtype=torch.float32, device="cuda")
+    y16 = torch.zeros((t, m), dtype=torch.bfloat16, device="cuda")
+    g.encode(dq, xd, y32, m, n, t, output_float32=True)
+    g.encode(dq, xd, y16, m, n, t)
+    _sync()
+    got = y32.cpu().numpy()
+    assert np.array_equal(got.view(np.uint32), exact.view(np.uint32))
+    assert np.abs(got - ref).max() / max(np.abs(ref).max(), 1e-6) < 2e-5
+    assert np.array_equal(ops.bf16_bits(y16), oracle.bf16_bits(got))
+    for i in range(t):
+        yi = torch.zeros((1, m), dtype=torch.float32, device="cuda")
+        g.encode(dq, xd[i:i + 1].contiguous(), yi, m, n, 1, output_float32=True)
+        _sync()
+        assert np.array_equal(yi.cpu().numpy()[0].view(np.uint32), got[i].view(np.uint32))
+    raw = torch.zeros(q.packed.size + 16, dtype=torch.uint8, device="cuda")
+    raw[2:2 + q.packed.size] = torch.from_numpy(q.packed.reshape(-1)).cuda()
+    odd = ops.QuantizedTensor(raw[2:2 + q.packed.size].view(m, n), dq.scales, dq.biases, 8, m, n)
+    yo = torch.zeros((t, m), dtype=torch.float32, device="cuda")
+    g.encode(odd, xd, yo, m, n, t, output_float32=True)
+    _sync()
+    assert np.array_equal(yo.cpu().numpy().view(np.uint32), exact.view(np.uint32))
+
+
+@pytest.mark.parametrize("d,f,e,k,fs,t", [(2048, 512, 256, 8, 512, 1), (2048, 512, 256, 8, 512, 4), (512, 256, 32, 4, 256, 3)])
+def test_layer_with_int8_scalar_gate(gpu, oracle, d, f, e, k, fs, t):
+    """The scalar shared gate as the reference's model files store it -- an 8-bit affine row
+    (RealForwardRunner.swift:2925-2941): the fused launch and the chain of launches give the same bits, the
+    layer agrees with the checker, and so does the ragged prefill call on the same weights."""
+    root = ROOT_SEED + 0x8A7E + d + t
+    layer = oracle.synth_layer(root, d, f, e, k, bits=4, fs=fs)
+    gate_row = oracle.Rng.key(root, "w_sg.q8").normal(0.0, 0.05, d).reshape(1, d)
+    layer.w_sg_q8 = oracle.quantize(gate_row, 8)
+    layer.w_sg = None
+    x = oracle.synth_x(root, t, d)
+    ref_y, ref_idx, ref_w = oracle.moe_layer(layer, x)
+    plain = oracle.synth_layer(root, d, f, e, k, bits=4, fs=fs, with_w_sg=False)
+    assert not np.array_equal(oracle.moe_layer(plain, x)[0], ref_y), "the gate has to matter in this case"
+    moe = make_moe(gpu, layer)
+    wts = to_device_layer(layer)
+    xd = ops.bf16_tensor(x)
+    outs = []
+    try:
+        for fused in (True, False):
+            moe.set_fused(fused)
+            y = torch.zeros((t, d), dtype=torch.bfloat16, device="cuda")
+            idx = torch.zeros((t, k), dtype=torch.int32, device="cuda")
+            moe.encode_decode_layer(wts, xd, y, t=t, out_indices=idx)
+            moe.status()
+            assert np.array_equal(idx.cpu().numpy().astype(np.uint32), ref_idx)
+            assert_layer_close(oracle.bf16_to_float(ops.bf16_bits(y)), oracle.bf16_to_float(ref_y),
+                               f"int8 gate fused={fused}")
+            outs.append(ops.bf16_bits(y))
+    finally:
+        moe.set_fused(True)
+    assert np.array_equal(outs[0], outs[1])
+    tp = 70
+    xp = oracle.synth_x(root + 1, tp, d)
+    ref_yp, ref_idxp, _ = oracle.moe_layer(layer, xp)
+    yp = torch.zeros((tp, d), dtype=torch.bfloat16, device="cuda")
+    idxp = torch.zeros((tp, k), dtype=torch.int32, device="cuda")
+    moe.encode_prefill_layer(wts, ops.bf16_tensor(xp), yp, tp, out_indices=idxp)
+    _sync()
+    assert np.array_equal(idxp.cpu().numpy().astype(np.uint32), ref_idxp)
+    assert_layer_close(oracle.bf16_to_float(ops.bf16_bits(yp)), oracle.bf16_to_float(ref_yp), "int8 gate prefill")

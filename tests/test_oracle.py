@@ -683,3 +683,40 @@ def test_gate_projection_at_group_32_against_float64(oracle):
     assert rc == 0 and np.array_equal(y64.view(np.uint32), oracle.gemv(q64, x).view(np.uint32))
     assert lib.mfo_gemv_group(oracle._p(q.packed), oracle._p(q.scales), oracle._p(q.biases), 2,
                               C.c_size_t(rows), C.c_size_t(n), C.c_size_t(16), oracle._p(x), oracle._p(y)) != 0
+
+
+def test_layer_with_int8_scalar_gate_matches_its_bf16_twin():
+    """The layer with its scalar shared gate as an 8-bit affine row (RealForwardRunner.swift:2925-2941;
+    dequant_int8.metal:66-107) against the same layer with the gate as bf16 numbers, for a row whose dequantized
+    weights q / 128 - 1 are bf16 numbers themselves: the two gate logits differ by fp32 summation order only, so
+    the layers agree to a bf16 step of the gated shared output -- and the gate is not a no-op."""
+    import numpy as np
+    from oracle import mf_oracle as O
+    d, f, e, k, fs, t = 256, 128, 16, 4, 128, 6
+    root = 0x4D464D4F00000000 + 0x1808
+    layer = O.synth_layer(root, d, f, e, k, bits=4, fs=fs)
+    codes = (np.array([O.Rng.key(root, "gate.codes").next() % 256 for _ in range(d)], np.uint8)).reshape(1, d)
+    scales = np.full((1, d // 64), O.bf16_bits(np.array([1.0 / 128], np.float32))[0], np.uint16)
+    biases = np.full((1, d // 64), O.bf16_bits(np.array([-1.0], np.float32))[0], np.uint16)
+    q8 = O.QTensor(codes, scales, biases, 8, 1, d)
+    twin = O.bf16_bits(O.dequantize(q8).reshape(d))
+    assert np.array_equal(O.bf16_to_float(twin), O.dequantize(q8).reshape(d))   # exactly representable
+    x = O.synth_x(root, t, d)
+    layer.w_sg, layer.w_sg_q8 = twin, None
+    y_bf16, idx_a, _ = O.moe_layer(layer, x)
+    layer.w_sg, layer.w_sg_q8 = None, q8
+    y_q8, idx_b, _ = O.moe_layer(layer, x)
+    layer.w_sg_q8 = None
+    y_none, _, _ = O.moe_layer(layer, x)
+    assert np.array_equal(idx_a, idx_b)
+    a, b = O.bf16_to_float(y_bf16).astype(np.float64), O.bf16_to_float(y_q8).astype(np.float64)
+    assert np.abs(a - b).max() <= 2.0 ** -7 * max(np.abs(a).max(), 1e-3)
+    assert (y_bf16 == y_q8).mean() > 0.9
+    assert not np.array_equal(y_none, y_q8)
+    # the gate logit itself: lane-order value against fp64 on the dequantized row
+    ones = np.full(d, 0x3F80, np.uint16)
+    w64 = O.dequantize(q8).reshape(d).astype(np.float64)
+    for i in range(t):
+        got = O.router_logits_int8(codes, scales, biases, x[i], ones)[0]
+        ref = float(w64 @ O.bf16_to_float(x[i]).astype(np.float64))
+        assert abs(got - ref) <= 1e-5 * max(1.0, abs(ref))

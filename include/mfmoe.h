@@ -465,7 +465,11 @@ mf_status mf_moe_decode_layer(mf_moe* h, mf_stream stream, const mf_moe_layer_we
  * launches (router, top-k, shared expert, phase 1, phase 2) inside
  * mf_moe_decode_layer.  Both give bit-identical results; the chain is the
  * structure of the reference's decode step and handles operands that are not
- * 16-byte aligned.  No counterpart in the reference. */
+ * 16-byte aligned.  enabled = 2: the fused launch, but through the kernel instance that reads every
+ * dimension from its arguments even when the build holds an instance with this layer's shape as
+ * literals (the reference specialises every shape through function constants, Kernels/MoE/MoE.swift:80-91;
+ * here the build specialises the shapes listed in mference_amd/fused_shapes.json) -- same bits, for
+ * measuring what the literals buy.  No counterpart in the reference. */
 mf_status mf_moe_set_fused(mf_moe* h, int enabled);
 
 /* Phase trace of the fused launch: when device_buffer is not NULL every

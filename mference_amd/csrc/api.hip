@@ -642,6 +642,7 @@ mf_status mf_moe_decode_layer(mf_moe* h, mf_stream stream, const mf_moe_layer_we
 mf_status mf_moe_set_fused(mf_moe* h, int enabled) {
   if (!h) return MF_ERR_INVALID_ARGUMENT;
   h->fused = enabled != 0;
+  h->generic_shape = enabled == 2;
   return MF_OK;
 }
 

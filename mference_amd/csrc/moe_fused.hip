@@ -940,6 +940,11 @@ hipError_t launch_fused_decode(hipStream_t s, const mf_moe& h, const mf_moe_laye
   const bool maple = c.bits == MF_BITS_TERNARY && c.d == 2048 && c.f == 512 && c.num_experts == 256 &&
                      c.top_k == 8 && c.shared_f == 0;
   const bool no_limit = c.swiglu_limit == 0.0f;  // the one-token instances of the benchmark shapes have these flags as literals
+  // the instances of the shapes listed for the build (fused_shapes.json): declarations here, the branches
+  // that pick them below, ahead of the instances that read every dimension from the arguments
+#define MF_SHAPES_DECLARE
+#include "fused_shapes.inc"
+#undef MF_SHAPES_DECLARE
   using Given = RuntimeShapeT<true>;
   using Big2T1Given = StaticShape<4096, 2048, 256, 6, 1, 2048, true>;
   using QwenT1Given = StaticShape<2048, 512, 256, 8, 1, 512, true, kDyn, 0, 1, 1>;
@@ -947,14 +952,29 @@ hipError_t launch_fused_decode(hipStream_t s, const mf_moe& h, const mf_moe_laye
   // (with the routing given the router mode plays no part: the shapes are recognised without it)
   const bool qwen_dims = c.bits == MF_BITS_4 && c.shared_bits == MF_BITS_4 && c.d == 2048 && c.f == 512 &&
                          c.num_experts == 256 && c.top_k == 8 && c.shared_f == 512;
+  const bool lit = !h.generic_shape;  // shape instances allowed
   if (!w.router_w) {  // caller-given routing
-    if (big2 && t == 1) MF_FUSED(kBits2, kBits4, Big2T1Given);
+    if (!lit) {
+      if (c.bits == MF_BITS_4) MF_FUSED(kBits4, kBits4, Given);
+      else if (c.bits == MF_BITS_2 && c.shared_f && c.shared_bits == MF_BITS_2) MF_FUSED(kBits2, kBits2, Given);
+      else if (c.bits == MF_BITS_2) MF_FUSED(kBits2, kBits4, Given);
+      else MF_FUSED(kBitsTernary, kBits4, Given);
+    }
+    else if (big2 && t == 1) MF_FUSED(kBits2, kBits4, Big2T1Given);
     else if (qwen_dims && t == 1 && !c.maple_rounding && no_limit && a.xprep) MF_FUSED(kBits4, kBits4, QwenT1Given);
     else if (qwen_dims) MF_FUSED(kBits4, kBits4, QwenTnGiven);
+#define MF_SHAPES_PICK_GIVEN
+#include "fused_shapes.inc"
+#undef MF_SHAPES_PICK_GIVEN
     else if (c.bits == MF_BITS_4) MF_FUSED(kBits4, kBits4, Given);
     else if (c.bits == MF_BITS_2 && c.shared_f && c.shared_bits == MF_BITS_2) MF_FUSED(kBits2, kBits2, Given);
     else if (c.bits == MF_BITS_2) MF_FUSED(kBits2, kBits4, Given);
     else MF_FUSED(kBitsTernary, kBits4, Given);
+  } else if (!lit) {
+    if (c.bits == MF_BITS_4) MF_FUSED(kBits4, kBits4, RuntimeShape);
+    else if (c.bits == MF_BITS_2 && c.shared_f && c.shared_bits == MF_BITS_2) MF_FUSED(kBits2, kBits2, RuntimeShape);
+    else if (c.bits == MF_BITS_2) MF_FUSED(kBits2, kBits4, RuntimeShape);
+    else MF_FUSED(kBitsTernary, kBits4, RuntimeShape);
   } else if (qwen && t == 1 && !c.maple_rounding && no_limit && a.xprep) MF_FUSED(kBits4, kBits4, QwenT1);
   else if (qwen) MF_FUSED(kBits4, kBits4, QwenTn);
   else if (big2 && t == 1 && !c.maple_rounding && a.xprep) MF_FUSED(kBits2, kBits4, Big2T1);
@@ -965,6 +985,9 @@ hipError_t launch_fused_decode(hipStream_t s, const mf_moe& h, const mf_moe_laye
   else if (maple && t == 1 && c.router_mode == MF_ROUTER_FULL_SOFTMAX && c.maple_rounding && no_limit && a.xprep)
     MF_FUSED(kBitsTernary, kBits4, MapleT1);
   else if (maple) MF_FUSED(kBitsTernary, kBits4, MapleTn);
+#define MF_SHAPES_PICK_OWN
+#include "fused_shapes.inc"
+#undef MF_SHAPES_PICK_OWN
   else if (c.bits == MF_BITS_4) MF_FUSED(kBits4, kBits4, RuntimeShape);
   else if (c.bits == MF_BITS_2 && c.shared_f && c.shared_bits == MF_BITS_2)
     MF_FUSED(kBits2, kBits2, RuntimeShape);

@@ -376,9 +376,10 @@ class MoE:
         except Exception:
             pass
 
-    def set_fused(self, enabled: bool) -> None:
-        """single fused launch (default) or the chain of separate launches"""
-        check(_capi.lib().mf_moe_set_fused(self._h, 1 if enabled else 0), self.context.handle)
+    def set_fused(self, enabled) -> None:
+        """single fused launch (True / 1, default) or the chain of separate launches (False / 0); 2: the fused
+        launch through the instance that reads every dimension from its arguments"""
+        check(_capi.lib().mf_moe_set_fused(self._h, int(enabled)), self.context.handle)
 
     def set_phase_trace(self, buffer: Optional[torch.Tensor]) -> None:
         """int64 device tensor of num_cu*8 entries receiving per-workgroup stage

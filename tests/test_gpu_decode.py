@@ -993,3 +993,42 @@ def test_layer_with_int8_scalar_gate(gpu, oracle, d, f, e, k, fs, t):
     _sync()
     assert np.array_equal(idxp.cpu().numpy().astype(np.uint32), ref_idxp)
     assert_layer_close(oracle.bf16_to_float(ops.bf16_bits(yp)), oracle.bf16_to_float(ref_yp), "int8 gate prefill")
+
+
+@pytest.mark.parametrize("t", [1, 4])
+def test_listed_shape_instance_at_full_size(gpu, oracle, t):
+    """A layer shape that is no benchmark shape -- Gemma 4's (hidden 2816, 128 experts of 704, top-8;
+    ArchConfig.gemma4_26B_A4B, ModelTypes.swift:376-398) -- listed in fused_shapes.json: the build holds
+    instances of the fused launch with its dimensions as literals.  At full size against the checker, and the
+    same bits as the instance that reads every dimension from its arguments and as the chain of launches;
+    with the routing given by the caller too (Gemma routes through its 8-bit router)."""
+    d, f, e, k = 2816, 704, 128, 8
+    root = ROOT_SEED + 0x6E44A + t
+    layer = oracle.synth_layer(root, d, f, e, k, bits=4, fs=0)
+    x = oracle.synth_x(root, t, d)
+    ref_y, ref_idx, ref_w = oracle.moe_layer(layer, x)
+    moe = make_moe(gpu, layer)
+    wts = to_device_layer(layer)
+    xd = ops.bf16_tensor(x)
+    got = {}
+    try:
+        for mode in (1, 2, 0):
+            moe.set_fused(mode)
+            y = torch.zeros((t, d), dtype=torch.bfloat16, device="cuda")
+            idx = torch.zeros((t, k), dtype=torch.int32, device="cuda")
+            w = torch.zeros((t, k), dtype=torch.float32, device="cuda")
+            moe.encode_decode_layer(wts, xd, y, t=t, out_indices=idx, out_weights=w)
+            moe.status()
+            assert np.array_equal(idx.cpu().numpy().astype(np.uint32), ref_idx)
+            assert np.array_equal(w.cpu().numpy().view(np.uint32), ref_w.view(np.uint32))
+            got[mode] = ops.bf16_bits(y)
+        moe.set_fused(1)
+        given = ops.MoELayerWeights(None, wts.experts, wts.offsets, None, None)
+        yg = torch.zeros((t, d), dtype=torch.bfloat16, device="cuda")
+        moe.encode_decode_layer(given, xd, yg, t=t, out_indices=idx, out_weights=w)
+        moe.status()
+    finally:
+        moe.set_fused(1)
+    assert_layer_close(oracle.bf16_to_float(got[1]), oracle.bf16_to_float(ref_y), f"gemma shape t={t}")
+    assert np.array_equal(got[1], got[2]) and np.array_equal(got[1], got[0])
+    assert np.array_equal(ops.bf16_bits(yg), got[1])

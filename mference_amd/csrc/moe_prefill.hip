@@ -929,10 +929,10 @@ struct QmmArgs {
   // added afterwards): rows of weights, tables and group sums are ng_ld groups apart (0: kdim / 64)
   // and the window starts at group g_off (a multiple of 8)
   uint32_t ng_ld, g_off;
-  // several windows in one launch (dense mode): tile slots [w * win_tiles, (w + 1) * win_tiles) belong to
-  // window w, which covers the groups from dense_window_start(ng_ld, n_win, w) on and writes its fp32
-  // result out_win_stride elements behind the previous window's
-  uint32_t n_win, win_tiles;
+  // several windows in one launch (dense mode): window w covers the groups from
+  // dense_window_start(ng_ld, n_win, w) on and writes its fp32 result out_win_stride elements behind the
+  // previous window's
+  uint32_t n_win;
   size_t out_win_stride;
   // epilogue
   int epi;              // 0 swiglu -> bf16 [pair, rows] in prep order; 1 fp32 [token*K+rank, rows]; 2 bf16 [pair, rows]
@@ -941,9 +941,16 @@ struct QmmArgs {
   int ternary;          // 2-bit codes {0,1,2} with bias = -scale: b_off / dense[].biases name the SCALE table
   int maple;            // MapleMoE's bf16-stepped activation in the SwiGLU epilogue
   void* out;
+  void* out2;           // epi 1 / 2 with two projections that are not row blocks of one: where projection 1 goes (null: dropped)
   uint32_t top_k;
   float limit;
-  uint32_t dense_tiles;  // dense mode: number of 64-row tiles
+  // dense mode: number of 64-row tiles and of work items; every XCD gets an eighth of the items however few
+  // tiles there are.  With few tiles (tile_major = 0: x is small, the weights are not) work item w is tile
+  // w % dense_tiles of row slice (w / dense_tiles) % slices: the items that read the same weight rows follow
+  // one another (same XCD, same moment).  With many tiles (tile_major = 1) the slices of one tile follow one
+  // another and an XCD's L2 holds the x rows of the few tiles it works on.  The window is w / (tiles * slices).
+  uint32_t dense_tiles, dense_items;
+  int tile_major;
   // optional stage stamps: 8 per work item, 100 MHz clock
   unsigned long long* trace;
   uint32_t trace_items;
@@ -984,7 +991,7 @@ struct QmmLaunch {
   uint32_t per_xcd[2];  // work items of each part on one XCD (grid = 8 * their sum)
 };
 
-template <int BITS, int NPROJ, bool NG8>
+template <int BITS, int NPROJ, bool NG8, bool TAB16>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(NPROJ == 1 ? 3 : 2, NPROJ == 1 ? 3 : 2)))
 void qmm_kernel(const QmmLaunch launch) {
   constexpr uint32_t kGB = QmmCodes<BITS>::kGroupBytes;  // bytes of one K group of one weight row
@@ -1001,22 +1008,29 @@ void qmm_kernel(const QmmLaunch launch) {
   const uint32_t work = (blockIdx.x & 7u) * launch.per_xcd[second ? 1 : 0] + (xcd_slot - (second ? launch.per_xcd[0] : 0u));
   const uint32_t wave_rows = a.pair_rows ? 32u * NPROJ : 32u;  // weight rows of one wave
   const uint32_t n_slices = a.rows / (kQmmWaves * wave_rows);
-  uint32_t tile_id = work / n_slices;
-  const uint32_t slice = work % n_slices;
+  uint32_t tile_id = work / n_slices, slice = work % n_slices, win = 0;
+  if (a.dense_mode) {
+    if (work >= a.dense_items) return;
+    const uint32_t inner = a.tile_major ? n_slices : a.dense_tiles, outer = a.tile_major ? a.dense_tiles : n_slices;
+    const uint32_t lo = work % inner, rest = work / inner, hi = rest % outer;
+    tile_id = a.tile_major ? hi : lo;
+    slice = a.tile_major ? lo : hi;
+    win = rest / outer;
+    if (tile_id >= a.dense_tiles) return;
+  }
   uint32_t ng = a.kdim / kGroup, g_off = a.g_off;
   uint8_t* out_base = static_cast<uint8_t*>(a.out);
+  uint8_t* out2_base = static_cast<uint8_t*>(a.out2);
   if (a.n_win > 1) {  // this work item's window of the contraction
-    const uint32_t win = tile_id / a.win_tiles;
-    tile_id -= win * a.win_tiles;
     g_off = dense_window_start(a.ng_ld, a.n_win, win);
     ng = dense_window_start(a.ng_ld, a.n_win, win + 1) - g_off;
     out_base += win * a.out_win_stride * sizeof(float);
+    if (out2_base) out2_base += win * a.out_win_stride * sizeof(float);
   }
   qmm_trace(a, work, 0);
 
   uint32_t expert = 0, pair_start, count;
   if (a.dense_mode) {
-    if (tile_id >= a.dense_tiles) return;
     pair_start = tile_id * kTileTokens;
     count = min(kTileTokens, a.dense_rows - pair_start);
   } else {
@@ -1028,8 +1042,12 @@ void qmm_kernel(const QmmLaunch launch) {
   }
 
   uint4* s_x = reinterpret_cast<uint4*>(smem);                      // 2 stages x 2 groups x 512 uint4
-  float* s_scale = reinterpret_cast<float*>(smem + kQmmXBytes);     // [NPROJ][4][ng][32]
-  uint32_t* s_slot = reinterpret_cast<uint32_t*>(smem + kQmmXBytes + NPROJ * kQmmWaves * ng * 32 * 4);
+  // The scale of every (row, group): fp32, or (TAB16, long contractions) a bf16 number -- 2 * scale for 4-bit
+  // codes is one (exponent + 1), so the upper half of the fp32 product is all of it.  That is half the LDS,
+  // which lets two workgroups share a CU up to 112 K groups (K = 7168), for one more instruction per read.
+  using tab_t = std::conditional_t<TAB16, uint16_t, float>;
+  tab_t* s_scale = reinterpret_cast<tab_t*>(smem + kQmmXBytes);  // [NPROJ][4][ng][32]
+  uint32_t* s_slot = reinterpret_cast<uint32_t*>(smem + kQmmXBytes + ((NPROJ * kQmmWaves * ng * 32 * sizeof(tab_t) + 15) & ~15u));
 
   // weight pointers of this workgroup's projections
   const uint8_t* Wp[NPROJ];
@@ -1160,12 +1178,16 @@ void qmm_kernel(const QmmLaunch launch) {
     uint4 ab[NPROJ], as[NPROJ];
 #pragma unroll
     for (int p = 0; p < NPROJ; ++p) {
-      float* tab = s_scale + (p * kQmmWaves + wv) * ng * 32;
+      tab_t* tab = s_scale + (p * kQmmWaves + wv) * ng * 32;
+      auto entry = [](float v) -> tab_t {
+        if constexpr (TAB16) return static_cast<uint16_t>(__float_as_uint(v) >> 16);
+        else return v;
+      };
       const uint32_t pr[4] = {t.S[p].x, t.S[p].y, t.S[p].z, t.S[p].w};
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
-        if (have && (NG8 || gl + 2 * i < ng)) tab[(gl + 2 * i) * 32 + m] = QmmCodes<BITS>::kScaleMul * bf16_lo(pr[i]);
-        if (have && (NG8 || gl + 2 * i + 1 < ng)) tab[(gl + 2 * i + 1) * 32 + m] = QmmCodes<BITS>::kScaleMul * bf16_hi(pr[i]);
+        if (have && (NG8 || gl + 2 * i < ng)) tab[(gl + 2 * i) * 32 + m] = entry(QmmCodes<BITS>::kScaleMul * bf16_lo(pr[i]));
+        if (have && (NG8 || gl + 2 * i + 1 < ng)) tab[(gl + 2 * i + 1) * 32 + m] = entry(QmmCodes<BITS>::kScaleMul * bf16_hi(pr[i]));
       }
       constexpr uint32_t kAdd = QmmCodes<BITS>::kNegOffsetAdd;
       // ternary rows store no biases: the bias is -scale (the table pointer is the scale table then)
@@ -1267,7 +1289,9 @@ void qmm_kernel(const QmmLaunch launch) {
           for (int s = 0; s < 4; ++s) bx[nt][s] = buf[((nt * 4 + s) * 2 + h) * 32 + rd_col[s]];
 #pragma unroll
         for (int p = 0; p < NPROJ; ++p) {
-          const float sc = s_scale[((p * kQmmWaves + wv) * ng + g) * 32 + m];
+          float sc;
+          if constexpr (TAB16) sc = bf16_to_f(s_scale[((p * kQmmWaves + wv) * ng + g) * 32 + m]);
+          else sc = s_scale[((p * kQmmWaves + wv) * ng + g) * 32 + m];
           f32x16_t tmp[2];
 #pragma unroll
           for (int nt = 0; nt < NTA; ++nt)
@@ -1367,9 +1391,10 @@ void qmm_kernel(const QmmLaunch launch) {
           const size_t at = static_cast<size_t>(slot[i]) * a.rows;
 #pragma unroll
           for (int p = 0; p < NPROJ; ++p) {
-            if (p > 0 && !a.pair_rows) break;
-            if (a.epi == 1) reinterpret_cast<float*>(out_base)[at + row_base[p] + m] = acc[p][nt][4 * j + i];
-            else reinterpret_cast<uint16_t*>(out_base)[at + row_base[p] + m] = f_to_bf16(acc[p][nt][4 * j + i]);
+            if (p > 0 && !a.pair_rows && !out2_base) break;
+            uint8_t* ob = (p > 0 && !a.pair_rows) ? out2_base : out_base;  // the second projection's own buffer
+            if (a.epi == 1) reinterpret_cast<float*>(ob)[at + row_base[p] + m] = acc[p][nt][4 * j + i];
+            else reinterpret_cast<uint16_t*>(ob)[at + row_base[p] + m] = f_to_bf16(acc[p][nt][4 * j + i]);
           }
         }
       }
@@ -1420,12 +1445,17 @@ void qmm_kres_kernel(const KresLaunch launch) {
   const uint32_t work = (blockIdx.x & 7u) * launch.per_xcd[second ? 1 : 0] + (xcd_slot - (second ? launch.per_xcd[0] : 0u));
   const uint32_t n_walk = launch.slices[second ? 1 : 0];
   const uint32_t items_per_tile = a.rows / (256u * n_walk);
-  const uint32_t tile_id = work / items_per_tile, slice0 = (work % items_per_tile) * n_walk;
+  uint32_t tile_id = work / items_per_tile, slice0 = (work % items_per_tile) * n_walk;
+  if (a.dense_mode) {
+    if (work >= a.dense_items) return;
+    tile_id = a.tile_major ? work / items_per_tile : work % a.dense_tiles;
+    slice0 = (a.tile_major ? work % items_per_tile : work / a.dense_tiles) * n_walk;
+    if (tile_id >= a.dense_tiles) return;
+  }
   qmm_trace(a, work, 0);
 
   uint32_t expert = 0, pair_start, count;
   if (a.dense_mode) {
-    if (tile_id >= a.dense_tiles) return;
     pair_start = tile_id * kTileTokens;
     count = min(kTileTokens, a.dense_rows - pair_start);
   } else {
@@ -1901,10 +1931,13 @@ hipError_t launch_topk_group(hipStream_t s, const float* logits, uint32_t t, uin
   return hipGetLastError();
 }
 
-size_t qmm_lds_bytes(uint32_t kdim, int nproj) {
+size_t qmm_lds_bytes(uint32_t kdim, int nproj, bool tab16) {
   const uint32_t ng = kdim / kGroup;
-  return kQmmXBytes + static_cast<size_t>(nproj) * kQmmWaves * ng * 32 * 4 + kTileTokens * 4;
+  return kQmmXBytes + ((static_cast<size_t>(nproj) * kQmmWaves * ng * 32 * (tab16 ? 2 : 4) + 15) & ~static_cast<size_t>(15)) +
+         kTileTokens * 4;
 }
+// the scale tables as bf16 where fp32 tables would leave a CU (160 KB of LDS) room for one workgroup only
+bool qmm_tab16(uint32_t kdim, int nproj) { return 2 * qmm_lds_bytes(kdim, nproj, false) > 160 * 1024; }
 
 hipError_t launch_prep_rows(hipStream_t s, const uint16_t* src, uint16_t* dst, float* sums, size_t elems,
                             const uint16_t* src1 = nullptr, uint16_t* dst1 = nullptr, float* sums1 = nullptr,
@@ -1917,6 +1950,17 @@ hipError_t launch_prep_rows(hipStream_t s, const uint16_t* src, uint16_t* dst, f
   if (!blocks) return hipSuccess;
   prep_rows_kernel<<<dim3(blocks), dim3(256), 0, s>>>(a);
   return hipGetLastError();
+}
+
+// Work items of a dense problem that one XCD gets: an eighth, but at least 4 while there are any -- a handful
+// of items (the shared expert beside the routed experts of a short batch) runs faster on few XCDs, whose L2
+// serves the x rows and weight rows they share, than spread one to an XCD (Qwen shape, 128 tokens: layer 81 us
+// against 89 us).
+static uint32_t dense_per_xcd(uint32_t items) { return std::max((items + 7) / 8, std::min(items, 4u)); }
+// Whether an XCD should own tiles (and stream all weight rows) or row slices (and stream all of x): whichever
+// streams fewer bytes.  code_bits: 4 or 2.
+static int dense_tile_major(uint32_t rows, uint32_t x_rows, int code_bits) {
+  return static_cast<uint64_t>(rows) * code_bits <= static_cast<uint64_t>(x_rows) * 16;
 }
 
 // Whether qmm_kres_kernel takes the problem: a down-projection epilogue, K of 128, 256 or 512, whole
@@ -1936,17 +1980,20 @@ hipError_t launch_qmm_kres(hipStream_t s, int bits, const QmmArgs& a, uint32_t t
   for (int part = 0; part < (b ? 2 : 1); ++part) {
     QmmArgs& q = launch.part[part];
     q = part ? *b : a;
-    uint32_t slots = part ? b_tile_slots : tile_slots;
-    if (q.dense_mode) {
-      q.dense_tiles = slots;
-      slots = (slots + 7) / 8 * 8;
-    }
+    const uint32_t slots = part ? b_tile_slots : tile_slots;
     const uint32_t n_slices = q.rows / 256;
     // two slices per work item halve the set-up per slice and still leave several rounds of work items
     // (Qwen shape, 2048 tokens, whole layer: 331 us with one slice, 325 with two, 330 with four, 334 with eight)
     const uint32_t walk = n_slices % 2 == 0 ? 2 : 1;
     launch.slices[part] = walk;
-    launch.per_xcd[part] = slots / 8 * (n_slices / walk);
+    if (q.dense_mode) {
+      q.dense_tiles = slots;
+      q.tile_major = dense_tile_major(q.rows, q.dense_rows, bits);
+      q.dense_items = slots * (n_slices / walk);
+      launch.per_xcd[part] = dense_per_xcd(q.dense_items);
+    } else {
+      launch.per_xcd[part] = slots / 8 * (n_slices / walk);
+    }
   }
   const dim3 grid(8 * (launch.per_xcd[0] + launch.per_xcd[1])), block(256);
   if (grid.x == 0) return hipSuccess;
@@ -1976,47 +2023,52 @@ hipError_t launch_qmm(hipStream_t s, int bits, QmmArgs a, int nproj, uint32_t ti
                       uint32_t b_tile_slots) {
   QmmLaunch launch{};
   size_t lds = 0;
-  bool ng8 = true;
+  bool ng8 = true, tab16 = false;
   for (int part = 0; part < (b ? 2 : 1); ++part) {
     QmmArgs& q = launch.part[part];
     q = part ? *b : a;
-    uint32_t slots = part ? b_tile_slots : tile_slots;
+    const uint32_t slots = part ? b_tile_slots : tile_slots;
     const uint32_t n_slices = q.rows / (kQmmRows * (q.pair_rows ? nproj : 1));
     if (q.dense_mode) {
       q.dense_tiles = slots;
-      slots = (slots + 7) / 8 * 8;
-      if (q.n_win > 1) {  // every window of the contraction has its own run of tile slots
-        q.win_tiles = slots;
-        slots *= q.n_win;
-      }
+      q.tile_major = dense_tile_major(q.rows * (q.pair_rows ? 1 : nproj), q.dense_rows, bits);
+      q.dense_items = slots * n_slices * std::max(1u, q.n_win);
+      launch.per_xcd[part] = dense_per_xcd(q.dense_items);
+    } else {
+      launch.per_xcd[part] = slots / 8 * n_slices;
     }
-    launch.per_xcd[part] = slots / 8 * n_slices;
     q.tab_aligned = q.dense_mode
         ? aligned16(q.dense[0].scales) && aligned16(q.dense[0].biases) && aligned16(q.dense[1].scales) &&
               aligned16(q.dense[1].biases)
         : aligned16(q.expert_base) && q.expert_stride % 16 == 0 &&
               (q.s_off[0] | q.b_off[0] | q.s_off[1] | q.b_off[1]) % 16 == 0;
-    lds = std::max(lds, qmm_lds_bytes(q.kdim, nproj));  // with windows: kdim is the longest window
+    tab16 = tab16 || qmm_tab16(q.kdim, nproj);  // with windows: kdim is the longest window
     ng8 = ng8 && (q.n_win > 1 ? q.ng_ld : q.kdim / kGroup) % 8 == 0;
   }
+  for (int part = 0; part < (b ? 2 : 1); ++part) lds = std::max(lds, qmm_lds_bytes(launch.part[part].kdim, nproj, tab16));
   const dim3 grid(8 * (launch.per_xcd[0] + launch.per_xcd[1])), block(256);
   if (grid.x == 0) return hipSuccess;
-#define MF_QMM(B, P, G)                                                                                \
+#define MF_QMM(B, P, G, T)                                                                             \
   do {                                                                                                 \
     if (lds > 48 * 1024) {                                                                             \
-      hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(qmm_kernel<B, P, G>),           \
+      hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(qmm_kernel<B, P, G, T>),        \
                                          hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds)); \
       if (e != hipSuccess) return e;                                                                   \
     }                                                                                                  \
-    qmm_kernel<B, P, G><<<grid, block, lds, s>>>(launch);                                              \
+    qmm_kernel<B, P, G, T><<<grid, block, lds, s>>>(launch);                                           \
+  } while (0)
+#define MF_QMM_G(B, P, G)                                            \
+  do {                                                               \
+    if (tab16) MF_QMM(B, P, G, true); else MF_QMM(B, P, G, false);   \
   } while (0)
 #define MF_QMM_B(B)                                                        \
   do {                                                                     \
-    if (nproj == 2) { if (ng8) MF_QMM(B, 2, true); else MF_QMM(B, 2, false); } \
-    else { if (ng8) MF_QMM(B, 1, true); else MF_QMM(B, 1, false); }        \
+    if (nproj == 2) { if (ng8) MF_QMM_G(B, 2, true); else MF_QMM_G(B, 2, false); } \
+    else { if (ng8) MF_QMM_G(B, 1, true); else MF_QMM_G(B, 1, false); }    \
   } while (0)
   if (bits == 4) MF_QMM_B(4); else MF_QMM_B(2);
 #undef MF_QMM_B
+#undef MF_QMM_G
 #undef MF_QMM
   return hipGetLastError();
 }
@@ -2032,9 +2084,10 @@ size_t up256(size_t v) { return (v + 255) / 256 * 256; }
 // workgroup's rows for the whole contraction in LDS, so a long K is cut into windows of at most
 // kDenseWindow groups (multiples of 8 groups, the last takes the rest): every window is a launch that
 // writes fp32 [m, n], and dense_combine_kernel adds the windows in order and narrows the sum.
+// A gate / up pair whose K does not fit one launch's tables (kDenseFusedMax groups) goes the same way:
+// both projections as fp32 per window, then dense_swiglu_combine_kernel.
 constexpr uint32_t kDenseWindow = 64;   // K groups per launch (4096 values)
 constexpr uint32_t kDenseFusedMax = 112;  // K groups a gate/up + SwiGLU launch can hold (both projections' scales in LDS)
-
 __global__ __launch_bounds__(256) void dense_combine_kernel(const float* __restrict__ parts, uint32_t n_parts,
                                                             size_t part_stride, void* __restrict__ y, size_t count,
                                                             int out_f32) {
@@ -2046,12 +2099,70 @@ __global__ __launch_bounds__(256) void dense_combine_kernel(const float* __restr
   else static_cast<uint16_t*>(y)[i] = f_to_bf16(acc);
 }
 
-static uint32_t dense_windows(uint32_t ng) { return (ng + kDenseWindow - 1) / kDenseWindow; }
+// windows of a contraction of length k
+static uint32_t dense_windows(uint32_t k, uint32_t max_groups = kDenseWindow) {
+  return std::max(1u, (k / kGroup + max_groups - 1) / max_groups);
+}
 
 // bytes of fp32 window results a projection of n rows over m tokens needs (0: one window, written directly)
 static size_t dense_parts_bytes(uint32_t m, uint32_t n, uint32_t k) {
-  const uint32_t n_win = dense_windows(k / kGroup);
+  const uint32_t n_win = dense_windows(k);
   return n_win > 1 ? up256(sizeof(float) * static_cast<size_t>(m) * n) * n_win : 0;
+}
+// ... and of the gate / up pair of an MLP (both projections of a work item: kQmmRows rows each)
+static uint32_t dense_gate_up_windows(uint32_t d) {
+  return dense_windows(d, kDenseFusedMax);
+}
+static size_t dense_gate_up_parts_bytes(uint32_t t, uint32_t f, uint32_t d) {
+  const uint32_t n_win = dense_gate_up_windows(d);
+  return n_win > 1 ? 2 * up256(sizeof(float) * static_cast<size_t>(t) * f) * n_win : 0;
+}
+
+// The windows of a gate / up pair meet here: sums in window order, gate and up narrowed to bf16
+// (dequant_int4.metal:240-245), act = bf16(silu(gate) * up) written in the matmul's order (0,4,1,5,2,6,3,7 inside
+// every run of 8) with the fp32 sum of every 64-wide group beside it -- what the SwiGLU epilogue of the
+// one-window launch and prep_rows_kernel produce together.  One thread per run of 8.
+__global__ __launch_bounds__(256) void dense_swiglu_combine_kernel(const float* __restrict__ pg, const float* __restrict__ pu,
+                                                                   uint32_t n_parts, size_t part_stride,
+                                                                   uint16_t* __restrict__ act, float* __restrict__ sums,
+                                                                   size_t chunks, float limit) {
+  const size_t c = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+  float g[8], u[8];
+#pragma unroll
+  for (int i = 0; i < 8; ++i) g[i] = u[i] = 0.0f;
+  if (c < chunks) {
+    for (uint32_t p = 0; p < n_parts; ++p) {
+      const float4 g0 = *reinterpret_cast<const float4*>(pg + p * part_stride + c * 8);
+      const float4 g1 = *reinterpret_cast<const float4*>(pg + p * part_stride + c * 8 + 4);
+      const float4 u0 = *reinterpret_cast<const float4*>(pu + p * part_stride + c * 8);
+      const float4 u1 = *reinterpret_cast<const float4*>(pu + p * part_stride + c * 8 + 4);
+      const float gv[8] = {g0.x, g0.y, g0.z, g0.w, g1.x, g1.y, g1.z, g1.w};
+      const float uv[8] = {u0.x, u0.y, u0.z, u0.w, u1.x, u1.y, u1.z, u1.w};
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {
+        g[i] = p == 0 ? gv[i] : g[i] + gv[i];
+        u[i] = p == 0 ? uv[i] : u[i] + uv[i];
+      }
+    }
+  }
+  uint32_t a[8];
+  float v[8];
+#pragma unroll
+  for (int i = 0; i < 8; ++i) {
+    float gr = round_bf16(g[i]), ur = round_bf16(u[i]);
+    if (limit > 0.0f) {
+      gr = fminf(gr, limit);
+      ur = fminf(fmaxf(ur, -limit), limit);
+    }
+    a[i] = f_to_bf16(fast_silu(gr) * ur);
+    v[i] = bf16_to_f(static_cast<uint16_t>(a[i]));
+  }
+  float sum = ((v[0] + v[1]) + (v[2] + v[3])) + ((v[4] + v[5]) + (v[6] + v[7]));
+  sum = group_sum(sum, 8);
+  if (c >= chunks) return;
+  *reinterpret_cast<uint4*>(act + c * 8) = make_uint4(a[0] | (a[4] << 16), a[1] | (a[5] << 16), a[2] | (a[6] << 16),
+                                                      a[3] | (a[7] << 16));
+  if ((c & 7) == 0) sums[c >> 3] = sum;
 }
 
 bool dense_qmm_takes(const mf_qtensor& w, int bits, const void* x, const void* y, uint32_t m, uint32_t n, uint32_t k) {
@@ -2069,7 +2180,7 @@ size_t dense_qmm_workspace_bytes(uint32_t m, uint32_t n, uint32_t k) {
 // x_prepared: rows already in the matmul's order with their group sums in sumx (x is then ignored)
 static hipError_t dense_project(hipStream_t s, const mf_qtensor& w, int bits, const uint16_t* xp, const float* sumx,
                                 void* y, uint32_t m, uint32_t n, uint32_t k, bool out_f32, void* parts) {
-  const uint32_t ng = k / kGroup, n_win = dense_windows(ng);
+  const uint32_t ng = k / kGroup, n_win = dense_windows(k);
   const int code_bits = bits == MF_BITS_4 ? 4 : 2;
   QmmArgs d{};
   d.dense_mode = 1; d.dense_rows = m; d.top_k = 1;
@@ -2119,7 +2230,7 @@ hipError_t launch_dense_qmm(hipStream_t s, const mf_qtensor& w, int bits, const 
 // (gate and up narrowed first, dequant_int4.metal:240-245), then the down projection.
 bool dense_mlp_takes(const mf_qtensor& gate, const mf_qtensor& up, const mf_qtensor& down, const void* x,
                      const void* y, const void* scratch, uint32_t d, uint32_t f, uint32_t t) {
-  if (d % kQmmRows || f % kQmmRows || d / kGroup > kDenseFusedMax || t == 0) return false;
+  if (d % kQmmRows || f % kQmmRows || t == 0) return false;
   return aligned16(gate.weights) && aligned16(up.weights) && aligned16(down.weights) && aligned16(x) && aligned16(y) &&
          aligned16(scratch) && static_cast<uint64_t>(t) * std::max(d, f) < (1ull << 31);
 }
@@ -2127,7 +2238,7 @@ bool dense_mlp_takes(const mf_qtensor& gate, const mf_qtensor& up, const mf_qten
 size_t dense_mlp_scratch_bytes(uint32_t d, uint32_t f, uint32_t t) {
   return up256(sizeof(uint16_t) * static_cast<size_t>(t) * f) + up256(sizeof(uint16_t) * static_cast<size_t>(t) * d) +
          up256(sizeof(float) * static_cast<size_t>(t) * (d / kGroup)) + up256(sizeof(float) * static_cast<size_t>(t) * (f / kGroup)) +
-         dense_parts_bytes(t, d, f);
+         std::max(dense_parts_bytes(t, d, f), dense_gate_up_parts_bytes(t, f, d));  // (the two uses follow one another)
 }
 
 hipError_t launch_dense_mlp(hipStream_t s, const mf_qtensor& gate, const mf_qtensor& up, const mf_qtensor& down,
@@ -2153,10 +2264,32 @@ hipError_t launch_dense_mlp(hipStream_t s, const mf_qtensor& gate, const mf_qten
     q.dense[1].biases = up.scales;
   }
   q.x = xp; q.sumx = sumx; q.x_stride = d; q.rows = f; q.kdim = d; q.epi = 0; q.out = act;
-  e = launch_qmm(s, code_bits, q, 2, (t + kTileTokens - 1) / kTileTokens, nullptr, 0);
-  if (e != hipSuccess) return e;
-  e = launch_prep_rows(s, act, nullptr, sum_act, static_cast<size_t>(t) * f);  // the activations are in matmul order already
-  if (e != hipSuccess) return e;
+  const uint32_t gu_win = dense_gate_up_windows(d);
+  if (gu_win > 1) {
+    // few rows (or a K too long for one launch's scale tables): the contraction in windows, both projections as
+    // fp32 per window, then one pass that adds the windows, activates and sums the groups
+    const uint32_t ng = d / kGroup;
+    const size_t part_stride = up256(sizeof(float) * static_cast<size_t>(t) * f) / sizeof(float);
+    float* pg = reinterpret_cast<float*>(base);
+    float* pu = pg + part_stride * gu_win;
+    uint32_t longest = 0;
+    for (uint32_t wdx = 0; wdx < gu_win; ++wdx)
+      longest = std::max(longest, dense_window_start(ng, gu_win, wdx + 1) - dense_window_start(ng, gu_win, wdx));
+    q.ng_ld = ng; q.kdim = longest * kGroup; q.n_win = gu_win; q.out_win_stride = part_stride;
+    q.epi = 1; q.out = pg; q.out2 = pu;
+    e = launch_qmm(s, code_bits, q, 2, (t + kTileTokens - 1) / kTileTokens, nullptr, 0);
+    if (e != hipSuccess) return e;
+    const size_t chunks = static_cast<size_t>(t) * f / 8;
+    dense_swiglu_combine_kernel<<<dim3(static_cast<uint32_t>((chunks + 255) / 256)), dim3(256), 0, s>>>(
+        pg, pu, gu_win, part_stride, act, sum_act, chunks, 0.0f);
+    e = hipGetLastError();
+    if (e != hipSuccess) return e;
+  } else {
+    e = launch_qmm(s, code_bits, q, 2, (t + kTileTokens - 1) / kTileTokens, nullptr, 0);
+    if (e != hipSuccess) return e;
+    e = launch_prep_rows(s, act, nullptr, sum_act, static_cast<size_t>(t) * f);  // the activations are in matmul order already
+    if (e != hipSuccess) return e;
+  }
   return dense_project(s, down, bits, act, sum_act, y, t, d, f, false, base);
 }
 

@@ -134,7 +134,9 @@ def _close_or_one_step(oracle, got_bits, ref_bits, what):
     assert rel_l2 <= 1e-3 and max_abs <= max(2e-2, step + 1e-9), (what, rel_l2, max_abs, step)
 
 
-@pytest.mark.parametrize("d,f,t", [(2048, 512, 40), (1024, 1536, 128), (5120, 1536, 33)])
+# (d = 7680: 120 K groups, more than one gate/up launch holds tables for -- the contraction goes in two windows
+# that meet in the SwiGLU combine pass)
+@pytest.mark.parametrize("d,f,t", [(2048, 512, 40), (1024, 1536, 128), (5120, 1536, 33), (7680, 256, 70)])
 def test_shared_expert_block_form(gpu, oracle, d, f, t):
     """PrefillSharedExpert.encodeBlock: t >= 32 rows through the matrix cores == the checker's shared
     expert row by row within the layer tolerance; with only t*f of scratch the call goes row by row and

@@ -164,6 +164,7 @@ void prefill_router_mfma_kernel(const uint16_t* __restrict__ W,
                                                                   const RouterTail tail) {
   constexpr int WAVES = 4, kPairs = 32 / WAVES;  // waves of a workgroup, chain pairs of one wave
   __shared__ float s_part[WAVES - 1][16 * 64];
+  __shared__ uint4 s_stage[N_I > 0 ? WAVES : 1][2][N_I > 0 ? 2 * 128 : 1];  // per wave: x and w, two buffers of 32 rows x 64 B
   const uint32_t lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
   if (tail.xp && blockIdx.y >= tail.router_cols) {  // an x-preparation workgroup (rows behind the expert blocks)
     const uint32_t row = ((blockIdx.y - tail.router_cols) * gridDim.x + blockIdx.x) * WAVES + wv;
@@ -182,61 +183,107 @@ void prefill_router_mfma_kernel(const uint16_t* __restrict__ W,
 #pragma unroll
   for (int r = 0; r < 16; ++r) lev0[r] = lev1[r] = lev2[r] = total[r] = 0.0f;
   if constexpr (N_I > 0) {
-    // step q = pp * N_I + i, operands 4 steps ahead in a ring of 8 slots
-    constexpr int kSteps = kPairs * N_I, kAhead = 4;
-    uint4 rx[2 * kAhead], rw[2 * kAhead];
+    // A lane needs 16 bytes of its token row and of its expert row per step -- read straight from memory
+    // that is 32 rows, 32 cache lines, per load instruction, and the L1's line rate, not the matrix core,
+    // sets the pace.  So the wave fetches 64 contiguous bytes of every row at a time (the operands of two
+    // chain pairs: four lanes side by side, 16 lines per instruction) and hands them to itself through a
+    // wave-private LDS buffer.  A stage is (pair group pg, K run i): 2 steps, 16 matrix instructions.  The
+    // two chain pairs of a group keep an accumulator each across the runs.
+    constexpr int kGroups = kPairs / 2, kStages = kGroups * N_I;
+    const uint32_t ld_row = lane >> 2, ld_chunk = lane & 3;  // fetch: rows ld_row, ld_row + 16; 16-byte chunk
+    const uint16_t* xsrc[2];
+    const uint16_t* wsrc[2];
 #pragma unroll
-    for (int q = 0; q < kAhead && q < kSteps; ++q) {
-      rx[q] = *reinterpret_cast<const uint4*>(xrow + 16 * (q / N_I) + 512 * (q % N_I));
-      rw[q] = *reinterpret_cast<const uint4*>(wrow + 16 * (q / N_I) + 512 * (q % N_I));
+    for (int j = 0; j < 2; ++j) {
+      xsrc[j] = x + static_cast<size_t>(min(t0 + ld_row + 16 * j, T - 1)) * x_stride + 8 * (2 * kPairs * wv + ld_chunk);
+      wsrc[j] = W + static_cast<size_t>(e0 + ld_row + 16 * j) * D + 8 * (2 * kPairs * wv + ld_chunk);
     }
-    f32x32_t acc;
+    // LDS rows of 64 bytes; chunk c of row r sits in slot c ^ ((r >> 2) & 3): 16 lanes that read the same
+    // chunk of 16 consecutive rows then cover 256 bytes of distinct banks
+    uint4* stage_x = s_stage[wv][0];
+    uint4* stage_w = s_stage[wv][1];
+    uint32_t st_at[2], rd_at[2];
 #pragma unroll
-    for (int q = 0; q < kSteps; ++q) {
-      if (q + kAhead < kSteps) {
-        const int qa = q + kAhead;
-        rx[qa % (2 * kAhead)] = *reinterpret_cast<const uint4*>(xrow + 16 * (qa / N_I) + 512 * (qa % N_I));
-        rw[qa % (2 * kAhead)] = *reinterpret_cast<const uint4*>(wrow + 16 * (qa / N_I) + 512 * (qa % N_I));
-      }
-      const uint4 cxq = rx[q % (2 * kAhead)], cwq = rw[q % (2 * kAhead)];
-      const uint32_t xw[4] = {cxq.x, cxq.y, cxq.z, cxq.w}, ww[4] = {cwq.x, cwq.y, cwq.z, cwq.w};
-      float xa[8], wa[8];
+    for (int j = 0; j < 2; ++j) {
+      const uint32_t r = ld_row + 16 * j;
+      st_at[j] = r * 4 + (ld_chunk ^ ((r >> 2) & 3));
+      rd_at[j] = m * 4 + ((2 * j + b) ^ ((m >> 2) & 3));  // pair j of the group, block b
+    }
+    typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
+    u32x4_t fx0, fx1, fw0, fw1;  // the stage on its way from memory to LDS
+#define MF_ROUTER_FETCH(ST)                                                                          \
+  do {                                                                                               \
+    const int f_off = 32 * ((ST) / N_I) + 512 * ((ST) % N_I);                                        \
+    fx0 = *reinterpret_cast<const u32x4_t*>(xsrc[0] + f_off);                                        \
+    fx1 = *reinterpret_cast<const u32x4_t*>(xsrc[1] + f_off);                                        \
+    fw0 = *reinterpret_cast<const u32x4_t*>(wsrc[0] + f_off);                                        \
+    fw1 = *reinterpret_cast<const u32x4_t*>(wsrc[1] + f_off);                                        \
+  } while (0)
+#define MF_ROUTER_PUT(BUF)                                                                           \
+  do {                                                                                               \
+    *reinterpret_cast<u32x4_t*>(stage_x + (BUF) * 128 + st_at[0]) = fx0;                             \
+    *reinterpret_cast<u32x4_t*>(stage_x + (BUF) * 128 + st_at[1]) = fx1;                             \
+    *reinterpret_cast<u32x4_t*>(stage_w + (BUF) * 128 + st_at[0]) = fw0;                             \
+    *reinterpret_cast<u32x4_t*>(stage_w + (BUF) * 128 + st_at[1]) = fw1;                             \
+  } while (0)
+    MF_ROUTER_FETCH(0);
+    MF_ROUTER_PUT(0);
+    if (kStages > 1) MF_ROUTER_FETCH(1);
+    f32x32_t acc[2];
 #pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        xa[2 * j] = bf16_lo(xw[j]); xa[2 * j + 1] = bf16_hi(xw[j]);
-        wa[2 * j] = bf16_lo(ww[j]); wa[2 * j + 1] = bf16_hi(ww[j]);
-      }
-      // all 16 operands in registers of their own before the step's first matrix instruction (see below)
-      asm volatile("" : "+v"(xa[0]), "+v"(xa[1]), "+v"(xa[2]), "+v"(xa[3]), "+v"(xa[4]), "+v"(xa[5]), "+v"(xa[6]), "+v"(xa[7]),
-                        "+v"(wa[0]), "+v"(wa[1]), "+v"(wa[2]), "+v"(wa[3]), "+v"(wa[4]), "+v"(wa[5]), "+v"(wa[6]), "+v"(wa[7]));
-      if (q % N_I == 0) {  // a chain's first product lands on 0
-        f32x32_t zero;
+    for (int st = 0; st < kStages; ++st) {
+      const int pg = st / N_I, i = st % N_I;
 #pragma unroll
-        for (int r = 0; r < 32; ++r) zero[r] = 0.0f;
-        acc = __builtin_amdgcn_mfma_f32_32x32x1f32(xa[0], wa[0], zero, 0, 0, 0);
-      } else {
-        acc = __builtin_amdgcn_mfma_f32_32x32x1f32(xa[0], wa[0], acc, 0, 0, 0);
-      }
+      for (int j = 0; j < 2; ++j) {
+        const uint4 cxq = stage_x[(st & 1) * 128 + rd_at[j]], cwq = stage_w[(st & 1) * 128 + rd_at[j]];
+        const uint32_t xw[4] = {cxq.x, cxq.y, cxq.z, cxq.w}, ww[4] = {cwq.x, cwq.y, cwq.z, cwq.w};
+        float xa[8], wa[8];
 #pragma unroll
-      for (int j = 1; j < 8; ++j) acc = __builtin_amdgcn_mfma_f32_32x32x1f32(xa[j], wa[j], acc, 0, 0, 0);
-      if (q % N_I == N_I - 1) {  // the pair of chains is complete: stride-1 level, then the binary counter
-        constexpr int kLevels = kPairs == 8 ? 3 : 2;
-        const int pp = q / N_I;
-        float carry[16];
-#pragma unroll
-        for (int r = 0; r < 16; ++r) carry[r] = acc[r] + acc[16 + r];
-        int level = 0;
-#pragma unroll
-        for (; level < kLevels && ((pp >> level) & 1); ++level) {
-          float* lv = level == 0 ? lev0 : level == 1 ? lev1 : lev2;
-#pragma unroll
-          for (int r = 0; r < 16; ++r) carry[r] = lv[r] + carry[r];
+        for (int u = 0; u < 4; ++u) {
+          xa[2 * u] = bf16_lo(xw[u]); xa[2 * u + 1] = bf16_hi(xw[u]);
+          wa[2 * u] = bf16_lo(ww[u]); wa[2 * u + 1] = bf16_hi(ww[u]);
         }
-        float* dst = level == kLevels ? total : level == 0 ? lev0 : level == 1 ? lev1 : lev2;
+        // all 16 operands in registers of their own before the step's first matrix instruction (see below)
+        asm volatile("" : "+v"(xa[0]), "+v"(xa[1]), "+v"(xa[2]), "+v"(xa[3]), "+v"(xa[4]), "+v"(xa[5]), "+v"(xa[6]), "+v"(xa[7]),
+                          "+v"(wa[0]), "+v"(wa[1]), "+v"(wa[2]), "+v"(wa[3]), "+v"(wa[4]), "+v"(wa[5]), "+v"(wa[6]), "+v"(wa[7]));
+        if (i == 0) {  // a chain's first product lands on 0
+          f32x32_t zero;
 #pragma unroll
-        for (int r = 0; r < 16; ++r) dst[r] = carry[r];
+          for (int r = 0; r < 32; ++r) zero[r] = 0.0f;
+          acc[j] = __builtin_amdgcn_mfma_f32_32x32x1f32(xa[0], wa[0], zero, 0, 0, 0);
+        } else {
+          acc[j] = __builtin_amdgcn_mfma_f32_32x32x1f32(xa[0], wa[0], acc[j], 0, 0, 0);
+        }
+#pragma unroll
+        for (int u = 1; u < 8; ++u) acc[j] = __builtin_amdgcn_mfma_f32_32x32x1f32(xa[u], wa[u], acc[j], 0, 0, 0);
+      }
+      if (st + 1 < kStages) {  // the next stage into the other buffer (read last a stage ago), the one after it on its way
+        MF_ROUTER_PUT((st + 1) & 1);
+        if (st + 2 < kStages) MF_ROUTER_FETCH(st + 2);
+      }
+      if (i == N_I - 1) {  // two pairs of chains are complete: stride-1 level, then the binary counter
+        constexpr int kLevels = kPairs == 8 ? 3 : 2;
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+          const int pp = 2 * pg + j;
+          float carry[16];
+#pragma unroll
+          for (int r = 0; r < 16; ++r) carry[r] = acc[j][r] + acc[j][16 + r];
+          int level = 0;
+#pragma unroll
+          for (; level < kLevels && ((pp >> level) & 1); ++level) {
+            float* lv = level == 0 ? lev0 : level == 1 ? lev1 : lev2;
+#pragma unroll
+            for (int r = 0; r < 16; ++r) carry[r] = lv[r] + carry[r];
+          }
+          float* dst = level == kLevels ? total : level == 0 ? lev0 : level == 1 ? lev1 : lev2;
+#pragma unroll
+          for (int r = 0; r < 16; ++r) dst[r] = carry[r];
+        }
       }
     }
+#undef MF_ROUTER_FETCH
+#undef MF_ROUTER_PUT
   } else {
   // step q = pp * n_i + i: chain pair pp (chains 16 wv + 2 pp + b), K run i; operands run 4 steps ahead
   const uint32_t steps = 8 * n_i;

@@ -208,35 +208,45 @@ def measure_prefill(ctx, w, layer, device, tokens=(128, 512, 2048), steps=100, w
                 routing_bit_exact=bool(np.array_equal(idx[:n_par].cpu().numpy().astype(np.uint32), ref_idx)),
                 max_abs=float(np.abs(got - ref).max()),
                 rel_l2=float(np.linalg.norm(got - ref) / np.linalg.norm(ref)))
-        # the layer call is eleven launches: replayed from a HIP graph (ten calls per graph) so that
+        # the layer call is several launches: replayed from a HIP graph (ten calls per graph) so that
         # short batches measure the kernels and not the host's launch rate
         per_graph = 10 if use_graph else 1
-        def calls():
-            for _ in range(per_graph):
-                moe.encode_prefill_layer(lw, x, y, t, workspace=ws)
-        go = calls
-        if use_graph:
-            side = torch.cuda.Stream()
-            side.wait_stream(torch.cuda.current_stream())
-            with torch.cuda.stream(side):
-                calls()
-            torch.cuda.current_stream().wait_stream(side)
+
+        def timed_us():
+            def calls():
+                for _ in range(per_graph):
+                    moe.encode_prefill_layer(lw, x, y, t, workspace=ws)
+            go = calls
+            if use_graph:
+                side = torch.cuda.Stream()
+                side.wait_stream(torch.cuda.current_stream())
+                with torch.cuda.stream(side):
+                    calls()
+                torch.cuda.current_stream().wait_stream(side)
+                torch.cuda.synchronize()
+                graph = torch.cuda.CUDAGraph()
+                with torch.cuda.graph(graph):
+                    calls()
+                go = graph.replay
+            reps = max(1, steps // per_graph)
+            for _ in range(max(1, warmup // per_graph)):
+                go()
             torch.cuda.synchronize()
-            graph = torch.cuda.CUDAGraph()
-            with torch.cuda.graph(graph):
-                calls()
-            go = graph.replay
-        reps = max(1, steps // per_graph)
-        for _ in range(max(1, warmup // per_graph)):
-            go()
-        torch.cuda.synchronize()
-        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-        e0.record()
-        for _ in range(reps):
-            go()
-        e1.record()
-        torch.cuda.synchronize()
-        us = e0.elapsed_time(e1) / (reps * per_graph) * 1e3
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            for _ in range(reps):
+                go()
+            e1.record()
+            torch.cuda.synchronize()
+            return e0.elapsed_time(e1) / (reps * per_graph) * 1e3
+
+        us = timed_us()
+        if not w.get("maple"):
+            # the reference's prefill rule: a route's result is a 16-bit number before its weight (half the
+            # bytes between the down projection and the reduce); the default keeps fp32 as the decode step does
+            moe.set_prefill_route_rounding(True)
+            run["us_per_layer_routes_bf16"] = round(timed_us(), 1)
+            moe.set_prefill_route_rounding(False)
         flops = 2.0 * 3 * w["d"] * (t * w["k"] * w["f"] + t * w["fs"])
         tflops = flops / us / 1e6
         # algorithmic bytes of the call: the experts that got a token + the shared expert + router, once each,

@@ -547,6 +547,16 @@ mf_status mf_moe_prefill_layer(mf_moe* h, mf_stream stream, const mf_moe_layer_w
                                const uint16_t* x, uint32_t t, uint16_t* y, void* workspace,
                                size_t workspace_bytes, uint32_t* out_idx, float* out_w);
 
+/* How mf_moe_prefill_layer rounds a route's down-projection result before it meets its routing weight.
+ * narrow = 0 (default): kept in fp32, as the decode step keeps it (moe.metal:1262-1270) -- prefill and
+ * decode then agree to the last rounding of the sum.  narrow = 1: narrowed to a 16-bit number first, the
+ * rule of the reference's prefill kernels (prefill_moe_int4_down_route_partials writes 16-bit
+ * route_partials, prefill_moe_reduce_token_major reads them, Metal/Prefill/prefill.metal:817-819,
+ * 644-651; 16-bit is bf16 here, as everywhere on this path): half the bytes between the down projection
+ * and the reduce.  A handle with maple_rounding narrows either way (maple_moe.metal:258) and always
+ * stores 16-bit results.  mf_moe_ragged_qmm's route_partials stay fp32. */
+mf_status mf_moe_set_prefill_route_rounding(mf_moe* h, int narrow);
+
 
 /* The two halves of the ragged layer on their own, for callers that hold a grouping already.
  *

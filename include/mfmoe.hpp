@@ -361,6 +361,7 @@ class MoE {
     check(mf_moe_unpermute(h_, cb, routePartials, routeWeights, indices, residual, tokens, h2), ctx_);
   }
   void setFused(bool enabled) const { check(mf_moe_set_fused(h_, enabled ? 1 : 0), ctx_); }
+  void setPrefillRouteRounding(bool narrow) const { check(mf_moe_set_prefill_route_rounding(h_, narrow ? 1 : 0), ctx_); }
   void status(mf_stream cb) const { check(mf_moe_status(h_, cb), ctx_); }
 
  private:

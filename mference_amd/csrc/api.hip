@@ -646,6 +646,12 @@ mf_status mf_moe_set_fused(mf_moe* h, int enabled) {
   return MF_OK;
 }
 
+mf_status mf_moe_set_prefill_route_rounding(mf_moe* h, int narrow) {
+  if (!h) return MF_ERR_INVALID_ARGUMENT;
+  h->narrow_routes = narrow != 0;
+  return MF_OK;
+}
+
 mf_status mf_moe_set_phase_trace(mf_moe* h, uint64_t* device_buffer, size_t bytes) {
   if (!h) return MF_ERR_INVALID_ARGUMENT;
   if (device_buffer && bytes < static_cast<size_t>(h->ctx->num_cu) * 8 * sizeof(uint64_t))

@@ -38,6 +38,7 @@ struct mf_moe {
   mf_moe_config cfg{};
   bool fused = true;  // mf_moe_set_fused
   bool generic_shape = false;  // mf_moe_set_fused(h, 2): the fused launch through the instance that reads every dimension from its arguments
+  bool narrow_routes = false;  // mf_moe_set_prefill_route_rounding
   unsigned long long* trace = nullptr;  // mf_moe_set_phase_trace
   size_t trace_bytes = 0;
   void* ws_base = nullptr;

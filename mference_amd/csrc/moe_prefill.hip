@@ -153,9 +153,10 @@ typedef __attribute__((ext_vector_type(32))) float f32x32_t;
 // vector instructions per matrix instruction where the loop for any width (N_I = 0) issues 10.6, and the
 // matrix instructions of a SIMD wait for its vector instructions (T=2048: 38.6 -> 34.1 us, T=512: 18.5 ->
 // 14.8 us).  (The unrolled form needs 123 registers; eight waves of 8 chains per block, four to a SIMD,
-// measured no faster than these four of 16 chains: 34.7 / 15.8 us.)
+// measured no faster than these four of 16 chains: 34.7 / 15.8 us.)  Three waves per SIMD: the x-preparation
+// workgroups behind the router's then share the CUs with them instead of waiting for a second round (-1.3 us).
 template <int N_I>
-__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2)))
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(N_I > 0 ? 3 : 2, N_I > 0 ? 3 : 2)))
 void prefill_router_mfma_kernel(const uint16_t* __restrict__ W,
                                                                   const uint16_t* __restrict__ x,
                                                                   uint32_t E, uint32_t D, uint32_t T,
@@ -982,7 +983,8 @@ struct QmmArgs {
   uint32_t n_win;
   size_t out_win_stride;
   // epilogue
-  int epi;              // 0 swiglu -> bf16 [pair, rows] in prep order; 1 fp32 [token*K+rank, rows]; 2 bf16 [pair, rows]
+  int epi;              // 0 swiglu -> bf16 [pair, rows] in prep order; 1 fp32 [token*K+rank, rows]; 2 bf16 [pair, rows];
+                        // 3 bf16 [token*K+rank, rows]
   int narrow;           // shared-expert rounding points (dequant_int4.metal:240-245)
   int tab_aligned;      // scale / bias rows start on 16-byte boundaries (set by the launcher)
   int ternary;          // 2-bit codes {0,1,2} with bias = -scale: b_off / dense[].biases name the SCALE table
@@ -1133,7 +1135,7 @@ void qmm_kernel(const QmmLaunch launch) {
       xrow[0] = a.sorted[ti_pair[0]].token;
       xrow[1] = a.sorted[ti_pair[1]].token;
     }
-    if (a.epi == 1) slot = pr.token * a.top_k + pr.rank;
+    if (a.epi == 1 || a.epi == 3) slot = pr.token * a.top_k + pr.rank;
   }
   const uint8_t* wrow[NPROJ];
   QmmCodes<BITS> cur[NPROJ][4];
@@ -1558,7 +1560,7 @@ void qmm_kres_kernel(const KresLaunch launch) {
   if (threadIdx.x < kTileTokens) {
     const uint32_t pi = pair_start + min(threadIdx.x, count - 1);
     slot = pi;
-    if (!a.dense_mode && a.epi == 1) {
+    if (!a.dense_mode && (a.epi == 1 || a.epi == 3)) {
       const mf_pair pr = a.sorted[pi];
       slot = pr.token * a.top_k + pr.rank;
     }
@@ -1751,6 +1753,7 @@ void qmm_kres_kernel(const KresLaunch launch) {
 // y[t,d] = bf16(h1[t,d] + sum_r w[t,r] * partial[t*K+r, d]), residual first, rank
 // order, product then add (moe.metal:1262-1270; reduce of prefill.metal:631-652).
 // h1 = bf16(hs / (1 + exp(-gate_t))) when a scalar gate is given (utility.metal:49-59).
+template <bool NARROW>  // the per-route results are bf16 numbers (stored as such) instead of fp32
 __global__ __launch_bounds__(256) void prefill_reduce_kernel(const float* __restrict__ partials,
                                                              const float* __restrict__ w,
                                                              const uint32_t* __restrict__ idx,
@@ -1782,14 +1785,20 @@ __global__ __launch_bounds__(256) void prefill_reduce_kernel(const float* __rest
     if (r < K) {
       ex[r] = idx ? idx[t * K + r] : 0u;
       wt[r] = w[t * K + r];
-      v[r] = *reinterpret_cast<const float4*>(partials + (static_cast<size_t>(t) * K + r) * D + d);
+      if constexpr (NARROW) {
+        const uint2 q = *reinterpret_cast<const uint2*>(reinterpret_cast<const uint16_t*>(partials) +
+                                                        (static_cast<size_t>(t) * K + r) * D + d);
+        v[r] = make_float4(bf16_lo(q.x), bf16_hi(q.x), bf16_lo(q.y), bf16_hi(q.y));
+      } else {
+        v[r] = *reinterpret_cast<const float4*>(partials + (static_cast<size_t>(t) * K + r) * D + d);
+      }
     }
   }
 #pragma unroll
   for (uint32_t r = 0; r < MF_MAX_TOPK; ++r) {
     if (r < K && ex[r] < E) {  // a route without an expert adds nothing
       float4 q = v[r];
-      if (maple) {  // maple_moe.metal:258: the down output is a bf16 number before its weight
+      if (maple && !NARROW) {  // maple_moe.metal:258: the down output is a bf16 number before its weight
         q.x = round_bf16(q.x); q.y = round_bf16(q.y); q.z = round_bf16(q.z); q.w = round_bf16(q.w);
       }
       const float p0 = wt[r] * q.x, p1 = wt[r] * q.y, p2 = wt[r] * q.z, p3 = wt[r] * q.w;
@@ -2429,7 +2438,7 @@ hipError_t launch_unpermute(hipStream_t s, const mf_moe_config& c, const float* 
                             const uint32_t* idx, const uint16_t* residual, uint32_t t, uint16_t* y) {
   const size_t n4 = static_cast<size_t>(t) * c.d / 4;
   if (!n4) return hipSuccess;
-  prefill_reduce_kernel<<<dim3(static_cast<uint32_t>((n4 + 255) / 256)), dim3(256), 0, s>>>(
+  prefill_reduce_kernel<false><<<dim3(static_cast<uint32_t>((n4 + 255) / 256)), dim3(256), 0, s>>>(
       partials, w, idx, residual, nullptr, y, t, c.top_k, c.d, c.num_experts, static_cast<int>(c.maple_rounding));
   return hipGetLastError();
 }
@@ -2544,7 +2553,13 @@ hipError_t launch_prefill_layer(hipStream_t s, const mf_moe& h, const mf_moe_lay
   // phase 2: routed down -> fp32 partials [token*K+rank, D]; shared down -> hs [token, D]
   q.w_off[0] = w.offsets.down_w; q.s_off[0] = w.offsets.down_s; q.b_off[0] = ternary ? w.offsets.down_s : w.offsets.down_b;
   q.w_off[1] = q.s_off[1] = q.b_off[1] = 0;
-  q.x = ws.acts; q.sumx = ws.sum_acts; q.x_stride = c.f; q.gather = 0; q.rows = c.d; q.kdim = c.f; q.epi = 1; q.out = ws.partials;
+  // Per-route results as bf16 numbers where the rounding rule narrows them anyway before they meet their
+  // weights -- MapleMoE's (maple_moe.metal:258), or on request (mf_moe_set_prefill_route_rounding; the
+  // reference's prefill keeps 16-bit per-route results, prefill.metal:817-819, 644-651): half the bytes
+  // written here and read by the reduce.  The caller's buffer of a ragged call stays fp32.
+  const bool narrow_routes = !ragged && (c.maple_rounding || h.narrow_routes);
+  q.x = ws.acts; q.sumx = ws.sum_acts; q.x_stride = c.f; q.gather = 0; q.rows = c.d; q.kdim = c.f;
+  q.epi = narrow_routes ? 3 : 1; q.out = ws.partials;
   q.limit = 0.0f;
   q.trace = nullptr;
   q.pair_rows = c.d % (2 * kQmmRows) == 0;
@@ -2586,8 +2601,13 @@ hipError_t launch_prefill_layer(hipStream_t s, const mf_moe& h, const mf_moe_lay
     if (want_gate) gate = ws.gate;
   }
   const size_t n4 = static_cast<size_t>(t) * c.d / 4;
-  prefill_reduce_kernel<<<dim3(static_cast<uint32_t>((n4 + 255) / 256)), dim3(256), 0, s>>>(
-      ws.partials, ws.w, ws.idx, hs, gate, y, t, c.top_k, c.d, c.num_experts, static_cast<int>(c.maple_rounding));
+  const dim3 reduce_grid(static_cast<uint32_t>((n4 + 255) / 256));
+  if (narrow_routes)
+    prefill_reduce_kernel<true><<<reduce_grid, dim3(256), 0, s>>>(ws.partials, ws.w, ws.idx, hs, gate, y, t, c.top_k, c.d,
+                                                                  c.num_experts, static_cast<int>(c.maple_rounding));
+  else
+    prefill_reduce_kernel<false><<<reduce_grid, dim3(256), 0, s>>>(ws.partials, ws.w, ws.idx, hs, gate, y, t, c.top_k, c.d,
+                                                                   c.num_experts, static_cast<int>(c.maple_rounding));
   MF_TRY(hipGetLastError());
 #undef MF_TRY
   return hipSuccess;

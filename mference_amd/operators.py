@@ -381,6 +381,11 @@ class MoE:
         launch through the instance that reads every dimension from its arguments"""
         check(_capi.lib().mf_moe_set_fused(self._h, int(enabled)), self.context.handle)
 
+    def set_prefill_route_rounding(self, narrow: bool) -> None:
+        """per-route down results of the prefill layer narrowed to bf16 before their routing weights (True: the
+        reference's prefill rule, prefill.metal:817-819) or kept in fp32 as the decode step keeps them (False)"""
+        check(_capi.lib().mf_moe_set_prefill_route_rounding(self._h, 1 if narrow else 0), self.context.handle)
+
     def set_phase_trace(self, buffer: Optional[torch.Tensor]) -> None:
         """int64 device tensor of num_cu*8 entries receiving per-workgroup stage
         timestamps of the fused launch (100 MHz clock); None switches it off"""

@@ -821,7 +821,8 @@ int mfo_moe_layer(const mfo_layer* L, const uint16_t* x, uint16_t* y, uint32_t* 
     if (!rc)
       for (size_t i = 0; i < d; ++i) {
         /* maple_moe.metal:258: the down output is a bf16 number before it meets its weight */
-        float partial = w[s] * (L->maple_rounding ? bf16r(v[i]) : v[i]);
+        /* prefill.metal:817-819: the prefill kernels keep a route's result as a 16-bit number */
+        float partial = w[s] * (L->maple_rounding || L->narrow_routes ? bf16r(v[i]) : v[i]);
         acc[i] += partial;
       }
   }

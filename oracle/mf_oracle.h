@@ -170,6 +170,9 @@ typedef struct {
   /* the scalar shared gate as an 8-bit affine row [1,d] (RealForwardRunner.swift:2925-2941,
    * dequant_int8.metal:66-107); used instead of w_sg when gqw != NULL */
   const uint8_t* gqw; const uint16_t* gqs; const uint16_t* gqb;
+  /* a route's down output narrowed to a 16-bit number (bf16) before it meets its weight, the rule of the
+   * reference's prefill kernels (prefill.metal:817-819 writes 16-bit route_partials, :644-651 reads them) */
+  int narrow_routes;
 } mfo_layer;
 
 /* one token through router -> routed experts -> shared expert -> combine.

@@ -54,6 +54,7 @@ class _Layer(C.Structure):
         ("sdw", C.c_void_p), ("sds", C.c_void_p), ("sdb", C.c_void_p),
         ("w_sg", C.c_void_p), ("maple_rounding", C.c_int), ("gate_group", C.c_int),
         ("gqw", C.c_void_p), ("gqs", C.c_void_p), ("gqb", C.c_void_p),
+        ("narrow_routes", C.c_int),
     ]
 
 
@@ -418,6 +419,7 @@ class Layer:
     maple_rounding: bool = False    # MapleMoE's activation and bf16 down outputs
     gate_group: int = GROUP         # group of the routed gate tables (32: the DeepSeek-V4 conversion)
     w_sg_q8: Optional["QTensor"] = None  # the scalar gate as an 8-bit affine row [1, d] (replaces w_sg)
+    narrow_routes: bool = False     # a route's down output narrowed to bf16 before its weight (prefill.metal:817-819)
 
     def _struct(self) -> _Layer:
         L = _Layer()
@@ -425,6 +427,7 @@ class Layer:
         L.bits, L.shared_bits = self.bits, self.shared_bits
         L.router_mode, L.swiglu_limit = self.router_mode, self.swiglu_limit
         L.maple_rounding = 1 if self.maple_rounding else 0
+        L.narrow_routes = 1 if self.narrow_routes else 0
         L.gate_group = self.gate_group
         L.router_w = self.router_w.ctypes.data
         L.experts = self.experts.ctypes.data

@@ -217,3 +217,48 @@ def test_ragged_qmm_refuses_a_grouping_that_does_not_fit(gpu, oracle):
         odd.encode_streamed_batched(wts.experts, wts.offsets, xd, sorted_pairs, counts, partials, t)
     assert err.value.status == -2
     torch.cuda.synchronize()
+
+
+@pytest.mark.parametrize("bits,d,f,e,k,t", [(4, 512, 256, 32, 8, 200),     # down projection with K = 256 (x tile resident)
+                                            (4, 256, 1024, 16, 4, 150),    # ... with K = 1024 (x tile ring)
+                                            (2, 256, 128, 16, 4, 70)])
+def test_prefill_route_rounding_narrows_every_route(gpu, oracle, bits, d, f, e, k, t):
+    """mf_moe_set_prefill_route_rounding(h, 1): the layer call gives, bit for bit, what narrowing the fp32
+    per-route results of the ragged call to bf16 and reducing them in rank order gives; it agrees with the
+    checker under the same rule; and it differs from the default somewhere."""
+    root = ROOT_SEED + 0xB700 + d + f
+    layer = oracle.synth_layer(root, d, f, e, k, bits=bits, fs=0)
+    x = oracle.synth_x(root, t, d)
+    moe = make_moe(gpu, layer)
+    wts = to_device_layer(layer)
+    xd = ops.bf16_tensor(x)
+    idx = torch.zeros((t, k), dtype=torch.int32, device="cuda")
+    w = torch.zeros((t, k), dtype=torch.float32, device="cuda")
+    y_wide = torch.zeros((t, d), dtype=torch.bfloat16, device="cuda")
+    moe.encode_prefill_layer(wts, xd, y_wide, t, out_indices=idx, out_weights=w)
+    moe.set_prefill_route_rounding(True)
+    y = torch.zeros_like(y_wide)
+    moe.encode_prefill_layer(wts, xd, y, t)
+    moe.set_prefill_route_rounding(False)
+
+    sorted_pairs = torch.zeros((t * k, 4), dtype=torch.int32, device="cuda")
+    offsets = torch.zeros(e, dtype=torch.int32, device="cuda")
+    counts = torch.zeros(e, dtype=torch.int32, device="cuda")
+    moe.encode_group(idx, w, t, sorted_pairs, offsets, counts)
+    partials = torch.zeros((t * k, d), dtype=torch.float32, device="cuda")
+    moe.encode_streamed_batched(wts.experts, wts.offsets, xd, sorted_pairs, counts, partials, t)
+    torch.cuda.synchronize()
+    moe.group_status()
+    q = oracle.bf16_to_float(oracle.bf16_bits(partials.cpu().numpy())).astype(np.float32).reshape(t, k, d)
+    w_h = w.cpu().numpy()
+    acc = np.zeros((t, d), dtype=np.float32)
+    for r in range(k):
+        acc = acc + (w_h[:, r:r + 1] * q[:, r, :]).astype(np.float32)
+    assert np.array_equal(ops.bf16_bits(y), oracle.bf16_bits(acc))
+    assert not np.array_equal(ops.bf16_bits(y), ops.bf16_bits(y_wide))
+
+    layer.narrow_routes = True
+    rows = np.random.default_rng(t).choice(t, size=24, replace=False)
+    ref_y, ref_idx, _ = oracle.moe_layer(layer, x[rows])
+    assert np.array_equal(idx.cpu().numpy().astype(np.uint32)[rows], ref_idx)
+    assert_layer_close(oracle.bf16_to_float(ops.bf16_bits(y)[rows]), oracle.bf16_to_float(ref_y), "narrow routes")

@@ -720,3 +720,25 @@ def test_layer_with_int8_scalar_gate_matches_its_bf16_twin():
         got = O.router_logits_int8(codes, scales, biases, x[i], ones)[0]
         ref = float(w64 @ O.bf16_to_float(x[i]).astype(np.float64))
         assert abs(got - ref) <= 1e-5 * max(1.0, abs(ref))
+
+
+def test_layer_with_narrow_routes_rounds_each_route(oracle):
+    """narrow_routes: a route's down output is a bf16 number before it meets its weight -- rebuilt here from
+    the per-route functions (prefill.metal:817-819, 644-651)"""
+    d, f, e, k = 128, 64, 8, 4
+    layer = oracle.synth_layer(0x5EED0000 + 0x7A0, d, f, e, k, bits=4, fs=0)
+    x = oracle.synth_x(0x5EED0000 + 0x7A0, 3, d)
+    layer.narrow_routes = True
+    y, idx, w = oracle.moe_layer(layer, x)
+    for t in range(3):
+        acc = np.zeros(d, dtype=np.float32)
+        for r in range(k):
+            ex = int(idx[t, r])
+            acts = oracle.expert_phase1(layer.experts[ex], layer.off, 4, d, f, x[t])
+            v = oracle.expert_down(layer.experts[ex], layer.off, 4, d, f, acts)
+            v = oracle.bf16_to_float(oracle.bf16_bits(v)).astype(np.float32)
+            acc = acc + (np.float32(w[t, r]) * v).astype(np.float32)
+        assert np.array_equal(oracle.bf16_bits(acc), y[t])
+    layer.narrow_routes = False
+    y0, _, _ = oracle.moe_layer(layer, x)
+    assert not np.array_equal(y0, y)

@@ -207,6 +207,18 @@ mf_status mf_shared_expert(mf_ctx* ctx, mf_stream stream, const uint16_t* x, mf_
                            uint32_t t, uint16_t* y, uint16_t* scratch_act,
                            size_t scratch_act_bytes);
 
+/* SharedExpertInt8.encode (Kernels/MoE/SharedExpertInt8.swift:78-181; SharedExpertInt4's bits == 8 case,
+ * SharedExpertInt4.swift:187): the dense MLP on 8-bit affine tensors (MF_BITS_8: one code per byte, bf16
+ * scale and bias per 64).  gate and up rows in one launch (shared_int8_gate_up_act_simd,
+ * Metal/Quant/dequant_int8.metal:110-164): both narrowed to 16 bits, act[f] = narrow(a(gate) * up) with
+ * a = the tanh form of GELU (int8_gelu_pytorch_tanh, :44-49) or, silu_activation != 0, SiLU
+ * (FC_SHARED_INT8_ACT_SILU, :51-57); then y[d] = narrow(down . act) (dequant_int8_gemv_simd, :66-107).
+ * Any t; scratch_act holds t*f bf16.  tanh is built on this library's exp (as every exp on this path). */
+mf_status mf_shared_expert_int8(mf_ctx* ctx, mf_stream stream, const uint16_t* x, mf_qtensor gate,
+                                mf_qtensor up, mf_qtensor down, uint32_t d, uint32_t f, uint32_t t,
+                                int silu_activation, uint16_t* y, uint16_t* scratch_act,
+                                size_t scratch_act_bytes);
+
 /* mf_shared_expert for callers that cannot allocate device memory and bring no scratch buffer:
  * code under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc.
  * It has no counterpart in the reference, whose operators always take the caller's scratch buffer.

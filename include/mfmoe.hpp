@@ -220,6 +220,24 @@ class SharedExpertInt4 {
   mf_bits bits_;
 };
 
+// SharedExpertInt8 (Kernels/MoE/SharedExpertInt8.swift:78-181): the dense MLP on 8-bit affine tensors; the
+// activation is the tanh form of GELU, or SiLU with siluActivation
+class SharedExpertInt8 {
+ public:
+  explicit SharedExpertInt8(const MetalContext& context, bool siluActivation = false)
+      : ctx_(context.raw()), silu_(siluActivation) {}
+  void encode(mf_stream commandBuffer, const uint16_t* x, mf_qtensor gate, mf_qtensor up, mf_qtensor down,
+              uint32_t d, uint32_t f, uint16_t* y, uint16_t* scratchAct, size_t scratchActBytes,
+              uint32_t tokens = 1) const {
+    check(mf_shared_expert_int8(ctx_, commandBuffer, x, gate, up, down, d, f, tokens, silu_ ? 1 : 0, y, scratchAct,
+                                scratchActBytes), ctx_);
+  }
+
+ private:
+  mf_ctx* ctx_;
+  bool silu_;
+};
+
 // MPPPrefillInt4QMM (Kernels/TensorCore/MPPPrefillInt4QMM.swift:34-78): y[m, n] = x[m, k] . deq(W[n, k])^T.
 // encode returns the path like the reference: Unavailable for sizes or offsets it rejects.
 class MPPPrefillInt4QMM {

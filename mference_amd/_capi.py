@@ -83,6 +83,7 @@ SIGNATURES = {
     "mf_shared_expert": (_I, [_P, _P, _P, QTensor, QTensor, QTensor, _I, _U32, _U32, _U32, _P, _P,
                               _SZ]),
     "mf_shared_expert_scratch_bytes": (_SZ, [_U32, _U32, _U32]),
+    "mf_shared_expert_int8": (_I, [_P, _P, _P, QTensor, QTensor, QTensor, _U32, _U32, _U32, _I, _P, _P, _SZ]),
     "mf_qmm_workspace_bytes": (_SZ, [_U32, _U32, _U32]),
     "mf_qmm": (_I, [_P, _P, QTensor, _I, _P, _P, _U32, _U32, _U32, _I, _P, _SZ]),
     "mf_qmm_path": (_I, [QTensor, _I, _P, _P, _U32, _U32, _U32, _P, _SZ]),

@@ -207,6 +207,28 @@ mf_status mf_shared_expert(mf_ctx* ctx, mf_stream stream, const uint16_t* x, mf_
   return MF_OK;
 }
 
+mf_status mf_shared_expert_int8(mf_ctx* ctx, mf_stream stream, const uint16_t* x, mf_qtensor gate, mf_qtensor up,
+                                mf_qtensor down, uint32_t d, uint32_t f, uint32_t t, int silu_activation,
+                                uint16_t* y, uint16_t* scratch_act, size_t scratch_act_bytes) {
+  if (!ctx || !x || !y || !scratch_act) return MF_ERR_INVALID_ARGUMENT;
+  if (d == 0 || f == 0 || d % MF_GROUP_SIZE != 0 || f % MF_GROUP_SIZE != 0) return MF_ERR_DIMENSION_MISMATCH;
+  if (t == 0 || t > MF_MAX_ROWS) return MF_ERR_INVALID_ARGUMENT;
+  if (!qtensor_ok(gate, MF_BITS_8) || !qtensor_ok(up, MF_BITS_8) || !qtensor_ok(down, MF_BITS_8))
+    return MF_ERR_INVALID_ARGUMENT;
+  if (!mf::aligned2(x) || !mf::aligned2(y) || !mf::aligned2(scratch_act)) return MF_ERR_INVALID_ARGUMENT;
+  if (scratch_act_bytes < static_cast<size_t>(t) * f * sizeof(uint16_t)) return MF_ERR_SCRATCH_TOO_SMALL;
+  auto s = static_cast<hipStream_t>(stream);
+  // rows in runs that keep the launch's wave count in range
+  const uint32_t step = 1u << 14;
+  for (uint32_t t0 = 0; t0 < t; t0 += step) {
+    const uint32_t tc = std::min<uint32_t>(t - t0, step);
+    uint16_t* act = scratch_act + static_cast<size_t>(t0) * f;
+    MF_HIP(ctx, mf::launch_gate_up_act_q8(s, gate, up, x + static_cast<size_t>(t0) * d, act, f, d, tc, silu_activation != 0));
+    MF_HIP(ctx, mf::launch_gemv(s, down, MF_BITS_8, act, y + static_cast<size_t>(t0) * d, d, f, tc, false));
+  }
+  return MF_OK;
+}
+
 size_t mf_qmm_workspace_bytes(uint32_t m, uint32_t n, uint32_t k) {
   if (m == 0 || n == 0 || k == 0 || k % MF_GROUP_SIZE) return 0;
   return mf::dense_qmm_workspace_bytes(m, n, k);

@@ -736,6 +736,32 @@ __global__ __launch_bounds__(256) void gemv_q8_kernel(const uint8_t* __restrict_
   }
 }
 
+// shared_int8_gate_up_act_simd (dequant_int8.metal:110-164): the gate and up rows of an 8-bit MLP in one pass,
+// both narrowed to 16 bits, act = narrow(activation(gate) * up); the activation is the tanh form of GELU or,
+// with the reference's FC_SHARED_INT8_ACT_SILU, SiLU.  One wave per (token, row), dot_q8_row's lane order.
+template <bool SILU>
+__global__ __launch_bounds__(256) void gate_up_act_q8_kernel(const uint8_t* __restrict__ Wg, const uint16_t* __restrict__ Sg,
+                                                             const uint16_t* __restrict__ Bg, const uint8_t* __restrict__ Wu,
+                                                             const uint16_t* __restrict__ Su, const uint16_t* __restrict__ Bu,
+                                                             const uint16_t* __restrict__ x, uint16_t* __restrict__ act,
+                                                             uint32_t m, uint32_t n, uint32_t t, int aligned) {
+  const uint32_t lane = threadIdx.x & 63;
+  const uint32_t wave = (blockIdx.x * blockDim.x + threadIdx.x) >> 6;
+  if (wave >= m * t) return;
+  const uint32_t tok = wave / m, row = wave % m;
+  const uint32_t ng = n / kGroup;
+  const uint16_t* xt = x + static_cast<size_t>(tok) * n;
+  const float g = dot_q8_row(Wg + static_cast<size_t>(row) * n, Sg + static_cast<size_t>(row) * ng,
+                             Bg + static_cast<size_t>(row) * ng, xt, n, lane, aligned != 0);
+  const float u = dot_q8_row(Wu + static_cast<size_t>(row) * n, Su + static_cast<size_t>(row) * ng,
+                             Bu + static_cast<size_t>(row) * ng, xt, n, lane, aligned != 0);
+  if (lane == 0) {
+    const float gh = round_bf16(g), uh = round_bf16(u);
+    const float a = SILU ? mf_silu(gh) : mf_gelu_tanh(gh);
+    act[static_cast<size_t>(tok) * m + row] = f_to_bf16(a * uh);
+  }
+}
+
 namespace {
 
 template <int BITS, bool ALIGNED>
@@ -1058,6 +1084,25 @@ __global__ __launch_bounds__(256) void residual_rmsnorm_kernel(uint16_t* __restr
   const float inv = 1.0f / __builtin_sqrtf(total / static_cast<float>(d) + eps);
   for (uint32_t i = threadIdx.x; i < d; i += blockDim.x)
     o[i] = f_to_bf16(bf16_to_f(h[i]) * inv * bf16_to_f(weight[i]));
+}
+
+hipError_t launch_gate_up_act_q8(hipStream_t s, const mf_qtensor& gate, const mf_qtensor& up, const uint16_t* x,
+                                 uint16_t* act, uint32_t f, uint32_t d, uint32_t t, bool silu) {
+  const uint64_t waves = static_cast<uint64_t>(f) * t;
+  if (!waves) return hipSuccess;
+  if (waves >= (1ull << 30)) return hipErrorInvalidValue;
+  const int al8 = (reinterpret_cast<uintptr_t>(gate.weights) % 8 == 0) && (reinterpret_cast<uintptr_t>(up.weights) % 8 == 0) &&
+                  d % 8 == 0 && aligned16(x);
+  const dim3 grid(static_cast<uint32_t>((waves + 3) / 4)), block(256);
+  if (silu)
+    gate_up_act_q8_kernel<true><<<grid, block, 0, s>>>(static_cast<const uint8_t*>(gate.weights), gate.scales, gate.biases,
+                                                        static_cast<const uint8_t*>(up.weights), up.scales, up.biases, x,
+                                                        act, f, d, t, al8);
+  else
+    gate_up_act_q8_kernel<false><<<grid, block, 0, s>>>(static_cast<const uint8_t*>(gate.weights), gate.scales, gate.biases,
+                                                         static_cast<const uint8_t*>(up.weights), up.scales, up.biases, x,
+                                                         act, f, d, t, al8);
+  return hipGetLastError();
 }
 
 hipError_t launch_residual_rmsnorm(hipStream_t s, uint16_t* hidden, const uint16_t* delta,

@@ -95,6 +95,17 @@ __device__ __forceinline__ float mf_sqrtsoftplus(float x) {
 // moe.metal:79-84
 __device__ __forceinline__ float mf_silu(float x) { return x / (1.0f + mf_exp(-x)); }
 
+// int8_gelu_pytorch_tanh (Metal/Quant/dequant_int8.metal:44-49): 0.5 x (1 + tanh(c (x + 0.044715 x^3))), the
+// argument clamped to +-20; tanh(z) = 1 - 2 / (exp(2 z) + 1) on this build's exp, the same IEEE sequence as the
+// CPU checker.
+__device__ __forceinline__ float mf_gelu_tanh(float x) {
+  const float x3 = x * x * x;
+  float inner = 0.7978845608028654f * (x + 0.044715f * x3);
+  inner = fminf(fmaxf(inner, -20.0f), 20.0f);
+  const float th = 1.0f - 2.0f / (mf_exp(2.0f * inner) + 1.0f);
+  return 0.5f * x * (1.0f + th);
+}
+
 // MapleMoE's activation (maple_swiglu, maple_moe.metal:153-164): every intermediate is a bf16 number.
 // min / clamp of bf16 numbers against +-7 and |x| stay bf16 numbers, so only the five arithmetic
 // results are narrowed here.

@@ -75,6 +75,8 @@ hipError_t launch_gemv(hipStream_t s, const mf_qtensor& w, int bits, const uint1
 hipError_t launch_gate_up_act(hipStream_t s, const mf_qtensor& gate, const mf_qtensor& up,
                               int bits, const uint16_t* x, uint16_t* act, uint32_t f, uint32_t d,
                               uint32_t t, bool lane_order = false);
+hipError_t launch_gate_up_act_q8(hipStream_t s, const mf_qtensor& gate, const mf_qtensor& up, const uint16_t* x,
+                                 uint16_t* act, uint32_t f, uint32_t d, uint32_t t, bool silu);
 hipError_t launch_residual_rmsnorm(hipStream_t s, uint16_t* hidden, const uint16_t* delta,
                                    const uint16_t* weight, uint16_t* out, uint32_t d, uint32_t t, float eps);
 hipError_t launch_silu_mul(hipStream_t s, const uint16_t* gate, const uint16_t* up, uint16_t* out,

@@ -259,6 +259,24 @@ class SharedExpertInt4:
             gate.n, gate.rows, t, _ptr(y)), self.context.handle)
 
 
+class SharedExpertInt8:
+    """Kernels/MoE/SharedExpertInt8.swift:78-181: the dense MLP on 8-bit affine tensors, GELU (tanh form) by
+    default, SiLU with silu_activation (the reference's siluActivation)."""
+
+    def __init__(self, context: MetalContext, silu_activation: bool = False):
+        self.context = context
+        self.silu_activation = silu_activation
+
+    def encode(self, x: torch.Tensor, gate: QuantizedTensor, up: QuantizedTensor, down: QuantizedTensor,
+               y: torch.Tensor, scratch_act: torch.Tensor, t: int = 1, stream=None) -> None:
+        if not (gate.rows == up.rows and gate.n == up.n and down.rows == gate.n and down.n == gate.rows):
+            raise MfError(-2, f"gate=({gate.rows},{gate.n}) up=({up.rows},{up.n}) down=({down.rows},{down.n})")
+        check(_capi.lib().mf_shared_expert_int8(
+            self.context.handle, _stream(stream), _ptr(x), gate.c(), up.c(), down.c(), gate.n, gate.rows, t,
+            1 if self.silu_activation else 0, _ptr(y), _ptr(scratch_act),
+            scratch_act.numel() * scratch_act.element_size()), self.context.handle)
+
+
 class FamilyRouters:
     """The family-specific routers of the reference's operator classes, stand-alone: every call
     runs the router GEMV into the caller's fp32 `logits` buffer [t, rows] and then the selection.

@@ -78,6 +78,11 @@
  *                                 down functions.  exp is mfo_exp, not Metal's:
  *                                 PARITY UNPINNED where an exp result sits on a
  *                                 bf16 rounding boundary.
+ *   mfo_gelu_tanh,                dequant_int8.metal:44-49, SharedExpertInt8.swift:78-181; the activation
+ *   mfo_shared_expert_int8        checked against fp64 tanh (1e-6), 0, +-large; the MLP against an fp64
+ *                                 composition of the dequantized weights.  tanh is built on mfo_exp:
+ *                                 PARITY UNPINNED against Metal's tanh where a result sits on a bf16
+ *                                 rounding boundary.
  *   mfo_residual_rmsnorm          utility.metal:83-92 + rmsnorm.metal:30-92; closed
  *                                 form, checked on hand-computed rows (3-4-0
  *                                 vector, unit vector, eps only) and fp64 numpy.
@@ -644,6 +649,42 @@ int mfo_gemv_multix(const uint8_t* packed, const uint16_t* scales, const uint16_
 
 /* moe.metal:79-84: x / (1 + exp(-x)) */
 float mfo_silu(float x) { return x / (1.0f + mfo_exp(-x)); }
+
+/* int8_gelu_pytorch_tanh (dequant_int8.metal:44-49) */
+float mfo_gelu_tanh(float x) {
+  const float x3 = x * x * x;
+  float inner = 0.7978845608028654f * (x + 0.044715f * x3);
+  inner = fminf(fmaxf(inner, -20.0f), 20.0f);
+  const float th = 1.0f - 2.0f / (mfo_exp(2.0f * inner) + 1.0f);
+  return 0.5f * x * (1.0f + th);
+}
+
+/* SharedExpertInt8.encode (SharedExpertInt8.swift:78-181): shared_int8_gate_up_act_simd
+ * (dequant_int8.metal:110-164), then dequant_int8_gemv_simd (:66-107) */
+int mfo_shared_expert_int8(const uint8_t* gw, const uint16_t* gs, const uint16_t* gb, const uint8_t* uw,
+                           const uint16_t* us, const uint16_t* ub, const uint8_t* dw, const uint16_t* ds,
+                           const uint16_t* db, size_t d, size_t f, int silu, const uint16_t* x, uint16_t* y) {
+  if (d == 0 || f == 0 || d % GROUP || f % GROUP) return MFO_ERR_ARG;
+  const size_t longest = d > f ? d : f;
+  uint16_t* ones = (uint16_t*)malloc(longest * sizeof(uint16_t));
+  uint16_t* act = (uint16_t*)malloc(f * sizeof(uint16_t));
+  if (!ones || !act) { free(ones); free(act); return MFO_ERR_ARG; }
+  for (size_t i = 0; i < longest; ++i) ones[i] = 0x3F80;
+#pragma omp parallel for schedule(static)
+  for (size_t r = 0; r < f; ++r) {
+    const float g = mfo_dot_int8_laneorder(gw + r * d, gs + r * (d / GROUP), gb + r * (d / GROUP), x, ones, d);
+    const float u = mfo_dot_int8_laneorder(uw + r * d, us + r * (d / GROUP), ub + r * (d / GROUP), x, ones, d);
+    const float gh = mfo_bf16_to_float(mfo_bf16_bits(g)), uh = mfo_bf16_to_float(mfo_bf16_bits(u));
+    const float a = silu ? gh / (1.0f + mfo_exp(-gh)) : mfo_gelu_tanh(gh);
+    act[r] = mfo_bf16_bits(a * uh);
+  }
+#pragma omp parallel for schedule(static)
+  for (size_t r = 0; r < d; ++r)
+    y[r] = mfo_bf16_bits(mfo_dot_int8_laneorder(dw + r * f, ds + r * (f / GROUP), db + r * (f / GROUP), act, ones, f));
+  free(ones);
+  free(act);
+  return 0;
+}
 
 /* maple_swiglu (maple_moe.metal:153-164): every intermediate is a bf16 number */
 static float bf16r(float x) { return mfo_bf16_to_float(mfo_bf16_bits(x)); }

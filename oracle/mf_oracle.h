@@ -129,6 +129,14 @@ int mfo_expert_phase1_gate(const uint8_t* blob, const mfo_expert_offsets* off, i
 int mfo_expert_phase1(const uint8_t* blob, const mfo_expert_offsets* off, int bits,
                       size_t d, size_t f, float swiglu_limit, int maple, const uint16_t* x,
                       uint16_t* acts);
+/* int8_gelu_pytorch_tanh (dequant_int8.metal:44-49) with tanh(z) = 1 - 2 / (mfo_exp(2 z) + 1) */
+float mfo_gelu_tanh(float x);
+/* SharedExpertInt8.encode (SharedExpertInt8.swift:78-181; dequant_int8.metal:66-164) for one token row:
+ * gate / up / down are 8-bit affine tensors [f,d], [f,d], [d,f] with bf16 tables per 64; rows are summed
+ * in the lane order of mfo_dot_int8_laneorder; silu != 0 selects SiLU instead of the tanh GELU */
+int mfo_shared_expert_int8(const uint8_t* gw, const uint16_t* gs, const uint16_t* gb, const uint8_t* uw,
+                           const uint16_t* us, const uint16_t* ub, const uint8_t* dw, const uint16_t* ds,
+                           const uint16_t* db, size_t d, size_t f, int silu, const uint16_t* x, uint16_t* y);
 /* MapleMoE's activation, every intermediate narrowed to bf16 (maple_moe.metal:153-164);
  * selected in mfo_expert_phase1 by maple != 0 (swiglu_limit is ignored then) */
 float mfo_maple_swiglu(float gate_projection, float up_projection);

@@ -372,6 +372,28 @@ def shared_expert(gate: QTensor, up: QTensor, down: QTensor, x_bits) -> np.ndarr
     return y
 
 
+def gelu_tanh(x: float) -> float:
+    """the tanh form of GELU on the build's exp (dequant_int8.metal:44-49)"""
+    fn = lib().mfo_gelu_tanh
+    fn.restype = C.c_float
+    fn.argtypes = [C.c_float]
+    return float(fn(C.c_float(x)))
+
+
+def shared_expert_int8(gate: QTensor, up: QTensor, down: QTensor, x_bits, silu: bool = False) -> np.ndarray:
+    """SharedExpertInt8.encode (SharedExpertInt8.swift:78-181) for one token row; 8-bit affine tensors"""
+    x_bits = _c(x_bits, np.uint16)
+    d, f = gate.n, gate.rows
+    y = np.empty(d, np.uint16)
+    rc = lib().mfo_shared_expert_int8(_p(gate.packed), _p(gate.scales), _p(gate.biases),
+                                      _p(up.packed), _p(up.scales), _p(up.biases),
+                                      _p(down.packed), _p(down.scales), _p(down.biases),
+                                      C.c_size_t(d), C.c_size_t(f), C.c_int(1 if silu else 0), _p(x_bits), _p(y))
+    if rc:
+        raise ValueError("mfo_shared_expert_int8")
+    return y
+
+
 def maple_swiglu(gate: float, up: float) -> float:
     """MapleMoE's activation, every intermediate a bf16 number (maple_moe.metal:153-164)"""
     fn = lib().mfo_maple_swiglu

@@ -1032,3 +1032,27 @@ def test_listed_shape_instance_at_full_size(gpu, oracle, t):
     assert_layer_close(oracle.bf16_to_float(got[1]), oracle.bf16_to_float(ref_y), f"gemma shape t={t}")
     assert np.array_equal(got[1], got[2]) and np.array_equal(got[1], got[0])
     assert np.array_equal(ops.bf16_bits(yg), got[1])
+
+
+@pytest.mark.parametrize("d,f,t,silu", [(256, 128, 1, False), (2816, 2112, 3, False), (512, 1024, 9, True)])
+def test_int8_shared_expert(gpu, oracle, d, f, t, silu):
+    """SharedExpertInt8.encode (SharedExpertInt8.swift:78-181): 8-bit gate / up rows in one launch with the tanh
+    GELU (or SiLU), 8-bit down rows -- the checker's bits (the lane order and the activation are defined)."""
+    rng = oracle.Rng.key(ROOT_SEED + 0x1E8, f"int8-mlp-{d}-{f}")
+    gq = oracle.quantize(rng.normal(0.0, 0.03, f * d).reshape(f, d), 8)
+    uq = oracle.quantize(rng.normal(0.0, 0.03, f * d).reshape(f, d), 8)
+    dq = oracle.quantize(rng.normal(0.0, 0.03, d * f).reshape(d, f), 8)
+    xb = oracle.bf16_bits(rng.normal(0.0, 1.0, t * d).reshape(t, d))
+    ref = np.stack([oracle.shared_expert_int8(gq, uq, dq, xb[i], silu=silu) for i in range(t)])
+    g, u, dn, x = to_device_q(gq), to_device_q(uq), to_device_q(dq), ops.bf16_tensor(xb)
+    op = ops.SharedExpertInt8(gpu, silu_activation=silu)
+    y = torch.zeros((t, d), dtype=torch.bfloat16, device="cuda")
+    scratch = torch.zeros((t, f), dtype=torch.bfloat16, device="cuda")
+    op.encode(x, g, u, dn, y, scratch, t=t)
+    torch.cuda.synchronize()
+    assert np.array_equal(ops.bf16_bits(y), ref)
+    lib = _capi.lib()
+    assert lib.mf_shared_expert_int8(gpu.handle, None, x.data_ptr(), g.c(), u.c(), dn.c(), d, f, t, 0, y.data_ptr(),
+                                     scratch.data_ptr(), t * f * 2 - 2) == -4
+    assert lib.mf_shared_expert_int8(gpu.handle, None, x.data_ptr(), g.c(), u.c(), dn.c(), d + 8, f, t, 0, y.data_ptr(),
+                                     scratch.data_ptr(), t * f * 2) == -2

@@ -742,3 +742,31 @@ def test_layer_with_narrow_routes_rounds_each_route(oracle):
     layer.narrow_routes = False
     y0, _, _ = oracle.moe_layer(layer, x)
     assert not np.array_equal(y0, y)
+
+
+def test_gelu_tanh_and_the_int8_shared_expert(oracle):
+    """mfo_gelu_tanh against the fp64 formula of dequant_int8.metal:44-49 and its limits; mfo_shared_expert_int8
+    against an fp64 composition of the dequantized 8-bit tensors (SharedExpertInt8.swift:78-181)."""
+    for x in (-30.0, -6.0, -1.5, -0.25, 0.0, 0.3, 1.0, 2.5, 7.0, 40.0):
+        want = 0.5 * x * (1.0 + math.tanh(max(-20.0, min(20.0, 0.7978845608028654 * (x + 0.044715 * x ** 3)))))
+        assert abs(oracle.gelu_tanh(x) - want) <= 1e-6 * max(1.0, abs(want)), x
+    assert oracle.gelu_tanh(0.0) == 0.0 and oracle.gelu_tanh(40.0) == 40.0 and oracle.gelu_tanh(-40.0) == 0.0
+    d, f = 128, 192
+    rng = oracle.Rng.key(0x5EED0000 + 0x1E8, "int8-mlp")
+    gq = oracle.quantize(rng.normal(0.0, 0.05, f * d).reshape(f, d), 8)
+    uq = oracle.quantize(rng.normal(0.0, 0.05, f * d).reshape(f, d), 8)
+    dq = oracle.quantize(rng.normal(0.0, 0.05, d * f).reshape(d, f), 8)
+    x = oracle.bf16_bits(rng.normal(0.0, 1.0, d))
+    xf = oracle.bf16_to_float(x).astype(np.float64)
+    wg, wu, wd = (oracle.dequantize(q).astype(np.float64) for q in (gq, uq, dq))
+    for silu in (False, True):
+        y = oracle.bf16_to_float(oracle.shared_expert_int8(gq, uq, dq, x, silu=silu)).astype(np.float64)
+        g = oracle.bf16_to_float(oracle.bf16_bits((wg @ xf).astype(np.float32))).astype(np.float64)
+        u = oracle.bf16_to_float(oracle.bf16_bits((wu @ xf).astype(np.float32))).astype(np.float64)
+        a = g / (1.0 + np.exp(-g)) if silu else 0.5 * g * (1.0 + np.tanh(0.7978845608028654 * (g + 0.044715 * g ** 3)))
+        act = oracle.bf16_to_float(oracle.bf16_bits((a * u).astype(np.float32))).astype(np.float64)
+        want = wd @ act
+        # (the dequantized weights carry two roundings the kernel's s * (q . x) + b * sum(x) form does not:
+        # a bf16 ulp on outputs of this size)
+        assert np.abs(y - want).max() <= 2e-2 * max(1.0, np.abs(want).max()), (silu, np.abs(y - want).max())
+    assert not np.array_equal(oracle.shared_expert_int8(gq, uq, dq, x), oracle.shared_expert_int8(gq, uq, dq, x, silu=True))

@@ -180,9 +180,14 @@ def measure_prefill(ctx, w, layer, device, tokens=(128, 512, 2048), steps=100, w
     moe = ops.MoE(ctx, w["d"], w["f"], w["e"], w["k"], bits=w["bits"], shared_f=w["fs"],
                   shared_bits=w["shared_bits"], maple_rounding=bool(w.get("maple")),
                   router_mode=ops.ROUTER_FULL_SOFTMAX if full_softmax else ops.ROUTER_TOPK_SOFTMAX)
+    # the routed experts a second time, in the prefill matmul's own order (mf_moe_tile_experts): what the layer
+    # call reads when it is given; same bits as from the row-by-row pool
+    lw.experts_tiled = moe.tile_experts(layer.experts, layer.offsets)
     qwen = w["config"] == QWEN["config"]
     import re
     out = {"launch": "hip_graph" if use_graph else "eager",
+           "expert_pool": "tiled copy of the layer's experts (mf_moe_tile_experts, +%d MB of HBM for this layer); "
+                          "us_per_layer_row_by_row_pool is the same call without it" % (layer.experts.numel() >> 20),
            "workload": ("qwen3.6-35b-a3b-moe-layer-ragged-prefill-4bit-g64" if qwen
                         else re.sub(r"-T\d+$", "", w["name"]).replace("decode", "ragged-prefill")) + ", skewed routing",
            "dtype": "u%d codes (exact, as bf16) x bf16 activations on bf16 MFMA, fp32 accumulate"
@@ -241,6 +246,10 @@ def measure_prefill(ctx, w, layer, device, tokens=(128, 512, 2048), steps=100, w
             return e0.elapsed_time(e1) / (reps * per_graph) * 1e3
 
         us = timed_us()
+        tiled = lw.experts_tiled
+        lw.experts_tiled = None
+        run["us_per_layer_row_by_row_pool"] = round(timed_us(), 1)
+        lw.experts_tiled = tiled
         if not w.get("maple"):
             # the reference's prefill rule: a route's result is a 16-bit number before its weight (half the
             # bytes between the down projection and the reduce); the default keeps fp32 as the decode step does

@@ -446,6 +446,10 @@ typedef struct {
                                * Metal/Quant/dequant_int8.metal:66-107).  Used when w_sg_q8.weights != NULL
                                * (w_sg is then ignored); all three pointers zero: w_sg decides.  The gate
                                * logit is the mf_gemv(MF_BITS_8) value of that row, narrowed to bf16. */
+  const void* expert_tiled;   /* NULL, or a second copy of the expert pool in the prefill matmul's own order
+                               * (mf_moe_tile_experts: same stride, same offsets).  mf_moe_prefill_layer reads the
+                               * routed experts from it when it is given (and the configuration takes the
+                               * matrix-core path); the decode calls never do.  Same results, bit for bit. */
 } mf_moe_layer_weights;
 
 /* The fused decode layer, one launch: router -> top-k -> routed gate/up/act ->
@@ -558,6 +562,18 @@ size_t mf_moe_prefill_workspace_bytes(const mf_moe* h, uint32_t t);
 mf_status mf_moe_prefill_layer(mf_moe* h, mf_stream stream, const mf_moe_layer_weights* wts,
                                const uint16_t* x, uint32_t t, uint16_t* y, void* workspace,
                                size_t workspace_bytes, uint32_t* out_idx, float* out_w);
+
+/* A copy of the expert pool for the prefill matmuls.  The reference repacks a model's experts once, offline,
+ * into the layout its kernels read best (MferenceRepack, RepackPlanner.swift:414-651); the counterpart here
+ * is done at load time on the device: `tiled` (expert_stride * num_experts bytes, 16-byte aligned, not
+ * overlapping the source) receives every blob with its three code sub-tensors re-ordered so that a load
+ * instruction of the matrix-core matmul reads consecutive bytes (inside a sub-tensor: blocks of 32 rows, K
+ * group by K group, the 64 half-group pieces of a block and group side by side); tables, offsets and stride
+ * are unchanged.  Costs a second pool in HBM (Qwen shape: 453 MB per layer) and buys 4..7 % of a prefill
+ * layer.  Needs the matrix-core configuration (mf_moe_prefill_workspace_bytes(h, t) != 0), else
+ * MF_ERR_DIMENSION_MISMATCH. */
+mf_status mf_moe_tile_experts(mf_moe* h, mf_stream stream, const void* expert_base, size_t expert_stride,
+                              const mf_expert_offsets* offsets, void* tiled);
 
 /* How mf_moe_prefill_layer rounds a route's down-projection result before it meets its routing weight.
  * narrow = 0 (default): kept in fp32, as the decode step keeps it (moe.metal:1262-1270) -- prefill and

@@ -379,6 +379,11 @@ class MoE {
     check(mf_moe_unpermute(h_, cb, routePartials, routeWeights, indices, residual, tokens, h2), ctx_);
   }
   void setFused(bool enabled) const { check(mf_moe_set_fused(h_, enabled ? 1 : 0), ctx_); }
+  // a copy of the expert pool in the prefill matmul's own order (mf_moe_layer_weights.expert_tiled)
+  void tileExperts(mf_stream cb, const void* expertBase, size_t expertStride, const mf_expert_offsets& offsets,
+                   void* tiled) const {
+    check(mf_moe_tile_experts(h_, cb, expertBase, expertStride, &offsets, tiled), ctx_);
+  }
   void setPrefillRouteRounding(bool narrow) const { check(mf_moe_set_prefill_route_rounding(h_, narrow ? 1 : 0), ctx_); }
   void status(mf_stream cb) const { check(mf_moe_status(h_, cb), ctx_); }
 

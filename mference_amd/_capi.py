@@ -57,6 +57,7 @@ class LayerWeights(C.Structure):
         ("shared_gate", QTensor), ("shared_up", QTensor), ("shared_down", QTensor),
         ("w_sg", C.c_void_p),
         ("w_sg_q8", QTensor),
+        ("expert_tiled", C.c_void_p),
     ]
 
 
@@ -105,6 +106,7 @@ SIGNATURES = {
     "mf_moe_decode_layer": (_I, [_P, _P, C.POINTER(LayerWeights), _P, _U32, _P, _P, _P, _P]),
     "mf_moe_set_fused": (_I, [_P, _I]),
     "mf_moe_set_prefill_route_rounding": (_I, [_P, _I]),
+    "mf_moe_tile_experts": (_I, [_P, _P, _P, _SZ, C.POINTER(ExpertOffsets), _P]),
     "mf_moe_status": (_I, [_P, _P]),
     "mf_moe_set_phase_trace": (_I, [_P, _P, _SZ]),
     "mf_ctx_num_cu": (_I, [_P]),

@@ -760,7 +760,7 @@ mf_status mf_moe_prefill_layer(mf_moe* h, mf_stream stream, const mf_moe_layer_w
   if ((!wts->router_w && (!out_idx || !out_w)) || !wts->expert_base || !offsets_ok(wts->offsets, c.bits) ||
       !mf::aligned16(wts->expert_base) || wts->expert_stride % 16 || offs % 16 ||
       !mf::aligned16(wts->router_w) || !mf::aligned16(x) || !mf::aligned16(y) ||
-      !mf::aligned16(workspace))
+      !mf::aligned16(workspace) || !mf::aligned16(wts->expert_tiled))
     return MF_ERR_INVALID_ARGUMENT;
   if (c.shared_f && (!qtensor_ok(wts->shared_gate, c.shared_bits) ||
                      !qtensor_ok(wts->shared_up, c.shared_bits) ||
@@ -793,6 +793,23 @@ mf_status mf_moe_ragged_qmm(mf_moe* h, mf_stream stream, const void* expert_base
     return MF_ERR_INVALID_ARGUMENT;
   MF_HIP(h->ctx, mf::launch_ragged_qmm(static_cast<hipStream_t>(stream), *h, expert_base, expert_stride, *offsets,
                                        x, sorted_pairs, expert_counts, t, route_partials, workspace));
+  return MF_OK;
+}
+
+mf_status mf_moe_tile_experts(mf_moe* h, mf_stream stream, const void* expert_base, size_t expert_stride,
+                              const mf_expert_offsets* offsets, void* tiled) {
+  if (!h || !expert_base || !offsets || !tiled) return MF_ERR_INVALID_ARGUMENT;
+  const mf_moe_config& c = h->cfg;
+  if (!mf::prefill_supported(c)) return MF_ERR_DIMENSION_MISMATCH;
+  const uint32_t offs = offsets->gate_w | offsets->up_w | offsets->down_w;
+  if (!offsets_ok(*offsets, c.bits) || !mf::aligned16(expert_base) || !mf::aligned16(tiled) || expert_stride % 16 ||
+      offs % 16)
+    return MF_ERR_INVALID_ARGUMENT;
+  const auto* a = static_cast<const uint8_t*>(expert_base);
+  const auto* b = static_cast<const uint8_t*>(tiled);
+  const size_t bytes = expert_stride * c.num_experts;
+  if (a < b + bytes && b < a + bytes) return MF_ERR_INVALID_ARGUMENT;  // the copy is not done in place
+  MF_HIP(h->ctx, mf::launch_tile_experts(static_cast<hipStream_t>(stream), c, expert_base, expert_stride, *offsets, tiled));
   return MF_OK;
 }
 

@@ -142,6 +142,8 @@ hipError_t launch_group(hipStream_t s, const uint32_t* idx, const float* w, uint
                         uint32_t* status, uint32_t* chunk_hist);
 size_t group_scratch_words();
 size_t prefill_workspace_bytes(const mf_moe_config& c, uint32_t t);
+hipError_t launch_tile_experts(hipStream_t s, const mf_moe_config& c, const void* src, size_t expert_stride,
+                               const mf_expert_offsets& off, void* dst);
 bool prefill_supported(const mf_moe_config& c);
 hipError_t launch_prefill_layer(hipStream_t s, const mf_moe& h, const mf_moe_layer_weights& w,
                                 const uint16_t* x, uint32_t t, uint16_t* y, void* workspace,

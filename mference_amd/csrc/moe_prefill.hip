@@ -872,6 +872,49 @@ __global__ __launch_bounds__(MF_MAX_EXPERTS) void group_place_kernel(const uint3
   }
 }
 
+// ---- the expert pool in the matmul's order
+// A lane of the matmul reads half a K group of ONE weight row per load (16 bytes of 4-bit codes, 8 of 2-bit):
+// row by row that is 32 rows, 32 memory lines, per load instruction, and the L1's line rate is a large part
+// of what a work item costs (Qwen shape, 2048 tokens: layer 273 -> 255 us with the loads below).  In the
+// tiled pool every sub-tensor keeps its place in the blob and its size; inside it, the pieces of the 32 rows
+// of a block for one K group sit side by side in lane order: piece (row block rb, group g, lane l = m + 32 h)
+// = row 32 rb + m, bytes [g * GB + h * GB / 2, + GB / 2) of the row, GB = 32 (4-bit) or 16 (2-bit, ternary)
+// bytes per group.  A load instruction then reads 1 KB (512 B) of consecutive bytes.  Scale and bias tables
+// stay row by row.  One thread per piece; sub-tensor w of every expert in one launch.
+__global__ __launch_bounds__(256) void tile_codes_kernel(const uint8_t* __restrict__ src, uint8_t* __restrict__ dst,
+                                                         size_t expert_stride, uint32_t w_off, uint32_t rows,
+                                                         uint32_t ng, uint32_t group_bytes) {
+  const uint32_t half = group_bytes / 2;
+  const uint64_t pieces = static_cast<uint64_t>(rows) * ng * 2;
+  const uint64_t i = static_cast<uint64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+  if (i >= pieces) return;
+  const uint32_t l = static_cast<uint32_t>(i & 63u), m = l & 31u, h = l >> 5;
+  const uint64_t bg = i >> 6;  // rb * ng + g
+  const uint32_t g = static_cast<uint32_t>(bg % ng), rb = static_cast<uint32_t>(bg / ng);
+  const size_t base = static_cast<size_t>(blockIdx.y) * expert_stride + w_off;
+  const uint8_t* from = src + base + (static_cast<size_t>(32u * rb + m) * ng + g) * group_bytes + h * half;
+  uint8_t* to = dst + base + i * half;
+  if (half == 16) *reinterpret_cast<uint4*>(to) = *reinterpret_cast<const uint4*>(from);
+  else *reinterpret_cast<uint2*>(to) = *reinterpret_cast<const uint2*>(from);
+}
+
+// dst = the pool `src` (E blobs, expert_stride apart) with the three code sub-tensors of every blob tiled
+hipError_t launch_tile_experts(hipStream_t s, const mf_moe_config& c, const void* src, size_t expert_stride,
+                               const mf_expert_offsets& off, void* dst) {
+  hipError_t e = hipMemcpyAsync(dst, src, expert_stride * c.num_experts, hipMemcpyDeviceToDevice, s);
+  if (e != hipSuccess) return e;
+  const uint32_t gb = c.bits == MF_BITS_4 ? 32u : 16u;
+  const struct { uint32_t off, rows, k; } parts[3] = {{off.gate_w, c.f, c.d}, {off.up_w, c.f, c.d}, {off.down_w, c.d, c.f}};
+  for (const auto& p : parts) {
+    const uint64_t pieces = static_cast<uint64_t>(p.rows) * (p.k / kGroup) * 2;
+    tile_codes_kernel<<<dim3(static_cast<uint32_t>((pieces + 255) / 256), c.num_experts), dim3(256), 0, s>>>(
+        static_cast<const uint8_t*>(src), static_cast<uint8_t*>(dst), expert_stride, p.off, p.rows, p.k / kGroup, gb);
+    e = hipGetLastError();
+    if (e != hipSuccess) return e;
+  }
+  return hipSuccess;
+}
+
 // --------------------------------------------------------------- the matmul
 
 // Activation rows as the matmul wants them: inside every run of 8 K values the
@@ -962,6 +1005,7 @@ struct QmmArgs {
   uint32_t w_off[2], s_off[2], b_off[2];
   mf_qtensor dense[2];
   int pair_rows;        // 1: the NPROJ blocks of a wave are consecutive 32-row blocks of projection 0
+  int tiled;            // 1: the routed experts' codes are in the matmul's own order (tile_codes_kernel), not row by row
   int dense_mode;       // 1: the "expert" is dense[], tiles are runs of consecutive rows
   uint32_t dense_rows;  // number of x rows in dense mode
   // activations: rows of kdim bf16 in prep_rows_kernel order + their group sums [row, kdim/64]
@@ -1138,12 +1182,16 @@ void qmm_kernel(const QmmLaunch launch) {
     if (a.epi == 1 || a.epi == 3) slot = pr.token * a.top_k + pr.rank;
   }
   const uint8_t* wrow[NPROJ];
+  const uint32_t gstride = a.tiled ? 32u * kGB : kGB;  // bytes from a group's codes to the next group's
   QmmCodes<BITS> cur[NPROJ][4];
 #pragma unroll
   for (int p = 0; p < NPROJ; ++p) {
-    wrow[p] = Wp[p] + (row_base[p] + m) * row_bytes + static_cast<size_t>(g_off) * kGB + h * (kGB / 2);
+    // row by row: the lane's half group of its row, groups kGB apart.  Tiled: the 32 rows' pieces of a group are
+    // one run of 64 x kGB / 2 bytes in lane order (one load instruction reads 1 KB of consecutive bytes)
+    wrow[p] = a.tiled ? Wp[p] + row_base[p] * row_bytes + static_cast<size_t>(g_off) * gstride + lane * (kGB / 2)
+                      : Wp[p] + (row_base[p] + m) * row_bytes + static_cast<size_t>(g_off) * gstride + h * (kGB / 2);
 #pragma unroll
-    for (int u = 0; u < 4; ++u) cur[p][u].load(wrow[p] + min(static_cast<uint32_t>(u), ng - 1) * kGB);
+    for (int u = 0; u < 4; ++u) cur[p][u].load(wrow[p] + min(static_cast<uint32_t>(u), ng - 1) * gstride);
   }
   // x rows of groups 0..2 and, for the bias terms, the group sums of the lane's two routes
   const uint16_t* st_src = a.x + static_cast<size_t>(st_row) * a.x_stride + static_cast<size_t>(g_off) * kGroup + st_q * 16;
@@ -1349,7 +1397,7 @@ void qmm_kernel(const QmmLaunch launch) {
           group_products<BITS, NTA>(cur[p][2 * uu + gi], bx, tmp, [](int) {});
           // the register that held this group's codes takes those of the group four ahead
           // (past the end the last group is read again: no branch inside the unrolled body)
-          cur[p][2 * uu + gi].load(wrow[p] + min(g + 4, ng - 1) * kGB);
+          cur[p][2 * uu + gi].load(wrow[p] + min(g + 4, ng - 1) * gstride);
 #pragma unroll
           for (int nt = 0; nt < NTA; ++nt)
 #pragma unroll
@@ -1534,7 +1582,9 @@ void qmm_kres_kernel(const KresLaunch launch) {
   constexpr uint32_t kRowBytes = NG * kGB;
   // the lane's weight row of block p of slice w: row0 + 256 w + 32 p
   const uint32_t row0 = (slice0 * kQmmWaves + wv) * 64 + m;
-  const uint8_t* wrow = W + static_cast<size_t>(row0) * kRowBytes + h * (kGB / 2);
+  const uint32_t gstride = a.tiled ? 32u * kGB : kGB;
+  const uint8_t* wrow = a.tiled ? W + static_cast<size_t>(row0 - m) * kRowBytes + lane * (kGB / 2)
+                                : W + static_cast<size_t>(row0) * kRowBytes + h * (kGB / 2);
   const uint16_t* srow = Sp + static_cast<size_t>(row0) * NG;
   const uint16_t* brow = Bp + static_cast<size_t>(row0) * NG;
 
@@ -1543,7 +1593,7 @@ void qmm_kres_kernel(const KresLaunch launch) {
 #pragma unroll
   for (int p = 0; p < 2; ++p)
 #pragma unroll
-    for (int u = 0; u < kRing; ++u) cur[p][u].load(wrow + p * 32 * kRowBytes + u * kGB);
+    for (int u = 0; u < kRing; ++u) cur[p][u].load(wrow + p * 32 * kRowBytes + u * gstride);
   uint4 nS[2], nB[2];
 #pragma unroll
   for (int p = 0; p < 2; ++p) {
@@ -1690,8 +1740,8 @@ void qmm_kres_kernel(const KresLaunch launch) {
         });
         // the register takes the codes kRing groups on: of this slice, or of the next one
         const int ahead = g + kRing;
-        cur[p][g % kRing].load(ahead < NG ? wrow + p * 32 * kRowBytes + ahead * kGB
-                                          : wnext + p * 32 * kRowBytes + (ahead - NG) * kGB);
+        cur[p][g % kRing].load(ahead < NG ? wrow + p * 32 * kRowBytes + ahead * gstride
+                                          : wnext + p * 32 * kRowBytes + (ahead - NG) * gstride);
 #pragma unroll
         for (int nt = 0; nt < NTA; ++nt)
 #pragma unroll
@@ -2510,7 +2560,9 @@ hipError_t launch_prefill_layer(hipStream_t s, const mf_moe& h, const mf_moe_lay
   if (gate_q8) MF_TRY(launch_gemv(s, w.w_sg_q8, MF_BITS_8, x, ws.gate, 1, c.d, t, false));
 
   QmmArgs q{};
-  q.expert_base = static_cast<const uint8_t*>(w.expert_base);
+  // the routed experts' blobs: the pool in the matmul's order when the caller built one (mf_moe_tile_experts)
+  q.expert_base = static_cast<const uint8_t*>(w.expert_tiled ? w.expert_tiled : w.expert_base);
+  q.tiled = w.expert_tiled != nullptr;
   q.expert_stride = w.expert_stride;
   q.sorted = ws.sorted;
   q.tiles = ws.tiles;

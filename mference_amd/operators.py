@@ -347,6 +347,7 @@ class MoELayerWeights:
     shared: Optional[Sequence[QuantizedTensor]] = None  # gate, up, down
     w_sg: Optional[torch.Tensor] = None    # bf16 [d]
     w_sg_q8: Optional[QuantizedTensor] = None  # the scalar gate as an 8-bit affine row [1, d] (replaces w_sg)
+    experts_tiled: Optional[torch.Tensor] = None  # uint8 [e, stride]: the pool in the prefill matmul's order (MoE.tile_experts)
 
     def c(self) -> _capi.LayerWeights:
         if self.experts.ndim != 2 or self.experts.stride(1) != 1:
@@ -362,6 +363,10 @@ class MoELayerWeights:
         L.w_sg = _ptr(self.w_sg)
         if self.w_sg_q8 is not None:
             L.w_sg_q8 = self.w_sg_q8.c()
+        if self.experts_tiled is not None:
+            if self.experts_tiled.shape != self.experts.shape or self.experts_tiled.stride(0) != self.experts.stride(0):
+                raise MfError(-1, "experts_tiled must have the pool's shape and stride")
+            L.expert_tiled = _ptr(self.experts_tiled)
         return L
 
 
@@ -398,6 +403,14 @@ class MoE:
         """single fused launch (True / 1, default) or the chain of separate launches (False / 0); 2: the fused
         launch through the instance that reads every dimension from its arguments"""
         check(_capi.lib().mf_moe_set_fused(self._h, int(enabled)), self.context.handle)
+
+    def tile_experts(self, experts: torch.Tensor, offsets: ExpertOffsets, stream=None) -> torch.Tensor:
+        """a copy of the expert pool [e, stride] in the prefill matmul's own order (mf_moe_tile_experts): pass it
+        as MoELayerWeights.experts_tiled"""
+        out = torch.empty_like(experts)
+        check(_capi.lib().mf_moe_tile_experts(self._h, _stream(stream), _ptr(experts), experts.stride(0),
+                                              C.byref(offsets), _ptr(out)), self.context.handle)
+        return out
 
     def set_prefill_route_rounding(self, narrow: bool) -> None:
         """per-route down results of the prefill layer narrowed to bf16 before their routing weights (True: the

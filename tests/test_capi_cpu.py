@@ -154,7 +154,7 @@ def _c_layout(tmp_path):
         "mf_moe_config": ["d", "f", "num_experts", "top_k", "bits", "router_mode", "swiglu_limit",
                           "shared_f", "shared_bits", "maple_rounding", "gate_group_size"],
         "mf_moe_layer_weights": ["router_w", "expert_base", "expert_stride", "offsets",
-                                 "shared_gate", "shared_up", "shared_down", "w_sg", "w_sg_q8"],
+                                 "shared_gate", "shared_up", "shared_down", "w_sg", "w_sg_q8", "expert_tiled"],
     }
     lines = ['#include <stdio.h>', '#include <stddef.h>', '#include "mfmoe.h"', 'int main(void){']
     for s, fields in structs.items():

@@ -471,3 +471,46 @@ def test_non_finite_token_takes_sentinel_routes(gpu, oracle, d, f, t):
     moe.status()
     assert np.array_equal(idd.cpu().numpy().astype(np.uint32), np.stack([ref_idx[r] for r in (2, 3, 4)]))
     assert (ops.bf16_bits(yd)[1] == 0).all()
+
+
+@pytest.mark.parametrize("bits,d,f,e,k,fs,t,mode", [
+    (4, 2048, 512, 256, 8, 512, 300, 0),   # the headline shape: K = 2048 through the ring, K = 512 resident
+    (4, 256, 1024, 16, 4, 128, 150, 0),    # down projection through the ring kernel (K = 1024)
+    (4, 384, 128, 32, 2, 128, 131, 1),     # K groups not a multiple of 8
+    (2, 512, 256, 32, 6, 256, 200, 0),     # 2-bit codes: 8-byte pieces
+    (1, 1024, 512, 64, 8, 0, 77, 1),       # ternary
+])
+def test_prefill_from_the_tiled_pool_gives_the_same_bits(gpu, oracle, bits, d, f, e, k, fs, t, mode):
+    """mf_moe_tile_experts: the expert pool in the matmul's own order (a second copy; codes re-ordered inside
+    each sub-tensor, tables in place) -- the prefill layer reads it and writes the bits it writes from the
+    row-by-row pool; a decode call with the same weights struct ignores it."""
+    root = ROOT_SEED + 0x711E + bits + d
+    layer = oracle.synth_layer(root, d, f, e, k, bits=bits, fs=fs, router_mode=mode)
+    x = oracle.synth_x(root, t, d)
+    moe = make_moe(gpu, layer)
+    wts = to_device_layer(layer)
+    y0, idx0, w0 = _run_prefill(moe, wts, x, t, d, k)
+    tiled = moe.tile_experts(wts.experts, wts.offsets)
+    torch.cuda.synchronize()
+    assert not torch.equal(tiled, wts.experts)
+    # tables and everything outside the three code sub-tensors are copied as they are
+    off = wts.offsets
+    assert torch.equal(tiled[:, off.gate_s:off.gate_s + f * (d // 64) * 2], wts.experts[:, off.gate_s:off.gate_s + f * (d // 64) * 2])
+    wts.experts_tiled = tiled
+    y1, idx1, w1 = _run_prefill(moe, wts, x, t, d, k)
+    assert np.array_equal(idx0, idx1) and np.array_equal(w0.view(np.uint32), w1.view(np.uint32))
+    assert np.array_equal(y0, y1)
+    # decode ignores the tiled pool
+    xd = ops.bf16_tensor(x[:3])
+    ya = torch.zeros((3, d), dtype=torch.bfloat16, device="cuda")
+    yb = torch.zeros_like(ya)
+    moe.encode_decode_layer(wts, xd, ya, 3)
+    wts.experts_tiled = None
+    moe.encode_decode_layer(wts, xd, yb, 3)
+    torch.cuda.synchronize()
+    assert torch.equal(ya, yb)
+    # in place is refused
+    lib = _capi.lib()
+    import ctypes as C
+    assert lib.mf_moe_tile_experts(moe._h, None, wts.experts.data_ptr(), wts.experts.stride(0), C.byref(wts.offsets),
+                                   wts.experts.data_ptr()) == -1

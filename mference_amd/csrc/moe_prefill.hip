@@ -1127,7 +1127,10 @@ void qmm_kernel(const QmmLaunch launch) {
     pair_start = tile_id * kTileTokens;
     count = min(kTileTokens, a.dense_rows - pair_start);
   } else {
-    const Tile t = a.tiles[tile_id];
+    // (the whole 16-byte record in one load: read field by field, the count was fetched, tested, and the rest
+    // fetched in a second round trip)
+    const uint4 tv = *reinterpret_cast<const uint4*>(a.tiles + tile_id);
+    const Tile t{tv.x, tv.y, tv.z, tv.w};
     if (t.count == 0) return;
     expert = t.expert;
     pair_start = t.pair_start;
@@ -1172,14 +1175,17 @@ void qmm_kernel(const QmmLaunch launch) {
   const uint32_t ti_pair[2] = {pair_start + min(m, count - 1), pair_start + min(32 + m, count - 1)};
   uint32_t st_row = st_pair, xrow[2] = {ti_pair[0], ti_pair[1]};
   uint32_t slot = pair_start + min(threadIdx.x & 63u, count - 1);
+  // the routes' records are requested here and looked at behind the code loads below, which do not depend on
+  // them: the first codes are then on their way one memory round trip earlier
+  mf_pair pr{};
+  uint32_t tok_st = 0, tok_0 = 0, tok_1 = 0;
   if (!a.dense_mode) {
-    const mf_pair pr = a.sorted[slot];
+    pr = a.sorted[slot];
     if (a.gather) {
-      st_row = a.sorted[st_pair].token;
-      xrow[0] = a.sorted[ti_pair[0]].token;
-      xrow[1] = a.sorted[ti_pair[1]].token;
+      tok_st = a.sorted[st_pair].token;
+      tok_0 = a.sorted[ti_pair[0]].token;
+      tok_1 = a.sorted[ti_pair[1]].token;
     }
-    if (a.epi == 1 || a.epi == 3) slot = pr.token * a.top_k + pr.rank;
   }
   const uint8_t* wrow[NPROJ];
   const uint32_t gstride = a.tiled ? 32u * kGB : kGB;  // bytes from a group's codes to the next group's
@@ -1192,6 +1198,15 @@ void qmm_kernel(const QmmLaunch launch) {
                       : Wp[p] + (row_base[p] + m) * row_bytes + static_cast<size_t>(g_off) * gstride + h * (kGB / 2);
 #pragma unroll
     for (int u = 0; u < 4; ++u) cur[p][u].load(wrow[p] + min(static_cast<uint32_t>(u), ng - 1) * gstride);
+  }
+  __builtin_amdgcn_sched_barrier(0);  // (keeps the look at the routes behind the code loads)
+  if (!a.dense_mode) {
+    if (a.gather) {
+      st_row = tok_st;
+      xrow[0] = tok_0;
+      xrow[1] = tok_1;
+    }
+    if (a.epi == 1 || a.epi == 3) slot = pr.token * a.top_k + pr.rank;
   }
   // x rows of groups 0..2 and, for the bias terms, the group sums of the lane's two routes
   const uint16_t* st_src = a.x + static_cast<size_t>(st_row) * a.x_stride + static_cast<size_t>(g_off) * kGroup + st_q * 16;
@@ -1556,7 +1571,10 @@ void qmm_kres_kernel(const KresLaunch launch) {
     pair_start = tile_id * kTileTokens;
     count = min(kTileTokens, a.dense_rows - pair_start);
   } else {
-    const Tile t = a.tiles[tile_id];
+    // (the whole 16-byte record in one load: read field by field, the count was fetched, tested, and the rest
+    // fetched in a second round trip)
+    const uint4 tv = *reinterpret_cast<const uint4*>(a.tiles + tile_id);
+    const Tile t{tv.x, tv.y, tv.z, tv.w};
     if (t.count == 0) return;
     expert = t.expert;
     pair_start = t.pair_start;

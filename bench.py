@@ -161,7 +161,8 @@ def pmc_calibration(device) -> str:
     return "3 x 256 MiB device-to-device copy (reads 268435456 B, writes 268435456 B)"
 
 
-def measure_prefill(ctx, w, layer, device, tokens=(128, 512, 2048), steps=100, warmup=100, use_graph=True):
+def measure_prefill(ctx, w, layer, device, tokens=(128, 512, 2048), steps=100, warmup=100, use_graph=True,
+                    side_runs=True):
     """Ragged prefill of one layer of the same shape: T tokens, top-k routing from skewed
     logits (router weights plus a per-expert bias ~ N(0, 1.5), carried by a constant-one last
     feature of x and the last column of the router, so expert loads are uneven and some
@@ -246,11 +247,12 @@ def measure_prefill(ctx, w, layer, device, tokens=(128, 512, 2048), steps=100, w
             return e0.elapsed_time(e1) / (reps * per_graph) * 1e3
 
         us = timed_us()
-        tiled = lw.experts_tiled
-        lw.experts_tiled = None
-        run["us_per_layer_row_by_row_pool"] = round(timed_us(), 1)
-        lw.experts_tiled = tiled
-        if not w.get("maple"):
+        if side_runs:
+            tiled = lw.experts_tiled
+            lw.experts_tiled = None
+            run["us_per_layer_row_by_row_pool"] = round(timed_us(), 1)
+            lw.experts_tiled = tiled
+        if side_runs and not w.get("maple"):
             # the reference's prefill rule: a route's result is a 16-bit number before its weight (half the
             # bytes between the down projection and the reduce); the default keeps fp32 as the decode step does
             moe.set_prefill_route_rounding(True)
@@ -818,6 +820,9 @@ def main() -> int:
     ap.add_argument("--no-prefill", action="store_true", help="skip the ragged prefill section")
     ap.add_argument("--no-other-configs", action="store_true",
                     help="skip the short runs of the other BASELINE configurations that the default run appends")
+    ap.add_argument("--no-side-runs", action="store_true",
+                    help="with --prefill-only: time the layer call as it is reported (tiled expert pool, fp32 per-route "
+                         "results) only, not the row-by-row pool and the 16-bit per-route results beside it (for profiling)")
     ap.add_argument("--prefill-only", action="store_true",
                     help="one layer, the ragged prefill section only (for profiling)")
     ap.add_argument("--phase-trace", action="store_true",
@@ -858,6 +863,7 @@ def main() -> int:
     if args.prefill_only:
         tokens = (args.tokens,) if args.tokens else (128, 512, 2048)
         res = {"prefill": measure_prefill(ctx, w, stack[0], device, tokens=tokens, steps=min(args.steps, 100),
+                                          side_runs=not args.no_side_runs,
                                           warmup=min(args.warmup, 100), use_graph=not args.no_graph)}
         if args.pmc_calibration:
             res["pmc_calibration"] = pmc_calibration(device)

@@ -500,6 +500,14 @@ def test_prefill_from_the_tiled_pool_gives_the_same_bits(gpu, oracle, bits, d, f
     y1, idx1, w1 = _run_prefill(moe, wts, x, t, d, k)
     assert np.array_equal(idx0, idx1) and np.array_equal(w0.view(np.uint32), w1.view(np.uint32))
     assert np.array_equal(y0, y1)
+    # ... also with 16-bit per-route results
+    moe.set_prefill_route_rounding(True)
+    y2, _, _ = _run_prefill(moe, wts, x, t, d, k)
+    wts.experts_tiled = None
+    y3, _, _ = _run_prefill(moe, wts, x, t, d, k)
+    moe.set_prefill_route_rounding(False)
+    wts.experts_tiled = tiled
+    assert np.array_equal(y2, y3)
     # decode ignores the tiled pool
     xd = ops.bf16_tensor(x[:3])
     ya = torch.zeros((3, d), dtype=torch.bfloat16, device="cuda")

@@ -990,6 +990,52 @@ def main() -> int:
                      "algorithmic_bytes_per_layer": ab["expert_bytes"]},
     }
 
+    if use_graph and args.workload == "qwen-decode":
+        # the layer with the step in front of it (hidden += delta, RMSNorm): one launch (mf_moe_decode_layer_normed)
+        # against mf_residual_rmsnorm + mf_moe_decode_layer, the same 40 layers replayed from a graph
+        hid = torch.randn((L, w["t"], w["d"]), generator=gen, device=device).to(torch.bfloat16)
+        dlt = (torch.randn((L, w["t"], w["d"]), generator=gen, device=device) * 0.1).to(torch.bfloat16)
+        nw = torch.ones((w["d"],), dtype=torch.bfloat16, device=device)
+        xn = torch.zeros_like(hid)
+        norm = ops.RMSNorm(ctx)
+
+        def step_two():
+            for l in range(L):
+                norm.encode_bf16w(hid[l], nw, xn[l], w["d"], 1e-6, t=w["t"], delta=dlt[l])
+                moes[l].encode_decode_layer(stack[l], xn[l], ys[l], t=w["t"], hidden=hid[l])
+
+        def step_one():
+            for l in range(L):
+                moes[l].encode_decode_layer_normed(stack[l], hid[l], nw, ys[l], t=w["t"], delta=dlt[l], eps=1e-6)
+
+        def graph_us(fn):
+            s2 = torch.cuda.Stream()
+            s2.wait_stream(torch.cuda.current_stream())
+            with torch.cuda.stream(s2):
+                fn()
+            torch.cuda.current_stream().wait_stream(s2)
+            torch.cuda.synchronize()
+            g = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(g):
+                fn()
+            for _ in range(3):
+                g.replay()
+            torch.cuda.synchronize()
+            a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            a.record()
+            for _ in range(max(1, K // 2)):
+                g.replay()
+            b.record()
+            torch.cuda.synchronize()
+            return a.elapsed_time(b) / max(1, K // 2) * 1e3 / L
+
+        out["layer_with_norm_in_front"] = {
+            "us_per_layer_two_launches": round(graph_us(step_two), 3),
+            "us_per_layer_one_launch": round(graph_us(step_one), 3),
+            "what": "hidden += delta, x = RMSNorm(hidden) * w, y = layer(x), hidden += y per layer "
+                    "(RealForwardRunner.swift:2799-2808 and the layer behind it); the two forms give the same bits"}
+        for m in moes:
+            m.status()
     if not args.no_prefill:
         out["prefill"] = measure_prefill(ctx, w, stack[0], device, use_graph=not args.no_graph)
     if not args.no_cpu_baseline:

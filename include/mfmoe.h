@@ -477,6 +477,20 @@ mf_status mf_moe_decode_layer(mf_moe* h, mf_stream stream, const mf_moe_layer_we
                               const uint16_t* x, uint32_t t, uint16_t* y, uint16_t* hidden,
                               uint32_t* out_idx, float* out_w);
 
+/* mf_moe_decode_layer with the step in front of it in the same launch (RealForwardRunner.produceToken,
+ * Runtime/Inference/RealForwardRunner.swift:2799-2808: Elementwise.encodeResidualAdd, RMSNorm.encodeBF16W,
+ * then the MoE layer and the residual add behind it): h' = bf16(hidden + delta) when delta is not NULL (else
+ * hidden), x = bf16(h' * rsqrt(mean(h'^2) + eps) * norm_weight[d]) as mf_residual_rmsnorm makes it, y = the
+ * layer on x, hidden[t,d] = bf16(h' + y).  One launch when the fused launch takes the layer (own routing,
+ * d <= 4096, the normalised rows fit its LDS): every workgroup normalises the rows for itself and reads x
+ * from LDS, the separate norm launch and the graph node between the two go away (Qwen shape, one token:
+ * see DESIGN).  Otherwise mf_residual_rmsnorm into rows of the handle followed by mf_moe_decode_layer.
+ * Both forms give the bits of those two calls.  When a bounded wait of the fused launch gives up
+ * (mf_moe_status), hidden is left as it was, delta not added. */
+mf_status mf_moe_decode_layer_normed(mf_moe* h, mf_stream stream, const mf_moe_layer_weights* wts,
+                                     uint16_t* hidden, const uint16_t* delta, const uint16_t* norm_weight,
+                                     float eps, uint32_t t, uint16_t* y, uint32_t* out_idx, float* out_w);
+
 /* Chooses between the single fused launch (default) and the chain of separate
  * launches (router, top-k, shared expert, phase 1, phase 2) inside
  * mf_moe_decode_layer.  Both give bit-identical results; the chain is the

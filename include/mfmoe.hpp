@@ -378,6 +378,12 @@ class MoE {
                               const uint16_t* residual = nullptr) const {
     check(mf_moe_unpermute(h_, cb, routePartials, routeWeights, indices, residual, tokens, h2), ctx_);
   }
+  // the residual add and RMSNorm in front of the layer, the layer and the residual add behind it in one call
+  void encodeDecodeLayerNormed(mf_stream cb, const mf_moe_layer_weights& weights, uint16_t* hidden, const uint16_t* delta,
+                               const uint16_t* normWeight, float eps, uint16_t* y, uint32_t tokens = 1,
+                               uint32_t* outIndices = nullptr, float* outWeights = nullptr) const {
+    check(mf_moe_decode_layer_normed(h_, cb, &weights, hidden, delta, normWeight, eps, tokens, y, outIndices, outWeights), ctx_);
+  }
   void setFused(bool enabled) const { check(mf_moe_set_fused(h_, enabled ? 1 : 0), ctx_); }
   // a copy of the expert pool in the prefill matmul's own order (mf_moe_layer_weights.expert_tiled)
   void tileExperts(mf_stream cb, const void* expertBase, size_t expertStride, const mf_expert_offsets& offsets,

@@ -104,6 +104,7 @@ SIGNATURES = {
     "mf_moe_phase1_subset": (_I, [_P, _P, _P, _SZ, C.POINTER(ExpertOffsets), _P, _P, _U32, _U32, _P, _P, _U32]),
     "mf_moe_phase2": (_I, [_P, _P, _P, _SZ, C.POINTER(ExpertOffsets), _P, _P, _P, _P, _U32, _P]),
     "mf_moe_decode_layer": (_I, [_P, _P, C.POINTER(LayerWeights), _P, _U32, _P, _P, _P, _P]),
+    "mf_moe_decode_layer_normed": (_I, [_P, _P, C.POINTER(LayerWeights), _P, _P, _P, C.c_float, _U32, _P, _P, _P]),
     "mf_moe_set_fused": (_I, [_P, _I]),
     "mf_moe_set_prefill_route_rounding": (_I, [_P, _I]),
     "mf_moe_tile_experts": (_I, [_P, _P, _P, _SZ, C.POINTER(ExpertOffsets), _P]),

@@ -359,6 +359,7 @@ mf_status mf_moe_create(mf_ctx* ctx, const mf_moe_config* cfg, mf_moe** out) {
   const size_t o_sact = take(T * std::max<uint32_t>(cfg->shared_f, 64) * sizeof(uint16_t));
   const size_t o_sy = take(T * cfg->d * sizeof(uint16_t));
   const size_t o_gate = take(T * sizeof(uint16_t));
+  const size_t o_xn = take(T * cfg->d * sizeof(uint16_t));
   const size_t o_tlogits = take(T * cfg->num_experts * sizeof(uint64_t));
   const size_t o_tsact = take(T * (std::max<uint32_t>(cfg->shared_f, 64) + 4) * sizeof(uint32_t));
   const size_t o_tacts = take(T * cfg->top_k * cfg->f * sizeof(uint32_t));
@@ -389,6 +390,7 @@ mf_status mf_moe_create(mf_ctx* ctx, const mf_moe_config* cfg, mf_moe** out) {
   h->ws.shared_act = reinterpret_cast<uint16_t*>(b + o_sact);
   h->ws.shared_y = reinterpret_cast<uint16_t*>(b + o_sy);
   h->ws.gate = reinterpret_cast<uint16_t*>(b + o_gate);
+  h->ws.xn = reinterpret_cast<uint16_t*>(b + o_xn);
   h->ws.t_logits = reinterpret_cast<unsigned long long*>(b + o_tlogits);
   h->ws.t_sact = reinterpret_cast<uint32_t*>(b + o_tsact);
   h->ws.t_acts = reinterpret_cast<uint32_t*>(b + o_tacts);
@@ -659,6 +661,29 @@ mf_status mf_moe_decode_layer(mf_moe* h, mf_stream stream, const mf_moe_layer_we
   if (out_w && !given)
     MF_HIP(h->ctx, hipMemcpyAsync(out_w, w, sizeof(float) * t * c.top_k, hipMemcpyDeviceToDevice, s));
   return MF_OK;
+}
+
+mf_status mf_moe_decode_layer_normed(mf_moe* h, mf_stream stream, const mf_moe_layer_weights* wts, uint16_t* hidden,
+                                     const uint16_t* delta, const uint16_t* norm_weight, float eps, uint32_t t,
+                                     uint16_t* y, uint32_t* out_idx, float* out_w) {
+  if (!h || !wts || !hidden || !norm_weight || !y) return MF_ERR_INVALID_ARGUMENT;
+  if (t == 0 || t > MF_MAX_TOKENS) return MF_ERR_INVALID_ARGUMENT;
+  if (!mf::aligned2(hidden) || !mf::aligned2(norm_weight) || (delta && !mf::aligned2(delta)) || !mf::aligned2(y))
+    return MF_ERR_INVALID_ARGUMENT;
+  const mf_moe_config& c = h->cfg;
+  auto s = static_cast<hipStream_t>(stream);
+  if (h->fused && wts->router_w && wts->expert_base && offsets_ok(wts->offsets, c.bits) &&
+      (!c.shared_f || (qtensor_ok(wts->shared_gate, c.shared_bits) && qtensor_ok(wts->shared_up, c.shared_bits) &&
+                       qtensor_ok(wts->shared_down, c.shared_bits) &&
+                       (!wts->w_sg_q8.weights || qtensor_ok(wts->w_sg_q8, MF_BITS_8)))) &&
+      mf::fused_norm_supported(*h, *wts, y, hidden, delta, norm_weight, t)) {
+    const mf::FusedNorm norm{delta, norm_weight, eps};
+    MF_HIP(h->ctx, mf::launch_fused_decode(s, *h, *wts, nullptr, t, y, hidden, out_idx, out_w, &norm));
+    return MF_OK;
+  }
+  // two launches: the norm into the handle's rows, then the layer on them (the same bits)
+  MF_HIP(h->ctx, mf::launch_residual_rmsnorm(s, hidden, delta, norm_weight, h->ws.xn, c.d, t, eps));
+  return mf_moe_decode_layer(h, stream, wts, h->ws.xn, t, y, hidden, out_idx, out_w);
 }
 
 mf_status mf_moe_set_fused(mf_moe* h, int enabled) {

@@ -23,6 +23,7 @@ struct mf_moe_workspace {
   uint16_t* shared_act; // [MF_MAX_TOKENS, shared_f]
   uint16_t* shared_y;   // [MF_MAX_TOKENS, d]
   uint16_t* gate;       // [MF_MAX_TOKENS]
+  uint16_t* xn;         // [MF_MAX_TOKENS, d]: the normalised rows of mf_moe_decode_layer_normed when it takes two launches
   // exchange buffers of the fused launch: every word carries an epoch tag
   unsigned long long* t_logits;  // [MF_MAX_TOKENS, num_experts]
   uint32_t* t_sact;              // [MF_MAX_TOKENS, shared_f]
@@ -128,9 +129,17 @@ hipError_t launch_slot_lookup(hipStream_t s, const uint32_t* idx, const int16_t*
 // moe_fused.hip
 bool fused_supported(const mf_moe& h, const mf_moe_layer_weights& w, const void* x, const void* y,
                      const void* hidden, uint32_t t);
+// the step in front of the layer made inside the fused launch (hidden += delta, x = RMSNorm(hidden) * weight)
+struct FusedNorm {
+  const uint16_t* delta;   // [t, d] or null
+  const uint16_t* weight;  // [d]
+  float eps;
+};
+bool fused_norm_supported(const mf_moe& h, const mf_moe_layer_weights& w, const void* y, const void* hidden,
+                          const void* delta, const void* norm_w, uint32_t t);
 hipError_t launch_fused_decode(hipStream_t s, const mf_moe& h, const mf_moe_layer_weights& w,
                                const uint16_t* x, uint32_t t, uint16_t* y, uint16_t* hidden,
-                               uint32_t* out_idx, float* out_w);
+                               uint32_t* out_idx, float* out_w, const FusedNorm* norm = nullptr);
 
 }  // namespace mf
 

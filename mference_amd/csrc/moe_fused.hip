@@ -162,6 +162,11 @@ struct FusedArgs {
   const uint16_t* x;
   uint16_t* y;
   uint16_t* hidden;
+  // NORM instances: x is made inside the launch from hidden (+ delta) -- see the kernel's prologue
+  const uint16_t* delta;   // [T, D] added to hidden first, or null
+  const uint16_t* norm_w;  // [D] RMSNorm weight
+  float norm_eps;
+  uint32_t xn_off;         // byte offset of the normalised rows [T, D] in LDS
   uint32_t* out_idx;
   float* out_w;
   // exchange buffers (workspace of the handle)
@@ -233,7 +238,7 @@ constexpr uint32_t static_rows_per_wave(uint32_t n, uint32_t elems_per_lane) {
   return 64u / lanes;
 }
 
-template <int BITS, int SBITS, class S>
+template <int BITS, int SBITS, class S, bool NORM = false>
 __global__ __launch_bounds__(kFusedThreads) void fused_decode_kernel(const FusedArgs a) {
   extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
   const uint32_t D = S::D != kDyn ? S::D : a.D, F = S::F != kDyn ? S::F : a.F;
@@ -284,6 +289,57 @@ __global__ __launch_bounds__(kFusedThreads) void fused_decode_kernel(const Fused
     return e + 1u;
   };
   trace_mark(a, 0);
+  // NORM: the step in front of the layer inside the launch (RealForwardRunner.swift:2799-2808: hidden += delta,
+  // x = RMSNorm(hidden) * weight).  Every workgroup makes the normalised rows for itself, in LDS, with the
+  // instruction order of residual_rmsnorm_kernel (256 threads per row, element i + 256 j on thread i, fmaf
+  // chain, neighbour-first butterfly, (s0 + s1) + (s2 + s3)), so x has the bits of that launch; everything
+  // below reads x from LDS.  hidden itself is written once, at the end, by the workgroup that owns the
+  // element: bf16(bf16(hidden + delta) + y).  A workgroup that other workgroups do not wait for (no row of
+  // stages A and B) may read hidden while it is being written: its x then is of no consequence.
+  const uint16_t* xin = a.x;
+  if constexpr (NORM) {
+    uint16_t* s_xn = reinterpret_cast<uint16_t*>(smem + a.xn_off);
+    float* s_part = s_v;  // [4 row groups][4 waves]; s_v is free until stage C
+    constexpr uint32_t kPer = 16;  // elements per thread: D <= 4096
+    const uint32_t grp = threadIdx.x >> 8, ti = threadIdx.x & 255u;
+    for (uint32_t tok0 = 0; tok0 < T; tok0 += 4) {
+      const uint32_t tok = tok0 + grp;
+      uint16_t hb[kPer];
+      float acc = 0.0f;
+      if (tok < T) {
+#pragma unroll
+        for (uint32_t j = 0; j < kPer; ++j) {
+          const uint32_t i = ti + 256u * j;
+          if (i < D) {
+            uint16_t v = a.hidden[static_cast<size_t>(tok) * D + i];
+            if (a.delta) v = f_to_bf16(bf16_to_f(v) + bf16_to_f(a.delta[static_cast<size_t>(tok) * D + i]));
+            hb[j] = v;
+          }
+        }
+#pragma unroll
+        for (uint32_t j = 0; j < kPer; ++j) {
+          if (ti + 256u * j < D) {
+            const float v = bf16_to_f(hb[j]);
+            acc = __builtin_fmaf(v, v, acc);
+          }
+        }
+      }
+      acc = wave_sum(acc);
+      if (lane == 0) s_part[wv] = acc;  // wave wv = 4 * grp + (wave of the row)
+      __syncthreads();
+      if (tok < T) {
+        const float total = (s_part[4 * grp] + s_part[4 * grp + 1]) + (s_part[4 * grp + 2] + s_part[4 * grp + 3]);
+        const float inv = 1.0f / __builtin_sqrtf(total / static_cast<float>(D) + a.norm_eps);
+#pragma unroll
+        for (uint32_t j = 0; j < kPer; ++j) {
+          const uint32_t i = ti + 256u * j;
+          if (i < D) s_xn[static_cast<size_t>(tok) * D + i] = f_to_bf16(bf16_to_f(hb[j]) * inv * bf16_to_f(a.norm_w[i]));
+        }
+      }
+      __syncthreads();
+    }
+    xin = s_xn;
+  }
   // rank counting selects the top-k when it is cheap enough, else one wave per token sorts
   const bool rank_count = !S::kGiven && T * E * E <= kRankCountLimit && T * E <= kRankWords;
   // Who does what while the logits are on their way: the top waves poll for them (n_poll waves),
@@ -310,7 +366,7 @@ __global__ __launch_bounds__(kFusedThreads) void fused_decode_kernel(const Fused
       if (wv < kRouterChunk && row < n_rows_r) {
         const uint32_t tok = row / E, e = row % E;
         const float v = dot_bf16_row(a.router_w + static_cast<size_t>(e) * D,
-                                     a.x + static_cast<size_t>(tok) * D, D, lane, true);
+                                     xin + static_cast<size_t>(tok) * D, D, lane, true);
         if (lane == 0) s_stage64[wv] = (static_cast<unsigned long long>(epoch_now()) << 32) | __float_as_uint(v);
       }
       __syncthreads();
@@ -326,8 +382,8 @@ __global__ __launch_bounds__(kFusedThreads) void fused_decode_kernel(const Fused
     for (uint32_t item = wg >= skip ? wv * Gs + (wg - skip) : n_items; item < n_items; item += kFusedWaves * Gs) {
       if (item < n_gate) {
         const uint32_t tok = item;
-        const float v = a.gq_w ? dot_q8_row(a.gq_w, a.gq_s, a.gq_b, a.x + static_cast<size_t>(tok) * D, D, lane, true)
-                               : dot_bf16_row(a.w_sg, a.x + static_cast<size_t>(tok) * D, D, lane, true);
+        const float v = a.gq_w ? dot_q8_row(a.gq_w, a.gq_s, a.gq_b, xin + static_cast<size_t>(tok) * D, D, lane, true)
+                               : dot_bf16_row(a.w_sg, xin + static_cast<size_t>(tok) * D, D, lane, true);
         if (lane < 4)  // the gate rides behind the token's shared activations
           store_u32_agent(&a.t_sact[static_cast<size_t>(tok) * sact_stride + Fs + lane],
                           (lane == 0 ? static_cast<uint32_t>(f_to_bf16(v)) : 0u) | (epoch_now() << 16));
@@ -347,7 +403,7 @@ __global__ __launch_bounds__(kFusedThreads) void fused_decode_kernel(const Fused
                                  a.sg.scales + r * ng, a.sg.biases + r * ng,
                                  static_cast<const uint8_t*>(a.su.weights) + r * rb,
                                  a.su.scales + r * ng, a.su.biases + r * ng,
-                                 a.x + static_cast<size_t>(tok) * D, D, sub, lpr, ga, ua);
+                                 xin + static_cast<size_t>(tok) * D, D, sub, lpr, ga, ua);
         const float g = group_sum(ga, static_cast<int>(lpr));
         const float u = group_sum(ua, static_cast<int>(lpr));
         if (ok && sub == 0) {
@@ -363,7 +419,7 @@ __global__ __launch_bounds__(kFusedThreads) void fused_decode_kernel(const Fused
       for (uint32_t q = (wv + n_poll + n_xw - kFusedWaves) * kWave + lane; q < T * n_sl; q += n_xw * kWave) {
         const uint32_t tok = q / n_sl, sl = q % n_sl;
         store_xslice_lds<BITS>(s_xq, s_xsum, tok, n_sl, sl,
-                               load_xslice<BITS, kXAligned>(a.x + static_cast<size_t>(tok) * D + sl * kEPL));
+                               load_xslice<BITS, kXAligned>(xin + static_cast<size_t>(tok) * D + sl * kEPL));
       }
     }
   }
@@ -500,7 +556,7 @@ __global__ __launch_bounds__(kFusedThreads) void fused_decode_kernel(const Fused
           const Chunk<BITS> uc = load_chunk<BITS>(uw, us, ub, e0);
           issue_fence();
           const XSlice<BITS> xs = xprep ? load_xslice_lds<BITS>(s_xq, s_xsum, tok, n_sl, e0 / kEPL)
-                                          : load_xslice<BITS, kXAligned>(a.x + static_cast<size_t>(tok) * D + e0);
+                                          : load_xslice<BITS, kXAligned>(xin + static_cast<size_t>(tok) * D + e0);
           const float gd = codes_dot<BITS>(gc.codes, xs), ud = codes_dot<BITS>(uc.codes, xs);
           if (ok) {
             ga = __builtin_fmaf(gc.s, gd, ga);
@@ -774,8 +830,13 @@ __global__ __launch_bounds__(kFusedThreads) void fused_decode_kernel(const Fused
           const bool failed = *s_fail != 0u;  // a wait gave up: no result, and hidden stays as it is
           const uint16_t yb = failed ? static_cast<uint16_t>(0x7FC0u) : f_to_bf16(acc);
           a.y[o] = yb;
-          if (a.hidden && !failed)  // residual_add_fp16, utility.metal:83-92
-            a.hidden[o] = f_to_bf16(bf16_to_f(a.hidden[o]) + bf16_to_f(yb));
+          if (a.hidden && !failed) {  // residual_add_fp16, utility.metal:83-92
+            uint16_t hv = a.hidden[o];
+            if constexpr (NORM) {  // the residual add in front of the norm, made here for good
+              if (a.delta) hv = f_to_bf16(bf16_to_f(hv) + bf16_to_f(a.delta[o]));
+            }
+            a.hidden[o] = f_to_bf16(bf16_to_f(hv) + bf16_to_f(yb));
+          }
         }
       }
       // The next round (or token) overwrites s_v.  Behind the last round nothing is left to protect, and a
@@ -860,9 +921,21 @@ bool fused_supported(const mf_moe& h, const mf_moe_layer_weights& w, const void*
   return true;
 }
 
+// Whether the launch can make x itself (NORM instances): own routing, rows of at most 4096 elements, room in
+// LDS for the normalised rows, everything the plain launch needs
+bool fused_norm_supported(const mf_moe& h, const mf_moe_layer_weights& w, const void* y, const void* hidden,
+                          const void* delta, const void* norm_w, uint32_t t) {
+  const mf_moe_config& c = h.cfg;
+  if (!w.router_w || !hidden || !norm_w || c.d > 4096) return false;
+  if (!aligned16(hidden) || !aligned16(norm_w) || (delta && !aligned16(delta))) return false;
+  if (!fused_supported(h, w, hidden, y, hidden, t)) return false;  // (x stands in as an aligned pointer)
+  const uint32_t num_cu = static_cast<uint32_t>(h.ctx->num_cu);
+  return fused_lds_bytes(c, num_cu, t) + 16 + static_cast<size_t>(t) * c.d * 2 <= kFusedLdsLimit;
+}
+
 hipError_t launch_fused_decode(hipStream_t s, const mf_moe& h, const mf_moe_layer_weights& w,
                                const uint16_t* x, uint32_t t, uint16_t* y, uint16_t* hidden,
-                               uint32_t* out_idx, float* out_w) {
+                               uint32_t* out_idx, float* out_w, const FusedNorm* norm) {
   const mf_moe_config& c = h.cfg;
   FusedArgs a{};
   a.router_w = w.router_w;
@@ -899,9 +972,16 @@ hipError_t launch_fused_decode(hipStream_t s, const mf_moe& h, const mf_moe_laye
   a.maple = static_cast<int>(c.maple_rounding);
   const dim3 grid(static_cast<uint32_t>(h.ctx->num_cu)), block(kFusedThreads);
   const uint32_t num_cu = static_cast<uint32_t>(h.ctx->num_cu);
-  const size_t lds = fused_lds_bytes(c, num_cu, t);
+  size_t lds = fused_lds_bytes(c, num_cu, t);
   a.stage_words = fused_stage_words(c, num_cu, t);
   a.xprep = fused_xprep(c, num_cu, t) ? 1 : 0;
+  if (norm) {  // the normalised rows behind everything else in LDS
+    a.delta = norm->delta;
+    a.norm_w = norm->weight;
+    a.norm_eps = norm->eps;
+    a.xn_off = static_cast<uint32_t>((lds + 15) & ~size_t(15));
+    lds = a.xn_off + static_cast<size_t>(t) * c.d * 2;
+  }
 #define MF_FUSED(B, SB, SHAPE)                                                                 \
   do {                                                                                         \
     auto kern = fused_decode_kernel<B, SB, SHAPE>;                                             \
@@ -953,6 +1033,27 @@ hipError_t launch_fused_decode(hipStream_t s, const mf_moe& h, const mf_moe_laye
   const bool qwen_dims = c.bits == MF_BITS_4 && c.shared_bits == MF_BITS_4 && c.d == 2048 && c.f == 512 &&
                          c.num_experts == 256 && c.top_k == 8 && c.shared_f == 512;
   const bool lit = !h.generic_shape;  // shape instances allowed
+#define MF_FUSED_N(B, SB, SHAPE)                                                               \
+  do {                                                                                         \
+    auto kern = fused_decode_kernel<B, SB, SHAPE, true>;                                       \
+    if (lds > 48 * 1024) {                                                                     \
+      hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),                  \
+                                         hipFuncAttributeMaxDynamicSharedMemorySize,           \
+                                         static_cast<int>(lds));                               \
+      if (e != hipSuccess) return e;                                                           \
+    }                                                                                          \
+    kern<<<grid, block, lds, s>>>(a);                                                          \
+  } while (0)
+  if (norm) {  // x made inside the launch: the Qwen shape's instances and the ones that read every dimension
+    if (lit && qwen && t == 1 && !c.maple_rounding && no_limit && a.xprep) MF_FUSED_N(kBits4, kBits4, QwenT1);
+    else if (lit && qwen) MF_FUSED_N(kBits4, kBits4, QwenTn);
+    else if (c.bits == MF_BITS_4) MF_FUSED_N(kBits4, kBits4, RuntimeShape);
+    else if (c.bits == MF_BITS_2 && c.shared_f && c.shared_bits == MF_BITS_2) MF_FUSED_N(kBits2, kBits2, RuntimeShape);
+    else if (c.bits == MF_BITS_2) MF_FUSED_N(kBits2, kBits4, RuntimeShape);
+    else MF_FUSED_N(kBitsTernary, kBits4, RuntimeShape);
+    return hipGetLastError();
+  }
+#undef MF_FUSED_N
   if (!w.router_w) {  // caller-given routing
     if (!lit) {
       if (c.bits == MF_BITS_4) MF_FUSED(kBits4, kBits4, Given);

@@ -399,6 +399,15 @@ class MoE:
         except Exception:
             pass
 
+    def encode_decode_layer_normed(self, weights: MoELayerWeights, hidden, norm_weight, y, t: int = 1, delta=None,
+                                   eps: float = 1e-6, out_indices=None, out_weights=None, stream=None):
+        """hidden += delta, x = RMSNorm(hidden) * norm_weight, y = layer(x), hidden += y: one launch where the
+        fused launch takes the layer (RealForwardRunner.swift:2799-2808 and the layer behind it)."""
+        lw = weights.c()
+        check(_capi.lib().mf_moe_decode_layer_normed(self._h, _stream(stream), C.byref(lw), _ptr(hidden), _ptr(delta),
+                                                     _ptr(norm_weight), eps, t, _ptr(y), _ptr(out_indices),
+                                                     _ptr(out_weights)), self.context.handle)
+
     def set_fused(self, enabled) -> None:
         """single fused launch (True / 1, default) or the chain of separate launches (False / 0); 2: the fused
         launch through the instance that reads every dimension from its arguments"""

@@ -1056,3 +1056,52 @@ def test_int8_shared_expert(gpu, oracle, d, f, t, silu):
                                      scratch.data_ptr(), t * f * 2 - 2) == -4
     assert lib.mf_shared_expert_int8(gpu.handle, None, x.data_ptr(), g.c(), u.c(), dn.c(), d + 8, f, t, 0, y.data_ptr(),
                                      scratch.data_ptr(), t * f * 2) == -2
+
+
+@pytest.mark.parametrize("bits,d,f,e,k,fs,t,with_delta", [
+    (4, 2048, 512, 256, 8, 512, 1, True),     # the headline shape's one-token instance
+    (4, 2048, 512, 256, 8, 512, 5, False),    # ... its several-rows instance, no delta
+    (4, 512, 256, 32, 4, 128, 8, True),       # the instance that reads every dimension; two rounds of four rows
+    (2, 1024, 512, 16, 6, 0, 3, True),        # 2-bit, no shared expert
+    (1, 512, 256, 32, 8, 0, 2, True),         # ternary, full-softmax router
+    (4, 4608, 128, 16, 2, 0, 2, True),        # rows wider than 4096: two launches behind the same call
+])
+def test_decode_layer_with_the_norm_in_front(gpu, oracle, bits, d, f, e, k, fs, t, with_delta):
+    """mf_moe_decode_layer_normed: hidden += delta, x = RMSNorm(hidden) * w, y = layer(x), hidden += y in one
+    call -- the bits of mf_residual_rmsnorm followed by mf_moe_decode_layer (also with the fused launch off),
+    and the checker's composition of the two."""
+    root = ROOT_SEED + 0x4042 + d + t
+    layer = oracle.synth_layer(root, d, f, e, k, bits=bits, fs=fs, router_mode=1 if bits == 1 else 0,
+                               maple_rounding=bits == 1)
+    rng = oracle.Rng.key(root, "norm")
+    hb = oracle.bf16_bits(rng.normal(0.0, 1.0, t * d).reshape(t, d))
+    db = oracle.bf16_bits(rng.normal(0.0, 0.5, t * d).reshape(t, d)) if with_delta else None
+    wb = oracle.bf16_bits(1.0 + rng.normal(0.0, 0.1, d))
+    moe = make_moe(gpu, layer)
+    wts = to_device_layer(layer)
+    # reference: the two calls
+    h_ref = ops.bf16_tensor(hb).clone()
+    xn = torch.zeros((t, d), dtype=torch.bfloat16, device="cuda")
+    ops.RMSNorm(gpu).encode_bf16w(h_ref, ops.bf16_tensor(wb), xn, d, 1e-6, t=t,
+                                  delta=None if db is None else ops.bf16_tensor(db))
+    y_ref = torch.zeros((t, d), dtype=torch.bfloat16, device="cuda")
+    moe.encode_decode_layer(wts, xn, y_ref, t, hidden=h_ref)
+    for fused in (1, 0):
+        moe.set_fused(fused)
+        h = ops.bf16_tensor(hb).clone()
+        y = torch.full((t, d), 3.0, dtype=torch.bfloat16, device="cuda")
+        idx = torch.zeros((t, k), dtype=torch.int32, device="cuda")
+        w = torch.zeros((t, k), dtype=torch.float32, device="cuda")
+        moe.encode_decode_layer_normed(wts, h, ops.bf16_tensor(wb), y, t, delta=None if db is None else ops.bf16_tensor(db),
+                                       eps=1e-6, out_indices=idx, out_weights=w)
+        torch.cuda.synchronize()
+        moe.status()
+        assert torch.equal(y, y_ref), f"y, fused={fused}"
+        assert torch.equal(h, h_ref), f"hidden, fused={fused}"
+    moe.set_fused(1)
+    # the checker: norm, layer, residual add
+    h1, x_ref = oracle.residual_rmsnorm(hb, wb, 1e-6, delta_bits=db)
+    ref_y, ref_idx, ref_w = oracle.moe_layer(layer, x_ref)
+    assert np.array_equal(ops.bf16_bits(xn), x_ref)
+    assert np.array_equal(idx.cpu().numpy().astype(np.uint32), ref_idx)
+    assert_layer_close(oracle.bf16_to_float(ops.bf16_bits(y)), oracle.bf16_to_float(ref_y), "normed layer")

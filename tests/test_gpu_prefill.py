@@ -173,6 +173,8 @@ def test_skewed_qwen_prefill_against_the_checker(gpu, oracle, t):
     x[:, -1] = 0x3F80
     moe = make_moe(gpu, layer)
     wts = to_device_layer(layer)
+    # (the form the benchmark reports: the routed experts read from the tiled copy of the pool)
+    wts.experts_tiled = moe.tile_experts(wts.experts, wts.offsets)
     y, idx, w = _run_prefill(moe, wts, x, t, d, k)
     rows = np.unique(np.concatenate([np.arange(8), np.arange(t - 8, t),
                                      np.random.default_rng(t).choice(t, size=48, replace=False)]))

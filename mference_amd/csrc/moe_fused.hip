@@ -297,6 +297,22 @@ __global__ __launch_bounds__(kFusedThreads) void fused_decode_kernel(const Fused
   // element: bf16(bf16(hidden + delta) + y).  A workgroup that other workgroups do not wait for (no row of
   // stages A and B) may read hidden while it is being written: its x then is of no consequence.
   const uint16_t* xin = a.x;
+  // (NORM) the first router row of a wave: its weights are requested ahead of the norm, which has a memory
+  // round trip of its own to wait for -- rows of up to 2048 elements, four chunks per lane
+  uint4 pre_w[4];
+  bool pre_router = false;
+  if constexpr (NORM && !S::kGiven) {
+    const uint32_t row = wg * kRouterChunk + wv;
+    pre_router = D <= 2048 && D % 8 == 0 && wv < kRouterChunk && row < E * T;
+    if (pre_router) {
+      const uint16_t* wr = a.router_w + static_cast<size_t>(row % E) * D;
+#pragma unroll
+      for (int sidx = 0; sidx < 4; ++sidx) {
+        const uint32_t c = lane + sidx * kWave;
+        pre_w[sidx] = c < D / 8 ? load_x8<true>(wr + c * 8) : make_uint4(0, 0, 0, 0);
+      }
+    }
+  }
   if constexpr (NORM) {
     uint16_t* s_xn = reinterpret_cast<uint16_t*>(smem + a.xn_off);
     float* s_part = s_v;  // [4 row groups][4 waves]; s_v is free until stage C
@@ -304,7 +320,7 @@ __global__ __launch_bounds__(kFusedThreads) void fused_decode_kernel(const Fused
     const uint32_t grp = threadIdx.x >> 8, ti = threadIdx.x & 255u;
     for (uint32_t tok0 = 0; tok0 < T; tok0 += 4) {
       const uint32_t tok = tok0 + grp;
-      uint16_t hb[kPer];
+      uint16_t hb[kPer], nwv[kPer];  // (the weights are requested with the row: one round trip, not two)
       float acc = 0.0f;
       if (tok < T) {
 #pragma unroll
@@ -314,6 +330,7 @@ __global__ __launch_bounds__(kFusedThreads) void fused_decode_kernel(const Fused
             uint16_t v = a.hidden[static_cast<size_t>(tok) * D + i];
             if (a.delta) v = f_to_bf16(bf16_to_f(v) + bf16_to_f(a.delta[static_cast<size_t>(tok) * D + i]));
             hb[j] = v;
+            nwv[j] = a.norm_w[i];
           }
         }
 #pragma unroll
@@ -333,7 +350,7 @@ __global__ __launch_bounds__(kFusedThreads) void fused_decode_kernel(const Fused
 #pragma unroll
         for (uint32_t j = 0; j < kPer; ++j) {
           const uint32_t i = ti + 256u * j;
-          if (i < D) s_xn[static_cast<size_t>(tok) * D + i] = f_to_bf16(bf16_to_f(hb[j]) * inv * bf16_to_f(a.norm_w[i]));
+          if (i < D) s_xn[static_cast<size_t>(tok) * D + i] = f_to_bf16(bf16_to_f(hb[j]) * inv * bf16_to_f(nwv[j]));
         }
       }
       __syncthreads();
@@ -365,8 +382,29 @@ __global__ __launch_bounds__(kFusedThreads) void fused_decode_kernel(const Fused
       const uint32_t row = ci * kRouterChunk + wv;
       if (wv < kRouterChunk && row < n_rows_r) {
         const uint32_t tok = row / E, e = row % E;
-        const float v = dot_bf16_row(a.router_w + static_cast<size_t>(e) * D,
-                                     xin + static_cast<size_t>(tok) * D, D, lane, true);
+        float v;
+        if (NORM && pre_router && ci == wg) {  // the weights are here already: dot_bf16_row's products in its order
+          const uint16_t* xr = xin + static_cast<size_t>(tok) * D;
+          float acc = 0.0f;
+#pragma unroll
+          for (int sidx = 0; sidx < 4; ++sidx) {
+            const uint32_t c = lane + sidx * kWave;
+            if (c < D / 8) {
+              const uint4 xv = load_x8<true>(xr + c * 8), wq = pre_w[sidx];
+              acc = __builtin_fmaf(bf16_lo(wq.x), bf16_lo(xv.x), acc);
+              acc = __builtin_fmaf(bf16_hi(wq.x), bf16_hi(xv.x), acc);
+              acc = __builtin_fmaf(bf16_lo(wq.y), bf16_lo(xv.y), acc);
+              acc = __builtin_fmaf(bf16_hi(wq.y), bf16_hi(xv.y), acc);
+              acc = __builtin_fmaf(bf16_lo(wq.z), bf16_lo(xv.z), acc);
+              acc = __builtin_fmaf(bf16_hi(wq.z), bf16_hi(xv.z), acc);
+              acc = __builtin_fmaf(bf16_lo(wq.w), bf16_lo(xv.w), acc);
+              acc = __builtin_fmaf(bf16_hi(wq.w), bf16_hi(xv.w), acc);
+            }
+          }
+          v = wave_sum(acc);
+        } else {
+          v = dot_bf16_row(a.router_w + static_cast<size_t>(e) * D, xin + static_cast<size_t>(tok) * D, D, lane, true);
+        }
         if (lane == 0) s_stage64[wv] = (static_cast<unsigned long long>(epoch_now()) << 32) | __float_as_uint(v);
       }
       __syncthreads();

@@ -94,3 +94,32 @@ def test_prefill_layer_replays_equal_eager(gpu, oracle, bits, d, f, e, k, fs, t)
         assert torch.equal(y.view(torch.int16), ye.view(torch.int16)), f"replay {rep}"
         seen.add(idx.cpu().numpy().tobytes())
     assert len(seen) == 4   # the replays did route differently
+
+
+@pytest.mark.parametrize("bits,d,f,e,k,fs,t", [(4, 2048, 512, 256, 8, 512, 1), (4, 512, 256, 32, 8, 256, 6)])
+def test_normed_decode_layer_replays_equal_eager(gpu, oracle, bits, d, f, e, k, fs, t):
+    """the layer with the residual add and the norm in its own launch: hidden is read at the start of the launch and
+    written at its end, replay after replay"""
+    root = ROOT_SEED + 0xC200 + d
+    layer = oracle.synth_layer(root, d, f, e, k, bits=bits, fs=fs)
+    moe = make_moe(gpu, layer)
+    wts = to_device_layer(layer)
+    nw = ops.bf16_tensor(oracle.bf16_bits(1.0 + oracle.Rng.key(root, "nw").normal(0.0, 0.1, d)))
+    hidden = torch.zeros((t, d), dtype=torch.bfloat16, device="cuda")
+    delta = torch.zeros_like(hidden)
+    y = torch.zeros_like(hidden)
+    graph = _capture(lambda: moe.encode_decode_layer_normed(wts, hidden, nw, y, t, delta=delta, eps=1e-6))
+    for rep in range(4):
+        hr = ops.bf16_tensor(oracle.synth_x(root + rep, t, d))
+        dr = ops.bf16_tensor(oracle.synth_x(root + 50 + rep, t, d))
+        ye, he = torch.zeros_like(y), hr.clone()
+        moe.encode_decode_layer_normed(wts, he, nw, ye, t, delta=dr, eps=1e-6)
+        moe.status()
+        hidden.copy_(hr)
+        delta.copy_(dr)
+        y.zero_()
+        graph.replay()
+        torch.cuda.synchronize()
+        moe.status()
+        assert torch.equal(y.view(torch.int16), ye.view(torch.int16)), f"replay {rep}"
+        assert torch.equal(hidden.view(torch.int16), he.view(torch.int16)), f"replay {rep}"

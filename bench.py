@@ -721,7 +721,7 @@ def prefill_phase_trace(ctx, w, layer, device, tokens) -> int:
     return 0
 
 
-def phase_trace(ctx, w, stack, moes, device) -> int:
+def phase_trace(ctx, w, stack, moes, device, with_norm=False) -> int:
     """Stage stamps every workgroup of the fused decode launch writes (100 MHz wall clock): per stamp
     the median over the layers of the earliest / median / latest workgroup, in us from the start of the
     layer's first workgroup, and the time from the end of one launch to the start of the next."""
@@ -735,9 +735,14 @@ def phase_trace(ctx, w, stack, moes, device) -> int:
     stamps = torch.zeros((L, ncu * 8), dtype=torch.int64, device=device)
     for l in range(L):
         moes[l].set_phase_trace(stamps[l])
+    nw = torch.ones((w["d"],), dtype=torch.bfloat16, device=device)
+    dl = torch.zeros_like(xs)
     for _ in range(6):
         for l in range(L):
-            moes[l].encode_decode_layer(stack[l], xs[l], ys[l], t=w["t"])
+            if with_norm:  # the residual add and the norm inside the launch: xs is the hidden state
+                moes[l].encode_decode_layer_normed(stack[l], xs[l], nw, ys[l], t=w["t"], delta=dl[l], eps=1e-6)
+            else:
+                moes[l].encode_decode_layer(stack[l], xs[l], ys[l], t=w["t"])
     torch.cuda.synchronize()
     for m in moes:
         m.status()
@@ -751,6 +756,7 @@ def phase_trace(ctx, w, stack, moes, device) -> int:
                           "median": round(float(np.median(np.median(rel[skip:, :, i], axis=1))), 2),
                           "latest": round(float(np.median(rel[skip:, :, i].max(axis=1))), 2)}
                       for i, n in enumerate(names)},
+           "norm_done_median": round(float(np.median(np.median((t[skip:, :, 7] - t[skip:, :, 0].min(axis=1)[:, None]) / 100.0, axis=1))), 2) if with_norm else None,
            "gap_end_to_next_start_us": round(float(np.median(
                [(t[l, :, 0].min() - t[l - 1, :, 6].max()) / 100.0 for l in range(skip + 1, L)])), 2)}
     print(json.dumps(out))
@@ -820,6 +826,8 @@ def main() -> int:
     ap.add_argument("--no-prefill", action="store_true", help="skip the ragged prefill section")
     ap.add_argument("--no-other-configs", action="store_true",
                     help="skip the short runs of the other BASELINE configurations that the default run appends")
+    ap.add_argument("--with-norm", action="store_true",
+                    help="with --phase-trace: the launch that makes x itself (mf_moe_decode_layer_normed)")
     ap.add_argument("--no-side-runs", action="store_true",
                     help="with --prefill-only: time the layer call as it is reported (tiled expert pool, fp32 per-route "
                          "results) only, not the row-by-row pool and the 16-bit per-route results beside it (for profiling)")
@@ -875,7 +883,7 @@ def main() -> int:
             for _ in range(L)]
 
     if args.phase_trace:
-        return phase_trace(ctx, w, stack, moes, device)
+        return phase_trace(ctx, w, stack, moes, device, with_norm=args.with_norm)
 
     gen = torch.Generator(device=device)
     gen.manual_seed(ROOT_SEED + 0x100 * w["config"] + 0xFF)

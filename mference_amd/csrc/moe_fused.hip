@@ -315,47 +315,80 @@ __global__ __launch_bounds__(kFusedThreads) void fused_decode_kernel(const Fused
   }
   if constexpr (NORM) {
     uint16_t* s_xn = reinterpret_cast<uint16_t*>(smem + a.xn_off);
-    float* s_part = s_v;  // [4 row groups][4 waves]; s_v is free until stage C
-    constexpr uint32_t kPer = 16;  // elements per thread: D <= 4096
+    float* s_part = s_v;  // [token][4 waves of its row]; s_v is free until stage C
+    // The rows come in as 16-byte pieces, every piece once per workgroup (piece c on thread c % 1024), with
+    // the matching piece of delta and of the weights in the same round trip; bf16(hidden + delta) goes to
+    // LDS, the sums read it from there in the norm kernel's order, and each piece's owner scales it in
+    // place.  (Element by element from global memory, the delta loads sat behind a branch each: eight
+    // round trips in a row, 3.9 us before the first row could start.)
+    constexpr uint32_t kPc = MF_MAX_TOKENS * 4096 / 8 / kFusedThreads;  // pieces per thread at most
+    const uint32_t ppr = D / 8, n_pc = T * ppr;
+    const uint16_t* dsrc = a.delta ? a.delta : a.hidden;  // (always a valid address: no branch around the load)
+    const bool has_delta = a.delta != nullptr;
+    uint4 hv[kPc], nv[kPc];
+#pragma unroll
+    for (uint32_t p = 0; p < kPc; ++p) {
+      const uint32_t c = threadIdx.x + kFusedThreads * p;
+      if (c < n_pc) {
+        const uint4 h4 = load_x8<true>(a.hidden + static_cast<size_t>(c) * 8);
+        const uint4 d4 = load_x8<true>(dsrc + static_cast<size_t>(c) * 8);
+        nv[p] = load_x8<true>(a.norm_w + static_cast<size_t>(c % ppr) * 8);
+        const uint32_t hw[4] = {h4.x, h4.y, h4.z, h4.w}, dw[4] = {d4.x, d4.y, d4.z, d4.w};
+        uint32_t o[4];
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+          const uint16_t lo = f_to_bf16(bf16_to_f(static_cast<uint16_t>(hw[q] & 0xffffu)) +
+                                        bf16_to_f(static_cast<uint16_t>(dw[q] & 0xffffu)));
+          const uint16_t hi = f_to_bf16(bf16_to_f(static_cast<uint16_t>(hw[q] >> 16)) +
+                                        bf16_to_f(static_cast<uint16_t>(dw[q] >> 16)));
+          o[q] = has_delta ? (static_cast<uint32_t>(lo) | (static_cast<uint32_t>(hi) << 16)) : hw[q];
+        }
+        hv[p] = make_uint4(o[0], o[1], o[2], o[3]);
+        *reinterpret_cast<uint4*>(s_xn + static_cast<size_t>(c) * 8) = hv[p];
+      }
+    }
+    __syncthreads();
     const uint32_t grp = threadIdx.x >> 8, ti = threadIdx.x & 255u;
     for (uint32_t tok0 = 0; tok0 < T; tok0 += 4) {
       const uint32_t tok = tok0 + grp;
-      uint16_t hb[kPer], nwv[kPer];  // (the weights are requested with the row: one round trip, not two)
       float acc = 0.0f;
       if (tok < T) {
 #pragma unroll
-        for (uint32_t j = 0; j < kPer; ++j) {
+        for (uint32_t j = 0; j < 16; ++j) {  // D <= 4096
           const uint32_t i = ti + 256u * j;
           if (i < D) {
-            uint16_t v = a.hidden[static_cast<size_t>(tok) * D + i];
-            if (a.delta) v = f_to_bf16(bf16_to_f(v) + bf16_to_f(a.delta[static_cast<size_t>(tok) * D + i]));
-            hb[j] = v;
-            nwv[j] = a.norm_w[i];
-          }
-        }
-#pragma unroll
-        for (uint32_t j = 0; j < kPer; ++j) {
-          if (ti + 256u * j < D) {
-            const float v = bf16_to_f(hb[j]);
+            const float v = bf16_to_f(s_xn[static_cast<size_t>(tok) * D + i]);
             acc = __builtin_fmaf(v, v, acc);
           }
         }
       }
       acc = wave_sum(acc);
-      if (lane == 0) s_part[wv] = acc;  // wave wv = 4 * grp + (wave of the row)
-      __syncthreads();
-      if (tok < T) {
-        const float total = (s_part[4 * grp] + s_part[4 * grp + 1]) + (s_part[4 * grp + 2] + s_part[4 * grp + 3]);
-        const float inv = 1.0f / __builtin_sqrtf(total / static_cast<float>(D) + a.norm_eps);
-#pragma unroll
-        for (uint32_t j = 0; j < kPer; ++j) {
-          const uint32_t i = ti + 256u * j;
-          if (i < D) s_xn[static_cast<size_t>(tok) * D + i] = f_to_bf16(bf16_to_f(hb[j]) * inv * bf16_to_f(nwv[j]));
-        }
-      }
-      __syncthreads();
+      if (lane == 0 && tok < T) s_part[4 * tok + (wv & 3u)] = acc;
     }
+    __syncthreads();
+#pragma unroll
+    for (uint32_t p = 0; p < kPc; ++p) {
+      const uint32_t c = threadIdx.x + kFusedThreads * p;
+      if (c < n_pc) {
+        const uint32_t tok = c / ppr;
+        const float total = (s_part[4 * tok] + s_part[4 * tok + 1]) + (s_part[4 * tok + 2] + s_part[4 * tok + 3]);
+        const float inv = 1.0f / __builtin_sqrtf(total / static_cast<float>(D) + a.norm_eps);
+        const uint32_t hw[4] = {hv[p].x, hv[p].y, hv[p].z, hv[p].w}, nw4[4] = {nv[p].x, nv[p].y, nv[p].z, nv[p].w};
+        uint32_t o[4];
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+          const uint16_t lo = f_to_bf16(bf16_to_f(static_cast<uint16_t>(hw[q] & 0xffffu)) * inv *
+                                        bf16_to_f(static_cast<uint16_t>(nw4[q] & 0xffffu)));
+          const uint16_t hi = f_to_bf16(bf16_to_f(static_cast<uint16_t>(hw[q] >> 16)) * inv *
+                                        bf16_to_f(static_cast<uint16_t>(nw4[q] >> 16)));
+          o[q] = static_cast<uint32_t>(lo) | (static_cast<uint32_t>(hi) << 16);
+        }
+        *reinterpret_cast<uint4*>(s_xn + static_cast<size_t>(c) * 8) = make_uint4(o[0], o[1], o[2], o[3]);
+      }
+    }
+    __syncthreads();
     xin = s_xn;
+    trace_mark(a, 7);
   }
   // rank counting selects the top-k when it is cheap enough, else one wave per token sorts
   const bool rank_count = !S::kGiven && T * E * E <= kRankCountLimit && T * E <= kRankWords;

@@ -254,6 +254,50 @@ static void test_layer() {
   EXPECT(std::memcmp(idx.data(), ref_idx.data(), t_pre * k * 4) == 0, "prefill routing indices");
   compare(to_host(dy, t_pre * d), ref_y, "ragged prefill layer");
 
+  // the same layer from the tiled copy of the expert pool: the bits of the row-by-row pool
+  {
+    auto y_rows = to_host(dy, t_pre * d);
+    void* tiled = nullptr;
+    HIP_OK(hipMalloc(&tiled, L.stride * e));
+    moe.tileExperts(nullptr, w.expert_base, w.expert_stride, w.offsets, tiled);
+    mf_moe_layer_weights wt2 = w;
+    wt2.expert_tiled = tiled;
+    moe.encodePrefillLayer(nullptr, wt2, dx, dy, t_pre, ws, ws_bytes, didx, dw);
+    HIP_OK(hipDeviceSynchronize());
+    EXPECT(to_host(dy, t_pre * d) == y_rows, "tiled pool != row-by-row pool");
+    std::printf("%-28s bit-identical\n", "prefill from the tiled pool");
+  }
+
+  // the residual add and the RMSNorm in front of the layer in the layer's launch == the two calls
+  {
+    std::vector<float> nf(d), df(t_dec * d);
+    mfo_rng rn = mfo_seed_tree_key(root, "norm");
+    mfo_rng_normal(&rn, 1.0f, 0.1f, nf.data(), nf.size());
+    mfo_rng_normal(&rn, 0.0f, 0.5f, df.data(), df.size());
+    std::vector<uint16_t> nw(d), dl(t_dec * d);
+    mfo_bf16_encode(nf.data(), nf.size(), nw.data());
+    mfo_bf16_encode(df.data(), df.size(), dl.data());
+    uint16_t* dnw = to_device(nw);
+    uint16_t* ddl = to_device(dl);
+    std::vector<uint16_t> h0(x.begin(), x.begin() + t_dec * d);
+    uint16_t* dh1 = to_device(h0);
+    uint16_t* dh2 = to_device(h0);
+    uint16_t* dxn = nullptr;
+    uint16_t* dya = nullptr;
+    uint16_t* dyb = nullptr;
+    HIP_OK(hipMalloc(&dxn, t_dec * d * 2));
+    HIP_OK(hipMalloc(&dya, t_dec * d * 2));
+    HIP_OK(hipMalloc(&dyb, t_dec * d * 2));
+    moe.encodeDecodeLayerNormed(nullptr, w, dh1, ddl, dnw, 1e-6f, dya, t_dec);
+    mf::RMSNorm norm(context);
+    norm.encodeBF16W(nullptr, dh2, dnw, dxn, d, 1e-6f, t_dec, ddl);
+    moe.encodeDecodeLayer(nullptr, w, dxn, dyb, t_dec, dh2);
+    moe.status(nullptr);
+    EXPECT(to_host(dya, t_dec * d) == to_host(dyb, t_dec * d), "normed layer: y != two calls");
+    EXPECT(to_host(dh1, t_dec * d) == to_host(dh2, t_dec * d), "normed layer: hidden != two calls");
+    std::printf("%-28s bit-identical\n", "normed decode layer");
+  }
+
   // argument errors throw and launch nothing (SharedExpertError.scratchTooSmall)
   bool thrown = false;
   try {

@@ -815,7 +815,9 @@ __global__ __launch_bounds__(kFusedThreads) void fused_decode_kernel(const Fused
     };
     // waves that own shared rows when the rows are dealt one wave step each
     const uint32_t sh_waves = Fs ? (n_slots + srpw - 1) / srpw : 0;
-    const bool split = Fs && sh_waves <= 4 && n_a <= (kFusedWaves - sh_waves) * 8 * kWave;
+    // (the first token only: the later tokens' routed words have arrived as well by then, and one fetch of
+    // everything is a trip past L2 shorter than two behind each other)
+    const bool split = tok == 0 && Fs && sh_waves <= 4 && n_a <= (kFusedWaves - sh_waves) * 8 * kWave;
     if (split) {
       gather(n_a, n_s, 0, kFusedWaves);  // first try succeeds: one round trip
       __syncthreads();

@@ -766,6 +766,8 @@ def phase_trace(ctx, w, stack, moes, device, with_norm=False) -> int:
 OTHER_CONFIGS = [
     # (key, BASELINE.json configuration, extra arguments of this script)
     ("single_expert_ffn_T1", 0, ["--workload", "single-expert", "--steps", "20", "--warmup", "5"]),
+    # the headline layer at the token count of an MTP verification step (not a BASELINE row of its own)
+    ("qwen_layer_T4", 1, ["--tokens", "4", "--steps", "100", "--warmup", "10"]),
     ("large_2bit_layer_T1", 3, ["--workload", "dsv4-2bit", "--steps", "100", "--warmup", "10"]),
     ("large_2bit_layer_T4", 3, ["--workload", "dsv4-2bit", "--tokens", "4", "--steps", "100", "--warmup", "10"]),
     ("ternary_layer_T1", 4, ["--workload", "maple-ternary", "--steps", "100", "--warmup", "10"]),
